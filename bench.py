@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the eden_utils compression hot path on one MI355X.
+
+A step = scaling_compress followed by scaling_decompress of one 25 MB DDP
+bucket (6,553,600 fp32 gradient elements, Student-t(3) * 1e-3 with 0.1 % of the
+entries multiplied by 100), hierarchical AEE (strategy 2), chunk 16, 4-bit
+codes, bf16 random pool -- the second configuration of BASELINE.json.  Inputs
+are resident in HBM before the timed region; the calls go through the C ABI of
+libdynamiq_eden.so on torch's current stream.
+
+Prints ONE JSON line (see the fields below).  `value` is fp32 gradient bytes
+(4 * N) per second of compress+decompress.  `roofline` prices the dominant
+kernel (compress) at its algorithmic bytes (4 + 2 + (q + 0.5625) / 8 per
+element) against the 8 TB/s HBM peak, with the kernel's average launch duration
+measured here with HIP events on the launch stream.  `cpu_baseline` times the
+scalar C oracle (a port of the reference algorithm) on the host, on one core.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+OVERHEAD_BITS = 0.5625  # hierarchical scale bytes per element, in bits
+
+
+def make_bucket(n, seed, device):
+    """Student-t(nu=3) * 1e-3 with 0.1 % outliers * 100, generated on the device."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    z = torch.randn(n, generator=g, device=device)
+    chi = torch.randn(3, n, generator=g, device=device).square_().sum(0)
+    x = z / torch.sqrt(chi / 3.0) * 1e-3
+    idx = torch.randint(0, n, (max(1, n // 1000),), generator=g, device=device)
+    x[idx] *= 100.0
+    return x.contiguous()
+
+
+def event_ms(fn, iters):
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--n", type=int, default=6553600, help="gradient elements in the bucket")
+    ap.add_argument("--nbits", type=int, default=4)
+    ap.add_argument("--strategy", type=int, default=2, help="2 = hierarchical AEE, 3 = hierarchical MEE")
+    ap.add_argument("--src", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the cpu_baseline leg (0 = skip)")
+    ap.add_argument("--no-check", action="store_true", help="skip the oracle parity check of a sample")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the path; --gpus must be 1 "
+              "(no collectives, sharding or multi-rank code is part of this build)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+
+    from dynamiq_sigcomm_artifact_amd import capi
+    capi.lib()  # fail loudly when the HIP library is missing
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    n = args.n // 256 * 256
+    nbits, strategy, C = args.nbits, args.strategy, 16
+    x32 = make_bucket(n, 0, dev)
+    src = x32 if args.src == "fp32" else x32.to(torch.bfloat16)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+    packed = torch.zeros(capi.required_bytes(n, nbits, C, strategy), dtype=torch.uint8, device=dev)
+    out = torch.empty_like(src)
+
+    def compress():
+        capi.scaling_compress(src, packed, rand, n, nbits, C, strategy)
+
+    def decompress():
+        capi.scaling_decompress(packed, out, n, nbits, C, strategy)
+
+    def step():
+        compress()
+        decompress()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly `steps` steps between two synchronisations ----
+    t0 = time.perf_counter()
+    ms_per_step = event_ms(step, args.steps)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = 4.0 * n / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-kernel launch durations (same stream, HIP events) ----
+    comp_ms = event_ms(compress, args.steps)
+    dec_ms = event_ms(decompress, args.steps)
+    sbytes = 4 if args.src == "fp32" else 2
+    comp_bytes = (sbytes + 2 + (nbits + OVERHEAD_BITS) / 8.0) * n
+    dec_bytes = (sbytes + (nbits + OVERHEAD_BITS) / 8.0) * n
+    comp_gbs = comp_bytes / (comp_ms * 1e-3) / 1e9
+    dec_gbs = dec_bytes / (dec_ms * 1e-3) / 1e9
+
+    # ---- quality: NMSE of the round trip ----
+    xf = x32.double()
+    nmse = float(((out.double() - xf) ** 2).sum() / (xf ** 2).sum())
+
+    # ---- parity of a sample against the oracle (the checker, not the product) ----
+    bit_exact = None
+    cpu = None
+    if not args.no_check or args.cpu_seconds > 0:
+        import oracle as O
+        odt = O.F32 if args.src == "fp32" else O.BF16
+        m = min(n, 1 << 20)
+
+        def host_bits(t):
+            t = t[:m].cpu().contiguous()
+            if t.dtype == torch.float32:
+                return t.numpy().copy()
+            return t.view(torch.int16).numpy().view(np.uint16).copy()
+
+        src_h = host_bits(src)
+        rand_h = host_bits(rand.float() if args.src == "fp32" else rand)
+        if not args.no_check:
+            enc_o = O.scaling_compress(src_h, rand_h, m, nbits, C, strategy, odt)
+            dec_o = np.zeros(m, src_h.dtype)
+            O.scaling_decompress(enc_o, dec_o, m, nbits, C, strategy, odt)
+            nb = O.required_bytes(m, nbits, C, strategy)
+            bit_exact = bool((packed[:nb].cpu().numpy() == enc_o).all() and (host_bits(out) == dec_o).all())
+        if args.cpu_seconds > 0:
+            reps, spent = 0, 0.0
+            dec_o = np.zeros(m, src_h.dtype)
+            while spent < args.cpu_seconds and reps < 64:
+                t1 = time.perf_counter()
+                enc_o = O.scaling_compress(src_h, rand_h, m, nbits, C, strategy, odt)
+                O.scaling_decompress(enc_o, dec_o, m, nbits, C, strategy, odt)
+                spent += time.perf_counter() - t1
+                reps += 1
+            cpu = {
+                "value": round(4.0 * m * reps / spent / 1e9, 4),
+                "unit": "GB/s",
+                "cores": 1,
+                "kind": "port",
+                "sample": "first %d elements of the same bucket, %d compress+decompress round trips of the scalar C oracle"
+                          % (m, reps),
+            }
+
+    result = {
+        "metric": "compress+decompress GB/s (fp32 grad in) on 1 MI355X, % of HBM peak; NMSE",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "one 25 MB DDP bucket: %d %s gradient elements, Student-t(3)*1e-3 with 0.1%% outliers x100; "
+                        "%d-bit hierarchical %s compress + decompress, chunk 16, bf16 rand_pool"
+                        % (n, args.src, nbits, "AEE" if strategy == 2 else "MEE"),
+            "elements": n,
+            "nbits": nbits,
+            "strategy": strategy,
+            "chunk_size": C,
+            "source_dtype": args.src,
+            "packed_bytes": int(packed.numel()),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "hier16_compress_kernel",
+            "achieved": round(comp_gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(comp_gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": int(comp_bytes),
+            "avg_launch_ms": round(comp_ms, 5),
+        },
+        "kernels": {
+            "compress": {"ms": round(comp_ms, 5), "algorithmic_GBps": round(comp_gbs, 1), "frac_hbm": round(comp_gbs / HBM_PEAK_GBS, 4)},
+            "decompress": {"ms": round(dec_ms, 5), "algorithmic_GBps": round(dec_gbs, 1), "frac_hbm": round(dec_gbs / HBM_PEAK_GBS, 4)},
+        },
+        "frac_hbm_roundtrip": round((comp_bytes + dec_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "nmse": nmse,
+        "bit_exact_vs_oracle": bit_exact,
+        "host_wall_ms_per_step": round(wall_ms, 5),
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

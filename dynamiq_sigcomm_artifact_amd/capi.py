@@ -1,0 +1,180 @@
+"""ctypes binding of the C ABI (``include/dynamiq_eden.h``) for torch tensors.
+
+Thin and explicit on purpose: each wrapper passes ``data_ptr()``, sizes, the
+device index and a stream handle straight to ``libdynamiq_eden.so`` and raises
+``RuntimeError`` with the library's message when the status is non-zero.  The
+library must be present; there is no fallback path.
+"""
+import ctypes
+import os
+
+import torch
+
+F16, BF16, F32 = 0, 1, 2
+RAND_BF16 = 0x10
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libdynamiq_eden.so")
+
+EXPORTS = [
+    "dq_status_string", "dq_last_error", "dq_version",
+    "dq_scaling_required_bytes", "dq_scaling_check_common",
+    "dq_init_lookup_table", "dq_mee_lookup_table",
+    "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
+    "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
+    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag",
+    "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
+]
+
+_lib = None
+
+
+def lib():
+    """The loaded shared library (raises if it has not been built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -m dynamiq_sigcomm_artifact_amd.build`" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        c = ctypes
+        vp, i64, i32, f32, u64 = c.c_void_p, c.c_int64, c.c_int, c.c_float, c.c_uint64
+        L.dq_status_string.restype = c.c_char_p
+        L.dq_status_string.argtypes = [i32]
+        L.dq_last_error.restype = c.c_char_p
+        L.dq_last_error.argtypes = []
+        L.dq_version.restype = c.c_char_p
+        L.dq_version.argtypes = []
+        L.dq_scaling_required_bytes.restype = i64
+        L.dq_scaling_required_bytes.argtypes = [i64, i32, i32, i32]
+        L.dq_scaling_check_common.restype = i32
+        L.dq_scaling_check_common.argtypes = [i64, i32, i32, i32, i32]
+        L.dq_init_lookup_table.restype = i32
+        L.dq_init_lookup_table.argtypes = []
+        L.dq_mee_lookup_table.restype = i32
+        L.dq_mee_lookup_table.argtypes = [i32, vp, vp]
+        L.dq_scaling_compress.restype = i32
+        L.dq_scaling_compress.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, i32, vp]
+        L.dq_scaling_decompress.restype = i32
+        L.dq_scaling_decompress.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, i32]
+        L.dq_scaling_dec_comp.restype = i32
+        L.dq_scaling_dec_comp.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp]
+        L.dq_superchunk_mean_center.restype = i32
+        L.dq_superchunk_mean_center.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, vp]
+        L.dq_superchunk_add_mean_copy.restype = i32
+        L.dq_superchunk_add_mean_copy.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
+        L.dq_hadamard.restype = i32
+        L.dq_hadamard.argtypes = [vp, i64, i32, vp, i32]
+        L.dq_rht_blocked.restype = i32
+        L.dq_rht_blocked.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp]
+        L.dq_rand_diag.restype = i32
+        L.dq_rand_diag.argtypes = [vp, i64, i64, i32, vp]
+        L.dq_bins_to_bits.restype = i32
+        L.dq_bins_to_bits.argtypes = [vp, i64, vp, i64, i32, i32, vp]
+        L.dq_bits_to_bins.restype = i32
+        L.dq_bits_to_bins.argtypes = [vp, i64, vp, i64, i32, i32, vp]
+        L.dq_quantization.restype = i32
+        L.dq_quantization.argtypes = [vp, i64, i32, f32, f32, u64, vp]
+        _lib = L
+    return _lib
+
+
+def dtype_code(t):
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.bfloat16:
+        return BF16
+    if t.dtype == torch.float32:
+        return F32
+    raise RuntimeError("unsupported element dtype %s" % t.dtype)
+
+
+def _pair_code(elem, rand_pool):
+    """dtype argument for the compress-side calls: fp32 gradients may come with a bf16 rand_pool."""
+    code = dtype_code(elem)
+    if rand_pool.dtype != elem.dtype:
+        if code == F32 and rand_pool.dtype == torch.bfloat16:
+            return code | RAND_BF16
+        raise RuntimeError("rand_pool dtype must match input dtype")
+    return code
+
+
+def _check(rc):
+    if rc != 0:
+        raise RuntimeError(lib().dq_last_error().decode())
+
+
+def _stream(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    return ctypes.c_void_p(int(stream))
+
+
+def _dev(t):
+    return t.device.index if t.device.index is not None else torch.cuda.current_device()
+
+
+def required_bytes(n, nbits, chunk_size, strategy):
+    return int(lib().dq_scaling_required_bytes(n, nbits, chunk_size, strategy))
+
+
+def check_common(n, nbits, chunk_size, strategy, strict=True):
+    _check(lib().dq_scaling_check_common(n, nbits, chunk_size, strategy, 1 if strict else 0))
+
+
+def mee_lookup_table(nbits):
+    import numpy as np
+    table = np.zeros(256, np.uint16)
+    params = np.zeros(4, np.uint16)
+    _check(lib().dq_mee_lookup_table(nbits, table.ctypes.data_as(ctypes.c_void_p), params.ctypes.data_as(ctypes.c_void_p)))
+    return table, params
+
+
+def scaling_compress(src, dst, rand_pool, n, nbits, chunk_size, strategy, stream=None):
+    _check(lib().dq_scaling_compress(src.data_ptr(), dst.data_ptr(), rand_pool.data_ptr(), n, nbits, chunk_size,
+                                     _pair_code(src, rand_pool), _dev(src), strategy, _stream(stream)))
+
+
+def scaling_decompress(src, dst, n, nbits, chunk_size, strategy, add=False, stream=None):
+    _check(lib().dq_scaling_decompress(src.data_ptr(), dst.data_ptr(), n, nbits, chunk_size, dtype_code(dst), _dev(dst),
+                                       strategy, _stream(stream), 1 if add else 0))
+
+
+def scaling_dec_comp(recv, inp, send, rand_pool, n, nbits, chunk_size, strategy, stream=None):
+    _check(lib().dq_scaling_dec_comp(recv.data_ptr(), inp.data_ptr(), send.data_ptr(), rand_pool.data_ptr(), n, nbits,
+                                     chunk_size, _pair_code(inp, rand_pool), _dev(inp), strategy, _stream(stream)))
+
+
+def superchunk_mean_center(src, residual, stats, n, world_size, superchunk_size=256, stream=None):
+    _check(lib().dq_superchunk_mean_center(src.data_ptr(), residual.data_ptr(), stats.data_ptr(), n, world_size,
+                                           superchunk_size, dtype_code(src), _dev(src), _stream(stream)))
+
+
+def superchunk_add_mean_copy(residual, dst, stats, n, superchunk_size=256, stream=None):
+    _check(lib().dq_superchunk_add_mean_copy(residual.data_ptr(), dst.data_ptr(), stats.data_ptr(), n, superchunk_size,
+                                             dtype_code(residual), _dev(residual), _stream(stream)))
+
+
+def hadamard(vec, stream=None):
+    _check(lib().dq_hadamard(vec.data_ptr(), vec.numel(), _dev(vec), _stream(stream), 0))
+
+
+def rht_blocked(vec, sign, block, scale, inverse=False, stream=None):
+    _check(lib().dq_rht_blocked(vec.data_ptr(), 0 if sign is None else sign.data_ptr(), vec.numel(), block, float(scale),
+                                1 if inverse else 0, _dev(vec), _stream(stream)))
+
+
+def rand_diag(out, seed, stream=None):
+    _check(lib().dq_rand_diag(out.data_ptr(), out.numel(), seed, _dev(out), _stream(stream)))
+
+
+def bins_to_bits(bins, arr, nbits, stream=None):
+    _check(lib().dq_bins_to_bits(bins.data_ptr(), bins.numel(), arr.data_ptr(), arr.numel(), nbits, _dev(bins), _stream(stream)))
+
+
+def bits_to_bins(bins, arr, nbits, stream=None):
+    _check(lib().dq_bits_to_bins(bins.data_ptr(), bins.numel(), arr.data_ptr(), arr.numel(), nbits, _dev(bins), _stream(stream)))
+
+
+def quantization(vec, div_factor, tensor_max, seed, stream=None):
+    _check(lib().dq_quantization(vec.data_ptr(), vec.numel(), _dev(vec), float(div_factor), float(tensor_max), int(seed),
+                                 _stream(stream)))

@@ -1,0 +1,365 @@
+// C ABI of libdynamiq_eden.so: argument validation, MEE table, kernel dispatch.
+// Declarations and the reference entry point each function replaces are in
+// include/dynamiq_eden.h.
+#include <math.h>
+#include <string.h>
+
+#include <mutex>
+#include <string>
+
+#include "dq_device.cuh"
+#include "dq_launch.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+const char *status_text(int s)
+{
+    switch (s) {
+    case DQ_OK: return "ok";
+    case DQ_ERR_N: return "n must be positive";
+    case DQ_ERR_NBITS: return "nbits must be one of {2, 4, 8}";
+    case DQ_ERR_STRATEGY: return "strategy must be 0 (AEE), 1 (MEE), 2 (hierarchical AEE), or 3 (hierarchical MEE)";
+    case DQ_ERR_CHUNK_RANGE: return "chunk_size must be in [1, 32]";
+    case DQ_ERR_CHUNK_POW2: return "chunk_size must be a power of two";
+    case DQ_ERR_CHUNK_BITS: return "chunk_size * nbits must be divisible by 8";
+    case DQ_ERR_N_CHUNK: return "n must be a multiple of chunk_size";
+    case DQ_ERR_N_SUPER: return "hierarchical mode requires n to contain a whole number of 16-chunk superchunks";
+    case DQ_ERR_DTYPE: return "unsupported element dtype";
+    case DQ_ERR_NULL: return "null pointer argument";
+    case DQ_ERR_SUPERCHUNK_SIZE: return "superchunk_size must be 256";
+    case DQ_ERR_WORLD_SIZE: return "world_size must be positive";
+    case DQ_ERR_POW2: return "input size must be a power of 2";
+    case DQ_ERR_SIZE: return "size mismatch";
+    case DQ_ERR_DEVICE: return "could not select the HIP device";
+    case DQ_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+    }
+}
+
+int fail(int status, const char *detail = nullptr)
+{
+    g_last_error = status_text(status);
+    if (detail) {
+        g_last_error += ": ";
+        g_last_error += detail;
+    }
+    return status;
+}
+
+int ok()
+{
+    g_last_error.clear();
+    return DQ_OK;
+}
+
+int finish(hipError_t e)
+{
+    if (e != hipSuccess) return fail(DQ_ERR_LAUNCH, hipGetErrorString(e));
+    return ok();
+}
+
+int select_device(int device)
+{
+    int cur = -1;
+    if (hipGetDevice(&cur) == hipSuccess && cur == device) return DQ_OK;
+    if (hipSetDevice(device) != hipSuccess) return fail(DQ_ERR_DEVICE);
+    return DQ_OK;
+}
+
+// ---- MEE lookup tables (host, built once) -----------------------------------------
+
+// binary32 -> binary16 bits, round to nearest even (host side)
+uint16_t host_f32_to_f16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x1ffu));
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);
+    if (a < 0x38800000u) {
+        float mag;
+        memcpy(&mag, &a, 4);
+        return (uint16_t)(sign | (uint16_t)nearbyintf(mag * 16777216.0f));
+    }
+    const uint32_t rounded = a + 0xfffu + ((a >> 13) & 1u);
+    return (uint16_t)(sign | (uint16_t)((rounded - 0x38000000u) >> 13));
+}
+
+float host_f16_to_f32(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t exp = (h >> 10) & 0x1fu, man = h & 0x3ffu;
+    uint32_t u;
+    if (exp == 0) {
+        float v = (float)man * 5.9604644775390625e-08f;
+        return sign ? -v : v;
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | (man << 13);
+    } else {
+        u = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+struct Lut {
+    uint16_t table[9][256];
+    uint16_t params[9][4];
+    dq::MeeParams mp[9];
+};
+
+Lut g_lut;
+std::once_flag g_lut_once;
+
+void build_lut()
+{
+    // csrc/cuda_hadamard.cu:873-899: fp32 host arithmetic, results kept as binary16
+    static const float epses[9] = {0.0f, 0.23f, 0.23f, 0.18f, 0.18f, 0.18f, 0.1f, 0.1f, 0.1f};
+    memset(&g_lut, 0, sizeof(g_lut));
+    for (int b = 1; b < 9; b++) {
+        const float eps = epses[b];
+        volatile float two_eps2 = 2.0f * eps * eps;
+        volatile float base = 1.0f + two_eps2;
+        volatile float one_plus_eps2 = 1.0f + eps * eps;
+        g_lut.params[b][0] = host_f32_to_f16(base);
+        g_lut.params[b][1] = host_f32_to_f16(one_plus_eps2 / two_eps2);
+        g_lut.params[b][3] = host_f32_to_f16(log2f(base));
+        const int anchor = (1 << (b - 1)) - 1;
+        volatile float pw = 1.0f;
+        for (int j = 1; j <= anchor; j++) {
+            pw = pw * base;
+            volatile float num = pw - 1.0f;
+            volatile float quo = num / two_eps2;
+            volatile float rep = quo * one_plus_eps2;
+            g_lut.table[b][anchor + j] = host_f32_to_f16(rep);
+            g_lut.table[b][anchor - j] = host_f32_to_f16(-rep);
+        }
+        g_lut.params[b][2] = g_lut.table[b][anchor * 2];
+        dq::MeeParams &m = g_lut.mp[b];
+        m.c = host_f16_to_f32(g_lut.params[b][1]);
+        m.cmm = host_f16_to_f32(g_lut.params[b][2]);
+        m.l2b = host_f16_to_f32(g_lut.params[b][3]);
+        m.pad = 0;
+        memcpy(m.table, g_lut.table[b], sizeof(m.table));
+    }
+}
+
+const dq::MeeParams &mee_params(int nbits)
+{
+    std::call_once(g_lut_once, build_lut);
+    return g_lut.mp[nbits];
+}
+
+int check_common(int64_t n, int nbits, int chunk_size, int strategy, int strict)
+{
+    if (!(n > 0)) return DQ_ERR_N;
+    if (strict) {
+        if (!(nbits == 2 || nbits == 4 || nbits == 8)) return DQ_ERR_NBITS;
+    } else if (nbits < 2 || nbits > 8) {
+        return DQ_ERR_NBITS;
+    }
+    if (strategy < 0 || strategy > 3) return DQ_ERR_STRATEGY;
+    if (!(chunk_size > 0 && chunk_size <= 32)) return DQ_ERR_CHUNK_RANGE;
+    if ((chunk_size & (chunk_size - 1)) != 0) return DQ_ERR_CHUNK_POW2;
+    if ((chunk_size * nbits) % 8 != 0) return DQ_ERR_CHUNK_BITS;
+    if (n % chunk_size != 0) return DQ_ERR_N_CHUNK;
+    if (strategy >= 2 && (n / chunk_size) % 16 != 0) return DQ_ERR_N_SUPER;
+    return DQ_OK;
+}
+
+inline bool dtype_ok(int dtype) { return dtype == DQ_F16 || dtype == DQ_BF16 || dtype == DQ_F32; }
+// compress-side dtype: the DQ_RAND_BF16 flag is only meaningful with DQ_F32 elements
+inline bool dtype_rand_ok(int dtype)
+{
+    if (dtype & ~(0xf | DQ_RAND_BF16)) return false;
+    if ((dtype & DQ_RAND_BF16) && (dtype & 0xf) != DQ_F32) return false;
+    return dtype_ok(dtype & 0xf);
+}
+
+// the vectorised kernels cover the production shape
+inline bool hier16_shape(int dtype, int chunk_size, int strategy)
+{
+    return (dtype == DQ_BF16 || dtype == DQ_F32) && chunk_size == 16 && strategy >= 2;
+}
+
+} // namespace
+
+extern "C" {
+
+const char *dq_status_string(int status) { return status_text(status); }
+const char *dq_last_error(void) { return g_last_error.c_str(); }
+const char *dq_version(void) { return "dynamiq_eden 0.1 gfx950"; }
+
+int64_t dq_scaling_required_bytes(int64_t n, int nbits, int chunk_size, int strategy)
+{
+    if (chunk_size <= 0) return 0;
+    const int64_t chunks = n / chunk_size;
+    const int64_t packed = ((int64_t)chunk_size * nbits) >> 3;
+    if (strategy >= 2) return (chunks / 16) * (16 * (packed + 1) + 2);
+    return chunks * (packed + 2);
+}
+
+int dq_scaling_check_common(int64_t n, int nbits, int chunk_size, int strategy, int strict)
+{
+    const int rc = check_common(n, nbits, chunk_size, strategy, strict);
+    return rc ? fail(rc) : ok();
+}
+
+int dq_init_lookup_table(void)
+{
+    (void)mee_params(2);
+    return ok();
+}
+
+int dq_mee_lookup_table(int nbits, uint16_t table[256], uint16_t params[4])
+{
+    if (nbits < 1 || nbits > 8) return fail(DQ_ERR_NBITS);
+    if (!table || !params) return fail(DQ_ERR_NULL);
+    (void)mee_params(nbits);
+    memcpy(table, g_lut.table[nbits], 256 * sizeof(uint16_t));
+    memcpy(params, g_lut.params[nbits], 4 * sizeof(uint16_t));
+    return ok();
+}
+
+int dq_scaling_compress(const void *src, uint8_t *dst, const void *rand_pool, int64_t n, int nbits, int chunk_size,
+                        int dtype, int device, int strategy, dq_stream_t stream)
+{
+    int rc = check_common(n, nbits, chunk_size, strategy, 0);
+    if (rc) return fail(rc);
+    if (!dtype_rand_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!src || !dst || !rand_pool) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dq::MeeParams &mp = mee_params(nbits);
+    if (hier16_shape(dtype & 0xf, chunk_size, strategy))
+        return finish(dq::launch_hier16_compress(src, dst, rand_pool, n, nbits, dtype, strategy == 3, mp, s));
+    return finish(dq::launch_generic_compress(src, dst, rand_pool, n, nbits, chunk_size, dtype, strategy, mp, s));
+}
+
+int dq_scaling_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int chunk_size, int dtype, int device,
+                          int strategy, dq_stream_t stream, int add_original)
+{
+    int rc = check_common(n, nbits, chunk_size, strategy, 0);
+    if (rc) return fail(rc);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!src || !dst) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dq::MeeParams &mp = mee_params(nbits);
+    if (hier16_shape(dtype, chunk_size, strategy))
+        return finish(dq::launch_hier16_decompress(src, dst, n, nbits, dtype, strategy == 3, mp, add_original, s));
+    return finish(dq::launch_generic_decompress(src, dst, n, nbits, chunk_size, dtype, strategy, mp, add_original, s));
+}
+
+int dq_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const void *rand_pool, int64_t n, int nbits,
+                        int chunk_size, int dtype, int device, int strategy, dq_stream_t stream)
+{
+    int rc = check_common(n, nbits, chunk_size, strategy, 0);
+    if (rc) return fail(rc);
+    if (!dtype_rand_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!recv || !inp || !send || !rand_pool) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dq::MeeParams &mp = mee_params(nbits);
+    if (hier16_shape(dtype & 0xf, chunk_size, strategy))
+        return finish(dq::launch_hier16_dec_comp(recv, inp, send, rand_pool, n, nbits, dtype, strategy == 3, mp, s));
+    // every other combination: decode into inp, then compress inp (two kernels, inp is modified)
+    hipError_t e = dq::launch_generic_decompress(recv, inp, n, nbits, chunk_size, dtype & 0xf, strategy, mp, 1, s);
+    if (e != hipSuccess) return finish(e);
+    return finish(dq::launch_generic_compress(inp, send, rand_pool, n, nbits, chunk_size, dtype, strategy, mp, s));
+}
+
+int dq_superchunk_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size,
+                              int superchunk_size, int dtype, int device, dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (!(world_size > 0)) return fail(DQ_ERR_WORLD_SIZE);
+    if (superchunk_size != 256) return fail(DQ_ERR_SUPERCHUNK_SIZE);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!src || !residual || !stats) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_mean_center(src, residual, stats, n, world_size, dtype, static_cast<hipStream_t>(stream)));
+}
+
+int dq_superchunk_add_mean_copy(const void *residual, void *dst, const void *stats, int64_t n, int superchunk_size,
+                                int dtype, int device, dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (superchunk_size != 256) return fail(DQ_ERR_SUPERCHUNK_SIZE);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!residual || !dst || !stats) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_add_mean_copy(residual, dst, stats, n, dtype, static_cast<hipStream_t>(stream)));
+}
+
+int dq_hadamard(float *vec, int64_t n, int device, dq_stream_t stream, int depth)
+{
+    (void)depth;
+    if (!(n > 0) || (n & (n - 1)) != 0) return fail(DQ_ERR_POW2);
+    if (!vec) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_hadamard(vec, n, static_cast<hipStream_t>(stream)));
+}
+
+int dq_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale, int inverse, int device,
+                   dq_stream_t stream)
+{
+    if (!(block > 0) || (block & (block - 1)) != 0) return fail(DQ_ERR_POW2, "block");
+    if (!(n > 0) || n % block != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of block");
+    if (!vec) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_rht_blocked(vec, sign, n, block, scale, inverse, static_cast<hipStream_t>(stream)));
+}
+
+int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t stream)
+{
+    if (!(size > 0)) return fail(DQ_ERR_N);
+    if (!out) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_rand_diag(out, size, seed, static_cast<hipStream_t>(stream)));
+}
+
+int dq_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int64_t narr, int nbits, int device,
+                    dq_stream_t stream)
+{
+    if (nbits < 1 || nbits > 32) return fail(DQ_ERR_NBITS, "nbits must be in [1, 32]");
+    if (!(nbins > 0) || (nbins & 31) != 0) return fail(DQ_ERR_SIZE, "bins size must be a multiple of 32");
+    if (narr != (nbins >> 5) * nbits) return fail(DQ_ERR_SIZE, "narr must equal nbins / 32 * nbits");
+    if (!bins || !arr) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_bins_to_bits(bins, nbins, arr, nbits, static_cast<hipStream_t>(stream)));
+}
+
+int dq_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int64_t narr, int nbits, int device,
+                    dq_stream_t stream)
+{
+    if (nbits < 1 || nbits > 32) return fail(DQ_ERR_NBITS, "nbits must be in [1, 32]");
+    if (!(nbins > 0) || (nbins & 31) != 0) return fail(DQ_ERR_SIZE, "bins size must be a multiple of 32");
+    if (narr != (nbins >> 5) * nbits) return fail(DQ_ERR_SIZE, "narr must equal nbins / 32 * nbits");
+    if (!bins || !arr) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_bits_to_bins(bins, nbins, arr, nbits, static_cast<hipStream_t>(stream)));
+}
+
+int dq_quantization(float *vec, int64_t n, int device, float div_factor, float tensor_max, uint64_t seed,
+                    dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (!vec) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_quantization(vec, n, div_factor, tensor_max, seed, static_cast<hipStream_t>(stream)));
+}
+
+} // extern "C"

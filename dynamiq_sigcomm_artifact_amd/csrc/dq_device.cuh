@@ -1,0 +1,240 @@
+// Device-side numeric primitives shared by the gfx950 kernels.
+//
+// Arithmetic contract (the kernels are checked byte-for-byte against a CPU
+// restatement that follows the same rules): IEEE binary32, round to nearest
+// even, denormals preserved, no implicit contraction (the translation units
+// are compiled with -ffp-contract=off); a multiply-add is fused only where
+// __builtin_fmaf is spelled out.  Half-precision operations are an fp32
+// operation followed by one rounding to binary16.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dynamiq_eden.h"
+
+namespace dq {
+
+// ---- storage formats -------------------------------------------------------
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+    __bf16 b = (__bf16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi)
+{
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {lo, hi};
+    bf16x2 b = __builtin_convertvector(v, bf16x2);
+    return __builtin_bit_cast(uint32_t, b);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
+{
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f)
+{
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// value of a binary16 result computed through fp32
+__device__ __forceinline__ float rh(float x) { return (float)(_Float16)x; }
+// value after a round trip through bfloat16
+__device__ __forceinline__ float rb(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+
+template <int DT> struct ElemIO;
+
+template <> struct ElemIO<DQ_F16> {
+    typedef uint16_t storage;
+    static __device__ __forceinline__ float load(const void *p, int64_t i) { return f16_bits_to_f32(((const uint16_t *)p)[i]); }
+    static __device__ __forceinline__ void store(void *p, int64_t i, float v) { ((uint16_t *)p)[i] = (uint16_t)f32_to_f16_bits(v); }
+    static __device__ __forceinline__ float round(float v) { return rh(v); }
+};
+template <> struct ElemIO<DQ_BF16> {
+    typedef uint16_t storage;
+    static __device__ __forceinline__ float load(const void *p, int64_t i) { return bf16_bits_to_f32(((const uint16_t *)p)[i]); }
+    static __device__ __forceinline__ void store(void *p, int64_t i, float v) { ((uint16_t *)p)[i] = (uint16_t)f32_to_bf16_bits(v); }
+    static __device__ __forceinline__ float round(float v) { return rb(v); }
+};
+template <> struct ElemIO<DQ_F32> {
+    typedef float storage;
+    static __device__ __forceinline__ float load(const void *p, int64_t i) { return ((const float *)p)[i]; }
+    static __device__ __forceinline__ void store(void *p, int64_t i, float v) { ((float *)p)[i] = v; }
+    static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+// ---- conversions with saturating / wrapping device semantics ---------------
+
+__device__ __forceinline__ int sat_i16(float x) // truncate, saturate, NaN -> 0
+{
+    int v = (int)x; // v_cvt_i32_f32: saturating, NaN -> 0
+    return min(max(v, -32768), 32767);
+}
+
+__device__ __forceinline__ int sat_u16(float x)
+{
+    int v = (int)x;
+    return min(max(v, 0), 65535);
+}
+
+__device__ __forceinline__ int wrap_i16(int x) { return (int)(int16_t)x; }
+
+__device__ __forceinline__ int clamp_code(int signed_val, int range)
+{
+    return min(max(signed_val, -range), range) + range;
+}
+
+// ---- scale guards (fp32 path) ---------------------------------------------
+
+__device__ __forceinline__ float pos_scale(float v)
+{
+    v = __builtin_isfinite(v) ? v : 1.0e-30f;
+    return __builtin_fmaxf(v, 1.0e-30f);
+}
+
+__device__ __forceinline__ float nonneg_scale(float v)
+{
+    v = __builtin_isfinite(v) ? v : 0.0f;
+    return __builtin_fmaxf(v, 0.0f);
+}
+
+// ---- deterministic log2 ----------------------------------------------------
+// x = 2^k * z, z in [sqrt(1/2), sqrt(2)); log2(z) = f*log2(e) + f^2*Q(f) with
+// f = z - 1 and Q a fixed degree-8 polynomial evaluated by Horner with fused
+// multiply-adds.  <= 1.7 ulp; identical on any IEEE machine.
+__device__ __forceinline__ float log2_det(float x)
+{
+    uint32_t ix = __float_as_uint(x);
+    int k = 0;
+    if (ix >= 0x7f800000u) {
+        if (ix == 0x7f800000u) return x;
+        if ((ix & 0x7fffffffu) > 0x7f800000u) return x + x;
+        if ((ix << 1) == 0) return -__builtin_inff();
+        return __uint_as_float(0x7fc00000u);
+    }
+    if (ix < 0x00800000u) {
+        if (ix == 0) return -__builtin_inff();
+        x *= 8388608.0f;
+        ix = __float_as_uint(x);
+        k = -23;
+    }
+    uint32_t t = ix - 0x3f3504f3u;
+    k += (int)t >> 23;
+    float z = __uint_as_float(ix - (t & 0xff800000u));
+    float f = z - 1.0f;
+    float q = -0x1.d0dd08p-4f;
+    q = __builtin_fmaf(q, f, 0x1.7ad622p-3f);
+    q = __builtin_fmaf(q, f, -0x1.831b24p-3f);
+    q = __builtin_fmaf(q, f, 0x1.a33bdap-3f);
+    q = __builtin_fmaf(q, f, -0x1.eb492p-3f);
+    q = __builtin_fmaf(q, f, 0x1.277e38p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715762p-2f);
+    q = __builtin_fmaf(q, f, 0x1.ec7092p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715476p-1f);
+    float p = (f * f) * q;
+    float r = __builtin_fmaf(f, 0x1.4ae0cp-26f, p);
+    r = __builtin_fmaf(f, 0x1.715476p+0f, r);
+    return (float)k + r;
+}
+
+// ---- stochastic rounding ----------------------------------------------------
+
+// floor(x) + ceil(frac - r) in int16 arithmetic, no guards
+__device__ __forceinline__ int sr_plain(float x, float r)
+{
+    float fl = __builtin_floorf(x);
+    int s = sat_i16(fl);
+    return wrap_i16(s + sat_i16(__builtin_ceilf((x - fl) - r)));
+}
+
+// non-finite and out-of-range inputs saturate to +-32767 (NaN -> 0); a
+// non-finite random value counts as 0
+__device__ __forceinline__ int sr_guarded(float x, float r)
+{
+    r = __builtin_isfinite(r) ? r : 0.0f;
+    int s = sr_plain(x, r);
+    if (!__builtin_isfinite(x)) s = (x > 0.0f) ? 32767 : ((x < 0.0f) ? -32767 : 0);
+    else if (x >= 32767.0f) s = 32767;
+    else if (x <= -32767.0f) s = -32767;
+    return s;
+}
+
+__device__ __forceinline__ float mee_inverse_plain(float x, float c, float l2b)
+{
+    float a = __builtin_fabsf(x);
+    if (!(a > 0.0f)) return 0.0f;
+    float lat = log2_det(a / c + 1.0f) / l2b;
+    return x < 0.0f ? -lat : lat;
+}
+
+__device__ __forceinline__ float mee_inverse_guarded(float x, float c, float l2b)
+{
+    if (!__builtin_isfinite(x)) return (x > 0.0f) ? 32767.0f : ((x < 0.0f) ? -32767.0f : 0.0f);
+    return mee_inverse_plain(x, c, l2b);
+}
+
+// ---- half-precision op set (fp32 op, one rounding to binary16) --------------
+
+__device__ __forceinline__ float h_add(float a, float b) { return rh(a + b); }
+__device__ __forceinline__ float h_sub(float a, float b) { return rh(a - b); }
+__device__ __forceinline__ float h_mul(float a, float b) { return rh(a * b); }
+__device__ __forceinline__ float h_div(float a, float b) { return rh(a / b); }
+__device__ __forceinline__ float h_max(float a, float b)
+{
+    if (a != a) return b;
+    if (b != b) return a;
+    return a > b ? a : b;
+}
+
+__device__ __forceinline__ int sr_half(float x, float r)
+{
+    float fl = __builtin_floorf(x);
+    int s = sat_i16(fl);
+    float frac = h_sub(x, fl);
+    return wrap_i16(s + sat_i16(__builtin_ceilf(h_sub(frac, r))));
+}
+
+__device__ __forceinline__ float mee_inverse_half(float x, float c, float l2b)
+{
+    float a = __builtin_fabsf(x);
+    if (!(a > 0.0f)) return 0.0f;
+    float arg = h_add(h_div(a, c), 1.0f);
+    float lat = h_div(rh(log2_det(arg)), l2b);
+    return x < 0.0f ? -lat : lat;
+}
+
+// ---- DPP row helpers (row = 16 lanes) ---------------------------------------
+
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// maximum over the 16 lanes of a DPP row with the fmaxf rule (NaN dropped)
+__device__ __forceinline__ float row16_max(float v)
+{
+    v = __builtin_fmaxf(v, dpp_f32<0xB1>(v));  // quad_perm [1,0,3,2]
+    v = __builtin_fmaxf(v, dpp_f32<0x4E>(v));  // quad_perm [2,3,0,1]
+    v = __builtin_fmaxf(v, dpp_f32<0x141>(v)); // row_half_mirror
+    v = __builtin_fmaxf(v, dpp_f32<0x140>(v)); // row_mirror
+    return v;
+}
+
+// parameters of the MEE lattice, built on the host and passed by value
+struct MeeParams {
+    float c;   // (1+e^2)/(2e^2), binary16 widened
+    float cmm; // chunk_max_mee, binary16 widened
+    float l2b; // log2(1+2e^2), binary16 widened
+    uint32_t pad;
+    uint16_t table[256]; // binary16 bit patterns
+};
+
+} // namespace dq

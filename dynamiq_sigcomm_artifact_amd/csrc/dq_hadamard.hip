@@ -1,0 +1,275 @@
+// Fast Walsh-Hadamard transform (unnormalised, Sylvester order) and the blocked
+// randomized transform built on it.
+//
+// One kernel does everything: a workgroup owns a tile of 2^kt floats in LDS and
+// applies the butterfly stages of a contiguous range of index bits to it.
+//   * contiguous pass: the tile is 2^kt consecutive floats and the stages are
+//     strides 1 .. 2^(kt-1) (or fewer when the transform block is smaller than
+//     the tile, so several small blocks share one tile);
+//   * strided pass (vectors longer than one tile): the tile is 2^r "rows" of
+//     2^c consecutive floats taken at stride 2^s, and the stages are the row
+//     bits, i.e. strides 2^s .. 2^(s+r-1) of the vector.
+// A whole-vector transform of n = 2^k is one contiguous pass plus
+// ceil((k-kt)/r) strided passes; each pass is one read and one write of the
+// vector.  Stages always run in ascending stride with butterflies (a+b, a-b),
+// which is the order of csrc/cuda_hadamard.cu:66-157,205-274,534-605, so the
+// result is bit-identical to a plain stage-by-stage FWHT.
+//
+// Inside the tile the stages are done four at a time (radix 16) on registers;
+// the LDS index is padded by one float per 16 (i + i/16), which keeps every
+// access pattern used here free of bank conflicts.
+#include "dq_device.cuh"
+#include "dq_launch.h"
+
+namespace dq {
+
+__device__ __forceinline__ int pad_idx(int i) { return i + (i >> 4); }
+
+template <int M> __device__ __forceinline__ void butterflies(float (&v)[1 << M])
+{
+#pragma unroll
+    for (int h = 1; h < (1 << M); h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < (1 << M); i++) {
+            if ((i & h) == 0) {
+                float a = v[i], b = v[i + h];
+                v[i] = a + b;
+                v[i + h] = a - b;
+            }
+        }
+    }
+}
+
+// stages for index bits [p, p+M) of the tile
+template <int M> __device__ __forceinline__ void lds_pass(float *lds, int p, int ntuples, int tid, int nthreads)
+{
+    for (int u = tid; u < ntuples; u += nthreads) {
+        const int lo = u & ((1 << p) - 1);
+        const int base = ((u >> p) << (p + M)) | lo;
+        float v[1 << M];
+#pragma unroll
+        for (int j = 0; j < (1 << M); j++) v[j] = lds[pad_idx(base + (j << p))];
+        butterflies<M>(v);
+#pragma unroll
+        for (int j = 0; j < (1 << M); j++) lds[pad_idx(base + (j << p))] = v[j];
+    }
+}
+
+struct FwhtArgs {
+    float *x;
+    const float *sign; // may be null
+    int64_t n;         // elements in the vector (for bounds of ragged tiles)
+    int kt;            // log2 tile elements
+    int b0, b1;        // tile-index bits to transform: [b0, b1)
+    int cbits;         // low cbits of the tile index are contiguous in memory
+    int sbits;         // vector stride of a tile row is 2^sbits (== cbits for a contiguous tile)
+    float scale;
+    int apply_scale;
+    int sign_mode;     // 0 none, 1 multiply on load, 2 multiply on store
+    int vec;           // 16-byte accesses allowed
+};
+
+__global__ void fwht_tile_kernel(FwhtArgs a)
+{
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int tile = 1 << a.kt;
+    const int cmask = (1 << a.cbits) - 1;
+    const int rbits = a.kt - a.cbits;
+
+    // tile -> position in the vector.  A contiguous tile (sbits == cbits) starts
+    // at blockIdx * 2^kt.  A strided tile covers rows rho = 0..2^rbits-1 at
+    // stride 2^sbits and columns [mid*2^cbits, +2^cbits):
+    //   index = hi * 2^(sbits+rbits) + rho * 2^sbits + mid * 2^cbits + col
+    int64_t origin;
+    if (a.sbits == a.cbits) {
+        origin = (int64_t)blockIdx.x << a.kt;
+    } else {
+        const int64_t mids = (int64_t)1 << (a.sbits - a.cbits);
+        const int64_t hi = blockIdx.x / mids, mid = blockIdx.x % mids;
+        origin = (hi << (a.sbits + rbits)) + (mid << a.cbits);
+    }
+
+    // load (coalesced), optional sign flip
+    if (a.vec) {
+        for (int i = tid * 4; i < tile; i += nthreads * 4) {
+            const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (g < a.n) {
+                v = *reinterpret_cast<const float4 *>(a.x + g);
+                if (a.sign_mode == 1) {
+                    const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
+                    v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
+                }
+            }
+            const int q = pad_idx(i); // i % 4 == 0: the four floats stay inside one padded group of 16
+            lds[q] = v.x; lds[q + 1] = v.y; lds[q + 2] = v.z; lds[q + 3] = v.w;
+        }
+    } else {
+        for (int i = tid; i < tile; i += nthreads) {
+            const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
+            float v = 0.0f;
+            if (g < a.n) {
+                v = a.x[g];
+                if (a.sign_mode == 1) v *= a.sign[g];
+            }
+            lds[pad_idx(i)] = v;
+        }
+    }
+    __syncthreads();
+
+    // butterfly stages, four index bits at a time
+    for (int p = a.b0; p < a.b1; p += 4) {
+        const int m = min(4, a.b1 - p);
+        const int ntuples = tile >> m;
+        switch (m) {
+        case 4: lds_pass<4>(lds, p, ntuples, tid, nthreads); break;
+        case 3: lds_pass<3>(lds, p, ntuples, tid, nthreads); break;
+        case 2: lds_pass<2>(lds, p, ntuples, tid, nthreads); break;
+        default: lds_pass<1>(lds, p, ntuples, tid, nthreads); break;
+        }
+        __syncthreads();
+    }
+
+    // store (coalesced), optional scale then sign flip
+    if (a.vec) {
+        for (int i = tid * 4; i < tile; i += nthreads * 4) {
+            const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
+            if (g >= a.n) continue;
+            const int q = pad_idx(i);
+            float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
+            if (a.apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
+            if (a.sign_mode == 2) {
+                const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
+                v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
+            }
+            *reinterpret_cast<float4 *>(a.x + g) = v;
+        }
+    } else {
+        for (int i = tid; i < tile; i += nthreads) {
+            const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
+            if (g >= a.n) continue;
+            float v = lds[pad_idx(i)];
+            if (a.apply_scale) v *= a.scale;
+            if (a.sign_mode == 2) v *= a.sign[g];
+            a.x[g] = v;
+        }
+    }
+}
+
+static inline int ilog2(int64_t v)
+{
+    int k = 0;
+    while (((int64_t)1 << (k + 1)) <= v) k++;
+    return k;
+}
+
+static hipError_t launch_tile(const FwhtArgs &a, int64_t ntiles, hipStream_t stream)
+{
+    const int tile = 1 << a.kt;
+    int threads = tile / 16;
+    threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+    const size_t lds_bytes = (size_t)(tile + tile / 16 + 1) * sizeof(float);
+    if (lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(fwht_tile_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(fwht_tile_kernel, dim3((unsigned)ntiles), dim3(threads), lds_bytes, stream, a);
+    return hipGetLastError();
+}
+
+constexpr int kMaxTileBits = 15; // 2^15 floats = 128 KiB (+ padding) of the 160 KiB LDS
+constexpr int kPrefTileBits = 13; // 32 KiB tiles keep several workgroups per CU in flight
+constexpr int kStridedCols = 5;   // 32 consecutive floats (128 B) per row of a strided tile
+
+// transform index bits [0, kb) of every aligned block of 2^kb elements of x[0..n)
+static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, float scale, int apply_scale,
+                              int inverse, hipStream_t stream)
+{
+    const bool vec16 = (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                       (sign == nullptr || (reinterpret_cast<uintptr_t>(sign) & 15) == 0);
+    FwhtArgs a;
+    a.x = x; a.sign = sign; a.n = n; a.scale = scale;
+    const int sign_fwd = (sign && !inverse) ? 1 : 0, sign_inv = (sign && inverse) ? 2 : 0;
+
+    if (kb <= kMaxTileBits) {
+        // single pass; small blocks share a tile
+        int kt = kb < kPrefTileBits ? kPrefTileBits : kb;
+        while (kt > kb && ((int64_t)1 << kt) > n) kt--;
+        a.kt = kt; a.b0 = 0; a.b1 = kb; a.cbits = kt; a.sbits = kt;
+        a.apply_scale = apply_scale; a.sign_mode = sign_fwd | sign_inv;
+        a.vec = vec16 && kt >= 2 && (n & 3) == 0;
+        const int64_t ntiles = (n + ((int64_t)1 << kt) - 1) >> kt;
+        return launch_tile(a, ntiles, stream);
+    }
+
+    // long transform: contiguous pass over the low bits, strided passes above
+    int kt = kPrefTileBits;
+    a.kt = kt; a.b0 = 0; a.b1 = kt; a.cbits = kt; a.sbits = kt;
+    a.apply_scale = 0; a.sign_mode = sign_fwd; a.vec = vec16;
+    hipError_t e = launch_tile(a, n >> kt, stream);
+    if (e != hipSuccess) return e;
+    int s = kt;
+    const int max_rows = kMaxTileBits - kStridedCols;
+    while (s < kb) {
+        // split the remaining bits evenly over as few passes as the LDS allows
+        const int rem = kb - s;
+        const int passes = (rem + max_rows - 1) / max_rows;
+        const int r = (rem + passes - 1) / passes;
+        a.kt = r + kStridedCols; a.b0 = kStridedCols; a.b1 = kStridedCols + r;
+        a.cbits = kStridedCols; a.sbits = s;
+        const bool last = (s + r == kb);
+        a.apply_scale = last ? apply_scale : 0;
+        a.sign_mode = last ? sign_inv : 0;
+        a.vec = vec16;
+        e = launch_tile(a, n >> a.kt, stream);
+        if (e != hipSuccess) return e;
+        s += r;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_hadamard(float *vec, int64_t n, hipStream_t stream)
+{
+    return fwht_blocks(vec, nullptr, n, ilog2(n), 1.0f, 0, 0, stream);
+}
+
+hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale, int inverse,
+                              hipStream_t stream)
+{
+    return fwht_blocks(vec, sign, n, ilog2(block), scale, 1, inverse, stream);
+}
+
+// ---- randDiag -----------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void rand_diag_kernel(float *__restrict__ out, int64_t size, int64_t s8, uint64_t ss)
+{
+    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (j >= s8) return;
+    const uint64_t M = 0xffffffffull;
+    uint64_t r = (uint64_t)j + ss;
+    r = (1103515245ull * r + 12345ull + ss) & M;
+    r = (1140671485ull * r + 12820163ull + ss) & M;
+    r += 0x9e3779b9ull; // the carry into bit 32 is kept
+    r = ((r ^ (r >> 16)) * 0x85ebca6bull) & M;
+    r = ((r ^ (r >> 13)) * 0xc2b2ae35ull) & M;
+    r = (r ^ (r >> 16)) & M;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const int64_t idx = (int64_t)k * s8 + j;
+        if (idx < size) out[idx] = ((r >> (4 * k)) & 15u) >= 8u ? 1.0f : -1.0f;
+    }
+}
+
+hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream)
+{
+    const uint64_t M = 0xffffffffull;
+    uint64_t ss = ((uint64_t)seed * 1664525ull + 1013904223ull) & M;
+    ss = (ss * 8121ull + 28411ull) & M;
+    const int64_t s8 = size / 8 + (size % 8 != 0);
+    hipLaunchKernelGGL(rand_diag_kernel, dim3((unsigned)((s8 + 255) / 256)), dim3(256), 0, stream, out, size, s8, ss);
+    return hipGetLastError();
+}
+
+} // namespace dq

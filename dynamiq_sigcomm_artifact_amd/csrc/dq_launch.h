@@ -1,0 +1,52 @@
+// Host-side launcher declarations shared by the translation units of
+// libdynamiq_eden.so.  Each launcher enqueues on `stream` and returns the
+// launch status; argument validation happens in the C ABI layer (dq_api.hip).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dq_device.cuh"
+
+namespace dq {
+
+// scaling quantisation, catch-all kernels (dq_scaling_generic.hip)
+hipError_t launch_generic_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n,
+                                   int nbits, int C, int dtype, int strategy, const MeeParams &mp,
+                                   hipStream_t stream);
+hipError_t launch_generic_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int C,
+                                     int dtype, int strategy, const MeeParams &mp, int add,
+                                     hipStream_t stream);
+
+// scaling quantisation, vectorised chunk-16 hierarchical kernels
+// (dq_scaling_hier16.hip); dtype BF16 or F32, element pointers 16-byte aligned
+hipError_t launch_hier16_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n,
+                                  int nbits, int dtype, bool mee, const MeeParams &mp,
+                                  hipStream_t stream);
+hipError_t launch_hier16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype,
+                                    bool mee, const MeeParams &mp, int add, hipStream_t stream);
+hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t *send,
+                                  const void *rnd, int64_t n, int nbits, int dtype, bool mee,
+                                  const MeeParams &mp, hipStream_t stream);
+
+// superchunk mean-centring (dq_superchunk.hip)
+hipError_t launch_mean_center(const void *src, void *residual, void *stats, int64_t n,
+                              int world_size, int dtype, hipStream_t stream);
+hipError_t launch_add_mean_copy(const void *residual, void *dst, const void *stats, int64_t n,
+                                int dtype, hipStream_t stream);
+
+// Walsh-Hadamard (dq_hadamard.hip)
+hipError_t launch_hadamard(float *vec, int64_t n, hipStream_t stream);
+hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale,
+                              int inverse, hipStream_t stream);
+hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream);
+
+// EDEN bit-plane packing and THC rounding (dq_packing.hip)
+hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits,
+                               hipStream_t stream);
+hipError_t launch_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int nbits,
+                               hipStream_t stream);
+hipError_t launch_quantization(float *vec, int64_t n, float div_factor, float tensor_max,
+                               uint64_t seed, hipStream_t stream);
+
+} // namespace dq

@@ -1,0 +1,98 @@
+// EDEN bit-plane packing (csrc/cuda_packing.cu:11-29,76-95) and the THC-style
+// in-place stochastic rounding (csrc/cuda_hadamard.cu:607-627).
+//
+// Packing on wave64: one lane per bin, one 64-bit ballot per bit plane, whose
+// halves are the two consecutive 32-bin words of that plane.
+#include "dq_device.cuh"
+#include "dq_launch.h"
+
+namespace dq {
+
+__global__ __launch_bounds__(256) void bins_to_bits_kernel(const int32_t *__restrict__ bins, int64_t nbins,
+                                                           uint32_t *__restrict__ arr, int nbits)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t words = nbins >> 5;
+    const int lane = threadIdx.x & 63;
+    const uint32_t b = (i < nbins) ? (uint32_t)bins[i] : 0u;
+    const int64_t w = i >> 5;
+    for (int p = 0; p < nbits; p++) {
+        const uint64_t m = __ballot((b >> p) & 1u);
+        if ((lane & 31) == 0 && w < words) arr[(int64_t)p * words + w] = (uint32_t)(m >> (lane & 32));
+    }
+}
+
+__global__ __launch_bounds__(256) void bits_to_bins_kernel(int32_t *__restrict__ bins, int64_t nbins,
+                                                           const uint32_t *__restrict__ arr, int nbits)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nbins) return;
+    const int64_t words = nbins >> 5;
+    const int64_t w = i >> 5;
+    const int t = (int)(i & 31);
+    int32_t v = 0;
+    for (int p = 0; p < nbits; p++) v += (int32_t)((arr[(int64_t)p * words + w] >> t) & 1u) << p;
+    bins[i] = v;
+}
+
+hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits, hipStream_t stream)
+{
+    hipLaunchKernelGGL(bins_to_bits_kernel, dim3((unsigned)((nbins + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
+    return hipGetLastError();
+}
+
+hipError_t launch_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int nbits, hipStream_t stream)
+{
+    hipLaunchKernelGGL(bits_to_bins_kernel, dim3((unsigned)((nbins + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
+    return hipGetLastError();
+}
+
+// ---- Philox4x32-10 -------------------------------------------------------------------
+
+__device__ __forceinline__ void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1)
+{
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+// four consecutive elements per thread share one Philox block keyed by
+// (seed, element index / 4); u = top 24 bits * 2^-24 in [0, 1)
+__global__ __launch_bounds__(256) void quantization_kernel(float *__restrict__ vec, int64_t n, float div_factor,
+                                                           float tensor_max, uint32_t k0, uint32_t k1)
+{
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i0 = g * 4;
+    if (i0 >= n) return;
+    uint32_t c[4] = {(uint32_t)g, (uint32_t)((uint64_t)g >> 32), 0u, 0u};
+    philox4x32_10(c, k0, k1);
+    const int cnt = (int)min((int64_t)4, n - i0);
+    for (int k = 0; k < cnt; k++) {
+        float t = vec[i0 + k] / div_factor;
+        t = t < tensor_max ? t : tensor_max;
+        t = t > -tensor_max ? t : -tensor_max;
+        const float fl = __builtin_floorf(t);
+        const float prob = t - fl;
+        const float u = (float)(c[k] >> 8) * 5.9604644775390625e-08f;
+        vec[i0 + k] = fl + ((u < prob) ? 1.0f : 0.0f);
+    }
+}
+
+hipError_t launch_quantization(float *vec, int64_t n, float div_factor, float tensor_max, uint64_t seed, hipStream_t stream)
+{
+    const int64_t groups = (n + 3) / 4;
+    hipLaunchKernelGGL(quantization_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, vec, n, div_factor,
+                       tensor_max, (uint32_t)seed, (uint32_t)(seed >> 32));
+    return hipGetLastError();
+}
+
+} // namespace dq

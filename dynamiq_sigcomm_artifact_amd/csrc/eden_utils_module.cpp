@@ -1,0 +1,376 @@
+// Python module `eden_utils`: the binding layer of the reference
+// (cuda_kernels/src/srrcomp/eden_utils/eden_utils.cpp:417-433) re-created on
+// top of the C ABI of libdynamiq_eden.so.  Same function names, argument order,
+// keyword names, defaults, dtypes, ownership rules and TORCH_CHECK messages, so
+// testbed_evaluation/new_comm_hooks/utils_aggregation.py, thc_hooks.py and
+// srrcomp.py import it unchanged.  On ROCm builds of PyTorch a HIP device
+// reports itself as torch::kCUDA, which is what the checks below test.
+//
+// Additions (not in the reference): the *_ex variants accept float32 buffers
+// and 3/5/6/7-bit codes, plus rht_blocked, rand_diag, scaling_required_bytes,
+// set_quantization_seed and abi_version.
+#include <torch/extension.h>
+
+#include <atomic>
+
+#include "dynamiq_eden.h"
+
+namespace {
+
+std::atomic<uint64_t> g_quant_seed{0x243F6A8885A308D3ull};
+
+bool is_supported_data_dtype(c10::ScalarType dtype, bool extended)
+{
+    if (dtype == torch::kFloat16 || dtype == torch::kBFloat16) return true;
+    return extended && dtype == torch::kFloat32;
+}
+
+int dq_dtype_of(c10::ScalarType dtype)
+{
+    if (dtype == torch::kFloat16) return DQ_F16;
+    if (dtype == torch::kBFloat16) return DQ_BF16;
+    return DQ_F32;
+}
+
+int64_t superchunk_num_chunks(int n, int superchunk_size)
+{
+    return (static_cast<int64_t>(n) + superchunk_size - 1) / superchunk_size;
+}
+
+// eden_utils.cpp:42-53, same order and wording
+void scaling_check_common(int n, int nbits, int chunk_size, int strategy, bool extended)
+{
+    TORCH_CHECK(n > 0, "n must be positive");
+    if (extended) {
+        TORCH_CHECK(nbits >= 2 && nbits <= 8, "nbits must be in [2, 8]");
+    } else {
+        TORCH_CHECK(nbits == 2 || nbits == 4 || nbits == 8, "nbits must be one of {2, 4, 8}");
+    }
+    TORCH_CHECK(strategy >= 0 && strategy <= 3, "strategy must be 0 (AEE), 1 (MEE), 2 (hierarchical AEE), or 3 (hierarchical MEE)");
+    TORCH_CHECK(chunk_size > 0 && chunk_size <= 32, "chunk_size must be in [1, 32]");
+    TORCH_CHECK((chunk_size & (chunk_size - 1)) == 0, "chunk_size must be a power of two");
+    TORCH_CHECK((chunk_size * nbits) % 8 == 0, "chunk_size * nbits must be divisible by 8");
+    TORCH_CHECK(n % chunk_size == 0, "n must be a multiple of chunk_size");
+    if (strategy >= 2) {
+        TORCH_CHECK((n / chunk_size) % 16 == 0, "hierarchical mode requires n to contain a whole number of 16-chunk superchunks");
+    }
+}
+
+void check_status(int status, const char *what)
+{
+    TORCH_CHECK(status == DQ_OK, what, ": ", dq_last_error());
+}
+
+dq_stream_t as_stream(uint64_t stream_p) { return reinterpret_cast<dq_stream_t>(static_cast<uintptr_t>(stream_p)); }
+
+// ---- Hadamard --------------------------------------------------------------------
+
+torch::Tensor Hadamard(torch::Tensor vec, uint64_t stream_p = 0, int depth = 0)
+{
+    TORCH_CHECK(vec.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(vec.dtype() == torch::kFloat32, "input must be a torch.float32 CUDA tensor");
+    auto n = vec.size(-1);
+    TORCH_CHECK(n == vec.numel(), "input must be 1D");
+    TORCH_CHECK((n & (n - 1)) == 0 && n > 0, "input size must be a power of 2");
+    auto output = vec.clone(); // contiguous copy, as in the reference
+    check_status(dq_hadamard(output.data_ptr<float>(), n, output.device().index(), as_stream(stream_p), depth), "Hadamard");
+    return output;
+}
+
+void Hadamard_inplace(torch::Tensor vec, uint64_t stream_p = 0, int depth = 0)
+{
+    TORCH_CHECK(vec.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(vec.dtype() == torch::kFloat32, "input must be a torch.float32 CUDA tensor");
+    auto n = vec.size(-1);
+    TORCH_CHECK(n == vec.numel(), "input must be 1D");
+    TORCH_CHECK((n & (n - 1)) == 0 && n > 0, "input size must be a power of 2");
+    check_status(dq_hadamard(vec.data_ptr<float>(), n, vec.device().index(), as_stream(stream_p), depth), "Hadamard_inplace");
+}
+
+void Hadamard_inplace_ptr(long long vec, int n, int device, uint64_t stream_p = 0, int depth = 0)
+{
+    check_status(dq_hadamard(reinterpret_cast<float *>(vec), n, device, as_stream(stream_p), depth), "Hadamard_inplace_ptr");
+}
+
+// The reference stores the pointer as curand state storage and launches
+// nothing (cuda_hadamard.cu:674-686).  Randomness here is counter based, so
+// there is no state to place in the caller's buffer: both calls are no-ops.
+void Hadamard_init(torch::Tensor vec) { (void)vec.data_ptr<int>(); }
+void Hadamard_init_ptr(long long vec, int device = 0) { (void)vec; (void)device; }
+
+void quantization_compression(torch::Tensor vec, float div_factor, float tensor_max, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(vec.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(vec.dtype() == torch::kFloat32, "input must be a torch.float32 CUDA tensor");
+    auto n = vec.size(-1);
+    const uint64_t seed = g_quant_seed.fetch_add(0x9E3779B97F4A7C15ull);
+    check_status(dq_quantization(vec.data_ptr<float>(), n, vec.device().index(), div_factor, tensor_max, seed, as_stream(stream_p)),
+                 "quantization_compression");
+}
+
+void set_quantization_seed(uint64_t seed) { g_quant_seed.store(seed); }
+
+torch::Tensor rht_blocked(torch::Tensor vec, c10::optional<torch::Tensor> sign, int64_t block, double scale, bool inverse,
+                          uint64_t stream_p = 0)
+{
+    TORCH_CHECK(vec.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(vec.dtype() == torch::kFloat32, "input must be a torch.float32 CUDA tensor");
+    TORCH_CHECK(vec.is_contiguous(), "input must be contiguous");
+    const float *sp = nullptr;
+    if (sign.has_value()) {
+        TORCH_CHECK(sign->device() == vec.device(), "sign must be on the same device as the input");
+        TORCH_CHECK(sign->dtype() == torch::kFloat32, "sign must be torch.float32");
+        TORCH_CHECK(sign->is_contiguous(), "sign must be contiguous");
+        TORCH_CHECK(sign->numel() >= vec.numel(), "sign has fewer elements than the input");
+        sp = sign->data_ptr<float>();
+    }
+    check_status(dq_rht_blocked(vec.data_ptr<float>(), sp, vec.numel(), block, (float)scale, inverse ? 1 : 0,
+                                vec.device().index(), as_stream(stream_p)),
+                 "rht_blocked");
+    return vec;
+}
+
+torch::Tensor rand_diag(int64_t size, int64_t seed, torch::Device device, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(device.type() == torch::kCUDA, "device must be a CUDA device");
+    auto out = torch::empty({size}, torch::TensorOptions().device(device).dtype(torch::kFloat32));
+    check_status(dq_rand_diag(out.data_ptr<float>(), size, seed, out.device().index(), as_stream(stream_p)), "rand_diag");
+    return out;
+}
+
+// ---- scaling quantisation ---------------------------------------------------------
+
+void scaling_compress_impl(torch::Tensor src, torch::Tensor dst, torch::Tensor rand_pool, int n, int nbits, int chunk_size,
+                           uint64_t stream_p, int strategy, bool ex)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(rand_pool.device().type() == torch::kCUDA, "rand_pool must be a CUDA tensor");
+    TORCH_CHECK(is_supported_data_dtype(src.scalar_type(), ex), "input must be torch.float16 or torch.bfloat16");
+    TORCH_CHECK(dst.dtype() == torch::kUInt8, "output must be torch.uint8");
+    TORCH_CHECK(rand_pool.dtype() == src.dtype(), "rand_pool dtype must match input dtype");
+    TORCH_CHECK(src.is_contiguous(), "input must be contiguous");
+    TORCH_CHECK(dst.is_contiguous(), "output must be contiguous");
+    TORCH_CHECK(rand_pool.is_contiguous(), "rand_pool must be contiguous");
+    scaling_check_common(n, nbits, chunk_size, strategy, ex);
+    TORCH_CHECK(src.numel() >= n, "input has fewer than n elements");
+    TORCH_CHECK(rand_pool.numel() >= n, "rand_pool has fewer than n elements");
+    TORCH_CHECK(dst.numel() >= dq_scaling_required_bytes(n, nbits, chunk_size, strategy), "output buffer is too small");
+    check_status(dq_scaling_compress(src.data_ptr(), dst.data_ptr<uint8_t>(), rand_pool.data_ptr(), n, nbits, chunk_size,
+                                     dq_dtype_of(src.scalar_type()), src.device().index(), strategy, as_stream(stream_p)),
+                 "scaling_compress");
+}
+
+void scaling_decompress_impl(torch::Tensor src, torch::Tensor dst, int n, int nbits, int chunk_size, uint64_t stream_p,
+                             int strategy, bool ex, int add)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(src.dtype() == torch::kUInt8, "input must be torch.uint8");
+    TORCH_CHECK(is_supported_data_dtype(dst.scalar_type(), ex), "output must be torch.float16 or torch.bfloat16");
+    TORCH_CHECK(src.is_contiguous(), "input must be contiguous");
+    TORCH_CHECK(dst.is_contiguous(), "output must be contiguous");
+    scaling_check_common(n, nbits, chunk_size, strategy, ex);
+    TORCH_CHECK(src.numel() >= dq_scaling_required_bytes(n, nbits, chunk_size, strategy), "input buffer is too small");
+    TORCH_CHECK(dst.numel() >= n, "output has fewer than n elements");
+    check_status(dq_scaling_decompress(src.data_ptr<uint8_t>(), dst.data_ptr(), n, nbits, chunk_size,
+                                       dq_dtype_of(dst.scalar_type()), src.device().index(), strategy, as_stream(stream_p), add),
+                 add ? "scaling_decompress_add" : "scaling_decompress");
+}
+
+void scaling_dec_comp_impl(torch::Tensor recv, torch::Tensor inp, torch::Tensor send, torch::Tensor rand_pool, int n, int nbits,
+                           int chunk_size, uint64_t stream_p, int strategy, bool ex)
+{
+    TORCH_CHECK(recv.device().type() == torch::kCUDA, "recv must be a CUDA tensor");
+    TORCH_CHECK(inp.device().type() == torch::kCUDA, "inp must be a CUDA tensor");
+    TORCH_CHECK(send.device().type() == torch::kCUDA, "send must be a CUDA tensor");
+    TORCH_CHECK(rand_pool.device().type() == torch::kCUDA, "rand_pool must be a CUDA tensor");
+    TORCH_CHECK(recv.dtype() == torch::kUInt8, "recv must be torch.uint8");
+    TORCH_CHECK(is_supported_data_dtype(inp.scalar_type(), ex), "inp must be torch.float16 or torch.bfloat16");
+    TORCH_CHECK(send.dtype() == torch::kUInt8, "send must be torch.uint8");
+    TORCH_CHECK(rand_pool.dtype() == inp.dtype(), "rand_pool dtype must match inp dtype");
+    TORCH_CHECK(recv.is_contiguous(), "recv must be contiguous");
+    TORCH_CHECK(inp.is_contiguous(), "inp must be contiguous");
+    TORCH_CHECK(send.is_contiguous(), "send must be contiguous");
+    TORCH_CHECK(rand_pool.is_contiguous(), "rand_pool must be contiguous");
+    scaling_check_common(n, nbits, chunk_size, strategy, ex);
+    const int64_t required_bytes = dq_scaling_required_bytes(n, nbits, chunk_size, strategy);
+    TORCH_CHECK(recv.numel() >= required_bytes, "recv buffer is too small");
+    TORCH_CHECK(send.numel() >= required_bytes, "send buffer is too small");
+    TORCH_CHECK(inp.numel() >= n, "inp has fewer than n elements");
+    TORCH_CHECK(rand_pool.numel() >= n, "rand_pool has fewer than n elements");
+    check_status(dq_scaling_dec_comp(recv.data_ptr<uint8_t>(), inp.data_ptr(), send.data_ptr<uint8_t>(), rand_pool.data_ptr(), n,
+                                     nbits, chunk_size, dq_dtype_of(inp.scalar_type()), recv.device().index(), strategy,
+                                     as_stream(stream_p)),
+                 "scaling_dec_comp");
+}
+
+void scaling_compress(torch::Tensor src, torch::Tensor dst, torch::Tensor rand_pool, int n, int nbits, int chunk_size,
+                      uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_compress_impl(src, dst, rand_pool, n, nbits, chunk_size, stream_p, strategy, false);
+}
+void scaling_compress_ex(torch::Tensor src, torch::Tensor dst, torch::Tensor rand_pool, int n, int nbits, int chunk_size,
+                         uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_compress_impl(src, dst, rand_pool, n, nbits, chunk_size, stream_p, strategy, true);
+}
+void scaling_decompress(torch::Tensor src, torch::Tensor dst, int n, int nbits, int chunk_size, uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_decompress_impl(src, dst, n, nbits, chunk_size, stream_p, strategy, false, 0);
+}
+void scaling_decompress_ex(torch::Tensor src, torch::Tensor dst, int n, int nbits, int chunk_size, uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_decompress_impl(src, dst, n, nbits, chunk_size, stream_p, strategy, true, 0);
+}
+void scaling_decompress_add(torch::Tensor src, torch::Tensor dst, int n, int nbits, int chunk_size, uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_decompress_impl(src, dst, n, nbits, chunk_size, stream_p, strategy, false, 1);
+}
+void scaling_decompress_add_ex(torch::Tensor src, torch::Tensor dst, int n, int nbits, int chunk_size, uint64_t stream_p = 0,
+                               int strategy = 0)
+{
+    scaling_decompress_impl(src, dst, n, nbits, chunk_size, stream_p, strategy, true, 1);
+}
+void scaling_dec_comp(torch::Tensor recv, torch::Tensor inp, torch::Tensor send, torch::Tensor rand_pool, int n, int nbits,
+                      int chunk_size, uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_dec_comp_impl(recv, inp, send, rand_pool, n, nbits, chunk_size, stream_p, strategy, false);
+}
+void scaling_dec_comp_ex(torch::Tensor recv, torch::Tensor inp, torch::Tensor send, torch::Tensor rand_pool, int n, int nbits,
+                         int chunk_size, uint64_t stream_p = 0, int strategy = 0)
+{
+    scaling_dec_comp_impl(recv, inp, send, rand_pool, n, nbits, chunk_size, stream_p, strategy, true);
+}
+
+int64_t scaling_required_bytes(int64_t n, int nbits, int chunk_size, int strategy)
+{
+    return dq_scaling_required_bytes(n, nbits, chunk_size, strategy);
+}
+
+// ---- superchunk ops ---------------------------------------------------------------
+
+void superchunk_mean_center(torch::Tensor src, torch::Tensor residual, torch::Tensor stats, int n, int world_size,
+                            int superchunk_size = 256, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "src must be a CUDA tensor");
+    TORCH_CHECK(residual.device().type() == torch::kCUDA, "residual must be a CUDA tensor");
+    TORCH_CHECK(stats.device().type() == torch::kCUDA, "stats must be a CUDA tensor");
+    TORCH_CHECK(residual.device() == src.device(), "residual must be on the same CUDA device as src");
+    TORCH_CHECK(stats.device() == src.device(), "stats must be on the same CUDA device as src");
+    TORCH_CHECK(is_supported_data_dtype(src.scalar_type(), false), "src must be torch.float16 or torch.bfloat16");
+    TORCH_CHECK(residual.scalar_type() == src.scalar_type(), "residual dtype must match src dtype");
+    TORCH_CHECK(stats.dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+    TORCH_CHECK(src.is_contiguous(), "src must be contiguous");
+    TORCH_CHECK(residual.is_contiguous(), "residual must be contiguous");
+    TORCH_CHECK(stats.is_contiguous(), "stats must be contiguous");
+    TORCH_CHECK(n > 0, "n must be positive");
+    TORCH_CHECK(world_size > 0, "world_size must be positive");
+    TORCH_CHECK(superchunk_size == 256, "superchunk_size must be 256");
+    TORCH_CHECK(src.numel() >= n, "src has fewer than n elements");
+    const int64_t num_superchunks = superchunk_num_chunks(n, superchunk_size);
+    TORCH_CHECK(residual.numel() >= num_superchunks * superchunk_size, "residual buffer is too small");
+    TORCH_CHECK(stats.numel() >= num_superchunks * 2, "stats buffer is too small");
+    check_status(dq_superchunk_mean_center(src.data_ptr(), residual.data_ptr(), stats.data_ptr(), n, world_size, superchunk_size,
+                                           dq_dtype_of(src.scalar_type()), src.device().index(), as_stream(stream_p)),
+                 "superchunk_mean_center");
+}
+
+void superchunk_add_mean_copy(torch::Tensor residual, torch::Tensor dst, torch::Tensor stats, int n, int superchunk_size = 256,
+                              uint64_t stream_p = 0)
+{
+    TORCH_CHECK(residual.device().type() == torch::kCUDA, "residual must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "dst must be a CUDA tensor");
+    TORCH_CHECK(stats.device().type() == torch::kCUDA, "stats must be a CUDA tensor");
+    TORCH_CHECK(dst.device() == residual.device(), "dst must be on the same CUDA device as residual");
+    TORCH_CHECK(stats.device() == residual.device(), "stats must be on the same CUDA device as residual");
+    TORCH_CHECK(is_supported_data_dtype(residual.scalar_type(), false), "residual must be torch.float16 or torch.bfloat16");
+    TORCH_CHECK(dst.scalar_type() == residual.scalar_type(), "dst dtype must match residual dtype");
+    TORCH_CHECK(stats.dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+    TORCH_CHECK(residual.is_contiguous(), "residual must be contiguous");
+    TORCH_CHECK(dst.is_contiguous(), "dst must be contiguous");
+    TORCH_CHECK(stats.is_contiguous(), "stats must be contiguous");
+    TORCH_CHECK(n > 0, "n must be positive");
+    TORCH_CHECK(superchunk_size == 256, "superchunk_size must be 256");
+    TORCH_CHECK(dst.numel() >= n, "dst has fewer than n elements");
+    const int64_t num_superchunks = superchunk_num_chunks(n, superchunk_size);
+    TORCH_CHECK(residual.numel() >= num_superchunks * superchunk_size, "residual buffer is too small");
+    TORCH_CHECK(stats.numel() >= num_superchunks * 2, "stats buffer is too small");
+    check_status(dq_superchunk_add_mean_copy(residual.data_ptr(), dst.data_ptr(), stats.data_ptr(), n, superchunk_size,
+                                             dq_dtype_of(residual.scalar_type()), residual.device().index(), as_stream(stream_p)),
+                 "superchunk_add_mean_copy");
+}
+
+// ---- EDEN bit-plane packing (default stream, fresh outputs, as the reference) -------
+
+torch::Tensor EdenBinsToBits(torch::Tensor bins, int nbits)
+{
+    TORCH_CHECK(bins.device().type() == torch::kCUDA, "bins must be a CUDA tensor");
+    TORCH_CHECK(bins.dtype() == torch::kInt32, "bins must be a torch.int32 CUDA tensor");
+    auto nbins = bins.size(-1);
+    TORCH_CHECK(nbins == bins.numel(), "bins must be 1D");
+    TORCH_CHECK((nbins & 31) == 0, "bins size must be a multiple of 32");
+    auto cbins = bins.clone();
+    const int device = cbins.device().index();
+    auto opts = torch::TensorOptions().device(bins.device().type(), device).dtype(torch::kInt32);
+    torch::Tensor carr = torch::zeros({(nbins >> 5) * nbits}, opts);
+    if (nbins > 0)
+        check_status(dq_bins_to_bits(cbins.data_ptr<int32_t>(), nbins, reinterpret_cast<uint32_t *>(carr.data_ptr<int32_t>()),
+                                     (nbins >> 5) * nbits, nbits, device, nullptr),
+                     "EdenBinsToBits");
+    return carr;
+}
+
+torch::Tensor EdenBitsToBins(torch::Tensor arr, int nbits)
+{
+    TORCH_CHECK(arr.device().type() == torch::kCUDA, "arr must be a CUDA tensor");
+    TORCH_CHECK(arr.dtype() == torch::kInt32, "arr must be a torch.int32 CUDA tensor");
+    auto narr = arr.size(-1);
+    TORCH_CHECK(narr == arr.numel(), "arr must be 1D");
+    auto carr = arr.clone();
+    const int device = carr.device().index();
+    auto opts = torch::TensorOptions().device(arr.device().type(), device).dtype(torch::kInt32);
+    const int64_t nbins = (narr / nbits) << 5;
+    torch::Tensor cbins = torch::zeros({nbins}, opts);
+    if (nbins > 0)
+        check_status(dq_bits_to_bins(cbins.data_ptr<int32_t>(), nbins, reinterpret_cast<const uint32_t *>(carr.data_ptr<int32_t>()),
+                                     (nbins >> 5) * nbits, nbits, device, nullptr),
+                     "EdenBitsToBins");
+    return cbins;
+}
+
+void init_lookup_table() { check_status(dq_init_lookup_table(), "init_lookup_table"); }
+
+std::string abi_version() { return dq_version(); }
+
+} // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
+{
+    modul.def("Hadamard", &Hadamard, "fast Hadamard transform", py::arg("vec"), py::arg("stream_p") = 0, py::arg("depth") = 0);
+    modul.def("EdenBinsToBits", &EdenBinsToBits, "EDEN's packing bins to bits");
+    modul.def("EdenBitsToBins", &EdenBitsToBins, "EDEN's unpacking bits to bins");
+    modul.def("Hadamard_init", &Hadamard_init, "hadamard init", py::arg("vec"));
+    modul.def("Hadamard_init_ptr", &Hadamard_init_ptr, "hadamard init", py::arg("vec"), py::arg("device") = 0);
+    modul.def("Hadamard_inplace", &Hadamard_inplace, "fast Hadamard transform", py::arg("vec"), py::arg("stream_p") = 0, py::arg("depth") = 0);
+    modul.def("Hadamard_inplace_ptr", &Hadamard_inplace_ptr, "fast Hadamard transform", py::arg("vec"), py::arg("n"), py::arg("device"), py::arg("stream_p") = 0, py::arg("depth") = 0);
+    modul.def("quantization_compression", &quantization_compression, "quantization compression", py::arg("vec"), py::arg("div_factor"), py::arg("tensor_max"), py::arg("stream_p") = 0);
+    modul.def("scaling_compress", &scaling_compress, "scaling compress", py::arg("src"), py::arg("dst"), py::arg("rand_pool"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_decompress", &scaling_decompress, "scaling decompress", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_decompress_add", &scaling_decompress_add, "scaling decompress and add", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_dec_comp", &scaling_dec_comp, "scaling decompress and compress", py::arg("recv"), py::arg("inp"), py::arg("send"), py::arg("rand_pool"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("superchunk_mean_center", &superchunk_mean_center, "mean-center 256-element superchunks and write per-superchunk mean/norm stats", py::arg("src"), py::arg("residual"), py::arg("stats"), py::arg("n"), py::arg("world_size"), py::arg("superchunk_size") = 256, py::arg("stream_p") = 0);
+    modul.def("superchunk_add_mean_copy", &superchunk_add_mean_copy, "add reduced per-superchunk means to residuals and copy back valid elements", py::arg("residual"), py::arg("dst"), py::arg("stats"), py::arg("n"), py::arg("superchunk_size") = 256, py::arg("stream_p") = 0);
+    modul.def("init_lookup_table", &init_lookup_table, "init lookup table");
+
+    // additions
+    modul.def("scaling_compress_ex", &scaling_compress_ex, "scaling compress (also float32 buffers, 2..8-bit codes)", py::arg("src"), py::arg("dst"), py::arg("rand_pool"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_decompress_ex", &scaling_decompress_ex, "scaling decompress (also float32 buffers, 2..8-bit codes)", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_decompress_add_ex", &scaling_decompress_add_ex, "scaling decompress and add (also float32 buffers, 2..8-bit codes)", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_dec_comp_ex", &scaling_dec_comp_ex, "scaling decompress and compress (also float32 buffers, 2..8-bit codes)", py::arg("recv"), py::arg("inp"), py::arg("send"), py::arg("rand_pool"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_required_bytes", &scaling_required_bytes, "packed size in bytes", py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("strategy"));
+    modul.def("rht_blocked", &rht_blocked, "in-place blocked randomized Hadamard transform", py::arg("vec"), py::arg("sign"), py::arg("block"), py::arg("scale"), py::arg("inverse") = false, py::arg("stream_p") = 0);
+    modul.def("rand_diag", &rand_diag, "EDEN's seeded +-1 diagonal", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
+    modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
+    modul.def("abi_version", &abi_version, "version string of libdynamiq_eden.so");
+}

@@ -1,0 +1,167 @@
+/*
+ * C ABI of libdynamiq_eden.so -- the MI355X (gfx950) implementation of the
+ * on-GPU gradient-compression path behind DynamiQ's `eden_utils` module.
+ *
+ * Every entry point takes plain device pointers, sizes, a HIP device index and
+ * a HIP stream handle (hipStream_t passed as void*; NULL = the null stream).
+ * All work is enqueued asynchronously on that stream; nothing synchronises,
+ * nothing allocates device memory, no state is kept between calls, and the
+ * functions are re-entrant (they may be called concurrently from several host
+ * threads on distinct streams with sub-buffer pointers at record-aligned
+ * offsets, as ring_allreduce_backend.cu:1262-1289 does).
+ *
+ * Return value: DQ_OK (0) or a dq_status code.  Argument errors carry the same
+ * message text as the TORCH_CHECKs of the reference binding
+ * (eden_utils.cpp:42-53); dq_last_error() returns the text for the calling
+ * thread.  Unlike the reference (which only prints launch failures,
+ * cuda_hadamard.cu:1496-1499) a failed launch is reported as DQ_ERR_LAUNCH.
+ *
+ * "reference" paths below are relative to
+ * cuda_kernels/src/srrcomp/eden_utils/ of the DynamiQ artifact.
+ */
+#ifndef DYNAMIQ_EDEN_H
+#define DYNAMIQ_EDEN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *dq_stream_t; /* hipStream_t */
+
+/* element type of gradient / random buffers */
+enum dq_dtype {
+    DQ_F16 = 0,  /* reference __half path: every intermediate in binary16   */
+    DQ_BF16 = 1, /* reference __nv_bfloat16 path: fp32 math, bf16 storage   */
+    DQ_F32 = 2   /* extension: the bf16 path's math on fp32 storage         */
+};
+/* OR-ed into the dtype argument of dq_scaling_compress / dq_scaling_dec_comp:
+ * rand_pool holds bfloat16 values although the gradient elements are DQ_F32
+ * (the reference's pools are bf16, utils_aggregation.py:384-389; this saves
+ * 2 bytes per element of HBM traffic for fp32 gradients). */
+#define DQ_RAND_BF16 0x10
+
+enum dq_status {
+    DQ_OK = 0,
+    DQ_ERR_N = 1,
+    DQ_ERR_NBITS = 2,
+    DQ_ERR_STRATEGY = 3,
+    DQ_ERR_CHUNK_RANGE = 4,
+    DQ_ERR_CHUNK_POW2 = 5,
+    DQ_ERR_CHUNK_BITS = 6,
+    DQ_ERR_N_CHUNK = 7,
+    DQ_ERR_N_SUPER = 8,
+    DQ_ERR_DTYPE = 9,
+    DQ_ERR_NULL = 10,
+    DQ_ERR_SUPERCHUNK_SIZE = 11,
+    DQ_ERR_WORLD_SIZE = 12,
+    DQ_ERR_POW2 = 13,
+    DQ_ERR_SIZE = 14,
+    DQ_ERR_DEVICE = 15,
+    DQ_ERR_LAUNCH = 16
+};
+
+const char *dq_status_string(int status);
+const char *dq_last_error(void);
+/* library build identification: "dynamiq_eden <version> gfx950" */
+const char *dq_version(void);
+
+/* ---- sizes and validation -------------------------------------------- */
+
+/* eden_utils.cpp:33-40 (scaling_required_bytes) */
+int64_t dq_scaling_required_bytes(int64_t n, int nbits, int chunk_size, int strategy);
+/* eden_utils.cpp:42-53 (scaling_check_common).  nbits in {2,4,8} when
+ * strict != 0; strict == 0 also admits the 3/5/6/7-bit extension codes. */
+int dq_scaling_check_common(int64_t n, int nbits, int chunk_size, int strategy, int strict);
+
+/* ---- MEE lookup table ------------------------------------------------- */
+
+/* csrc/cuda_hadamard.cu:935-939 (init_lookup_table).  The table is built on
+ * the host once per process and travels to the kernels as launch arguments,
+ * so this call is optional and never touches the device. */
+int dq_init_lookup_table(void);
+/* csrc/cuda_hadamard.cu:873-899: copies the 256 binary16 table entries and the
+ * four binary16 parameters {1+2e^2, (1+e^2)/(2e^2), chunk_max_mee,
+ * log2(1+2e^2)} for nbits in 1..8. */
+int dq_mee_lookup_table(int nbits, uint16_t table[256], uint16_t params[4]);
+
+/* ---- scaling quantisation -------------------------------------------- */
+
+/* csrc/cuda_hadamard.h:18,20 (scaling_compress_with_cuda, both overloads).
+ * src, rand_pool: `dtype` elements [>= n]; dst: packed records
+ * [>= dq_scaling_required_bytes].  strategy 0 AEE, 1 MEE, 2/3 hierarchical. */
+int dq_scaling_compress(const void *src, uint8_t *dst, const void *rand_pool, int64_t n,
+                        int nbits, int chunk_size, int dtype, int device, int strategy,
+                        dq_stream_t stream);
+
+/* csrc/cuda_hadamard.h:19,21 (scaling_decompress_with_cuda).  add_original
+ * != 0 accumulates into dst (scaling_decompress_add). */
+int dq_scaling_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int chunk_size,
+                          int dtype, int device, int strategy, dq_stream_t stream,
+                          int add_original);
+
+/* csrc/cuda_hadamard.h:22 (scaling_dec_comp_with_cuda) plus the fp16 split of
+ * eden_utils.cpp:212-214.  send = compress(round(inp + decode(recv))).  With
+ * bf16/f32, chunk_size 16 and strategy 2/3 this is one fused kernel and inp is
+ * left untouched; every other combination decodes INTO inp first, exactly like
+ * the reference dispatch (csrc/cuda_hadamard.cu:1744-1747). */
+int dq_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const void *rand_pool,
+                        int64_t n, int nbits, int chunk_size, int dtype, int device,
+                        int strategy, dq_stream_t stream);
+
+/* ---- superchunk mean-centring ---------------------------------------- */
+
+/* csrc/cuda_hadamard.h:23-24 (superchunk_mean_center_with_cuda).  residual
+ * [>= 256*ceil(n/256)] (padded tail zero-filled), stats bf16
+ * [>= 2*ceil(n/256)] interleaved (mean, sum of squares).  dtype F16 or BF16
+ * (F32 accepted as an extension). */
+int dq_superchunk_mean_center(const void *src, void *residual, void *stats, int64_t n,
+                              int world_size, int superchunk_size, int dtype, int device,
+                              dq_stream_t stream);
+/* csrc/cuda_hadamard.h:25-26 (superchunk_add_mean_copy_with_cuda) */
+int dq_superchunk_add_mean_copy(const void *residual, void *dst, const void *stats, int64_t n,
+                                int superchunk_size, int dtype, int device, dq_stream_t stream);
+
+/* ---- Walsh-Hadamard --------------------------------------------------- */
+
+/* csrc/cuda_hadamard.h:14 (HadamardWithCuda): in-place unnormalised FWHT of
+ * n = 2^k floats; depth is accepted and ignored as in the reference. */
+int dq_hadamard(float *vec, int64_t n, int device, dq_stream_t stream, int depth);
+/* Extension (no reference entry point; fuses thc_hooks.py:95-107 /
+ * srrcomp.py:317-319): per block of `block` = 2^k floats, in place,
+ *   forward: y = FWHT(sign .* x) * scale,   inverse: y = sign .* (FWHT(x) * scale).
+ * sign may be NULL (all +1).  n must be a multiple of block. */
+int dq_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale,
+                   int inverse, int device, dq_stream_t stream);
+/* srrcomp.py:61-106 (SRRCompUtils.randDiag, torchRNG=False) computed on the
+ * device: out[size] of +-1.0f. */
+int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t stream);
+
+/* ---- EDEN bit-plane packing ------------------------------------------ */
+
+/* csrc/cuda_packing.h:10 (BinsToBits).  arr[p*(nbins/32) + w] bit t = bit p of
+ * bins[32*w + t]; nbins % 32 == 0; narr == nbins/32*nbits.  Unlike the
+ * reference launch (cuda_packing.cu:58-65) every bin is processed, also when
+ * nbins is not a multiple of 1024, and the caller's stream is honoured. */
+int dq_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int64_t narr, int nbits,
+                    int device, dq_stream_t stream);
+/* csrc/cuda_packing.h:11 (BitsToBins) */
+int dq_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int64_t narr, int nbits,
+                    int device, dq_stream_t stream);
+
+/* ---- THC-style stochastic rounding ------------------------------------ */
+
+/* csrc/cuda_hadamard.h:16 (quantization_with_cuda): in place
+ *   t = clamp(v / div_factor, +-tensor_max); v = floor(t) + (u < t - floor(t)).
+ * The reference draws u from curand states it never initialises
+ * (cuda_hadamard.cu:669-686); here u is a counter-based Philox4x32-10 uniform
+ * keyed by (seed, element index). */
+int dq_quantization(float *vec, int64_t n, int device, float div_factor, float tensor_max,
+                    uint64_t seed, dq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,213 @@
+"""GPU parity of the scaling-quantisation entry points against the CPU oracle.
+
+Everything here calls the HIP kernels through the C ABI (ctypes) or through the
+`eden_utils` binding that sits on top of it, and compares packed bytes / decoded
+bit patterns with the oracle: bit-exact, no tolerance.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, F16, F32, TORCH_DT, bits_to_f32, from_bits, make_input, make_rand, to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _cmp_bits(name, got, want):
+    got = np.asarray(got)
+    want = np.asarray(want)
+    assert got.shape == want.shape, name
+    if got.dtype == np.float32:
+        # bit patterns, except that any NaN matches any NaN
+        nan = np.isnan(got) & np.isnan(want)
+        got = np.where(nan, 0, got.view(np.uint32))
+        want = np.where(nan, 0, want.view(np.uint32))
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, "%s: %d mismatches, first at %d: got %r want %r" % (
+        name, bad.size, bad[0], got[bad[0]], want[bad[0]])
+
+
+def _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src_t, rand_t, tag):
+    nbytes = oracle.required_bytes(n, nbits, C, strategy)
+    assert capi.required_bytes(n, nbits, C, strategy) == nbytes
+    src_d, rand_d = src_t.to(DEV), rand_t.to(DEV)
+    enc_d = torch.full((nbytes + 7,), 0xAB, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(src_d, enc_d, rand_d, n, nbits, C, strategy)
+    torch.cuda.synchronize()
+    enc_o = oracle.scaling_compress(to_bits(src_t), to_bits(rand_t), n, nbits, C, strategy, dt)
+    enc_g = enc_d.cpu().numpy()
+    _cmp_bits(tag + " compress", enc_g[:nbytes], enc_o)
+    assert (enc_g[nbytes:] == 0xAB).all(), tag + " wrote past the packed stream"
+
+    # decompress (overwrite)
+    dec_d = torch.zeros(n, dtype=TORCH_DT[dt], device=DEV)
+    capi.scaling_decompress(enc_d, dec_d, n, nbits, C, strategy)
+    dec_o = np.zeros(n, np.float32 if dt == F32 else np.uint16)
+    oracle.scaling_decompress(enc_o, dec_o, n, nbits, C, strategy, dt)
+    _cmp_bits(tag + " decompress", to_bits(dec_d), dec_o)
+
+    # decompress_add
+    base_t = (src_t.float() * 0.125).to(TORCH_DT[dt])
+    add_d = base_t.to(DEV)
+    capi.scaling_decompress(enc_d, add_d, n, nbits, C, strategy, add=True)
+    add_o = to_bits(base_t)
+    oracle.scaling_decompress(enc_o, add_o, n, nbits, C, strategy, dt, add=True)
+    _cmp_bits(tag + " decompress_add", to_bits(add_d), add_o)
+    return enc_o
+
+
+def _dec_comp(capi, oracle, dt, n, nbits, C, strategy, recv_src_t, inp_t, rand_recv_t, rand_send_t, tag):
+    nbytes = oracle.required_bytes(n, nbits, C, strategy)
+    recv_o = oracle.scaling_compress(to_bits(recv_src_t), to_bits(rand_recv_t), n, nbits, C, strategy, dt)
+    recv_d = torch.from_numpy(recv_o).to(DEV)
+    inp_d = inp_t.to(DEV)
+    send_d = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    capi.scaling_dec_comp(recv_d, inp_d, send_d, rand_send_t.to(DEV), n, nbits, C, strategy)
+    torch.cuda.synchronize()
+    inp_o = to_bits(inp_t)
+    send_o = oracle.scaling_dec_comp(recv_o, inp_o, to_bits(rand_send_t), n, nbits, C, strategy, dt)
+    _cmp_bits(tag + " dec_comp send", send_d.cpu().numpy(), send_o)
+    # inp: untouched by the fused path, holds the sum on the split path -- same as the oracle
+    _cmp_bits(tag + " dec_comp inp", to_bits(inp_d), inp_o)
+
+    # the reference's own invariant: fused bytes == decompress_add + compress bytes
+    inp2_d = inp_t.to(DEV)
+    capi.scaling_decompress(recv_d, inp2_d, n, nbits, C, strategy, add=True)
+    send2_d = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(inp2_d, send2_d, rand_send_t.to(DEV), n, nbits, C, strategy)
+    assert torch.equal(send_d, send2_d), tag + " fused != split"
+
+
+@pytest.mark.parametrize("dt", [F16, BF16])
+@pytest.mark.parametrize("C", [16, 32])
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+def test_functional_sweep(capi, oracle, dt, C, nbits, strategy):
+    """The 48-case sweep of the reference's functional test, bit-exact."""
+    tdt = TORCH_DT[dt]
+    n = C * (32 if strategy >= 2 else 19)
+    src = make_input(n, tdt)
+    rnd = make_rand(n, 1000 + nbits * 31 + C * 7 + strategy, tdt)
+    tag = "dt=%d C=%d b=%d s=%d" % (dt, C, nbits, strategy)
+    _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src, rnd, tag)
+    recv_src = (make_input(n, tdt).float() * 0.5).to(tdt)
+    inp = (make_input(n, tdt).float() * -0.25).to(tdt)
+    _dec_comp(capi, oracle, dt, n, nbits, C, strategy, recv_src, inp,
+              make_rand(n, 2000 + nbits * 17 + C + strategy, tdt),
+              make_rand(n, 3000 + nbits * 19 + C + strategy, tdt), tag)
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_production_shape_random(capi, oracle, dt, nbits, strategy):
+    """chunk 16 / superchunk 16 on random gradients, ragged superchunk counts."""
+    tdt = TORCH_DT[dt]
+    g = torch.Generator().manual_seed(77 + nbits * 5 + strategy)
+    for nsc in (1, 3, 4, 5, 16, 67, 1030):
+        n = nsc * 256
+        scale = torch.exp(torch.randn(nsc, 1, generator=g) * 3.0 - 7.0)
+        src = (torch.randn(nsc, 256, generator=g) * scale).reshape(-1).to(tdt)
+        rnd = torch.rand(n, generator=g).to(tdt)
+        tag = "dt=%d b=%d s=%d nsc=%d" % (dt, nbits, strategy, nsc)
+        _roundtrip(capi, oracle, dt, n, nbits, 16, strategy, src, rnd, tag)
+        inp = (torch.randn(n, generator=g) * 2e-3).to(tdt)
+        _dec_comp(capi, oracle, dt, n, nbits, 16, strategy, src, inp, rnd, torch.rand(n, generator=g).to(tdt), tag)
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_special_values(capi, oracle, dt, strategy):
+    """zeros, denormals, huge values, inf/nan inputs, rand exactly 0 and 1."""
+    tdt = TORCH_DT[dt]
+    n = 256 * 8
+    g = torch.Generator().manual_seed(5)
+    src = torch.randn(n, generator=g) * 1e-3
+    src[0:256] = 0.0
+    src[256:512] *= 1e-38
+    src[512:768] *= 1e35
+    src[768] = float("inf")
+    src[800] = float("-inf")
+    src[1030] = float("nan")
+    src[1280:1536] = 3.0e38
+    src[1536:1552] = 0.0
+    src[1792:2048] = torch.randn(256, generator=g) * 1e-3
+    src[1800] = 1e30
+    src = src.to(tdt)
+    rnd = torch.rand(n, generator=g)
+    rnd[::7] = 0.0
+    rnd[3::11] = 1.0
+    rnd = rnd.to(tdt)
+    for nbits in (2, 4, 8):
+        _roundtrip_nan_safe = _roundtrip  # codes and scale bytes never hold NaN: exact compare is valid
+        _roundtrip_nan_safe(capi, oracle, dt, n, nbits, 16, strategy, src, rnd, "special b=%d" % nbits)
+
+
+def test_fp32_gradient_with_bf16_rand_pool(capi, oracle):
+    """fp32 elements + bf16 random pool (DQ_RAND_BF16) == fp32 elements + the same values widened"""
+    g = torch.Generator().manual_seed(21)
+    n = 256 * 37
+    src = torch.randn(n, generator=g) * 1e-3
+    rnd16 = torch.rand(n, generator=g).to(torch.bfloat16)
+    inp = torch.randn(n, generator=g) * 1e-3
+    for nbits, strategy in ((4, 2), (8, 2), (4, 3), (5, 2)):
+        nbytes = oracle.required_bytes(n, nbits, 16, strategy)
+        enc_d = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+        capi.scaling_compress(src.to(DEV), enc_d, rnd16.to(DEV), n, nbits, 16, strategy)
+        enc_o = oracle.scaling_compress(to_bits(src), to_bits(rnd16.float()), n, nbits, 16, strategy, F32)
+        _cmp_bits("mixed compress", enc_d.cpu().numpy(), enc_o)
+        send_d = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+        capi.scaling_dec_comp(enc_d, inp.to(DEV), send_d, rnd16.to(DEV), n, nbits, 16, strategy)
+        send_o = oracle.scaling_dec_comp(enc_o, to_bits(inp), to_bits(rnd16.float()), n, nbits, 16, strategy, F32)
+        _cmp_bits("mixed dec_comp", send_d.cpu().numpy(), send_o)
+
+
+def test_unaligned_buffers(capi, oracle):
+    """views with storage offsets: element pointers off the 16-byte grid, packed
+    pointers at record-aligned (odd) offsets"""
+    n = 256 * 9
+    g = torch.Generator().manual_seed(9)
+    for nbits, strategy in ((4, 2), (8, 3), (2, 2)):
+        nbytes = oracle.required_bytes(n, nbits, 16, strategy)
+        rec = nbytes // 9
+        src_t = (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16)
+        rnd_t = torch.rand(n, generator=g).to(torch.bfloat16)
+        big_src = torch.zeros(n + 64, dtype=torch.bfloat16, device=DEV)
+        big_rnd = torch.zeros(n + 64, dtype=torch.bfloat16, device=DEV)
+        big_src[3:3 + n] = src_t.to(DEV)
+        big_rnd[16:16 + n] = rnd_t.to(DEV)
+        enc_o = oracle.scaling_compress(to_bits(src_t), to_bits(rnd_t), n, nbits, 16, strategy, BF16)
+        for off in (rec, 2 * rec + 0, 5 * rec):
+            buf = torch.zeros(nbytes + 6 * rec, dtype=torch.uint8, device=DEV)
+            capi.scaling_compress(big_src[3:3 + n], buf[off:], big_rnd[16:16 + n], n, nbits, 16, strategy)
+            got = buf.cpu().numpy()
+            assert (got[:off] == 0).all() and (got[off + nbytes:] == 0).all()
+            assert (got[off:off + nbytes] == enc_o).all()
+            out = torch.zeros(n + 8, dtype=torch.bfloat16, device=DEV)
+            capi.scaling_decompress(buf[off:], out[5:5 + n], n, nbits, 16, strategy)
+            dec_o = np.zeros(n, np.uint16)
+            oracle.scaling_decompress(enc_o, dec_o, n, nbits, 16, strategy, BF16)
+            assert (to_bits(out[5:5 + n]) == dec_o).all()
+            assert float(out[:5].abs().sum()) == 0.0 and float(out[5 + n:].abs().sum()) == 0.0
+
+
+def test_eden_utils_binding(eden_utils, oracle):
+    """same calls as the reference's test, through the pybind module"""
+    n, nbits, C, strategy = 16 * 32, 4, 16, 2
+    src = make_input(n, torch.bfloat16, DEV)
+    rnd = make_rand(n, 1234, torch.bfloat16, DEV)
+    enc = torch.zeros(oracle.required_bytes(n, nbits, C, strategy), dtype=torch.uint8, device=DEV)
+    dec = torch.empty_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+    eden_utils.scaling_compress(src, enc, rnd, n, nbits, C, stream, strategy)
+    eden_utils.scaling_decompress(enc, dec, n, nbits, C, stream, strategy)
+    torch.cuda.synchronize()
+    enc_o = oracle.scaling_compress(to_bits(src), to_bits(rnd), n, nbits, C, strategy, BF16)
+    assert (enc.cpu().numpy() == enc_o).all()
+    with pytest.raises(RuntimeError, match="nbits must be one of"):
+        eden_utils.scaling_compress(src, enc, rnd, n, 5, C, stream, strategy)
+    with pytest.raises(RuntimeError, match="input must be torch.float16 or torch.bfloat16"):
+        eden_utils.scaling_compress(src.float(), enc, rnd.float(), n, nbits, C, stream, strategy)
+    with pytest.raises(RuntimeError, match="output buffer is too small"):
+        eden_utils.scaling_compress(src, enc[:-1], rnd, n, nbits, C, stream, strategy)
