@@ -46,3 +46,30 @@ def make_rand(n, seed, dtype, device="cpu"):
     g = torch.Generator(device="cpu")
     g.manual_seed(seed)
     return torch.rand(n, generator=g, dtype=torch.float32).to(dtype).to(device)
+
+
+def unpack_stream(enc, n, nbits, C, strategy):
+    """Parse a packed stream by the documented layout
+    (cuda_kernels/documentation/scaling_quantization_algorithm.md:183-196,347-388).
+    Returns codes[n], and for hierarchical streams (q[nchunks] uint8, unit[nsc] uint16),
+    for flat streams (scale[nchunks] uint16, None)."""
+    enc = np.asarray(enc, np.uint8)
+    PB = C * nbits // 8
+    nch = n // C
+    if strategy >= 2:
+        CB = PB + 1
+        REC = 16 * CB + 2
+        nsc = nch // 16
+        rec = enc[:nsc * REC].reshape(nsc, REC)
+        chunks = rec[:, :16 * CB].reshape(nsc, 16, CB)
+        code_bytes = np.ascontiguousarray(chunks[:, :, :PB]).reshape(-1)
+        q = np.ascontiguousarray(chunks[:, :, PB]).reshape(-1)
+        unit = np.ascontiguousarray(rec[:, 16 * CB:]).view(np.uint16).reshape(-1)
+        aux = (q, unit)
+    else:
+        rec = enc[:nch * (PB + 2)].reshape(nch, PB + 2)
+        code_bytes = np.ascontiguousarray(rec[:, :PB]).reshape(-1)
+        aux = (np.ascontiguousarray(rec[:, PB:]).view(np.uint16).reshape(-1), None)
+    bits = np.unpackbits(code_bytes, bitorder="little").reshape(-1, nbits)
+    codes = (bits.astype(np.int64) << np.arange(nbits)).sum(axis=1)
+    return codes, aux

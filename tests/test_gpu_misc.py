@@ -1,0 +1,176 @@
+"""GPU parity of the superchunk, Hadamard, randDiag, bit-plane packing and
+rounding entry points against the CPU oracle (bit-exact unless stated)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, F16, F32, TORCH_DT, from_bits, to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _eq(name, got, want):
+    got, want = np.asarray(got), np.asarray(want)
+    if got.dtype == np.float32:
+        nan = np.isnan(got) & np.isnan(want)
+        got = np.where(nan, 0, got.view(np.uint32))
+        want = np.where(nan, 0, want.view(np.uint32))
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, "%s: %d mismatches, first at %d (%r vs %r)" % (name, bad.size, bad[0], got[bad[0]], want[bad[0]])
+
+
+@pytest.mark.parametrize("dt", [F16, BF16, F32])
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 1000, 256 * 33, 256 * 1000 + 17])
+@pytest.mark.parametrize("world", [1, 8, 3])
+def test_superchunk_mean_center_and_back(capi, oracle, dt, n, world):
+    tdt = TORCH_DT[dt]
+    g = torch.Generator().manual_seed(n * 7 + world)
+    src = (torch.randn(n, generator=g) * 1e-2 + 3e-3).to(tdt)
+    nsc = (n + 255) // 256
+    res_d = torch.full((nsc * 256,), 7.0, dtype=tdt, device=DEV)
+    stats_d = torch.zeros(nsc * 2, dtype=torch.bfloat16, device=DEV)
+    capi.superchunk_mean_center(src.to(DEV), res_d, stats_d, n, world)
+    res_o, stats_o = oracle.superchunk_mean_center(to_bits(src), n, world, dt)
+    _eq("residual", to_bits(res_d), res_o)
+    _eq("stats", to_bits(stats_d), stats_o)
+    out_d = torch.full((n + 3,), 5.0, dtype=tdt, device=DEV)
+    capi.superchunk_add_mean_copy(res_d, out_d, stats_d, n)
+    out_o = oracle.superchunk_add_mean_copy(res_o, stats_o, n, dt)
+    _eq("add_mean", to_bits(out_d[:n]), out_o)
+    assert (out_d[n:] == 5.0).all()
+
+
+def test_superchunk_constant_block(capi):
+    """closed form: a constant block has residual 0 and stats (c/W, 256*(c/W)^2)"""
+    c, W = 0.5, 4
+    src = torch.full((512,), c, dtype=torch.bfloat16, device=DEV)
+    res = torch.ones(512, dtype=torch.bfloat16, device=DEV)
+    stats = torch.zeros(4, dtype=torch.bfloat16, device=DEV)
+    capi.superchunk_mean_center(src, res, stats, 512, W)
+    assert float(res.abs().max()) == 0.0
+    assert stats.float().tolist() == [c / W, 256 * (c / W) ** 2] * 2
+
+
+@pytest.mark.parametrize("k", [0, 1, 2, 3, 5, 8, 10, 12, 13, 14, 15, 16, 18, 20, 22])
+def test_hadamard_whole_vector(capi, oracle, k):
+    n = 1 << k
+    g = torch.Generator().manual_seed(k)
+    x = torch.randn(n, generator=g)
+    x_d = x.to(DEV)
+    capi.hadamard(x_d)
+    _eq("fwht 2^%d" % k, x_d.cpu().numpy(), oracle.fwht(x.numpy()))
+
+
+def test_hadamard_identities(capi):
+    """H(e_i) = i-th Walsh row (+-1), H(1) = n e_0, H(H(x)) = n x on small integers"""
+    n = 1 << 14
+    e = torch.zeros(n, device=DEV)
+    e[12345] = 1.0
+    capi.hadamard(e)
+    idx = torch.arange(n, device=DEV)
+    par = torch.zeros(n, dtype=torch.int64, device=DEV)
+    v = idx & 12345
+    for b in range(14):
+        par ^= (v >> b) & 1
+    assert torch.equal(e, 1.0 - 2.0 * par.float())
+    ones = torch.ones(n, device=DEV)
+    capi.hadamard(ones)
+    assert float(ones[0]) == n and float(ones[1:].abs().max()) == 0.0
+    x = torch.randint(-8, 9, (n,), device=DEV).float()
+    y = x.clone()
+    capi.hadamard(y)
+    capi.hadamard(y)
+    assert torch.equal(y, x * n)
+
+
+def test_hadamard_module_functions(eden_utils, oracle):
+    n = 1 << 11
+    x = torch.randn(n, device=DEV)
+    ref = oracle.fwht(x.cpu().numpy())
+    y = eden_utils.Hadamard(x, torch.cuda.current_stream().cuda_stream)
+    assert y.data_ptr() != x.data_ptr()
+    _eq("Hadamard", y.cpu().numpy(), ref)
+    z = x.clone()
+    eden_utils.Hadamard_inplace(z)
+    _eq("Hadamard_inplace", z.cpu().numpy(), ref)
+    w = x.clone()
+    eden_utils.Hadamard_inplace_ptr(w.data_ptr(), n, 0)
+    torch.cuda.synchronize()
+    _eq("Hadamard_inplace_ptr", w.cpu().numpy(), ref)
+    with pytest.raises(RuntimeError, match="power of 2"):
+        eden_utils.Hadamard(torch.zeros(12, device=DEV))
+    with pytest.raises(RuntimeError, match="torch.float32"):
+        eden_utils.Hadamard(torch.zeros(16, device=DEV, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("kb", [4, 10, 11, 12, 13, 14, 15, 17])
+@pytest.mark.parametrize("inverse", [False, True])
+def test_rht_blocked(capi, oracle, kb, inverse):
+    block = 1 << kb
+    nblocks = 3 if kb <= 15 else 2
+    n = block * nblocks
+    g = torch.Generator().manual_seed(kb)
+    x = torch.randn(n, generator=g) * 1e-3
+    sign = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    scale = 1.0 / math.sqrt(block)
+    x_d = x.to(DEV)
+    capi.rht_blocked(x_d, sign.to(DEV), block, scale, inverse)
+    ref = oracle.rht_blocked(x.numpy(), sign.numpy(), block, np.float32(scale), inverse)
+    _eq("rht", x_d.cpu().numpy(), ref)
+
+
+def test_rht_roundtrip_is_identity(capi):
+    """inverse(forward(x)) == x up to fp32 rounding (orthonormal transform)"""
+    block, n = 1 << 12, 1 << 20
+    x = torch.randn(n, device=DEV) * 1e-3
+    sign = (torch.randint(0, 2, (n,), device=DEV) * 2 - 1).float()
+    y = x.clone()
+    s = 1.0 / math.sqrt(block)
+    capi.rht_blocked(y, sign, block, s, False)
+    # energy is preserved
+    assert abs(float(y.double().pow(2).sum() / x.double().pow(2).sum()) - 1.0) < 1e-5
+    capi.rht_blocked(y, sign, block, s, True)
+    assert float((y - x).abs().max()) <= 1e-5 * float(x.abs().max())
+
+
+@pytest.mark.parametrize("size", [8, 64, 100, 4096, 1000003])
+@pytest.mark.parametrize("seed", [0, 1, 42, 2 ** 31])
+def test_rand_diag(capi, oracle, size, seed):
+    out = torch.zeros(size, device=DEV)
+    capi.rand_diag(out, seed)
+    _eq("rand_diag", out.cpu().numpy(), oracle.rand_diag(size, seed))
+
+
+@pytest.mark.parametrize("nbits", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("nbins", [32, 64, 96, 1024, 1056, 100000 * 32])
+def test_bit_plane_packing(capi, oracle, eden_utils, nbits, nbins):
+    g = torch.Generator().manual_seed(nbits * 100 + nbins % 97)
+    bins = torch.randint(0, 1 << nbits, (nbins,), generator=g, dtype=torch.int32)
+    arr_o = oracle.bins_to_bits(bins.numpy(), nbits)
+    arr_d = eden_utils.EdenBinsToBits(bins.to(DEV), nbits)
+    assert arr_d.dtype == torch.int32 and arr_d.numel() == nbins // 32 * nbits
+    _eq("bins_to_bits", arr_d.cpu().numpy().view(np.uint32), arr_o)
+    back = eden_utils.EdenBitsToBins(arr_d, nbits)
+    assert torch.equal(back.cpu(), bins)
+
+
+def test_quantization_compression(eden_utils):
+    """values land on floor/ceil of t = clamp(v/div, +-max), unbiased in the mean"""
+    n = 1 << 20
+    v = (torch.rand(n, device=DEV) * 12.0 - 6.0)
+    t = (v / 0.5).clamp(-10.0, 10.0)
+    eden_utils.set_quantization_seed(123)
+    q = v.clone()
+    eden_utils.quantization_compression(q, 0.5, 10.0)
+    assert bool(((q == t.floor()) | (q == t.floor() + 1)).all())
+    assert abs(float((q - t).mean())) < 5e-3
+    eden_utils.set_quantization_seed(123)
+    q2 = v.clone()
+    eden_utils.quantization_compression(q2, 0.5, 10.0)
+    assert torch.equal(q, q2)
+    q3 = v.clone()
+    eden_utils.quantization_compression(q3, 0.5, 10.0)
+    assert not torch.equal(q, q3)

@@ -1,0 +1,217 @@
+"""Pins of the remaining oracle functions (no GPU): number formats, log2, the
+superchunk statistics, Walsh-Hadamard, randDiag / bit-plane packing golden
+vectors written from the reference's own torch code, the bit-width rule."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, F16, F32, TORCH_DT, bits_to_f32, to_bits
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "srrcomp_golden.npz")
+
+
+# ---- number formats ------------------------------------------------------------------------
+
+def test_conversions_match_numpy_and_torch(oracle):
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(50000) * np.exp(rng.uniform(-45, 45, 50000))).astype(np.float32)
+    x[:8] = [0.0, -0.0, np.inf, -np.inf, 65519.99, 65520.0, 5.96e-8, 2.98e-8]
+    with np.errstate(over="ignore"):
+        assert (oracle.f32_to_f16(x) == x.astype(np.float16).view(np.uint16)).all()
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert (oracle.f32_to_bf16(x) == want).all()
+    xs = rng.uniform(-7e-5, 7e-5, 50000).astype(np.float32)          # half subnormals
+    assert (oracle.f32_to_f16(xs) == xs.astype(np.float16).view(np.uint16)).all()
+    allh = np.arange(65536, dtype=np.uint16)
+    L = oracle.lib()
+    got = np.array([L.dqo_f16_to_f32(int(h)) for h in allh[::7]], np.float32)
+    want = allh[::7].view(np.float16).astype(np.float32)
+    assert ((got == want) | (np.isnan(got) & np.isnan(want))).all()
+    # ties to even
+    assert oracle.f32_to_bf16(np.array([1.00390625, 1.01171875], np.float32)).tolist() == [0x3F80, 0x3F82]
+
+
+def test_log2_accuracy_and_special_values(oracle):
+    rng = np.random.default_rng(1)
+    a = np.concatenate([np.exp(rng.uniform(-87, 88, 40000)), 1 + rng.uniform(0, 1e-3, 5000),
+                        rng.uniform(0.5, 2.0, 20000), 2.0 ** np.arange(-126, 127)]).astype(np.float32)
+    got = oracle.log2f(a).astype(np.float64)
+    ref = np.log2(a.astype(np.float64))
+    ulp = np.spacing(np.abs(ref).astype(np.float32)).astype(np.float64)
+    assert (np.abs(got - ref) <= 1.75 * ulp).all()
+    exact = oracle.log2f(np.array([1.0, 2.0, 0.5, 1024.0, 2.0 ** -130], np.float32))
+    assert exact.tolist() == [0.0, 1.0, -1.0, 10.0, -130.0]
+    sp = oracle.log2f(np.array([0.0, np.inf, -1.0, np.nan], np.float32))
+    assert sp[0] == -np.inf and sp[1] == np.inf and np.isnan(sp[2]) and np.isnan(sp[3])
+
+
+# ---- superchunk statistics -------------------------------------------------------------------
+
+@pytest.mark.parametrize("dt", [F16, BF16, F32])
+def test_mean_center_closed_forms(oracle, dt):
+    tdt = TORCH_DT[dt]
+    # constant block: residual 0, stats (c/W, 256 (c/W)^2)
+    src = to_bits(torch.full((512,), 0.5).to(tdt))
+    res, stats = oracle.superchunk_mean_center(src, 512, 4, dt)
+    assert (bits_to_f32(res, dt) == 0).all()
+    assert bits_to_f32(stats, BF16).tolist() == [0.125, 4.0, 0.125, 4.0]
+    # ragged tail: mean over the valid elements only, padded residual is zero
+    n = 256 + 10
+    x = torch.arange(n, dtype=torch.float32).remainder(5).to(tdt)
+    res, stats = oracle.superchunk_mean_center(to_bits(x), n, 1, dt)
+    st = bits_to_f32(stats, BF16)
+    tail = x[256:].float().numpy()
+    assert st[2] == bits_to_f32(to_bits(torch.tensor([tail.mean()]).to(torch.bfloat16)), BF16)[0]
+    assert st[3] == float((tail ** 2).sum())             # un-centred sum of squares
+    assert (bits_to_f32(res, dt)[n:] == 0).all() and res.size == 512
+    # tree order (stride 128 -> 1) == numpy pairwise halving in float32
+    g = torch.Generator().manual_seed(2)
+    y = (torch.randn(256, generator=g) * 3).to(tdt)
+    v = (bits_to_f32(to_bits(y), dt) / np.float32(3.0)).astype(np.float32)
+    s, q = v.copy(), (v * v).astype(np.float32)
+    while s.size > 1:
+        h = s.size // 2
+        s = (s[:h] + s[h:]).astype(np.float32)
+        q = (q[:h] + q[h:]).astype(np.float32)
+    res, stats = oracle.superchunk_mean_center(to_bits(y), 256, 3, dt)
+    mean = np.float32(s[0] / np.float32(256))
+    assert stats[0] == to_bits(torch.tensor([mean]).to(torch.bfloat16))[0]
+    assert stats[1] == to_bits(torch.tensor([q[0]]).to(torch.bfloat16))[0]
+    want_res = to_bits(torch.from_numpy((v - mean).astype(np.float32)).to(tdt))
+    assert (res == want_res).all()
+
+
+def test_add_mean_restores_input(oracle):
+    g = torch.Generator().manual_seed(4)
+    n, W = 256 * 5 + 77, 8
+    x = (torch.randn(n, generator=g) * 1e-2 + 0.02).to(torch.bfloat16)
+    res, stats = oracle.superchunk_mean_center(to_bits(x), n, W, BF16)
+    back = bits_to_f32(oracle.superchunk_add_mean_copy(res, stats, n, BF16), BF16)
+    want = x.float().numpy() / W
+    assert np.abs(back - want).max() <= 2 ** -7 * np.abs(want).max()
+
+
+# ---- Walsh-Hadamard -------------------------------------------------------------------------------
+
+def _sylvester(n):
+    h = np.array([[1.0]])
+    while h.shape[0] < n:
+        h = np.block([[h, h], [h, -h]])
+    return h
+
+
+@pytest.mark.parametrize("n", [1, 2, 4, 16, 64, 256])
+def test_fwht_equals_sylvester_matrix(oracle, n):
+    rng = np.random.default_rng(n)
+    x = rng.integers(-50, 50, n).astype(np.float32)          # integers: every sum is exact
+    assert (oracle.fwht(x) == (_sylvester(n) @ x.astype(np.float64)).astype(np.float32)).all()
+
+
+def test_fwht_identities(oracle):
+    n = 1 << 12
+    rng = np.random.default_rng(0)
+    x = rng.integers(-8, 9, n).astype(np.float32)
+    assert (oracle.fwht(oracle.fwht(x)) == n * x).all()
+    ones = oracle.fwht(np.ones(n, np.float32))
+    assert ones[0] == n and (ones[1:] == 0).all()
+    e = np.zeros(n, np.float32)
+    e[1234] = 1
+    row = oracle.fwht(e)
+    par = np.array([bin(i & 1234).count("1") & 1 for i in range(n)])
+    assert (row == 1 - 2 * par).all()
+    y = rng.standard_normal(n).astype(np.float32)
+    ref = _sylvester(256) @ y[:256].astype(np.float64)
+    assert np.abs(oracle.fwht(y[:256]) - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
+def test_fwht_against_reference_torch_butterfly():
+    import oracle as O
+    gold = np.load(GOLDEN)
+    for k in (3, 6, 10):
+        got = O.fwht(gold["had_in_%d" % k])
+        ref = gold["had_out_%d" % k]
+        assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
+def test_rht_blocked_is_diag_fwht_scale(oracle):
+    rng = np.random.default_rng(5)
+    n, B = 4096, 1024
+    x = rng.standard_normal(n).astype(np.float32)
+    s = rng.choice([-1.0, 1.0], n).astype(np.float32)
+    sc = np.float32(1 / math.sqrt(B))
+    fwd = oracle.rht_blocked(x, s, B, sc)
+    for b in range(n // B):
+        blk = slice(b * B, (b + 1) * B)
+        assert (fwd[blk] == (oracle.fwht(x[blk] * s[blk]) * sc).astype(np.float32)).all()
+    back = oracle.rht_blocked(fwd, s, B, sc, inverse=True)
+    assert np.abs(back - x).max() <= 1e-5 * np.abs(x).max()
+
+
+# ---- golden vectors from the reference's torch code -----------------------------------------------------
+
+def test_rand_diag_golden(oracle):
+    gold = np.load(GOLDEN)
+    for size, seed in gold["randdiag_cases"]:
+        size, seed = int(size), int(seed)
+        want = np.unpackbits(gold["randdiag_%d_%d" % (size, seed)])[:size]
+        got = (oracle.rand_diag(size, seed) > 0).astype(np.uint8)
+        assert (got == want).all(), (size, seed)
+    # roughly balanced signs
+    s = oracle.rand_diag(1 << 16, 7)
+    assert set(np.unique(s)) == {-1.0, 1.0} and abs(s.mean()) < 0.02
+
+
+def test_bit_plane_packing_golden_and_roundtrip(oracle):
+    gold = np.load(GOLDEN)
+    for nbits in range(1, 9):
+        for nbins in (64, 256):
+            bins = gold["pack_bins_%d_%d" % (nbits, nbins)]
+            bits = gold["pack_bits_%d_%d" % (nbits, nbins)]
+            assert (oracle.bins_to_bits(bins, nbits).view(np.int32) == bits).all()
+            assert (oracle.bits_to_bins(bits.view(np.uint32).copy(), nbits) == bins).all()
+    rng = np.random.default_rng(3)
+    for nbits in range(1, 9):
+        bins = rng.integers(0, 1 << nbits, 32 * 37).astype(np.int32)
+        arr = oracle.bins_to_bits(bins, nbits)
+        # closed form: word w of plane p, bit t = bit p of bins[32 w + t]
+        w, t, p = 11, 5, nbits - 1
+        assert (arr[p * 37 + w] >> t) & 1 == (bins[32 * w + t] >> p) & 1
+        assert (oracle.bits_to_bins(arr, nbits) == bins).all()
+
+
+# ---- dynamic bit-width rule ------------------------------------------------------------------------------
+
+def _torch_qbits(norms, u):
+    """testbed_evaluation/new_comm_hooks/comm_hooks.py:64-70, torch ops on the tensor as given"""
+    eps = 1e-20
+    log_norms = torch.log2(torch.clamp(norms, min=eps))
+    score = log_norms.mul(4.0 / (512.0 / 17.0)).add(float(u))
+    z = torch.floor(torch.log2(torch.clamp(score, min=eps))).to(torch.int64)
+    z.clamp_(1, 3)
+    return torch.bitwise_left_shift(torch.ones_like(z), z)
+
+
+def test_dynamic_bitrate_rule(oracle):
+    g = torch.Generator().manual_seed(6)
+    norms = torch.exp(torch.randn(20000, generator=g) * 6 - 8).to(torch.bfloat16)
+    nb = to_bits(norms)
+    assert (oracle.dynamic_bitrate_qbits(nb, 60.0) == 8).all()          # score >= 51 -> z clamps to 3
+    assert (oracle.dynamic_bitrate_qbits(nb, -10.0) == 2).all()         # score < 0 -> eps -> z = 1
+    prev = None
+    for u in np.linspace(-10, 60, 71):
+        q = oracle.dynamic_bitrate_qbits(nb, float(u))
+        assert set(np.unique(q)) <= {2, 4, 8}
+        if prev is not None:
+            assert (q >= prev).all()                                   # monotone in u
+        prev = q
+        tq = _torch_qbits(norms, float(u)).numpy()
+        assert (q != tq).mean() < 1e-3                                  # log2 ulps at bf16 ties only
+    # norm 1 -> log2 = 0 -> score = bf16(u): 2 bits below 4, 4 bits in [4, 8), 8 bits from 8 on;
+    # bf16(7.97) = 7.96875 has log2 = 2.9943, which ROUNDS to 3.0 in bf16 and therefore already gets 8 bits
+    one = to_bits(torch.tensor([1.0]).to(torch.bfloat16))
+    us = (3.98, 4.0, 7.9, 7.97, 8.0)
+    assert [int(oracle.dynamic_bitrate_qbits(one, u)[0]) for u in us] == [2, 4, 4, 8, 8]
+    assert [int(_torch_qbits(torch.tensor([1.0]).to(torch.bfloat16), u)[0]) for u in us] == [2, 4, 4, 8, 8]

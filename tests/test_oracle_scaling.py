@@ -1,0 +1,285 @@
+"""Pins of the CPU oracle's scaling quantiser (no GPU): closed-form layouts and
+special cases, statistical identities, and an independently written numpy model."""
+import numpy as np
+import pytest
+import torch
+
+import ref_model
+from helpers import BF16, F16, F32, TORCH_DT, bits_to_f32, make_input, make_rand, to_bits, unpack_stream
+
+bf16_of = lambda x: to_bits(torch.as_tensor(np.asarray(x, np.float32)).to(torch.bfloat16))
+
+
+# ---- sizes and validation ------------------------------------------------------------
+
+def test_record_sizes_closed_form(oracle):
+    # 256-element superchunk records: 82 / 146 / 274 bytes (eden_utils.cpp:33-40)
+    assert [oracle.required_bytes(256, b, 16, 2) for b in (2, 4, 8)] == [82, 146, 274]
+    # 25 MB bucket (6,553,600 elements)
+    assert [oracle.required_bytes(6553600, b, 16, 2) for b in (2, 4, 8)] == [2099200, 3737600, 7014400]
+    # flat: chunk*nbits/8 + 2 bytes per chunk
+    assert oracle.required_bytes(16 * 19, 4, 16, 0) == 19 * 10
+    assert oracle.required_bytes(32 * 19, 2, 32, 1) == 19 * 10
+    # compressed_numel of the caller (utils_aggregation.py:403-407)
+    for n in (256, 1000, 15555072):
+        padded = (n + 255) // 256 * 256
+        assert oracle.required_bytes(padded, 4, 16, 3) == padded // 256 * (16 * 9 + 2)
+
+
+@pytest.mark.parametrize("args,code", [
+    ((0, 4, 16, 0), 1), ((256, 3, 16, 0), 2), ((256, 4, 16, 4), 3), ((256, 4, 64, 0), 4),
+    ((256, 4, 12, 0), 5), ((256, 2, 2, 0), 6), ((250, 4, 16, 0), 7), ((16 * 17, 4, 16, 2), 8),
+    ((256, 4, 16, 2), 0), ((16 * 19, 8, 16, 1), 0),
+])
+def test_check_common(oracle, args, code):
+    assert oracle.scaling_check(*args, strict=True) == code
+
+
+# ---- special cases with known answers ---------------------------------------------------
+
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+def test_all_zero_superchunk(oracle, nbits):
+    n, R = 256, (1 << (nbits - 1)) - 1
+    src = np.zeros(n, np.uint16)
+    rnd = bf16_of(np.linspace(0, 0.99, n))
+    enc = oracle.scaling_compress(src, rnd, n, nbits, 16, 2, BF16)
+    codes, (q, unit) = unpack_stream(enc, n, nbits, 16, 2)
+    assert (codes == R).all()                      # ceil(0 - r) = 0 for r < 1
+    assert (q == 255).all()                        # all chunk scales equal the maximum
+    want_unit = bf16_of([np.float32(np.float32(0.0) / np.float32(R) + np.float32(1e-7)) / np.float32(255.0)])
+    assert unit[0] == want_unit[0]
+    # r == 1.0 exactly (bf16-rounded torch.rand can produce it): floor - 1
+    rnd1 = bf16_of(np.ones(n))
+    codes1, _ = unpack_stream(oracle.scaling_compress(src, rnd1, n, nbits, 16, 2, BF16), n, nbits, 16, 2)
+    assert (codes1 == max(R - 1, 0)).all()
+    # flat layout stores bf16(1e-7) as the scale
+    encf = oracle.scaling_compress(src, rnd, n, nbits, 16, 0, BF16)
+    _, (scale, _) = unpack_stream(encf, n, nbits, 16, 0)
+    assert (scale == bf16_of([1e-7])[0]).all()
+
+
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("strategy", [0, 2])
+def test_single_extreme_element(oracle, nbits, strategy):
+    """one +-max element in an otherwise zero superchunk -> code 2R / 0 there, R elsewhere"""
+    n, R = 256, (1 << (nbits - 1)) - 1
+    for pos, sign in ((0, 1.0), (37, -1.0), (255, 1.0)):
+        v = np.zeros(n, np.float32)
+        v[pos] = sign * 0.5
+        enc = oracle.scaling_compress(bf16_of(v), bf16_of(np.full(n, 0.5)), n, nbits, 16, strategy, BF16)
+        codes, _ = unpack_stream(enc, n, nbits, 16, strategy)
+        want = np.full(n, R)
+        # |x| = 0.5/scale is just below R (scale carries +1e-7 and is rounded up); rand 0.5 decides
+        want[pos] = codes[pos]
+        assert (codes == want).all()
+        assert codes[pos] in ((2 * R, 2 * R - 1) if sign > 0 else (0, 1))
+        dec = np.zeros(n, np.uint16)
+        oracle.scaling_decompress(enc, dec, n, nbits, 16, strategy, BF16)
+        d = bits_to_f32(dec, BF16)
+        assert (np.delete(d, pos) == 0).all() and abs(d[pos] - v[pos]) <= 0.5 / max(R, 1) * 1.02
+
+
+def test_rounding_direction_at_rand_extremes(oracle):
+    """rand = 0 rounds up unless x is an integer; rand = 1 floors (and gives x-1 on integers)"""
+    nbits, R, n = 8, 127, 256
+    # chunk maximum 127 * 2^-10 -> scale slightly above 2^-10; use values k * 2^-10 + small offsets
+    base = np.zeros(n, np.float32)
+    base[0] = 127.0 / 1024.0
+    base[1:16] = (np.arange(1, 16) + 0.25) / 1024.0      # fractional
+    enc0 = oracle.scaling_compress(bf16_of(base), bf16_of(np.zeros(n)), n, nbits, 16, 0, BF16)
+    enc1 = oracle.scaling_compress(bf16_of(base), bf16_of(np.ones(n)), n, nbits, 16, 0, BF16)
+    c0, (scale, _) = unpack_stream(enc0, n, nbits, 16, 0)
+    c1, _ = unpack_stream(enc1, n, nbits, 16, 0)
+    s = bits_to_f32(scale[:1], BF16)[0]
+    x = bits_to_f32(bf16_of(base[:16]), BF16) / s
+    assert (c0[:16] - R == np.ceil(x)).all()             # rand 0: up
+    assert (c1[:16] - R == np.where(x == np.floor(x), x - 1, np.floor(x))).all()   # rand 1: down
+    # exact zeros: rand 0 keeps 0, rand 1 gives -1
+    assert (c0[16:] == R).all() and (c1[16:] == R - 1).all()
+
+
+@pytest.mark.parametrize("strategy", [0, 2])
+@pytest.mark.parametrize("nbits", [4, 8])
+def test_stochastic_rounding_is_unbiased(oracle, strategy, nbits):
+    """E_r[decode(encode(x, r))] = x, and the error variance is scale^2 * frac * (1 - frac)"""
+    n, reps = 256, 2000
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16)
+    xs = to_bits(x)
+    acc = np.zeros(n, np.float64)
+    dec = np.zeros(n, np.float32)
+    xf = bits_to_f32(xs, BF16).astype(np.float32)
+    for _ in range(reps):
+        r = torch.rand(n, generator=g)
+        enc = oracle.scaling_compress(xf, r.numpy().copy(), n, nbits, 16, strategy, F32)
+        oracle.scaling_decompress(enc, dec, n, nbits, 16, strategy, F32)
+        acc += dec
+    step = np.abs(xf).reshape(-1, 16).max(axis=1).repeat(16) / ((1 << (nbits - 1)) - 1)
+    err = acc / reps - xf
+    assert np.abs(err).max() < 5.0 * step.max() * 0.5 / np.sqrt(reps)
+
+
+def test_nmse_band_gaussian(oracle):
+    """NMSE ~ E[scale^2]/(6 E[x^2]) with scale ~ absmax16/R: ~1.5e-2 (4-bit), ~4.7e-5 (8-bit)"""
+    n = 256 * 256
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(n, generator=g) * 1e-3).numpy().copy()
+    r = torch.rand(n, generator=g).numpy().copy()
+    out = np.zeros(n, np.float32)
+    for nbits, lo, hi in ((4, 1.3e-2, 1.8e-2), (8, 4.0e-5, 5.6e-5)):
+        enc = oracle.scaling_compress(x, r, n, nbits, 16, 2, F32)
+        oracle.scaling_decompress(enc, out, n, nbits, 16, 2, F32)
+        nmse = float(((out - x) ** 2).sum() / (x ** 2).sum())
+        assert lo < nmse < hi, nmse
+
+
+# ---- MEE table and lattice ----------------------------------------------------------------
+
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+def test_mee_table_closed_form(oracle, nbits):
+    table, params = oracle.mee_lut(nbits)
+    want, c, cmm, l2b = ref_model.mee_table(nbits)
+    assert (table[: 1 << nbits].view(np.float16) == want).all()
+    assert (table[1 << nbits:] == 0).all()
+    assert table[(1 << nbits) - 1] == 0                       # top code unused
+    assert params[1:].view(np.float16).tolist() == [c, cmm, l2b]
+    anchor = (1 << (nbits - 1)) - 1
+    t = table[: 2 * anchor + 1].view(np.float16).astype(np.float64)
+    assert (np.diff(t) > 0).all() and t[anchor] == 0 and np.allclose(t, -t[::-1])
+    # closed form in double: ((1+2e^2)^j - 1)/(2e^2) * (1+e^2)
+    e = ref_model.EPS[nbits]
+    j = np.arange(0, anchor + 1)
+    exact = ((1 + 2 * e * e) ** j - 1) / (2 * e * e) * (1 + e * e)
+    assert np.allclose(t[anchor:], exact, rtol=2e-3, atol=1e-6)
+
+
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("strategy", [1, 3])
+def test_mee_lattice_points_are_fixed_points(oracle, nbits, strategy):
+    """x = table[c] * s encodes to c for any rand in (0,1) and decodes to itself"""
+    table, _ = oracle.mee_lut(nbits)
+    R = (1 << (nbits - 1)) - 1
+    levels = table[: 2 * R + 1].view(np.float16).astype(np.float32)
+    n = 256
+    s = np.float32(2.0 ** -9)
+    codes_in = np.resize(np.arange(2 * R + 1), n)
+    codes_in[::16] = 2 * R          # every chunk holds the top level, so the chunk scale is ~s
+    x = levels[codes_in] * s
+    for rv in (0.25, 0.75):
+        enc = oracle.scaling_compress(x.astype(np.float32), np.full(n, rv, np.float32), n, nbits, 16, strategy, F32)
+        codes, _ = unpack_stream(enc, n, nbits, 16, strategy)
+        # the stored scale is s*(1+tiny) rounded (bf16 / 8-bit ratio), so the lattice coordinate
+        # lands within a small fraction below the integer: rand 0.25 rounds it back up
+        if rv == 0.25:
+            assert (np.abs(codes - codes_in) <= 0).mean() > 0.9
+        assert (np.abs(codes - codes_in) <= 1).all()
+
+
+def test_mee_monotone(oracle):
+    """codes are non-decreasing in the input value (fixed rand)"""
+    n = 256
+    x = np.sort(np.random.default_rng(0).normal(0, 1e-3, n)).astype(np.float32)
+    x[-1] = 4e-3
+    for nbits in (2, 4, 8):
+        enc = oracle.scaling_compress(x, np.full(n, 0.5, np.float32), n, nbits, 16, 1, F32)
+        codes, (scale, _) = unpack_stream(enc, n, nbits, 16, 1)
+        lattice = codes.reshape(-1, 16)
+        xs = x.reshape(-1, 16) / bits_to_f32(scale, BF16)[:, None]
+        order = np.argsort(xs.reshape(-1), kind="stable")
+        # within a chunk (same scale) the code is monotone in x
+        for k in range(lattice.shape[0]):
+            assert (np.diff(lattice[k][np.argsort(xs[k], kind="stable")]) >= 0).all()
+
+
+# ---- independent numpy model ------------------------------------------------------------------
+
+@pytest.mark.parametrize("C", [16, 32])
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+def test_bf16_matches_numpy_model(oracle, C, nbits, strategy):
+    n = C * (32 if strategy >= 2 else 19)
+    src = make_input(n, torch.bfloat16)
+    rnd = make_rand(n, 1000 + nbits * 31 + C * 7 + strategy, torch.bfloat16)
+    enc = oracle.scaling_compress(to_bits(src), to_bits(rnd), n, nbits, C, strategy, BF16)
+    codes, _ = unpack_stream(enc, n, nbits, C, strategy)
+    mcodes, mdec = ref_model.model_bf16(src.float().numpy(), rnd.float().numpy(), nbits, C, strategy)
+    dec = np.zeros(n, np.uint16)
+    oracle.scaling_decompress(enc, dec, n, nbits, C, strategy, BF16)
+    d = bits_to_f32(dec, BF16)
+    if strategy in (0, 2):
+        assert (codes == mcodes).all()
+        assert (d == ref_model.bf16_round(mdec)).all()
+    else:
+        # log2 implementations differ by ulps: at most a rare off-by-one code
+        assert (np.abs(codes - mcodes) <= 1).all() and (codes != mcodes).mean() < 0.01
+    # the reference test's own tolerances (:287-290)
+    tol = 4e-2 if strategy in (0, 2) else 8e-2
+    assert (np.abs(d - mdec) <= tol + tol * np.abs(mdec)).all()
+
+
+@pytest.mark.parametrize("C", [16, 32])
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+def test_f16_matches_numpy_model(oracle, C, nbits, strategy):
+    n = C * (32 if strategy >= 2 else 19)
+    src = make_input(n, torch.float16)
+    rnd = make_rand(n, 1000 + nbits * 31 + C * 7 + strategy, torch.float16)
+    enc = oracle.scaling_compress(to_bits(src), to_bits(rnd), n, nbits, C, strategy, F16)
+    codes, _ = unpack_stream(enc, n, nbits, C, strategy)
+    mcodes, mdec = ref_model.model_f16(src.numpy(), rnd.numpy(), nbits, C, strategy)
+    dec = np.zeros(n, np.uint16)
+    oracle.scaling_decompress(enc, dec, n, nbits, C, strategy, F16)
+    d = bits_to_f32(dec, F16)
+    if strategy in (0, 2):
+        assert (codes == mcodes).all()
+        assert (d == mdec).all()
+    else:
+        assert (np.abs(codes - mcodes) <= 1).all() and (codes != mcodes).mean() < 0.02
+    atol, rtol = ((2e-3, 2e-3) if strategy in (0, 2) else (2e-2, 6e-2))
+    same = codes == mcodes
+    assert (np.abs(d - mdec)[same] <= atol + rtol * np.abs(mdec)[same]).all()
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+def test_random_data_matches_numpy_model(oracle, dt):
+    g = torch.Generator().manual_seed(17)
+    n = 256 * 300
+    scale = torch.exp(torch.randn(n // 256, 1, generator=g) * 3 - 7)
+    src = (torch.randn(n // 256, 256, generator=g) * scale).reshape(-1).to(TORCH_DT[dt])
+    rnd = torch.rand(n, generator=g).to(TORCH_DT[dt])
+    for nbits in (2, 3, 4, 5, 6, 7, 8):
+        enc = oracle.scaling_compress(to_bits(src), to_bits(rnd), n, nbits, 16, 2, dt)
+        codes, _ = unpack_stream(enc, n, nbits, 16, 2)
+        mcodes, _ = ref_model.model_bf16(src.float().numpy(), rnd.float().numpy(), nbits, 16, 2)
+        assert (codes == mcodes).all()
+
+
+# ---- invariants of the reference's own test --------------------------------------------------------
+
+@pytest.mark.parametrize("dt", [F16, BF16, F32])
+@pytest.mark.parametrize("C", [16, 32])
+@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+def test_fused_equals_split_and_add_is_rounded_sum(oracle, dt, C, nbits, strategy):
+    tdt = TORCH_DT[dt]
+    n = C * (32 if strategy >= 2 else 19)
+    recv_src = (make_input(n, tdt).float() * 0.5).to(tdt)
+    inp = (make_input(n, tdt).float() * -0.25).to(tdt)
+    r1 = make_rand(n, 2000 + nbits * 17 + C + strategy, tdt)
+    r2 = make_rand(n, 3000 + nbits * 19 + C + strategy, tdt)
+    recv = oracle.scaling_compress(to_bits(recv_src), to_bits(r1), n, nbits, C, strategy, dt)
+    inp_f = to_bits(inp)
+    send = oracle.scaling_dec_comp(recv, inp_f, to_bits(r2), n, nbits, C, strategy, dt)
+    fused = dt != F16 and C == 16 and strategy >= 2
+    inp_s = to_bits(inp)
+    oracle.scaling_decompress(recv, inp_s, n, nbits, C, strategy, dt, add=True)
+    send_s = oracle.scaling_compress(inp_s, to_bits(r2), n, nbits, C, strategy, dt)
+    assert (send == send_s).all()
+    # fused leaves inp alone, split leaves the sum in it (cuda_hadamard.cu:1744-1747)
+    assert (inp_f == (to_bits(inp) if fused else inp_s)).all()
+    # decompress_add == round(base + decoded) within the reference tolerances (:338-349)
+    dec = np.zeros(n, inp_s.dtype)
+    oracle.scaling_decompress(recv, dec, n, nbits, C, strategy, dt)
+    want = (torch.as_tensor(bits_to_f32(to_bits(inp), dt)) + torch.as_tensor(bits_to_f32(dec, dt))).to(tdt).float().numpy()
+    tol = {F16: (2e-3 if strategy in (0, 2) else 6e-2), BF16: (4e-2 if strategy in (0, 2) else 8e-2), F32: 1e-6}[dt]
+    assert (np.abs(bits_to_f32(inp_s, dt) - want) <= tol + tol * np.abs(want)).all()
