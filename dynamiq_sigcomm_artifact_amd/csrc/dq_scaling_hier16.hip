@@ -2,56 +2,90 @@
 // shape: chunk 16, superchunk 16 chunks (256 elements), bf16 or fp32 elements,
 // strategies 2 (AEE) and 3 (MEE), code widths 2..8.
 //
-// Work decomposition (wave64):
+// Work decomposition (wave64, one wave per workgroup, no barriers):
 //   * one lane owns one chunk: 16 consecutive elements = 32 B (bf16) / 64 B
-//     (fp32) of 128-bit loads, so the chunk maximum needs no cross-lane
-//     traffic and every per-chunk scalar is computed once per 16 elements;
+//     (fp32) of 128-bit loads, so the chunk maximum needs no cross-lane traffic
+//     and every per-chunk scalar is computed once per 16 elements;
 //   * one 16-lane DPP row owns one superchunk: the superchunk maximum is four
-//     v_max_f32_dpp steps, no LDS, no barrier;
-//   * one wave owns 4 consecutive superchunks = one contiguous run of 4
-//     records (328..1096 bytes) in the packed stream.  Records are 82/146/274
-//     bytes and never 16-byte aligned, so the run is assembled in a per-wave
-//     LDS window whose offset equals the global address modulo 16 and then
-//     streamed out with aligned 128-bit stores (ragged head / tail bytes are
-//     stored singly).  The receive side of the fused kernel and the decoder
-//     pull their run of records through the same kind of window with aligned
-//     128-bit loads.
-//   Waves never synchronise with each other.
+//     DPP max steps, no LDS;
+//   * one wave owns a tile of 4 consecutive superchunks = one contiguous run of
+//     4 records (328..1096 bytes) of the packed stream.  Records are 82/146/274
+//     bytes and never 16-byte aligned, so a run is assembled in an LDS window
+//     whose offset equals the global address modulo 16 and streamed out with
+//     aligned 128-bit stores (ragged head / tail bytes singly); packed input is
+//     pulled through the same kind of window with aligned 128-bit loads;
+//   * a wave walks tiles blockIdx, blockIdx + gridDim, ... and issues the loads
+//     of its next tile before it computes the current one, so HBM latency hides
+//     behind the VALU work even when the whole grid is resident at once (a
+//     25 MB bucket is only ~1.5 tiles per wave slot of the chip).
+//
+// VALU budget.  The quantiser is VALU-bound if written naively (IEEE division,
+// NaN/Inf/out-of-range guards per element).  Two measures keep it HBM-bound:
+//   * exact division by a chunk-constant: x/d == (float)((double)x * (1/d in
+//     double)).  The product carries a relative error < 2^-51 while a binary32
+//     quotient of binary32 operands is never closer than 2^-49 (relative) to a
+//     rounding boundary without being exactly representable, so the result is
+//     the correctly rounded quotient for every finite x -- three full-rate
+//     instructions per element instead of the ~10-instruction division
+//     expansion;
+//   * a wave-uniform fast path: if every element of the wave is finite and
+//     below 2^100 and every random value lies in [0, 1] (one packed integer
+//     maximum per element finds out), the guards of the general formula cannot
+//     fire and are skipped; otherwise the whole wave takes the guarded path.
+//     Both paths produce the same bytes on the inputs the fast path accepts.
 //
 // Numerics: csrc/cuda_hierarchical_mee.cu:203-343 (compress), 345-505
 // (decompress) and 526-696 (fused decompress-accumulate-recompress).
+#include <stdlib.h>
+
+#include <mutex>
+
 #include "dq_device.cuh"
 #include "dq_launch.h"
 
 namespace dq {
 
-constexpr int kWavesPerBlock = 4;
-constexpr int kRowsPerWave = 4; // superchunks per wave
+constexpr int kRowsPerWave = 4; // superchunks per tile
 
 template <int NBITS> struct Rec {
     static constexpr int R = (1 << (NBITS - 1)) - 1;
-    static constexpr int PB = 2 * NBITS;          // code bytes per chunk
-    static constexpr int CB = PB + 1;             // + one scale byte
-    static constexpr int REC = 16 * CB + 2;       // + bf16 unit
-    static constexpr int WORDS = (PB + 3) / 4;    // dwords holding one chunk's codes
-    // per-wave LDS window: 4 records + up to 15 bytes of misalignment, padded
+    static constexpr int PB = 2 * NBITS;       // code bytes per chunk
+    static constexpr int CB = PB + 1;          // + one scale byte
+    static constexpr int REC = 16 * CB + 2;    // + bf16 unit
+    static constexpr int WORDS = (PB + 3) / 4; // dwords holding one chunk's codes
+    // LDS window: 4 records + up to 15 bytes of misalignment, padded to 16
     static constexpr int WIN = ((kRowsPerWave * REC + 15 + 15) / 16) * 16;
+    static constexpr int WIN_VECS = WIN / 16;  // <= 70: at most two 128-bit registers per lane
 };
 
 template <int NBITS, bool MEE> struct MeeArg {
     float c, cmm, l2b;
-    uint16_t table[MEE ? (1 << NBITS) : 2];
+    uint32_t pad;
+    double inv_c, inv_cmm, inv_l2b; // correctly rounded double reciprocals
+    uint16_t table[MEE ? (1 << NBITS) : 4];
 };
 
-// ---- element vectors -----------------------------------------------------------
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
-template <int DT> struct Vec16;
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
 
-template <> struct Vec16<DQ_BF16> {
-    static __device__ __forceinline__ void load(const void *p, int64_t e, float (&v)[16], bool vec)
+// ---- 16 raw elements of one lane ----------------------------------------------------
+
+template <int DT> struct Raw16;
+
+template <> struct Raw16<DQ_BF16> {
+    uint32_t w[8];
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int k = 0; k < 8; k++) w[k] = 0;
+    }
+    __device__ __forceinline__ void load(const void *p, int64_t e, bool vec)
     {
         const uint16_t *h = static_cast<const uint16_t *>(p) + e;
-        uint32_t w[8];
         if (vec) {
             const uint4 *q = reinterpret_cast<const uint4 *>(h);
             uint4 a = q[0], b = q[1];
@@ -60,17 +94,9 @@ template <> struct Vec16<DQ_BF16> {
 #pragma unroll
             for (int k = 0; k < 8; k++) w[k] = (uint32_t)h[2 * k] | ((uint32_t)h[2 * k + 1] << 16);
         }
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            v[2 * k] = __uint_as_float(w[k] << 16);
-            v[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
-        }
     }
-    static __device__ __forceinline__ void store(void *p, int64_t e, const float (&v)[16], bool vec)
+    __device__ __forceinline__ void store(void *p, int64_t e, bool vec) const
     {
-        uint32_t w[8];
-#pragma unroll
-        for (int k = 0; k < 8; k++) w[k] = f32x2_to_bf16x2(v[2 * k], v[2 * k + 1]);
         uint16_t *h = static_cast<uint16_t *>(p) + e;
         if (vec) {
             uint4 *q = reinterpret_cast<uint4 *>(h);
@@ -81,50 +107,122 @@ template <> struct Vec16<DQ_BF16> {
             for (int k = 0; k < 8; k++) { h[2 * k] = (uint16_t)w[k]; h[2 * k + 1] = (uint16_t)(w[k] >> 16); }
         }
     }
-    static __device__ __forceinline__ float round(float x) { return rb(x); }
+    __device__ __forceinline__ float get(int i) const
+    {
+        return (i & 1) ? __uint_as_float(w[i >> 1] & 0xffff0000u) : __uint_as_float(w[i >> 1] << 16);
+    }
+    __device__ __forceinline__ void set(const float (&t)[16])
+    {
+#pragma unroll
+        for (int k = 0; k < 8; k++) w[k] = f32x2_to_bf16x2(t[2 * k], t[2 * k + 1]);
+    }
+    // binary32 bit pattern of max |element| in integer order (a NaN sorts above infinity)
+    __device__ __forceinline__ uint32_t absmax_bits() const
+    {
+        uint32_t m = w[0] & 0x7fff7fffu;
+#pragma unroll
+        for (int k = 1; k < 8; k++) m = pk_max_u16(m, w[k] & 0x7fff7fffu);
+        return max(m << 16, m & 0xffff0000u);
+    }
+    // every element in [+0, 1]
+    __device__ __forceinline__ bool unit_interval() const
+    {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int k = 1; k < 8; k++) m = pk_max_u16(m, w[k]);
+        return max(m & 0xffffu, m >> 16) <= 0x3f80u;
+    }
+    static constexpr int kSlots = 2; // 16-byte pieces per lane
+    __device__ __forceinline__ uint4 slot(int j) const { return make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]); }
 };
 
-template <> struct Vec16<DQ_F32> {
-    static __device__ __forceinline__ void load(const void *p, int64_t e, float (&v)[16], bool vec)
+template <> struct Raw16<DQ_F32> {
+    uint32_t w[16];
+    __device__ __forceinline__ void zero()
     {
-        const float *f = static_cast<const float *>(p) + e;
+#pragma unroll
+        for (int k = 0; k < 16; k++) w[k] = 0;
+    }
+    __device__ __forceinline__ void load(const void *p, int64_t e, bool vec)
+    {
+        const uint32_t *f = static_cast<const uint32_t *>(p) + e;
         if (vec) {
-            const float4 *q = reinterpret_cast<const float4 *>(f);
+            const uint4 *q = reinterpret_cast<const uint4 *>(f);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                float4 t = q[k];
-                v[4 * k] = t.x; v[4 * k + 1] = t.y; v[4 * k + 2] = t.z; v[4 * k + 3] = t.w;
+                uint4 t = q[k];
+                w[4 * k] = t.x; w[4 * k + 1] = t.y; w[4 * k + 2] = t.z; w[4 * k + 3] = t.w;
             }
         } else {
 #pragma unroll
-            for (int k = 0; k < 16; k++) v[k] = f[k];
+            for (int k = 0; k < 16; k++) w[k] = f[k];
         }
     }
-    static __device__ __forceinline__ void store(void *p, int64_t e, const float (&v)[16], bool vec)
+    __device__ __forceinline__ void store(void *p, int64_t e, bool vec) const
     {
-        float *f = static_cast<float *>(p) + e;
+        uint32_t *f = static_cast<uint32_t *>(p) + e;
         if (vec) {
-            float4 *q = reinterpret_cast<float4 *>(f);
+            uint4 *q = reinterpret_cast<uint4 *>(f);
 #pragma unroll
-            for (int k = 0; k < 4; k++) q[k] = make_float4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+            for (int k = 0; k < 4; k++) q[k] = make_uint4(w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
         } else {
 #pragma unroll
-            for (int k = 0; k < 16; k++) f[k] = v[k];
+            for (int k = 0; k < 16; k++) f[k] = w[k];
         }
     }
-    static __device__ __forceinline__ float round(float x) { return x; }
+    __device__ __forceinline__ float get(int i) const { return __uint_as_float(w[i]); }
+    __device__ __forceinline__ void set(const float (&t)[16])
+    {
+#pragma unroll
+        for (int k = 0; k < 16; k++) w[k] = __float_as_uint(t[k]);
+    }
+    __device__ __forceinline__ uint32_t absmax_bits() const
+    {
+        uint32_t m = w[0] & 0x7fffffffu;
+#pragma unroll
+        for (int k = 1; k < 16; k++) m = max(m, w[k] & 0x7fffffffu);
+        return m;
+    }
+    __device__ __forceinline__ bool unit_interval() const
+    {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int k = 1; k < 16; k++) m = max(m, w[k]);
+        return m <= 0x3f800000u;
+    }
+    static constexpr int kSlots = 4;
+    __device__ __forceinline__ uint4 slot(int j) const { return make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]); }
 };
 
-// ---- record windows --------------------------------------------------------------
+// ---- record windows --------------------------------------------------------------------
 
-// pull `total` bytes starting at g (any alignment) into the window so that
-// byte k of the run sits at win[(g & 15) + k]
-__device__ __forceinline__ int window_fill(uint8_t *win, const uint8_t *g, int total, int lane)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// the (up to two) aligned 128-bit pieces of a packed run this lane moves
+struct WinRegs {
+    u32x4 a, b;
+};
+
+// every lane loads (indices are clamped into the run), so the registers are
+// always defined and the prefetch is two plain vector loads
+__device__ __forceinline__ WinRegs window_fetch(const uint8_t *g, int total, int lane)
 {
     const int mis = (int)(reinterpret_cast<uintptr_t>(g) & 15);
-    const uint4 *ga = reinterpret_cast<const uint4 *>(g - mis);
+    const u32x4 *ga = reinterpret_cast<const u32x4 *>(g - mis);
     const int nvec = (mis + total + 15) >> 4;
-    for (int v = lane; v < nvec; v += 64) reinterpret_cast<uint4 *>(win)[v] = ga[v];
+    WinRegs r;
+    r.a = ga[min(lane, nvec - 1)];
+    r.b = ga[min(lane + 64, nvec - 1)];
+    return r;
+}
+
+// byte k of the run lands at win[(g & 15) + k]
+__device__ __forceinline__ int window_commit(uint8_t *win, const WinRegs &r, const uint8_t *g, int total, int lane)
+{
+    const int mis = (int)(reinterpret_cast<uintptr_t>(g) & 15);
+    const int nvec = (mis + total + 15) >> 4;
+    if (lane < nvec) reinterpret_cast<u32x4 *>(win)[lane] = r.a;
+    if (lane + 64 < nvec) reinterpret_cast<u32x4 *>(win)[lane + 64] = r.b;
     return mis;
 }
 
@@ -143,6 +241,8 @@ __device__ __forceinline__ void window_flush(const uint8_t *win, uint8_t *g, int
     if (tl >= 0 && tl < tail) g[head + body + tl] = win[mis + head + body + tl];
 }
 
+// LDS accesses of one wave execute in order; the fence only stops the compiler
+// from moving them across the hand-over between lanes
 __device__ __forceinline__ void wave_lds_sync()
 {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -150,7 +250,7 @@ __device__ __forceinline__ void wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// ---- per-chunk code words ---------------------------------------------------------
+// ---- per-chunk code words -----------------------------------------------------------------
 
 template <int NBITS> __device__ __forceinline__ void words_put(uint32_t (&w)[Rec<NBITS>::WORDS], int i, uint32_t code)
 {
@@ -167,7 +267,7 @@ template <int NBITS> __device__ __forceinline__ uint32_t words_get(const uint32_
     return v & ((1u << NBITS) - 1u);
 }
 
-// read one chunk's CB bytes (codes + scale byte) from a window
+// one chunk's CB bytes (codes + scale byte) from / to a window
 template <int NBITS>
 __device__ __forceinline__ void chunk_read(const uint8_t *p, uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q)
 {
@@ -186,10 +286,50 @@ __device__ __forceinline__ void chunk_write(uint8_t *p, const uint32_t (&w)[Rec<
     p[Rec<NBITS>::PB] = (uint8_t)q;
 }
 
-// ---- the math of one chunk ---------------------------------------------------------
+// ---- exact division by a chunk constant ------------------------------------------------------
 
-// decode 16 levels of one chunk and accumulate: t = round(lev*sc + acc)
-template <int DT, int NBITS, bool MEE, bool ADD>
+// 1/b in double to within one double ulp, b a normal binary32 in [2^-100, 2^100]
+__device__ __forceinline__ double recip_f64(float b)
+{
+    const double bd = (double)b;
+    double y = (double)__builtin_amdgcn_rcpf(b);
+    double e = __builtin_fma(-bd, y, 1.0);
+    y = __builtin_fma(y, e, y);
+    e = __builtin_fma(-bd, y, 1.0);
+    y = __builtin_fma(y, e, y);
+    return y;
+}
+
+// correctly rounded binary32 quotient a / b given yb ~= 1/b in double
+__device__ __forceinline__ float div_by(float a, double yb) { return (float)((double)a * yb); }
+
+// log2_det() for a finite argument >= 1 (same operations, special cases dropped)
+__device__ __forceinline__ float log2_det_ge1(float x)
+{
+    const uint32_t ix = __float_as_uint(x);
+    const uint32_t t = ix - 0x3f3504f3u;
+    const int k = (int)t >> 23;
+    const float z = __uint_as_float(ix - (t & 0xff800000u));
+    const float f = z - 1.0f;
+    float q = -0x1.d0dd08p-4f;
+    q = __builtin_fmaf(q, f, 0x1.7ad622p-3f);
+    q = __builtin_fmaf(q, f, -0x1.831b24p-3f);
+    q = __builtin_fmaf(q, f, 0x1.a33bdap-3f);
+    q = __builtin_fmaf(q, f, -0x1.eb492p-3f);
+    q = __builtin_fmaf(q, f, 0x1.277e38p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715762p-2f);
+    q = __builtin_fmaf(q, f, 0x1.ec7092p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715476p-1f);
+    const float p = (f * f) * q;
+    float r = __builtin_fmaf(f, 0x1.4ae0cp-26f, p);
+    r = __builtin_fmaf(f, 0x1.715476p+0f, r);
+    return (float)k + r;
+}
+
+// ---- the math of one chunk ---------------------------------------------------------------------
+
+// decode 16 levels of one chunk: t = lev*sc (+ t when ADD)
+template <int NBITS, bool MEE, bool ADD>
 __device__ __forceinline__ void chunk_decode(const uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t q, uint32_t unit_bits,
                                              const float *table, float (&t)[16])
 {
@@ -203,16 +343,16 @@ __device__ __forceinline__ void chunk_decode(const uint32_t (&w)[Rec<NBITS>::WOR
     }
 }
 
-// quantise one chunk held in v[] against the superchunk (row) it belongs to
-template <int NBITS, bool MEE>
-__device__ __forceinline__ void chunk_encode(const float (&v)[16], const float (&r)[16], float c, float cmm, float l2b,
-                                             uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q, uint32_t &unit_bits)
+// general (guarded) quantiser of one chunk against its superchunk row
+template <int NBITS, bool MEE, class RV, class RR, class ARG>
+__device__ __forceinline__ void chunk_encode_guarded(const RV &v, const RR &r, const ARG &mp,
+                                                     uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q, uint32_t &unit_bits)
 {
     constexpr int R = Rec<NBITS>::R;
-    float a = __builtin_fabsf(v[0]);
+    float a = __builtin_fabsf(v.get(0));
 #pragma unroll
-    for (int i = 1; i < 16; i++) a = __builtin_fmaxf(a, __builtin_fabsf(v[i]));
-    const float s = pos_scale(MEE ? a / pos_scale(cmm) + 1e-7f : a / (float)R + 1e-7f);
+    for (int i = 1; i < 16; i++) a = __builtin_fmaxf(a, __builtin_fabsf(v.get(i)));
+    const float s = pos_scale(MEE ? a / pos_scale(mp.cmm) + 1e-7f : a / (float)R + 1e-7f);
     const float g = pos_scale(row16_max(s));
     unit_bits = f32_to_bf16_bits(pos_scale(g / 255.0f));
     const float unit = pos_scale(bf16_bits_to_f32(unit_bits));
@@ -226,134 +366,311 @@ __device__ __forceinline__ void chunk_encode(const float (&v)[16], const float (
     for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        float x = v[i] / d;
-        if (MEE) x = mee_inverse_guarded(x, c, l2b);
-        words_put<NBITS>(w, i, (uint32_t)clamp_code(sr_guarded(x, r[i]), R));
+        float x = v.get(i) / d;
+        if (MEE) x = mee_inverse_guarded(x, mp.c, mp.l2b);
+        words_put<NBITS>(w, i, (uint32_t)clamp_code(sr_guarded(x, r.get(i)), R));
     }
 }
 
-// ---- kernels ------------------------------------------------------------------------
+// the same quantiser for a wave whose elements are all finite and <= 2^100 in
+// magnitude (amax_bits is the integer-order maximum of |v|) and whose random
+// values all lie in [0, 1]: none of the guards can fire
+template <int NBITS, bool MEE, class RV, class RR, class ARG>
+__device__ __forceinline__ void chunk_encode_fast(const RV &v, const RR &r, uint32_t amax_bits, const ARG &mp,
+                                                  uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q, uint32_t &unit_bits)
+{
+    constexpr int R = Rec<NBITS>::R;
+    const float a = __uint_as_float(amax_bits);
+    float s;
+    if (MEE)
+        s = div_by(a, mp.inv_cmm) + 1e-7f;
+    else
+        s = (R == 1 ? a : div_by(a, 1.0 / (double)R)) + 1e-7f; // >= 1e-7, finite
+    const float g = row16_max(s);
+    unit_bits = f32_to_bf16_bits(div_by(g, 1.0 / 255.0));
+    const float unit = bf16_bits_to_f32(unit_bits);
+    const float ratio = div_by(s, recip_f64(g)) * 255.0f;
+    int qi = (int)__builtin_ceilf(ratio);
+    qi = min(max(qi, 1), 255);
+    q = (uint32_t)qi;
+    const float d = (float)qi * unit; // exact: 8 x 8 significant bits
+    const double yd = recip_f64(d);
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float x = div_by(v.get(i), yd);
+        if (MEE) {
+            const float arg = div_by(__builtin_fabsf(x), mp.inv_c) + 1.0f;
+            const float lat = div_by(log2_det_ge1(arg), mp.inv_l2b);
+            x = __builtin_copysignf(lat, x);
+        }
+        const float fl = __builtin_floorf(x);
+        const float c = __builtin_ceilf((x - fl) - r.get(i));
+        const int sv = (int)(fl + c); // |fl| <= R + 1 and c in {-1, 0, 1}: exact
+        words_put<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
+    }
+}
+
+constexpr uint32_t kFastMaxBits = 0x71800000u; // 2^100
+
+// ---- kernels ------------------------------------------------------------------------------------
 
 // compress (FUSED = false) or decode-accumulate-recompress (FUSED = true)
-template <int DT, int RDT, int NBITS, bool MEE, bool FUSED>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void hier16_compress_kernel(
-    const void *__restrict__ src, const uint8_t *__restrict__ recv, uint8_t *__restrict__ dst,
-    const void *__restrict__ rnd, int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
+template <int DT, int RDT, int NBITS, bool MEE, bool FUSED, bool LOOP>
+__global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restrict__ src, const uint8_t *__restrict__ recv,
+                                                            uint8_t *__restrict__ dst, const void *__restrict__ rnd,
+                                                            int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
-    __shared__ __attribute__((aligned(16))) uint8_t win_out[kWavesPerBlock][RC::WIN];
-    __shared__ __attribute__((aligned(16))) uint8_t win_in[FUSED ? kWavesPerBlock : 1][FUSED ? RC::WIN : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t win_out[RC::WIN];
+    __shared__ __attribute__((aligned(16))) uint8_t win_in[FUSED ? RC::WIN : 16];
     __shared__ float table[(MEE && FUSED) ? (1 << NBITS) : 1];
 
+    const int lane = threadIdx.x;
     if (MEE && FUSED) {
-        for (int k = threadIdx.x; k < (1 << NBITS); k += kWavesPerBlock * 64) table[k] = f16_bits_to_f32(mp.table[k]);
-        __syncthreads();
-    }
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int64_t sc0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
-    if (sc0 >= nsc) return;
-    const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-    const int row = lane >> 4, j = lane & 15;
-    const bool active = row < rows;
-    const int64_t e = (sc0 * 16 + lane) * 16;
-    const int total = rows * RC::REC;
-
-    float v[16], r[16];
-    if (active) {
-        Vec16<DT>::load(src, e, v, vec & 1);
-        Vec16<RDT>::load(rnd, e, r, vec & 2);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 16; i++) { v[i] = 0.0f; r[i] = 0.0f; }
-    }
-
-    if (FUSED) {
-        const int mis_in = window_fill(win_in[wave], recv + sc0 * RC::REC, total, lane);
+        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
         wave_lds_sync();
-        if (active) {
-            const uint8_t *rec = win_in[wave] + mis_in + row * RC::REC;
-            uint32_t w[RC::WORDS], q;
-            chunk_read<NBITS>(rec + j * RC::CB, w, q);
-            const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
-            chunk_decode<DT, NBITS, MEE, true>(w, q, ub, table, v);
+    }
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t ntiles = (nsc + kRowsPerWave - 1) / kRowsPerWave;
+    int64_t tile = blockIdx.x;
+    if (tile >= ntiles) return;
+
+    Raw16<DT> v;
+    Raw16<RDT> r;
+    WinRegs wr;
+    wr.a = wr.b = (u32x4)(0u);
+    {
+        const int64_t sc0 = tile * kRowsPerWave;
+        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+        if (row < rows) {
+            v.load(src, (sc0 * 16 + lane) * 16, vec & 1);
+            r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
+        } else {
+            v.zero();
+            r.zero();
+        }
+        if (FUSED) wr = window_fetch(recv + sc0 * RC::REC, rows * RC::REC, lane);
+    }
+
+    for (;;) {
+        const int64_t sc0 = tile * kRowsPerWave;
+        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+        const bool active = row < rows;
+        const int total = rows * RC::REC;
+
+        // issue the next tile's loads before touching the current one
+        const int64_t next = tile + gridDim.x;
+        const bool has_next = LOOP && next < ntiles;
+        Raw16<DT> vn;
+        Raw16<RDT> rn;
+        WinRegs wn = wr;
+        if (has_next) {
+            const int64_t nsc0 = next * kRowsPerWave;
+            const int nrows = (int)min((int64_t)kRowsPerWave, nsc - nsc0);
+            if (row < nrows) {
+                vn.load(src, (nsc0 * 16 + lane) * 16, vec & 1);
+                rn.load(rnd, (nsc0 * 16 + lane) * 16, vec & 2);
+            } else {
+                vn.zero();
+                rn.zero();
+            }
+            if (FUSED) wn = window_fetch(recv + nsc0 * RC::REC, nrows * RC::REC, lane);
+        }
+
+        if (FUSED) {
+            const int mis_in = window_commit(win_in, wr, recv + sc0 * RC::REC, total, lane);
+            wave_lds_sync();
+            if (active) {
+                const uint8_t *rec = win_in + mis_in + row * RC::REC;
+                uint32_t cw[RC::WORDS], cq;
+                chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+                const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+                float t[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) v[i] = Vec16<DT>::round(v[i]);
+                for (int i = 0; i < 16; i++) t[i] = v.get(i);
+                chunk_decode<NBITS, MEE, true>(cw, cq, ub, table, t);
+                v.set(t); // rounds the sum to the element type
+            }
         }
-    }
 
-    uint32_t w[RC::WORDS], q, ub;
-    chunk_encode<NBITS, MEE>(v, r, mp.c, mp.cmm, mp.l2b, w, q, ub);
+        uint32_t w[RC::WORDS], q, ub;
+        const uint32_t amax = v.absmax_bits();
+        const bool lane_fast = amax <= kFastMaxBits && r.unit_interval();
+        if (__builtin_amdgcn_ballot_w64(!lane_fast) == 0)
+            chunk_encode_fast<NBITS, MEE>(v, r, amax, mp, w, q, ub);
+        else
+            chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
 
-    uint8_t *gout = dst + sc0 * RC::REC;
-    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
-    if (active) {
-        uint8_t *rec = win_out[wave] + mis + row * RC::REC;
-        chunk_write<NBITS>(rec + j * RC::CB, w, q);
-        if (j == 0) {
-            rec[16 * RC::CB] = (uint8_t)ub;
-            rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+        uint8_t *gout = dst + sc0 * RC::REC;
+        const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
+        if (active) {
+            uint8_t *rec = win_out + mis + row * RC::REC;
+            chunk_write<NBITS>(rec + j * RC::CB, w, q);
+            if (j == 0) {
+                rec[16 * RC::CB] = (uint8_t)ub;
+                rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+            }
         }
+        wave_lds_sync();
+        window_flush(win_out, gout, mis, total, lane);
+        wave_lds_sync();
+
+        if (!has_next) break;
+        v = vn;
+        r = rn;
+        if (FUSED) wr = wn;
+        tile = next;
     }
-    wave_lds_sync();
-    window_flush(win_out[wave], gout, mis, total, lane);
 }
 
-template <int DT, int NBITS, bool MEE, bool ADD>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void hier16_decompress_kernel(
-    const uint8_t *__restrict__ src, void *__restrict__ dst, int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
+// 16-byte slot s of a wave's output tile lives at LDS slot s ^ ((s >> 3) & 7): both
+// the per-lane writes (slots S*lane + j) and the lane-contiguous reads (slots
+// 64*k + lane) then touch eight distinct bank groups per eight lanes
+__device__ __forceinline__ int swz(int s) { return s ^ ((s >> 3) & 7); }
+
+template <int DT, int NBITS, bool MEE, bool ADD, bool LOOP>
+__global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
+                                                              int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
-    __shared__ __attribute__((aligned(16))) uint8_t win_in[kWavesPerBlock][RC::WIN];
+    constexpr int S = Raw16<DT>::kSlots;
+    __shared__ __attribute__((aligned(16))) uint8_t win_in[RC::WIN];
+    __shared__ __attribute__((aligned(16))) uint4 tile_out[64 * S];
     __shared__ float table[MEE ? (1 << NBITS) : 1];
 
+    const int lane = threadIdx.x;
     if (MEE) {
-        for (int k = threadIdx.x; k < (1 << NBITS); k += kWavesPerBlock * 64) table[k] = f16_bits_to_f32(mp.table[k]);
-        __syncthreads();
+        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
+        wave_lds_sync();
+    }
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t ntiles = (nsc + kRowsPerWave - 1) / kRowsPerWave;
+    int64_t tile = blockIdx.x;
+    if (tile >= ntiles) return;
+
+    WinRegs wr;
+    Raw16<DT> acc;
+    {
+        const int64_t sc0 = tile * kRowsPerWave;
+        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+        wr = window_fetch(src + sc0 * RC::REC, rows * RC::REC, lane);
+        if (ADD && row < rows) acc.load(dst, (sc0 * 16 + lane) * 16, vec);
     }
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int64_t sc0 = ((int64_t)blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
-    if (sc0 >= nsc) return;
-    const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-    const int row = lane >> 4, j = lane & 15;
-    const bool active = row < rows;
-    const int64_t e = (sc0 * 16 + lane) * 16;
-    const int total = rows * RC::REC;
+    for (;;) {
+        const int64_t sc0 = tile * kRowsPerWave;
+        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+        const bool active = row < rows;
+        const int total = rows * RC::REC;
 
-    float t[16];
-    if (ADD && active) Vec16<DT>::load(dst, e, t, vec);
+        const int64_t next = tile + gridDim.x;
+        const bool has_next = LOOP && next < ntiles;
+        WinRegs wn = wr;
+        Raw16<DT> accn;
+        if (has_next) {
+            const int64_t nsc0 = next * kRowsPerWave;
+            const int nrows = (int)min((int64_t)kRowsPerWave, nsc - nsc0);
+            wn = window_fetch(src + nsc0 * RC::REC, nrows * RC::REC, lane);
+            if (ADD && row < nrows) accn.load(dst, (nsc0 * 16 + lane) * 16, vec);
+        }
 
-    const int mis_in = window_fill(win_in[wave], src + sc0 * RC::REC, total, lane);
-    wave_lds_sync();
-    if (!active) return;
+        const int mis_in = window_commit(win_in, wr, src + sc0 * RC::REC, total, lane);
+        wave_lds_sync();
+        Raw16<DT> out;
+        if (active) {
+            const uint8_t *rec = win_in + mis_in + row * RC::REC;
+            uint32_t cw[RC::WORDS], cq;
+            chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+            const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+            float t[16];
+            if (ADD) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) t[i] = acc.get(i);
+            }
+            chunk_decode<NBITS, MEE, ADD>(cw, cq, ub, table, t);
+            out.set(t);
+        } else {
+            out.zero();
+        }
+        const int64_t e0 = sc0 * 256; // first element of the tile
+        if (vec) {
+            // transpose through LDS so that every store instruction writes 1 KiB contiguously
+            if (active) {
+#pragma unroll
+                for (int k = 0; k < S; k++) tile_out[swz(S * lane + k)] = out.slot(k);
+            }
+            wave_lds_sync();
+            const int nslots = rows * 16 * S;
+            uint4 *g = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + e0 * (DT == DQ_F32 ? 4 : 2));
+#pragma unroll
+            for (int k = 0; k < S; k++) {
+                const int s = 64 * k + lane;
+                if (s < nslots) g[s] = tile_out[swz(s)];
+            }
+        } else if (active) {
+            out.store(dst, e0 + lane * 16, false);
+        }
+        wave_lds_sync();
 
-    const uint8_t *rec = win_in[wave] + mis_in + row * RC::REC;
-    uint32_t w[RC::WORDS], q;
-    chunk_read<NBITS>(rec + j * RC::CB, w, q);
-    const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
-    chunk_decode<DT, NBITS, MEE, ADD>(w, q, ub, table, t);
-    Vec16<DT>::store(dst, e, t, vec);
+        if (!has_next) break;
+        wr = wn;
+        if (ADD) acc = accn;
+        tile = next;
+    }
 }
 
-// ---- launchers ------------------------------------------------------------------------
+// ---- launchers ------------------------------------------------------------------------------------
 
 template <int NBITS, bool MEE> static MeeArg<NBITS, MEE> make_arg(const MeeParams &mp)
 {
     MeeArg<NBITS, MEE> a;
-    a.c = mp.c; a.cmm = mp.cmm; a.l2b = mp.l2b;
-    for (int k = 0; k < (MEE ? (1 << NBITS) : 2); k++) a.table[k] = mp.table[k];
+    a.c = mp.c; a.cmm = mp.cmm; a.l2b = mp.l2b; a.pad = 0;
+    a.inv_c = 1.0 / (double)mp.c; a.inv_cmm = 1.0 / (double)mp.cmm; a.inv_l2b = 1.0 / (double)mp.l2b;
+    for (int k = 0; k < (MEE ? (1 << NBITS) : 4); k++) a.table[k] = mp.table[k];
     return a;
 }
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-static inline unsigned grid_for(int64_t nsc)
+// resident wave slots to aim for on the current device: CUs x waves per CU
+// (default 32; DYNAMIQ_WAVES_PER_CU overrides it for tuning)
+static int wave_slots()
 {
-    const int64_t per_block = (int64_t)kWavesPerBlock * kRowsPerWave;
-    return (unsigned)((nsc + per_block - 1) / per_block);
+    static std::once_flag once;
+    static int slots[64];
+    static int fallback = 256 * 16;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fallback;
+    std::call_once(once, [] {
+        int per_cu = 32;
+        if (const char *env = getenv("DYNAMIQ_WAVES_PER_CU")) {
+            const int v = atoi(env);
+            if (v >= 1 && v <= 64) per_cu = v;
+        }
+        int n = 0;
+        if (hipGetDeviceCount(&n) != hipSuccess) n = 0;
+        for (int d = 0; d < 64; d++) {
+            int cus = 0;
+            if (d < n && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, d) == hipSuccess && cus > 0)
+                slots[d] = cus * per_cu;
+            else
+                slots[d] = 256 * per_cu;
+        }
+    });
+    return slots[dev];
+}
+
+// number of single-wave workgroups: every wave gets the same number of tiles (+-1);
+// `loop` tells whether any wave gets more than one
+static inline unsigned grid_for(int64_t nsc, bool &loop)
+{
+    const int64_t ntiles = (nsc + kRowsPerWave - 1) / kRowsPerWave;
+    const int64_t slots = wave_slots();
+    const int64_t per_wave = (ntiles + slots - 1) / slots;
+    loop = per_wave > 1;
+    return (unsigned)((ntiles + per_wave - 1) / per_wave);
 }
 
 template <int DT, int RDT, int NBITS, bool MEE>
@@ -361,12 +678,16 @@ static hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *ds
                                bool fused, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
-    dim3 grid(grid_for(nsc)), block(kWavesPerBlock * 64);
+    bool loop;
+    dim3 grid(grid_for(nsc, loop)), block(64);
     const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
-    if (fused)
-        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg);
-    else
-        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg);
+#define DQ_LAUNCH_C(F, L) hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, F, L>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg)
+    if (fused) {
+        if (loop) DQ_LAUNCH_C(true, true); else DQ_LAUNCH_C(true, false);
+    } else {
+        if (loop) DQ_LAUNCH_C(false, true); else DQ_LAUNCH_C(false, false);
+    }
+#undef DQ_LAUNCH_C
     return hipGetLastError();
 }
 
@@ -374,12 +695,16 @@ template <int DT, int NBITS, bool MEE>
 static hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nsc, int add, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
-    dim3 grid(grid_for(nsc)), block(kWavesPerBlock * 64);
+    bool loop;
+    dim3 grid(grid_for(nsc, loop)), block(64);
     const int vec = aligned16(dst) ? 1 : 0;
-    if (add)
-        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, true>), grid, block, 0, stream, src, dst, nsc, vec, arg);
-    else
-        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false>), grid, block, 0, stream, src, dst, nsc, vec, arg);
+#define DQ_LAUNCH_D(A, L) hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, A, L>), grid, block, 0, stream, src, dst, nsc, vec, arg)
+    if (add) {
+        if (loop) DQ_LAUNCH_D(true, true); else DQ_LAUNCH_D(true, false);
+    } else {
+        if (loop) DQ_LAUNCH_D(false, true); else DQ_LAUNCH_D(false, false);
+    }
+#undef DQ_LAUNCH_D
     return hipGetLastError();
 }
 
