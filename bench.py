@@ -66,6 +66,10 @@ def main():
     ap.add_argument("--src", choices=["fp32", "bf16"], default="fp32")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the cpu_baseline leg (0 = skip)")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle parity check of a sample")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain elementwise fp32 copy kernel (out = in * 1.0) of the same element count, "
+                         "4*N bytes read + 4*N bytes written per launch, so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -120,6 +124,13 @@ def main():
     dec_bytes = (sbytes + (nbits + OVERHEAD_BITS) / 8.0) * n
     comp_gbs = comp_bytes / (comp_ms * 1e-3) / 1e9
     dec_gbs = dec_bytes / (dec_ms * 1e-3) / 1e9
+
+    if args.pmc_calibration:
+        cal_src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
+        cal_dst = torch.empty_like(cal_src)
+        for _ in range(5):
+            torch.mul(cal_src, 1.0, out=cal_dst)
+        torch.cuda.synchronize()
 
     # ---- quality: NMSE of the round trip ----
     xf = x32.double()

@@ -148,7 +148,9 @@ void scaling_compress_impl(torch::Tensor src, torch::Tensor dst, torch::Tensor r
     TORCH_CHECK(rand_pool.device().type() == torch::kCUDA, "rand_pool must be a CUDA tensor");
     TORCH_CHECK(is_supported_data_dtype(src.scalar_type(), ex), "input must be torch.float16 or torch.bfloat16");
     TORCH_CHECK(dst.dtype() == torch::kUInt8, "output must be torch.uint8");
-    TORCH_CHECK(rand_pool.dtype() == src.dtype(), "rand_pool dtype must match input dtype");
+    // extended calls also take a bf16 pool next to float32 gradients (the reference's pools are bf16)
+    const bool mixed = ex && src.scalar_type() == torch::kFloat32 && rand_pool.scalar_type() == torch::kBFloat16;
+    TORCH_CHECK(mixed || rand_pool.dtype() == src.dtype(), "rand_pool dtype must match input dtype");
     TORCH_CHECK(src.is_contiguous(), "input must be contiguous");
     TORCH_CHECK(dst.is_contiguous(), "output must be contiguous");
     TORCH_CHECK(rand_pool.is_contiguous(), "rand_pool must be contiguous");
@@ -157,7 +159,8 @@ void scaling_compress_impl(torch::Tensor src, torch::Tensor dst, torch::Tensor r
     TORCH_CHECK(rand_pool.numel() >= n, "rand_pool has fewer than n elements");
     TORCH_CHECK(dst.numel() >= dq_scaling_required_bytes(n, nbits, chunk_size, strategy), "output buffer is too small");
     check_status(dq_scaling_compress(src.data_ptr(), dst.data_ptr<uint8_t>(), rand_pool.data_ptr(), n, nbits, chunk_size,
-                                     dq_dtype_of(src.scalar_type()), src.device().index(), strategy, as_stream(stream_p)),
+                                     dq_dtype_of(src.scalar_type()) | (mixed ? DQ_RAND_BF16 : 0), src.device().index(), strategy,
+                                     as_stream(stream_p)),
                  "scaling_compress");
 }
 
@@ -188,7 +191,8 @@ void scaling_dec_comp_impl(torch::Tensor recv, torch::Tensor inp, torch::Tensor 
     TORCH_CHECK(recv.dtype() == torch::kUInt8, "recv must be torch.uint8");
     TORCH_CHECK(is_supported_data_dtype(inp.scalar_type(), ex), "inp must be torch.float16 or torch.bfloat16");
     TORCH_CHECK(send.dtype() == torch::kUInt8, "send must be torch.uint8");
-    TORCH_CHECK(rand_pool.dtype() == inp.dtype(), "rand_pool dtype must match inp dtype");
+    const bool mixed = ex && inp.scalar_type() == torch::kFloat32 && rand_pool.scalar_type() == torch::kBFloat16;
+    TORCH_CHECK(mixed || rand_pool.dtype() == inp.dtype(), "rand_pool dtype must match inp dtype");
     TORCH_CHECK(recv.is_contiguous(), "recv must be contiguous");
     TORCH_CHECK(inp.is_contiguous(), "inp must be contiguous");
     TORCH_CHECK(send.is_contiguous(), "send must be contiguous");
@@ -200,8 +204,8 @@ void scaling_dec_comp_impl(torch::Tensor recv, torch::Tensor inp, torch::Tensor 
     TORCH_CHECK(inp.numel() >= n, "inp has fewer than n elements");
     TORCH_CHECK(rand_pool.numel() >= n, "rand_pool has fewer than n elements");
     check_status(dq_scaling_dec_comp(recv.data_ptr<uint8_t>(), inp.data_ptr(), send.data_ptr<uint8_t>(), rand_pool.data_ptr(), n,
-                                     nbits, chunk_size, dq_dtype_of(inp.scalar_type()), recv.device().index(), strategy,
-                                     as_stream(stream_p)),
+                                     nbits, chunk_size, dq_dtype_of(inp.scalar_type()) | (mixed ? DQ_RAND_BF16 : 0),
+                                     recv.device().index(), strategy, as_stream(stream_p)),
                  "scaling_dec_comp");
 }
 

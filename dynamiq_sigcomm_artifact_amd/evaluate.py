@@ -1,0 +1,281 @@
+"""Runs the synthetic workloads of the build's baseline configurations on one GPU
+and prints one JSON line per measurement (NMSE, GB/s, fraction of the 8 TB/s HBM
+peak).  ``python -m dynamiq_sigcomm_artifact_amd.evaluate --config 1|2|3|4|5``.
+
+  1  2^20 fp32 N(0,1e-3^2): blocked randomized Hadamard + quantise + pack and back
+  2  25 MB bucket, Student-t with outliers: 4/8-bit round trips, fp32 and bf16
+  3  8 simulated ranks x 124,439,808 elements: compressed ring all-reduce
+  4  Llama-3-8B shaped gradient set in 25 MB buckets: dynamic {2,4,8}-bit allocation
+  5  2^30 fp32: compress / decompress / fused sweep, and the blocked transform
+
+Timings use HIP events on the launch stream, 10 warm-up + 50 timed launches
+(cuda_kernels/tests/benchmark_scaling_quantization.py:41-57).
+"""
+import argparse
+import json
+import math
+import types
+
+import torch
+
+from . import bitrate, capi
+from .compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
+from .dynamiq_pipeline import dynamic_bitrate_allreduce
+from .ring_sim import ring_allreduce, split_chunks
+
+HBM_PEAK = 8000.0  # GB/s
+OV = 0.5625        # scale overhead, bits per element
+
+
+def _time_us(fn, warmup=10, iters=50):
+    for _ in range(warmup):
+        fn()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    e.synchronize()
+    return s.elapsed_time(e) / iters * 1e3
+
+
+def _nmse(x, xhat):
+    x = x.double()
+    return float(((xhat.double() - x) ** 2).sum() / (x ** 2).sum())
+
+
+def _emit(**kw):
+    print(json.dumps(kw), flush=True)
+
+
+def _student_bucket(n, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    z = torch.randn(n, generator=g, device=dev)
+    chi = torch.randn(3, n, generator=g, device=dev).square_().sum(0)
+    x = z / torch.sqrt(chi / 3.0) * 1e-3
+    idx = torch.randint(0, n, (max(1, n // 1000),), generator=g, device=dev)
+    x[idx] *= 100.0
+    return x.contiguous()
+
+
+def config1(dev):
+    n = 1 << 20
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(n, generator=g, device=dev) * 1e-3
+    rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+    sign = torch.empty(n, device=dev)
+    capi.rand_diag(sign, 0)
+    for kb in (10, 11, 12, 13, 14, 15, 20):
+        B = 1 << kb
+        scale = 1.0 / math.sqrt(B)
+        for nbits in (4, 5, 8):
+            y = x.clone()
+            capi.rht_blocked(y, sign, B, scale, False)
+            packed = torch.zeros(capi.required_bytes(n, nbits, 16, 2), dtype=torch.uint8, device=dev)
+            capi.scaling_compress(y, packed, rand, n, nbits, 16, 2)
+            z = torch.empty_like(y)
+            capi.scaling_decompress(packed, z, n, nbits, 16, 2)
+            capi.rht_blocked(z, sign, B, scale, True)
+            plain = torch.empty_like(x)
+            packed2 = torch.zeros_like(packed)
+            capi.scaling_compress(x, packed2, rand, n, nbits, 16, 2)
+            capi.scaling_decompress(packed2, plain, n, nbits, 16, 2)
+            t_rht = _time_us(lambda: capi.rht_blocked(y, sign, B, scale, False))
+            _emit(config=1, block=B, nbits=nbits, nmse_rht=_nmse(x, z), nmse_no_rht=_nmse(x, plain),
+                  rht_us=round(t_rht, 2), rht_GBps=round(8.0 * n / t_rht / 1e3, 1))
+
+
+def config2(dev):
+    n = 6553600
+    x32 = _student_bucket(n, dev)
+    g = torch.Generator(device=dev).manual_seed(1)
+    rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+    for src_name, src in (("fp32", x32), ("bf16", x32.to(torch.bfloat16))):
+        sb = src.element_size()
+        for strategy in (2, 3):
+            for nbits in (4, 8):
+                packed = torch.zeros(capi.required_bytes(n, nbits, 16, strategy), dtype=torch.uint8, device=dev)
+                out = torch.empty_like(src)
+                capi.scaling_compress(src, packed, rand, n, nbits, 16, strategy)
+                capi.scaling_decompress(packed, out, n, nbits, 16, strategy)
+                tc = _time_us(lambda: capi.scaling_compress(src, packed, rand, n, nbits, 16, strategy))
+                td = _time_us(lambda: capi.scaling_decompress(packed, out, n, nbits, 16, strategy))
+                pb = (nbits + OV) / 8
+                _emit(config=2, source=src_name, strategy=strategy, nbits=nbits, nmse=_nmse(x32, out),
+                      compress_us=round(tc, 2), decompress_us=round(td, 2),
+                      roundtrip_GBps_of_fp32_input=round(4.0 * n / (tc + td) / 1e3, 1),
+                      compress_frac_hbm=round((sb + 2 + pb) * n / tc / 1e3 / HBM_PEAK, 4),
+                      decompress_frac_hbm=round((sb + pb) * n / td / 1e3 / HBM_PEAK, 4))
+
+
+def _params(d, W, r):
+    return {"d": {(0, 0): d}, "world_size": W, "rank": r, "args": types.SimpleNamespace(aggregation_method="dynamiQ")}
+
+
+def config3(dev, n=124439808, W=8):
+    g = torch.Generator(device=dev).manual_seed(0)
+    sig = torch.pow(10.0, torch.rand(W, generator=g, device=dev) * 2.0 - 4.0)   # log-uniform [1e-4, 1e-2]
+    npad = (n + 255) // 256 * 256
+    exact = torch.zeros(npad, dtype=torch.float64, device=dev)
+    grads = []
+    for r in range(W):
+        x = torch.zeros(npad, device=dev)
+        x[:n] = torch.randn(n, generator=g, device=dev) * sig[r]
+        exact += x.double()
+        grads.append(x.to(torch.bfloat16))          # the DDP hook hands bf16 buckets to the compressor
+        del x
+    for nbits in (4, 5, 8):
+        for cls, name in ((Aee_Dynamic_Range_GPU_kern, "aee"), (Mee_Dynamic_Range_GPU_kern, "mee")):
+            gen = torch.Generator(device=dev).manual_seed(7)
+            comps = [cls(nbits, 16, _params(npad, W, r), generator=gen) for r in range(W)]
+            vecs = [x.clone() for x in grads]
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            ring_allreduce(vecs, comps)
+            e.record()
+            e.synchronize()
+            ms = s.elapsed_time(e)
+            same = all(torch.equal(vecs[0], v) for v in vecs[1:])
+            # one fused reduce-scatter step of one rank on its ring chunk
+            chunk = split_chunks(vecs[0], W, 256)[0]
+            m = chunk.numel()
+            recv = comps[0].create_tensor(chunk, torch.uint8)
+            send = comps[0].create_tensor(chunk, torch.uint8)
+            comps[0].compression(chunk, recv)
+            t = _time_us(lambda: comps[0].dec_compression(recv, chunk, send), 5, 25)
+            pb = (nbits + OV) / 8
+            _emit(config=3, world=W, elements_per_rank=n, nbits=nbits, method=name, nmse_vs_fp64_sum=_nmse(exact, vecs[0]),
+                  ranks_identical=same, ring_total_ms=round(ms, 3), step_elements=m, step_us=round(t, 2),
+                  step_GBps_algorithmic=round((2 + 2 + 2 * pb) * m / t / 1e3, 1),
+                  step_frac_hbm=round((2 + 2 + 2 * pb) * m / t / 1e3 / HBM_PEAK, 4))
+            del vecs, comps
+
+
+LLAMA3_8B = [("embed", 128256 * 4096)] + [
+    (name, numel) for _ in range(32) for name, numel in (
+        ("q", 4096 * 4096), ("k", 1024 * 4096), ("v", 1024 * 4096), ("o", 4096 * 4096),
+        ("gate", 14336 * 4096), ("up", 14336 * 4096), ("down", 4096 * 14336))]
+
+
+def _llama_buckets(dev, bucket=6553600, limit=None):
+    """yields fp32 buckets of the flattened gradient set; per-tensor scale log-normal(ln 1e-3, 1.5)"""
+    g = torch.Generator(device=dev).manual_seed(0)
+    gs = torch.Generator().manual_seed(1)
+    scales = torch.exp(torch.randn(len(LLAMA3_8B), generator=gs) * 1.5 + math.log(1e-3)).tolist()
+    buf = torch.empty(bucket, device=dev)
+    fill, count = 0, 0
+    for (name, numel), sc in zip(LLAMA3_8B, scales):
+        left = numel
+        while left > 0:
+            take = min(left, bucket - fill)
+            buf[fill:fill + take] = torch.randn(take, generator=g, device=dev) * sc
+            fill += take
+            left -= take
+            if fill == bucket:
+                yield buf
+                count += 1
+                if limit and count >= limit:
+                    return
+                fill = 0
+    if fill:
+        yield buf[:fill // 256 * 256]
+
+
+def config4(dev, limit=None):
+    target = 5.0 - bitrate.DYNAMIC_BITRATE_HEADROOM
+    from .compressors import superchunk_mean_center
+    # pass 1: norms of every superchunk -> u
+    norms_list = []
+    for b in _llama_buckets(dev, limit=limit):
+        x = b.to(torch.bfloat16)
+        n = x.numel()
+        res = torch.empty(n, dtype=torch.bfloat16, device=dev)
+        st = torch.empty((n // 256, 2), dtype=torch.bfloat16, device=dev)
+        superchunk_mean_center(x, res, st, n, 1, 256)
+        norms_list.append(st[:, 1].clone())
+    u, avg_bits, delta = bitrate.dynamic_bitrate_binary_search_u(norms_list, target)
+    # pass 2: quantise
+    for cls, name in ((Aee_Dynamic_Range_GPU_kern, "aee"), (Mee_Dynamic_Range_GPU_kern, "mee")):
+        gen = torch.Generator(device=dev).manual_seed(3)
+        comps = {q: [cls(q, 16, _params(6553600 * 8, 1, 0), generator=gen)] for q in (2, 4, 8)}
+        num = den = 0.0
+        bits = elems = 0
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        gpu_ms = 0.0
+        nb = 0
+        for b in _llama_buckets(dev, limit=limit):
+            x = b.to(torch.bfloat16)
+            s.record()
+            outs, _, qbits = dynamic_bitrate_allreduce([x], u, comps)
+            e.record()
+            e.synchronize()
+            gpu_ms += s.elapsed_time(e)
+            num += float(((outs[0].double() - b.double()) ** 2).sum())
+            den += float((b.double() ** 2).sum())
+            bits += int(qbits.sum())
+            elems += qbits.numel()
+            nb += 1
+        _emit(config=4, method=name, buckets=nb, elements=elems * 256, target_avg_bits=target, u=u,
+              search_avg_bits=avg_bits, achieved_avg_code_bits=bits / elems,
+              achieved_bits_with_scales=bits / elems + OV, nmse=num / den,
+              pipeline_GBps_of_bf16_input=round(2.0 * elems * 256 / (gpu_ms * 1e-3) / 1e9, 1))
+
+
+def config5(dev, n=1 << 30):
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(n, generator=g, device=dev) * 1e-3
+    rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty_like(x)
+    for nbits in (2, 4, 5, 8):
+        packed = torch.zeros(capi.required_bytes(n, nbits, 16, 2), dtype=torch.uint8, device=dev)
+        send = torch.zeros_like(packed)
+        capi.scaling_compress(x, packed, rand, n, nbits, 16, 2)
+        tc = _time_us(lambda: capi.scaling_compress(x, packed, rand, n, nbits, 16, 2), 3, 10)
+        td = _time_us(lambda: capi.scaling_decompress(packed, out, n, nbits, 16, 2), 3, 10)
+        tf = _time_us(lambda: capi.scaling_dec_comp(packed, x, send, rand, n, nbits, 16, 2), 3, 10)
+        pb = (nbits + OV) / 8
+        _emit(config=5, op="quantise", nbits=nbits, nmse=_nmse(x, out), compress_us=round(tc, 1), decompress_us=round(td, 1),
+              fused_us=round(tf, 1), compress_GBps_fp32_in=round(4.0 * n / tc / 1e3, 1),
+              compress_frac_hbm=round((4 + 2 + pb) * n / tc / 1e3 / HBM_PEAK, 4),
+              decompress_frac_hbm=round((4 + pb) * n / td / 1e3 / HBM_PEAK, 4),
+              fused_frac_hbm=round((4 + 2 + 2 * pb) * n / tf / 1e3 / HBM_PEAK, 4))
+        del packed, send
+    del out, rand
+    sign = torch.empty(n, device=dev)
+    capi.rand_diag(sign, 0)
+    for kb in (10, 11, 12, 13, 14, 15):
+        B = 1 << kb
+        t = _time_us(lambda: capi.rht_blocked(x, sign, B, 1.0, False), 2, 5)
+        _emit(config=5, op="rht_blocked", block=B, us=round(t, 1), GBps=round(12.0 * n / t / 1e3, 1),
+              frac_hbm=round(12.0 * n / t / 1e3 / HBM_PEAK, 4))
+    t = _time_us(lambda: capi.hadamard(x), 1, 3)
+    _emit(config=5, op="hadamard_whole_vector", n=n, us=round(t, 1))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", type=int, required=True, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--limit", type=int, default=None, help="config 4: number of 25 MB buckets to process")
+    ap.add_argument("--n", type=int, default=None, help="configs 3 and 5: element count override")
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        raise SystemExit("evaluate needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.config == 1:
+        config1(dev)
+    elif args.config == 2:
+        config2(dev)
+    elif args.config == 3:
+        config3(dev, **({"n": args.n} if args.n else {}))
+    elif args.config == 4:
+        config4(dev, args.limit)
+    else:
+        config5(dev, **({"n": args.n} if args.n else {}))
+
+
+if __name__ == "__main__":
+    main()
