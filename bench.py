@@ -31,6 +31,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 OVERHEAD_BITS = 0.5625  # hierarchical scale bytes per element, in bits
 
+# HBM bytes per launch of the compress kernel from two `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for
+# the --pmc-calibration copy kernel: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0.
+# key: (source dtype, nbits, strategy, elements)
+MEASURED_TRAFFIC_BYTES = {
+    ("fp32", 4, 2, 6553600): int((2.0 * 19237.0 + 1.0 * 3800.0) * 1024),
+}
+
 
 def make_bucket(n, seed, device):
     """Student-t(nu=3) * 1e-3 with 0.1 % outliers * 100, generated on the device."""
@@ -67,7 +75,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the cpu_baseline leg (0 = skip)")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle parity check of a sample")
     ap.add_argument("--pmc-calibration", action="store_true",
-                    help="also run a plain elementwise fp32 copy kernel (out = in * 1.0) of the same element count, "
+                    help="also run a plain elementwise fp32 copy kernel (out = -in) of the same element count, "
                          "4*N bytes read + 4*N bytes written per launch, so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
@@ -129,7 +137,7 @@ def main():
         cal_src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
         cal_dst = torch.empty_like(cal_src)
         for _ in range(5):
-            torch.mul(cal_src, 1.0, out=cal_dst)
+            torch.neg(cal_src, out=cal_dst)
         torch.cuda.synchronize()
 
     # ---- quality: NMSE of the round trip ----
@@ -207,7 +215,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(comp_gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.src, nbits, strategy, n)),
             "algorithmic_bytes_per_launch": int(comp_bytes),
             "avg_launch_ms": round(comp_ms, 5),
         },
