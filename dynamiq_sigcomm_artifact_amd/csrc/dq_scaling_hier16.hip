@@ -14,10 +14,10 @@
 //     whose offset equals the global address modulo 16 and streamed out with
 //     aligned 128-bit stores (ragged head / tail bytes singly); packed input is
 //     pulled through the same kind of window with aligned 128-bit loads;
-//   * a wave walks tiles blockIdx, blockIdx + gridDim, ... and issues the loads
-//     of its next tile before it computes the current one, so HBM latency hides
-//     behind the VALU work even when the whole grid is resident at once (a
-//     25 MB bucket is only ~1.5 tiles per wave slot of the chip).
+//   * one single-wave workgroup per tile, ~50 VGPRs, 8 waves per SIMD: many
+//     small workgroups let the dispatcher balance the chip better than a
+//     persistent loop with software prefetch did (4.7 -> 5.4 TB/s at 1 GiB), and
+//     a 25 MB bucket (6400 tiles) fits the machine in one resident round.
 //
 // VALU budget.  The quantiser is VALU-bound if written naively (IEEE division,
 // NaN/Inf/out-of-range guards per element).  Two measures keep it HBM-bound:
@@ -36,10 +36,6 @@
 //
 // Numerics: csrc/cuda_hierarchical_mee.cu:203-343 (compress), 345-505
 // (decompress) and 526-696 (fused decompress-accumulate-recompress).
-#include <stdlib.h>
-
-#include <mutex>
-
 #include "dq_device.cuh"
 #include "dq_launch.h"
 
@@ -416,8 +412,8 @@ constexpr uint32_t kFastMaxBits = 0x71800000u; // 2^100
 
 // ---- kernels ------------------------------------------------------------------------------------
 
-// compress (FUSED = false) or decode-accumulate-recompress (FUSED = true)
-template <int DT, int RDT, int NBITS, bool MEE, bool FUSED, bool LOOP>
+// compress (FUSED = false) or decode-accumulate-recompress (FUSED = true); workgroup = one wave = one tile
+template <int DT, int RDT, int NBITS, bool MEE, bool FUSED>
 __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restrict__ src, const uint8_t *__restrict__ recv,
                                                             uint8_t *__restrict__ dst, const void *__restrict__ rnd,
                                                             int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
@@ -428,101 +424,65 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     __shared__ float table[(MEE && FUSED) ? (1 << NBITS) : 1];
 
     const int lane = threadIdx.x;
-    if (MEE && FUSED) {
-        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
-        wave_lds_sync();
-    }
     const int row = lane >> 4, j = lane & 15;
-    const int64_t ntiles = (nsc + kRowsPerWave - 1) / kRowsPerWave;
-    int64_t tile = blockIdx.x;
-    if (tile >= ntiles) return;
+    const int64_t sc0 = (int64_t)blockIdx.x * kRowsPerWave;
+    if (sc0 >= nsc) return;
+    const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+    const bool active = row < rows;
+    const int total = rows * RC::REC;
 
+    // all global loads of the tile are issued before anything waits on them
     Raw16<DT> v;
     Raw16<RDT> r;
+    if (active) {
+        v.load(src, (sc0 * 16 + lane) * 16, vec & 1);
+        r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
+    } else {
+        v.zero();
+        r.zero();
+    }
     WinRegs wr;
-    wr.a = wr.b = (u32x4)(0u);
-    {
-        const int64_t sc0 = tile * kRowsPerWave;
-        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-        if (row < rows) {
-            v.load(src, (sc0 * 16 + lane) * 16, vec & 1);
-            r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
-        } else {
-            v.zero();
-            r.zero();
-        }
-        if (FUSED) wr = window_fetch(recv + sc0 * RC::REC, rows * RC::REC, lane);
+    if (FUSED) wr = window_fetch(recv + sc0 * RC::REC, total, lane);
+    if (MEE && FUSED) {
+        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
     }
 
-    for (;;) {
-        const int64_t sc0 = tile * kRowsPerWave;
-        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-        const bool active = row < rows;
-        const int total = rows * RC::REC;
-
-        // issue the next tile's loads before touching the current one
-        const int64_t next = tile + gridDim.x;
-        const bool has_next = LOOP && next < ntiles;
-        Raw16<DT> vn;
-        Raw16<RDT> rn;
-        WinRegs wn = wr;
-        if (has_next) {
-            const int64_t nsc0 = next * kRowsPerWave;
-            const int nrows = (int)min((int64_t)kRowsPerWave, nsc - nsc0);
-            if (row < nrows) {
-                vn.load(src, (nsc0 * 16 + lane) * 16, vec & 1);
-                rn.load(rnd, (nsc0 * 16 + lane) * 16, vec & 2);
-            } else {
-                vn.zero();
-                rn.zero();
-            }
-            if (FUSED) wn = window_fetch(recv + nsc0 * RC::REC, nrows * RC::REC, lane);
-        }
-
-        if (FUSED) {
-            const int mis_in = window_commit(win_in, wr, recv + sc0 * RC::REC, total, lane);
-            wave_lds_sync();
-            if (active) {
-                const uint8_t *rec = win_in + mis_in + row * RC::REC;
-                uint32_t cw[RC::WORDS], cq;
-                chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
-                const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
-                float t[16];
-#pragma unroll
-                for (int i = 0; i < 16; i++) t[i] = v.get(i);
-                chunk_decode<NBITS, MEE, true>(cw, cq, ub, table, t);
-                v.set(t); // rounds the sum to the element type
-            }
-        }
-
-        uint32_t w[RC::WORDS], q, ub;
-        const uint32_t amax = v.absmax_bits();
-        const bool lane_fast = amax <= kFastMaxBits && r.unit_interval();
-        if (__builtin_amdgcn_ballot_w64(!lane_fast) == 0)
-            chunk_encode_fast<NBITS, MEE>(v, r, amax, mp, w, q, ub);
-        else
-            chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
-
-        uint8_t *gout = dst + sc0 * RC::REC;
-        const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
+    if (FUSED) {
+        const int mis_in = window_commit(win_in, wr, recv + sc0 * RC::REC, total, lane);
+        wave_lds_sync();
         if (active) {
-            uint8_t *rec = win_out + mis + row * RC::REC;
-            chunk_write<NBITS>(rec + j * RC::CB, w, q);
-            if (j == 0) {
-                rec[16 * RC::CB] = (uint8_t)ub;
-                rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
-            }
+            const uint8_t *rec = win_in + mis_in + row * RC::REC;
+            uint32_t cw[RC::WORDS], cq;
+            chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+            const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+            float t[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = v.get(i);
+            chunk_decode<NBITS, MEE, true>(cw, cq, ub, table, t);
+            v.set(t); // rounds the sum to the element type
         }
-        wave_lds_sync();
-        window_flush(win_out, gout, mis, total, lane);
-        wave_lds_sync();
-
-        if (!has_next) break;
-        v = vn;
-        r = rn;
-        if (FUSED) wr = wn;
-        tile = next;
     }
+
+    uint32_t w[RC::WORDS], q, ub;
+    const uint32_t amax = v.absmax_bits();
+    const bool lane_fast = amax <= kFastMaxBits && r.unit_interval();
+    if (__builtin_amdgcn_ballot_w64(!lane_fast) == 0)
+        chunk_encode_fast<NBITS, MEE>(v, r, amax, mp, w, q, ub);
+    else
+        chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
+
+    uint8_t *gout = dst + sc0 * RC::REC;
+    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
+    if (active) {
+        uint8_t *rec = win_out + mis + row * RC::REC;
+        chunk_write<NBITS>(rec + j * RC::CB, w, q);
+        if (j == 0) {
+            rec[16 * RC::CB] = (uint8_t)ub;
+            rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+        }
+    }
+    wave_lds_sync();
+    window_flush(win_out, gout, mis, total, lane);
 }
 
 // 16-byte slot s of a wave's output tile lives at LDS slot s ^ ((s >> 3) & 7): both
@@ -530,7 +490,7 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
 // 64*k + lane) then touch eight distinct bank groups per eight lanes
 __device__ __forceinline__ int swz(int s) { return s ^ ((s >> 3) & 7); }
 
-template <int DT, int NBITS, bool MEE, bool ADD, bool LOOP>
+template <int DT, int NBITS, bool MEE, bool ADD>
 __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
                                                               int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
 {
@@ -541,83 +501,55 @@ __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__
     __shared__ float table[MEE ? (1 << NBITS) : 1];
 
     const int lane = threadIdx.x;
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t sc0 = (int64_t)blockIdx.x * kRowsPerWave;
+    if (sc0 >= nsc) return;
+    const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+    const bool active = row < rows;
+    const int total = rows * RC::REC;
+    const int64_t e0 = sc0 * 256; // first element of the tile
+
+    const WinRegs wr = window_fetch(src + sc0 * RC::REC, total, lane);
+    Raw16<DT> acc;
+    if (ADD && active) acc.load(dst, e0 + lane * 16, vec);
     if (MEE) {
         for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
-        wave_lds_sync();
-    }
-    const int row = lane >> 4, j = lane & 15;
-    const int64_t ntiles = (nsc + kRowsPerWave - 1) / kRowsPerWave;
-    int64_t tile = blockIdx.x;
-    if (tile >= ntiles) return;
-
-    WinRegs wr;
-    Raw16<DT> acc;
-    {
-        const int64_t sc0 = tile * kRowsPerWave;
-        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-        wr = window_fetch(src + sc0 * RC::REC, rows * RC::REC, lane);
-        if (ADD && row < rows) acc.load(dst, (sc0 * 16 + lane) * 16, vec);
     }
 
-    for (;;) {
-        const int64_t sc0 = tile * kRowsPerWave;
-        const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-        const bool active = row < rows;
-        const int total = rows * RC::REC;
-
-        const int64_t next = tile + gridDim.x;
-        const bool has_next = LOOP && next < ntiles;
-        WinRegs wn = wr;
-        Raw16<DT> accn;
-        if (has_next) {
-            const int64_t nsc0 = next * kRowsPerWave;
-            const int nrows = (int)min((int64_t)kRowsPerWave, nsc - nsc0);
-            wn = window_fetch(src + nsc0 * RC::REC, nrows * RC::REC, lane);
-            if (ADD && row < nrows) accn.load(dst, (nsc0 * 16 + lane) * 16, vec);
+    const int mis_in = window_commit(win_in, wr, src + sc0 * RC::REC, total, lane);
+    wave_lds_sync();
+    Raw16<DT> out;
+    if (active) {
+        const uint8_t *rec = win_in + mis_in + row * RC::REC;
+        uint32_t cw[RC::WORDS], cq;
+        chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+        const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+        float t[16];
+        if (ADD) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = acc.get(i);
         }
-
-        const int mis_in = window_commit(win_in, wr, src + sc0 * RC::REC, total, lane);
-        wave_lds_sync();
-        Raw16<DT> out;
+        chunk_decode<NBITS, MEE, ADD>(cw, cq, ub, table, t);
+        out.set(t);
+    } else {
+        out.zero();
+    }
+    if (vec) {
+        // transpose through LDS so that every store instruction writes 1 KiB contiguously
         if (active) {
-            const uint8_t *rec = win_in + mis_in + row * RC::REC;
-            uint32_t cw[RC::WORDS], cq;
-            chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
-            const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
-            float t[16];
-            if (ADD) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) t[i] = acc.get(i);
-            }
-            chunk_decode<NBITS, MEE, ADD>(cw, cq, ub, table, t);
-            out.set(t);
-        } else {
-            out.zero();
-        }
-        const int64_t e0 = sc0 * 256; // first element of the tile
-        if (vec) {
-            // transpose through LDS so that every store instruction writes 1 KiB contiguously
-            if (active) {
-#pragma unroll
-                for (int k = 0; k < S; k++) tile_out[swz(S * lane + k)] = out.slot(k);
-            }
-            wave_lds_sync();
-            const int nslots = rows * 16 * S;
-            uint4 *g = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + e0 * (DT == DQ_F32 ? 4 : 2));
-#pragma unroll
-            for (int k = 0; k < S; k++) {
-                const int s = 64 * k + lane;
-                if (s < nslots) g[s] = tile_out[swz(s)];
-            }
-        } else if (active) {
-            out.store(dst, e0 + lane * 16, false);
+            for (int k = 0; k < S; k++) tile_out[swz(S * lane + k)] = out.slot(k);
         }
         wave_lds_sync();
-
-        if (!has_next) break;
-        wr = wn;
-        if (ADD) acc = accn;
-        tile = next;
+        const int nslots = rows * 16 * S;
+        uint4 *g = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + e0 * (DT == DQ_F32 ? 4 : 2));
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const int s = 64 * k + lane;
+            if (s < nslots) g[s] = tile_out[swz(s)];
+        }
+    } else if (active) {
+        out.store(dst, e0 + lane * 16, false);
     }
 }
 
@@ -634,60 +566,20 @@ template <int NBITS, bool MEE> static MeeArg<NBITS, MEE> make_arg(const MeeParam
 
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// resident wave slots to aim for on the current device: CUs x waves per CU
-// (default 32; DYNAMIQ_WAVES_PER_CU overrides it for tuning)
-static int wave_slots()
-{
-    static std::once_flag once;
-    static int slots[64];
-    static int fallback = 256 * 16;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fallback;
-    std::call_once(once, [] {
-        int per_cu = 32;
-        if (const char *env = getenv("DYNAMIQ_WAVES_PER_CU")) {
-            const int v = atoi(env);
-            if (v >= 1 && v <= 64) per_cu = v;
-        }
-        int n = 0;
-        if (hipGetDeviceCount(&n) != hipSuccess) n = 0;
-        for (int d = 0; d < 64; d++) {
-            int cus = 0;
-            if (d < n && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, d) == hipSuccess && cus > 0)
-                slots[d] = cus * per_cu;
-            else
-                slots[d] = 256 * per_cu;
-        }
-    });
-    return slots[dev];
-}
-
-// number of single-wave workgroups: every wave gets the same number of tiles (+-1);
-// `loop` tells whether any wave gets more than one
-static inline unsigned grid_for(int64_t nsc, bool &loop)
-{
-    const int64_t ntiles = (nsc + kRowsPerWave - 1) / kRowsPerWave;
-    const int64_t slots = wave_slots();
-    const int64_t per_wave = (ntiles + slots - 1) / slots;
-    loop = per_wave > 1;
-    return (unsigned)((ntiles + per_wave - 1) / per_wave);
-}
+// one single-wave workgroup per tile of 4 superchunks
+static inline unsigned grid_for(int64_t nsc) { return (unsigned)((nsc + kRowsPerWave - 1) / kRowsPerWave); }
 
 template <int DT, int RDT, int NBITS, bool MEE>
 static hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, int64_t nsc,
                                bool fused, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
-    bool loop;
-    dim3 grid(grid_for(nsc, loop)), block(64);
+    dim3 grid(grid_for(nsc)), block(64);
     const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
-#define DQ_LAUNCH_C(F, L) hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, F, L>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg)
-    if (fused) {
-        if (loop) DQ_LAUNCH_C(true, true); else DQ_LAUNCH_C(true, false);
-    } else {
-        if (loop) DQ_LAUNCH_C(false, true); else DQ_LAUNCH_C(false, false);
-    }
-#undef DQ_LAUNCH_C
+    if (fused)
+        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg);
+    else
+        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg);
     return hipGetLastError();
 }
 
@@ -695,16 +587,12 @@ template <int DT, int NBITS, bool MEE>
 static hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nsc, int add, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
-    bool loop;
-    dim3 grid(grid_for(nsc, loop)), block(64);
+    dim3 grid(grid_for(nsc)), block(64);
     const int vec = aligned16(dst) ? 1 : 0;
-#define DQ_LAUNCH_D(A, L) hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, A, L>), grid, block, 0, stream, src, dst, nsc, vec, arg)
-    if (add) {
-        if (loop) DQ_LAUNCH_D(true, true); else DQ_LAUNCH_D(true, false);
-    } else {
-        if (loop) DQ_LAUNCH_D(false, true); else DQ_LAUNCH_D(false, false);
-    }
-#undef DQ_LAUNCH_D
+    if (add)
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, true>), grid, block, 0, stream, src, dst, nsc, vec, arg);
+    else
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false>), grid, block, 0, stream, src, dst, nsc, vec, arg);
     return hipGetLastError();
 }
 
