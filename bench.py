@@ -33,10 +33,10 @@ OVERHEAD_BITS = 0.5625  # hierarchical scale bytes per element, in bits
 
 # HBM bytes per launch of the compress kernel from two `rocprofv3 --pmc` runs of this script
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for
-# the --pmc-calibration copy kernel: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0.
+# the --pmc-calibration copy kernel: FETCH_SIZE x 1.999, WRITE_SIZE x 1.000.
 # key: (source dtype, nbits, strategy, elements)
 MEASURED_TRAFFIC_BYTES = {
-    ("fp32", 4, 2, 6553600): int((2.0 * 19237.0 + 1.0 * 3800.0) * 1024),
+    ("fp32", 4, 2, 6553600): int((25600.0 / 12806.7 * 19228.5 + 1.0 * 3800.0) * 1024),
 }
 
 
