@@ -1,0 +1,271 @@
+"""The baseline configurations at their real sizes: bit-exact against the oracle where the
+oracle finishes in seconds, and through size-independent properties beyond that
+(fused == split bytes, per-element error bound, oracle-checked slices -- tiles are
+independent, so any 256-aligned slice can be verified on its own)."""
+import math
+import threading
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, F32, TORCH_DT, bits_to_f32, to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _student_bucket(n, seed=0):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    z = torch.randn(n, generator=g, device=DEV)
+    chi = torch.randn(3, n, generator=g, device=DEV).square_().sum(0)
+    x = z / torch.sqrt(chi / 3.0) * 1e-3
+    idx = torch.randint(0, n, (max(1, n // 1000),), generator=g, device=DEV)
+    x[idx] *= 100.0
+    return x.contiguous()
+
+
+@pytest.mark.parametrize("src_dt", [F32, BF16])
+@pytest.mark.parametrize("nbits,strategy", [(4, 2), (8, 2), (4, 3), (8, 3)])
+def test_config2_bucket_bit_exact(capi, oracle, src_dt, nbits, strategy):
+    """25 MB bucket, Student-t with outliers: packed bytes and decoded values of the WHOLE bucket"""
+    n = 6553600
+    x = _student_bucket(n)
+    src = x if src_dt == F32 else x.to(torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    rnd = torch.rand(n, generator=g, device=DEV).to(torch.bfloat16)
+    nbytes = capi.required_bytes(n, nbits, 16, strategy)
+    enc = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    out = torch.empty_like(src)
+    capi.scaling_compress(src, enc, rnd, n, nbits, 16, strategy)
+    capi.scaling_decompress(enc, out, n, nbits, 16, strategy)
+    rnd_h = to_bits(rnd.float()) if src_dt == F32 else to_bits(rnd)
+    enc_o = oracle.scaling_compress(to_bits(src), rnd_h, n, nbits, 16, strategy, src_dt)
+    assert (enc.cpu().numpy() == enc_o).all()
+    dec_o = np.zeros(n, np.float32 if src_dt == F32 else np.uint16)
+    oracle.scaling_decompress(enc_o, dec_o, n, nbits, 16, strategy, src_dt)
+    assert (to_bits(out) == dec_o).all()
+    nmse = float(((out.double() - x.double()) ** 2).sum() / (x.double() ** 2).sum())
+    assert nmse < (2e-2 if nbits == 4 else 3e-4)
+
+
+def test_config1_rht_5bit_bit_exact(capi, oracle):
+    """2^20 N(0,1e-3^2): randDiag + blocked FWHT + 5-bit codes + bit-plane packing, and back"""
+    n = 1 << 20
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(n, generator=g, device=DEV) * 1e-3
+    rnd = torch.rand(n, generator=g, device=DEV).to(torch.bfloat16)
+    sign = torch.empty(n, device=DEV)
+    capi.rand_diag(sign, 0)
+    sign_o = oracle.rand_diag(n, 0)
+    assert (sign.cpu().numpy() == sign_o).all()
+    for kb in (10, 15, 20):
+        B, sc = 1 << kb, np.float32(1.0 / math.sqrt(1 << kb))
+        y = x.clone()
+        capi.rht_blocked(y, sign, B, float(sc), False)
+        y_o = oracle.rht_blocked(x.cpu().numpy(), sign_o, B, sc)
+        assert (y.cpu().numpy().view(np.uint32) == y_o.view(np.uint32)).all()
+        enc = torch.zeros(capi.required_bytes(n, 5, 16, 2), dtype=torch.uint8, device=DEV)
+        capi.scaling_compress(y, enc, rnd, n, 5, 16, 2)
+        enc_o = oracle.scaling_compress(y_o, to_bits(rnd.float()), n, 5, 16, 2, F32)
+        assert (enc.cpu().numpy() == enc_o).all()
+        z = torch.empty_like(y)
+        capi.scaling_decompress(enc, z, n, 5, 16, 2)
+        capi.rht_blocked(z, sign, B, float(sc), True)
+        dec_o = np.zeros(n, np.float32)
+        oracle.scaling_decompress(enc_o, dec_o, n, 5, 16, 2, F32)
+        z_o = oracle.rht_blocked(dec_o, sign_o, B, sc, inverse=True)
+        assert (z.cpu().numpy().view(np.uint32) == z_o.view(np.uint32)).all()
+        nmse = float(((z - x).double() ** 2).sum() / (x.double() ** 2).sum())
+        assert 2.5e-3 < nmse < 4.0e-3
+    # the reference-legal 5-bit packer: bit planes of 5-bit bins
+    bins = torch.randint(0, 32, (n,), generator=torch.Generator().manual_seed(3), dtype=torch.int32)
+    arr = torch.zeros(n // 32 * 5, dtype=torch.int32, device=DEV)
+    capi.bins_to_bits(bins.to(DEV), arr, 5)
+    assert (arr.cpu().numpy().view(np.uint32) == oracle.bins_to_bits(bins.numpy(), 5)).all()
+
+
+def test_config3_ring_chunk_bit_exact(capi, oracle):
+    """one fused reduce-scatter step on a GPT-2-small ring chunk (15,555,072 bf16 elements), 4-bit"""
+    n = 15555072
+    g = torch.Generator(device=DEV).manual_seed(4)
+    a = (torch.randn(n, generator=g, device=DEV) * 3e-3).to(torch.bfloat16)
+    b = (torch.randn(n, generator=g, device=DEV) * 7e-4).to(torch.bfloat16)
+    r1 = torch.rand(n, generator=g, device=DEV).to(torch.bfloat16)
+    r2 = torch.rand(n, generator=g, device=DEV).to(torch.bfloat16)
+    nbytes = capi.required_bytes(n, 4, 16, 2)
+    assert nbytes == 60762 * 146
+    recv = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    send = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(a, recv, r1, n, 4, 16, 2)
+    capi.scaling_dec_comp(recv, b, send, r2, n, 4, 16, 2)
+    recv_o = oracle.scaling_compress(to_bits(a), to_bits(r1), n, 4, 16, 2, BF16)
+    send_o = oracle.scaling_dec_comp(recv_o, to_bits(b), to_bits(r2), n, 4, 16, 2, BF16)
+    assert (recv.cpu().numpy() == recv_o).all() and (send.cpu().numpy() == send_o).all()
+
+
+@pytest.mark.parametrize("nbits", [2, 4, 5, 8])
+def test_config5_properties_at_2_pow_28(capi, oracle, nbits):
+    """1 GiB of fp32: fused == split, error bound, and oracle-checked slices"""
+    n = 1 << 28
+    g = torch.Generator(device=DEV).manual_seed(nbits)
+    x = torch.randn(n, generator=g, device=DEV) * 1e-3
+    rnd = torch.rand(n, generator=g, device=DEV).to(torch.bfloat16)
+    nbytes = capi.required_bytes(n, nbits, 16, 2)
+    rec = nbytes // (n // 256)
+    enc = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    out = torch.empty_like(x)
+    capi.scaling_compress(x, enc, rnd, n, nbits, 16, 2)
+    capi.scaling_decompress(enc, out, n, nbits, 16, 2)
+    # |x - decode| <= one quantisation step; the chunk's step is its absmax / R rounded UP to a multiple of
+    # the superchunk unit (superchunk absmax / R / 255), both carried in bf16 (relative 2^-7)
+    R = (1 << (nbits - 1)) - 1
+    cmax = x.abs().view(-1, 16).max(dim=1).values
+    smax = x.abs().view(-1, 256).max(dim=1).values.repeat_interleave(16)
+    step = (cmax / R + smax / R / 255) * (1 + 2 ** -7) + 2e-7
+    assert bool(((out - x).abs().view(-1, 16) <= step[:, None]).all())
+    del cmax, smax, step
+    # fused ring step == decompress_add + compress, byte for byte, over the whole GiB
+    inp = torch.randn(n, generator=g, device=DEV) * 1e-3
+    send = torch.zeros_like(enc)
+    capi.scaling_dec_comp(enc, inp, send, rnd, n, nbits, 16, 2)
+    inp2 = inp.clone()
+    capi.scaling_decompress(enc, inp2, n, nbits, 16, 2, add=True)
+    send2 = torch.zeros_like(enc)
+    capi.scaling_compress(inp2, send2, rnd, n, nbits, 16, 2)
+    assert torch.equal(send, send2)
+    del inp2, send2
+    # slices against the oracle: start, an odd tile in the middle, the very end
+    m = 256 * 1021
+    for off in (0, 256 * 524287, n - m):
+        sl = slice(off, off + m)
+        enc_o = oracle.scaling_compress(to_bits(x[sl]), to_bits(rnd[sl].float()), m, nbits, 16, 2, F32)
+        got = enc[off // 256 * rec: (off + m) // 256 * rec].cpu().numpy()
+        assert (got == enc_o).all()
+        dec_o = np.zeros(m, np.float32)
+        oracle.scaling_decompress(enc_o, dec_o, m, nbits, 16, 2, F32)
+        assert (to_bits(out[sl]).view(np.uint32) == dec_o.view(np.uint32)).all()
+
+
+def test_hadamard_2_pow_28_involution(capi):
+    """H(H(x)) = n x exactly on small integers; four passes over 1 GiB"""
+    n = 1 << 28
+    x = torch.randint(-2, 3, (n,), device=DEV).float()
+    y = x.clone()
+    capi.hadamard(y)
+    assert float(y[0]) == float(x.double().sum())
+    capi.hadamard(y)
+    assert torch.equal(y, x * n)
+
+
+def test_dynamic_bitrate_pipeline_matches_oracle(eden_utils, oracle):
+    """mean-centre -> q in {2,4,8} -> per-width compress/decompress -> add mean, one rank, against the
+    same steps done with oracle calls (Llama-like tensors with very different scales)"""
+    from dynamiq_sigcomm_artifact_amd import bitrate
+    from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import dynamic_bitrate_allreduce
+    n = 256 * 3000
+    g = torch.Generator().manual_seed(8)
+    scale = torch.exp(torch.randn(n // 256 // 100, 1, generator=g) * 1.5 + math.log(1e-3)).repeat_interleave(100 * 256)
+    x = (torch.randn(n, generator=g) * scale.reshape(-1)[:n]).to(torch.bfloat16)
+    params = {"d": {(0, 0): n * 4}, "world_size": 1, "rank": 0, "args": types.SimpleNamespace(aggregation_method="dynamiQ_aee")}
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    comps = {q: [Aee_Dynamic_Range_GPU_kern(q, 16, params, generator=gen)] for q in (2, 4, 8)}
+    # u from the CPU statistics
+    res_o, stats_o = oracle.superchunk_mean_center(to_bits(x), n, 1, BF16)
+    norms = torch.from_numpy(bits_to_f32(stats_o[1::2], BF16)).to(torch.bfloat16)
+    u, avg, _ = bitrate.dynamic_bitrate_binary_search_u([norms], 4.375)
+    outs, total, qbits = dynamic_bitrate_allreduce([x.to(DEV)], u, comps)
+    assert (to_bits(total.reshape(-1)) == stats_o).all()
+    q_cpu = bitrate.dynamic_bitrate_qbits(norms, u)
+    assert torch.equal(qbits.cpu(), q_cpu) and abs(float(q_cpu.float().mean()) - avg) < 1e-6
+    # oracle pipeline with the same random-pool offsets (first call of each compressor)
+    res2d = res_o.reshape(-1, 256).copy()
+    for q in (8, 4, 2):
+        idx = np.nonzero(q_cpu.numpy() == q)[0]
+        if idx.size == 0:
+            continue
+        grp = np.ascontiguousarray(res2d[idx].reshape(-1))
+        c = comps[q][0]
+        seed = ((q * 998244353) & 0xFFFFFFFF) * 671431 + 1000000007 & 0xFFFFFFFF
+        rows = c.randomized_vec_pool.shape[0]
+        randl = seed % (rows - grp.size // 16 - 1)
+        rnd = to_bits(c.randomized_vec_pool[randl:randl + grp.size // 16].reshape(-1))
+        enc = oracle.scaling_compress(grp, rnd, grp.size, q, 16, 2, BF16)
+        oracle.scaling_decompress(enc, grp, grp.size, q, 16, 2, BF16)
+        res2d[idx] = grp.reshape(-1, 256)
+    want = oracle.superchunk_add_mean_copy(res2d.reshape(-1), stats_o, n, BF16)
+    assert (to_bits(outs[0]) == want).all()
+
+
+def test_concurrent_streams_and_sub_buffers(capi, oracle):
+    """two host threads, two streams, tiles of one bucket at record-aligned offsets (the transport's call pattern)"""
+    n, tile = 256 * 4096, 256 * 512
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16)
+    rnd = torch.rand(n, generator=g).to(torch.bfloat16)
+    x_d, r_d = x.to(DEV), rnd.to(DEV)
+    nbytes = capi.required_bytes(n, 4, 16, 2)
+    rec_tile = capi.required_bytes(tile, 4, 16, 2)
+    enc = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    out = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(k):
+        try:
+            s = streams[k]
+            for t in range(k, n // tile, 2):
+                e = slice(t * tile, (t + 1) * tile)
+                p = enc[t * rec_tile:(t + 1) * rec_tile]
+                capi.scaling_compress(x_d[e], p, r_d[e], tile, 4, 16, 2, stream=s.cuda_stream)
+                capi.scaling_decompress(p, out[e], tile, 4, 16, 2, stream=s.cuda_stream)
+        except Exception as exc:  # pragma: no cover
+            errors.append(exc)
+
+    th = [threading.Thread(target=worker, args=(k,)) for k in (0, 1)]
+    [t.start() for t in th]
+    [t.join() for t in th]
+    torch.cuda.synchronize()
+    assert not errors
+    enc_o = oracle.scaling_compress(to_bits(x), to_bits(rnd), n, 4, 16, 2, BF16)
+    assert (enc.cpu().numpy() == enc_o).all()
+    dec_o = np.zeros(n, np.uint16)
+    oracle.scaling_decompress(enc_o, dec_o, n, 4, 16, 2, BF16)
+    assert (to_bits(out) == dec_o).all()
+
+
+def test_hip_graph_replay(capi):
+    """compress + fused step + decompress captured once and replayed: same bytes on every replay"""
+    n = 256 * 2048
+    x = (torch.randn(n, device=DEV) * 1e-3).to(torch.bfloat16)
+    inp = (torch.randn(n, device=DEV) * 1e-3).to(torch.bfloat16)
+    rnd = torch.rand(n, device=DEV).to(torch.bfloat16)
+    nbytes = capi.required_bytes(n, 4, 16, 3)
+    enc = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    send = torch.zeros_like(enc)
+    out = torch.zeros_like(x)
+
+    def run(stream=None):
+        capi.scaling_compress(x, enc, rnd, n, 4, 16, 3, stream=stream)
+        capi.scaling_dec_comp(enc, inp, send, rnd, n, 4, 16, 3, stream=stream)
+        capi.scaling_decompress(send, out, n, 4, 16, 3, stream=stream)
+
+    run()
+    torch.cuda.synchronize()
+    want_send, want_out = send.clone(), out.clone()
+    s = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        with torch.cuda.graph(graph, stream=s):
+            run(stream=s.cuda_stream)
+    for k in range(4):
+        send.zero_()
+        out.zero_()
+        x.add_(0)      # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(send, want_send) and torch.equal(out, want_out), k
