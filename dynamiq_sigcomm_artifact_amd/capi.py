@@ -20,6 +20,8 @@ EXPORTS = [
     "dq_scaling_required_bytes", "dq_scaling_check_common",
     "dq_init_lookup_table", "dq_mee_lookup_table",
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
+    "dq_group_plan_work_ints", "dq_group_plan",
+    "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
@@ -58,6 +60,16 @@ def lib():
         L.dq_scaling_decompress.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, i32]
         L.dq_scaling_dec_comp.restype = i32
         L.dq_scaling_dec_comp.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp]
+        L.dq_group_plan_work_ints.restype = i64
+        L.dq_group_plan_work_ints.argtypes = [i64]
+        L.dq_group_plan.restype = i32
+        L.dq_group_plan.argtypes = [vp, i64, vp, vp, i64, i32, vp]
+        L.dq_scaling_compress_rows.restype = i32
+        L.dq_scaling_compress_rows.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
+        L.dq_scaling_dec_comp_rows.restype = i32
+        L.dq_scaling_dec_comp_rows.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
+        L.dq_scaling_decompress_rows.restype = i32
+        L.dq_scaling_decompress_rows.argtypes = [vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, vp, i32]
         L.dq_superchunk_mean_center.restype = i32
         L.dq_superchunk_mean_center.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_superchunk_add_mean_copy.restype = i32
@@ -142,6 +154,41 @@ def scaling_decompress(src, dst, n, nbits, chunk_size, strategy, add=False, stre
 def scaling_dec_comp(recv, inp, send, rand_pool, n, nbits, chunk_size, strategy, stream=None):
     _check(lib().dq_scaling_dec_comp(recv.data_ptr(), inp.data_ptr(), send.data_ptr(), rand_pool.data_ptr(), n, nbits,
                                      chunk_size, _pair_code(inp, rand_pool), _dev(inp), strategy, _stream(stream)))
+
+
+def group_plan_work_ints(nsc):
+    return int(lib().dq_group_plan_work_ints(nsc))
+
+
+def group_plan(qbits, order, work, stream=None):
+    """qbits int64 [nsc] -> order int32 [nsc] (8-bit rows, then 4-bit, then 2-bit), work[0:3] = counts"""
+    if qbits.dtype != torch.int64 or order.dtype != torch.int32 or work.dtype != torch.int32:
+        raise RuntimeError("group_plan: qbits must be int64, order and work int32")
+    if order.numel() < qbits.numel():
+        raise RuntimeError("group_plan: order has fewer entries than qbits")
+    _check(lib().dq_group_plan(qbits.data_ptr(), qbits.numel(), order.data_ptr(), work.data_ptr(), work.numel(),
+                               _dev(qbits), _stream(stream)))
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def scaling_compress_rows(src, rows, dst, rand_pool, nrows, nbits, strategy, stream=None):
+    _check(lib().dq_scaling_compress_rows(src.data_ptr(), _ptr(rows), dst.data_ptr(), rand_pool.data_ptr(), nrows, nbits,
+                                          _pair_code(src, rand_pool), _dev(src), strategy, _stream(stream)))
+
+
+def scaling_dec_comp_rows(recv, inp, rows, send, rand_pool, nrows, nbits, strategy, stream=None):
+    _check(lib().dq_scaling_dec_comp_rows(recv.data_ptr(), inp.data_ptr(), _ptr(rows), send.data_ptr(),
+                                          rand_pool.data_ptr(), nrows, nbits, _pair_code(inp, rand_pool), _dev(inp),
+                                          strategy, _stream(stream)))
+
+
+def scaling_decompress_rows(src, dst, rows, stats, n_limit, nrows, nbits, strategy, add=False, stream=None):
+    _check(lib().dq_scaling_decompress_rows(src.data_ptr(), dst.data_ptr(), _ptr(rows), _ptr(stats), n_limit, nrows,
+                                            nbits, dtype_code(dst), _dev(dst), strategy, _stream(stream),
+                                            1 if add else 0))
 
 
 def superchunk_mean_center(src, residual, stats, n, world_size, superchunk_size=256, stream=None):

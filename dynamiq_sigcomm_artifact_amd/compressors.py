@@ -138,6 +138,37 @@ class _DynamicRangeGPUKern(object):
                                                self.strategy)
 
 
+    # ---- the same three steps over a list of superchunk indices (no counterpart in the reference:
+    # they stand for index_select + the call above + index_copy_, comm_hooks.py:1001-1011) ----
+
+    def compression_rows(self, full_tensor, rows, send_chunk):
+        """send record k = compressed superchunk rows[k] of full_tensor"""
+        nrows = rows.numel()
+        if nrows == 0:
+            return
+        rand_vec = self.rand_pool(nrows * 256, full_tensor.dtype)
+        self.eden_utils.scaling_compress_rows(full_tensor, rows, send_chunk, rand_vec, nrows, self.nbits,
+                                              self._stream(), self.strategy)
+
+    def dec_compression_rows(self, recv_chunk, full_tensor, rows, send_chunk):
+        nrows = rows.numel()
+        if nrows == 0:
+            return
+        rand_vec = self.rand_pool(nrows * 256, full_tensor.dtype)
+        self.eden_utils.scaling_dec_comp_rows(recv_chunk, full_tensor, rows, send_chunk, rand_vec, nrows, self.nbits,
+                                              self._stream(), self.strategy)
+
+    def decompression_rows(self, recv_chunk, full_output, rows, stats=None, n_limit=None):
+        """superchunk rows[k] of full_output = decoded record k (+ its mean from stats)"""
+        nrows = rows.numel()
+        if nrows == 0:
+            return
+        if n_limit is None:
+            n_limit = full_output.numel()
+        self.eden_utils.scaling_decompress_rows(recv_chunk, full_output, rows, stats, n_limit, nrows, self.nbits,
+                                                self._stream(), self.strategy)
+
+
 class Aee_Dynamic_Range_GPU_kern(_DynamicRangeGPUKern):
     """utils_aggregation.py:369-466 (hierarchical AEE, strategy 2)"""
     strategy = 2

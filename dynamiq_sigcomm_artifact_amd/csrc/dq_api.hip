@@ -273,6 +273,66 @@ int dq_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const voi
     return finish(dq::launch_generic_compress(inp, send, rand_pool, n, nbits, chunk_size, dtype, strategy, mp, s));
 }
 
+int64_t dq_group_plan_work_ints(int64_t nsc) { return nsc > 0 ? dq::group_plan_work_ints(nsc) : 4; }
+
+int dq_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work, int64_t work_ints, int device,
+                  dq_stream_t stream)
+{
+    if (!(nsc > 0) || nsc > (int64_t)0x7fffffff) return fail(DQ_ERR_N, "nsc must be in [1, 2^31)");
+    if (!qbits || !order || !work) return fail(DQ_ERR_NULL);
+    if (work_ints < dq::group_plan_work_ints(nsc)) return fail(DQ_ERR_SIZE, "work buffer is too small");
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_group_plan(qbits, nsc, order, work, static_cast<hipStream_t>(stream)));
+}
+
+static int check_rows(int64_t nrows, int nbits, int dtype, int strategy, bool rand)
+{
+    if (!(nrows > 0) || nrows > (int64_t)0x7fffffff) return DQ_ERR_N;
+    if (nbits < 2 || nbits > 8) return DQ_ERR_NBITS;
+    if (strategy != 2 && strategy != 3) return DQ_ERR_STRATEGY;
+    if (rand ? !dtype_rand_ok(dtype) : !dtype_ok(dtype)) return DQ_ERR_DTYPE;
+    if ((dtype & 0xf) == DQ_F16) return DQ_ERR_DTYPE;
+    return DQ_OK;
+}
+
+int dq_scaling_compress_rows(const void *src, const int32_t *rows, uint8_t *dst, const void *rand_pool, int64_t nrows,
+                             int nbits, int dtype, int device, int strategy, dq_stream_t stream)
+{
+    int rc = check_rows(nrows, nbits, dtype, strategy, true);
+    if (rc) return fail(rc);
+    if (!src || !dst || !rand_pool) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_hier16_compress_rows(src, nullptr, rows, dst, rand_pool, nrows, nbits, dtype, strategy == 3,
+                                                  mee_params(nbits), static_cast<hipStream_t>(stream)));
+}
+
+int dq_scaling_dec_comp_rows(const uint8_t *recv, const void *inp, const int32_t *rows, uint8_t *send,
+                             const void *rand_pool, int64_t nrows, int nbits, int dtype, int device, int strategy,
+                             dq_stream_t stream)
+{
+    int rc = check_rows(nrows, nbits, dtype, strategy, true);
+    if (rc) return fail(rc);
+    if (!recv || !inp || !send || !rand_pool) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_hier16_compress_rows(inp, recv, rows, send, rand_pool, nrows, nbits, dtype, strategy == 3,
+                                                  mee_params(nbits), static_cast<hipStream_t>(stream)));
+}
+
+int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *rows, const void *stats, int64_t n_limit,
+                               int64_t nrows, int nbits, int dtype, int device, int strategy, dq_stream_t stream,
+                               int add_original)
+{
+    int rc = check_rows(nrows, nbits, dtype, strategy, false);
+    if (rc) return fail(rc);
+    if (!src || !dst) return fail(DQ_ERR_NULL);
+    if (!(n_limit > 0)) return fail(DQ_ERR_N, "n_limit");
+    if (add_original && stats) return fail(DQ_ERR_SIZE, "stats cannot be combined with add_original");
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_hier16_decompress_rows(src, dst, rows, stats, n_limit, nrows, nbits, dtype, strategy == 3,
+                                                    mee_params(nbits), add_original, static_cast<hipStream_t>(stream)));
+}
+
 int dq_superchunk_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size,
                               int superchunk_size, int dtype, int device, dq_stream_t stream)
 {

@@ -29,6 +29,23 @@ hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t 
                                   const void *rnd, int64_t n, int nbits, int dtype, bool mee,
                                   const MeeParams &mp, hipStream_t stream);
 
+// the same kernels over a list of superchunk indices: record k <-> superchunk rows[k] of the
+// element buffer; recv != null makes compress the fused decode-accumulate-recompress step;
+// stats != null adds the destination superchunk's mean after decoding; elements >= limit are
+// not written
+hipError_t launch_hier16_compress_rows(const void *src, const uint8_t *recv, const int32_t *rows,
+                                       uint8_t *dst, const void *rnd, int64_t nrows, int nbits,
+                                       int dtype, bool mee, const MeeParams &mp, hipStream_t stream);
+hipError_t launch_hier16_decompress_rows(const uint8_t *src, void *dst, const int32_t *rows,
+                                         const void *stats, int64_t limit, int64_t nrows, int nbits,
+                                         int dtype, bool mee, const MeeParams &mp, int add,
+                                         hipStream_t stream);
+
+// stable partition of superchunk indices by bit width (dq_grouping.hip)
+int64_t group_plan_work_ints(int64_t nsc);
+hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work,
+                             hipStream_t stream);
+
 // superchunk mean-centring (dq_superchunk.hip)
 hipError_t launch_mean_center(const void *src, void *residual, void *stats, int64_t n,
                               int world_size, int dtype, hipStream_t stream);

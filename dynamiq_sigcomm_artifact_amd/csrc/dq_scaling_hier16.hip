@@ -81,9 +81,11 @@ template <> struct Raw16<DQ_BF16> {
     }
     __device__ __forceinline__ void load(const void *p, int64_t e, bool vec)
     {
-        const uint16_t *h = static_cast<const uint16_t *>(p) + e;
+        // the unaligned path goes through volatile accesses so that the compiler cannot fold the two
+        // paths into one narrow-load sequence
+        const volatile uint16_t *h = static_cast<const volatile uint16_t *>(p) + e;
         if (vec) {
-            const uint4 *q = reinterpret_cast<const uint4 *>(h);
+            const uint4 *q = reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(p) + e);
             uint4 a = q[0], b = q[1];
             w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
         } else {
@@ -93,9 +95,9 @@ template <> struct Raw16<DQ_BF16> {
     }
     __device__ __forceinline__ void store(void *p, int64_t e, bool vec) const
     {
-        uint16_t *h = static_cast<uint16_t *>(p) + e;
+        volatile uint16_t *h = static_cast<volatile uint16_t *>(p) + e;
         if (vec) {
-            uint4 *q = reinterpret_cast<uint4 *>(h);
+            uint4 *q = reinterpret_cast<uint4 *>(static_cast<uint16_t *>(p) + e);
             q[0] = make_uint4(w[0], w[1], w[2], w[3]);
             q[1] = make_uint4(w[4], w[5], w[6], w[7]);
         } else {
@@ -141,9 +143,9 @@ template <> struct Raw16<DQ_F32> {
     }
     __device__ __forceinline__ void load(const void *p, int64_t e, bool vec)
     {
-        const uint32_t *f = static_cast<const uint32_t *>(p) + e;
+        const volatile uint32_t *f = static_cast<const volatile uint32_t *>(p) + e;
         if (vec) {
-            const uint4 *q = reinterpret_cast<const uint4 *>(f);
+            const uint4 *q = reinterpret_cast<const uint4 *>(static_cast<const uint32_t *>(p) + e);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 uint4 t = q[k];
@@ -156,9 +158,9 @@ template <> struct Raw16<DQ_F32> {
     }
     __device__ __forceinline__ void store(void *p, int64_t e, bool vec) const
     {
-        uint32_t *f = static_cast<uint32_t *>(p) + e;
+        volatile uint32_t *f = static_cast<volatile uint32_t *>(p) + e;
         if (vec) {
-            uint4 *q = reinterpret_cast<uint4 *>(f);
+            uint4 *q = reinterpret_cast<uint4 *>(static_cast<uint32_t *>(p) + e);
 #pragma unroll
             for (int k = 0; k < 4; k++) q[k] = make_uint4(w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
         } else {
@@ -412,11 +414,14 @@ constexpr uint32_t kFastMaxBits = 0x71800000u; // 2^100
 
 // ---- kernels ------------------------------------------------------------------------------------
 
-// compress (FUSED = false) or decode-accumulate-recompress (FUSED = true); workgroup = one wave = one tile
+// compress (FUSED = false) or decode-accumulate-recompress (FUSED = true); workgroup = one wave = one tile.
+// Record k of the packed streams (and row k of rnd) belongs to superchunk rows[k] of src
+// (to superchunk k when rows is null).
 template <int DT, int RDT, int NBITS, bool MEE, bool FUSED>
 __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restrict__ src, const uint8_t *__restrict__ recv,
                                                             uint8_t *__restrict__ dst, const void *__restrict__ rnd,
-                                                            int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
+                                                            const int32_t *__restrict__ rows, int64_t nsc, int vec,
+                                                            MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
     __shared__ __attribute__((aligned(16))) uint8_t win_out[RC::WIN];
@@ -427,16 +432,17 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     const int row = lane >> 4, j = lane & 15;
     const int64_t sc0 = (int64_t)blockIdx.x * kRowsPerWave;
     if (sc0 >= nsc) return;
-    const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-    const bool active = row < rows;
-    const int total = rows * RC::REC;
+    const int rows_here = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+    const bool active = row < rows_here;
+    const int total = rows_here * RC::REC;
 
     // all global loads of the tile are issued before anything waits on them
     Raw16<DT> v;
     Raw16<RDT> r;
     if (active) {
-        v.load(src, (sc0 * 16 + lane) * 16, vec & 1);
         r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
+        const int64_t sc_src = rows ? (int64_t)rows[sc0 + row] : sc0 + row;
+        v.load(src, (sc_src * 16 + j) * 16, vec & 1);
     } else {
         v.zero();
         r.zero();
@@ -490,12 +496,19 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
 // 64*k + lane) then touch eight distinct bank groups per eight lanes
 __device__ __forceinline__ int swz(int s) { return s ^ ((s >> 3) & 7); }
 
+// Record k decodes into superchunk rows[k] of dst (superchunk k when rows is null). With stats
+// (interleaved bf16 pairs, the mean first) the stored value is T(float(T(decoded)) + mean of the
+// destination superchunk); elements at or beyond `limit` are not written.
 template <int DT, int NBITS, bool MEE, bool ADD>
 __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
+                                                              const int32_t *__restrict__ rows,
+                                                              const uint16_t *__restrict__ stats, int64_t limit,
                                                               int64_t nsc, int vec, MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
     constexpr int S = Raw16<DT>::kSlots;
+    constexpr int ESZ = DT == DQ_F32 ? 4 : 2;
+    constexpr int EP = 16 / ESZ; // elements per 16-byte slot
     __shared__ __attribute__((aligned(16))) uint8_t win_in[RC::WIN];
     __shared__ __attribute__((aligned(16))) uint4 tile_out[64 * S];
     __shared__ float table[MEE ? (1 << NBITS) : 1];
@@ -504,14 +517,28 @@ __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__
     const int row = lane >> 4, j = lane & 15;
     const int64_t sc0 = (int64_t)blockIdx.x * kRowsPerWave;
     if (sc0 >= nsc) return;
-    const int rows = (int)min((int64_t)kRowsPerWave, nsc - sc0);
-    const bool active = row < rows;
-    const int total = rows * RC::REC;
-    const int64_t e0 = sc0 * 256; // first element of the tile
+    const int rows_here = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+    const bool active = row < rows_here;
+    const int total = rows_here * RC::REC;
 
     const WinRegs wr = window_fetch(src + sc0 * RC::REC, total, lane);
+    // destination superchunk of this lane's chunk, and of the slots this lane stores after the transpose
+    int64_t d_own = sc0 + row;
+    int64_t d_slot[S];
+#pragma unroll
+    for (int k = 0; k < S; k++) d_slot[k] = sc0 + (64 * k + lane) / (16 * S);
+    if (rows) {
+        if (active) d_own = rows[sc0 + row];
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const int rr = (64 * k + lane) / (16 * S);
+            if (rr < rows_here) d_slot[k] = rows[sc0 + rr];
+        }
+    }
     Raw16<DT> acc;
-    if (ADD && active) acc.load(dst, e0 + lane * 16, vec);
+    if (ADD && active) acc.load(dst, d_own * 256 + j * 16, vec);
+    float mean = 0.0f;
+    if (stats && active) mean = bf16_bits_to_f32(stats[2 * d_own]);
     if (MEE) {
         for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
     }
@@ -531,25 +558,60 @@ __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__
         }
         chunk_decode<NBITS, MEE, ADD>(cw, cq, ub, table, t);
         out.set(t);
+        if (stats) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = out.get(i) + mean;
+            out.set(t);
+        }
     } else {
         out.zero();
     }
+    char *dbytes = static_cast<char *>(dst);
     if (vec) {
-        // transpose through LDS so that every store instruction writes 1 KiB contiguously
+        // transpose through LDS so that every store instruction writes whole superchunks contiguously
         if (active) {
 #pragma unroll
             for (int k = 0; k < S; k++) tile_out[swz(S * lane + k)] = out.slot(k);
         }
         wave_lds_sync();
-        const int nslots = rows * 16 * S;
-        uint4 *g = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + e0 * (DT == DQ_F32 ? 4 : 2));
+        const int nslots = rows_here * 16 * S;
 #pragma unroll
         for (int k = 0; k < S; k++) {
             const int s = 64 * k + lane;
-            if (s < nslots) g[s] = tile_out[swz(s)];
+            if (s < nslots) {
+                const int64_t e = d_slot[k] * 256 + (s % (16 * S)) * EP;
+                const uint4 val = tile_out[swz(s)];
+                if (e + EP <= limit) {
+                    *reinterpret_cast<uint4 *>(dbytes + e * ESZ) = val;
+                } else {
+                    const uint32_t part[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+                    for (int i = 0; i < EP; i++) {
+                        if (e + i < limit) {
+                            if (DT == DQ_F32)
+                                reinterpret_cast<uint32_t *>(dbytes)[e + i] = part[i];
+                            else
+                                reinterpret_cast<uint16_t *>(dbytes)[e + i] = (uint16_t)(part[i >> 1] >> (16 * (i & 1)));
+                        }
+                    }
+                }
+            }
         }
     } else if (active) {
-        out.store(dst, e0 + lane * 16, false);
+        const int64_t e = d_own * 256 + j * 16;
+        if (e + 16 <= limit) {
+            out.store(dst, e, false);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                if (e + i < limit) {
+                    if (DT == DQ_F32)
+                        reinterpret_cast<uint32_t *>(dbytes)[e + i] = out.w[i];
+                    else
+                        reinterpret_cast<uint16_t *>(dbytes)[e + i] = (uint16_t)(out.w[i >> 1] >> (16 * (i & 1)));
+                }
+            }
+        }
     }
 }
 
@@ -570,29 +632,30 @@ static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t
 static inline unsigned grid_for(int64_t nsc) { return (unsigned)((nsc + kRowsPerWave - 1) / kRowsPerWave); }
 
 template <int DT, int RDT, int NBITS, bool MEE>
-static hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, int64_t nsc,
-                               bool fused, const MeeParams &mp, hipStream_t stream)
+static hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, const int32_t *rows,
+                               int64_t nsc, bool fused, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
     dim3 grid(grid_for(nsc)), block(64);
     const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
     if (fused)
-        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, rows, nsc, vec, arg);
     else
-        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, rows, nsc, vec, arg);
     return hipGetLastError();
 }
 
 template <int DT, int NBITS, bool MEE>
-static hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nsc, int add, const MeeParams &mp, hipStream_t stream)
+static hipError_t run_decompress(const uint8_t *src, void *dst, const int32_t *rows, const uint16_t *stats, int64_t limit,
+                                 int64_t nsc, int add, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
     dim3 grid(grid_for(nsc)), block(64);
     const int vec = aligned16(dst) ? 1 : 0;
     if (add)
-        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, true>), grid, block, 0, stream, src, dst, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, true>), grid, block, 0, stream, src, dst, rows, stats, limit, nsc, vec, arg);
     else
-        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false>), grid, block, 0, stream, src, dst, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false>), grid, block, 0, stream, src, dst, rows, stats, limit, nsc, vec, arg);
     return hipGetLastError();
 }
 
@@ -610,41 +673,63 @@ static hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nsc, int
 
 #define DQ_COMMA ,
 
-static hipError_t dispatch_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, int64_t nsc,
-                                    bool fused, int nbits, int dtype, bool mee, const MeeParams &mp, hipStream_t stream)
+static hipError_t dispatch_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd,
+                                    const int32_t *rows, int64_t nsc, bool fused, int nbits, int dtype, bool mee,
+                                    const MeeParams &mp, hipStream_t stream)
 {
     const bool rb16 = (dtype & DQ_RAND_BF16) != 0;
     dtype &= 0xf;
     if (dtype == DQ_BF16) {
-        DQ_NBITS_MEE(run_compress, DQ_BF16 DQ_COMMA DQ_BF16, src, recv, dst, rnd, nsc, fused, mp, stream)
+        DQ_NBITS_MEE(run_compress, DQ_BF16 DQ_COMMA DQ_BF16, src, recv, dst, rnd, rows, nsc, fused, mp, stream)
     } else if (rb16) {
-        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_BF16, src, recv, dst, rnd, nsc, fused, mp, stream)
+        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_BF16, src, recv, dst, rnd, rows, nsc, fused, mp, stream)
     } else {
-        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_F32, src, recv, dst, rnd, nsc, fused, mp, stream)
+        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_F32, src, recv, dst, rnd, rows, nsc, fused, mp, stream)
     }
 }
 
 hipError_t launch_hier16_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n, int nbits, int dtype,
                                   bool mee, const MeeParams &mp, hipStream_t stream)
 {
-    return dispatch_compress(src, nullptr, dst, rnd, n / 256, false, nbits, dtype, mee, mp, stream);
+    return dispatch_compress(src, nullptr, dst, rnd, nullptr, n / 256, false, nbits, dtype, mee, mp, stream);
 }
 
 hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t *send, const void *rnd, int64_t n,
                                   int nbits, int dtype, bool mee, const MeeParams &mp, hipStream_t stream)
 {
-    return dispatch_compress(inp, recv, send, rnd, n / 256, true, nbits, dtype, mee, mp, stream);
+    return dispatch_compress(inp, recv, send, rnd, nullptr, n / 256, true, nbits, dtype, mee, mp, stream);
+}
+
+hipError_t launch_hier16_compress_rows(const void *src, const uint8_t *recv, const int32_t *rows, uint8_t *dst,
+                                       const void *rnd, int64_t nrows, int nbits, int dtype, bool mee,
+                                       const MeeParams &mp, hipStream_t stream)
+{
+    return dispatch_compress(src, recv, dst, rnd, rows, nrows, recv != nullptr, nbits, dtype, mee, mp, stream);
+}
+
+static hipError_t dispatch_decompress(const uint8_t *src, void *dst, const int32_t *rows, const uint16_t *stats,
+                                      int64_t limit, int64_t nsc, int nbits, int dtype, bool mee, const MeeParams &mp,
+                                      int add, hipStream_t stream)
+{
+    if ((dtype & 0xf) == DQ_BF16) {
+        DQ_NBITS_MEE(run_decompress, DQ_BF16, src, dst, rows, stats, limit, nsc, add, mp, stream)
+    } else {
+        DQ_NBITS_MEE(run_decompress, DQ_F32, src, dst, rows, stats, limit, nsc, add, mp, stream)
+    }
 }
 
 hipError_t launch_hier16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype, bool mee,
                                     const MeeParams &mp, int add, hipStream_t stream)
 {
-    const int64_t nsc = n / 256;
-    if ((dtype & 0xf) == DQ_BF16) {
-        DQ_NBITS_MEE(run_decompress, DQ_BF16, src, dst, nsc, add, mp, stream)
-    } else {
-        DQ_NBITS_MEE(run_decompress, DQ_F32, src, dst, nsc, add, mp, stream)
-    }
+    return dispatch_decompress(src, dst, nullptr, nullptr, n, n / 256, nbits, dtype, mee, mp, add, stream);
+}
+
+hipError_t launch_hier16_decompress_rows(const uint8_t *src, void *dst, const int32_t *rows, const void *stats,
+                                         int64_t limit, int64_t nrows, int nbits, int dtype, bool mee,
+                                         const MeeParams &mp, int add, hipStream_t stream)
+{
+    return dispatch_decompress(src, dst, rows, static_cast<const uint16_t *>(stats), limit, nrows, nbits, dtype, mee, mp,
+                               add, stream);
 }
 
 } // namespace dq

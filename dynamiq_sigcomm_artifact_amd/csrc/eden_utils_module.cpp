@@ -252,6 +252,112 @@ int64_t scaling_required_bytes(int64_t n, int nbits, int chunk_size, int strateg
     return dq_scaling_required_bytes(n, nbits, chunk_size, strategy);
 }
 
+// ---- dynamic-bitrate groups (additions; see include/dynamiq_eden.h) -----------------
+
+void check_rows_tensor(const torch::Tensor &rows, int64_t nrows)
+{
+    TORCH_CHECK(rows.device().type() == torch::kCUDA, "rows must be a CUDA tensor");
+    TORCH_CHECK(rows.dtype() == torch::kInt32, "rows must be torch.int32");
+    TORCH_CHECK(rows.is_contiguous(), "rows must be contiguous");
+    TORCH_CHECK(rows.numel() >= nrows, "rows has fewer than nrows entries");
+}
+
+void check_rows_common(int64_t nrows, int nbits, int strategy)
+{
+    TORCH_CHECK(nrows > 0, "nrows must be positive");
+    TORCH_CHECK(nbits >= 2 && nbits <= 8, "nbits must be in [2, 8]");
+    TORCH_CHECK(strategy == 2 || strategy == 3, "strategy must be 2 (hierarchical AEE) or 3 (hierarchical MEE)");
+}
+
+torch::Tensor group_plan(torch::Tensor qbits, torch::Tensor order, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(qbits.device().type() == torch::kCUDA, "qbits must be a CUDA tensor");
+    TORCH_CHECK(order.device().type() == torch::kCUDA, "order must be a CUDA tensor");
+    TORCH_CHECK(qbits.dtype() == torch::kInt64, "qbits must be torch.int64");
+    TORCH_CHECK(order.dtype() == torch::kInt32, "order must be torch.int32");
+    TORCH_CHECK(qbits.is_contiguous() && order.is_contiguous(), "qbits and order must be contiguous");
+    const int64_t nsc = qbits.numel();
+    TORCH_CHECK(nsc > 0, "qbits must not be empty");
+    TORCH_CHECK(order.numel() >= nsc, "order has fewer entries than qbits");
+    auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
+    check_status(dq_group_plan(qbits.data_ptr<int64_t>(), nsc, order.data_ptr<int32_t>(), work.data_ptr<int32_t>(),
+                               work.numel(), qbits.device().index(), as_stream(stream_p)),
+                 "group_plan");
+    return work.slice(0, 0, 4);
+}
+
+void scaling_compress_rows(torch::Tensor src, torch::Tensor rows, torch::Tensor dst, torch::Tensor rand_pool, int64_t nrows,
+                           int nbits, uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(rand_pool.device().type() == torch::kCUDA, "rand_pool must be a CUDA tensor");
+    TORCH_CHECK(src.scalar_type() == torch::kBFloat16 || src.scalar_type() == torch::kFloat32, "input must be torch.bfloat16 or torch.float32");
+    TORCH_CHECK(dst.dtype() == torch::kUInt8, "output must be torch.uint8");
+    const bool mixed = src.scalar_type() == torch::kFloat32 && rand_pool.scalar_type() == torch::kBFloat16;
+    TORCH_CHECK(mixed || rand_pool.dtype() == src.dtype(), "rand_pool dtype must match input dtype");
+    TORCH_CHECK(src.is_contiguous() && dst.is_contiguous() && rand_pool.is_contiguous(), "buffers must be contiguous");
+    check_rows_common(nrows, nbits, strategy);
+    check_rows_tensor(rows, nrows);
+    TORCH_CHECK(dst.numel() >= dq_scaling_required_bytes(nrows * 256, nbits, 16, strategy), "output buffer is too small");
+    TORCH_CHECK(rand_pool.numel() >= nrows * 256, "rand_pool has fewer than 256 * nrows elements");
+    check_status(dq_scaling_compress_rows(src.data_ptr(), rows.data_ptr<int32_t>(), dst.data_ptr<uint8_t>(), rand_pool.data_ptr(),
+                                          nrows, nbits, dq_dtype_of(src.scalar_type()) | (mixed ? DQ_RAND_BF16 : 0),
+                                          src.device().index(), strategy, as_stream(stream_p)),
+                 "scaling_compress_rows");
+}
+
+void scaling_dec_comp_rows(torch::Tensor recv, torch::Tensor inp, torch::Tensor rows, torch::Tensor send, torch::Tensor rand_pool,
+                           int64_t nrows, int nbits, uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(recv.device().type() == torch::kCUDA && inp.device().type() == torch::kCUDA &&
+                    send.device().type() == torch::kCUDA && rand_pool.device().type() == torch::kCUDA,
+                "all buffers must be CUDA tensors");
+    TORCH_CHECK(recv.dtype() == torch::kUInt8, "recv must be torch.uint8");
+    TORCH_CHECK(send.dtype() == torch::kUInt8, "send must be torch.uint8");
+    TORCH_CHECK(inp.scalar_type() == torch::kBFloat16 || inp.scalar_type() == torch::kFloat32, "inp must be torch.bfloat16 or torch.float32");
+    const bool mixed = inp.scalar_type() == torch::kFloat32 && rand_pool.scalar_type() == torch::kBFloat16;
+    TORCH_CHECK(mixed || rand_pool.dtype() == inp.dtype(), "rand_pool dtype must match inp dtype");
+    TORCH_CHECK(recv.is_contiguous() && inp.is_contiguous() && send.is_contiguous() && rand_pool.is_contiguous(), "buffers must be contiguous");
+    check_rows_common(nrows, nbits, strategy);
+    check_rows_tensor(rows, nrows);
+    const int64_t required_bytes = dq_scaling_required_bytes(nrows * 256, nbits, 16, strategy);
+    TORCH_CHECK(recv.numel() >= required_bytes, "recv buffer is too small");
+    TORCH_CHECK(send.numel() >= required_bytes, "send buffer is too small");
+    TORCH_CHECK(rand_pool.numel() >= nrows * 256, "rand_pool has fewer than 256 * nrows elements");
+    check_status(dq_scaling_dec_comp_rows(recv.data_ptr<uint8_t>(), inp.data_ptr(), rows.data_ptr<int32_t>(), send.data_ptr<uint8_t>(),
+                                          rand_pool.data_ptr(), nrows, nbits,
+                                          dq_dtype_of(inp.scalar_type()) | (mixed ? DQ_RAND_BF16 : 0), inp.device().index(),
+                                          strategy, as_stream(stream_p)),
+                 "scaling_dec_comp_rows");
+}
+
+void scaling_decompress_rows(torch::Tensor src, torch::Tensor dst, torch::Tensor rows, c10::optional<torch::Tensor> stats,
+                             int64_t n_limit, int64_t nrows, int nbits, uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(src.dtype() == torch::kUInt8, "input must be torch.uint8");
+    TORCH_CHECK(dst.scalar_type() == torch::kBFloat16 || dst.scalar_type() == torch::kFloat32, "output must be torch.bfloat16 or torch.float32");
+    TORCH_CHECK(src.is_contiguous() && dst.is_contiguous(), "buffers must be contiguous");
+    check_rows_common(nrows, nbits, strategy);
+    check_rows_tensor(rows, nrows);
+    TORCH_CHECK(src.numel() >= dq_scaling_required_bytes(nrows * 256, nbits, 16, strategy), "input buffer is too small");
+    TORCH_CHECK(n_limit > 0 && n_limit <= dst.numel(), "n_limit must be in (0, output elements]");
+    const void *stats_ptr = nullptr;
+    if (stats.has_value()) {
+        TORCH_CHECK(stats->device().type() == torch::kCUDA, "stats must be a CUDA tensor");
+        TORCH_CHECK(stats->dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+        TORCH_CHECK(stats->is_contiguous(), "stats must be contiguous");
+        TORCH_CHECK(stats->numel() >= 2 * ((n_limit + 255) / 256), "stats buffer is too small");
+        stats_ptr = stats->data_ptr();
+    }
+    check_status(dq_scaling_decompress_rows(src.data_ptr<uint8_t>(), dst.data_ptr(), rows.data_ptr<int32_t>(), stats_ptr, n_limit,
+                                            nrows, nbits, dq_dtype_of(dst.scalar_type()), dst.device().index(), strategy,
+                                            as_stream(stream_p), 0),
+                 "scaling_decompress_rows");
+}
+
 // ---- superchunk ops ---------------------------------------------------------------
 
 void superchunk_mean_center(torch::Tensor src, torch::Tensor residual, torch::Tensor stats, int n, int world_size,
@@ -376,5 +482,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("rht_blocked", &rht_blocked, "in-place blocked randomized Hadamard transform", py::arg("vec"), py::arg("sign"), py::arg("block"), py::arg("scale"), py::arg("inverse") = false, py::arg("stream_p") = 0);
     modul.def("rand_diag", &rand_diag, "EDEN's seeded +-1 diagonal", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
+    modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width; returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
+    modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("scaling_decompress_rows", &scaling_decompress_rows, "decode consecutive records into the superchunks rows[k] of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("rows"), py::arg("stats"), py::arg("n_limit"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("abi_version", &abi_version, "version string of libdynamiq_eden.so");
 }

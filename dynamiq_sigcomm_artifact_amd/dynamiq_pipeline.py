@@ -16,7 +16,8 @@ import torch
 
 from . import bitrate
 from .compressors import superchunk_add_mean_copy, superchunk_mean_center
-from .ring_sim import ring_allreduce
+from . import load_eden_utils
+from .ring_sim import ring_allreduce, ring_allreduce_rows
 
 SUPERCHUNK = 256
 
@@ -59,4 +60,54 @@ def dynamic_bitrate_allreduce(rank_vecs, u, compressors, out=None):
     outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
     for r in range(W):
         superchunk_add_mean_copy(residuals[r], outs[r], total, n, SUPERCHUNK)
+    return outs, total, qbits
+
+
+def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=None):
+    """Same inputs, same results (bit for bit) as dynamic_bitrate_allreduce, with the gather, the scatter
+    and the final mean add folded into the codec kernels: one device-side partition of the superchunk
+    indices by width (a single 16-byte read-back for the three group sizes, in place of three
+    torch.nonzero), no group tensors, no index_select / index_copy_ / superchunk_add_mean_copy passes."""
+    eu = load_eden_utils()
+    W = len(rank_vecs)
+    n = rank_vecs[0].numel()
+    nsc = (n + SUPERCHUNK - 1) // SUPERCHUNK
+    dev, dt = rank_vecs[0].device, rank_vecs[0].dtype
+    if work is None:
+        work = {}
+    key = (nsc, dt, W)
+    if work.get("key") != key:
+        work["key"] = key
+        work["residuals"] = [torch.empty(nsc * SUPERCHUNK, dtype=dt, device=dev) for _ in range(W)]
+        work["stats"] = [torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev) for _ in range(W)]
+        work["order"] = torch.empty(nsc, dtype=torch.int32, device=dev)
+    residuals, stats, order = work["residuals"], work["stats"], work["order"]
+    stream = torch.cuda.current_stream().cuda_stream
+    for r in range(W):
+        superchunk_mean_center(rank_vecs[r], residuals[r], stats[r], n, W, SUPERCHUNK)
+    total = stats[0] if W == 1 else stats[0].clone()
+    for r in range(1, W):
+        total.add_(stats[r])
+    qbits = bitrate.dynamic_bitrate_qbits(total[:, 1], u)
+    counts = eu.group_plan(qbits, order, stream).tolist()
+    assert counts[3] == 0, "bit widths outside {2, 4, 8}"
+
+    outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
+    start = 0
+    for q, cnt in zip((8, 4, 2), counts[:3]):
+        if cnt == 0:
+            continue
+        rows = order[start:start + cnt]
+        start += cnt
+        comps = compressors[q]
+        if W == 1:
+            c = comps[0]
+            send = work.get(("send", q))
+            need = c.compressed_numel(cnt * SUPERCHUNK)
+            if send is None or send.numel() < need:
+                send = work[("send", q)] = torch.empty(need, dtype=torch.uint8, device=dev)
+            c.compression_rows(residuals[0], rows, send)
+            c.decompression_rows(send, outs[0], rows, total, n)
+        else:
+            ring_allreduce_rows(residuals, rows, comps, outs, total, n)
     return outs, total, qbits

@@ -20,7 +20,7 @@ import torch
 
 from . import bitrate, capi
 from .compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
-from .dynamiq_pipeline import dynamic_bitrate_allreduce
+from .dynamiq_pipeline import dynamic_bitrate_allreduce, dynamic_bitrate_allreduce_grouped
 from .ring_sim import ring_allreduce, split_chunks
 
 HBM_PEAK = 8000.0  # GB/s
@@ -151,6 +151,32 @@ def config3(dev, n=124439808, W=8):
                   step_GBps_algorithmic=round((2 + 2 + 2 * pb) * m / t / 1e3, 1),
                   step_frac_hbm=round((2 + 2 + 2 * pb) * m / t / 1e3 / HBM_PEAK, 4))
             del vecs, comps
+    # "5 bits" as the dynamic {2, 4, 8} mix (target 5 - 0.625 code bits): mean-centre, allocate, one grouped ring per width
+    target = 5.0 - bitrate.DYNAMIC_BITRATE_HEADROOM
+    from .compressors import superchunk_mean_center
+    nsc = npad // 256
+    norms = torch.zeros(nsc, dtype=torch.bfloat16, device=dev)
+    res = torch.empty(npad, dtype=torch.bfloat16, device=dev)
+    st = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
+    for r in range(W):
+        superchunk_mean_center(grads[r], res, st, npad, W, 256)
+        norms += st[:, 1]
+    del res, st
+    u, avg_bits, _ = bitrate.dynamic_bitrate_binary_search_u([norms], target)
+    for cls, name in ((Aee_Dynamic_Range_GPU_kern, "aee"), (Mee_Dynamic_Range_GPU_kern, "mee")):
+        gen = torch.Generator(device=dev).manual_seed(7)
+        comps = {q: [cls(q, 16, _params(npad, W, r), generator=gen) for r in range(W)] for q in (2, 4, 8)}
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        outs, _, qbits = dynamic_bitrate_allreduce_grouped(grads, u, comps)
+        e.record()
+        e.synchronize()
+        same = all(torch.equal(outs[0], v) for v in outs[1:])
+        _emit(config=3, world=W, elements_per_rank=n, nbits="dynamic{2,4,8}", method=name, u=u,
+              avg_code_bits=float(qbits.float().mean()), nmse_vs_fp64_mean=_nmse(exact / W, outs[0]),
+              ranks_identical=same, pipeline_total_ms=round(s.elapsed_time(e), 3))
+        del outs, comps
 
 
 LLAMA3_8B = [("embed", 128256 * 4096)] + [
@@ -196,32 +222,37 @@ def config4(dev, limit=None):
         superchunk_mean_center(x, res, st, n, 1, 256)
         norms_list.append(st[:, 1].clone())
     u, avg_bits, delta = bitrate.dynamic_bitrate_binary_search_u(norms_list, target)
-    # pass 2: quantise
+    # pass 2: quantise, with the reference's op sequence and with the gather/scatter folded into the kernels
     for cls, name in ((Aee_Dynamic_Range_GPU_kern, "aee"), (Mee_Dynamic_Range_GPU_kern, "mee")):
-        gen = torch.Generator(device=dev).manual_seed(3)
-        comps = {q: [cls(q, 16, _params(6553600 * 8, 1, 0), generator=gen)] for q in (2, 4, 8)}
-        num = den = 0.0
-        bits = elems = 0
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        gpu_ms = 0.0
-        nb = 0
-        for b in _llama_buckets(dev, limit=limit):
-            x = b.to(torch.bfloat16)
-            s.record()
-            outs, _, qbits = dynamic_bitrate_allreduce([x], u, comps)
-            e.record()
-            e.synchronize()
-            gpu_ms += s.elapsed_time(e)
-            num += float(((outs[0].double() - b.double()) ** 2).sum())
-            den += float((b.double() ** 2).sum())
-            bits += int(qbits.sum())
-            elems += qbits.numel()
-            nb += 1
-        _emit(config=4, method=name, buckets=nb, elements=elems * 256, target_avg_bits=target, u=u,
-              search_avg_bits=avg_bits, achieved_avg_code_bits=bits / elems,
-              achieved_bits_with_scales=bits / elems + OV, nmse=num / den,
-              pipeline_GBps_of_bf16_input=round(2.0 * elems * 256 / (gpu_ms * 1e-3) / 1e9, 1))
+        for pipe_name, pipe in (("sequence", dynamic_bitrate_allreduce), ("grouped", dynamic_bitrate_allreduce_grouped)):
+            gen = torch.Generator(device=dev).manual_seed(3)
+            comps = {q: [cls(q, 16, _params(6553600 * 8, 1, 0), generator=gen)] for q in (2, 4, 8)}
+            kw = {"work": {}} if pipe_name == "grouped" else {}
+            num = den = 0.0
+            bits = elems = 0
+            check = 0
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            times = []
+            for b in _llama_buckets(dev, limit=limit):
+                x = b.to(torch.bfloat16)
+                s.record()
+                outs, _, qbits = pipe([x], u, comps, **kw)
+                e.record()
+                e.synchronize()
+                times.append((s.elapsed_time(e), x.numel()))
+                num += float(((outs[0].double() - b.double()) ** 2).sum())
+                den += float((b.double() ** 2).sum())
+                bits += int(qbits.sum())
+                elems += qbits.numel()
+                check ^= int(outs[0].view(torch.int16).to(torch.int64).sum()) & 0xFFFFFFFF
+            timed = times[1:] if len(times) > 1 else times       # the first bucket pays the one-time allocations
+            gpu_ms = sum(t for t, _ in timed)
+            _emit(config=4, method=name, pipeline=pipe_name, buckets=len(times), elements=elems * 256, target_avg_bits=target,
+                  u=u, search_avg_bits=avg_bits, achieved_avg_code_bits=bits / elems,
+                  achieved_bits_with_scales=bits / elems + OV, nmse=num / den, output_checksum=check,
+                  ms_per_25MB_bucket=round(gpu_ms / len(timed), 4),
+                  pipeline_GBps_of_bf16_input=round(2.0 * sum(m for _, m in timed) / (gpu_ms * 1e-3) / 1e9, 1))
 
 
 def config5(dev, n=1 << 30):

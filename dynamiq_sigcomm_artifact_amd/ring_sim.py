@@ -65,3 +65,49 @@ def ring_allreduce(rank_vecs, compressors, align=256):
         for r in range(W):
             compressors[r].decompression(bufs[(step ^ 1) & 1][r], chunks[r][(r - step + W) % W])
     return rank_vecs
+
+
+def split_rows(rows, world_size):
+    """the ring chunks of a group of superchunks: split_chunks() on its 256 * len(rows) elements"""
+    per = (rows.numel() * 256 + world_size - 1) // world_size
+    per = _align_up(per, 256) // 256
+    return [rows[per * i: min(per * (i + 1), rows.numel())] for i in range(world_size)]
+
+
+def ring_allreduce_rows(rank_residuals, rows, compressors, rank_outputs, stats, n_limit):
+    """The same schedule for one bit-width group without materialising the group tensor: ``rows`` (int32)
+    lists the group's superchunks; every rank reads them from its full residual buffer and the decoded
+    result lands, mean added, in the rank's output buffer.  Byte-identical to index_select ->
+    ring_allreduce -> index_copy_ -> superchunk_add_mean_copy on those superchunks."""
+    W = len(rank_residuals)
+    assert W == len(compressors) and W >= 2
+    chunks = split_rows(rows, W)
+    nbytes = compressors[0].compressed_numel(chunks[0].numel() * 256)
+    dev = rank_residuals[0].device
+    send = [torch.zeros(nbytes, dtype=torch.uint8, device=dev) for _ in range(W)]
+    recv = [torch.zeros(nbytes, dtype=torch.uint8, device=dev) for _ in range(W)]
+
+    def exchange(src_bufs, dst_bufs):
+        for r in range(W):
+            dst_bufs[(r + 1) % W].copy_(src_bufs[r])
+
+    for step in range(W - 1):
+        for r in range(W):
+            if step == 0:
+                compressors[r].compression_rows(rank_residuals[r], chunks[r], send[r])
+            else:
+                compressors[r].dec_compression_rows(recv[r], rank_residuals[r], chunks[(r - step + W) % W], send[r])
+        exchange(send, recv)
+
+    for r in range(W):
+        owner = chunks[(r + 1) % W]
+        compressors[r].dec_compression_rows(recv[r], rank_residuals[r], owner, send[r])
+        compressors[r].decompression_rows(send[r], rank_outputs[r], owner, stats, n_limit)
+
+    bufs = [send, recv]
+    for step in range(W - 1):
+        exchange(bufs[step & 1], bufs[(step ^ 1) & 1])
+        for r in range(W):
+            compressors[r].decompression_rows(bufs[(step ^ 1) & 1][r], rank_outputs[r], chunks[(r - step + W) % W],
+                                              stats, n_limit)
+    return rank_outputs

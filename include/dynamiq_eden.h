@@ -111,6 +111,58 @@ int dq_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const voi
                         int64_t n, int nbits, int chunk_size, int dtype, int device,
                         int strategy, dq_stream_t stream);
 
+/* ---- dynamic-bitrate groups: gather / scatter folded into the codec ----
+ *
+ * The reference's dynamic-bitrate hook builds, per bit width w in {8, 4, 2}, the
+ * list of superchunks with that width (three torch.nonzero calls,
+ * testbed_evaluation/new_comm_hooks/comm_hooks.py:964-966), copies them into a
+ * contiguous group tensor (index_select, :1001), runs the compressed ring on the
+ * group, copies the result back (index_copy_, :1011) and finally adds the means
+ * (superchunk_add_mean_copy, :1019).  The entry points below produce the same
+ * bytes without the group tensor: record k of a packed stream stands for
+ * superchunk rows[k] of the full residual / output buffer.  chunk_size is 16,
+ * strategy 2 or 3, dtype DQ_BF16 or DQ_F32 (DQ_RAND_BF16 allowed on the
+ * compress side); other combinations return DQ_ERR_DTYPE / DQ_ERR_STRATEGY. */
+
+/* number of int32 the `work` argument of dq_group_plan must hold */
+int64_t dq_group_plan_work_ints(int64_t nsc);
+
+/* comm_hooks.py:964-966.  qbits: int64 [nsc] on the device (the output of
+ * _dynamic_bitrate_qbits, :48-66).  order: int32 [nsc]; on return
+ * order[0..n8) lists, ascending, the superchunks with qbits == 8, then n4 with
+ * 4, then n2 with 2 (torch.nonzero order).  work[0..2] = n8, n4, n2 and
+ * work[3] = superchunks of any other width (they appear in no group); the rest
+ * of work is scratch.  Two launches on `stream`, no host synchronisation. */
+int dq_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work,
+                  int64_t work_ints, int device, dq_stream_t stream);
+
+/* comm_hooks.py:1001 + scaling_compress: dst record k (and rand_pool row k,
+ * 256 elements) encodes superchunk rows[k] of src.  rows: int32 [nrows] on the
+ * device, every entry in [0, src superchunks).  rows == NULL means rows[k] = k. */
+int dq_scaling_compress_rows(const void *src, const int32_t *rows, uint8_t *dst,
+                             const void *rand_pool, int64_t nrows, int nbits, int dtype,
+                             int device, int strategy, dq_stream_t stream);
+
+/* the ring's fused step on a group: send record k =
+ * compress(round(inp[rows[k]] + decode(recv record k))); inp is not modified. */
+int dq_scaling_dec_comp_rows(const uint8_t *recv, const void *inp, const int32_t *rows,
+                             uint8_t *send, const void *rand_pool, int64_t nrows, int nbits,
+                             int dtype, int device, int strategy, dq_stream_t stream);
+
+/* scaling_decompress + comm_hooks.py:1011 (+ :1019 when stats != NULL): record
+ * k decodes into superchunk rows[k] of dst.  With stats (bf16 pairs
+ * (mean, sum of squares) per superchunk of dst, as written by
+ * dq_superchunk_mean_center) the value stored is
+ * T(float(T(decoded)) + float(stats[2 * rows[k]])) -- what decompress into the
+ * residual followed by superchunk_add_mean_copy stores.  Elements at index >=
+ * n_limit of dst are not written (n_limit = the unpadded element count when dst
+ * is the final output; pass the padded count for a residual buffer).
+ * add_original != 0 accumulates into dst (stats must then be NULL). */
+int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *rows,
+                               const void *stats, int64_t n_limit, int64_t nrows, int nbits,
+                               int dtype, int device, int strategy, dq_stream_t stream,
+                               int add_original);
+
 /* ---- superchunk mean-centring ---------------------------------------- */
 
 /* csrc/cuda_hadamard.h:23-24 (superchunk_mean_center_with_cuda).  residual

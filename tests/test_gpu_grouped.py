@@ -1,0 +1,144 @@
+"""The codec over lists of superchunk indices (gather / scatter / mean add folded into the kernels)
+against what it replaces: torch.nonzero, index_select + codec + index_copy_, superchunk_add_mean_copy
+(testbed_evaluation/new_comm_hooks/comm_hooks.py:963-1019) -- byte for byte."""
+import math
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, F32, to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("nsc", [1, 5, 1023, 1024, 1025, 25600, 300001])
+def test_group_plan_matches_nonzero(capi, nsc):
+    g = torch.Generator().manual_seed(nsc)
+    q = torch.tensor([2, 4, 8, 16])[torch.randint(0, 4 if nsc > 5 else 3, (nsc,), generator=g)].to(DEV)
+    if nsc == 1023:
+        q[:] = 8            # a single group
+    order = torch.full((nsc,), -1, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    capi.group_plan(q, order, work)
+    counts = work[:4].tolist()
+    want = [torch.nonzero(q == w).view(-1) for w in (8, 4, 2)]
+    assert counts[:3] == [w.numel() for w in want] and counts[3] == int((q == 16).sum())
+    got = order[:sum(counts[:3])].cpu()
+    assert torch.equal(got, torch.cat(want).cpu().to(torch.int32))
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("nbits,strategy", [(2, 2), (4, 2), (8, 3), (5, 3)])
+def test_rows_entry_points_match_gather_codec_scatter(capi, dt, nbits, strategy):
+    nsc, n_valid = 1037, 1037 * 256 - 77
+    g = torch.Generator().manual_seed(nbits * 7 + strategy)
+    full = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+    peer = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+    stats = torch.randn(nsc, 2, generator=g).mul(1e-2).to(torch.bfloat16).to(DEV)
+    rows = torch.randperm(nsc, generator=g)[:701].sort().values.to(torch.int32).to(DEV)
+    nrows = rows.numel()
+    rnd = torch.rand(nrows * 256, generator=g).to(torch.bfloat16).to(DEV)
+    if dt == torch.float32 and nbits == 2:
+        rnd = rnd.float()       # same-dtype pool as well as the mixed one
+    nbytes = capi.required_bytes(nrows * 256, nbits, 16, strategy)
+    idx = rows.long()
+
+    # reference sequence
+    grp = full.view(-1, 256).index_select(0, idx).reshape(-1).contiguous()
+    enc_ref = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(grp, enc_ref, rnd, nrows * 256, nbits, 16, strategy)
+    grp2 = peer.view(-1, 256).index_select(0, idx).reshape(-1).contiguous()
+    send_ref = torch.zeros_like(enc_ref)
+    capi.scaling_dec_comp(enc_ref, grp2, send_ref, rnd, nrows * 256, nbits, 16, strategy)
+    dec = torch.empty_like(grp)
+    capi.scaling_decompress(send_ref, dec, nrows * 256, nbits, 16, strategy)
+    res = torch.zeros_like(full)
+    res.view(-1, 256).index_copy_(0, idx, dec.view(-1, 256))
+    out_ref = torch.full((n_valid,), 7.0, dtype=dt, device=DEV)
+    capi.superchunk_add_mean_copy(res, out_ref, stats, n_valid)
+
+    # folded
+    enc = torch.zeros_like(enc_ref)
+    capi.scaling_compress_rows(full, rows, enc, rnd, nrows, nbits, strategy)
+    assert torch.equal(enc, enc_ref)
+    send = torch.zeros_like(enc_ref)
+    peer_before = peer.clone()
+    capi.scaling_dec_comp_rows(enc, peer, rows, send, rnd, nrows, nbits, strategy)
+    assert torch.equal(send, send_ref) and torch.equal(peer, peer_before)
+    out = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
+    capi.scaling_decompress_rows(send, out, rows, stats, n_valid, nrows, nbits, strategy)
+    sel = torch.zeros(nsc * 256, dtype=torch.bool, device=DEV)
+    sel.view(-1, 256)[idx] = True
+    sel = sel[:n_valid]
+    assert torch.equal(to_bits_t(out[:n_valid][sel]), to_bits_t(out_ref[sel]))
+    assert bool((out[:n_valid][~sel] == 7.0).all()) and bool((out[n_valid:] == 7.0).all())    # nothing else touched
+
+    # without stats, scatter into a residual-sized buffer; rows == None is the identity list
+    plain = torch.zeros_like(full)
+    capi.scaling_decompress_rows(send, plain, rows, None, nsc * 256, nrows, nbits, strategy)
+    assert torch.equal(to_bits_t(plain), to_bits_t(res))
+    ident = torch.empty_like(dec)
+    capi.scaling_decompress_rows(send, ident, None, None, nrows * 256, nrows, nbits, strategy)
+    assert torch.equal(to_bits_t(ident), to_bits_t(dec))
+    # an element buffer that is only 2-byte aligned takes the per-lane store path
+    if dt == torch.bfloat16:
+        shifted = torch.zeros(nsc * 256 + 8, dtype=dt, device=DEV)[1:1 + nsc * 256]
+        capi.scaling_decompress_rows(send, shifted, rows, stats, n_valid, nrows, nbits, strategy)
+        assert torch.equal(to_bits_t(shifted[:n_valid][sel]), to_bits_t(out_ref[sel]))
+        assert bool((shifted[n_valid:] == 0).all())
+
+
+def to_bits_t(t):
+    return t.view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+def _tensors(n, W, seed):
+    g = torch.Generator().manual_seed(seed)
+    blocks = (n + 2559) // 2560
+    scale = torch.exp(torch.randn(blocks, generator=g) * 4.0 + math.log(1e-3)).repeat_interleave(2560)[:n]
+    return [(torch.randn(n, generator=g) * scale).to(torch.bfloat16).to(DEV) for _ in range(W)]
+
+
+def _compressors(cls, W, n, seed):
+    out = {}
+    for q in (2, 4, 8):
+        out[q] = []
+        for r in range(W):
+            params = {"d": {(0, 0): n * 4}, "world_size": W, "rank": r,
+                      "args": types.SimpleNamespace(aggregation_method="dynamiQ")}
+            gen = torch.Generator(device=DEV).manual_seed(seed * 100 + q * 10 + r)
+            out[q].append(cls(q, 16, params, generator=gen))
+    return out
+
+
+@pytest.mark.parametrize("W", [1, 2, 5])
+@pytest.mark.parametrize("method", ["aee", "mee"])
+def test_grouped_pipeline_equals_reference_sequence(eden_utils, W, method):
+    from dynamiq_sigcomm_artifact_amd import bitrate
+    from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import dynamic_bitrate_allreduce, dynamic_bitrate_allreduce_grouped
+    cls = Aee_Dynamic_Range_GPU_kern if method == "aee" else Mee_Dynamic_Range_GPU_kern
+    n = 256 * 2111 + 19            # a ragged tail: the last superchunk is mostly padding
+    vecs = _tensors(n, W, 3)
+    # u from the reduced norms, as the hook does at its first compressed round (comm_hooks.py:94-114)
+    nsc = (n + 255) // 256
+    norms = torch.zeros(nsc, dtype=torch.bfloat16, device=DEV)
+    for v in vecs:
+        st = torch.empty(nsc, 2, dtype=torch.bfloat16, device=DEV)
+        eden_utils.superchunk_mean_center(v, torch.empty(nsc * 256, dtype=v.dtype, device=DEV), st, n, W)
+        norms += st[:, 1]
+    u, _, _ = bitrate.dynamic_bitrate_binary_search_u([norms], 4.375)
+    a_out, a_stats, a_q = dynamic_bitrate_allreduce([v.clone() for v in vecs], u, _compressors(cls, W, n, 1))
+    b_out, b_stats, b_q = dynamic_bitrate_allreduce_grouped([v.clone() for v in vecs], u, _compressors(cls, W, n, 1))
+    assert torch.equal(a_q, b_q) and len({int(x) for x in a_q.unique().tolist()}) == 3
+    assert torch.equal(to_bits_t(a_stats), to_bits_t(b_stats))
+    for r in range(W):
+        assert torch.equal(to_bits_t(a_out[r]), to_bits_t(b_out[r])), r
+    for r in range(1, W):
+        assert torch.equal(to_bits_t(b_out[0]), to_bits_t(b_out[r]))
+    ref = torch.stack([v.double() for v in vecs]).mean(0)
+    nmse = float(((b_out[0].double() - ref) ** 2).sum() / (ref ** 2).sum())
+    assert nmse < 0.2
