@@ -20,7 +20,7 @@ EXPORTS = [
     "dq_scaling_required_bytes", "dq_scaling_check_common",
     "dq_init_lookup_table", "dq_mee_lookup_table",
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
-    "dq_group_plan_work_ints", "dq_group_plan",
+    "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag",
@@ -64,6 +64,8 @@ def lib():
         L.dq_group_plan_work_ints.argtypes = [i64]
         L.dq_group_plan.restype = i32
         L.dq_group_plan.argtypes = [vp, i64, vp, vp, i64, i32, vp]
+        L.dq_group_plan_stats.restype = i32
+        L.dq_group_plan_stats.argtypes = [vp, c.c_double, i64, vp, vp, vp, i64, i32, vp]
         L.dq_scaling_compress_rows.restype = i32
         L.dq_scaling_compress_rows.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_scaling_dec_comp_rows.restype = i32
@@ -172,6 +174,17 @@ def group_plan(qbits, order, work, stream=None):
 
 def _ptr(t):
     return 0 if t is None else t.data_ptr()
+
+
+def group_plan_stats(stats, u, qbits_out, order, work, stream=None):
+    """stats bf16 [nsc, 2] (mean, reduced sum of squares), offset u -> qbits_out (int64 or None), order, work"""
+    if stats.dtype != torch.bfloat16 or order.dtype != torch.int32 or work.dtype != torch.int32:
+        raise RuntimeError("group_plan_stats: stats must be bfloat16, order and work int32")
+    nsc = stats.numel() // 2
+    if order.numel() < nsc or (qbits_out is not None and (qbits_out.dtype != torch.int64 or qbits_out.numel() < nsc)):
+        raise RuntimeError("group_plan_stats: order / qbits_out too small or of the wrong dtype")
+    _check(lib().dq_group_plan_stats(stats.data_ptr(), float(u), nsc, _ptr(qbits_out), order.data_ptr(), work.data_ptr(),
+                                     work.numel(), _dev(stats), _stream(stream)))
 
 
 def scaling_compress_rows(src, rows, dst, rand_pool, nrows, nbits, strategy, stream=None):

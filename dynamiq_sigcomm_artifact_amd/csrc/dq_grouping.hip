@@ -20,12 +20,42 @@ constexpr int kPer = kTile / kThreads;
 
 __device__ __forceinline__ int width_class(int64_t q) { return q == 8 ? 0 : q == 4 ? 1 : q == 2 ? 2 : 3; }
 
+__device__ __forceinline__ float round_bf16(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+
+// testbed_evaluation/new_comm_hooks/comm_hooks.py:64-70 on a bf16 norm: every torch op computes in
+// binary32 and rounds its result to bf16
+__device__ __forceinline__ int64_t qbits_of_norm(uint32_t norm_bits, float u)
+{
+    const float eps = 1e-20f;
+    float x = bf16_bits_to_f32(norm_bits);
+    x = (x != x) ? x : round_bf16(x > eps ? x : eps);
+    x = round_bf16(log2_det(x));
+    x = round_bf16(x * (float)(4.0 / (512.0 / 17.0)));
+    x = round_bf16(x + u);
+    x = (x != x) ? x : round_bf16(x > eps ? x : eps);
+    x = round_bf16(log2_det(x));
+    x = __builtin_floorf(x);
+    int z = (x != x) ? 1 : (x < 1.0f ? 1 : (x > 3.0f ? 3 : (int)x));
+    return (int64_t)1 << z;
+}
+
+// where the widths come from: an int64 array, or the norm column of the interleaved bf16 stats
+struct WidthsFromArray {
+    const int64_t *qbits;
+    __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
+};
+struct WidthsFromStats {
+    const uint16_t *stats;
+    float u;
+    __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits_of_norm(stats[2 * i + 1], u); }
+};
+
 // three 21-bit counters in one word
 __device__ __forceinline__ uint64_t one_of(int cls) { return cls < 3 ? (uint64_t)1 << (21 * cls) : 0; }
 __device__ __forceinline__ int field(uint64_t p, int cls) { return (int)((p >> (21 * cls)) & 0x1fffff); }
 
-__global__ __launch_bounds__(kThreads) void plan_count_kernel(const int64_t *__restrict__ qbits, int64_t nsc,
-                                                              int32_t *__restrict__ work)
+template <class W>
+__global__ __launch_bounds__(kThreads) void plan_count_kernel(W widths, int64_t nsc, int32_t *__restrict__ work)
 {
     __shared__ int cnt[4];
     if (threadIdx.x < 4) cnt[threadIdx.x] = 0;
@@ -34,7 +64,7 @@ __global__ __launch_bounds__(kThreads) void plan_count_kernel(const int64_t *__r
     int c[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int k = 0; k < kPer; k++) {
-        if (base + k < nsc) c[width_class(qbits[base + k])]++;
+        if (base + k < nsc) c[width_class(widths(base + k))]++;
     }
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -44,8 +74,10 @@ __global__ __launch_bounds__(kThreads) void plan_count_kernel(const int64_t *__r
     if (threadIdx.x < 4) work[4 + 4 * blockIdx.x + threadIdx.x] = cnt[threadIdx.x];
 }
 
-__global__ __launch_bounds__(kThreads) void plan_place_kernel(const int64_t *__restrict__ qbits, int64_t nsc, int ntiles,
-                                                              int32_t *__restrict__ order, int32_t *__restrict__ work)
+template <class W>
+__global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t *__restrict__ qbits_out, int64_t nsc,
+                                                              int ntiles, int32_t *__restrict__ order,
+                                                              int32_t *__restrict__ work)
 {
     __shared__ int before[4], total[4];
     __shared__ uint64_t wave_sum[kThreads / 64];
@@ -78,7 +110,12 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(const int64_t *__r
     uint64_t mine = 0;
 #pragma unroll
     for (int k = 0; k < kPer; k++) {
-        cls[k] = base + k < nsc ? width_class(qbits[base + k]) : 3;
+        cls[k] = 3;
+        if (base + k < nsc) {
+            const int64_t q = widths(base + k);
+            if (qbits_out) qbits_out[base + k] = q;
+            cls[k] = width_class(q);
+        }
         mine += one_of(cls[k]);
     }
     // inclusive scan over the wave, then over the waves of the workgroup
@@ -111,14 +148,26 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(const int64_t *__r
 
 int64_t group_plan_work_ints(int64_t nsc) { return 4 + 4 * ((nsc + kTile - 1) / kTile); }
 
-hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work, hipStream_t stream)
+template <class W>
+static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *order, int32_t *work, hipStream_t stream)
 {
     const int ntiles = (int)((nsc + kTile - 1) / kTile);
-    hipLaunchKernelGGL(plan_count_kernel, dim3(ntiles), dim3(kThreads), 0, stream, qbits, nsc, work);
+    hipLaunchKernelGGL(plan_count_kernel<W>, dim3(ntiles), dim3(kThreads), 0, stream, widths, nsc, work);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(plan_place_kernel, dim3(ntiles), dim3(kThreads), 0, stream, qbits, nsc, ntiles, order, work);
+    hipLaunchKernelGGL(plan_place_kernel<W>, dim3(ntiles), dim3(kThreads), 0, stream, widths, qbits_out, nsc, ntiles, order, work);
     return hipGetLastError();
+}
+
+hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work, hipStream_t stream)
+{
+    return run_plan(WidthsFromArray{qbits}, nullptr, nsc, order, work, stream);
+}
+
+hipError_t launch_group_plan_stats(const void *stats, float u, int64_t nsc, int64_t *qbits_out, int32_t *order,
+                                   int32_t *work, hipStream_t stream)
+{
+    return run_plan(WidthsFromStats{static_cast<const uint16_t *>(stats), u}, qbits_out, nsc, order, work, stream);
 }
 
 } // namespace dq

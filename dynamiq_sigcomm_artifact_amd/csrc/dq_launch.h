@@ -45,6 +45,9 @@ hipError_t launch_hier16_decompress_rows(const uint8_t *src, void *dst, const in
 int64_t group_plan_work_ints(int64_t nsc);
 hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work,
                              hipStream_t stream);
+// the same with the widths computed from the norm column of the bf16 stats and the offset u
+hipError_t launch_group_plan_stats(const void *stats, float u, int64_t nsc, int64_t *qbits_out,
+                                   int32_t *order, int32_t *work, hipStream_t stream);
 
 // superchunk mean-centring (dq_superchunk.hip)
 hipError_t launch_mean_center(const void *src, void *residual, void *stats, int64_t n,

@@ -286,6 +286,31 @@ torch::Tensor group_plan(torch::Tensor qbits, torch::Tensor order, uint64_t stre
     return work.slice(0, 0, 4);
 }
 
+torch::Tensor group_plan_stats(torch::Tensor stats, double u, torch::Tensor order, c10::optional<torch::Tensor> qbits_out,
+                               uint64_t stream_p = 0)
+{
+    TORCH_CHECK(stats.device().type() == torch::kCUDA, "stats must be a CUDA tensor");
+    TORCH_CHECK(order.device().type() == torch::kCUDA, "order must be a CUDA tensor");
+    TORCH_CHECK(stats.dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+    TORCH_CHECK(order.dtype() == torch::kInt32, "order must be torch.int32");
+    TORCH_CHECK(stats.is_contiguous() && order.is_contiguous(), "stats and order must be contiguous");
+    const int64_t nsc = stats.numel() / 2;
+    TORCH_CHECK(nsc > 0 && stats.numel() == 2 * nsc, "stats must hold (mean, norm) pairs");
+    TORCH_CHECK(order.numel() >= nsc, "order has fewer entries than superchunks");
+    int64_t *qptr = nullptr;
+    if (qbits_out.has_value()) {
+        TORCH_CHECK(qbits_out->device().type() == torch::kCUDA && qbits_out->dtype() == torch::kInt64 &&
+                        qbits_out->is_contiguous() && qbits_out->numel() >= nsc,
+                    "qbits_out must be a contiguous torch.int64 CUDA tensor with one entry per superchunk");
+        qptr = qbits_out->data_ptr<int64_t>();
+    }
+    auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
+    check_status(dq_group_plan_stats(stats.data_ptr(), u, nsc, qptr, order.data_ptr<int32_t>(), work.data_ptr<int32_t>(),
+                                     work.numel(), stats.device().index(), as_stream(stream_p)),
+                 "group_plan_stats");
+    return work.slice(0, 0, 4);
+}
+
 void scaling_compress_rows(torch::Tensor src, torch::Tensor rows, torch::Tensor dst, torch::Tensor rand_pool, int64_t nrows,
                            int nbits, uint64_t stream_p = 0, int strategy = 2)
 {
@@ -483,6 +508,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("rand_diag", &rand_diag, "EDEN's seeded +-1 diagonal", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
     modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width; returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
+    modul.def("group_plan_stats", &group_plan_stats, "bit widths from the reduced bf16 norms and the offset u, and the partition by width, in one call; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
     modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_decompress_rows", &scaling_decompress_rows, "decode consecutive records into the superchunks rows[k] of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("rows"), py::arg("stats"), py::arg("n_limit"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);

@@ -63,11 +63,15 @@ def dynamic_bitrate_allreduce(rank_vecs, u, compressors, out=None):
     return outs, total, qbits
 
 
-def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=None):
+def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=None, device_qbits=False):
     """Same inputs, same results (bit for bit) as dynamic_bitrate_allreduce, with the gather, the scatter
     and the final mean add folded into the codec kernels: one device-side partition of the superchunk
     indices by width (a single 16-byte read-back for the three group sizes, in place of three
-    torch.nonzero), no group tensors, no index_select / index_copy_ / superchunk_add_mean_copy passes."""
+    torch.nonzero), no group tensors, no index_select / index_copy_ / superchunk_add_mean_copy passes.
+
+    device_qbits=True also computes the bit widths inside the partition call (the rule of
+    bitrate.dynamic_bitrate_qbits with the library's fixed-polynomial log2 in place of torch.log2; the two
+    agree except where a log2 value lies within a few binary32 ulps of a bf16 rounding boundary)."""
     eu = load_eden_utils()
     W = len(rank_vecs)
     n = rank_vecs[0].numel()
@@ -88,8 +92,14 @@ def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=
     total = stats[0] if W == 1 else stats[0].clone()
     for r in range(1, W):
         total.add_(stats[r])
-    qbits = bitrate.dynamic_bitrate_qbits(total[:, 1], u)
-    counts = eu.group_plan(qbits, order, stream).tolist()
+    if device_qbits:
+        qbits = work.get("qbits")
+        if qbits is None or qbits.numel() != nsc:
+            qbits = work["qbits"] = torch.empty(nsc, dtype=torch.int64, device=dev)
+        counts = eu.group_plan_stats(total, float(u), order, qbits, stream).tolist()
+    else:
+        qbits = bitrate.dynamic_bitrate_qbits(total[:, 1], u)
+        counts = eu.group_plan(qbits, order, stream).tolist()
     assert counts[3] == 0, "bit widths outside {2, 4, 8}"
 
     outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]

@@ -224,10 +224,11 @@ def config4(dev, limit=None):
     u, avg_bits, delta = bitrate.dynamic_bitrate_binary_search_u(norms_list, target)
     # pass 2: quantise, with the reference's op sequence and with the gather/scatter folded into the kernels
     for cls, name in ((Aee_Dynamic_Range_GPU_kern, "aee"), (Mee_Dynamic_Range_GPU_kern, "mee")):
-        for pipe_name, pipe in (("sequence", dynamic_bitrate_allreduce), ("grouped", dynamic_bitrate_allreduce_grouped)):
+        for pipe_name, pipe in (("sequence", dynamic_bitrate_allreduce), ("grouped", dynamic_bitrate_allreduce_grouped),
+                                ("grouped+device_qbits", dynamic_bitrate_allreduce_grouped)):
             gen = torch.Generator(device=dev).manual_seed(3)
             comps = {q: [cls(q, 16, _params(6553600 * 8, 1, 0), generator=gen)] for q in (2, 4, 8)}
-            kw = {"work": {}} if pipe_name == "grouped" else {}
+            kw = {} if pipe_name == "sequence" else {"work": {}, "device_qbits": pipe_name.endswith("device_qbits")}
             num = den = 0.0
             bits = elems = 0
             check = 0

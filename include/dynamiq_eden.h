@@ -136,6 +136,15 @@ int64_t dq_group_plan_work_ints(int64_t nsc);
 int dq_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work,
                   int64_t work_ints, int device, dq_stream_t stream);
 
+/* comm_hooks.py:48-70 (_dynamic_bitrate_qbits on the bf16 norms, every torch op
+ * rounding its result to bf16) + :964-966 in one call: the width of superchunk
+ * i is computed from stats[2 * i + 1] (the reduced sum of squares written by
+ * dq_superchunk_mean_center) and the offset u, log2 being the library's fixed
+ * polynomial.  qbits_out: int64 [nsc] or NULL. */
+int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits_out,
+                        int32_t *order, int32_t *work, int64_t work_ints, int device,
+                        dq_stream_t stream);
+
 /* comm_hooks.py:1001 + scaling_compress: dst record k (and rand_pool row k,
  * 256 elements) encodes superchunk rows[k] of src.  rows: int32 [nrows] on the
  * device, every entry in [0, src superchunks).  rows == NULL means rows[k] = k. */

@@ -818,9 +818,8 @@ void dqo_dynamic_bitrate_qbits(const uint16_t *norms_bf16, int64_t stride, int64
         x = (x != x) ? x : rb(x > eps ? x : eps);          /* clamp(min=eps)  */
         x = rb(dqo_log2f(x));                              /* log2            */
         x = floorf(x);                                     /* floor           */
-        int64_t z = (x != x) ? INT64_MIN : (int64_t)x;
-        if (z < 1) z = 1;
-        if (z > 3) z = 3;
+        /* .to(torch.int64) on the device saturates (+inf -> INT64_MAX) and sends NaN below the clamp */
+        int64_t z = (x != x) ? 1 : (x < 1.0f ? 1 : (x > 3.0f ? 3 : (int64_t)x));
         qbits[i] = (int64_t)1 << z;
     }
 }

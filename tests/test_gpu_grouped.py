@@ -30,6 +30,33 @@ def test_group_plan_matches_nonzero(capi, nsc):
     assert torch.equal(got, torch.cat(want).cpu().to(torch.int32))
 
 
+def test_group_plan_stats_all_bf16_norms(capi, oracle):
+    """widths computed in the kernel == the oracle's restatement of the allocation rule for EVERY bf16 norm
+    pattern and a sweep of offsets; torch's own op sequence on the device agrees as well"""
+    from dynamiq_sigcomm_artifact_amd import bitrate
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    norms = pats.view(torch.bfloat16)
+    nsc = norms.numel()
+    stats = torch.zeros(nsc, 2, dtype=torch.bfloat16)
+    stats[:, 1] = norms
+    stats_d = stats.to(DEV)
+    order = torch.empty(nsc, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    qout = torch.empty(nsc, dtype=torch.int64, device=DEV)
+    finite = torch.isfinite(norms.float())
+    for u in (-10.0, 0.0, 3.3, 7.25, 10.38818359375, 11.0, 13.7, 25.0, 60.0):
+        capi.group_plan_stats(stats_d, u, qout, order, work)
+        want = oracle.dynamic_bitrate_qbits(to_bits(norms), u)
+        got = qout.cpu().numpy()
+        assert (got == want).all(), (u, np.nonzero(got != want)[0][:10], got[got != want][:10], want[got != want][:10])
+        counts = work[:4].tolist()
+        assert counts == [int((want == 8).sum()), int((want == 4).sum()), int((want == 2).sum()), 0]
+        idx = np.concatenate([np.nonzero(want == w)[0] for w in (8, 4, 2)])
+        assert (order.cpu().numpy() == idx).all()
+        t = bitrate.dynamic_bitrate_qbits(stats_d[:, 1], u).cpu()
+        assert int((t[finite] != qout.cpu()[finite]).sum()) == 0, u
+
+
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("nbits,strategy", [(2, 2), (4, 2), (8, 3), (5, 3)])
 def test_rows_entry_points_match_gather_codec_scatter(capi, dt, nbits, strategy):
@@ -139,6 +166,9 @@ def test_grouped_pipeline_equals_reference_sequence(eden_utils, W, method):
         assert torch.equal(to_bits_t(a_out[r]), to_bits_t(b_out[r])), r
     for r in range(1, W):
         assert torch.equal(to_bits_t(b_out[0]), to_bits_t(b_out[r]))
+    c_out, _, c_q = dynamic_bitrate_allreduce_grouped([v.clone() for v in vecs], u, _compressors(cls, W, n, 1),
+                                                      device_qbits=True)
+    assert torch.equal(c_q, a_q) and torch.equal(to_bits_t(c_out[0]), to_bits_t(a_out[0]))
     ref = torch.stack([v.double() for v in vecs]).mean(0)
     nmse = float(((b_out[0].double() - ref) ** 2).sum() / (ref ** 2).sum())
     assert nmse < 0.2

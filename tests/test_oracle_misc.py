@@ -215,3 +215,13 @@ def test_dynamic_bitrate_rule(oracle):
     us = (3.98, 4.0, 7.9, 7.97, 8.0)
     assert [int(oracle.dynamic_bitrate_qbits(one, u)[0]) for u in us] == [2, 4, 4, 8, 8]
     assert [int(_torch_qbits(torch.tensor([1.0]).to(torch.bfloat16), u)[0]) for u in us] == [2, 4, 4, 8, 8]
+
+
+def test_bit_width_rule_non_finite_norms(oracle):
+    """the device conversion to int64 saturates: +inf norms land in the 8-bit group, NaN norms in the 2-bit group"""
+    import numpy as np
+    from helpers import to_bits
+    import torch
+    norms = torch.tensor([float("inf"), float("nan"), 0.0, -1.0, 1e-30], dtype=torch.bfloat16)
+    assert oracle.dynamic_bitrate_qbits(to_bits(norms), 60.0).tolist() == [8, 2, 8, 8, 8]
+    assert oracle.dynamic_bitrate_qbits(to_bits(norms), -10.0).tolist() == [8, 2, 2, 2, 2]
