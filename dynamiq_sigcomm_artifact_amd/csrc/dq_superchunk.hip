@@ -1,11 +1,17 @@
 // Superchunk (256-element) mean-centring and its inverse.
 //
-// superchunk_mean_center: one wave owns one superchunk.  Lane L holds elements
-// L, L+64, L+128, L+192, which makes the reference's fixed reduction tree
-// (shared-memory halving, stride 128 -> 1, csrc/cuda_hadamard.cu:1286-1292)
-// two in-lane adds followed by six "lane L += lane L+stride" steps; the sum is
-// therefore associated exactly as in the reference and the statistics are
+// superchunk_mean_center reproduces the reference's fixed reduction tree
+// (shared-memory halving, stride 128 -> 1, csrc/cuda_hadamard.cu:1286-1292), so the
+// sums are associated exactly as in the reference and the statistics are
 // bit-identical.  Numerics: csrc/cuda_hadamard.cu:1257-1349.
+//
+//  * mean_center_tile_kernel (16-byte aligned buffers, whole superchunks): one wave owns
+//    four superchunks; the tile comes in with 16-byte loads, is staged in LDS, and the
+//    lane (row r, column j) picks up elements j + 16 k of superchunk r.  Strides 128..16
+//    of the tree are then fifteen in-lane adds and strides 8..1 four row-shift steps.
+//    The residual takes the same way back and leaves with 16-byte stores.
+//  * mean_center_kernel (anything else, and the ragged last superchunk): one wave per
+//    superchunk, lane L holds elements L + 64 k.
 //
 // superchunk_add_mean_copy: pure streaming, csrc/cuda_hadamard.cu:1351-1369.
 #include "dq_device.cuh"
@@ -20,14 +26,134 @@ template <int CTRL> __device__ __forceinline__ float dpp_shift(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// LDS accesses of one wave execute in order; the fence only stops the compiler from moving them
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// v / world, correctly rounded: world = 2^k multiplies by the exact reciprocal; otherwise the product with
+// the double reciprocal is within 2^-51 of the quotient, closer than a quotient of two binary32 numbers
+// can come to a rounding boundary without lying on it
+struct WorldDiv {
+    float inv;
+    double inv_d;
+    int pow2;
+    __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
+};
+
+template <int DT>
+__global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__restrict__ src, void *__restrict__ residual,
+                                                             uint32_t *__restrict__ stats, int64_t nsc, WorldDiv wd)
+{
+    constexpr int ESZ = DT == DQ_F32 ? 4 : 2;
+    constexpr int SPR = 16 * ESZ;            // 16-byte slots per superchunk
+    constexpr int RS = 256 * ESZ + 16 * ESZ; // padded LDS row stride: the four rows of a tile use disjoint banks
+    __shared__ __attribute__((aligned(16))) uint8_t tile[4 * RS];
+
+    const int lane = threadIdx.x;
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t sc0 = (int64_t)blockIdx.x * 4;
+    if (sc0 >= nsc) return;
+    const int rows_here = (int)min((int64_t)4, nsc - sc0);
+    const int nslots = rows_here * SPR;
+    const u32x4 *gin = reinterpret_cast<const u32x4 *>(static_cast<const char *>(src) + sc0 * 256 * ESZ);
+    u32x4 *gout = reinterpret_cast<u32x4 *>(static_cast<char *>(residual) + sc0 * 256 * ESZ);
+
+    // every lane loads (the slot index is clamped into the tile), so all loads are in flight together
+    const u32x4 raw0 = gin[min(lane, nslots - 1)];
+    const u32x4 raw1 = gin[min(lane + 64, nslots - 1)];
+    u32x4 raw2 = raw0, raw3 = raw0;
+    if (ESZ == 4) {
+        raw2 = gin[min(lane + 128, nslots - 1)];
+        raw3 = gin[min(lane + 192, nslots - 1)];
+    }
+#define DQ_SLOT_PTR(s) reinterpret_cast<u32x4 *>(tile + ((s) / SPR) * RS + ((s) % SPR) * 16)
+    if (lane < nslots) *DQ_SLOT_PTR(lane) = raw0;
+    if (lane + 64 < nslots) *DQ_SLOT_PTR(lane + 64) = raw1;
+    if (ESZ == 4) {
+        if (lane + 128 < nslots) *DQ_SLOT_PTR(lane + 128) = raw2;
+        if (lane + 192 < nslots) *DQ_SLOT_PTR(lane + 192) = raw3;
+    }
+    wave_lds_sync();
+
+    uint8_t *mine = tile + row * RS + j * ESZ;
+    float v[16];
+    if (row < rows_here) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            float x;
+            if (DT == DQ_F32)
+                x = *reinterpret_cast<const float *>(mine + 16 * k * ESZ);
+            else if (DT == DQ_BF16)
+                x = bf16_bits_to_f32(*reinterpret_cast<const uint16_t *>(mine + 16 * k * ESZ));
+            else
+                x = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(mine + 16 * k * ESZ));
+            v[k] = wd(x);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) v[k] = 0.0f;
+    }
+    // strides 128, 64, 32, 16: element j + 16 k pairs with k + 8, k + 4, k + 2, k + 1
+    float a[8], b[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        a[k] = v[k] + v[k + 8];
+        b[k] = v[k] * v[k] + v[k + 8] * v[k + 8];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        a[k] += a[k + 4];
+        b[k] += b[k + 4];
+    }
+    float sum = (a[0] + a[2]) + (a[1] + a[3]);
+    float sq = (b[0] + b[2]) + (b[1] + b[3]);
+    // strides 8, 4, 2, 1 inside the row of 16 lanes
+    sum += dpp_shift<0x108>(sum);
+    sq += dpp_shift<0x108>(sq);
+    sum += dpp_shift<0x104>(sum);
+    sq += dpp_shift<0x104>(sq);
+    sum += dpp_shift<0x102>(sum);
+    sq += dpp_shift<0x102>(sq);
+    sum += dpp_shift<0x101>(sum);
+    sq += dpp_shift<0x101>(sq);
+    const float mean = __shfl(sum, lane & 48, 64) * 0.00390625f; // / 256, exact
+    if (row < rows_here) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const float r = v[k] - mean;
+            if (DT == DQ_F32)
+                *reinterpret_cast<float *>(mine + 16 * k * ESZ) = r;
+            else if (DT == DQ_BF16)
+                *reinterpret_cast<uint16_t *>(mine + 16 * k * ESZ) = (uint16_t)f32_to_bf16_bits(r);
+            else
+                *reinterpret_cast<uint16_t *>(mine + 16 * k * ESZ) = (uint16_t)f32_to_f16_bits(r);
+        }
+        if (j == 0) stats[sc0 + row] = f32_to_bf16_bits(mean) | (f32_to_bf16_bits(sq) << 16);
+    }
+    wave_lds_sync();
+    if (lane < nslots) gout[lane] = *DQ_SLOT_PTR(lane);
+    if (lane + 64 < nslots) gout[lane + 64] = *DQ_SLOT_PTR(lane + 64);
+    if (ESZ == 4) {
+        if (lane + 128 < nslots) gout[lane + 128] = *DQ_SLOT_PTR(lane + 128);
+        if (lane + 192 < nslots) gout[lane + 192] = *DQ_SLOT_PTR(lane + 192);
+    }
+#undef DQ_SLOT_PTR
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void mean_center_kernel(const void *__restrict__ src, void *__restrict__ residual,
-                                                          uint16_t *__restrict__ stats, int64_t n, int64_t nsc,
-                                                          float world)
+                                                          uint16_t *__restrict__ stats, int64_t n, int64_t sc_begin,
+                                                          int64_t nsc, float world)
 {
     typedef ElemIO<DT> IO;
     const int lane = threadIdx.x & 63;
-    const int64_t sc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t sc = sc_begin + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (sc >= nsc) return;
     const int64_t start = sc * 256;
     int64_t valid64 = n - start;
@@ -107,19 +233,38 @@ __global__ __launch_bounds__(256) void add_mean_copy_vec_kernel(const uint4 *__r
     dst[i] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+template <int DT>
+static hipError_t run_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size,
+                                  hipStream_t stream)
+{
+    const int64_t nsc = (n + 255) / 256;
+    int64_t done = 0;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(residual)) & 15) == 0 &&
+                         (reinterpret_cast<uintptr_t>(stats) & 3) == 0;
+    if (aligned && n >= 256) {
+        done = n / 256;
+        WorldDiv wd;
+        wd.inv = 1.0f / (float)world_size;
+        wd.inv_d = 1.0 / (double)world_size;
+        wd.pow2 = (world_size & (world_size - 1)) == 0;
+        hipLaunchKernelGGL(mean_center_tile_kernel<DT>, dim3((unsigned)((done + 3) / 4)), dim3(64), 0, stream, src, residual,
+                           static_cast<uint32_t *>(stats), done, wd);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess || done == nsc) return e;
+    }
+    hipLaunchKernelGGL(mean_center_kernel<DT>, dim3((unsigned)((nsc - done + 3) / 4)), dim3(256), 0, stream, src, residual,
+                       static_cast<uint16_t *>(stats), n, done, nsc, (float)world_size);
+    return hipGetLastError();
+}
+
 hipError_t launch_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size, int dtype,
                               hipStream_t stream)
 {
-    const int64_t nsc = (n + 255) / 256;
-    dim3 grid((unsigned)((nsc + 3) / 4)), block(256);
-    uint16_t *st = static_cast<uint16_t *>(stats);
-    const float world = (float)world_size;
     switch (dtype) {
-    case DQ_F16: hipLaunchKernelGGL(mean_center_kernel<DQ_F16>, grid, block, 0, stream, src, residual, st, n, nsc, world); break;
-    case DQ_BF16: hipLaunchKernelGGL(mean_center_kernel<DQ_BF16>, grid, block, 0, stream, src, residual, st, n, nsc, world); break;
-    default: hipLaunchKernelGGL(mean_center_kernel<DQ_F32>, grid, block, 0, stream, src, residual, st, n, nsc, world); break;
+    case DQ_F16: return run_mean_center<DQ_F16>(src, residual, stats, n, world_size, stream);
+    case DQ_BF16: return run_mean_center<DQ_BF16>(src, residual, stats, n, world_size, stream);
+    default: return run_mean_center<DQ_F32>(src, residual, stats, n, world_size, stream);
     }
-    return hipGetLastError();
 }
 
 hipError_t launch_add_mean_copy(const void *residual, void *dst, const void *stats, int64_t n, int dtype,

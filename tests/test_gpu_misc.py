@@ -43,6 +43,29 @@ def test_superchunk_mean_center_and_back(capi, oracle, dt, n, world):
     assert (out_d[n:] == 5.0).all()
 
 
+@pytest.mark.parametrize("dt", [F16, BF16, F32])
+def test_superchunk_mean_center_wide_range_and_worlds(capi, oracle, dt):
+    """every exponent (subnormal quotients, overflow to inf in fp16 squares), world sizes that are not
+    powers of two (the division must stay correctly rounded), a view that is not 16-byte aligned"""
+    tdt = TORCH_DT[dt]
+    n = 256 * 517 + 100
+    g = torch.Generator().manual_seed(31)
+    expo = torch.randint(-40 if dt != F16 else -24, 30 if dt != F16 else 12, (n,), generator=g).float()
+    src = (torch.randn(n, generator=g) * torch.pow(2.0, expo)).to(tdt)
+    src[1000:1256] = 0.0
+    nsc = (n + 255) // 256
+    for world, shift in ((1, 0), (2, 0), (3, 0), (5, 3), (6, 0), (7, 0), (8, 0), (12, 0), (64, 0), (100, 8)):
+        buf = torch.zeros(n + 16, dtype=tdt, device=DEV)
+        view = buf[shift:shift + n]
+        view.copy_(src)
+        res_d = torch.full((nsc * 256,), 7.0, dtype=tdt, device=DEV)
+        stats_d = torch.zeros(nsc * 2, dtype=torch.bfloat16, device=DEV)
+        capi.superchunk_mean_center(view, res_d, stats_d, n, world)
+        res_o, stats_o = oracle.superchunk_mean_center(to_bits(src), n, world, dt)
+        _eq("residual W=%d" % world, to_bits(res_d), res_o)
+        _eq("stats W=%d" % world, to_bits(stats_d), stats_o)
+
+
 def test_superchunk_constant_block(capi):
     """closed form: a constant block has residual 0 and stats (c/W, 256*(c/W)^2)"""
     c, W = 0.5, 4
