@@ -24,6 +24,7 @@ HIP_SOURCES = [
     "dq_api.hip",
     "dq_scaling_generic.hip",
     "dq_scaling_hier16.hip",
+    "dq_scaling_tile16.hip",
     "dq_grouping.hip",
     "dq_superchunk.hip",
     "dq_hadamard.hip",

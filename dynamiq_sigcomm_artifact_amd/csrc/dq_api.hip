@@ -180,10 +180,15 @@ inline bool dtype_rand_ok(int dtype)
     return dtype_ok(dtype & 0xf);
 }
 
-// the vectorised kernels cover the production shape
+// the production shape: one fused-capable vectorised kernel family
 inline bool hier16_shape(int dtype, int chunk_size, int strategy)
 {
     return (dtype == DQ_BF16 || dtype == DQ_F32) && chunk_size == 16 && strategy >= 2;
+}
+// every other chunk-16 shape: binary16 elements, flat strategies
+inline bool tile16_shape(int dtype, int chunk_size, int strategy)
+{
+    return chunk_size == 16 && !hier16_shape(dtype, chunk_size, strategy);
 }
 
 } // namespace
@@ -237,6 +242,8 @@ int dq_scaling_compress(const void *src, uint8_t *dst, const void *rand_pool, in
     const dq::MeeParams &mp = mee_params(nbits);
     if (hier16_shape(dtype & 0xf, chunk_size, strategy))
         return finish(dq::launch_hier16_compress(src, dst, rand_pool, n, nbits, dtype, strategy == 3, mp, s));
+    if (tile16_shape(dtype & 0xf, chunk_size, strategy))
+        return finish(dq::launch_tile16_compress(src, dst, rand_pool, n, nbits, dtype, strategy, mp, s));
     return finish(dq::launch_generic_compress(src, dst, rand_pool, n, nbits, chunk_size, dtype, strategy, mp, s));
 }
 
@@ -252,6 +259,8 @@ int dq_scaling_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, i
     const dq::MeeParams &mp = mee_params(nbits);
     if (hier16_shape(dtype, chunk_size, strategy))
         return finish(dq::launch_hier16_decompress(src, dst, n, nbits, dtype, strategy == 3, mp, add_original, s));
+    if (tile16_shape(dtype, chunk_size, strategy))
+        return finish(dq::launch_tile16_decompress(src, dst, n, nbits, dtype, strategy, mp, add_original, s));
     return finish(dq::launch_generic_decompress(src, dst, n, nbits, chunk_size, dtype, strategy, mp, add_original, s));
 }
 
@@ -268,6 +277,11 @@ int dq_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const voi
     if (hier16_shape(dtype & 0xf, chunk_size, strategy))
         return finish(dq::launch_hier16_dec_comp(recv, inp, send, rand_pool, n, nbits, dtype, strategy == 3, mp, s));
     // every other combination: decode into inp, then compress inp (two kernels, inp is modified)
+    if (tile16_shape(dtype & 0xf, chunk_size, strategy)) {
+        hipError_t e = dq::launch_tile16_decompress(recv, inp, n, nbits, dtype & 0xf, strategy, mp, 1, s);
+        if (e != hipSuccess) return finish(e);
+        return finish(dq::launch_tile16_compress(inp, send, rand_pool, n, nbits, dtype, strategy, mp, s));
+    }
     hipError_t e = dq::launch_generic_decompress(recv, inp, n, nbits, chunk_size, dtype & 0xf, strategy, mp, 1, s);
     if (e != hipSuccess) return finish(e);
     return finish(dq::launch_generic_compress(inp, send, rand_pool, n, nbits, chunk_size, dtype, strategy, mp, s));

@@ -185,7 +185,14 @@ __device__ __forceinline__ float mee_inverse_guarded(float x, float c, float l2b
 
 __device__ __forceinline__ float h_add(float a, float b) { return rh(a + b); }
 __device__ __forceinline__ float h_sub(float a, float b) { return rh(a - b); }
-__device__ __forceinline__ float h_mul(float a, float b) { return rh(a * b); }
+// The product passes through an empty asm: otherwise "round to binary16 of a * b" is selected as
+// v_fma_mixlo_f16 a, b, +0, and (-0) + (+0) turns a negative-zero product into +0.
+__device__ __forceinline__ float h_mul(float a, float b)
+{
+    float p = a * b;
+    asm("" : "+v"(p));
+    return rh(p);
+}
 __device__ __forceinline__ float h_div(float a, float b) { return rh(a / b); }
 __device__ __forceinline__ float h_max(float a, float b)
 {

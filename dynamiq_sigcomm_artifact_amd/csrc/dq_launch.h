@@ -29,6 +29,13 @@ hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t 
                                   const void *rnd, int64_t n, int nbits, int dtype, bool mee,
                                   const MeeParams &mp, hipStream_t stream);
 
+// vectorised chunk-16 kernels for the remaining shapes (dq_scaling_tile16.hip): binary16 elements
+// with any strategy, bf16 / fp32 elements with the flat strategies 0 / 1
+hipError_t launch_tile16_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n, int nbits,
+                                  int dtype, int strategy, const MeeParams &mp, hipStream_t stream);
+hipError_t launch_tile16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype,
+                                    int strategy, const MeeParams &mp, int add, hipStream_t stream);
+
 // the same kernels over a list of superchunk indices: record k <-> superchunk rows[k] of the
 // element buffer; recv != null makes compress the fused decode-accumulate-recompress step;
 // stats != null adds the destination superchunk's mean after decoding; elements >= limit are

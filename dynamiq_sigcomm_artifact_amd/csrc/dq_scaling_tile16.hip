@@ -1,0 +1,326 @@
+// Vectorised chunk-16 kernels for the shapes outside the production kernel of
+// dq_scaling_hier16.hip: binary16 elements (every strategy; all arithmetic is the
+// reference's op-by-op half arithmetic, i.e. an fp32 operation followed by one rounding to
+// binary16) and the flat strategies 0 / 1 for bf16 and fp32 elements (PB code bytes + a
+// 2-byte scale per chunk, no superchunk level).
+//
+// Same decomposition as the production kernel: one lane = one chunk (128-bit loads), one
+// single-wave workgroup = 64 chunks = one contiguous run of the packed stream, assembled in
+// (or pulled through) an LDS window whose offset equals the global address modulo 16;
+// decoded elements are transposed through a swizzled LDS tile so that every store
+// instruction covers 1 KiB.  Divisions by the chunk's scale use the exact double-reciprocal
+// product when every scale of the wave is an ordinary number, IEEE division otherwise.
+//
+// Numerics: csrc/cuda_hadamard.cu:768-861,941-1234 (flat), csrc/cuda_hierarchical_mee.cu:698-930
+// (binary16 hierarchical) of the reference.
+#include "dq_launch.h"
+#include "dq_tile16.cuh"
+
+namespace dq {
+
+namespace {
+
+constexpr int kChunksPerWave = 64;
+
+template <int NBITS, bool HIER> struct Geo {
+    static constexpr int PB = 2 * NBITS;
+    static constexpr int CB = HIER ? PB + 1 : PB + 2; // bytes of one chunk in the stream
+    static constexpr int REC = 16 * CB + 2;           // hierarchical record
+    static constexpr int FULL = HIER ? 4 * REC : kChunksPerWave * CB;
+    static constexpr int WIN = ((FULL + 15 + 15) / 16) * 16;
+    __device__ static __forceinline__ int bytes(int chunks) { return HIER ? (chunks >> 4) * REC : chunks * CB; }
+    __device__ static __forceinline__ int offset(int chunk) { return HIER ? (chunk >> 4) * REC + (chunk & 15) * CB : chunk * CB; }
+    __host__ __device__ static __forceinline__ int64_t stream_offset(int64_t chunk) { return HIER ? (chunk >> 4) * REC : chunk * CB; }
+};
+
+// maximum over a 16-lane row with the half-precision max rule (a NaN operand is dropped)
+__device__ __forceinline__ float row16_hmax(float v)
+{
+    v = h_max(v, dpp_f32<0xB1>(v));
+    v = h_max(v, dpp_f32<0x4E>(v));
+    v = h_max(v, dpp_f32<0x141>(v));
+    v = h_max(v, dpp_f32<0x140>(v));
+    return v;
+}
+
+// a scale the double-reciprocal division is proven for: normal, 2^-100 <= d <= 2^100
+__device__ __forceinline__ bool ordinary_scale(float d)
+{
+    const uint32_t b = __float_as_uint(d);
+    return b >= 0x0d800000u && b <= 0x71800000u;
+}
+
+template <int DT, int RDT, int NBITS, bool HIER, bool MEE>
+__global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restrict__ src, uint8_t *__restrict__ dst,
+                                                            const void *__restrict__ rnd, int64_t nchunks, int vec,
+                                                            MeeArg<NBITS, MEE> mp)
+{
+    typedef Geo<NBITS, HIER> G;
+    constexpr int R = Rec<NBITS>::R;
+    __shared__ __attribute__((aligned(16))) uint8_t win_out[G::WIN];
+
+    const int lane = threadIdx.x;
+    const int64_t c0 = (int64_t)blockIdx.x * kChunksPerWave;
+    if (c0 >= nchunks) return;
+    const int chunks_here = (int)min((int64_t)kChunksPerWave, nchunks - c0);
+    const bool active = lane < chunks_here;
+    const int total = G::bytes(chunks_here);
+
+    Raw16<DT> v;
+    Raw16<RDT> r;
+    if (active) {
+        v.load(src, (c0 + lane) * 16, vec & 1);
+        r.load(rnd, (c0 + lane) * 16, vec & 2);
+    } else {
+        v.zero();
+        r.zero();
+    }
+
+    float a = __builtin_fabsf(v.get(0));
+#pragma unroll
+    for (int i = 1; i < 16; i++) {
+        const float e = __builtin_fabsf(v.get(i));
+        a = (DT == DQ_F16) ? h_max(a, e) : __builtin_fmaxf(a, e);
+    }
+
+    float d;             // the scale the codes are computed against
+    uint32_t tail_bits;  // what follows the code bytes of this chunk: q (hier) or the 2-byte scale (flat)
+    uint32_t unit_bits = 0;
+    if (DT == DQ_F16) {
+        const float eps_h = rh(1e-7f);
+        const float s = h_add(h_div(a, MEE ? mp.cmm : (float)R), eps_h);
+        if (HIER) {
+            const float g = row16_hmax(s);
+            const float unit = h_div(g, 255.0f);
+            int q = sat_u16(__builtin_ceilf(h_mul(h_div(s, g), 255.0f)));
+            q = min(q, 255);
+            d = h_mul((float)q, unit);
+            tail_bits = (uint32_t)q;
+            unit_bits = f32_to_f16_bits(unit);
+        } else {
+            d = s;
+            tail_bits = f32_to_f16_bits(s);
+        }
+    } else {
+        // flat, fp32 arithmetic: the codes are computed against the bf16-rounded scale
+        tail_bits = f32_to_bf16_bits(MEE ? a / mp.cmm + 1e-7f : a / (float)R + 1e-7f);
+        d = bf16_bits_to_f32(tail_bits);
+    }
+
+    const bool fast = __builtin_amdgcn_ballot_w64(!ordinary_scale(d)) == 0;
+    const double yd = fast ? recip_f64(d) : 0.0;
+    uint32_t w[Rec<NBITS>::WORDS];
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float e = v.get(i);
+        float x = fast ? div_by(e, yd) : e / d;
+        int sv;
+        if (DT == DQ_F16) {
+            x = rh(x);
+            if (MEE) {
+                // mee_inverse_half with the divisions by the table constants done exactly
+                const float ax = __builtin_fabsf(x);
+                if (!(ax > 0.0f)) {
+                    x = 0.0f;
+                } else {
+                    const float arg = h_add(rh(div_by(ax, mp.inv_c)), 1.0f);
+                    const float lat = rh(div_by(rh(log2_det(arg)), mp.inv_l2b));
+                    x = x < 0.0f ? -lat : lat;
+                }
+            }
+            sv = sr_half(x, r.get(i));
+        } else {
+            if (MEE) {
+                const float ax = __builtin_fabsf(x);
+                if (!(ax > 0.0f)) {
+                    x = 0.0f;
+                } else {
+                    const float lat = div_by(log2_det(div_by(ax, mp.inv_c) + 1.0f), mp.inv_l2b);
+                    x = x < 0.0f ? -lat : lat;
+                }
+            }
+            sv = sr_plain(x, r.get(i));
+        }
+        words_put<NBITS>(w, i, (uint32_t)clamp_code(sv, R));
+    }
+
+    uint8_t *gout = dst + G::stream_offset(c0);
+    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
+    if (active) {
+        uint8_t *p = win_out + mis + G::offset(lane);
+        chunk_write<NBITS>(p, w, tail_bits); // PB code bytes + the low byte of tail_bits
+        if (!HIER) p[G::PB + 1] = (uint8_t)(tail_bits >> 8);
+        if (HIER && (lane & 15) == 0) {
+            p[16 * G::CB] = (uint8_t)unit_bits;
+            p[16 * G::CB + 1] = (uint8_t)(unit_bits >> 8);
+        }
+    }
+    wave_lds_sync();
+    window_flush(win_out, gout, mis, total, lane);
+}
+
+template <int DT, int NBITS, bool HIER, bool MEE, bool ADD>
+__global__ __launch_bounds__(64) void tile16_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
+                                                              int64_t nchunks, int vec, MeeArg<NBITS, MEE> mp)
+{
+    typedef Geo<NBITS, HIER> G;
+    constexpr int R = Rec<NBITS>::R;
+    constexpr int S = Raw16<DT>::kSlots;
+    __shared__ __attribute__((aligned(16))) uint8_t win_in[G::WIN];
+    __shared__ __attribute__((aligned(16))) uint4 tile_out[64 * S];
+    __shared__ float table[MEE ? (1 << NBITS) : 1];
+
+    const int lane = threadIdx.x;
+    const int64_t c0 = (int64_t)blockIdx.x * kChunksPerWave;
+    if (c0 >= nchunks) return;
+    const int chunks_here = (int)min((int64_t)kChunksPerWave, nchunks - c0);
+    const bool active = lane < chunks_here;
+    const int total = G::bytes(chunks_here);
+    const int64_t e0 = c0 * 16;
+    const uint8_t *gin = src + G::stream_offset(c0);
+
+    const WinRegs wr = window_fetch(gin, total, lane);
+    Raw16<DT> acc;
+    if (ADD && active) acc.load(dst, e0 + lane * 16, vec);
+    if (MEE) {
+        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
+    }
+    const int mis_in = window_commit(win_in, wr, gin, total, lane);
+    wave_lds_sync();
+
+    Raw16<DT> out;
+    if (active) {
+        const uint8_t *p = win_in + mis_in + G::offset(lane);
+        uint32_t cw[Rec<NBITS>::WORDS], tail;
+        chunk_read<NBITS>(p, cw, tail);
+        float sc;
+        if (HIER) {
+            const uint8_t *rec_end = win_in + mis_in + (lane >> 4) * G::REC + 16 * G::CB;
+            const uint32_t ub = (uint32_t)rec_end[0] | ((uint32_t)rec_end[1] << 8);
+            sc = h_mul((float)tail, f16_bits_to_f32(ub)); // HIER is instantiated for binary16 only
+        } else {
+            const uint32_t sb = tail | ((uint32_t)p[G::PB + 1] << 8);
+            sc = (DT == DQ_F16) ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb);
+        }
+        float t[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t code = words_get<NBITS>(cw, i);
+            const float lev = MEE ? table[code] : (float)((int)code - R);
+            if (DT == DQ_F16) {
+                const float val = h_mul(lev, sc);
+                t[i] = ADD ? h_add(acc.get(i), val) : val;
+            } else {
+                t[i] = ADD ? __builtin_fmaf(lev, sc, acc.get(i)) : lev * sc;
+            }
+        }
+        out.set(t);
+    } else {
+        out.zero();
+    }
+    if (vec) {
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < S; k++) tile_out[swz(S * lane + k)] = out.slot(k);
+        }
+        wave_lds_sync();
+        const int nslots = chunks_here * S;
+        uint4 *g = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + e0 * (DT == DQ_F32 ? 4 : 2));
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const int s = 64 * k + lane;
+            if (s < nslots) g[s] = tile_out[swz(s)];
+        }
+    } else if (active) {
+        out.store(dst, e0 + lane * 16, false);
+    }
+}
+
+inline unsigned grid_for(int64_t nchunks) { return (unsigned)((nchunks + kChunksPerWave - 1) / kChunksPerWave); }
+
+template <int DT, int RDT, int NBITS, bool MEE>
+hipError_t run_compress(const void *src, uint8_t *dst, const void *rnd, int64_t nchunks, bool hier, const MeeParams &mp,
+                        hipStream_t stream)
+{
+    auto arg = make_arg<NBITS, MEE>(mp);
+    const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
+    dim3 grid(grid_for(nchunks)), block(64);
+    if (DT == DQ_F16 && hier)
+        hipLaunchKernelGGL((tile16_compress_kernel<DQ_F16, DQ_F16, NBITS, true, MEE>), grid, block, 0, stream, src, dst, rnd, nchunks, vec, arg);
+    else
+        hipLaunchKernelGGL((tile16_compress_kernel<DT, RDT, NBITS, false, MEE>), grid, block, 0, stream, src, dst, rnd, nchunks, vec, arg);
+    return hipGetLastError();
+}
+
+template <int DT, int NBITS, bool MEE>
+hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nchunks, bool hier, int add, const MeeParams &mp,
+                          hipStream_t stream)
+{
+    auto arg = make_arg<NBITS, MEE>(mp);
+    const int vec = aligned16(dst) ? 1 : 0;
+    dim3 grid(grid_for(nchunks)), block(64);
+    if (DT == DQ_F16 && hier) {
+        if (add)
+            hipLaunchKernelGGL((tile16_decompress_kernel<DQ_F16, NBITS, true, MEE, true>), grid, block, 0, stream, src, dst, nchunks, vec, arg);
+        else
+            hipLaunchKernelGGL((tile16_decompress_kernel<DQ_F16, NBITS, true, MEE, false>), grid, block, 0, stream, src, dst, nchunks, vec, arg);
+    } else {
+        if (add)
+            hipLaunchKernelGGL((tile16_decompress_kernel<DT, NBITS, false, MEE, true>), grid, block, 0, stream, src, dst, nchunks, vec, arg);
+        else
+            hipLaunchKernelGGL((tile16_decompress_kernel<DT, NBITS, false, MEE, false>), grid, block, 0, stream, src, dst, nchunks, vec, arg);
+    }
+    return hipGetLastError();
+}
+
+#define DQ_T16_NBITS_MEE(FN, PRE, ...)                                                                    \
+    switch (nbits) {                                                                                      \
+    case 2: return mee ? FN<PRE, 2, true>(__VA_ARGS__) : FN<PRE, 2, false>(__VA_ARGS__);                  \
+    case 3: return mee ? FN<PRE, 3, true>(__VA_ARGS__) : FN<PRE, 3, false>(__VA_ARGS__);                  \
+    case 4: return mee ? FN<PRE, 4, true>(__VA_ARGS__) : FN<PRE, 4, false>(__VA_ARGS__);                  \
+    case 5: return mee ? FN<PRE, 5, true>(__VA_ARGS__) : FN<PRE, 5, false>(__VA_ARGS__);                  \
+    case 6: return mee ? FN<PRE, 6, true>(__VA_ARGS__) : FN<PRE, 6, false>(__VA_ARGS__);                  \
+    case 7: return mee ? FN<PRE, 7, true>(__VA_ARGS__) : FN<PRE, 7, false>(__VA_ARGS__);                  \
+    default: return mee ? FN<PRE, 8, true>(__VA_ARGS__) : FN<PRE, 8, false>(__VA_ARGS__);                 \
+    }
+#define DQ_T16_COMMA ,
+
+} // namespace
+
+// dtype F16 with any strategy, or BF16 / F32 with strategy 0 / 1; chunk size 16
+hipError_t launch_tile16_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n, int nbits, int dtype,
+                                  int strategy, const MeeParams &mp, hipStream_t stream)
+{
+    const bool rb16 = (dtype & DQ_RAND_BF16) != 0;
+    dtype &= 0xf;
+    const bool mee = (strategy & 1) != 0, hier = strategy >= 2;
+    const int64_t nchunks = n / 16;
+    if (dtype == DQ_F16) {
+        DQ_T16_NBITS_MEE(run_compress, DQ_F16 DQ_T16_COMMA DQ_F16, src, dst, rnd, nchunks, hier, mp, stream)
+    } else if (dtype == DQ_BF16) {
+        DQ_T16_NBITS_MEE(run_compress, DQ_BF16 DQ_T16_COMMA DQ_BF16, src, dst, rnd, nchunks, false, mp, stream)
+    } else if (rb16) {
+        DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_BF16, src, dst, rnd, nchunks, false, mp, stream)
+    } else {
+        DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_F32, src, dst, rnd, nchunks, false, mp, stream)
+    }
+}
+
+hipError_t launch_tile16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype, int strategy,
+                                    const MeeParams &mp, int add, hipStream_t stream)
+{
+    dtype &= 0xf;
+    const bool mee = (strategy & 1) != 0, hier = strategy >= 2;
+    const int64_t nchunks = n / 16;
+    if (dtype == DQ_F16) {
+        DQ_T16_NBITS_MEE(run_decompress, DQ_F16, src, dst, nchunks, hier, add, mp, stream)
+    } else if (dtype == DQ_BF16) {
+        DQ_T16_NBITS_MEE(run_decompress, DQ_BF16, src, dst, nchunks, false, add, mp, stream)
+    } else {
+        DQ_T16_NBITS_MEE(run_decompress, DQ_F32, src, dst, nchunks, false, add, mp, stream)
+    }
+}
+
+} // namespace dq

@@ -1,0 +1,335 @@
+// Building blocks shared by the vectorised chunk-16 kernels (dq_scaling_hier16.hip,
+// dq_scaling_tile16.hip): one lane owns one chunk of 16 elements, one wave owns a tile of
+// 64 chunks whose packed bytes form one contiguous run of the record stream.
+#pragma once
+
+#include "dq_device.cuh"
+
+namespace dq {
+
+constexpr int kRowsPerWave = 4; // superchunks per tile
+
+template <int NBITS> struct Rec {
+    static constexpr int R = (1 << (NBITS - 1)) - 1;
+    static constexpr int PB = 2 * NBITS;       // code bytes per chunk
+    static constexpr int CB = PB + 1;          // + one scale byte
+    static constexpr int REC = 16 * CB + 2;    // + bf16 unit
+    static constexpr int WORDS = (PB + 3) / 4; // dwords holding one chunk's codes
+    // LDS window: 4 records + up to 15 bytes of misalignment, padded to 16
+    static constexpr int WIN = ((kRowsPerWave * REC + 15 + 15) / 16) * 16;
+    static constexpr int WIN_VECS = WIN / 16;  // <= 70: at most two 128-bit registers per lane
+};
+
+template <int NBITS, bool MEE> struct MeeArg {
+    float c, cmm, l2b;
+    uint32_t pad;
+    double inv_c, inv_cmm, inv_l2b; // correctly rounded double reciprocals
+    uint16_t table[MEE ? (1 << NBITS) : 4];
+};
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+
+// ---- 16 raw elements of one lane ----------------------------------------------------
+
+template <int DT> struct Raw16;
+
+template <> struct Raw16<DQ_BF16> {
+    uint32_t w[8];
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int k = 0; k < 8; k++) w[k] = 0;
+    }
+    __device__ __forceinline__ void load(const void *p, int64_t e, bool vec)
+    {
+        // the unaligned path goes through volatile accesses so that the compiler cannot fold the two
+        // paths into one narrow-load sequence
+        const volatile uint16_t *h = static_cast<const volatile uint16_t *>(p) + e;
+        if (vec) {
+            const uint4 *q = reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(p) + e);
+            uint4 a = q[0], b = q[1];
+            w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) w[k] = (uint32_t)h[2 * k] | ((uint32_t)h[2 * k + 1] << 16);
+        }
+    }
+    __device__ __forceinline__ void store(void *p, int64_t e, bool vec) const
+    {
+        volatile uint16_t *h = static_cast<volatile uint16_t *>(p) + e;
+        if (vec) {
+            uint4 *q = reinterpret_cast<uint4 *>(static_cast<uint16_t *>(p) + e);
+            q[0] = make_uint4(w[0], w[1], w[2], w[3]);
+            q[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) { h[2 * k] = (uint16_t)w[k]; h[2 * k + 1] = (uint16_t)(w[k] >> 16); }
+        }
+    }
+    __device__ __forceinline__ float get(int i) const
+    {
+        return (i & 1) ? __uint_as_float(w[i >> 1] & 0xffff0000u) : __uint_as_float(w[i >> 1] << 16);
+    }
+    __device__ __forceinline__ void set(const float (&t)[16])
+    {
+#pragma unroll
+        for (int k = 0; k < 8; k++) w[k] = f32x2_to_bf16x2(t[2 * k], t[2 * k + 1]);
+    }
+    // binary32 bit pattern of max |element| in integer order (a NaN sorts above infinity)
+    __device__ __forceinline__ uint32_t absmax_bits() const
+    {
+        uint32_t m = w[0] & 0x7fff7fffu;
+#pragma unroll
+        for (int k = 1; k < 8; k++) m = pk_max_u16(m, w[k] & 0x7fff7fffu);
+        return max(m << 16, m & 0xffff0000u);
+    }
+    // every element in [+0, 1]
+    __device__ __forceinline__ bool unit_interval() const
+    {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int k = 1; k < 8; k++) m = pk_max_u16(m, w[k]);
+        return max(m & 0xffffu, m >> 16) <= 0x3f80u;
+    }
+    static constexpr int kSlots = 2; // 16-byte pieces per lane
+    __device__ __forceinline__ uint4 slot(int j) const { return make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]); }
+};
+
+template <> struct Raw16<DQ_F32> {
+    uint32_t w[16];
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int k = 0; k < 16; k++) w[k] = 0;
+    }
+    __device__ __forceinline__ void load(const void *p, int64_t e, bool vec)
+    {
+        const volatile uint32_t *f = static_cast<const volatile uint32_t *>(p) + e;
+        if (vec) {
+            const uint4 *q = reinterpret_cast<const uint4 *>(static_cast<const uint32_t *>(p) + e);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                uint4 t = q[k];
+                w[4 * k] = t.x; w[4 * k + 1] = t.y; w[4 * k + 2] = t.z; w[4 * k + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++) w[k] = f[k];
+        }
+    }
+    __device__ __forceinline__ void store(void *p, int64_t e, bool vec) const
+    {
+        volatile uint32_t *f = static_cast<volatile uint32_t *>(p) + e;
+        if (vec) {
+            uint4 *q = reinterpret_cast<uint4 *>(static_cast<uint32_t *>(p) + e);
+#pragma unroll
+            for (int k = 0; k < 4; k++) q[k] = make_uint4(w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++) f[k] = w[k];
+        }
+    }
+    __device__ __forceinline__ float get(int i) const { return __uint_as_float(w[i]); }
+    __device__ __forceinline__ void set(const float (&t)[16])
+    {
+#pragma unroll
+        for (int k = 0; k < 16; k++) w[k] = __float_as_uint(t[k]);
+    }
+    __device__ __forceinline__ uint32_t absmax_bits() const
+    {
+        uint32_t m = w[0] & 0x7fffffffu;
+#pragma unroll
+        for (int k = 1; k < 16; k++) m = max(m, w[k] & 0x7fffffffu);
+        return m;
+    }
+    __device__ __forceinline__ bool unit_interval() const
+    {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int k = 1; k < 16; k++) m = max(m, w[k]);
+        return m <= 0x3f800000u;
+    }
+    static constexpr int kSlots = 4;
+    __device__ __forceinline__ uint4 slot(int j) const { return make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]); }
+};
+
+// binary16 elements: the storage and the moves of the bf16 case, other conversions
+template <> struct Raw16<DQ_F16> : Raw16<DQ_BF16> {
+    __device__ __forceinline__ float get(int i) const { return f16_bits_to_f32((w[i >> 1] >> (16 * (i & 1))) & 0xffffu); }
+    __device__ __forceinline__ void set(const float (&t)[16])
+    {
+#pragma unroll
+        for (int k = 0; k < 8; k++) w[k] = f32_to_f16_bits(t[2 * k]) | (f32_to_f16_bits(t[2 * k + 1]) << 16);
+    }
+    // binary16 bit pattern of max |element| in integer order (a NaN sorts above infinity)
+    __device__ __forceinline__ uint32_t absmax_half_bits() const
+    {
+        uint32_t m = w[0] & 0x7fff7fffu;
+#pragma unroll
+        for (int k = 1; k < 8; k++) m = pk_max_u16(m, w[k] & 0x7fff7fffu);
+        return max(m & 0xffffu, m >> 16);
+    }
+    // every element in [+0, 1]
+    __device__ __forceinline__ bool unit_interval() const
+    {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int k = 1; k < 8; k++) m = pk_max_u16(m, w[k]);
+        return max(m & 0xffffu, m >> 16) <= 0x3c00u;
+    }
+};
+
+// ---- record windows --------------------------------------------------------------------
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// the (up to two) aligned 128-bit pieces of a packed run this lane moves
+struct WinRegs {
+    u32x4 a, b;
+};
+
+// every lane loads (indices are clamped into the run), so the registers are
+// always defined and the prefetch is two plain vector loads
+__device__ __forceinline__ WinRegs window_fetch(const uint8_t *g, int total, int lane)
+{
+    const int mis = (int)(reinterpret_cast<uintptr_t>(g) & 15);
+    const u32x4 *ga = reinterpret_cast<const u32x4 *>(g - mis);
+    const int nvec = (mis + total + 15) >> 4;
+    WinRegs r;
+    r.a = ga[min(lane, nvec - 1)];
+    r.b = ga[min(lane + 64, nvec - 1)];
+    return r;
+}
+
+// byte k of the run lands at win[(g & 15) + k]
+__device__ __forceinline__ int window_commit(uint8_t *win, const WinRegs &r, const uint8_t *g, int total, int lane)
+{
+    const int mis = (int)(reinterpret_cast<uintptr_t>(g) & 15);
+    const int nvec = (mis + total + 15) >> 4;
+    if (lane < nvec) reinterpret_cast<u32x4 *>(win)[lane] = r.a;
+    if (lane + 64 < nvec) reinterpret_cast<u32x4 *>(win)[lane + 64] = r.b;
+    return mis;
+}
+
+// stream `total` bytes from win[mis ...] to g (g & 15 == mis)
+__device__ __forceinline__ void window_flush(const uint8_t *win, uint8_t *g, int mis, int total, int lane)
+{
+    int head = (16 - mis) & 15;
+    head = min(head, total);
+    const int body = (total - head) & ~15;
+    const int tail = total - head - body;
+    if (lane < head) g[lane] = win[mis + lane];
+    const uint4 *wv = reinterpret_cast<const uint4 *>(win + mis + head);
+    uint4 *gv = reinterpret_cast<uint4 *>(g + head);
+    for (int v = lane; v < (body >> 4); v += 64) gv[v] = wv[v];
+    const int tl = lane - 32; // lanes 32.. store the tail so head and tail overlap in time
+    if (tl >= 0 && tl < tail) g[head + body + tl] = win[mis + head + body + tl];
+}
+
+// LDS accesses of one wave execute in order; the fence only stops the compiler
+// from moving them across the hand-over between lanes
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---- per-chunk code words -----------------------------------------------------------------
+
+template <int NBITS> __device__ __forceinline__ void words_put(uint32_t (&w)[Rec<NBITS>::WORDS], int i, uint32_t code)
+{
+    const int bit = i * NBITS;
+    w[bit >> 5] |= code << (bit & 31);
+    if ((bit & 31) + NBITS > 32) w[(bit >> 5) + 1] |= code >> (32 - (bit & 31));
+}
+
+template <int NBITS> __device__ __forceinline__ uint32_t words_get(const uint32_t (&w)[Rec<NBITS>::WORDS], int i)
+{
+    const int bit = i * NBITS;
+    uint32_t v = w[bit >> 5] >> (bit & 31);
+    if ((bit & 31) + NBITS > 32) v |= w[(bit >> 5) + 1] << (32 - (bit & 31));
+    return v & ((1u << NBITS) - 1u);
+}
+
+// one chunk's CB bytes (codes + scale byte) from / to a window
+template <int NBITS>
+__device__ __forceinline__ void chunk_read(const uint8_t *p, uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q)
+{
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::PB; k++) w[k >> 2] |= (uint32_t)p[k] << (8 * (k & 3));
+    q = p[Rec<NBITS>::PB];
+}
+
+template <int NBITS>
+__device__ __forceinline__ void chunk_write(uint8_t *p, const uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t q)
+{
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::PB; k++) p[k] = (uint8_t)(w[k >> 2] >> (8 * (k & 3)));
+    p[Rec<NBITS>::PB] = (uint8_t)q;
+}
+
+// ---- exact division by a chunk constant ------------------------------------------------------
+
+// 1/b in double to within one double ulp, b a normal binary32 in [2^-100, 2^100]
+__device__ __forceinline__ double recip_f64(float b)
+{
+    const double bd = (double)b;
+    double y = (double)__builtin_amdgcn_rcpf(b);
+    double e = __builtin_fma(-bd, y, 1.0);
+    y = __builtin_fma(y, e, y);
+    e = __builtin_fma(-bd, y, 1.0);
+    y = __builtin_fma(y, e, y);
+    return y;
+}
+
+// correctly rounded binary32 quotient a / b given yb ~= 1/b in double
+__device__ __forceinline__ float div_by(float a, double yb) { return (float)((double)a * yb); }
+
+// log2_det() for a finite argument >= 1 (same operations, special cases dropped)
+__device__ __forceinline__ float log2_det_ge1(float x)
+{
+    const uint32_t ix = __float_as_uint(x);
+    const uint32_t t = ix - 0x3f3504f3u;
+    const int k = (int)t >> 23;
+    const float z = __uint_as_float(ix - (t & 0xff800000u));
+    const float f = z - 1.0f;
+    float q = -0x1.d0dd08p-4f;
+    q = __builtin_fmaf(q, f, 0x1.7ad622p-3f);
+    q = __builtin_fmaf(q, f, -0x1.831b24p-3f);
+    q = __builtin_fmaf(q, f, 0x1.a33bdap-3f);
+    q = __builtin_fmaf(q, f, -0x1.eb492p-3f);
+    q = __builtin_fmaf(q, f, 0x1.277e38p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715762p-2f);
+    q = __builtin_fmaf(q, f, 0x1.ec7092p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715476p-1f);
+    const float p = (f * f) * q;
+    float r = __builtin_fmaf(f, 0x1.4ae0cp-26f, p);
+    r = __builtin_fmaf(f, 0x1.715476p+0f, r);
+    return (float)k + r;
+}
+
+// 16-byte slot s of a wave's output tile lives at LDS slot s ^ ((s >> 3) & 7): both
+// the per-lane writes (slots S*lane + j) and the lane-contiguous reads (slots
+// 64*k + lane) then touch eight distinct bank groups per eight lanes
+__device__ __forceinline__ int swz(int s) { return s ^ ((s >> 3) & 7); }
+
+template <int NBITS, bool MEE> static MeeArg<NBITS, MEE> make_arg(const MeeParams &mp)
+{
+    MeeArg<NBITS, MEE> a;
+    a.c = mp.c; a.cmm = mp.cmm; a.l2b = mp.l2b; a.pad = 0;
+    a.inv_c = 1.0 / (double)mp.c; a.inv_cmm = 1.0 / (double)mp.cmm; a.inv_l2b = 1.0 / (double)mp.l2b;
+    for (int k = 0; k < (MEE ? (1 << NBITS) : 4); k++) a.table[k] = mp.table[k];
+    return a;
+}
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+} // namespace dq

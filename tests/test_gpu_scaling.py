@@ -144,6 +144,80 @@ def test_special_values(capi, oracle, dt, strategy):
         _roundtrip_nan_safe(capi, oracle, dt, n, nbits, 16, strategy, src, rnd, "special b=%d" % nbits)
 
 
+def _wide_source(n, tdt, seed):
+    """random magnitudes over the whole exponent range of the type, plus zeros, infinities, NaN and
+    values the type cannot hold without rounding to the extremes"""
+    g = torch.Generator().manual_seed(seed)
+    lo, hi = (-24, 15) if tdt == torch.float16 else (-60, 60)
+    expo = torch.randint(lo, hi, (n // 16,), generator=g).float().repeat_interleave(16)
+    src = torch.randn(n, generator=g) * torch.pow(2.0, expo) * torch.pow(2.0, torch.randint(-6, 1, (n,), generator=g).float())
+    src[0:64] = 0.0
+    src[100] = float("inf")
+    src[333] = float("-inf")
+    src[517] = float("nan")
+    src[640:656] = float("nan")            # a whole chunk of NaN
+    src[700:716] = 65504.0 if tdt == torch.float16 else 3.0e38
+    return src.to(tdt)
+
+
+@pytest.mark.parametrize("dt,strategies", [(F16, (0, 1, 2, 3)), (BF16, (0, 1)), (F32, (0, 1))])
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+def test_tile16_shapes(capi, oracle, dt, strategies, nbits):
+    """chunk 16 outside the production kernel -- binary16 elements, flat strategies: ordinary data over
+    several tiles with a ragged last tile, then the special values; the ring step is the split one"""
+    tdt = TORCH_DT[dt]
+    for strategy in strategies:
+        n = 16 * (64 * 5 + 16 * 3 + (0 if strategy >= 2 else 7))
+        g = torch.Generator().manual_seed(nbits * 10 + strategy)
+        src = (torch.randn(n, generator=g) * 1e-2).to(tdt)
+        rnd = torch.rand(n, generator=g).to(tdt)
+        tag = "tile16 dt=%d b=%d s=%d" % (dt, nbits, strategy)
+        _roundtrip(capi, oracle, dt, n, nbits, 16, strategy, src, rnd, tag)
+        inp = (torch.randn(n, generator=g) * 1e-2).to(tdt)
+        _dec_comp(capi, oracle, dt, n, nbits, 16, strategy, src, inp, rnd, torch.rand(n, generator=g).to(tdt), tag)
+        wide = _wide_source(n, tdt, nbits + strategy)
+        rnd2 = torch.rand(n, generator=g)
+        rnd2[::7] = 0.0
+        rnd2[3::11] = 1.0
+        _roundtrip(capi, oracle, dt, n, nbits, 16, strategy, wide, rnd2.to(tdt), tag + " wide")
+
+
+def test_tile16_unaligned_and_mixed_pool(capi, oracle):
+    """element views off the 16-byte grid, packed pointers at odd chunk offsets, bf16 pool beside fp32 elements"""
+    g = torch.Generator().manual_seed(77)
+    n = 16 * 151
+    for tdt, dt, strategy, nbits in ((torch.float16, F16, 2, 4), (torch.float16, F16, 1, 8), (torch.bfloat16, BF16, 0, 4),
+                                     (torch.float32, F32, 1, 5)):
+        if strategy >= 2:
+            n = 256 * 9
+        src_t = (torch.randn(n, generator=g) * 1e-3).to(tdt)
+        rnd_t = torch.rand(n, generator=g).to(tdt)
+        nbytes = oracle.required_bytes(n, nbits, 16, strategy)
+        enc_o = oracle.scaling_compress(to_bits(src_t), to_bits(rnd_t), n, nbits, 16, strategy, dt)
+        big_src = torch.zeros(n + 64, dtype=tdt, device=DEV)
+        big_rnd = torch.zeros(n + 64, dtype=tdt, device=DEV)
+        big_src[3:3 + n] = src_t.to(DEV)
+        big_rnd[1:1 + n] = rnd_t.to(DEV)
+        for off in (1, 7, 16):
+            buf = torch.zeros(nbytes + 32, dtype=torch.uint8, device=DEV)
+            capi.scaling_compress(big_src[3:3 + n], buf[off:], big_rnd[1:1 + n], n, nbits, 16, strategy)
+            got = buf.cpu().numpy()
+            assert (got[:off] == 0).all() and (got[off + nbytes:] == 0).all()
+            assert (got[off:off + nbytes] == enc_o).all()
+            out = torch.zeros(n + 8, dtype=tdt, device=DEV)
+            capi.scaling_decompress(buf[off:], out[5:5 + n], n, nbits, 16, strategy)
+            dec_o = np.zeros(n, np.float32 if dt == F32 else np.uint16)
+            oracle.scaling_decompress(enc_o, dec_o, n, nbits, 16, strategy, dt)
+            _cmp_bits("unaligned", to_bits(out[5:5 + n]), dec_o)
+            assert float(out[:5].abs().sum()) == 0.0 and float(out[5 + n:].abs().sum()) == 0.0
+    # fp32 elements with a bf16 pool, flat
+    src = torch.randn(n, generator=g) * 1e-3
+    rnd16 = torch.rand(n, generator=g).to(torch.bfloat16)
+    enc_d = torch.zeros(oracle.required_bytes(n, 4, 16, 0), dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(src.to(DEV), enc_d, rnd16.to(DEV), n, 4, 16, 0)
+    _cmp_bits("mixed flat", enc_d.cpu().numpy(), oracle.scaling_compress(to_bits(src), to_bits(rnd16.float()), n, 4, 16, 0, F32))
+
+
 def test_fp32_gradient_with_bf16_rand_pool(capi, oracle):
     """fp32 elements + bf16 random pool (DQ_RAND_BF16) == fp32 elements + the same values widened"""
     g = torch.Generator().manual_seed(21)
