@@ -29,6 +29,7 @@ HIP_SOURCES = [
     "dq_superchunk.hip",
     "dq_hadamard.hip",
     "dq_packing.hip",
+    "dq_eden.hip",
 ]
 
 HIPCC_FLAGS = [

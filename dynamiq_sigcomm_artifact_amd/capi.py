@@ -25,6 +25,7 @@ EXPORTS = [
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
+    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_thc_quantize", "dq_thc_dequantize",
 ]
 
 _lib = None
@@ -86,6 +87,16 @@ def lib():
         L.dq_bins_to_bits.argtypes = [vp, i64, vp, i64, i32, i32, vp]
         L.dq_bits_to_bins.restype = i32
         L.dq_bits_to_bins.argtypes = [vp, i64, vp, i64, i32, i32, vp]
+        L.dq_eden_work_doubles.restype = i64
+        L.dq_eden_work_doubles.argtypes = [i64]
+        L.dq_eden_quantize.restype = i32
+        L.dq_eden_quantize.argtypes = [vp, i64, vp, vp, i32, vp, vp, vp, i64, i32, vp]
+        L.dq_eden_dequantize.restype = i32
+        L.dq_eden_dequantize.argtypes = [vp, i64, vp, i32, vp, i32, vp]
+        L.dq_thc_quantize.restype = i32
+        L.dq_thc_quantize.argtypes = [vp, vp, vp, i64, vp, vp, i32, i32, vp]
+        L.dq_thc_dequantize.restype = i32
+        L.dq_thc_dequantize.argtypes = [vp, vp, i64, vp, vp, i32, vp]
         L.dq_quantization.restype = i32
         L.dq_quantization.argtypes = [vp, i64, i32, f32, f32, u64, vp]
         _lib = L
@@ -238,3 +249,53 @@ def bits_to_bins(bins, arr, nbits, stream=None):
 def quantization(vec, div_factor, tensor_max, seed, stream=None):
     _check(lib().dq_quantization(vec.data_ptr(), vec.numel(), _dev(vec), float(div_factor), float(tensor_max), int(seed),
                                  _stream(stream)))
+
+
+def eden_work_doubles(n):
+    return int(lib().dq_eden_work_doubles(n))
+
+
+def eden_quantize(vec, boundaries, centroids, nbits, packed, result, work, stream=None):
+    """vec float32 [n] -> packed int32/uint32 [n / 32 * nbits], result float32 [4] = (sumsq, dot, scale, norm)"""
+    for t, name in ((vec, "vec"), (boundaries, "boundaries"), (centroids, "centroids"), (result, "result")):
+        if t.dtype != torch.float32:
+            raise RuntimeError("eden_quantize: %s must be float32" % name)
+    if packed.dtype != torch.int32 or work.dtype != torch.float64:
+        raise RuntimeError("eden_quantize: packed must be int32 and work float64")
+    n = vec.numel()
+    if boundaries.numel() < (1 << nbits) - 1 or centroids.numel() < (1 << nbits) or result.numel() < 4 \
+            or packed.numel() < n // 32 * nbits:
+        raise RuntimeError("eden_quantize: a buffer is too small")
+    _check(lib().dq_eden_quantize(vec.data_ptr(), n, boundaries.data_ptr(), centroids.data_ptr(), nbits, packed.data_ptr(),
+                                  result.data_ptr(), work.data_ptr(), work.numel(), _dev(vec), _stream(stream)))
+
+
+def eden_dequantize(packed, n, centroids, nbits, out, stream=None):
+    if packed.dtype != torch.int32 or centroids.dtype != torch.float32 or out.dtype != torch.float32:
+        raise RuntimeError("eden_dequantize: packed must be int32, centroids and out float32")
+    if packed.numel() < n // 32 * nbits or out.numel() < n or centroids.numel() < (1 << nbits):
+        raise RuntimeError("eden_dequantize: a buffer is too small")
+    _check(lib().dq_eden_dequantize(packed.data_ptr(), n, centroids.data_ptr(), nbits, out.data_ptr(), _dev(out),
+                                    _stream(stream)))
+
+
+def thc_quantize(rotated, uniform, levels_out, lo, delta, levels, stream=None):
+    if rotated.dtype != torch.float32 or uniform.dtype != torch.float32 or levels_out.dtype != torch.bfloat16 \
+            or lo.dtype != torch.float32 or delta.dtype != torch.float32:
+        raise RuntimeError("thc_quantize: rotated, uniform, lo, delta must be float32 and the output bfloat16")
+    n = rotated.numel()
+    if uniform.numel() < n or levels_out.numel() < n:
+        raise RuntimeError("thc_quantize: a buffer is too small")
+    _check(lib().dq_thc_quantize(rotated.data_ptr(), uniform.data_ptr(), levels_out.data_ptr(), n, lo.data_ptr(),
+                                 delta.data_ptr(), levels, _dev(rotated), _stream(stream)))
+
+
+def thc_dequantize(levels_in, out, step, lo, stream=None):
+    if levels_in.dtype != torch.bfloat16 or out.dtype != torch.float32 or step.dtype != torch.float32 \
+            or lo.dtype != torch.float32:
+        raise RuntimeError("thc_dequantize: levels must be bfloat16, out, step, lo float32")
+    n = levels_in.numel()
+    if out.numel() < n:
+        raise RuntimeError("thc_dequantize: out is too small")
+    _check(lib().dq_thc_dequantize(levels_in.data_ptr(), out.data_ptr(), n, step.data_ptr(), lo.data_ptr(), _dev(out),
+                                   _stream(stream)))

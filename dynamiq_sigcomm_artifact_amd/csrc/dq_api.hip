@@ -437,6 +437,53 @@ int dq_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int64_t n
     return finish(dq::launch_bits_to_bins(bins, nbins, arr, nbits, static_cast<hipStream_t>(stream)));
 }
 
+int64_t dq_eden_work_doubles(int64_t n) { return n > 0 ? dq::eden_work_doubles(n) : 1; }
+
+int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids, int nbits,
+                     uint32_t *packed, float *result, double *work, int64_t work_doubles, int device, dq_stream_t stream)
+{
+    if (!(n > 0) || (n & 31) != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of 32");
+    if (nbits < 1 || nbits > 8) return fail(DQ_ERR_NBITS, "nbits must be in [1, 8]");
+    if (!vec || !boundaries || !centroids || !packed || !result || !work) return fail(DQ_ERR_NULL);
+    if (work_doubles < dq::eden_work_doubles(n)) return fail(DQ_ERR_SIZE, "work buffer is too small");
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_eden_quantize(vec, n, boundaries, centroids, nbits, packed, result, work,
+                                           static_cast<hipStream_t>(stream)));
+}
+
+int dq_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits, float *out, int device,
+                       dq_stream_t stream)
+{
+    if (!(n > 0) || (n & 31) != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of 32");
+    if (nbits < 1 || nbits > 8) return fail(DQ_ERR_NBITS, "nbits must be in [1, 8]");
+    if (!packed || !centroids || !out) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_eden_dequantize(packed, n, centroids, nbits, out, static_cast<hipStream_t>(stream)));
+}
+
+int dq_thc_quantize(const float *rotated, const float *uniform, void *levels_bf16, int64_t n, const float *lo,
+                    const float *delta, int levels, int device, dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (levels < 2 || levels > 256) return fail(DQ_ERR_SIZE, "levels must be in [2, 256]");
+    if (!rotated || !uniform || !levels_bf16 || !lo || !delta) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_thc_quantize(rotated, uniform, levels_bf16, n, lo, delta, levels, static_cast<hipStream_t>(stream)));
+}
+
+int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const float *step, const float *lo, int device,
+                      dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (!levels_bf16 || !out || !step || !lo) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_thc_dequantize(levels_bf16, out, n, step, lo, static_cast<hipStream_t>(stream)));
+}
+
 int dq_quantization(float *vec, int64_t n, int device, float div_factor, float tensor_max, uint64_t seed,
                     dq_stream_t stream)
 {

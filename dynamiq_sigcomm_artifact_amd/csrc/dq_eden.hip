@@ -1,0 +1,253 @@
+// The consumers of the rotated vector: EDEN's Lloyd-Max quantiser with its bit-plane packer
+// (cuda_kernels/src/srrcomp/srrcomp.py:293-361) and THC's uniform stochastic quantiser
+// (testbed_evaluation/new_comm_hooks/thc_hooks.py:149-181), which the reference runs as chains of
+// torch element-wise ops and reductions around eden_utils.Hadamard.
+//
+// EDEN quantise, four launches, no host synchronisation:
+//   sumsq   tile b = elements [4096 b, 4096 b + 4096): thread t adds v^2 of elements t + 256 k (k ascending)
+//           in double, the 256 sums are halved (stride 128 .. 1) -> work[b]
+//   norm    one workgroup folds work[] the same way -> sumsq (double); norm = sqrtf((float)sumsq)
+//   bins    x = (v * (float)sqrt(n)) / norm; bin = number of boundaries < x (torch.bucketize, right=False);
+//           bit plane p of 32 consecutive bins -> packed[p * n/32 + w]; the products centroid[bin] * v are
+//           summed in double with the tile scheme above -> work[b]
+//   scale   dot = fold(work[]); scale = (norm * norm) / (float)dot
+// The sums are in double with a fixed association, so the result does not depend on the launch geometry
+// and the CPU restatement reproduces it bit for bit.
+#include "dq_launch.h"
+#include "dq_tile16.cuh"
+
+namespace dq {
+
+namespace {
+
+constexpr int kEdenThreads = 256;
+constexpr int kEdenPerThread = 16;
+constexpr int kEdenTile = kEdenThreads * kEdenPerThread; // 4096 elements
+
+// sum[l] += sum[l + stride], stride 128 .. 1; returns the total in every thread
+__device__ __forceinline__ double fold256(double v, double *lds)
+{
+    const int t = threadIdx.x;
+    lds[t] = v;
+    __syncthreads();
+#pragma unroll
+    for (int stride = 128; stride > 0; stride >>= 1) {
+        if (t < stride) lds[t] += lds[t + stride];
+        __syncthreads();
+    }
+    const double total = lds[0];
+    __syncthreads();
+    return total;
+}
+
+__global__ __launch_bounds__(kEdenThreads) void eden_sumsq_kernel(const float *__restrict__ vec, int64_t n,
+                                                                 double *__restrict__ work)
+{
+    __shared__ double lds[kEdenThreads];
+    const int64_t base = (int64_t)blockIdx.x * kEdenTile;
+    double acc = 0.0;
+#pragma unroll
+    for (int k = 0; k < kEdenPerThread; k++) {
+        const int64_t i = base + threadIdx.x + (int64_t)kEdenThreads * k;
+        if (i < n) {
+            const double v = (double)vec[i];
+            acc += v * v;
+        }
+    }
+    const double total = fold256(acc, lds);
+    if (threadIdx.x == 0) work[blockIdx.x] = total;
+}
+
+// folds work[0 .. count): thread t adds entries t + 256 k (k ascending), then the halving tree
+__device__ __forceinline__ double fold_array(const double *work, int64_t count, double *lds)
+{
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < count; i += kEdenThreads) acc += work[i];
+    return fold256(acc, lds);
+}
+
+// result[0] = (float)sumsq, result[3] = norm
+__global__ __launch_bounds__(kEdenThreads) void eden_norm_kernel(const double *__restrict__ work, int64_t count,
+                                                                float *__restrict__ result)
+{
+    __shared__ double lds[kEdenThreads];
+    const double sumsq = fold_array(work, count, lds);
+    if (threadIdx.x == 0) {
+        const float s = (float)sumsq;
+        result[0] = s;
+        result[3] = __builtin_sqrtf(s);
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__restrict__ vec, int64_t n,
+                                                                const float *__restrict__ boundaries,
+                                                                const float *__restrict__ centroids,
+                                                                const float *__restrict__ result, float sqrt_n,
+                                                                uint32_t *__restrict__ packed, double *__restrict__ work)
+{
+    constexpr int L = 1 << NBITS;
+    __shared__ double lds[kEdenThreads];
+    __shared__ float bnd[L], cen[L];
+    for (int k = threadIdx.x; k < L; k += kEdenThreads) {
+        bnd[k] = k < L - 1 ? boundaries[k] : 0.0f;
+        cen[k] = centroids[k];
+    }
+    __syncthreads();
+    const float norm = result[3];
+    const uint32_t nb = __float_as_uint(norm);
+    const bool ordinary = nb >= 0x0d800000u && nb <= 0x71800000u; // uniform over the grid
+    const double yn = ordinary ? recip_f64(norm) : 0.0;
+    const int64_t words = n >> 5;
+    const int64_t base = (int64_t)blockIdx.x * kEdenTile;
+    const int lane = threadIdx.x & 63;
+    double acc = 0.0;
+#pragma unroll 4
+    for (int k = 0; k < kEdenPerThread; k++) {
+        const int64_t i = base + threadIdx.x + (int64_t)kEdenThreads * k;
+        const bool in = i < n;
+        const float v = in ? vec[i] : 0.0f;
+        const float scaled = v * sqrt_n;
+        const float x = ordinary ? div_by(scaled, yn) : scaled / norm;
+        int bin = 0;
+#pragma unroll
+        for (int step = L >> 1; step > 0; step >>= 1) {
+            if (bnd[bin + step - 1] < x) bin += step;
+        }
+        if (in) acc += (double)cen[bin] * (double)v;
+        const int64_t w = i >> 5;
+#pragma unroll
+        for (int p = 0; p < NBITS; p++) {
+            const uint64_t m = __ballot(in && ((bin >> p) & 1));
+            if ((lane & 31) == 0 && in) packed[(int64_t)p * words + w] = (uint32_t)(m >> (lane & 32));
+        }
+    }
+    const double total = fold256(acc, lds);
+    if (threadIdx.x == 0) work[blockIdx.x] = total;
+}
+
+// result[1] = (float)dot, result[2] = scale
+__global__ __launch_bounds__(kEdenThreads) void eden_scale_kernel(const double *__restrict__ work, int64_t count,
+                                                                 float *__restrict__ result)
+{
+    __shared__ double lds[kEdenThreads];
+    const double dot = fold_array(work, count, lds);
+    if (threadIdx.x == 0) {
+        const float d = (float)dot;
+        const float norm = result[3];
+        result[1] = d;
+        result[2] = (norm * norm) / d;
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void eden_dequantize_kernel(const uint32_t *__restrict__ packed, int64_t n,
+                                                              const float *__restrict__ centroids, float *__restrict__ out)
+{
+    constexpr int L = 1 << NBITS;
+    __shared__ float cen[L];
+    for (int k = threadIdx.x; k < L; k += 256) cen[k] = centroids[k];
+    __syncthreads();
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t words = n >> 5, w = i >> 5;
+    const int t = (int)(i & 31);
+    int bin = 0;
+#pragma unroll
+    for (int p = 0; p < NBITS; p++) bin |= (int)((packed[(int64_t)p * words + w] >> t) & 1u) << p;
+    out[i] = cen[bin];
+}
+
+// ---- THC ------------------------------------------------------------------------------------------
+
+// x = clamp((v - lo) / delta, 0, levels - 1); level = floor(x) + (u < x - floor(x)); stored as bf16
+__global__ __launch_bounds__(256) void thc_quantize_kernel(const float *__restrict__ rotated, const float *__restrict__ uniform,
+                                                           uint16_t *__restrict__ out, int64_t n,
+                                                           const float *__restrict__ lo_p, const float *__restrict__ delta_p,
+                                                           float top)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float lo = *lo_p, delta = *delta_p;
+    float x = (rotated[i] - lo) / delta;
+    // torch.clamp_ keeps NaN
+    if (x < 0.0f) x = 0.0f;
+    if (x > top) x = top;
+    const float fl = __builtin_floorf(x);
+    const float prob = x - fl;
+    const float level = fl + ((uniform[i] < prob) ? 1.0f : 0.0f);
+    out[i] = (uint16_t)f32_to_bf16_bits(level);
+}
+
+// v = float(level sum) * step + lo, two roundings
+__global__ __launch_bounds__(256) void thc_dequantize_kernel(const uint16_t *__restrict__ levels, float *__restrict__ out,
+                                                             int64_t n, const float *__restrict__ step_p,
+                                                             const float *__restrict__ lo_p)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float prod = bf16_bits_to_f32(levels[i]) * *step_p;
+    out[i] = prod + *lo_p;
+}
+
+inline int64_t eden_tiles(int64_t n) { return (n + kEdenTile - 1) / kEdenTile; }
+
+} // namespace
+
+int64_t eden_work_doubles(int64_t n) { return eden_tiles(n); }
+
+hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids, int nbits,
+                                uint32_t *packed, float *result, double *work, hipStream_t stream)
+{
+    const int64_t tiles = eden_tiles(n);
+    const float sqrt_n = (float)sqrt((double)n);
+    dim3 grid((unsigned)tiles), block(kEdenThreads);
+    hipLaunchKernelGGL(eden_sumsq_kernel, grid, block, 0, stream, vec, n, work);
+    hipLaunchKernelGGL(eden_norm_kernel, dim3(1), block, 0, stream, work, tiles, result);
+    switch (nbits) {
+#define DQ_EDEN_CASE(B)                                                                                                  \
+    case B:                                                                                                              \
+        hipLaunchKernelGGL(eden_bins_kernel<B>, grid, block, 0, stream, vec, n, boundaries, centroids, result, sqrt_n, packed, \
+                           work);                                                                                        \
+        break;
+        DQ_EDEN_CASE(1) DQ_EDEN_CASE(2) DQ_EDEN_CASE(3) DQ_EDEN_CASE(4) DQ_EDEN_CASE(5) DQ_EDEN_CASE(6) DQ_EDEN_CASE(7)
+    default:
+        hipLaunchKernelGGL(eden_bins_kernel<8>, grid, block, 0, stream, vec, n, boundaries, centroids, result, sqrt_n, packed, work);
+        break;
+#undef DQ_EDEN_CASE
+    }
+    hipLaunchKernelGGL(eden_scale_kernel, dim3(1), block, 0, stream, work, tiles, result);
+    return hipGetLastError();
+}
+
+hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits, float *out,
+                                  hipStream_t stream)
+{
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    switch (nbits) {
+#define DQ_EDEN_CASE(B)                                                                                      \
+    case B: hipLaunchKernelGGL(eden_dequantize_kernel<B>, grid, block, 0, stream, packed, n, centroids, out); break;
+        DQ_EDEN_CASE(1) DQ_EDEN_CASE(2) DQ_EDEN_CASE(3) DQ_EDEN_CASE(4) DQ_EDEN_CASE(5) DQ_EDEN_CASE(6) DQ_EDEN_CASE(7)
+    default: hipLaunchKernelGGL(eden_dequantize_kernel<8>, grid, block, 0, stream, packed, n, centroids, out); break;
+#undef DQ_EDEN_CASE
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_thc_quantize(const float *rotated, const float *uniform, void *out, int64_t n, const float *lo,
+                               const float *delta, int levels, hipStream_t stream)
+{
+    hipLaunchKernelGGL(thc_quantize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, rotated, uniform,
+                       static_cast<uint16_t *>(out), n, lo, delta, (float)(levels - 1));
+    return hipGetLastError();
+}
+
+hipError_t launch_thc_dequantize(const void *levels, float *out, int64_t n, const float *step, const float *lo,
+                                 hipStream_t stream)
+{
+    hipLaunchKernelGGL(thc_dequantize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<const uint16_t *>(levels), out, n, step, lo);
+    return hipGetLastError();
+}
+
+} // namespace dq

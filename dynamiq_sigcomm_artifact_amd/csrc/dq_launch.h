@@ -68,6 +68,18 @@ hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t 
                               int inverse, hipStream_t stream);
 hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream);
 
+// EDEN Lloyd-Max quantiser + packer, THC uniform quantiser (dq_eden.hip)
+int64_t eden_work_doubles(int64_t n);
+hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,
+                                int nbits, uint32_t *packed, float *result, double *work,
+                                hipStream_t stream);
+hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits,
+                                  float *out, hipStream_t stream);
+hipError_t launch_thc_quantize(const float *rotated, const float *uniform, void *out, int64_t n,
+                               const float *lo, const float *delta, int levels, hipStream_t stream);
+hipError_t launch_thc_dequantize(const void *levels, float *out, int64_t n, const float *step,
+                                 const float *lo, hipStream_t stream);
+
 // EDEN bit-plane packing and THC rounding (dq_packing.hip)
 hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits,
                                hipStream_t stream);

@@ -12,6 +12,7 @@
 #include <torch/extension.h>
 
 #include <atomic>
+#include <vector>
 
 #include "dynamiq_eden.h"
 
@@ -474,6 +475,85 @@ torch::Tensor EdenBitsToBins(torch::Tensor arr, int nbits)
     return cbins;
 }
 
+// ---- EDEN / THC consumers (additions; see include/dynamiq_eden.h) --------------------------
+
+void check_f32_cuda(const torch::Tensor &t, const char *name)
+{
+    TORCH_CHECK(t.device().type() == torch::kCUDA, name, " must be a CUDA tensor");
+    TORCH_CHECK(t.dtype() == torch::kFloat32, name, " must be torch.float32");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+
+// returns (packed int32 [n / 32 * nbits], result float32 [4] = sum of squares, dot, scale, norm)
+std::vector<torch::Tensor> eden_quantize(torch::Tensor vec, torch::Tensor boundaries, torch::Tensor centroids, int nbits,
+                                         uint64_t stream_p = 0)
+{
+    check_f32_cuda(vec, "vec");
+    check_f32_cuda(boundaries, "boundaries");
+    check_f32_cuda(centroids, "centroids");
+    TORCH_CHECK(nbits >= 1 && nbits <= 8, "nbits must be in [1, 8]");
+    const int64_t n = vec.numel();
+    TORCH_CHECK(n > 0 && (n & 31) == 0, "vec size must be a positive multiple of 32");
+    TORCH_CHECK(boundaries.numel() == (1 << nbits) - 1, "boundaries must hold 2^nbits - 1 values");
+    TORCH_CHECK(centroids.numel() == (1 << nbits), "centroids must hold 2^nbits values");
+    auto packed = torch::empty({n / 32 * nbits}, vec.options().dtype(torch::kInt32));
+    auto result = torch::empty({4}, vec.options());
+    auto work = torch::empty({dq_eden_work_doubles(n)}, vec.options().dtype(torch::kFloat64));
+    check_status(dq_eden_quantize(vec.data_ptr<float>(), n, boundaries.data_ptr<float>(), centroids.data_ptr<float>(), nbits,
+                                  reinterpret_cast<uint32_t *>(packed.data_ptr<int32_t>()), result.data_ptr<float>(),
+                                  work.data_ptr<double>(), work.numel(), vec.device().index(), as_stream(stream_p)),
+                 "eden_quantize");
+    return {packed, result};
+}
+
+torch::Tensor eden_dequantize(torch::Tensor packed, torch::Tensor centroids, int nbits, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(packed.device().type() == torch::kCUDA && packed.dtype() == torch::kInt32 && packed.is_contiguous(),
+                "packed must be a contiguous torch.int32 CUDA tensor");
+    check_f32_cuda(centroids, "centroids");
+    TORCH_CHECK(nbits >= 1 && nbits <= 8, "nbits must be in [1, 8]");
+    TORCH_CHECK(packed.numel() > 0 && packed.numel() % nbits == 0, "packed size must be a multiple of nbits");
+    TORCH_CHECK(centroids.numel() == (1 << nbits), "centroids must hold 2^nbits values");
+    const int64_t n = packed.numel() / nbits * 32;
+    auto out = torch::empty({n}, centroids.options());
+    check_status(dq_eden_dequantize(reinterpret_cast<const uint32_t *>(packed.data_ptr<int32_t>()), n, centroids.data_ptr<float>(),
+                                    nbits, out.data_ptr<float>(), packed.device().index(), as_stream(stream_p)),
+                 "eden_dequantize");
+    return out;
+}
+
+torch::Tensor thc_quantize(torch::Tensor rotated, torch::Tensor uniform, torch::Tensor lo, torch::Tensor delta, int levels,
+                           uint64_t stream_p = 0)
+{
+    check_f32_cuda(rotated, "rotated");
+    check_f32_cuda(uniform, "uniform");
+    check_f32_cuda(lo, "lo");
+    check_f32_cuda(delta, "delta");
+    TORCH_CHECK(uniform.numel() >= rotated.numel(), "uniform has fewer elements than rotated");
+    TORCH_CHECK(lo.numel() == 1 && delta.numel() == 1, "lo and delta must hold one value");
+    TORCH_CHECK(levels >= 2 && levels <= 256, "levels must be in [2, 256]");
+    auto out = torch::empty({rotated.numel()}, rotated.options().dtype(torch::kBFloat16));
+    check_status(dq_thc_quantize(rotated.data_ptr<float>(), uniform.data_ptr<float>(), out.data_ptr(), rotated.numel(),
+                                 lo.data_ptr<float>(), delta.data_ptr<float>(), levels, rotated.device().index(),
+                                 as_stream(stream_p)),
+                 "thc_quantize");
+    return out;
+}
+
+void thc_dequantize(torch::Tensor levels, torch::Tensor out, torch::Tensor step, torch::Tensor lo, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(levels.device().type() == torch::kCUDA && levels.dtype() == torch::kBFloat16 && levels.is_contiguous(),
+                "levels must be a contiguous torch.bfloat16 CUDA tensor");
+    check_f32_cuda(out, "out");
+    check_f32_cuda(step, "step");
+    check_f32_cuda(lo, "lo");
+    TORCH_CHECK(out.numel() >= levels.numel(), "out has fewer elements than levels");
+    TORCH_CHECK(step.numel() == 1 && lo.numel() == 1, "step and lo must hold one value");
+    check_status(dq_thc_dequantize(levels.data_ptr(), out.data_ptr<float>(), levels.numel(), step.data_ptr<float>(),
+                                   lo.data_ptr<float>(), levels.device().index(), as_stream(stream_p)),
+                 "thc_dequantize");
+}
+
 void init_lookup_table() { check_status(dq_init_lookup_table(), "init_lookup_table"); }
 
 std::string abi_version() { return dq_version(); }
@@ -512,5 +592,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_decompress_rows", &scaling_decompress_rows, "decode consecutive records into the superchunks rows[k] of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("rows"), py::arg("stats"), py::arg("n_limit"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("eden_quantize", &eden_quantize, "EDEN: normalise, bucketize against the Lloyd-Max boundaries, pack bit planes, scale; returns [packed, result]", py::arg("vec"), py::arg("boundaries"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
+    modul.def("eden_dequantize", &eden_dequantize, "EDEN: centroids of the packed bins", py::arg("packed"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
+    modul.def("thc_quantize", &thc_quantize, "THC: uniform stochastic quantiser of the rotated vector, bfloat16 levels", py::arg("rotated"), py::arg("uniform"), py::arg("lo"), py::arg("delta"), py::arg("levels"), py::arg("stream_p") = 0);
+    modul.def("thc_dequantize", &thc_dequantize, "THC: out = float(levels) * step + lo", py::arg("levels"), py::arg("out"), py::arg("step"), py::arg("lo"), py::arg("stream_p") = 0);
     modul.def("abi_version", &abi_version, "version string of libdynamiq_eden.so");
 }

@@ -95,6 +95,24 @@ def config1(dev):
             t_rht = _time_us(lambda: capi.rht_blocked(y, sign, B, scale, False))
             _emit(config=1, block=B, nbits=nbits, nmse_rht=_nmse(x, z), nmse_no_rht=_nmse(x, plain),
                   rht_us=round(t_rht, 2), rht_GBps=round(8.0 * n / t_rht / 1e3, 1))
+    # the reference-legal path for this configuration: EDEN (whole-vector rotation, Lloyd-Max bins, bit planes)
+    from .eden import Eden
+    eden = Eden(device=dev)
+    for nbits in (4, 5, 8):
+        data = eden.compress(x, nbits, 0)
+        rec = eden.decompress(data)
+        cen, bnd = eden._tables(nbits)
+        y = x.clone()
+        capi.rht_blocked(y, sign, n, 1.0 / math.sqrt(n), False)
+        packed = torch.empty(n // 32 * nbits, dtype=torch.int32, device=dev)
+        result = torch.empty(4, device=dev)
+        work = torch.empty(capi.eden_work_doubles(n), dtype=torch.float64, device=dev)
+        out = torch.empty(n, device=dev)
+        tq = _time_us(lambda: capi.eden_quantize(y, bnd, cen, nbits, packed, result, work))
+        td = _time_us(lambda: capi.eden_dequantize(packed, n, cen, nbits, out))
+        _emit(config=1, path="eden", nbits=nbits, nmse=_nmse(x, rec), slices=len(data), quantize_us=round(tq, 2),
+              dequantize_us=round(td, 2), quantize_GBps=round((8.0 + nbits / 8.0) * n / tq / 1e3, 1),
+              dequantize_GBps=round((4.0 + nbits / 8.0) * n / td / 1e3, 1))
 
 
 def config2(dev):

@@ -172,6 +172,48 @@ int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *row
                                int dtype, int device, int strategy, dq_stream_t stream,
                                int add_original);
 
+/* ---- consumers of the rotated vector: EDEN and THC ----------------------
+ *
+ * "reference" here: cuda_kernels/src/srrcomp/srrcomp.py (EDEN) and
+ * testbed_evaluation/new_comm_hooks/thc_hooks.py (THC); both run these steps
+ * as chains of torch ops around eden_utils.Hadamard. */
+
+/* number of doubles the `work` argument of dq_eden_quantize must hold */
+int64_t dq_eden_work_doubles(int64_t n);
+
+/* srrcomp.py:356-361 (Eden._quantize) + :124-145 (EdenBinsToBits) in one call.
+ * vec: float32 [n], n a positive multiple of 32 (the caller pads, :300-309).
+ * boundaries: float32 [2^nbits - 1] ascending, centroids: float32 [2^nbits]
+ * (Eden.boundaries[nbits], Eden.centroids[nbits]); nbits 1..8.
+ *   bin_i   = #{ boundaries < (vec_i * (float)sqrt(n)) / ||vec|| }   (torch.bucketize, right=False)
+ *   packed  = bit planes of the bins, uint32 [n / 32 * nbits]
+ *   result  = float32 [4] on the device: sum of squares, <centroids[bin], vec>,
+ *             scale = ||vec||^2 / <centroids[bin], vec>, ||vec||
+ * Sums are accumulated in double in a fixed order (4096-element tiles, stride
+ * 256 inside a tile, halving trees), so the result is independent of the launch
+ * shape; torch's own reduction order is not specified, hence `scale` agrees with
+ * the reference to rounding error, not bit for bit. */
+int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,
+                     int nbits, uint32_t *packed, float *result, double *work,
+                     int64_t work_doubles, int device, dq_stream_t stream);
+
+/* srrcomp.py:343-345: out_i = centroids[bin_i] from the bit planes. */
+int dq_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits,
+                       float *out, int device, dq_stream_t stream);
+
+/* thc_hooks.py:161-166: level = floor(x) + (uniform < x - floor(x)) with
+ * x = clamp((rotated - *lo) / *delta, 0, levels - 1), stored as bfloat16.
+ * lo, delta: device scalars (they derive from the all-reduced norm,
+ * thc_hooks.py:143-147).  uniform: float32 [n] in [0, 1) -- the caller draws it
+ * (torch's bernoulli_ stream cannot be reproduced outside torch). */
+int dq_thc_quantize(const float *rotated, const float *uniform, void *levels_bf16, int64_t n,
+                    const float *lo, const float *delta, int levels, int device,
+                    dq_stream_t stream);
+
+/* thc_hooks.py:176-178: out = float(levels) * *step + *lo (two roundings). */
+int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const float *step,
+                      const float *lo, int device, dq_stream_t stream);
+
 /* ---- superchunk mean-centring ---------------------------------------- */
 
 /* csrc/cuda_hadamard.h:23-24 (superchunk_mean_center_with_cuda).  residual

@@ -256,6 +256,53 @@ def bits_to_bins(arr, nbits):
     return bins
 
 
+def eden_quantize(vec, boundaries, centroids, nbits):
+    """-> (bins int32 [n], result float32 [4] = sumsq, dot, scale, norm)"""
+    _chk(vec, np.float32, "vec")
+    _chk(boundaries, np.float32, "boundaries")
+    _chk(centroids, np.float32, "centroids")
+    assert boundaries.size == (1 << nbits) - 1 and centroids.size == 1 << nbits
+    bins = np.zeros(vec.size, np.int32)
+    result = np.zeros(4, np.float32)
+    f = lib().dqo_eden_quantize
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    f(_p(vec), vec.size, _p(boundaries), _p(centroids), nbits, _p(bins), _p(result))
+    return bins, result
+
+
+def eden_dequantize(bins, centroids):
+    _chk(bins, np.int32, "bins")
+    _chk(centroids, np.float32, "centroids")
+    out = np.zeros(bins.size, np.float32)
+    f = lib().dqo_eden_dequantize
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+    f(_p(bins), bins.size, _p(centroids), _p(out))
+    return out
+
+
+def thc_quantize(rotated, uniform, lo, delta, levels):
+    _chk(rotated, np.float32, "rotated")
+    _chk(uniform, np.float32, "uniform")
+    out = np.zeros(rotated.size, np.uint16)
+    f = lib().dqo_thc_quantize
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_float, ctypes.c_int]
+    f(_p(rotated), _p(uniform), _p(out), rotated.size, float(lo), float(delta), levels)
+    return out
+
+
+def thc_dequantize(levels_bf16, step, lo):
+    _chk(levels_bf16, np.uint16, "levels")
+    out = np.zeros(levels_bf16.size, np.float32)
+    f = lib().dqo_thc_dequantize
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_float]
+    f(_p(levels_bf16), _p(out), levels_bf16.size, float(step), float(lo))
+    return out
+
+
 def dynamic_bitrate_qbits(norms_bf16, u, stride=1):
     _chk(norms_bf16, np.uint16, "norms")
     count = (norms_bf16.size + stride - 1) // stride

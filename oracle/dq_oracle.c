@@ -799,6 +799,110 @@ void dqo_bits_to_bins(const uint32_t *arr, int64_t narr, int32_t *bins, int nbit
 }
 
 /* ------------------------------------------------------------------------ */
+/* EDEN Lloyd-Max quantiser, THC uniform quantiser                           */
+/* ------------------------------------------------------------------------ */
+
+/* sum of term(i), i < n, in double: tiles of 4096 indices, inside a tile 256 lanes that add
+ * indices lane + 256 k (k ascending), a halving tree over the lanes (stride 128 .. 1); the tile
+ * sums are folded the same way (lane adds tiles lane + 256 k, then the tree).  torch leaves the
+ * order of its reductions unspecified; this is the order the library documents for itself. */
+typedef double (*dqo_term_fn)(int64_t i, void *ctx);
+
+static double halve256(double *lane)
+{
+    for (int stride = 128; stride > 0; stride >>= 1)
+        for (int l = 0; l < stride; l++) lane[l] += lane[l + stride];
+    return lane[0];
+}
+
+static double tiled_sum(int64_t n, dqo_term_fn term, void *ctx)
+{
+    const int64_t tiles = (n + 4095) / 4096;
+    double *tile_sum = (double *)malloc((size_t)tiles * sizeof(double));
+    double lane[256];
+    for (int64_t b = 0; b < tiles; b++) {
+        for (int l = 0; l < 256; l++) {
+            double acc = 0.0;
+            for (int k = 0; k < 16; k++) {
+                int64_t i = b * 4096 + l + 256 * k;
+                if (i < n) acc += term(i, ctx);
+            }
+            lane[l] = acc;
+        }
+        tile_sum[b] = halve256(lane);
+    }
+    for (int l = 0; l < 256; l++) {
+        double acc = 0.0;
+        for (int64_t i = l; i < tiles; i += 256) acc += tile_sum[i];
+        lane[l] = acc;
+    }
+    free(tile_sum);
+    return halve256(lane);
+}
+
+struct eden_ctx { const float *vec; const float *cen; const int32_t *bins; };
+static double term_sq(int64_t i, void *c) { double v = (double)((struct eden_ctx *)c)->vec[i]; return v * v; }
+static double term_dot(int64_t i, void *c)
+{
+    struct eden_ctx *e = (struct eden_ctx *)c;
+    return (double)e->cen[e->bins[i]] * (double)e->vec[i];
+}
+
+/* srrcomp.py:356-361: bins = bucketize(vec * sqrt(n) / ||vec||, boundaries) with right=False, i.e. the
+ * number of boundaries strictly below the value; scale = ||vec||^2 / <centroids[bins], vec>.
+ * result = {sum of squares, dot, scale, norm}. */
+void dqo_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids, int nbits,
+                       int32_t *bins, float *result)
+{
+    const int nb = (1 << nbits) - 1;
+    struct eden_ctx ctx = {vec, centroids, bins};
+    const float sumsq = (float)tiled_sum(n, term_sq, &ctx);
+    const float norm = sqrtf(sumsq);
+    const float sqrt_n = (float)sqrt((double)n);
+    for (int64_t i = 0; i < n; i++) {
+        const float x = (vec[i] * sqrt_n) / norm;
+        int b = 0;
+        while (b < nb && boundaries[b] < x) b++;
+        bins[i] = b;
+    }
+    const float dot = (float)tiled_sum(n, term_dot, &ctx);
+    result[0] = sumsq;
+    result[1] = dot;
+    result[2] = (norm * norm) / dot;
+    result[3] = norm;
+}
+
+/* srrcomp.py:343-345 */
+void dqo_eden_dequantize(const int32_t *bins, int64_t n, const float *centroids, float *out)
+{
+    for (int64_t i = 0; i < n; i++) out[i] = centroids[bins[i]];
+}
+
+/* thc_hooks.py:161-166 with the Bernoulli draw given as a uniform value: 1 when uniform < probability */
+void dqo_thc_quantize(const float *rotated, const float *uniform, uint16_t *levels_bf16, int64_t n, float lo,
+                      float delta, int levels)
+{
+    const float top = (float)(levels - 1);
+    for (int64_t i = 0; i < n; i++) {
+        float x = (rotated[i] - lo) / delta;
+        if (x < 0.0f) x = 0.0f;
+        if (x > top) x = top;
+        const float fl = floorf(x);
+        const float prob = x - fl;
+        levels_bf16[i] = dqo_f32_to_bf16(fl + (uniform[i] < prob ? 1.0f : 0.0f));
+    }
+}
+
+/* thc_hooks.py:176-178 */
+void dqo_thc_dequantize(const uint16_t *levels_bf16, float *out, int64_t n, float step, float lo)
+{
+    for (int64_t i = 0; i < n; i++) {
+        const float prod = dqo_bf16_to_f32(levels_bf16[i]) * step;
+        out[i] = prod + lo;
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* dynamic bit-width rule                                                    */
 /* ------------------------------------------------------------------------ */
 

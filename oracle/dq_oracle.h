@@ -108,6 +108,20 @@ void dqo_rand_diag(float *out, int64_t size, int64_t seed);
 void dqo_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits);
 void dqo_bits_to_bins(const uint32_t *arr, int64_t narr, int32_t *bins, int nbits);
 
+/* cuda_kernels/src/srrcomp/srrcomp.py:356-361 (Eden._quantize) and :343-345; sums in double in the
+ * library's documented order (torch's reduction order is unspecified: "parity unpinned" for the
+ * last bits of `scale`, pinned within tolerance by the reference's own outputs in
+ * tests/golden/eden_golden.npz).  result = {sum of squares, dot, scale, norm}. */
+void dqo_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,
+                       int nbits, int32_t *bins, float *result);
+void dqo_eden_dequantize(const int32_t *bins, int64_t n, const float *centroids, float *out);
+
+/* testbed_evaluation/new_comm_hooks/thc_hooks.py:161-166 and :176-178; the Bernoulli draw is an
+ * input (uniform < probability): torch's bernoulli_ stream is "parity unpinned". */
+void dqo_thc_quantize(const float *rotated, const float *uniform, uint16_t *levels_bf16, int64_t n,
+                      float lo, float delta, int levels);
+void dqo_thc_dequantize(const uint16_t *levels_bf16, float *out, int64_t n, float step, float lo);
+
 /* testbed_evaluation/new_comm_hooks/comm_hooks.py:64-70 evaluated on bf16
  * norms with bf16 rounding after every tensor op (what torch does for a bf16
  * tensor); qbits out as int64. */
