@@ -432,6 +432,7 @@ int dq_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int64_t n
     if (!(nbins > 0) || (nbins & 31) != 0) return fail(DQ_ERR_SIZE, "bins size must be a multiple of 32");
     if (narr != (nbins >> 5) * nbits) return fail(DQ_ERR_SIZE, "narr must equal nbins / 32 * nbits");
     if (!bins || !arr) return fail(DQ_ERR_NULL);
+    if (reinterpret_cast<uintptr_t>(bins) & 15) return fail(DQ_ERR_SIZE, "bins must be 16-byte aligned");
     int rc;
     if ((rc = select_device(device))) return rc;
     return finish(dq::launch_bits_to_bins(bins, nbins, arr, nbits, static_cast<hipStream_t>(stream)));
@@ -458,6 +459,7 @@ int dq_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids
     if (!(n > 0) || (n & 31) != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of 32");
     if (nbits < 1 || nbits > 8) return fail(DQ_ERR_NBITS, "nbits must be in [1, 8]");
     if (!packed || !centroids || !out) return fail(DQ_ERR_NULL);
+    if (reinterpret_cast<uintptr_t>(out) & 15) return fail(DQ_ERR_SIZE, "out must be 16-byte aligned");
     int rc;
     if ((rc = select_device(device))) return rc;
     return finish(dq::launch_eden_dequantize(packed, n, centroids, nbits, out, static_cast<hipStream_t>(stream)));

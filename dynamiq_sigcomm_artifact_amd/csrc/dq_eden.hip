@@ -140,6 +140,7 @@ __global__ __launch_bounds__(kEdenThreads) void eden_scale_kernel(const double *
     }
 }
 
+// four consecutive elements per thread: they share the 32-bin word of every bit plane
 template <int NBITS>
 __global__ __launch_bounds__(256) void eden_dequantize_kernel(const uint32_t *__restrict__ packed, int64_t n,
                                                               const float *__restrict__ centroids, float *__restrict__ out)
@@ -148,46 +149,80 @@ __global__ __launch_bounds__(256) void eden_dequantize_kernel(const uint32_t *__
     __shared__ float cen[L];
     for (int k = threadIdx.x; k < L; k += 256) cen[k] = centroids[k];
     __syncthreads();
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= n) return;
     const int64_t words = n >> 5, w = i >> 5;
     const int t = (int)(i & 31);
-    int bin = 0;
+    uint32_t bins[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int p = 0; p < NBITS; p++) bin |= (int)((packed[(int64_t)p * words + w] >> t) & 1u) << p;
-    out[i] = cen[bin];
+    for (int p = 0; p < NBITS; p++) {
+        const uint32_t word = packed[(int64_t)p * words + w] >> t;
+#pragma unroll
+        for (int k = 0; k < 4; k++) bins[k] |= ((word >> k) & 1u) << p;
+    }
+    *reinterpret_cast<float4 *>(out + i) = make_float4(cen[bins[0]], cen[bins[1]], cen[bins[2]], cen[bins[3]]);
 }
 
 // ---- THC ------------------------------------------------------------------------------------------
 
-// x = clamp((v - lo) / delta, 0, levels - 1); level = floor(x) + (u < x - floor(x)); stored as bf16
-__global__ __launch_bounds__(256) void thc_quantize_kernel(const float *__restrict__ rotated, const float *__restrict__ uniform,
-                                                           uint16_t *__restrict__ out, int64_t n,
-                                                           const float *__restrict__ lo_p, const float *__restrict__ delta_p,
-                                                           float top)
+// x = clamp((v - lo) / delta, 0, levels - 1); level = floor(x) + (u < x - floor(x))
+__device__ __forceinline__ float thc_level(float v, float u, float lo, float delta, float top)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    const float lo = *lo_p, delta = *delta_p;
-    float x = (rotated[i] - lo) / delta;
+    float x = (v - lo) / delta;
     // torch.clamp_ keeps NaN
     if (x < 0.0f) x = 0.0f;
     if (x > top) x = top;
     const float fl = __builtin_floorf(x);
     const float prob = x - fl;
-    const float level = fl + ((uniform[i] < prob) ? 1.0f : 0.0f);
-    out[i] = (uint16_t)f32_to_bf16_bits(level);
+    return fl + ((u < prob) ? 1.0f : 0.0f);
+}
+
+// levels stored as bf16; VEC: four elements per thread through 16-byte loads and one 8-byte store
+template <bool VEC>
+__global__ __launch_bounds__(256) void thc_quantize_kernel(const float *__restrict__ rotated, const float *__restrict__ uniform,
+                                                           uint16_t *__restrict__ out, int64_t begin, int64_t n,
+                                                           const float *__restrict__ lo_p, const float *__restrict__ delta_p,
+                                                           float top)
+{
+    const float lo = *lo_p, delta = *delta_p;
+    if (VEC) {
+        const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+        if (i + 4 > n) return;
+        const float4 v = *reinterpret_cast<const float4 *>(rotated + i);
+        const float4 u = *reinterpret_cast<const float4 *>(uniform + i);
+        uint2 o;
+        o.x = f32x2_to_bf16x2(thc_level(v.x, u.x, lo, delta, top), thc_level(v.y, u.y, lo, delta, top));
+        o.y = f32x2_to_bf16x2(thc_level(v.z, u.z, lo, delta, top), thc_level(v.w, u.w, lo, delta, top));
+        *reinterpret_cast<uint2 *>(out + i) = o;
+    } else {
+        const int64_t i = begin + (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (i >= n) return;
+        out[i] = (uint16_t)f32_to_bf16_bits(thc_level(rotated[i], uniform[i], lo, delta, top));
+    }
 }
 
 // v = float(level sum) * step + lo, two roundings
+template <bool VEC>
 __global__ __launch_bounds__(256) void thc_dequantize_kernel(const uint16_t *__restrict__ levels, float *__restrict__ out,
-                                                             int64_t n, const float *__restrict__ step_p,
+                                                             int64_t begin, int64_t n, const float *__restrict__ step_p,
                                                              const float *__restrict__ lo_p)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    const float prod = bf16_bits_to_f32(levels[i]) * *step_p;
-    out[i] = prod + *lo_p;
+    const float step = *step_p, lo = *lo_p;
+    if (VEC) {
+        const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+        if (i + 4 > n) return;
+        const uint2 l = *reinterpret_cast<const uint2 *>(levels + i);
+        float4 o;
+        float p0 = bf16_bits_to_f32(l.x & 0xffffu) * step, p1 = bf16_bits_to_f32(l.x >> 16) * step;
+        float p2 = bf16_bits_to_f32(l.y & 0xffffu) * step, p3 = bf16_bits_to_f32(l.y >> 16) * step;
+        o.x = p0 + lo; o.y = p1 + lo; o.z = p2 + lo; o.w = p3 + lo;
+        *reinterpret_cast<float4 *>(out + i) = o;
+    } else {
+        const int64_t i = begin + (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (i >= n) return;
+        const float prod = bf16_bits_to_f32(levels[i]) * step;
+        out[i] = prod + lo;
+    }
 }
 
 inline int64_t eden_tiles(int64_t n) { return (n + kEdenTile - 1) / kEdenTile; }
@@ -223,7 +258,9 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
 hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits, float *out,
                                   hipStream_t stream)
 {
-    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    // n is a multiple of 32, so groups of four never straddle a word; out comes from an allocator (16-byte aligned)
+    // or at a multiple-of-32 element offset into one
+    dim3 grid((unsigned)((n / 4 + 255) / 256)), block(256);
     switch (nbits) {
 #define DQ_EDEN_CASE(B)                                                                                      \
     case B: hipLaunchKernelGGL(eden_dequantize_kernel<B>, grid, block, 0, stream, packed, n, centroids, out); break;
@@ -237,16 +274,36 @@ hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float
 hipError_t launch_thc_quantize(const float *rotated, const float *uniform, void *out, int64_t n, const float *lo,
                                const float *delta, int levels, hipStream_t stream)
 {
-    hipLaunchKernelGGL(thc_quantize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, rotated, uniform,
-                       static_cast<uint16_t *>(out), n, lo, delta, (float)(levels - 1));
+    uint16_t *o = static_cast<uint16_t *>(out);
+    const float top = (float)(levels - 1);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(rotated) | reinterpret_cast<uintptr_t>(uniform)) & 15) == 0 &&
+                         (reinterpret_cast<uintptr_t>(out) & 7) == 0;
+    int64_t done = 0;
+    if (aligned && n >= 4) {
+        done = n / 4 * 4;
+        hipLaunchKernelGGL(thc_quantize_kernel<true>, dim3((unsigned)((done / 4 + 255) / 256)), dim3(256), 0, stream, rotated,
+                           uniform, o, (int64_t)0, done, lo, delta, top);
+    }
+    if (done < n)
+        hipLaunchKernelGGL(thc_quantize_kernel<false>, dim3((unsigned)((n - done + 255) / 256)), dim3(256), 0, stream, rotated,
+                           uniform, o, done, n, lo, delta, top);
     return hipGetLastError();
 }
 
 hipError_t launch_thc_dequantize(const void *levels, float *out, int64_t n, const float *step, const float *lo,
                                  hipStream_t stream)
 {
-    hipLaunchKernelGGL(thc_dequantize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
-                       static_cast<const uint16_t *>(levels), out, n, step, lo);
+    const uint16_t *l = static_cast<const uint16_t *>(levels);
+    const bool aligned = (reinterpret_cast<uintptr_t>(levels) & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    int64_t done = 0;
+    if (aligned && n >= 4) {
+        done = n / 4 * 4;
+        hipLaunchKernelGGL(thc_dequantize_kernel<true>, dim3((unsigned)((done / 4 + 255) / 256)), dim3(256), 0, stream, l, out,
+                           (int64_t)0, done, step, lo);
+    }
+    if (done < n)
+        hipLaunchKernelGGL(thc_dequantize_kernel<false>, dim3((unsigned)((n - done + 255) / 256)), dim3(256), 0, stream, l, out,
+                           done, n, step, lo);
     return hipGetLastError();
 }
 

@@ -22,17 +22,22 @@ __global__ __launch_bounds__(256) void bins_to_bits_kernel(const int32_t *__rest
     }
 }
 
+// four consecutive bins per thread: they share the word of every bit plane
 __global__ __launch_bounds__(256) void bits_to_bins_kernel(int32_t *__restrict__ bins, int64_t nbins,
                                                            const uint32_t *__restrict__ arr, int nbits)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= nbins) return;
     const int64_t words = nbins >> 5;
     const int64_t w = i >> 5;
     const int t = (int)(i & 31);
-    int32_t v = 0;
-    for (int p = 0; p < nbits; p++) v += (int32_t)((arr[(int64_t)p * words + w] >> t) & 1u) << p;
-    bins[i] = v;
+    int32_t v[4] = {0, 0, 0, 0};
+    for (int p = 0; p < nbits; p++) {
+        const uint32_t word = arr[(int64_t)p * words + w] >> t;
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] += (int32_t)((word >> k) & 1u) << p;
+    }
+    *reinterpret_cast<int4 *>(bins + i) = make_int4(v[0], v[1], v[2], v[3]);
 }
 
 hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits, hipStream_t stream)
@@ -43,7 +48,8 @@ hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr
 
 hipError_t launch_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int nbits, hipStream_t stream)
 {
-    hipLaunchKernelGGL(bits_to_bins_kernel, dim3((unsigned)((nbins + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
+    // nbins is a multiple of 32 and bins a whole tensor: groups of four are 16-byte aligned
+    hipLaunchKernelGGL(bits_to_bins_kernel, dim3((unsigned)((nbins / 4 + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
     return hipGetLastError();
 }
 

@@ -7,6 +7,7 @@ peak).  ``python -m dynamiq_sigcomm_artifact_amd.evaluate --config 1|2|3|4|5``.
   3  8 simulated ranks x 124,439,808 elements: compressed ring all-reduce
   4  Llama-3-8B shaped gradient set in 25 MB buckets: dynamic {2,4,8}-bit allocation
   5  2^30 fp32: compress / decompress / fused sweep, and the blocked transform
+``--kernels`` times every entry point of the library on one 25 MB bucket.
 
 Timings: 10 warm-up launches, then 50 launches replayed from a HIP graph between two
 events (cuda_kernels/tests/benchmark_scaling_quantization.py:41-57 times eager launches;
@@ -323,9 +324,110 @@ def config5(dev, n=1 << 30):
     _emit(config=5, op="hadamard_whole_vector", n=n, us=round(t, 1))
 
 
+def kernels(dev, n=6553600):
+    """every entry point of the library on one 25 MB bucket (n elements): device time per call and the fraction of
+    the 8 TB/s HBM peak its algorithmic bytes amount to"""
+    g = torch.Generator(device=dev).manual_seed(0)
+    x32 = torch.randn(n, generator=g, device=dev) * 1e-3
+    nsc = n // 256
+
+    def line(name, fn, nbytes, **kw):
+        t = _time_us(fn)
+        _emit(kernel=name, us=round(t, 2), algorithmic_MB=round(nbytes / 1e6, 2), GBps=round(nbytes / t / 1e3, 1),
+              frac_hbm=round(nbytes / t / 1e3 / HBM_PEAK, 4), **kw)
+
+    # scaling quantisation: every element type and strategy at chunk 16, 4 and 8 bits
+    for tdt, name, sb in ((torch.float32, "fp32", 4), (torch.bfloat16, "bf16", 2), (torch.float16, "fp16", 2)):
+        src = x32.to(tdt)
+        rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16 if tdt != torch.float16 else tdt)
+        out = torch.empty_like(src)
+        for strategy in (2, 3, 0, 1):
+            for nbits in (4, 8):
+                nb = capi.required_bytes(n, nbits, 16, strategy)
+                packed = torch.zeros(nb, dtype=torch.uint8, device=dev)
+                send = torch.zeros_like(packed)
+                rnd = rand              # a bf16 pool beside fp32 elements as well
+                capi.scaling_compress(src, packed, rnd, n, nbits, 16, strategy)
+                tag = dict(elements=name, strategy=strategy, nbits=nbits)
+                line("scaling_compress", lambda: capi.scaling_compress(src, packed, rnd, n, nbits, 16, strategy),
+                     (sb + 2) * n + nb, **tag)
+                line("scaling_decompress", lambda: capi.scaling_decompress(packed, out, n, nbits, 16, strategy),
+                     sb * n + nb, **tag)
+                line("scaling_decompress_add", lambda: capi.scaling_decompress(packed, out, n, nbits, 16, strategy, add=True),
+                     2 * sb * n + nb, **tag)
+                if strategy >= 2 and tdt != torch.float16:
+                    line("scaling_dec_comp (fused)", lambda: capi.scaling_dec_comp(packed, src, send, rnd, n, nbits, 16, strategy),
+                         (sb + 2) * n + 2 * nb, **tag)
+        del src, rand, out
+    # chunk sizes other than 16: the thread-per-chunk kernels
+    src = x32.to(torch.bfloat16)
+    rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty_like(src)
+    for C in (8, 32):
+        nb = capi.required_bytes(n, 4, C, 2)
+        packed = torch.zeros(nb, dtype=torch.uint8, device=dev)
+        line("scaling_compress", lambda: capi.scaling_compress(src, packed, rand, n, 4, C, 2), 4 * n + nb,
+             elements="bf16", strategy=2, nbits=4, chunk_size=C)
+        line("scaling_decompress", lambda: capi.scaling_decompress(packed, out, n, 4, C, 2), 2 * n + nb,
+             elements="bf16", strategy=2, nbits=4, chunk_size=C)
+    # superchunk statistics, groups
+    res = torch.empty_like(src)
+    stats = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
+    line("superchunk_mean_center", lambda: capi.superchunk_mean_center(src, res, stats, n, 8), 4 * n + 4 * nsc, elements="bf16")
+    line("superchunk_add_mean_copy", lambda: capi.superchunk_add_mean_copy(res, out, stats, n), 4 * n + 2 * nsc, elements="bf16")
+    order = torch.empty(nsc, dtype=torch.int32, device=dev)
+    work = torch.empty(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
+    qbits = torch.empty(nsc, dtype=torch.int64, device=dev)
+    u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)
+    line("group_plan_stats", lambda: capi.group_plan_stats(stats, u, qbits, order, work), 4 * nsc + 12 * nsc, superchunks=nsc)
+    line("group_plan", lambda: capi.group_plan(qbits, order, work), 8 * nsc + 4 * nsc, superchunks=nsc)
+    rows = torch.arange(0, nsc, 2, dtype=torch.int32, device=dev)
+    nr = rows.numel()
+    nb = capi.required_bytes(nr * 256, 4, 16, 2)
+    packed = torch.zeros(nb, dtype=torch.uint8, device=dev)
+    line("scaling_compress_rows", lambda: capi.scaling_compress_rows(res, rows, packed, rand, nr, 4, 2), 4 * nr * 256 + nb + 4 * nr,
+         elements="bf16", rows="every second superchunk")
+    line("scaling_decompress_rows (+mean)", lambda: capi.scaling_decompress_rows(packed, out, rows, stats, n, nr, 4, 2),
+         2 * nr * 256 + nb + 8 * nr, elements="bf16", rows="every second superchunk")
+    del src, rand, out, res
+    # transforms: whole-vector Hadamard on the padded bucket (THC: d = 2^23), blocked RHT
+    d = 1 << 23
+    y = torch.randn(d, generator=g, device=dev)
+    sign = torch.empty(d, device=dev)
+    line("rand_diag", lambda: capi.rand_diag(sign, 0), 4 * d, n=d)
+    line("Hadamard (whole vector)", lambda: capi.hadamard(y), 16 * d, n=d, passes=2)
+    y.normal_(generator=g)
+    line("rht_blocked (whole vector, sign + scale)", lambda: capi.rht_blocked(y, sign, d, 1.0, False), 20 * d, n=d, passes=2)
+    for kb in (10, 15):
+        y.normal_(generator=g)
+        line("rht_blocked", lambda: capi.rht_blocked(y, sign, 1 << kb, 1.0, False), 12 * d, n=d, block=1 << kb)
+    # consumers of the rotated vector
+    from .eden import normal_centroids_and_boundaries
+    y.normal_(generator=g)
+    for nbits in (4, 8):
+        cen, bnd = (t.to(dev) for t in normal_centroids_and_boundaries(nbits))
+        packed = torch.empty(d // 32 * nbits, dtype=torch.int32, device=dev)
+        result = torch.empty(4, device=dev)
+        work64 = torch.empty(capi.eden_work_doubles(d), dtype=torch.float64, device=dev)
+        out = torch.empty(d, device=dev)
+        line("eden_quantize", lambda: capi.eden_quantize(y, bnd, cen, nbits, packed, result, work64), 8 * d + d // 8 * nbits, n=d, nbits=nbits)
+        line("eden_dequantize", lambda: capi.eden_dequantize(packed, d, cen, nbits, out), 4 * d + d // 8 * nbits, n=d, nbits=nbits)
+    uni = torch.rand(d, generator=g, device=dev)
+    lev = torch.empty(d, dtype=torch.bfloat16, device=dev)
+    lo, delta = torch.tensor([-4.0], device=dev), torch.tensor([8.0 / 63], device=dev)
+    line("thc_quantize", lambda: capi.thc_quantize(y, uni, lev, lo, delta, 64), 10 * d, n=d)
+    line("thc_dequantize", lambda: capi.thc_dequantize(lev, y, delta, lo), 6 * d, n=d)
+    bins = torch.randint(0, 32, (d,), generator=g, device=dev, dtype=torch.int32)
+    arr = torch.empty(d // 32 * 5, dtype=torch.int32, device=dev)
+    line("EdenBinsToBits", lambda: capi.bins_to_bits(bins, arr, 5), 4 * d + d // 32 * 5 * 4, n=d, nbits=5)
+    line("EdenBitsToBins", lambda: capi.bits_to_bins(bins, arr, 5), 4 * d + d // 32 * 5 * 4, n=d, nbits=5)
+    line("quantization_compression", lambda: capi.quantization(y, 0.5, 15.0, 1), 8 * d, n=d)
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", type=int, required=True, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--config", type=int, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--kernels", action="store_true", help="time every entry point of the library on a 25 MB bucket")
     ap.add_argument("--limit", type=int, default=None, help="config 4: number of 25 MB buckets to process")
     ap.add_argument("--n", type=int, default=None, help="configs 3 and 5: element count override")
     args = ap.parse_args()
@@ -333,6 +435,11 @@ def main():
         raise SystemExit("evaluate needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.kernels:
+        kernels(dev, **({"n": args.n} if args.n else {}))
+        return
+    if args.config is None:
+        raise SystemExit("give --config N or --kernels")
     if args.config == 1:
         config1(dev)
     elif args.config == 2:

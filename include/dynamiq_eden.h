@@ -197,7 +197,8 @@ int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const
                      int nbits, uint32_t *packed, float *result, double *work,
                      int64_t work_doubles, int device, dq_stream_t stream);
 
-/* srrcomp.py:343-345: out_i = centroids[bin_i] from the bit planes. */
+/* srrcomp.py:343-345: out_i = centroids[bin_i] from the bit planes.  out must be
+ * 16-byte aligned. */
 int dq_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits,
                        float *out, int device, dq_stream_t stream);
 
@@ -250,7 +251,7 @@ int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t
  * nbins is not a multiple of 1024, and the caller's stream is honoured. */
 int dq_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int64_t narr, int nbits,
                     int device, dq_stream_t stream);
-/* csrc/cuda_packing.h:11 (BitsToBins) */
+/* csrc/cuda_packing.h:11 (BitsToBins); bins must be 16-byte aligned */
 int dq_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int64_t narr, int nbits,
                     int device, dq_stream_t stream);
 

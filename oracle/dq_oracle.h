@@ -23,6 +23,25 @@
  *     reproducible on any IEEE machine;
  *   - float -> int16 conversions saturate and map NaN to 0, int16 additions
  *     wrap (what the reference's cvt/add instructions do).
+ *
+ * What pins this file (tests/test_oracle_*.py): the reference's golden vectors
+ * for randDiag, the bit-plane packer, the torch butterfly and 50 Eden
+ * compress / decompress runs (tests/golden/*.npz, written by the reference's own
+ * CPU code); closed forms, special cases and invariants of the reference's
+ * functional test for the scaling quantiser; an independently written numpy
+ * model of the bf16 / fp16 arithmetic.
+ *
+ * Parity unpinned (no reference output can exist or be reproduced):
+ *   - bit patterns of MEE codes on the reference's own GPU (device log2f under
+ *     fast-math); pinned to dqo_log2f instead;
+ *   - the last bits of dqo_eden_quantize's scale and bins within rounding error
+ *     of a boundary (torch's reduction order is unspecified); tolerance-pinned;
+ *   - dqo_thc_quantize's individual roundings (torch's bernoulli_ stream); the
+ *     uniform draws are an input here;
+ *   - fp32-element and 3/5/6/7-bit scaling modes (extensions of the reference's
+ *     formulas, checked against the numpy model only).
+ * quantization_compression has no restatement at all: the reference's curand
+ * states are never initialised (csrc/cuda_hadamard.cu:669-686).
  */
 #ifndef DQ_ORACLE_H
 #define DQ_ORACLE_H
