@@ -72,6 +72,8 @@ def main():
     ap.add_argument("--nbits", type=int, default=4)
     ap.add_argument("--strategy", type=int, default=2, help="2 = hierarchical AEE, 3 = hierarchical MEE")
     ap.add_argument("--src", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--rand", choices=["pool", "philox"], default="pool",
+                    help="pool: the reference's rand_pool tensor (default); philox: uniform values drawn in the kernel")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the cpu_baseline leg (0 = skip)")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle parity check of a sample")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -104,7 +106,10 @@ def main():
     out = torch.empty_like(src)
 
     def compress():
-        capi.scaling_compress(src, packed, rand, n, nbits, C, strategy)
+        if args.rand == "philox":
+            capi.scaling_compress_philox(src, packed, n, nbits, C, strategy, 2026, 0)
+        else:
+            capi.scaling_compress(src, packed, rand, n, nbits, C, strategy)
 
     def decompress():
         capi.scaling_decompress(packed, out, n, nbits, C, strategy)
@@ -128,7 +133,7 @@ def main():
     comp_ms = event_ms(compress, args.steps)
     dec_ms = event_ms(decompress, args.steps)
     sbytes = 4 if args.src == "fp32" else 2
-    comp_bytes = (sbytes + 2 + (nbits + OVERHEAD_BITS) / 8.0) * n
+    comp_bytes = (sbytes + (2 if args.rand == "pool" else 0) + (nbits + OVERHEAD_BITS) / 8.0) * n
     dec_bytes = (sbytes + (nbits + OVERHEAD_BITS) / 8.0) * n
     comp_gbs = comp_bytes / (comp_ms * 1e-3) / 1e9
     dec_gbs = dec_bytes / (dec_ms * 1e-3) / 1e9
@@ -159,7 +164,11 @@ def main():
             return t.view(torch.int16).numpy().view(np.uint16).copy()
 
         src_h = host_bits(src)
-        rand_h = host_bits(rand.float() if args.src == "fp32" else rand)
+        if args.rand == "philox":
+            uni = O.philox_uniform(m, 2026, 0)
+            rand_h = uni if args.src == "fp32" else (uni.view(np.uint32) >> 16).astype(np.uint16)   # k/256 is exact in bf16
+        else:
+            rand_h = host_bits(rand.float() if args.src == "fp32" else rand)
         if not args.no_check:
             enc_o = O.scaling_compress(src_h, rand_h, m, nbits, C, strategy, odt)
             dec_o = np.zeros(m, src_h.dtype)
@@ -199,8 +208,9 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "one 25 MB DDP bucket: %d %s gradient elements, Student-t(3)*1e-3 with 0.1%% outliers x100; "
-                        "%d-bit hierarchical %s compress + decompress, chunk 16, bf16 rand_pool"
-                        % (n, args.src, nbits, "AEE" if strategy == 2 else "MEE"),
+                        "%d-bit hierarchical %s compress + decompress, chunk 16, %s"
+                        % (n, args.src, nbits, "AEE" if strategy == 2 else "MEE",
+                           "bf16 rand_pool" if args.rand == "pool" else "in-kernel Philox rounding"),
             "elements": n,
             "nbits": nbits,
             "strategy": strategy,
@@ -215,7 +225,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(comp_gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.src, nbits, strategy, n)),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.src, nbits, strategy, n)) if args.rand == "pool" else None,
             "algorithmic_bytes_per_launch": int(comp_bytes),
             "avg_launch_ms": round(comp_ms, 5),
         },

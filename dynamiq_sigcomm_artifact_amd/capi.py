@@ -20,6 +20,7 @@ EXPORTS = [
     "dq_scaling_required_bytes", "dq_scaling_check_common",
     "dq_init_lookup_table", "dq_mee_lookup_table",
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
+    "dq_scaling_compress_philox", "dq_scaling_dec_comp_philox", "dq_philox_uniform",
     "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
@@ -61,6 +62,12 @@ def lib():
         L.dq_scaling_decompress.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, vp, i32]
         L.dq_scaling_dec_comp.restype = i32
         L.dq_scaling_dec_comp.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp]
+        L.dq_scaling_compress_philox.restype = i32
+        L.dq_scaling_compress_philox.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32, u64, u64, vp]
+        L.dq_scaling_dec_comp_philox.restype = i32
+        L.dq_scaling_dec_comp_philox.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, i32, u64, u64, vp]
+        L.dq_philox_uniform.restype = i32
+        L.dq_philox_uniform.argtypes = [vp, i64, i32, i32, u64, u64, vp]
         L.dq_group_plan_work_ints.restype = i64
         L.dq_group_plan_work_ints.argtypes = [i64]
         L.dq_group_plan.restype = i32
@@ -213,6 +220,23 @@ def scaling_decompress_rows(src, dst, rows, stats, n_limit, nrows, nbits, strate
     _check(lib().dq_scaling_decompress_rows(src.data_ptr(), dst.data_ptr(), _ptr(rows), _ptr(stats), n_limit, nrows,
                                             nbits, dtype_code(dst), _dev(dst), strategy, _stream(stream),
                                             1 if add else 0))
+
+
+def scaling_compress_philox(src, dst, n, nbits, chunk_size, strategy, seed, step, stream=None):
+    """scaling_compress with the uniform values drawn in the kernel (Philox keyed by seed, counter = chunk, step)"""
+    _check(lib().dq_scaling_compress_philox(src.data_ptr(), dst.data_ptr(), n, nbits, chunk_size, dtype_code(src), _dev(src),
+                                            strategy, int(seed), int(step), _stream(stream)))
+
+
+def scaling_dec_comp_philox(recv, inp, send, n, nbits, chunk_size, strategy, seed, step, stream=None):
+    _check(lib().dq_scaling_dec_comp_philox(recv.data_ptr(), inp.data_ptr(), send.data_ptr(), n, nbits, chunk_size,
+                                            dtype_code(inp), _dev(inp), strategy, int(seed), int(step), _stream(stream)))
+
+
+def philox_uniform(out, seed, step, stream=None):
+    """the uniform values of that stream as a tensor (any of the three element types)"""
+    _check(lib().dq_philox_uniform(out.data_ptr(), out.numel(), dtype_code(out), _dev(out), int(seed), int(step),
+                                   _stream(stream)))
 
 
 def superchunk_mean_center(src, residual, stats, n, world_size, superchunk_size=256, stream=None):

@@ -57,6 +57,16 @@ class _DynamicRangeGPUKern(object):
 
         self.three_times_cur_max_size = (3 * self.cur_max_size) // self.nclients
         pool = params.get("rand_pool_tensor")
+        # not in the reference: params["philox_seed"] draws the rounding randomness inside the kernels (one stream per
+        # rank, one step per call) and allocates no pool
+        self.philox_seed = params.get("philox_seed")
+        if self.philox_seed is not None:
+            self.philox_seed = (int(self.philox_seed) + self.client_rank * 0x9E3779B97F4A7C15) & 0xFFFFFFFFFFFFFFFF
+            self.philox_step = (self.nbits << 32)
+            self.randomized_vec_pool = None
+            self.randomized_vec_pools = {}
+            self.rand_seed = (self.nbits * 998244353) & 0xFFFFFFFF
+            return
         if pool is not None:
             # caller-provided pool (the reference's "correlated" mode loads one from disk)
             self.randomized_vec_pool = pool.to(device=device)[: self.three_times_cur_max_size * self.chunk_size].view(
@@ -107,9 +117,17 @@ class _DynamicRangeGPUKern(object):
     def _stream(self):
         return torch.cuda.current_stream().cuda_stream
 
+    def _next_step(self):
+        self.philox_step += 1
+        return self.philox_step
+
     def compression(self, input_chunk, send_chunk, interm_chunk=None):
         n = input_chunk.numel()
         if n == 0:
+            return
+        if self.philox_seed is not None:
+            self.eden_utils.scaling_compress_philox(input_chunk, send_chunk, n, self.nbits, self.chunk_size, self.philox_seed,
+                                                    self._next_step(), self._stream(), self.strategy)
             return
         rand_vec = self.rand_pool(n, input_chunk.dtype)
         self._compress(input_chunk, send_chunk, rand_vec, n, self.nbits, self.chunk_size,
@@ -125,6 +143,10 @@ class _DynamicRangeGPUKern(object):
     def dec_compression(self, recv_chunk, input_chunk, send_chunk, interm_chunk=None, interm_chunk2=None):
         n = input_chunk.numel()
         if n == 0:
+            return
+        if self.philox_seed is not None:
+            self.eden_utils.scaling_dec_comp_philox(recv_chunk, input_chunk, send_chunk, n, self.nbits, self.chunk_size,
+                                                    self.philox_seed, self._next_step(), self._stream(), self.strategy)
             return
         rand_vec = self.rand_pool(n, input_chunk.dtype)
         self._dec_comp(recv_chunk, input_chunk, send_chunk, rand_vec, n, self.nbits, self.chunk_size,

@@ -358,6 +358,52 @@ int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *row
                                                     mee_params(nbits), add_original, static_cast<hipStream_t>(stream)));
 }
 
+int dq_scaling_compress_philox(const void *src, uint8_t *dst, int64_t n, int nbits, int chunk_size, int dtype, int device,
+                               int strategy, uint64_t seed, uint64_t step, dq_stream_t stream)
+{
+    int rc = check_common(n, nbits, chunk_size, strategy, 0);
+    if (rc) return fail(rc);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (chunk_size != 16) return fail(DQ_ERR_CHUNK_RANGE, "the in-kernel random stream is defined for chunk_size 16");
+    if (!src || !dst) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dq::MeeParams &mp = mee_params(nbits);
+    if (hier16_shape(dtype, chunk_size, strategy))
+        return finish(dq::launch_hier16_compress_philox(src, nullptr, dst, n, nbits, dtype, strategy == 3, mp, seed, step, s));
+    const dq::RandKey key{seed, step};
+    return finish(dq::launch_tile16_compress(src, dst, nullptr, n, nbits, dtype, strategy, mp, s, &key));
+}
+
+int dq_scaling_dec_comp_philox(const uint8_t *recv, void *inp, uint8_t *send, int64_t n, int nbits, int chunk_size, int dtype,
+                               int device, int strategy, uint64_t seed, uint64_t step, dq_stream_t stream)
+{
+    int rc = check_common(n, nbits, chunk_size, strategy, 0);
+    if (rc) return fail(rc);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (chunk_size != 16) return fail(DQ_ERR_CHUNK_RANGE, "the in-kernel random stream is defined for chunk_size 16");
+    if (!recv || !inp || !send) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dq::MeeParams &mp = mee_params(nbits);
+    if (hier16_shape(dtype, chunk_size, strategy))
+        return finish(dq::launch_hier16_compress_philox(inp, recv, send, n, nbits, dtype, strategy == 3, mp, seed, step, s));
+    hipError_t e = dq::launch_tile16_decompress(recv, inp, n, nbits, dtype, strategy, mp, 1, s);
+    if (e != hipSuccess) return finish(e);
+    const dq::RandKey key{seed, step};
+    return finish(dq::launch_tile16_compress(inp, send, nullptr, n, nbits, dtype, strategy, mp, s, &key));
+}
+
+int dq_philox_uniform(void *out, int64_t n, int dtype, int device, uint64_t seed, uint64_t step, dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!out) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_philox_uniform(out, n, dtype, seed, step, static_cast<hipStream_t>(stream)));
+}
+
 int dq_superchunk_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size,
                               int superchunk_size, int dtype, int device, dq_stream_t stream)
 {

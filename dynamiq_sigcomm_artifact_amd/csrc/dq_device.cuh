@@ -244,4 +244,42 @@ struct MeeParams {
     uint16_t table[256]; // binary16 bit patterns
 };
 
+// ---- counter-based random stream ----------------------------------------------------
+
+// Philox4x32-10 (Salmon et al., SC'11): counter c, key (k0, k1)
+__host__ __device__ __forceinline__ void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1)
+{
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+// The in-kernel random stream of the scaling quantiser: key = seed, counter = (chunk index, step).
+// One block gives the 16 uniform values of one 16-element chunk: element i takes byte i of the four
+// output words (little endian), u = (byte | 1) * 2^-8, i.e. the 128 odd multiples of 1/256: centred in
+// their cells (a value k/256 would round up with probability ceil(256 f)/256 > f, a bias of 1/512 of a
+// step on every element) and exactly representable in binary16, bfloat16 and binary32.
+struct RandKey {
+    uint64_t seed;
+    uint64_t step;
+};
+
+__host__ __device__ __forceinline__ void chunk_uniform_words(const RandKey &key, int64_t chunk, uint32_t (&w)[4])
+{
+    w[0] = (uint32_t)chunk;
+    w[1] = (uint32_t)((uint64_t)chunk >> 32);
+    w[2] = (uint32_t)key.step;
+    w[3] = (uint32_t)(key.step >> 32);
+    philox4x32_10(w, (uint32_t)key.seed, (uint32_t)(key.seed >> 32));
+}
+
 } // namespace dq

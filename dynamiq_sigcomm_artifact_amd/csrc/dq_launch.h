@@ -25,6 +25,10 @@ hipError_t launch_hier16_compress(const void *src, uint8_t *dst, const void *rnd
                                   hipStream_t stream);
 hipError_t launch_hier16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype,
                                     bool mee, const MeeParams &mp, int add, hipStream_t stream);
+// compress (recv == null) or the fused ring step with the uniform values drawn in the kernel
+hipError_t launch_hier16_compress_philox(const void *src, const uint8_t *recv, uint8_t *dst, int64_t n,
+                                         int nbits, int dtype, bool mee, const MeeParams &mp,
+                                         uint64_t seed, uint64_t step, hipStream_t stream);
 hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t *send,
                                   const void *rnd, int64_t n, int nbits, int dtype, bool mee,
                                   const MeeParams &mp, hipStream_t stream);
@@ -32,7 +36,11 @@ hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t 
 // vectorised chunk-16 kernels for the remaining shapes (dq_scaling_tile16.hip): binary16 elements
 // with any strategy, bf16 / fp32 elements with the flat strategies 0 / 1
 hipError_t launch_tile16_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n, int nbits,
-                                  int dtype, int strategy, const MeeParams &mp, hipStream_t stream);
+                                  int dtype, int strategy, const MeeParams &mp, hipStream_t stream,
+                                  const RandKey *philox = nullptr);
+// the in-kernel random stream (dq_device.cuh: chunk_uniform_words) written out as a tensor
+hipError_t launch_philox_uniform(void *out, int64_t n, int dtype, uint64_t seed, uint64_t step,
+                                 hipStream_t stream);
 hipError_t launch_tile16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype,
                                     int strategy, const MeeParams &mp, int add, hipStream_t stream);
 

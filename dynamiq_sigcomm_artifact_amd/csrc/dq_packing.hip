@@ -53,24 +53,6 @@ hipError_t launch_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr
     return hipGetLastError();
 }
 
-// ---- Philox4x32-10 -------------------------------------------------------------------
-
-__device__ __forceinline__ void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1)
-{
-#pragma unroll
-    for (int r = 0; r < 10; r++) {
-        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
-        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
-        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
-        const uint32_t n1 = (uint32_t)p1;
-        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
-        const uint32_t n3 = (uint32_t)p0;
-        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
-        k0 += 0x9E3779B9u;
-        k1 += 0xBB67AE85u;
-    }
-}
-
 // four consecutive elements per thread share one Philox block keyed by
 // (seed, element index / 4); u = top 24 bits * 2^-24 in [0, 1)
 __global__ __launch_bounds__(256) void quantization_kernel(float *__restrict__ vec, int64_t n, float div_factor,

@@ -140,7 +140,7 @@ template <int DT, int RDT, int NBITS, bool MEE, bool FUSED>
 __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restrict__ src, const uint8_t *__restrict__ recv,
                                                             uint8_t *__restrict__ dst, const void *__restrict__ rnd,
                                                             const int32_t *__restrict__ rows, int64_t nsc, int vec,
-                                                            MeeArg<NBITS, MEE> mp)
+                                                            RandKey key, MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
     __shared__ __attribute__((aligned(16))) uint8_t win_out[RC::WIN];
@@ -159,7 +159,10 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     Raw16<DT> v;
     Raw16<RDT> r;
     if (active) {
-        r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
+        if constexpr (RDT == DQ_PHILOX)
+            r.generate(key, sc0 * 16 + lane);
+        else
+            r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
         const int64_t sc_src = rows ? (int64_t)rows[sc0 + row] : sc0 + row;
         v.load(src, (sc_src * 16 + j) * 16, vec & 1);
     } else {
@@ -338,15 +341,15 @@ static inline unsigned grid_for(int64_t nsc) { return (unsigned)((nsc + kRowsPer
 
 template <int DT, int RDT, int NBITS, bool MEE>
 static hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, const int32_t *rows,
-                               int64_t nsc, bool fused, const MeeParams &mp, hipStream_t stream)
+                               int64_t nsc, bool fused, const MeeParams &mp, RandKey key, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
     dim3 grid(grid_for(nsc)), block(64);
     const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
     if (fused)
-        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, rows, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, rows, nsc, vec, key, arg);
     else
-        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, rows, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_compress_kernel<DT, RDT, NBITS, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, rows, nsc, vec, key, arg);
     return hipGetLastError();
 }
 
@@ -380,16 +383,24 @@ static hipError_t run_decompress(const uint8_t *src, void *dst, const int32_t *r
 
 static hipError_t dispatch_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd,
                                     const int32_t *rows, int64_t nsc, bool fused, int nbits, int dtype, bool mee,
-                                    const MeeParams &mp, hipStream_t stream)
+                                    const MeeParams &mp, hipStream_t stream, const RandKey *philox = nullptr)
 {
     const bool rb16 = (dtype & DQ_RAND_BF16) != 0;
     dtype &= 0xf;
+    const RandKey key = philox ? *philox : RandKey{0, 0};
+    if (philox) {
+        if (dtype == DQ_BF16) {
+            DQ_NBITS_MEE(run_compress, DQ_BF16 DQ_COMMA DQ_PHILOX, src, recv, dst, rnd, rows, nsc, fused, mp, key, stream)
+        } else {
+            DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_PHILOX, src, recv, dst, rnd, rows, nsc, fused, mp, key, stream)
+        }
+    }
     if (dtype == DQ_BF16) {
-        DQ_NBITS_MEE(run_compress, DQ_BF16 DQ_COMMA DQ_BF16, src, recv, dst, rnd, rows, nsc, fused, mp, stream)
+        DQ_NBITS_MEE(run_compress, DQ_BF16 DQ_COMMA DQ_BF16, src, recv, dst, rnd, rows, nsc, fused, mp, key, stream)
     } else if (rb16) {
-        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_BF16, src, recv, dst, rnd, rows, nsc, fused, mp, stream)
+        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_BF16, src, recv, dst, rnd, rows, nsc, fused, mp, key, stream)
     } else {
-        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_F32, src, recv, dst, rnd, rows, nsc, fused, mp, stream)
+        DQ_NBITS_MEE(run_compress, DQ_F32 DQ_COMMA DQ_F32, src, recv, dst, rnd, rows, nsc, fused, mp, key, stream)
     }
 }
 
@@ -403,6 +414,13 @@ hipError_t launch_hier16_dec_comp(const uint8_t *recv, const void *inp, uint8_t 
                                   int nbits, int dtype, bool mee, const MeeParams &mp, hipStream_t stream)
 {
     return dispatch_compress(inp, recv, send, rnd, nullptr, n / 256, true, nbits, dtype, mee, mp, stream);
+}
+
+hipError_t launch_hier16_compress_philox(const void *src, const uint8_t *recv, uint8_t *dst, int64_t n, int nbits, int dtype,
+                                         bool mee, const MeeParams &mp, uint64_t seed, uint64_t step, hipStream_t stream)
+{
+    const RandKey key{seed, step};
+    return dispatch_compress(src, recv, dst, nullptr, nullptr, n / 256, recv != nullptr, nbits, dtype, mee, mp, stream, &key);
 }
 
 hipError_t launch_hier16_compress_rows(const void *src, const uint8_t *recv, const int32_t *rows, uint8_t *dst,

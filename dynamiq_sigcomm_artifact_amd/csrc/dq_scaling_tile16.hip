@@ -53,7 +53,7 @@ __device__ __forceinline__ bool ordinary_scale(float d)
 template <int DT, int RDT, int NBITS, bool HIER, bool MEE>
 __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restrict__ src, uint8_t *__restrict__ dst,
                                                             const void *__restrict__ rnd, int64_t nchunks, int vec,
-                                                            MeeArg<NBITS, MEE> mp)
+                                                            RandKey key, MeeArg<NBITS, MEE> mp)
 {
     typedef Geo<NBITS, HIER> G;
     constexpr int R = Rec<NBITS>::R;
@@ -70,7 +70,10 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
     Raw16<RDT> r;
     if (active) {
         v.load(src, (c0 + lane) * 16, vec & 1);
-        r.load(rnd, (c0 + lane) * 16, vec & 2);
+        if constexpr (RDT == DQ_PHILOX)
+            r.generate(key, c0 + lane);
+        else
+            r.load(rnd, (c0 + lane) * 16, vec & 2);
     } else {
         v.zero();
         r.zero();
@@ -242,15 +245,15 @@ inline unsigned grid_for(int64_t nchunks) { return (unsigned)((nchunks + kChunks
 
 template <int DT, int RDT, int NBITS, bool MEE>
 hipError_t run_compress(const void *src, uint8_t *dst, const void *rnd, int64_t nchunks, bool hier, const MeeParams &mp,
-                        hipStream_t stream)
+                        RandKey key, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
     const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
     dim3 grid(grid_for(nchunks)), block(64);
     if (DT == DQ_F16 && hier)
-        hipLaunchKernelGGL((tile16_compress_kernel<DQ_F16, DQ_F16, NBITS, true, MEE>), grid, block, 0, stream, src, dst, rnd, nchunks, vec, arg);
+        hipLaunchKernelGGL((tile16_compress_kernel<DQ_F16, RDT, NBITS, true, MEE>), grid, block, 0, stream, src, dst, rnd, nchunks, vec, key, arg);
     else
-        hipLaunchKernelGGL((tile16_compress_kernel<DT, RDT, NBITS, false, MEE>), grid, block, 0, stream, src, dst, rnd, nchunks, vec, arg);
+        hipLaunchKernelGGL((tile16_compress_kernel<DT, RDT, NBITS, false, MEE>), grid, block, 0, stream, src, dst, rnd, nchunks, vec, key, arg);
     return hipGetLastError();
 }
 
@@ -275,6 +278,18 @@ hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nchunks, bool h
     return hipGetLastError();
 }
 
+// the uniform values of the in-kernel stream written out as a tensor: element e = chunk e / 16, byte e % 16
+template <int DT>
+__global__ __launch_bounds__(256) void philox_uniform_kernel(void *__restrict__ out, int64_t n, RandKey key)
+{
+    const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (chunk * 16 >= n) return;
+    Raw16<DQ_PHILOX> r;
+    r.generate(key, chunk);
+    const int cnt = (int)min((int64_t)16, n - chunk * 16);
+    for (int i = 0; i < cnt; i++) ElemIO<DT>::store(out, chunk * 16 + i, r.get(i));
+}
+
 #define DQ_T16_NBITS_MEE(FN, PRE, ...)                                                                    \
     switch (nbits) {                                                                                      \
     case 2: return mee ? FN<PRE, 2, true>(__VA_ARGS__) : FN<PRE, 2, false>(__VA_ARGS__);                  \
@@ -291,21 +306,43 @@ hipError_t run_decompress(const uint8_t *src, void *dst, int64_t nchunks, bool h
 
 // dtype F16 with any strategy, or BF16 / F32 with strategy 0 / 1; chunk size 16
 hipError_t launch_tile16_compress(const void *src, uint8_t *dst, const void *rnd, int64_t n, int nbits, int dtype,
-                                  int strategy, const MeeParams &mp, hipStream_t stream)
+                                  int strategy, const MeeParams &mp, hipStream_t stream, const RandKey *philox)
 {
     const bool rb16 = (dtype & DQ_RAND_BF16) != 0;
     dtype &= 0xf;
     const bool mee = (strategy & 1) != 0, hier = strategy >= 2;
     const int64_t nchunks = n / 16;
-    if (dtype == DQ_F16) {
-        DQ_T16_NBITS_MEE(run_compress, DQ_F16 DQ_T16_COMMA DQ_F16, src, dst, rnd, nchunks, hier, mp, stream)
-    } else if (dtype == DQ_BF16) {
-        DQ_T16_NBITS_MEE(run_compress, DQ_BF16 DQ_T16_COMMA DQ_BF16, src, dst, rnd, nchunks, false, mp, stream)
-    } else if (rb16) {
-        DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_BF16, src, dst, rnd, nchunks, false, mp, stream)
-    } else {
-        DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_F32, src, dst, rnd, nchunks, false, mp, stream)
+    const RandKey key = philox ? *philox : RandKey{0, 0};
+    if (philox) {
+        if (dtype == DQ_F16) {
+            DQ_T16_NBITS_MEE(run_compress, DQ_F16 DQ_T16_COMMA DQ_PHILOX, src, dst, rnd, nchunks, hier, mp, key, stream)
+        } else if (dtype == DQ_BF16) {
+            DQ_T16_NBITS_MEE(run_compress, DQ_BF16 DQ_T16_COMMA DQ_PHILOX, src, dst, rnd, nchunks, false, mp, key, stream)
+        } else {
+            DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_PHILOX, src, dst, rnd, nchunks, false, mp, key, stream)
+        }
     }
+    if (dtype == DQ_F16) {
+        DQ_T16_NBITS_MEE(run_compress, DQ_F16 DQ_T16_COMMA DQ_F16, src, dst, rnd, nchunks, hier, mp, key, stream)
+    } else if (dtype == DQ_BF16) {
+        DQ_T16_NBITS_MEE(run_compress, DQ_BF16 DQ_T16_COMMA DQ_BF16, src, dst, rnd, nchunks, false, mp, key, stream)
+    } else if (rb16) {
+        DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_BF16, src, dst, rnd, nchunks, false, mp, key, stream)
+    } else {
+        DQ_T16_NBITS_MEE(run_compress, DQ_F32 DQ_T16_COMMA DQ_F32, src, dst, rnd, nchunks, false, mp, key, stream)
+    }
+}
+
+hipError_t launch_philox_uniform(void *out, int64_t n, int dtype, uint64_t seed, uint64_t step, hipStream_t stream)
+{
+    const RandKey key{seed, step};
+    dim3 grid((unsigned)(((n + 15) / 16 + 255) / 256)), block(256);
+    switch (dtype) {
+    case DQ_F16: hipLaunchKernelGGL(philox_uniform_kernel<DQ_F16>, grid, block, 0, stream, out, n, key); break;
+    case DQ_BF16: hipLaunchKernelGGL(philox_uniform_kernel<DQ_BF16>, grid, block, 0, stream, out, n, key); break;
+    default: hipLaunchKernelGGL(philox_uniform_kernel<DQ_F32>, grid, block, 0, stream, out, n, key); break;
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_tile16_decompress(const uint8_t *src, void *dst, int64_t n, int nbits, int dtype, int strategy,

@@ -184,6 +184,21 @@ template <> struct Raw16<DQ_F16> : Raw16<DQ_BF16> {
     }
 };
 
+// the 16 uniform values of a chunk drawn in the kernel (element type tag for the random operand)
+constexpr int DQ_PHILOX = 3;
+
+template <> struct Raw16<DQ_PHILOX> {
+    uint32_t w[4];
+    __device__ __forceinline__ void zero() { w[0] = w[1] = w[2] = w[3] = 0; }
+    __device__ __forceinline__ void generate(const RandKey &key, int64_t chunk) { chunk_uniform_words(key, chunk, w); }
+    __device__ __forceinline__ void load(const void *, int64_t, bool) {}
+    __device__ __forceinline__ float get(int i) const
+    {
+        return (float)(((w[i >> 2] >> (8 * (i & 3))) & 0xffu) | 1u) * 0.00390625f;
+    }
+    __device__ __forceinline__ bool unit_interval() const { return true; }
+};
+
 // ---- record windows --------------------------------------------------------------------
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

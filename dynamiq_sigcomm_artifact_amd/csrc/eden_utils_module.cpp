@@ -475,6 +475,58 @@ torch::Tensor EdenBitsToBins(torch::Tensor arr, int nbits)
     return cbins;
 }
 
+// ---- in-kernel random stream (additions; see include/dynamiq_eden.h) ------------------------
+
+void scaling_compress_philox(torch::Tensor src, torch::Tensor dst, int64_t n, int nbits, int chunk_size, uint64_t seed,
+                             uint64_t step, uint64_t stream_p = 0, int strategy = 0)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(is_supported_data_dtype(src.scalar_type(), true), "input must be torch.float16, torch.bfloat16 or torch.float32");
+    TORCH_CHECK(dst.dtype() == torch::kUInt8, "output must be torch.uint8");
+    TORCH_CHECK(src.is_contiguous(), "input must be contiguous");
+    TORCH_CHECK(dst.is_contiguous(), "output must be contiguous");
+    scaling_check_common((int)n, nbits, chunk_size, strategy, true);
+    TORCH_CHECK(chunk_size == 16, "the in-kernel random stream is defined for chunk_size 16");
+    TORCH_CHECK(src.numel() >= n, "input has fewer than n elements");
+    TORCH_CHECK(dst.numel() >= dq_scaling_required_bytes(n, nbits, chunk_size, strategy), "output buffer is too small");
+    check_status(dq_scaling_compress_philox(src.data_ptr(), dst.data_ptr<uint8_t>(), n, nbits, chunk_size,
+                                            dq_dtype_of(src.scalar_type()), src.device().index(), strategy, seed, step,
+                                            as_stream(stream_p)),
+                 "scaling_compress_philox");
+}
+
+void scaling_dec_comp_philox(torch::Tensor recv, torch::Tensor inp, torch::Tensor send, int64_t n, int nbits, int chunk_size,
+                             uint64_t seed, uint64_t step, uint64_t stream_p = 0, int strategy = 0)
+{
+    TORCH_CHECK(recv.device().type() == torch::kCUDA && inp.device().type() == torch::kCUDA && send.device().type() == torch::kCUDA,
+                "all buffers must be CUDA tensors");
+    TORCH_CHECK(recv.dtype() == torch::kUInt8, "recv must be torch.uint8");
+    TORCH_CHECK(send.dtype() == torch::kUInt8, "send must be torch.uint8");
+    TORCH_CHECK(is_supported_data_dtype(inp.scalar_type(), true), "inp must be torch.float16, torch.bfloat16 or torch.float32");
+    TORCH_CHECK(recv.is_contiguous() && inp.is_contiguous() && send.is_contiguous(), "buffers must be contiguous");
+    scaling_check_common((int)n, nbits, chunk_size, strategy, true);
+    TORCH_CHECK(chunk_size == 16, "the in-kernel random stream is defined for chunk_size 16");
+    const int64_t required_bytes = dq_scaling_required_bytes(n, nbits, chunk_size, strategy);
+    TORCH_CHECK(recv.numel() >= required_bytes, "recv buffer is too small");
+    TORCH_CHECK(send.numel() >= required_bytes, "send buffer is too small");
+    TORCH_CHECK(inp.numel() >= n, "inp has fewer than n elements");
+    check_status(dq_scaling_dec_comp_philox(recv.data_ptr<uint8_t>(), inp.data_ptr(), send.data_ptr<uint8_t>(), n, nbits, chunk_size,
+                                            dq_dtype_of(inp.scalar_type()), inp.device().index(), strategy, seed, step,
+                                            as_stream(stream_p)),
+                 "scaling_dec_comp_philox");
+}
+
+void philox_uniform(torch::Tensor out, uint64_t seed, uint64_t step, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(out.device().type() == torch::kCUDA, "out must be a CUDA tensor");
+    TORCH_CHECK(is_supported_data_dtype(out.scalar_type(), true), "out must be torch.float16, torch.bfloat16 or torch.float32");
+    TORCH_CHECK(out.is_contiguous() && out.numel() > 0, "out must be contiguous and not empty");
+    check_status(dq_philox_uniform(out.data_ptr(), out.numel(), dq_dtype_of(out.scalar_type()), out.device().index(), seed, step,
+                                   as_stream(stream_p)),
+                 "philox_uniform");
+}
+
 // ---- EDEN / THC consumers (additions; see include/dynamiq_eden.h) --------------------------
 
 void check_f32_cuda(const torch::Tensor &t, const char *name)
@@ -592,6 +644,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_decompress_rows", &scaling_decompress_rows, "decode consecutive records into the superchunks rows[k] of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("rows"), py::arg("stats"), py::arg("n_limit"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("scaling_compress_philox", &scaling_compress_philox, "scaling compress with the uniform values drawn in the kernel (Philox: key = seed, counter = chunk, step)", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("scaling_dec_comp_philox", &scaling_dec_comp_philox, "scaling decompress and compress with the uniform values drawn in the kernel", py::arg("recv"), py::arg("inp"), py::arg("send"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
+    modul.def("philox_uniform", &philox_uniform, "the uniform values of that stream written out as a tensor", py::arg("out"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0);
     modul.def("eden_quantize", &eden_quantize, "EDEN: normalise, bucketize against the Lloyd-Max boundaries, pack bit planes, scale; returns [packed, result]", py::arg("vec"), py::arg("boundaries"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
     modul.def("eden_dequantize", &eden_dequantize, "EDEN: centroids of the packed bins", py::arg("packed"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
     modul.def("thc_quantize", &thc_quantize, "THC: uniform stochastic quantiser of the rotated vector, bfloat16 levels", py::arg("rotated"), py::arg("uniform"), py::arg("lo"), py::arg("delta"), py::arg("levels"), py::arg("stream_p") = 0);

@@ -111,6 +111,27 @@ int dq_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const voi
                         int64_t n, int nbits, int chunk_size, int dtype, int device,
                         int strategy, dq_stream_t stream);
 
+/* ---- in-kernel random stream -------------------------------------------
+ *
+ * No counterpart in the reference, whose random values always arrive as the
+ * rand_pool tensor (utils_aggregation.py:384-397).  Here the uniform values of
+ * the stochastic rounding are drawn inside the kernel from Philox4x32-10:
+ * key = seed, counter = (chunk index, step); the 16 bytes of one block are the
+ * 16 values of one chunk, u = (byte | 1) / 256 (the odd multiples of 1/256:
+ * unbiased rounding, exact in all three element types).  This removes the 2 (4) bytes per
+ * element the pool costs in HBM reads.  chunk_size must be 16; every dtype and
+ * strategy.  The result equals dq_scaling_compress / dq_scaling_dec_comp fed
+ * with the tensor dq_philox_uniform writes for the same (seed, step). */
+int dq_scaling_compress_philox(const void *src, uint8_t *dst, int64_t n, int nbits, int chunk_size,
+                               int dtype, int device, int strategy, uint64_t seed, uint64_t step,
+                               dq_stream_t stream);
+int dq_scaling_dec_comp_philox(const uint8_t *recv, void *inp, uint8_t *send, int64_t n, int nbits,
+                               int chunk_size, int dtype, int device, int strategy, uint64_t seed,
+                               uint64_t step, dq_stream_t stream);
+/* out: `dtype` elements [n]; element e = (byte e % 16 of the block of chunk e / 16, low bit set) * 2^-8 */
+int dq_philox_uniform(void *out, int64_t n, int dtype, int device, uint64_t seed, uint64_t step,
+                      dq_stream_t stream);
+
 /* ---- dynamic-bitrate groups: gather / scatter folded into the codec ----
  *
  * The reference's dynamic-bitrate hook builds, per bit width w in {8, 4, 2}, the

@@ -256,6 +256,26 @@ def bits_to_bins(arr, nbits):
     return bins
 
 
+def philox4x32_10(ctr, key):
+    c = np.asarray(ctr, np.uint32)
+    k = np.asarray(key, np.uint32)
+    out = np.zeros(4, np.uint32)
+    f = lib().dqo_philox4x32_10
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p] * 3
+    f(_p(c), _p(k), _p(out))
+    return out
+
+
+def philox_uniform(n, seed, step):
+    out = np.zeros(n, np.float32)
+    f = lib().dqo_philox_uniform
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_uint64]
+    f(_p(out), n, int(seed), int(step))
+    return out
+
+
 def eden_quantize(vec, boundaries, centroids, nbits):
     """-> (bins int32 [n], result float32 [4] = sumsq, dot, scale, norm)"""
     _chk(vec, np.float32, "vec")

@@ -799,6 +799,42 @@ void dqo_bits_to_bins(const uint32_t *arr, int64_t narr, int32_t *bins, int nbit
 }
 
 /* ------------------------------------------------------------------------ */
+/* counter-based random stream of the in-kernel rounding                     */
+/* ------------------------------------------------------------------------ */
+
+/* Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11) */
+void dqo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+{
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* element e: block with key = seed, counter = (chunk e / 16, step); u = (byte e % 16 of the four output
+ * words, little endian, with its low bit set) * 2^-8: the odd multiples of 1/256 */
+void dqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t step)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    for (int64_t chunk = 0; chunk * 16 < n; chunk++) {
+        const uint32_t ctr[4] = {(uint32_t)chunk, (uint32_t)((uint64_t)chunk >> 32), (uint32_t)step, (uint32_t)(step >> 32)};
+        uint32_t w[4];
+        dqo_philox4x32_10(ctr, key, w);
+        for (int i = 0; i < 16 && chunk * 16 + i < n; i++)
+            out[chunk * 16 + i] = (float)(((w[i >> 2] >> (8 * (i & 3))) & 0xffu) | 1u) * 0.00390625f;
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* EDEN Lloyd-Max quantiser, THC uniform quantiser                           */
 /* ------------------------------------------------------------------------ */
 

@@ -26,7 +26,7 @@
  *
  * What pins this file (tests/test_oracle_*.py): the reference's golden vectors
  * for randDiag, the bit-plane packer, the torch butterfly and 50 Eden
- * compress / decompress runs (tests/golden/*.npz, written by the reference's own
+ * compress / decompress runs (the .npz files under tests/golden, written by the reference's own
  * CPU code); closed forms, special cases and invariants of the reference's
  * functional test for the scaling quantiser; an independently written numpy
  * model of the bf16 / fp16 arithmetic.
@@ -126,6 +126,11 @@ void dqo_rand_diag(float *out, int64_t size, int64_t seed);
 /* csrc/cuda_packing.cu:11-29 / 76-95 and srrcomp.py:124-167 */
 void dqo_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits);
 void dqo_bits_to_bins(const uint32_t *arr, int64_t narr, int32_t *bins, int nbits);
+
+/* The random stream of the library's in-kernel rounding mode (no counterpart in the reference, whose
+ * random values are an input tensor): Philox4x32-10, pinned by the published known-answer vectors. */
+void dqo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+void dqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t step);
 
 /* cuda_kernels/src/srrcomp/srrcomp.py:356-361 (Eden._quantize) and :343-345; sums in double in the
  * library's documented order (torch's reduction order is unspecified: "parity unpinned" for the

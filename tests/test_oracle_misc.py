@@ -225,3 +225,24 @@ def test_bit_width_rule_non_finite_norms(oracle):
     norms = torch.tensor([float("inf"), float("nan"), 0.0, -1.0, 1e-30], dtype=torch.bfloat16)
     assert oracle.dynamic_bitrate_qbits(to_bits(norms), 60.0).tolist() == [8, 2, 8, 8, 8]
     assert oracle.dynamic_bitrate_qbits(to_bits(norms), -10.0).tolist() == [8, 2, 2, 2, 2]
+
+
+def test_philox_known_answers(oracle):
+    """Philox4x32-10 known-answer vectors published with Random123 (kat_vectors: zeros, all ones, digits of pi)"""
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+        ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+         [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+    ]
+    for ctr, key, want in kat:
+        assert oracle.philox4x32_10(ctr, key).tolist() == want
+    # the stream of the rounding mode: element e = byte e % 16 of block (chunk e / 16, step), key = seed
+    import numpy as np
+    seed, step = 0x299f31d0a4093822, 0x0370734413198a2e
+    u = oracle.philox_uniform(40, seed, step)
+    for chunk in (0, 1, 2):
+        w = oracle.philox4x32_10([chunk, 0, step & 0xffffffff, step >> 32], [seed & 0xffffffff, seed >> 32])
+        want = (np.frombuffer(w.astype("<u4").tobytes(), np.uint8) | 1).astype(np.float32) / 256
+        got = u[16 * chunk: 16 * chunk + 16]
+        assert (got == want[:got.size]).all()
