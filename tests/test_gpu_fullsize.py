@@ -148,6 +148,40 @@ def test_config5_properties_at_2_pow_28(capi, oracle, nbits):
         assert (to_bits(out[sl]).view(np.uint32) == dec_o.view(np.uint32)).all()
 
 
+def test_more_than_2_pow_31_elements(capi, oracle):
+    """64-bit indexing: 2^31 + 2^20 bf16 elements in one call (the binding's `int n` cannot say this, the C ABI can);
+    the tiles on both sides of the 2^31 boundary and the very last one against the oracle"""
+    n = (1 << 31) + (1 << 20)
+    g = torch.Generator(device=DEV).manual_seed(9)
+    x = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    rnd = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    step = 1 << 28
+    for off in range(0, n, step):
+        m = min(step, n - off)
+        x[off:off + m] = (torch.randn(m, generator=g, device=DEV) * 1e-3).to(torch.bfloat16)
+        rnd[off:off + m] = torch.rand(m, generator=g, device=DEV).to(torch.bfloat16)
+    nbytes = capi.required_bytes(n, 4, 16, 3)
+    assert nbytes == n // 256 * 146
+    enc = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(x, enc, rnd, n, 4, 16, 3)
+    out = torch.zeros_like(x)
+    capi.scaling_decompress(enc, out, n, 4, 16, 3)
+    send = torch.zeros_like(enc)
+    capi.scaling_dec_comp(enc, x, send, rnd, n, 4, 16, 3)
+    m = 256 * 64
+    for off in ((1 << 31) - m, 1 << 31, n - m):
+        sl = slice(off, off + m)
+        enc_o = oracle.scaling_compress(to_bits(x[sl]), to_bits(rnd[sl]), m, 4, 16, 3, BF16)
+        rec = slice(off // 256 * 146, (off + m) // 256 * 146)
+        assert (enc[rec].cpu().numpy() == enc_o).all()
+        dec_o = np.zeros(m, np.uint16)
+        oracle.scaling_decompress(enc_o, dec_o, m, 4, 16, 3, BF16)
+        assert (to_bits(out[sl]) == dec_o).all()
+        send_o = oracle.scaling_dec_comp(enc_o, to_bits(x[sl]), to_bits(rnd[sl]), m, 4, 16, 3, BF16)
+        assert (send[rec].cpu().numpy() == send_o).all()
+    assert int(out[-1].view(torch.int16)) != 0 or float(x[-1]) == 0.0
+
+
 def test_hadamard_2_pow_28_involution(capi):
     """H(H(x)) = n x exactly on small integers; four passes over 1 GiB"""
     n = 1 << 28

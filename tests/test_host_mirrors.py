@@ -153,3 +153,13 @@ def test_simulated_ring_matches_oracle_schedule(eden_utils, oracle, W, nbits, st
     assert (to_bits(vecs[0]) == want[0]).all()
     nmse = float(((vecs[0].double().cpu() - exact) ** 2).sum() / (exact ** 2).sum())
     assert nmse < {2: 4.0, 4: 0.12, 8: 6e-4}[nbits], nmse
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """no multi-GPU figure is produced: bench.py --gpus 2 exits with a message before touching a device"""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "--gpus must be 1" in r.stderr and r.stdout.strip() == ""
