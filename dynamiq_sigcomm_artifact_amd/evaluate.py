@@ -137,6 +137,44 @@ def config2(dev):
                       roundtrip_GBps_of_fp32_input=round(4.0 * n / (tc + td) / 1e3, 1),
                       compress_frac_hbm=round((sb + 2 + pb) * n / tc / 1e3 / HBM_PEAK, 4),
                       decompress_frac_hbm=round((sb + pb) * n / td / 1e3 / HBM_PEAK, 4))
+    for nbits in (4, 8):
+        _cpu_torch_line(x32, nbits)
+
+
+def _torch_cpu_roundtrip(x, rand, nbits, chunk=16):
+    """the chunk-scaling quantiser as a torch op sequence of the shape the reference's own torch implementation has
+    (csrc/logic.py:225-296: abs, row max, div, add 1e-7, div, floor, stochastic carry from the random tensor, nibble pack;
+    unpack, mul), here on CPU tensors"""
+    rng = (1 << (nbits - 1)) - 1
+    v = x.view(-1, chunk).clone()
+    scale = v.abs().max(dim=1, keepdim=True)[0].div_(rng).add_(1e-7)
+    v.div_(scale)
+    fl = torch.floor(v)
+    codes = fl.add_(rand.view(-1, chunk) < v.sub_(fl)).clamp_(-rng, rng).add_(rng).to(torch.uint8)
+    if nbits == 4:
+        packed = codes[:, 0::2] | (codes[:, 1::2] << 4)
+        codes = torch.stack((packed & 15, packed >> 4), dim=2).reshape(-1, chunk)
+    return codes.float().sub_(rng).mul_(scale).reshape(-1)
+
+
+def _cpu_torch_line(x32, nbits):
+    """median of 5 round trips on all host cores, one warm-up"""
+    import os
+    import time
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    xc = x32.cpu()
+    rc = torch.rand(xc.numel())
+    _torch_cpu_roundtrip(xc, rc, nbits)
+    ts = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        out = _torch_cpu_roundtrip(xc, rc, nbits)
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    _emit(config=2, path="cpu torch op sequence (csrc/logic.py:225-296)", nbits=nbits, threads=threads,
+          roundtrip_ms=round(ts[2] * 1e3, 2), roundtrip_GBps_of_fp32_input=round(4.0 * xc.numel() / ts[2] / 1e9, 3),
+          nmse=_nmse(xc, out))
 
 
 def _params(d, W, r):
