@@ -5,9 +5,9 @@ Every superchunk (256 elements) gets q in {2, 4, 8} bits from its reduced
 squared norm F and a scalar offset u:
     z = clamp(floor(log2(max(NORM_SCALE * log2(max(F, 1e-20)) + u, 1e-20))), 1, 3),  q = 2^z
 and u is steered so that the average q meets a target (nominal bits - 0.625 for
-the scale overhead).  The functions are the reference's torch-op sequences, so
-they run on whatever device and dtype the norms live in (the testbed feeds bf16
-norms, the simulation casts to fp32 first).
+the scale overhead).  ``dynamic_bitrate_qbits`` keeps the reference's torch op
+order exactly (each op rounds in the dtype of the norms, which is what makes the
+widths reproducible); the two searches are written around one evaluation helper.
 """
 import torch
 
@@ -17,88 +17,88 @@ DYNAMIC_BITRATE_U_MAX = 60.0
 DYNAMIC_BITRATE_TOL = 0.1
 DYNAMIC_BITRATE_MAX_ITERS = 32
 DYNAMIC_BITRATE_NORM_SCALE = 4.0 / (512.0 / 17.0)
+_EPS = 1e-20
 
 
 def dynamic_bitrate_target_bitrate(aggregation_method):
-    """comm_hooks.py:56-61: "<n>bit" in the method name, default 5"""
-    method = aggregation_method.lower()
-    for nbits in (8, 7, 6, 5, 4, 3, 2):
-        if f"{nbits}bit" in method:
-            return float(nbits)
-    return 5.0
+    """comm_hooks.py:56-61: the "<n>bit" token of the method name (n = 8 .. 2), 5 when there is none"""
+    name = aggregation_method.lower()
+    found = [b for b in range(8, 1, -1) if "%dbit" % b in name]
+    return float(found[0]) if found else 5.0
 
 
 def dynamic_bitrate_qbits(norms, u):
-    """comm_hooks.py:64-70"""
-    eps = 1e-20
-    log_norms = torch.log2(torch.clamp(norms, min=eps))
-    score = log_norms.mul(DYNAMIC_BITRATE_NORM_SCALE).add(float(u))
-    z = torch.floor(torch.log2(torch.clamp(score, min=eps))).to(torch.int64)
-    z.clamp_(1, 3)
+    """comm_hooks.py:64-70, op for op: clamp, log2, mul, add, clamp, log2, floor, int64, clamp, shift"""
+    score = torch.log2(torch.clamp(norms, min=_EPS)).mul(DYNAMIC_BITRATE_NORM_SCALE).add(float(u))
+    z = torch.floor(torch.log2(torch.clamp(score, min=_EPS))).to(torch.int64).clamp_(1, 3)
     return torch.bitwise_left_shift(torch.ones_like(z), z)
 
 
 def dynamic_bitrate_average_bits(norms_list, u):
-    """comm_hooks.py:73-86"""
-    total_chunks = 0
-    total_bits = None
-    for norms in norms_list:
-        if norms.numel() == 0:
-            continue
-        qbits = dynamic_bitrate_qbits(norms, u)
-        qbits_sum = qbits.sum()
-        total_bits = qbits_sum if total_bits is None else total_bits + qbits_sum
-        total_chunks += qbits.numel()
-    if total_bits is None or total_chunks == 0:
+    """comm_hooks.py:73-86: mean width over all superchunks of all tensors (0.0 for no superchunks)"""
+    tensors = [t for t in norms_list if t.numel() > 0]
+    if not tensors:
         return 0.0
-    return float(total_bits.item()) / total_chunks
+    bits = sum(dynamic_bitrate_qbits(t, u).sum() for t in tensors)
+    return float(bits.item()) / sum(t.numel() for t in tensors)
 
 
 def dynamic_bitrate_avg_delta(norms_list, u, target_avg_bits):
-    avg_bits = dynamic_bitrate_average_bits(norms_list, u)
-    return avg_bits, target_avg_bits - avg_bits
+    """(average width at u, target - average)"""
+    avg = dynamic_bitrate_average_bits(norms_list, u)
+    return avg, target_avg_bits - avg
+
+
+def _clip_u(u):
+    return min(DYNAMIC_BITRATE_U_MAX, max(DYNAMIC_BITRATE_U_MIN, float(u)))
+
+
+class _Best(object):
+    """the candidate with the smallest |delta| seen so far (the first one wins ties)"""
+
+    def __init__(self, u, avg, delta):
+        self.u, self.avg, self.delta = u, avg, delta
+
+    def offer(self, u, avg, delta):
+        if abs(delta) < abs(self.delta):
+            self.u, self.avg, self.delta = u, avg, delta
+
+    def triple(self):
+        return self.u, self.avg, self.delta
 
 
 def dynamic_bitrate_binary_search_u(norms_list, target_avg_bits):
-    """comm_hooks.py:94-114: bisection on u in [-10, 60], at most 32 steps, tolerance 0.1 bit"""
-    low = DYNAMIC_BITRATE_U_MIN
-    high = DYNAMIC_BITRATE_U_MAX
-    best_u = high
-    best_avg, best_delta = dynamic_bitrate_avg_delta(norms_list, best_u, target_avg_bits)
+    """comm_hooks.py:94-114: bisection of u over [-10, 60]; stops at |delta| <= 0.1 bit or after 32 midpoints, then
+    returns the best point seen (the upper end of the interval is the starting candidate)"""
+    lo, hi = DYNAMIC_BITRATE_U_MIN, DYNAMIC_BITRATE_U_MAX
+    best = _Best(hi, *dynamic_bitrate_avg_delta(norms_list, hi, target_avg_bits))
     for _ in range(DYNAMIC_BITRATE_MAX_ITERS):
-        mid = (low + high) * 0.5
-        avg_bits, delta = dynamic_bitrate_avg_delta(norms_list, mid, target_avg_bits)
-        if abs(delta) < abs(best_delta):
-            best_u = mid
-            best_avg = avg_bits
-            best_delta = delta
+        mid = 0.5 * (lo + hi)
+        avg, delta = dynamic_bitrate_avg_delta(norms_list, mid, target_avg_bits)
+        best.offer(mid, avg, delta)
         if abs(delta) <= DYNAMIC_BITRATE_TOL:
-            return mid, avg_bits, delta
-        if delta > 0:
-            low = mid
+            return mid, avg, delta
+        if delta > 0:       # too few bits: raise u
+            lo = mid
         else:
-            high = mid
-    return best_u, best_avg, best_delta
+            hi = mid
+    return best.triple()
 
 
 def dynamic_bitrate_adjust_u(norms_list, prev_u, target_avg_bits):
-    """comm_hooks.py:117-139: incremental correction used after the first compressed round"""
-    prev_u = max(DYNAMIC_BITRATE_U_MIN, min(DYNAMIC_BITRATE_U_MAX, float(prev_u)))
-    old_avg, old_delta = dynamic_bitrate_avg_delta(norms_list, prev_u, target_avg_bits)
-    if abs(old_delta) <= DYNAMIC_BITRATE_TOL:
-        return prev_u, old_avg, old_delta
-    step = old_delta
-    best_u = prev_u
-    best_avg = old_avg
-    best_delta = old_delta
+    """comm_hooks.py:117-139: the correction used after the first compressed round.  Steps from the previous u by the
+    current deficit, halving the step each time, until the tolerance is met or the deficit no longer changes sign."""
+    start = _clip_u(prev_u)
+    avg0, delta0 = dynamic_bitrate_avg_delta(norms_list, start, target_avg_bits)
+    if abs(delta0) <= DYNAMIC_BITRATE_TOL:
+        return start, avg0, delta0
+    best = _Best(start, avg0, delta0)
+    step = delta0
     for _ in range(DYNAMIC_BITRATE_MAX_ITERS):
-        candidate_u = max(DYNAMIC_BITRATE_U_MIN, min(DYNAMIC_BITRATE_U_MAX, prev_u + step))
-        avg_bits, delta = dynamic_bitrate_avg_delta(norms_list, candidate_u, target_avg_bits)
-        if abs(delta) < abs(best_delta):
-            best_u = candidate_u
-            best_avg = avg_bits
-            best_delta = delta
-        if abs(delta) <= DYNAMIC_BITRATE_TOL or old_delta * delta >= 0:
-            return candidate_u, avg_bits, delta
+        u = _clip_u(start + step)
+        avg, delta = dynamic_bitrate_avg_delta(norms_list, u, target_avg_bits)
+        best.offer(u, avg, delta)
+        if abs(delta) <= DYNAMIC_BITRATE_TOL or delta0 * delta >= 0:
+            return u, avg, delta
         step *= 0.5
-    return best_u, best_avg, best_delta
+    return best.triple()
