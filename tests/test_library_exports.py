@@ -66,3 +66,56 @@ def test_module_imports_without_gpu():
     with pytest.raises(RuntimeError, match="src must be a CUDA tensor"):
         eu.superchunk_mean_center(x, x, x, 256, 1)
     eu.init_lookup_table()
+
+
+def test_argument_errors_are_reported_before_any_device_work():
+    """every entry point rejects bad arguments with a status code and a message for the calling thread; these calls
+    return before the first HIP call, so they run without a GPU (the pointers are never dereferenced)"""
+    from dynamiq_sigcomm_artifact_amd import capi
+    L = capi.lib()
+    P = ctypes.c_void_p(0x1000)          # non-null placeholder
+    N = ctypes.c_void_p(0)
+    S = ctypes.c_void_p(0)               # stream
+
+    def err(rc, text):
+        assert rc != 0
+        assert text in L.dq_last_error().decode(), (L.dq_last_error().decode(), text)
+
+    err(L.dq_scaling_compress(P, P, P, 0, 4, 16, 1, 0, 2, S), "n must be positive")
+    err(L.dq_scaling_compress(P, P, P, 256, 9, 16, 1, 0, 2, S), "nbits")
+    err(L.dq_scaling_compress(P, P, P, 256, 4, 16, 7, 0, 2, S), "unsupported element dtype")
+    err(L.dq_scaling_compress(P, P, P, 256, 4, 16, 1 | 0x10, 0, 2, S), "unsupported element dtype")   # bf16 pool flag needs f32
+    err(L.dq_scaling_compress(N, P, P, 256, 4, 16, 1, 0, 2, S), "null pointer")
+    err(L.dq_scaling_decompress(P, N, 256, 4, 16, 1, 0, 2, S, 0), "null pointer")
+    err(L.dq_scaling_decompress(P, P, 250, 4, 16, 1, 0, 0, S, 0), "multiple of chunk_size")
+    err(L.dq_scaling_dec_comp(P, P, P, P, 272, 4, 16, 1, 0, 3, S), "whole number of 16-chunk superchunks")
+    err(L.dq_scaling_compress_philox(P, P, 512, 4, 32, 1, 0, 2, 1, 1, S), "chunk_size 16")
+    err(L.dq_scaling_dec_comp_philox(P, P, N, 256, 4, 16, 1, 0, 2, 1, 1, S), "null pointer")
+    err(L.dq_philox_uniform(P, 0, 1, 0, 1, 1, S), "n must be positive")
+    err(L.dq_superchunk_mean_center(P, P, P, 256, 0, 256, 1, 0, S), "world_size must be positive")
+    err(L.dq_superchunk_mean_center(P, P, P, 256, 2, 128, 1, 0, S), "superchunk_size must be 256")
+    err(L.dq_superchunk_add_mean_copy(P, P, N, 256, 256, 1, 0, S), "null pointer")
+    err(L.dq_hadamard(P, 1000, 0, S, 0), "power of 2")
+    err(L.dq_rht_blocked(P, P, 1024, 48, ctypes.c_float(1.0), 0, 0, S), "block")
+    err(L.dq_rht_blocked(P, P, 1000, 64, ctypes.c_float(1.0), 0, 0, S), "multiple of block")
+    err(L.dq_rand_diag(P, 0, 1, 0, S), "n must be positive")
+    err(L.dq_bins_to_bits(P, 48, P, 6, 4, 0, S), "multiple of 32")
+    err(L.dq_bits_to_bins(P, 64, P, 9, 4, 0, S), "narr")
+    err(L.dq_quantization(N, 16, 0, ctypes.c_float(1.0), ctypes.c_float(1.0), 1, S), "null pointer")
+    err(L.dq_group_plan(P, 0, P, P, 100, 0, S), "nsc")
+    err(L.dq_group_plan(P, 5000, P, P, 8, 0, S), "work buffer is too small")
+    err(L.dq_group_plan_stats(N, ctypes.c_double(1.0), 100, N, P, P, 100, 0, S), "null pointer")
+    err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 0, 0, 2, S), "unsupported element dtype")        # binary16 has no row-list kernels
+    err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 1, 0, 1, S), "strategy")
+    err(L.dq_scaling_dec_comp_rows(P, P, P, P, P, 0, 4, 1, 0, 2, S), "n must be positive")
+    err(L.dq_scaling_decompress_rows(P, P, P, P, 2560, 10, 4, 1, 0, 2, S, 1), "stats cannot be combined")
+    err(L.dq_eden_quantize(P, 100, P, P, 4, P, P, P, 10, 0, S), "multiple of 32")
+    err(L.dq_eden_quantize(P, 8192, P, P, 4, P, P, P, 1, 0, S), "work buffer is too small")
+    err(L.dq_eden_dequantize(P, 64, P, 9, P, 0, S), "nbits")
+    err(L.dq_eden_dequantize(P, 64, P, 4, ctypes.c_void_p(0x1004), 0, S), "16-byte aligned")
+    err(L.dq_thc_quantize(P, P, P, 64, P, P, 1, 0, S), "levels")
+    err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
+    assert capi.group_plan_work_ints(25600) == 4 + 4 * 25 and capi.eden_work_doubles(8192) == 2
+    # a good call clears the message
+    assert L.dq_scaling_check_common(256, 4, 16, 2, 1) == 0 and L.dq_last_error().decode() == ""
+    assert L.dq_status_string(16).decode() == "kernel launch failed"
