@@ -89,6 +89,7 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
     constexpr int L = 1 << NBITS;
     __shared__ double lds[kEdenThreads];
     __shared__ float bnd[L], cen[L];
+    __shared__ uint32_t planes[NBITS][kEdenTile / 32]; // the tile's 128 words of every bit plane
     for (int k = threadIdx.x; k < L; k += kEdenThreads) {
         bnd[k] = k < L - 1 ? boundaries[k] : 0.0f;
         cen[k] = centroids[k];
@@ -101,25 +102,48 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
     const int64_t words = n >> 5;
     const int64_t base = (int64_t)blockIdx.x * kEdenTile;
     const int lane = threadIdx.x & 63;
+    // all sixteen elements of the thread walk the boundary table in lockstep: sixteen independent LDS reads
+    // per search step instead of one dependent chain per element
+    float v[kEdenPerThread], x[kEdenPerThread];
+    int bin[kEdenPerThread];
+#pragma unroll
+    for (int k = 0; k < kEdenPerThread; k++) {
+        const int64_t i = base + threadIdx.x + (int64_t)kEdenThreads * k;
+        v[k] = i < n ? vec[i] : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < kEdenPerThread; k++) {
+        const float scaled = v[k] * sqrt_n;
+        x[k] = ordinary ? div_by(scaled, yn) : scaled / norm;
+        bin[k] = 0;
+    }
+#pragma unroll
+    for (int step = L >> 1; step > 0; step >>= 1) {
+#pragma unroll
+        for (int k = 0; k < kEdenPerThread; k++) {
+            if (bnd[bin[k] + step - 1] < x[k]) bin[k] += step;
+        }
+    }
     double acc = 0.0;
-#pragma unroll 4
+#pragma unroll
     for (int k = 0; k < kEdenPerThread; k++) {
         const int64_t i = base + threadIdx.x + (int64_t)kEdenThreads * k;
         const bool in = i < n;
-        const float v = in ? vec[i] : 0.0f;
-        const float scaled = v * sqrt_n;
-        const float x = ordinary ? div_by(scaled, yn) : scaled / norm;
-        int bin = 0;
-#pragma unroll
-        for (int step = L >> 1; step > 0; step >>= 1) {
-            if (bnd[bin + step - 1] < x) bin += step;
-        }
-        if (in) acc += (double)cen[bin] * (double)v;
-        const int64_t w = i >> 5;
+        if (in) acc += (double)cen[bin[k]] * (double)v[k];
+        const int w = (threadIdx.x >> 5) + 8 * k; // word of the tile
 #pragma unroll
         for (int p = 0; p < NBITS; p++) {
-            const uint64_t m = __ballot(in && ((bin >> p) & 1));
-            if ((lane & 31) == 0 && in) packed[(int64_t)p * words + w] = (uint32_t)(m >> (lane & 32));
+            const uint64_t m = __ballot(in && ((bin[k] >> p) & 1));
+            if ((lane & 31) == 0) planes[p][w] = (uint32_t)(m >> (lane & 32));
+        }
+    }
+    __syncthreads();
+    // 512 contiguous bytes per plane and tile
+    if (threadIdx.x < kEdenTile / 32) {
+        const int64_t w = (base >> 5) + threadIdx.x;
+        if (w < words) {
+#pragma unroll
+            for (int p = 0; p < NBITS; p++) packed[(int64_t)p * words + w] = planes[p][threadIdx.x];
         }
     }
     const double total = fold256(acc, lds);
