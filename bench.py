@@ -13,7 +13,9 @@ Prints ONE JSON line (see the fields below).  `value` is fp32 gradient bytes
 kernel (compress) at its algorithmic bytes (4 + 2 + (q + 0.5625) / 8 per
 element) against the 8 TB/s HBM peak, with the kernel's average launch duration
 measured here with HIP events on the launch stream.  `cpu_baseline` times the
-scalar C oracle (a port of the reference algorithm) on the host, on one core.
+scalar C oracle (a port of the reference algorithm) on the host, on one core;
+`cpu_torch_path` times the same round trip written as torch CPU tensor ops (the
+shape of the reference's own torch implementation) on torch's thread pool.
 """
 import argparse
 import json
@@ -193,6 +195,26 @@ def main():
                           % (m, reps),
             }
 
+    # ---- the same round trip as a torch op sequence on the host cores (shape of the reference's own torch
+    #      implementation, csrc/logic.py:225-296); a second reported baseline beside the scalar port ----
+    cpu_torch = None
+    if args.cpu_seconds > 0 and nbits in (4, 8) and args.src == "fp32":
+        from dynamiq_sigcomm_artifact_amd.evaluate import _torch_cpu_roundtrip
+        xc, rc = src.cpu(), torch.rand(n)
+        _torch_cpu_roundtrip(xc, rc, nbits)
+        ts = []
+        while len(ts) < 9 and sum(ts) < args.cpu_seconds:
+            t1 = time.perf_counter()
+            _torch_cpu_roundtrip(xc, rc, nbits)
+            ts.append(time.perf_counter() - t1)
+        ts.sort()
+        cpu_torch = {
+            "value": round(4.0 * n / ts[len(ts) // 2] / 1e9, 3),
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "sample": "the whole bucket, median of %d round trips of the flat chunk-16 quantiser as torch CPU ops" % len(ts),
+        }
+
     result = {
         "metric": "compress+decompress GB/s (fp32 grad in) on 1 MI355X, % of HBM peak; NMSE",
         "value": round(value, 2),
@@ -238,6 +260,7 @@ def main():
         "bit_exact_vs_oracle": bit_exact,
         "host_wall_ms_per_step": round(wall_ms, 5),
         "cpu_baseline": cpu,
+        "cpu_torch_path": cpu_torch,
     }
     print(json.dumps(result))
 

@@ -26,6 +26,7 @@ HIP_SOURCES = [
     "dq_scaling_hier16.hip",
     "dq_scaling_tile16.hip",
     "dq_grouping.hip",
+    "dq_scaling_mixed.hip",
     "dq_superchunk.hip",
     "dq_hadamard.hip",
     "dq_packing.hip",

@@ -23,6 +23,7 @@ EXPORTS = [
     "dq_scaling_compress_philox", "dq_scaling_dec_comp_philox", "dq_philox_uniform",
     "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
+    "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
@@ -80,6 +81,14 @@ def lib():
         L.dq_scaling_dec_comp_rows.argtypes = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_scaling_decompress_rows.restype = i32
         L.dq_scaling_decompress_rows.argtypes = [vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, vp, i32]
+        L.dq_mixed_required_bytes.restype = i64
+        L.dq_mixed_required_bytes.argtypes = [i64, i32]
+        L.dq_mixed_compress.restype = i32
+        L.dq_mixed_compress.argtypes = [vp, vp, i32, i64, vp, vp, i32, i32, vp, vp, vp, u64, u64, i64, i32, i32, i32, vp]
+        L.dq_mixed_decompress.restype = i32
+        L.dq_mixed_decompress.argtypes = [vp, vp, vp, vp, i32, i32, vp, i64, i64, i32, i32, i32, vp]
+        L.dq_superchunk_stats.restype = i32
+        L.dq_superchunk_stats.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
         L.dq_superchunk_mean_center.restype = i32
         L.dq_superchunk_mean_center.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_superchunk_add_mean_copy.restype = i32
@@ -220,6 +229,33 @@ def scaling_decompress_rows(src, dst, rows, stats, n_limit, nrows, nbits, strate
     _check(lib().dq_scaling_decompress_rows(src.data_ptr(), dst.data_ptr(), _ptr(rows), _ptr(stats), n_limit, nrows,
                                             nbits, dtype_code(dst), _dev(dst), strategy, _stream(stream),
                                             1 if add else 0))
+
+
+def mixed_required_bytes(nsc, ring_world=1):
+    return int(lib().dq_mixed_required_bytes(nsc, ring_world))
+
+
+def mixed_compress(src, order, counts, dst, nsc, strategy, rand_pool=None, seed=0, step=0, recv=None, center_mean=None,
+                   center_world=1, n=0, ring_chunk=0, ring_world=1, stream=None):
+    """all three bit-width groups of the plan (order, counts = work[0:3] of group_plan*) in one launch; recv makes it
+    the ring's fused step; center_mean (float32 per superchunk, from superchunk_stats) centres src on load"""
+    code = dtype_code(src) if rand_pool is None else _pair_code(src, rand_pool)
+    _check(lib().dq_mixed_compress(src.data_ptr(), _ptr(center_mean), center_world, n, order.data_ptr(), counts.data_ptr(),
+                                   ring_chunk, ring_world, _ptr(recv), dst.data_ptr(), _ptr(rand_pool), int(seed), int(step),
+                                   nsc, code, _dev(src), strategy, _stream(stream)))
+
+
+def mixed_decompress(src, dst, order, counts, nsc, strategy, stats=None, n_limit=None, ring_chunk=0, ring_world=1,
+                     stream=None):
+    _check(lib().dq_mixed_decompress(src.data_ptr(), dst.data_ptr(), order.data_ptr(), counts.data_ptr(), ring_chunk,
+                                     ring_world, _ptr(stats), nsc * 256 if n_limit is None else n_limit, nsc,
+                                     dtype_code(dst), _dev(dst), strategy, _stream(stream)))
+
+
+def superchunk_stats(src, stats, mean, n, world_size, stream=None):
+    """the statistics of superchunk_mean_center without the residual; mean (float32 [nsc] or None) gets the unrounded means"""
+    _check(lib().dq_superchunk_stats(src.data_ptr(), stats.data_ptr(), _ptr(mean), n, world_size, dtype_code(src), _dev(src),
+                                     _stream(stream)))
 
 
 def scaling_compress_philox(src, dst, n, nbits, chunk_size, strategy, seed, step, stream=None):

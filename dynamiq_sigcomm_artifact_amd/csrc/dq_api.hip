@@ -358,6 +358,55 @@ int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *row
                                                     mee_params(nbits), add_original, static_cast<hipStream_t>(stream)));
 }
 
+static int check_mixed(int64_t nsc, int ring_chunk, int ring_world, int dtype, int strategy, bool rand)
+{
+    if (!(nsc > 0) || nsc > (int64_t)0x7fffffff) return DQ_ERR_N;
+    if (!(ring_world > 0) || ring_chunk < 0 || ring_chunk >= ring_world) return DQ_ERR_WORLD_SIZE;
+    if (strategy != 2 && strategy != 3) return DQ_ERR_STRATEGY;
+    if (rand ? !dtype_rand_ok(dtype) : !dtype_ok(dtype)) return DQ_ERR_DTYPE;
+    if ((dtype & 0xf) == DQ_F16) return DQ_ERR_DTYPE;
+    return DQ_OK;
+}
+
+int64_t dq_mixed_required_bytes(int64_t nsc, int ring_world)
+{
+    return (nsc > 0 && ring_world > 0) ? dq::mixed_stream_bytes(nsc, ring_world) : 0;
+}
+
+int dq_mixed_compress(const void *src, const float *center_mean, int center_world, int64_t n, const int32_t *order,
+                      const int32_t *counts, int ring_chunk, int ring_world, const uint8_t *recv, uint8_t *dst,
+                      const void *rand_pool, uint64_t seed, uint64_t step, int64_t nsc, int dtype, int device, int strategy,
+                      dq_stream_t stream)
+{
+    int rc = check_mixed(nsc, ring_chunk, ring_world, dtype, strategy, rand_pool != nullptr);
+    if (rc) return fail(rc);
+    if (!src || !order || !counts || !dst) return fail(DQ_ERR_NULL);
+    if (center_mean) {
+        if (!(center_world > 0)) return fail(DQ_ERR_WORLD_SIZE);
+        if (!(n > 0) || (n + 255) / 256 > nsc) return fail(DQ_ERR_N, "n must lie in [1, 256 * nsc]");
+    }
+    if ((rc = select_device(device))) return rc;
+    const dq::MeeParams mp[3] = {mee_params(8), mee_params(4), mee_params(2)};
+    const dq::RandKey key{seed, step};
+    return finish(dq::launch_mixed_compress(src, center_mean, center_mean ? center_world : 1, n, order, counts, ring_chunk,
+                                            ring_world, recv, dst, rand_pool, rand_pool ? nullptr : &key, nsc, dtype,
+                                            strategy == 3, mp, static_cast<hipStream_t>(stream)));
+}
+
+int dq_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, const int32_t *counts, int ring_chunk,
+                        int ring_world, const void *stats, int64_t n_limit, int64_t nsc, int dtype, int device,
+                        int strategy, dq_stream_t stream)
+{
+    int rc = check_mixed(nsc, ring_chunk, ring_world, dtype, strategy, false);
+    if (rc) return fail(rc);
+    if (!src || !dst || !order || !counts) return fail(DQ_ERR_NULL);
+    if (!(n_limit > 0)) return fail(DQ_ERR_N, "n_limit");
+    if ((rc = select_device(device))) return rc;
+    const dq::MeeParams mp[3] = {mee_params(8), mee_params(4), mee_params(2)};
+    return finish(dq::launch_mixed_decompress(src, dst, order, counts, ring_chunk, ring_world, stats, n_limit, nsc, dtype,
+                                              strategy == 3, mp, static_cast<hipStream_t>(stream)));
+}
+
 int dq_scaling_compress_philox(const void *src, uint8_t *dst, int64_t n, int nbits, int chunk_size, int dtype, int device,
                                int strategy, uint64_t seed, uint64_t step, dq_stream_t stream)
 {
@@ -414,7 +463,19 @@ int dq_superchunk_mean_center(const void *src, void *residual, void *stats, int6
     if (!src || !residual || !stats) return fail(DQ_ERR_NULL);
     int rc;
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_mean_center(src, residual, stats, n, world_size, dtype, static_cast<hipStream_t>(stream)));
+    return finish(dq::launch_mean_center(src, residual, stats, nullptr, n, world_size, dtype, static_cast<hipStream_t>(stream)));
+}
+
+int dq_superchunk_stats(const void *src, void *stats, float *mean, int64_t n, int world_size, int dtype, int device,
+                        dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (!(world_size > 0)) return fail(DQ_ERR_WORLD_SIZE);
+    if (!dtype_ok(dtype)) return fail(DQ_ERR_DTYPE);
+    if (!src || !stats) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_mean_center(src, nullptr, stats, mean, n, world_size, dtype, static_cast<hipStream_t>(stream)));
 }
 
 int dq_superchunk_add_mean_copy(const void *residual, void *dst, const void *stats, int64_t n, int superchunk_size,

@@ -282,4 +282,14 @@ __host__ __device__ __forceinline__ void chunk_uniform_words(const RandKey &key,
     philox4x32_10(w, (uint32_t)key.seed, (uint32_t)(key.seed >> 32));
 }
 
+// v / world, correctly rounded: world = 2^k multiplies by the exact reciprocal; otherwise the product with
+// the double reciprocal is within 2^-51 of the quotient, closer than a quotient of two binary32 numbers
+// can come to a rounding boundary without lying on it
+struct WorldDiv {
+    float inv;
+    double inv_d;
+    int pow2;
+    __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
+};
+
 } // namespace dq

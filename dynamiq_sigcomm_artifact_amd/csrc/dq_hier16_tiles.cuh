@@ -1,0 +1,326 @@
+// Tile bodies of the hierarchical chunk-16 kernels: the work of one wave on one tile of four
+// superchunks, shared by the single-width kernels (dq_scaling_hier16.hip) and the kernels that
+// serve all bit-width groups of a bucket in one launch (dq_scaling_mixed.hip).
+//
+// Numerics: csrc/cuda_hierarchical_mee.cu:203-343 (compress), 345-505 (decompress) and 526-696
+// (fused decompress-accumulate-recompress).
+#pragma once
+
+#include "dq_tile16.cuh"
+
+namespace dq {
+
+// ---- the math of one chunk ---------------------------------------------------------------------
+
+// decode 16 levels of one chunk: t = lev*sc (+ t when ADD)
+template <int NBITS, bool MEE, bool ADD>
+__device__ __forceinline__ void chunk_decode(const uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t q, uint32_t unit_bits,
+                                             const float *table, float (&t)[16])
+{
+    const float us = nonneg_scale(bf16_bits_to_f32(unit_bits));
+    const float sc = nonneg_scale((float)q * us);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const uint32_t code = words_get<NBITS>(w, i);
+        const float lev = MEE ? table[code] : (float)((int)code - Rec<NBITS>::R);
+        t[i] = ADD ? __builtin_fmaf(lev, sc, t[i]) : lev * sc;
+    }
+}
+
+// general (guarded) quantiser of one chunk against its superchunk row
+template <int NBITS, bool MEE, class RV, class RR, class ARG>
+__device__ __forceinline__ void chunk_encode_guarded(const RV &v, const RR &r, const ARG &mp,
+                                                     uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q, uint32_t &unit_bits)
+{
+    constexpr int R = Rec<NBITS>::R;
+    float a = __builtin_fabsf(v.get(0));
+#pragma unroll
+    for (int i = 1; i < 16; i++) a = __builtin_fmaxf(a, __builtin_fabsf(v.get(i)));
+    const float s = pos_scale(MEE ? a / pos_scale(mp.cmm) + 1e-7f : a / (float)R + 1e-7f);
+    const float g = pos_scale(row16_max(s));
+    unit_bits = f32_to_bf16_bits(pos_scale(g / 255.0f));
+    const float unit = pos_scale(bf16_bits_to_f32(unit_bits));
+    float ratio = pos_scale(s) / pos_scale(g) * 255.0f;
+    if (!__builtin_isfinite(ratio)) ratio = ratio > 0.0f ? 255.0f : 1.0f;
+    int qi = sat_u16(__builtin_ceilf(ratio));
+    qi = min(max(qi, 1), 255);
+    q = (uint32_t)qi;
+    const float d = pos_scale(pos_scale((float)qi * unit));
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float x = v.get(i) / d;
+        if (MEE) x = mee_inverse_guarded(x, mp.c, mp.l2b);
+        words_put<NBITS>(w, i, (uint32_t)clamp_code(sr_guarded(x, r.get(i)), R));
+    }
+}
+
+// the same quantiser for a wave whose elements are all finite and <= 2^100 in
+// magnitude (amax_bits is the integer-order maximum of |v|) and whose random
+// values all lie in [0, 1]: none of the guards can fire
+template <int NBITS, bool MEE, class RV, class RR, class ARG>
+__device__ __forceinline__ void chunk_encode_fast(const RV &v, const RR &r, uint32_t amax_bits, const ARG &mp,
+                                                  uint32_t (&w)[Rec<NBITS>::WORDS], uint32_t &q, uint32_t &unit_bits)
+{
+    constexpr int R = Rec<NBITS>::R;
+    const float a = __uint_as_float(amax_bits);
+    float s;
+    if (MEE)
+        s = div_by(a, mp.inv_cmm) + 1e-7f;
+    else
+        s = (R == 1 ? a : div_by(a, 1.0 / (double)R)) + 1e-7f; // >= 1e-7, finite
+    const float g = row16_max(s);
+    unit_bits = f32_to_bf16_bits(div_by(g, 1.0 / 255.0));
+    const float unit = bf16_bits_to_f32(unit_bits);
+    const float ratio = div_by(s, recip_f64(g)) * 255.0f;
+    int qi = (int)__builtin_ceilf(ratio);
+    qi = min(max(qi, 1), 255);
+    q = (uint32_t)qi;
+    const float d = (float)qi * unit; // exact: 8 x 8 significant bits
+    const double yd = recip_f64(d);
+#pragma unroll
+    for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float x = div_by(v.get(i), yd);
+        if (MEE) {
+            const float arg = div_by(__builtin_fabsf(x), mp.inv_c) + 1.0f;
+            const float lat = div_by(log2_det_ge1(arg), mp.inv_l2b);
+            x = __builtin_copysignf(lat, x);
+        }
+        const float fl = __builtin_floorf(x);
+        const float c = __builtin_ceilf((x - fl) - r.get(i));
+        const int sv = (int)(fl + c); // |fl| <= R + 1 and c in {-1, 0, 1}: exact
+        words_put<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
+    }
+}
+
+constexpr uint32_t kFastMaxBits = 0x71800000u; // 2^100
+
+
+// Mean-centring applied to the source elements as they are loaded (csrc/cuda_hadamard.cu:1304-1349):
+// element e of superchunk b becomes T(f32(src[e]) / world - mean[b]) with mean in binary32, zero at and
+// beyond n_valid.  mean == nullptr switches it off.
+struct Center {
+    const float *mean;
+    int64_t n_valid;
+    WorldDiv wd;
+};
+
+template <int DT>
+__device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int64_t e0, const Center &ctr, int64_t sc_src,
+                                             bool vec)
+{
+    float t[16];
+    const float mean = ctr.mean[sc_src];
+    if (e0 + 16 <= ctr.n_valid) {
+        v.load(src, e0, vec);
+#pragma unroll
+        for (int i = 0; i < 16; i++) t[i] = ctr.wd(v.get(i)) - mean;
+    } else {
+        // the ragged end of the vector: nothing at or beyond n_valid is read
+#pragma unroll
+        for (int i = 0; i < 16; i++) t[i] = e0 + i < ctr.n_valid ? ctr.wd(ElemIO<DT>::load(src, e0 + i)) - mean : 0.0f;
+    }
+    v.set(t);
+}
+
+// compress (FUSED = false) or decode-accumulate-recompress (FUSED = true) of tile `tile` of a run of nsc
+// records.  Record k of the packed streams (and row k of rnd) belongs to superchunk rows[k] of src
+// (to superchunk k when rows is null).  win_out / win_in: Rec<NBITS>::WIN bytes of LDS each, 16-byte
+// aligned (win_in only when FUSED); table: 2^NBITS floats of LDS (only when MEE && FUSED).
+template <int DT, int RDT, int NBITS, bool MEE, bool FUSED>
+__device__ __forceinline__ void compress_tile(const void *__restrict__ src, const uint8_t *__restrict__ recv,
+                                              uint8_t *__restrict__ dst, const void *__restrict__ rnd,
+                                              const int32_t *__restrict__ rows, int64_t nsc, int64_t tile, int vec,
+                                              const RandKey &key, const Center &ctr, const MeeArg<NBITS, MEE> &mp,
+                                              uint8_t *win_out, uint8_t *win_in, float *table)
+{
+    typedef Rec<NBITS> RC;
+    const int lane = threadIdx.x;
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t sc0 = tile * kRowsPerWave;
+    if (sc0 >= nsc) return;
+    const int rows_here = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+    const bool active = row < rows_here;
+    const int total = rows_here * RC::REC;
+
+    // all global loads of the tile are issued before anything waits on them
+    Raw16<DT> v;
+    Raw16<RDT> r;
+    if (active) {
+        if constexpr (RDT != DQ_PHILOX) r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
+        const int64_t sc_src = rows ? (int64_t)rows[sc0 + row] : sc0 + row;
+        if constexpr (RDT == DQ_PHILOX) r.generate(key, sc_src * 16 + j); // keyed by the chunk's place in the source vector
+        if (ctr.mean)
+            center_chunk<DT>(v, src, (sc_src * 16 + j) * 16, ctr, sc_src, vec & 1);
+        else
+            v.load(src, (sc_src * 16 + j) * 16, vec & 1);
+    } else {
+        v.zero();
+        r.zero();
+    }
+    WinRegs wr;
+    if (FUSED) wr = window_fetch(recv + sc0 * RC::REC, total, lane);
+    if (MEE && FUSED) {
+        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
+    }
+
+    if (FUSED) {
+        const int mis_in = window_commit(win_in, wr, recv + sc0 * RC::REC, total, lane);
+        wave_lds_sync();
+        if (active) {
+            const uint8_t *rec = win_in + mis_in + row * RC::REC;
+            uint32_t cw[RC::WORDS], cq;
+            chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+            const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+            float t[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = v.get(i);
+            chunk_decode<NBITS, MEE, true>(cw, cq, ub, table, t);
+            v.set(t); // rounds the sum to the element type
+        }
+    }
+
+    uint32_t w[RC::WORDS], q, ub;
+    const uint32_t amax = v.absmax_bits();
+    const bool lane_fast = amax <= kFastMaxBits && r.unit_interval();
+    if (__builtin_amdgcn_ballot_w64(!lane_fast) == 0)
+        chunk_encode_fast<NBITS, MEE>(v, r, amax, mp, w, q, ub);
+    else
+        chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
+
+    uint8_t *gout = dst + sc0 * RC::REC;
+    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
+    if (active) {
+        uint8_t *rec = win_out + mis + row * RC::REC;
+        chunk_write<NBITS>(rec + j * RC::CB, w, q);
+        if (j == 0) {
+            rec[16 * RC::CB] = (uint8_t)ub;
+            rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+        }
+    }
+    wave_lds_sync();
+    window_flush(win_out, gout, mis, total, lane);
+}
+
+// Tile `tile` of a run of nsc records: record k decodes into superchunk rows[k] of dst (superchunk k when
+// rows is null).  With stats (interleaved bf16 pairs, the mean first) the stored value is
+// T(float(T(decoded)) + mean of the destination superchunk); elements at or beyond `limit` are not
+// written.  win_in: Rec<NBITS>::WIN bytes of LDS, 16-byte aligned; tile_out: 64 * Raw16<DT>::kSlots
+// 16-byte slots of LDS; table: 2^NBITS floats of LDS (only when MEE).
+template <int DT, int NBITS, bool MEE, bool ADD>
+__device__ __forceinline__ void decompress_tile(const uint8_t *__restrict__ src, void *__restrict__ dst,
+                                                const int32_t *__restrict__ rows, const uint16_t *__restrict__ stats,
+                                                int64_t limit, int64_t nsc, int64_t tile, int vec,
+                                                const MeeArg<NBITS, MEE> &mp, uint8_t *win_in, uint4 *tile_out, float *table)
+{
+    typedef Rec<NBITS> RC;
+    constexpr int S = Raw16<DT>::kSlots;
+    constexpr int ESZ = DT == DQ_F32 ? 4 : 2;
+    constexpr int EP = 16 / ESZ; // elements per 16-byte slot
+
+    const int lane = threadIdx.x;
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t sc0 = tile * kRowsPerWave;
+    if (sc0 >= nsc) return;
+    const int rows_here = (int)min((int64_t)kRowsPerWave, nsc - sc0);
+    const bool active = row < rows_here;
+    const int total = rows_here * RC::REC;
+
+    const WinRegs wr = window_fetch(src + sc0 * RC::REC, total, lane);
+    // destination superchunk of this lane's chunk, and of the slots this lane stores after the transpose
+    int64_t d_own = sc0 + row;
+    int64_t d_slot[S];
+#pragma unroll
+    for (int k = 0; k < S; k++) d_slot[k] = sc0 + (64 * k + lane) / (16 * S);
+    if (rows) {
+        if (active) d_own = rows[sc0 + row];
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const int rr = (64 * k + lane) / (16 * S);
+            if (rr < rows_here) d_slot[k] = rows[sc0 + rr];
+        }
+    }
+    Raw16<DT> acc;
+    if (ADD && active) acc.load(dst, d_own * 256 + j * 16, vec);
+    float mean = 0.0f;
+    if (stats && active) mean = bf16_bits_to_f32(stats[2 * d_own]);
+    if (MEE) {
+        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
+    }
+
+    const int mis_in = window_commit(win_in, wr, src + sc0 * RC::REC, total, lane);
+    wave_lds_sync();
+    Raw16<DT> out;
+    if (active) {
+        const uint8_t *rec = win_in + mis_in + row * RC::REC;
+        uint32_t cw[RC::WORDS], cq;
+        chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+        const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+        float t[16];
+        if (ADD) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = acc.get(i);
+        }
+        chunk_decode<NBITS, MEE, ADD>(cw, cq, ub, table, t);
+        out.set(t);
+        if (stats) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = out.get(i) + mean;
+            out.set(t);
+        }
+    } else {
+        out.zero();
+    }
+    char *dbytes = static_cast<char *>(dst);
+    if (vec) {
+        // transpose through LDS so that every store instruction writes whole superchunks contiguously
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < S; k++) tile_out[swz(S * lane + k)] = out.slot(k);
+        }
+        wave_lds_sync();
+        const int nslots = rows_here * 16 * S;
+#pragma unroll
+        for (int k = 0; k < S; k++) {
+            const int s = 64 * k + lane;
+            if (s < nslots) {
+                const int64_t e = d_slot[k] * 256 + (s % (16 * S)) * EP;
+                const uint4 val = tile_out[swz(s)];
+                if (e + EP <= limit) {
+                    *reinterpret_cast<uint4 *>(dbytes + e * ESZ) = val;
+                } else {
+                    const uint32_t part[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+                    for (int i = 0; i < EP; i++) {
+                        if (e + i < limit) {
+                            if (DT == DQ_F32)
+                                reinterpret_cast<uint32_t *>(dbytes)[e + i] = part[i];
+                            else
+                                reinterpret_cast<uint16_t *>(dbytes)[e + i] = (uint16_t)(part[i >> 1] >> (16 * (i & 1)));
+                        }
+                    }
+                }
+            }
+        }
+    } else if (active) {
+        const int64_t e = d_own * 256 + j * 16;
+        if (e + 16 <= limit) {
+            out.store(dst, e, false);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                if (e + i < limit) {
+                    if (DT == DQ_F32)
+                        reinterpret_cast<uint32_t *>(dbytes)[e + i] = out.w[i];
+                    else
+                        reinterpret_cast<uint16_t *>(dbytes)[e + i] = (uint16_t)(out.w[i >> 1] >> (16 * (i & 1)));
+                }
+            }
+        }
+    }
+}
+
+} // namespace dq

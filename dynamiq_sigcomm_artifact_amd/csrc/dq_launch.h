@@ -64,8 +64,20 @@ hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, 
 hipError_t launch_group_plan_stats(const void *stats, float u, int64_t nsc, int64_t *qbits_out,
                                    int32_t *order, int32_t *work, hipStream_t stream);
 
+// all bit-width groups of a planned bucket in one launch (dq_scaling_mixed.hip); mp: the MEE
+// parameters of 8, 4 and 2 bits in this order
+int64_t mixed_stream_bytes(int64_t nsc, int world);
+hipError_t launch_mixed_compress(const void *src, const float *center_mean, int center_world, int64_t n_valid,
+                                 const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world,
+                                 const uint8_t *recv, uint8_t *dst, const void *rnd, const RandKey *philox,
+                                 int64_t nsc, int dtype, bool mee, const MeeParams *mp, hipStream_t stream);
+hipError_t launch_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, const int32_t *counts,
+                                   int ring_chunk, int ring_world, const void *stats, int64_t limit, int64_t nsc,
+                                   int dtype, bool mee, const MeeParams *mp, hipStream_t stream);
+
 // superchunk mean-centring (dq_superchunk.hip)
-hipError_t launch_mean_center(const void *src, void *residual, void *stats, int64_t n,
+// residual == nullptr: statistics only; mean_out (nullable) receives the binary32 means
+hipError_t launch_mean_center(const void *src, void *residual, void *stats, float *mean_out, int64_t n,
                               int world_size, int dtype, hipStream_t stream);
 hipError_t launch_add_mean_copy(const void *residual, void *dst, const void *stats, int64_t n,
                                 int dtype, hipStream_t stream);

@@ -1,0 +1,201 @@
+// All bit-width groups of a bucket in one launch.
+//
+// The reference's dynamic-bitrate all-reduce splits a bucket's superchunks into the groups that got 8, 4
+// and 2 bits, gathers each group into a tensor of its own and runs the ring three times
+// (testbed_evaluation/new_comm_hooks/comm_hooks.py:963-1018).  Here one launch serves the three groups:
+// the partition (`order`, group sizes `counts`, written by the plan kernels of dq_grouping.hip) stays in
+// device memory, every workgroup works out from the three counts which group and which tile of it it
+// owns, and runs the tile body of that width.  The host never learns the group sizes, so the whole
+// bucket pipeline is a fixed sequence of launches without a read-back (and can be replayed as a graph).
+//
+// Ring chunk c of `world` (the reference's split of a group into world pieces of whole superchunks,
+// ceil(n_g / world) each) is served as one stream of records:
+//     [8-bit records of chunk c | 4-bit records of chunk c | 2-bit records of chunk c]
+// The record formats are those of the single-width kernels, so each of the three runs is byte for byte
+// what dq_scaling_compress_rows writes for the same superchunks and random values.
+//
+// Rounding randomness: row k of rand_pool (256 values) belongs to position k of `order`; the in-kernel
+// stream is keyed by the chunk's index in the source vector.
+#include "dq_hier16_tiles.cuh"
+#include "dq_launch.h"
+
+namespace dq {
+
+namespace {
+
+struct MixedPlan {
+    const int32_t *order;  // superchunk indices, grouped 8 | 4 | 2
+    const int32_t *counts; // n8, n4, n2
+    int chunk, world;
+};
+
+struct Segment {
+    int cls;          // 0: 8-bit, 1: 4-bit, 2: 2-bit, 3: nothing to do
+    int tile;         // tile inside the run
+    int cnt;          // records in the run
+    int64_t pos0;     // position in `order` of the run's first record
+    int64_t byte_off; // where the run starts in the packed stream
+};
+
+__device__ __forceinline__ Segment locate(const MixedPlan &p, int block)
+{
+    constexpr int kRec[3] = {Rec<8>::REC, Rec<4>::REC, Rec<2>::REC};
+    Segment s;
+    s.cls = 3; s.tile = 0; s.cnt = 0; s.pos0 = 0; s.byte_off = 0;
+    int64_t pos = 0, off = 0;
+    int t = block;
+#pragma unroll
+    for (int g = 0; g < 3; g++) {
+        const int n = p.counts[g];
+        const int per = (n + p.world - 1) / p.world;
+        const int begin = (int)min((int64_t)per * p.chunk, (int64_t)n);
+        const int cnt = min(per, n - begin);
+        const int tiles = (cnt + kRowsPerWave - 1) / kRowsPerWave;
+        if (s.cls == 3 && t < tiles) {
+            s.cls = g; s.tile = t; s.cnt = cnt; s.pos0 = pos + begin; s.byte_off = off;
+        }
+        t -= tiles;
+        pos += n;
+        off += (int64_t)cnt * kRec[g];
+    }
+    return s;
+}
+
+template <int DT, int RDT, bool MEE, bool FUSED>
+__global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restrict__ src, const uint8_t *__restrict__ recv,
+                                                           uint8_t *__restrict__ dst, const void *__restrict__ rnd,
+                                                           MixedPlan plan, int vec, RandKey key, Center ctr,
+                                                           MeeArg<8, MEE> m8, MeeArg<4, MEE> m4, MeeArg<2, MEE> m2)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t win_out[Rec<8>::WIN];
+    __shared__ __attribute__((aligned(16))) uint8_t win_in[FUSED ? Rec<8>::WIN : 16];
+    __shared__ float table[(MEE && FUSED) ? 256 : 1];
+    constexpr int RESZ = RDT == DQ_F32 ? 4 : 2;
+
+    const Segment s = locate(plan, blockIdx.x);
+    if (s.cls == 3) return;
+    const int32_t *rows = plan.order + s.pos0;
+    const void *r = RDT == DQ_PHILOX ? nullptr : static_cast<const char *>(rnd) + s.pos0 * 256 * RESZ;
+    const uint8_t *in = FUSED ? recv + s.byte_off : nullptr;
+    uint8_t *out = dst + s.byte_off;
+    switch (s.cls) {
+    case 0:
+        compress_tile<DT, RDT, 8, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m8, win_out, win_in, table);
+        break;
+    case 1:
+        compress_tile<DT, RDT, 4, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m4, win_out, win_in, table);
+        break;
+    default:
+        compress_tile<DT, RDT, 2, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m2, win_out, win_in, table);
+        break;
+    }
+}
+
+template <int DT, bool MEE>
+__global__ __launch_bounds__(64) void mixed_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
+                                                             MixedPlan plan, const uint16_t *__restrict__ stats,
+                                                             int64_t limit, int vec, MeeArg<8, MEE> m8, MeeArg<4, MEE> m4,
+                                                             MeeArg<2, MEE> m2)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t win_in[Rec<8>::WIN];
+    __shared__ __attribute__((aligned(16))) uint4 tile_out[64 * Raw16<DT>::kSlots];
+    __shared__ float table[MEE ? 256 : 1];
+
+    const Segment s = locate(plan, blockIdx.x);
+    if (s.cls == 3) return;
+    const int32_t *rows = plan.order + s.pos0;
+    const uint8_t *in = src + s.byte_off;
+    switch (s.cls) {
+    case 0:
+        decompress_tile<DT, 8, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile, vec, m8, win_in, tile_out, table);
+        break;
+    case 1:
+        decompress_tile<DT, 4, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile, vec, m4, win_in, tile_out, table);
+        break;
+    default:
+        decompress_tile<DT, 2, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile, vec, m2, win_in, tile_out, table);
+        break;
+    }
+}
+
+// every group rounds its share of a ring chunk up to whole superchunks and its superchunks up to whole
+// tiles: at most nsc / world + 3 records and nsc / (4 world) + 3 tiles
+inline unsigned grid_for(int64_t nsc, int world) { return (unsigned)(nsc / ((int64_t)kRowsPerWave * world) + 4); }
+
+template <int DT, int RDT, bool MEE>
+hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, const MixedPlan &plan,
+                        int64_t nsc, const Center &ctr, const RandKey &key, const MeeParams *mp, hipStream_t stream)
+{
+    const auto m8 = make_arg<8, MEE>(mp[0]);
+    const auto m4 = make_arg<4, MEE>(mp[1]);
+    const auto m2 = make_arg<2, MEE>(mp[2]);
+    dim3 grid(grid_for(nsc, plan.world)), block(64);
+    const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
+    if (recv)
+        hipLaunchKernelGGL((mixed_compress_kernel<DT, RDT, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, plan, vec,
+                           key, ctr, m8, m4, m2);
+    else
+        hipLaunchKernelGGL((mixed_compress_kernel<DT, RDT, MEE, false>), grid, block, 0, stream, src, recv, dst, rnd, plan, vec,
+                           key, ctr, m8, m4, m2);
+    return hipGetLastError();
+}
+
+template <int DT, bool MEE>
+hipError_t run_decompress(const uint8_t *src, void *dst, const MixedPlan &plan, int64_t nsc, const uint16_t *stats,
+                          int64_t limit, const MeeParams *mp, hipStream_t stream)
+{
+    const auto m8 = make_arg<8, MEE>(mp[0]);
+    const auto m4 = make_arg<4, MEE>(mp[1]);
+    const auto m2 = make_arg<2, MEE>(mp[2]);
+    hipLaunchKernelGGL((mixed_decompress_kernel<DT, MEE>), dim3(grid_for(nsc, plan.world)), dim3(64), 0, stream, src, dst, plan,
+                       stats, limit, aligned16(dst) ? 1 : 0, m8, m4, m2);
+    return hipGetLastError();
+}
+
+} // namespace
+
+int64_t mixed_stream_bytes(int64_t nsc, int world) { return (nsc / world + 3) * Rec<8>::REC; }
+
+// mp: the MEE parameters of 8, 4 and 2 bits, in this order
+hipError_t launch_mixed_compress(const void *src, const float *center_mean, int center_world, int64_t n_valid,
+                                 const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world,
+                                 const uint8_t *recv, uint8_t *dst, const void *rnd, const RandKey *philox, int64_t nsc,
+                                 int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
+{
+    const MixedPlan plan{order, counts, ring_chunk, ring_world};
+    Center ctr;
+    ctr.mean = center_mean;
+    ctr.n_valid = n_valid;
+    ctr.wd.inv = 1.0f / (float)center_world;
+    ctr.wd.inv_d = 1.0 / (double)center_world;
+    ctr.wd.pow2 = (center_world & (center_world - 1)) == 0;
+    const RandKey key = philox ? *philox : RandKey{0, 0};
+    const bool rb16 = (dtype & DQ_RAND_BF16) != 0;
+    dtype &= 0xf;
+#define DQ_MIXED(DT, RDT)                                                                                              \
+    return mee ? run_compress<DT, RDT, true>(src, recv, dst, rnd, plan, nsc, ctr, key, mp, stream)                     \
+               : run_compress<DT, RDT, false>(src, recv, dst, rnd, plan, nsc, ctr, key, mp, stream)
+    if (dtype == DQ_BF16) {
+        if (philox) { DQ_MIXED(DQ_BF16, DQ_PHILOX); }
+        DQ_MIXED(DQ_BF16, DQ_BF16);
+    }
+    if (philox) { DQ_MIXED(DQ_F32, DQ_PHILOX); }
+    if (rb16) { DQ_MIXED(DQ_F32, DQ_BF16); }
+    DQ_MIXED(DQ_F32, DQ_F32);
+#undef DQ_MIXED
+}
+
+hipError_t launch_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, const int32_t *counts,
+                                   int ring_chunk, int ring_world, const void *stats, int64_t limit, int64_t nsc,
+                                   int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
+{
+    const MixedPlan plan{order, counts, ring_chunk, ring_world};
+    const uint16_t *st = static_cast<const uint16_t *>(stats);
+    if ((dtype & 0xf) == DQ_BF16)
+        return mee ? run_decompress<DQ_BF16, true>(src, dst, plan, nsc, st, limit, mp, stream)
+                   : run_decompress<DQ_BF16, false>(src, dst, plan, nsc, st, limit, mp, stream);
+    return mee ? run_decompress<DQ_F32, true>(src, dst, plan, nsc, st, limit, mp, stream)
+               : run_decompress<DQ_F32, false>(src, dst, plan, nsc, st, limit, mp, stream);
+}
+
+} // namespace dq

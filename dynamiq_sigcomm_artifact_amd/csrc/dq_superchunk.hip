@@ -36,19 +36,10 @@ __device__ __forceinline__ void wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// v / world, correctly rounded: world = 2^k multiplies by the exact reciprocal; otherwise the product with
-// the double reciprocal is within 2^-51 of the quotient, closer than a quotient of two binary32 numbers
-// can come to a rounding boundary without lying on it
-struct WorldDiv {
-    float inv;
-    double inv_d;
-    int pow2;
-    __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
-};
-
 template <int DT>
 __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__restrict__ src, void *__restrict__ residual,
-                                                             uint32_t *__restrict__ stats, int64_t nsc, WorldDiv wd)
+                                                             uint32_t *__restrict__ stats, float *__restrict__ mean_out,
+                                                             int64_t nsc, WorldDiv wd)
 {
     constexpr int ESZ = DT == DQ_F32 ? 4 : 2;
     constexpr int SPR = 16 * ESZ;            // 16-byte slots per superchunk
@@ -123,6 +114,11 @@ __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__rest
     sum += dpp_shift<0x101>(sum);
     sq += dpp_shift<0x101>(sq);
     const float mean = __shfl(sum, lane & 48, 64) * 0.00390625f; // / 256, exact
+    if (row < rows_here && j == 0) {
+        stats[sc0 + row] = f32_to_bf16_bits(mean) | (f32_to_bf16_bits(sq) << 16);
+        if (mean_out) mean_out[sc0 + row] = mean;
+    }
+    if (!residual) return; // statistics only
     if (row < rows_here) {
 #pragma unroll
         for (int k = 0; k < 16; k++) {
@@ -134,7 +130,6 @@ __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__rest
             else
                 *reinterpret_cast<uint16_t *>(mine + 16 * k * ESZ) = (uint16_t)f32_to_f16_bits(r);
         }
-        if (j == 0) stats[sc0 + row] = f32_to_bf16_bits(mean) | (f32_to_bf16_bits(sq) << 16);
     }
     wave_lds_sync();
     if (lane < nslots) gout[lane] = *DQ_SLOT_PTR(lane);
@@ -148,8 +143,8 @@ __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__rest
 
 template <int DT>
 __global__ __launch_bounds__(256) void mean_center_kernel(const void *__restrict__ src, void *__restrict__ residual,
-                                                          uint16_t *__restrict__ stats, int64_t n, int64_t sc_begin,
-                                                          int64_t nsc, float world)
+                                                          uint16_t *__restrict__ stats, float *__restrict__ mean_out,
+                                                          int64_t n, int64_t sc_begin, int64_t nsc, float world)
 {
     typedef ElemIO<DT> IO;
     const int lane = threadIdx.x & 63;
@@ -183,14 +178,17 @@ __global__ __launch_bounds__(256) void mean_center_kernel(const void *__restrict
     sq += dpp_shift<0x101>(sq);
     const float total = __shfl(sum, 0, 64);
     const float mean = valid > 0 ? total / (float)valid : 0.0f;
+    if (residual) {
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const int l = lane + 64 * k;
-        IO::store(residual, start + l, (l < valid) ? v[k] - mean : 0.0f);
+        for (int k = 0; k < 4; k++) {
+            const int l = lane + 64 * k;
+            IO::store(residual, start + l, (l < valid) ? v[k] - mean : 0.0f);
+        }
     }
     if (lane == 0) {
         stats[2 * sc] = (uint16_t)f32_to_bf16_bits(mean);
         stats[2 * sc + 1] = (uint16_t)f32_to_bf16_bits(sq);
+        if (mean_out) mean_out[sc] = mean;
     }
 }
 
@@ -234,8 +232,8 @@ __global__ __launch_bounds__(256) void add_mean_copy_vec_kernel(const uint4 *__r
 }
 
 template <int DT>
-static hipError_t run_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size,
-                                  hipStream_t stream)
+static hipError_t run_mean_center(const void *src, void *residual, void *stats, float *mean_out, int64_t n,
+                                  int world_size, hipStream_t stream)
 {
     const int64_t nsc = (n + 255) / 256;
     int64_t done = 0;
@@ -248,22 +246,23 @@ static hipError_t run_mean_center(const void *src, void *residual, void *stats, 
         wd.inv_d = 1.0 / (double)world_size;
         wd.pow2 = (world_size & (world_size - 1)) == 0;
         hipLaunchKernelGGL(mean_center_tile_kernel<DT>, dim3((unsigned)((done + 3) / 4)), dim3(64), 0, stream, src, residual,
-                           static_cast<uint32_t *>(stats), done, wd);
+                           static_cast<uint32_t *>(stats), mean_out, done, wd);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess || done == nsc) return e;
     }
     hipLaunchKernelGGL(mean_center_kernel<DT>, dim3((unsigned)((nsc - done + 3) / 4)), dim3(256), 0, stream, src, residual,
-                       static_cast<uint16_t *>(stats), n, done, nsc, (float)world_size);
+                       static_cast<uint16_t *>(stats), mean_out, n, done, nsc, (float)world_size);
     return hipGetLastError();
 }
 
-hipError_t launch_mean_center(const void *src, void *residual, void *stats, int64_t n, int world_size, int dtype,
-                              hipStream_t stream)
+// residual == nullptr: statistics only; mean_out (nullable) receives the binary32 means
+hipError_t launch_mean_center(const void *src, void *residual, void *stats, float *mean_out, int64_t n, int world_size,
+                              int dtype, hipStream_t stream)
 {
     switch (dtype) {
-    case DQ_F16: return run_mean_center<DQ_F16>(src, residual, stats, n, world_size, stream);
-    case DQ_BF16: return run_mean_center<DQ_BF16>(src, residual, stats, n, world_size, stream);
-    default: return run_mean_center<DQ_F32>(src, residual, stats, n, world_size, stream);
+    case DQ_F16: return run_mean_center<DQ_F16>(src, residual, stats, mean_out, n, world_size, stream);
+    case DQ_BF16: return run_mean_center<DQ_BF16>(src, residual, stats, mean_out, n, world_size, stream);
+    default: return run_mean_center<DQ_F32>(src, residual, stats, mean_out, n, world_size, stream);
     }
 }
 

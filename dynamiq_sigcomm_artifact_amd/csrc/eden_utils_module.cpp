@@ -384,6 +384,120 @@ void scaling_decompress_rows(torch::Tensor src, torch::Tensor dst, torch::Tensor
                  "scaling_decompress_rows");
 }
 
+// ---- all bit-width groups of a planned bucket in one launch ---------------------------------
+
+int64_t mixed_required_bytes(int64_t nsc, int ring_world = 1) { return dq_mixed_required_bytes(nsc, ring_world); }
+
+static void check_plan_tensors(const torch::Tensor &order, const torch::Tensor &counts, int64_t nsc)
+{
+    TORCH_CHECK(nsc > 0, "nsc must be positive");
+    TORCH_CHECK(order.device().type() == torch::kCUDA && counts.device().type() == torch::kCUDA, "order and counts must be CUDA tensors");
+    TORCH_CHECK(order.dtype() == torch::kInt32 && counts.dtype() == torch::kInt32, "order and counts must be torch.int32");
+    TORCH_CHECK(order.is_contiguous() && counts.is_contiguous(), "order and counts must be contiguous");
+    TORCH_CHECK(order.numel() >= nsc, "order has fewer entries than superchunks");
+    TORCH_CHECK(counts.numel() >= 3, "counts must hold the three group sizes");
+}
+
+void mixed_compress(torch::Tensor src, torch::Tensor order, torch::Tensor counts, torch::Tensor dst, int64_t nsc,
+                    c10::optional<torch::Tensor> rand_pool, c10::optional<torch::Tensor> recv,
+                    c10::optional<torch::Tensor> center_mean, int center_world = 1, int64_t n = 0, int ring_chunk = 0,
+                    int ring_world = 1, uint64_t seed = 0, uint64_t step = 0, uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(src.scalar_type() == torch::kBFloat16 || src.scalar_type() == torch::kFloat32, "input must be torch.bfloat16 or torch.float32");
+    TORCH_CHECK(dst.dtype() == torch::kUInt8, "output must be torch.uint8");
+    TORCH_CHECK(src.is_contiguous() && dst.is_contiguous(), "buffers must be contiguous");
+    TORCH_CHECK(strategy == 2 || strategy == 3, "strategy must be 2 or 3");
+    TORCH_CHECK(ring_world > 0 && ring_chunk >= 0 && ring_chunk < ring_world, "ring_chunk must lie in [0, ring_world)");
+    check_plan_tensors(order, counts, nsc);
+    const int64_t need = dq_mixed_required_bytes(nsc, ring_world);
+    TORCH_CHECK(dst.numel() >= need, "output buffer is smaller than mixed_required_bytes(nsc, ring_world)");
+    int code = dq_dtype_of(src.scalar_type());
+    const void *rand_ptr = nullptr, *recv_ptr = nullptr;
+    const float *mean_ptr = nullptr;
+    if (rand_pool.has_value()) {
+        TORCH_CHECK(rand_pool->device().type() == torch::kCUDA && rand_pool->is_contiguous(), "rand_pool must be a contiguous CUDA tensor");
+        const bool mixed = src.scalar_type() == torch::kFloat32 && rand_pool->scalar_type() == torch::kBFloat16;
+        TORCH_CHECK(mixed || rand_pool->dtype() == src.dtype(), "rand_pool dtype must match input dtype");
+        TORCH_CHECK(rand_pool->numel() >= nsc * 256, "rand_pool has fewer than 256 * nsc elements");
+        if (mixed) code |= DQ_RAND_BF16;
+        rand_ptr = rand_pool->data_ptr();
+    }
+    if (recv.has_value()) {
+        TORCH_CHECK(recv->device().type() == torch::kCUDA && recv->dtype() == torch::kUInt8 && recv->is_contiguous(),
+                    "recv must be a contiguous torch.uint8 CUDA tensor");
+        TORCH_CHECK(recv->numel() >= need, "recv buffer is smaller than mixed_required_bytes(nsc, ring_world)");
+        recv_ptr = recv->data_ptr();
+    }
+    if (center_mean.has_value()) {
+        TORCH_CHECK(center_mean->device().type() == torch::kCUDA && center_mean->dtype() == torch::kFloat32 &&
+                        center_mean->is_contiguous() && center_mean->numel() >= nsc,
+                    "center_mean must be a contiguous torch.float32 CUDA tensor with one entry per superchunk");
+        TORCH_CHECK(center_world > 0, "center_world must be positive");
+        TORCH_CHECK(n > 0 && (n + 255) / 256 <= nsc, "n must lie in [1, 256 * nsc]");
+        TORCH_CHECK(src.numel() >= n, "input has fewer than n elements");
+        mean_ptr = center_mean->data_ptr<float>();
+    } else {
+        TORCH_CHECK(src.numel() >= nsc * 256, "input has fewer than 256 * nsc elements");
+    }
+    check_status(dq_mixed_compress(src.data_ptr(), mean_ptr, center_world, n, order.data_ptr<int32_t>(), counts.data_ptr<int32_t>(),
+                                   ring_chunk, ring_world, static_cast<const uint8_t *>(recv_ptr), dst.data_ptr<uint8_t>(), rand_ptr,
+                                   seed, step, nsc, code, src.device().index(), strategy, as_stream(stream_p)),
+                 "mixed_compress");
+}
+
+void mixed_decompress(torch::Tensor src, torch::Tensor dst, torch::Tensor order, torch::Tensor counts, int64_t nsc,
+                      c10::optional<torch::Tensor> stats, int64_t n_limit, int ring_chunk = 0, int ring_world = 1,
+                      uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA, "output must be a CUDA tensor");
+    TORCH_CHECK(src.dtype() == torch::kUInt8, "input must be torch.uint8");
+    TORCH_CHECK(dst.scalar_type() == torch::kBFloat16 || dst.scalar_type() == torch::kFloat32, "output must be torch.bfloat16 or torch.float32");
+    TORCH_CHECK(src.is_contiguous() && dst.is_contiguous(), "buffers must be contiguous");
+    TORCH_CHECK(strategy == 2 || strategy == 3, "strategy must be 2 or 3");
+    TORCH_CHECK(ring_world > 0 && ring_chunk >= 0 && ring_chunk < ring_world, "ring_chunk must lie in [0, ring_world)");
+    check_plan_tensors(order, counts, nsc);
+    TORCH_CHECK(src.numel() >= dq_mixed_required_bytes(nsc, ring_world), "input buffer is smaller than mixed_required_bytes(nsc, ring_world)");
+    TORCH_CHECK(n_limit > 0 && n_limit <= dst.numel() && n_limit <= nsc * 256, "n_limit must be in (0, min(output elements, 256 * nsc)]");
+    const void *stats_ptr = nullptr;
+    if (stats.has_value()) {
+        TORCH_CHECK(stats->device().type() == torch::kCUDA && stats->dtype() == torch::kBFloat16 && stats->is_contiguous(),
+                    "stats must be a contiguous torch.bfloat16 CUDA tensor");
+        TORCH_CHECK(stats->numel() >= 2 * nsc, "stats buffer is too small");
+        stats_ptr = stats->data_ptr();
+    }
+    check_status(dq_mixed_decompress(src.data_ptr<uint8_t>(), dst.data_ptr(), order.data_ptr<int32_t>(), counts.data_ptr<int32_t>(),
+                                     ring_chunk, ring_world, stats_ptr, n_limit, nsc, dq_dtype_of(dst.scalar_type()),
+                                     dst.device().index(), strategy, as_stream(stream_p)),
+                 "mixed_decompress");
+}
+
+void superchunk_stats(torch::Tensor src, torch::Tensor stats, c10::optional<torch::Tensor> mean, int64_t n, int world_size,
+                      uint64_t stream_p = 0)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA && stats.device().type() == torch::kCUDA, "src and stats must be CUDA tensors");
+    TORCH_CHECK(is_supported_data_dtype(src.scalar_type(), true), "src must be torch.float16, torch.bfloat16 or torch.float32");
+    TORCH_CHECK(stats.dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+    TORCH_CHECK(src.is_contiguous() && stats.is_contiguous(), "buffers must be contiguous");
+    TORCH_CHECK(n > 0, "n must be positive");
+    TORCH_CHECK(world_size > 0, "world_size must be positive");
+    TORCH_CHECK(src.numel() >= n, "src has fewer than n elements");
+    const int64_t nsc = (n + 255) / 256;
+    TORCH_CHECK(stats.numel() >= 2 * nsc, "stats buffer is too small");
+    float *mean_ptr = nullptr;
+    if (mean.has_value()) {
+        TORCH_CHECK(mean->device().type() == torch::kCUDA && mean->dtype() == torch::kFloat32 && mean->is_contiguous() &&
+                        mean->numel() >= nsc,
+                    "mean must be a contiguous torch.float32 CUDA tensor with one entry per superchunk");
+        mean_ptr = mean->data_ptr<float>();
+    }
+    check_status(dq_superchunk_stats(src.data_ptr(), stats.data_ptr(), mean_ptr, n, world_size, dq_dtype_of(src.scalar_type()),
+                                     src.device().index(), as_stream(stream_p)),
+                 "superchunk_stats");
+}
+
 // ---- superchunk ops ---------------------------------------------------------------
 
 void superchunk_mean_center(torch::Tensor src, torch::Tensor residual, torch::Tensor stats, int n, int world_size,
@@ -644,6 +758,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_decompress_rows", &scaling_decompress_rows, "decode consecutive records into the superchunks rows[k] of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("rows"), py::arg("stats"), py::arg("n_limit"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("mixed_required_bytes", &mixed_required_bytes, "upper bound of the packed stream of one ring chunk over the three bit-width groups", py::arg("nsc"), py::arg("ring_world") = 1);
+    modul.def("mixed_compress", &mixed_compress, "compress (or, with recv, decode-accumulate-recompress) ring chunk ring_chunk of all three bit-width groups of a planned bucket in one launch", py::arg("src"), py::arg("order"), py::arg("counts"), py::arg("dst"), py::arg("nsc"), py::arg("rand_pool") = py::none(), py::arg("recv") = py::none(), py::arg("center_mean") = py::none(), py::arg("center_world") = 1, py::arg("n") = 0, py::arg("ring_chunk") = 0, py::arg("ring_world") = 1, py::arg("seed") = 0, py::arg("step") = 0, py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("mixed_decompress", &mixed_decompress, "decode ring chunk ring_chunk of all three bit-width groups into their superchunks of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("order"), py::arg("counts"), py::arg("nsc"), py::arg("stats"), py::arg("n_limit"), py::arg("ring_chunk") = 0, py::arg("ring_world") = 1, py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("superchunk_stats", &superchunk_stats, "the statistics of superchunk_mean_center without the residual, plus the unrounded float32 means", py::arg("src"), py::arg("stats"), py::arg("mean"), py::arg("n"), py::arg("world_size"), py::arg("stream_p") = 0);
     modul.def("scaling_compress_philox", &scaling_compress_philox, "scaling compress with the uniform values drawn in the kernel (Philox: key = seed, counter = chunk, step)", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
     modul.def("scaling_dec_comp_philox", &scaling_dec_comp_philox, "scaling decompress and compress with the uniform values drawn in the kernel", py::arg("recv"), py::arg("inp"), py::arg("send"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
     modul.def("philox_uniform", &philox_uniform, "the uniform values of that stream written out as a tensor", py::arg("out"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0);

@@ -121,3 +121,81 @@ def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=
         else:
             ring_allreduce_rows(residuals, rows, comps, outs, total, n)
     return outs, total, qbits
+
+
+def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=None, work=None, stream=None):
+    """The same all-reduce with every stage kept on the device: no residual buffers (the centring is folded
+    into the codec's loads), no group tensors, no per-width launches and no read-back of the group sizes --
+    a fixed sequence of launches per bucket (statistics, plan, and one codec launch per ring step for all
+    three bit widths), which can be captured once and replayed as a graph.
+
+    Per rank: superchunk_stats -> (stats sum) -> group_plan_stats -> ring over mixed_compress /
+    mixed_decompress.  The bit widths follow the device rule of group_plan_stats; the rounding randomness is
+    the in-kernel stream keyed by (seed + rank, ring step, index of the chunk in the vector), so results are
+    reproducible but not those of dynamic_bitrate_allreduce, whose random values come from the pool.
+
+    Returns (result tensors per rank, reduced stats, device int32 tensor [n8, n4, n2, other])."""
+    from . import capi
+    W = len(rank_vecs)
+    n = rank_vecs[0].numel()
+    nsc = (n + SUPERCHUNK - 1) // SUPERCHUNK
+    dev, dt = rank_vecs[0].device, rank_vecs[0].dtype
+    if work is None:
+        work = {}
+    key = ("single_pass", nsc, dt, W)
+    if work.get("key") != key:
+        work.clear()
+        work["key"] = key
+        cap = capi.mixed_required_bytes(nsc, W)
+        work["stats"] = [torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev) for _ in range(W)]
+        work["mean"] = [torch.empty(nsc, dtype=torch.float32, device=dev) for _ in range(W)]
+        work["total"] = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
+        work["order"] = torch.empty(nsc, dtype=torch.int32, device=dev)
+        work["plan"] = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
+        work["send"] = [torch.zeros(cap, dtype=torch.uint8, device=dev) for _ in range(W)]
+        work["recv"] = [torch.zeros(cap, dtype=torch.uint8, device=dev) for _ in range(W if W > 1 else 0)]
+    stats, mean, order, plan = work["stats"], work["mean"], work["order"], work["plan"]
+    send, recv = work["send"], work["recv"]
+    for r in range(W):
+        capi.superchunk_stats(rank_vecs[r], stats[r], mean[r], n, W, stream=stream)
+    if W == 1:
+        total = stats[0]
+    else:
+        total = work["total"]
+        total.copy_(stats[0])
+        for r in range(1, W):
+            total.add_(stats[r])
+    capi.group_plan_stats(total, float(u), None, order, plan, stream=stream)
+    outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
+
+    def encode(r, chunk, step, received=None):
+        capi.mixed_compress(rank_vecs[r], order, plan, send[r], nsc, strategy, seed=seed + r, step=step, recv=received,
+                            center_mean=mean[r], center_world=W, n=n, ring_chunk=chunk, ring_world=W, stream=stream)
+
+    def decode(r, packed, chunk):
+        capi.mixed_decompress(packed, outs[r], order, plan, nsc, strategy, stats=total, n_limit=n, ring_chunk=chunk,
+                              ring_world=W, stream=stream)
+
+    if W == 1:
+        encode(0, 0, 0)
+        decode(0, send[0], 0)
+        return outs, total, plan[:4]
+
+    def exchange(src_bufs, dst_bufs):
+        for r in range(W):
+            dst_bufs[(r + 1) % W].copy_(src_bufs[r])
+
+    # reduce-scatter: W - 1 steps, then the owner's step; all-gather of the owners' streams
+    for step in range(W - 1):
+        for r in range(W):
+            encode(r, (r - step + W) % W, step, None if step == 0 else recv[r])
+        exchange(send, recv)
+    for r in range(W):
+        encode(r, (r + 1) % W, W - 1, recv[r])
+        decode(r, send[r], (r + 1) % W)
+    bufs = [send, recv]
+    for step in range(W - 1):
+        exchange(bufs[step & 1], bufs[(step ^ 1) & 1])
+        for r in range(W):
+            decode(r, bufs[(step ^ 1) & 1][r], (r - step + W) % W)
+    return outs, total, plan[:4]

@@ -158,11 +158,9 @@ def _torch_cpu_roundtrip(x, rand, nbits, chunk=16):
 
 
 def _cpu_torch_line(x32, nbits):
-    """median of 5 round trips on all host cores, one warm-up"""
-    import os
+    """median of 5 round trips on torch's intra-op thread pool (its size follows OMP_NUM_THREADS), one warm-up"""
     import time
-    threads = os.cpu_count() or 1
-    torch.set_num_threads(threads)
+    threads = torch.get_num_threads()
     xc = x32.cpu()
     rc = torch.rand(xc.numel())
     _torch_cpu_roundtrip(xc, rc, nbits)

@@ -193,6 +193,57 @@ int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *row
                                int dtype, int device, int strategy, dq_stream_t stream,
                                int add_original);
 
+/* ---- the three bit-width groups of a bucket in one launch ----------------
+ *
+ * comm_hooks.py:963-1018 runs gather -> ring all-reduce -> scatter once per
+ * bit-width group (8, 4, 2), with the group sizes known on the host.  The
+ * calls below take the partition from device memory instead -- `order` and the
+ * first three ints of `work` as written by dq_group_plan / dq_group_plan_stats
+ * (n8, n4, n2) -- and serve all three groups with one launch and no host
+ * synchronisation.
+ *
+ * Ring chunk `ring_chunk` of `ring_world` is, per group, superchunks
+ * [per * ring_chunk, min(per * (ring_chunk + 1), n_g)) of the group with
+ * per = ceil(n_g / ring_world) (the split of ring_rdma.py:590-631 applied to a
+ * gathered group).  Its packed stream is the 8-bit records, then the 4-bit
+ * records, then the 2-bit records, each run byte for byte what
+ * dq_scaling_compress_rows writes for the same superchunks and random values;
+ * dq_mixed_required_bytes(nsc, ring_world) bounds its size.  ring_world = 1,
+ * ring_chunk = 0 addresses whole groups.
+ *
+ * Rounding randomness: rand_pool != NULL -> row k (256 values, element type of
+ * src, or bf16 with DQ_RAND_BF16) belongs to position k of `order`, so the
+ * pool holds >= 256 * nsc values; rand_pool == NULL -> the in-kernel Philox
+ * stream of dq_scaling_compress_philox, keyed by (seed, step, index of the
+ * chunk in src).
+ *
+ * center_mean != NULL folds superchunk_mean_center into the load: element e
+ * of src is replaced by T(float(src[e]) / center_world - center_mean[e / 256]),
+ * and by zero at e >= n; nothing at or beyond n is read.  center_mean is the
+ * binary32 mean array written by dq_superchunk_stats.  With center_mean ==
+ * NULL src is a residual buffer of 256 * nsc elements and n is ignored.
+ * recv != NULL makes the call the ring's fused step (decode recv, add the
+ * centred source, re-encode into dst; recv and dst share one layout).
+ * strategy 2 or 3, dtype DQ_BF16 or DQ_F32. */
+int64_t dq_mixed_required_bytes(int64_t nsc, int ring_world);
+int dq_mixed_compress(const void *src, const float *center_mean, int center_world, int64_t n,
+                      const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world,
+                      const uint8_t *recv, uint8_t *dst, const void *rand_pool, uint64_t seed,
+                      uint64_t step, int64_t nsc, int dtype, int device, int strategy,
+                      dq_stream_t stream);
+
+/* decode ring chunk `ring_chunk` of all three groups into their superchunks of
+ * dst; stats / n_limit as in dq_scaling_decompress_rows. */
+int dq_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, const int32_t *counts,
+                        int ring_chunk, int ring_world, const void *stats, int64_t n_limit,
+                        int64_t nsc, int dtype, int device, int strategy, dq_stream_t stream);
+
+/* cuda_hadamard.cu:1304-1349 without the residual: stats as written by
+ * dq_superchunk_mean_center, plus (mean != NULL) the unrounded binary32 mean
+ * of every superchunk, float [ceil(n / 256)]. */
+int dq_superchunk_stats(const void *src, void *stats, float *mean, int64_t n, int world_size,
+                        int dtype, int device, dq_stream_t stream);
+
 /* ---- consumers of the rotated vector: EDEN and THC ----------------------
  *
  * "reference" here: cuda_kernels/src/srrcomp/srrcomp.py (EDEN) and

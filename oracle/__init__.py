@@ -77,6 +77,8 @@ def _declare(L):
     L.dqo_scaling_decompress.argtypes = [vp, vp, i64, i32, i32, i32, i32, i32]
     L.dqo_scaling_dec_comp.restype = i32
     L.dqo_scaling_dec_comp.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32]
+    L.dqo_superchunk_stats.restype = None
+    L.dqo_superchunk_stats.argtypes = [vp, vp, vp, i64, i32, i32]
     L.dqo_superchunk_mean_center.restype = None
     L.dqo_superchunk_mean_center.argtypes = [vp, vp, vp, i64, i32, i32]
     L.dqo_superchunk_add_mean_copy.restype = None
@@ -206,6 +208,16 @@ def superchunk_mean_center(src, n, world_size, dtype):
     stats = np.zeros(nsc * 2, np.uint16)
     lib().dqo_superchunk_mean_center(_p(src), _p(residual), _p(stats), n, world_size, dtype)
     return residual, stats
+
+
+def superchunk_stats(src, n, world_size, dtype):
+    """(stats uint16 [2 nsc], means float32 [nsc]) of superchunk_mean_center, no residual"""
+    _chk(src, _elem_dtype(dtype), "src")
+    nsc = (n + 255) // 256
+    stats = np.zeros(nsc * 2, np.uint16)
+    mean = np.zeros(nsc, np.float32)
+    lib().dqo_superchunk_stats(_p(src), _p(stats), _p(mean), n, world_size, dtype)
+    return stats, mean
 
 
 def superchunk_add_mean_copy(residual, stats, n, dtype, dst=None):

@@ -675,8 +675,8 @@ int dqo_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const vo
 /* superchunk mean-centre / add-mean                                         */
 /* ------------------------------------------------------------------------ */
 
-void dqo_superchunk_mean_center(const void *src, void *residual, uint16_t *stats,
-                                int64_t n, int world_size, int dtype)
+static void mean_center_impl(const void *src, void *residual, uint16_t *stats, float *mean_out,
+                             int64_t n, int world_size, int dtype)
 {
     const int64_t nsc = (n + 255) / 256;
     float sum[256], sq[256], val[256];
@@ -698,11 +698,24 @@ void dqo_superchunk_mean_center(const void *src, void *residual, uint16_t *stats
                 sq[l] += sq[l + stride];
             }
         float mean = valid > 0 ? sum[0] / (float)valid : 0.0f;
-        for (int l = 0; l < 256; l++)
-            store_elem(residual, dtype, start + l, l < valid ? val[l] - mean : 0.0f);
+        if (residual)
+            for (int l = 0; l < 256; l++)
+                store_elem(residual, dtype, start + l, l < valid ? val[l] - mean : 0.0f);
         stats[2 * b] = dqo_f32_to_bf16(mean);
         stats[2 * b + 1] = dqo_f32_to_bf16(sq[0]);
+        if (mean_out) mean_out[b] = mean;
     }
+}
+
+void dqo_superchunk_mean_center(const void *src, void *residual, uint16_t *stats,
+                                int64_t n, int world_size, int dtype)
+{
+    mean_center_impl(src, residual, stats, NULL, n, world_size, dtype);
+}
+
+void dqo_superchunk_stats(const void *src, uint16_t *stats, float *mean, int64_t n, int world_size, int dtype)
+{
+    mean_center_impl(src, NULL, stats, mean, n, world_size, dtype);
 }
 
 void dqo_superchunk_add_mean_copy(const void *residual, void *dst, const uint16_t *stats,

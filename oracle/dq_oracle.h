@@ -108,6 +108,10 @@ int dqo_scaling_dec_comp(const uint8_t *recv, void *inp, uint8_t *send, const vo
 /* csrc/cuda_hadamard.cu:1257-1349; stats is bf16 [2*ceil(n/256)] */
 void dqo_superchunk_mean_center(const void *src, void *residual, uint16_t *stats,
                                 int64_t n, int world_size, int dtype);
+/* the same statistics without the residual, plus the unrounded binary32 mean of every superchunk
+ * (the value the residual is formed with) */
+void dqo_superchunk_stats(const void *src, uint16_t *stats, float *mean, int64_t n, int world_size,
+                          int dtype);
 /* csrc/cuda_hadamard.cu:1351-1369 */
 void dqo_superchunk_add_mean_copy(const void *residual, void *dst, const uint16_t *stats,
                                   int64_t n, int dtype);

@@ -1,0 +1,297 @@
+"""All bit-width groups of a bucket in one launch (dq_mixed_*), against the per-group calls they replace
+(testbed_evaluation/new_comm_hooks/comm_hooks.py:963-1018 runs the ring once per group) and against the
+oracle -- byte for byte."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, F32, to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+REC = {8: 274, 4: 146, 2: 82}
+
+
+def bits_t(t):
+    return t.view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+def make_plan(capi, nsc, seed, weights=(1, 1, 1)):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.tensor(weights, dtype=torch.float)
+    q = torch.tensor([8, 4, 2])[torch.multinomial(w, nsc, replacement=True, generator=g)].to(DEV)
+    order = torch.full((nsc,), -1, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    capi.group_plan(q, order, work)
+    return q, order, work
+
+
+def segments(counts, chunk, world):
+    """(width, position of the run in `order`, records, byte offset) of ring chunk `chunk`, and the stream size"""
+    out, pos, off = [], 0, 0
+    for q, n in zip((8, 4, 2), counts):
+        per = -(-n // world)
+        begin = min(per * chunk, n)
+        cnt = min(per, n - begin)
+        out.append((q, pos + begin, cnt, off))
+        pos += n
+        off += cnt * REC[q]
+    return out, off
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("strategy", [2, 3])
+@pytest.mark.parametrize("nsc,world,weights", [(1037, 1, (1, 1, 1)), (1037, 3, (1, 2, 3)), (2, 1, (1, 1, 1)),
+                                               (515, 4, (1, 0, 1)), (64, 8, (0, 1, 0)), (6403, 8, (1, 6, 2))])
+def test_mixed_matches_per_group_calls(capi, dt, strategy, nsc, world, weights):
+    n_valid = nsc * 256 - 77
+    q, order, work = make_plan(capi, nsc, nsc + world, weights)
+    counts = work[:3].tolist()
+    assert sum(counts) == nsc
+    g = torch.Generator().manual_seed(nsc * 3 + strategy)
+    full = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+    peer = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+    stats = torch.randn(nsc, 2, generator=g).mul(1e-2).to(torch.bfloat16).to(DEV)
+    pool = torch.rand(nsc * 256, generator=g).to(torch.bfloat16 if (dt == torch.bfloat16 or strategy == 2) else dt).to(DEV)
+    cap = capi.mixed_required_bytes(nsc, world)
+    out = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
+    out_ref = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
+    for chunk in range(world):
+        segs, total = segments(counts, chunk, world)
+        assert total <= cap
+        enc = torch.full((cap + 16,), 0xAB, dtype=torch.uint8, device=DEV)
+        send = torch.full((cap + 16,), 0xCD, dtype=torch.uint8, device=DEV)
+        capi.mixed_compress(full, order, work, enc, nsc, strategy, rand_pool=pool, ring_chunk=chunk, ring_world=world)
+        peer_before = peer.clone()
+        capi.mixed_compress(peer, order, work, send, nsc, strategy, rand_pool=pool, recv=enc, ring_chunk=chunk,
+                            ring_world=world)
+        assert torch.equal(peer, peer_before)
+        capi.mixed_decompress(send, out, order, work, nsc, strategy, stats=stats, n_limit=n_valid, ring_chunk=chunk,
+                              ring_world=world)
+        assert bool((enc[total:] == 0xAB).all()) and bool((send[total:] == 0xCD).all())    # nothing past the stream
+        for width, pos, cnt, off in segs:
+            if cnt == 0:
+                continue
+            rows = order[pos:pos + cnt]
+            rnd = pool[pos * 256:(pos + cnt) * 256]
+            nb = cnt * REC[width]
+            e = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+            s = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+            capi.scaling_compress_rows(full, rows, e, rnd, cnt, width, strategy)
+            capi.scaling_dec_comp_rows(e, peer, rows, s, rnd, cnt, width, strategy)
+            assert torch.equal(enc[off:off + nb], e), (chunk, width)
+            assert torch.equal(send[off:off + nb], s), (chunk, width)
+            capi.scaling_decompress_rows(s, out_ref, rows, stats, n_valid, cnt, width, strategy)
+    assert torch.equal(bits_t(out), bits_t(out_ref))
+    assert bool((out[n_valid:] == 7.0).all())
+
+
+@pytest.mark.parametrize("dt,odt", [(torch.bfloat16, BF16), (torch.float32, F32)])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_mixed_philox_matches_oracle(capi, oracle, dt, odt, strategy):
+    """in-kernel rounding stream keyed by the chunk's index in the source vector: every run equals the oracle's
+    compress of the gathered superchunks with the gathered uniform values"""
+    nsc, seed, step = 333, 2027, 5
+    q, order, work = make_plan(capi, nsc, 17)
+    counts = work[:3].tolist()
+    g = torch.Generator().manual_seed(5)
+    full = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+    enc = torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=DEV)
+    capi.mixed_compress(full, order, work, enc, nsc, strategy, seed=seed, step=step)
+    uni = oracle.philox_uniform(nsc * 256, seed, step)
+    if odt == BF16:
+        uni = (uni.view(np.uint32) >> 16).astype(np.uint16)     # k/256 is exact in bf16
+    src_h = to_bits(full.cpu())
+    ord_h = order.cpu().numpy()
+    segs, total = segments(counts, 0, 1)
+    got = enc.cpu().numpy()
+    for width, pos, cnt, off in segs:
+        rows = ord_h[pos:pos + cnt]
+        gs = src_h.reshape(-1, 256)[rows].reshape(-1).copy()
+        gu = uni.reshape(-1, 256)[rows].reshape(-1).copy()
+        want = oracle.scaling_compress(gs, gu, cnt * 256, width, 16, strategy, odt)
+        assert (got[off:off + cnt * REC[width]] == want).all(), width
+    # natural order (rows == identity) of the single-width Philox call uses the same key
+    e4 = torch.zeros(capi.required_bytes(nsc * 256, 4, 16, strategy), dtype=torch.uint8, device=DEV)
+    capi.scaling_compress_philox(full, e4, nsc * 256, 4, 16, strategy, seed, step)
+    want = oracle.scaling_compress(src_h, uni, nsc * 256, 4, 16, strategy, odt)
+    assert (e4.cpu().numpy() == want).all()
+
+
+@pytest.mark.parametrize("dt,odt", [(torch.bfloat16, BF16), (torch.float32, F32)])
+@pytest.mark.parametrize("world", [1, 2, 3, 8])
+@pytest.mark.parametrize("n", [256 * 40, 256 * 41 - 200, 256 * 41 - 1, 77])
+def test_stats_and_centre_on_load(capi, oracle, dt, odt, world, n):
+    """superchunk_stats == the oracle's statistics and binary32 means; compress with the centring folded into the
+    load == mean_center followed by compress of the residual, with nothing read beyond n"""
+    nsc = (n + 255) // 256
+    g = torch.Generator().manual_seed(n + world)
+    base = torch.randn(n, generator=g) * 1e-2 + 3e-3
+    src = torch.full((n + 64,), float("nan"), dtype=dt, device=DEV)     # a NaN beyond n must never be picked up
+    src[:n] = base.to(dt)
+    stats = torch.zeros(nsc, 2, dtype=torch.bfloat16, device=DEV)
+    mean = torch.zeros(nsc, dtype=torch.float32, device=DEV)
+    capi.superchunk_stats(src, stats, mean, n, world)
+    st_o, mean_o = oracle.superchunk_stats(to_bits(src[:n].cpu()), n, world, odt)
+    assert (to_bits(stats.cpu()).reshape(-1) == st_o).all()
+    assert (mean.cpu().numpy().view(np.uint32) == mean_o.view(np.uint32)).all()
+    stats2 = torch.zeros_like(stats)
+    capi.superchunk_stats(src, stats2, None, n, world)
+    assert torch.equal(bits_t(stats), bits_t(stats2))
+
+    residual = torch.zeros(nsc * 256, dtype=dt, device=DEV)
+    stats3 = torch.zeros_like(stats)
+    capi.superchunk_mean_center(src, residual, stats3, n, world)
+    assert torch.equal(bits_t(stats), bits_t(stats3))
+    q, order, work = make_plan(capi, nsc, n)
+    pool = torch.rand(nsc * 256, generator=g).to(dt).to(DEV)
+    cap = capi.mixed_required_bytes(nsc, 1)
+    for strategy in (2, 3):
+        a = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+        b = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+        capi.mixed_compress(residual, order, work, a, nsc, strategy, rand_pool=pool)
+        capi.mixed_compress(src, order, work, b, nsc, strategy, rand_pool=pool, center_mean=mean, center_world=world, n=n)
+        assert torch.equal(a, b), strategy
+        # the fused step centres its local operand the same way
+        a2, b2 = torch.zeros_like(a), torch.zeros_like(a)
+        capi.mixed_compress(residual, order, work, a2, nsc, strategy, seed=9, step=1, recv=a)
+        capi.mixed_compress(src, order, work, b2, nsc, strategy, seed=9, step=1, recv=a, center_mean=mean,
+                            center_world=world, n=n)
+        assert torch.equal(a2, b2), strategy
+
+
+def test_mixed_misaligned_buffers(capi):
+    """element buffers that are only element-aligned and streams at odd byte offsets"""
+    nsc = 203
+    q, order, work = make_plan(capi, nsc, 3)
+    g = torch.Generator().manual_seed(1)
+    dt = torch.bfloat16
+    full_al = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+    pool_al = torch.rand(nsc * 256, generator=g).to(dt).to(DEV)
+    full = torch.zeros(nsc * 256 + 8, dtype=dt, device=DEV)[3:3 + nsc * 256].copy_(full_al)
+    pool = torch.zeros(nsc * 256 + 8, dtype=dt, device=DEV)[1:1 + nsc * 256].copy_(pool_al)
+    cap = capi.mixed_required_bytes(nsc, 1)
+    ref = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+    capi.mixed_compress(full_al, order, work, ref, nsc, 2, rand_pool=pool_al)
+    enc = torch.zeros(cap + 16, dtype=torch.uint8, device=DEV)[5:5 + cap]
+    capi.mixed_compress(full, order, work, enc, nsc, 2, rand_pool=pool)
+    assert torch.equal(enc, ref)
+    out_ref = torch.zeros(nsc * 256, dtype=dt, device=DEV)
+    capi.mixed_decompress(ref, out_ref, order, work, nsc, 2)
+    out = torch.zeros(nsc * 256 + 8, dtype=dt, device=DEV)[1:1 + nsc * 256]
+    capi.mixed_decompress(enc, out, order, work, nsc, 2)
+    assert torch.equal(bits_t(out), bits_t(out_ref))
+
+
+def test_mixed_pipeline_replays_as_graph(capi):
+    """stats -> plan -> compress -> decompress of a bucket is a fixed launch sequence with no read-back: captured
+    once, replayed on new data, every replay equals the eager result"""
+    n = 6553600 // 4
+    nsc = n // 256
+    g = torch.Generator().manual_seed(11)
+    scales = torch.exp(torch.randn(nsc, 1, generator=g) * 6.0) * 1e-3
+    src = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    stats = torch.zeros(nsc, 2, dtype=torch.bfloat16, device=DEV)
+    mean = torch.zeros(nsc, dtype=torch.float32, device=DEV)
+    order = torch.zeros(nsc, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    enc = torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=DEV)
+    out = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    u = 7.1
+
+    def fill(seed):
+        gg = torch.Generator().manual_seed(seed)
+        src.copy_((torch.randn(nsc, 256, generator=gg) * scales).reshape(-1).to(torch.bfloat16))
+
+    def pipeline(stream=None):
+        capi.superchunk_stats(src, stats, mean, n, 1, stream=stream)
+        capi.group_plan_stats(stats, u, None, order, work, stream=stream)
+        capi.mixed_compress(src, order, work, enc, nsc, 2, seed=1, step=0, center_mean=mean, center_world=1, n=n,
+                            stream=stream)
+        capi.mixed_decompress(enc, out, order, work, nsc, 2, stats=stats, n_limit=n, stream=stream)
+
+    fill(0)
+    pipeline()
+    torch.cuda.synchronize()
+    counts0 = work[:3].tolist()
+    assert min(counts0) > 0, counts0
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            pipeline(side.cuda_stream)
+    for seed in (1, 2, 3):
+        fill(seed)
+        graph.replay()
+        torch.cuda.synchronize()
+        got, got_enc, got_counts = out.clone(), enc.clone(), work[:3].tolist()
+        out.zero_()
+        pipeline()
+        torch.cuda.synchronize()
+        assert got_counts == work[:3].tolist()
+        total = sum(c * REC[w] for c, w in zip(got_counts, (8, 4, 2)))
+        assert torch.equal(got_enc[:total], enc[:total])
+        assert torch.equal(bits_t(got), bits_t(out))
+        err = (out.float() - src.float()).pow(2).sum() / src.float().pow(2).sum()
+        assert float(err) < 0.05
+
+
+@pytest.mark.parametrize("W", [1, 2, 3])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_single_pass_pipeline_matches_oracle(capi, oracle, W, strategy):
+    """the whole device-resident all-reduce (statistics, widths, partition, ring of mixed launches, mean add) against
+    the oracle's functions chained on the host, bit for bit, for every simulated rank"""
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import dynamic_bitrate_allreduce_single_pass
+    n, seed, u = 256 * 301 - 100, 77, 6.0
+    nsc = (n + 255) // 256
+    g = torch.Generator().manual_seed(W * 10 + strategy)
+    scales = torch.exp(torch.randn(nsc, 1, generator=g) * 6.0) * 1e-3
+    vecs = [((torch.randn(nsc, 256, generator=g) * scales).reshape(-1)[:n] + 1e-4).to(torch.bfloat16) for _ in range(W)]
+    outs, total, counts = dynamic_bitrate_allreduce_single_pass([v.to(DEV) for v in vecs], u, strategy=strategy, seed=seed)
+    torch.cuda.synchronize()
+
+    # host chain
+    res, stats = [], []
+    for v in vecs:
+        r, s = oracle.superchunk_mean_center(to_bits(v), n, W, BF16)
+        res.append(r.reshape(-1, 256))
+        stats.append(torch.from_numpy(s.view(np.int16).copy()).view(torch.bfloat16))
+    tot = stats[0].clone()
+    for s in stats[1:]:
+        tot.add_(s)                                   # bf16 adds, the order of the pipeline
+    tot_bits = to_bits(tot)
+    assert (to_bits(total.cpu()).reshape(-1) == tot_bits).all()
+    qb = oracle.dynamic_bitrate_qbits(tot_bits[1::2].copy(), u)
+    cnt = [int((qb == w).sum()) for w in (8, 4, 2)]
+    assert counts.tolist() == cnt + [0] and min(cnt) > 0, (counts.tolist(), cnt)
+    uni = {}
+
+    def U(rank, step, rows):
+        if (rank, step) not in uni:
+            x = oracle.philox_uniform(nsc * 256, seed + rank, step)
+            uni[(rank, step)] = (x.view(np.uint32) >> 16).astype(np.uint16).reshape(-1, 256)
+        return uni[(rank, step)][rows].reshape(-1).copy()
+
+    want = np.zeros((nsc, 256), np.uint16)
+    for width in (8, 4, 2):
+        rows_g = np.nonzero(qb == width)[0]
+        per = -(-rows_g.size // W)
+        for c in range(W):
+            rows = rows_g[per * c:per * (c + 1)]
+            if rows.size == 0:
+                continue
+            m = rows.size * 256
+            stream = oracle.scaling_compress(res[c][rows].reshape(-1).copy(), U(c, 0, rows), m, width, 16, strategy, BF16)
+            for s in range(1, W):
+                rank = (c + s) % W
+                stream = oracle.scaling_dec_comp(stream, res[rank][rows].reshape(-1).copy(), U(rank, s, rows), m, width, 16,
+                                                 strategy, BF16)
+            dec = np.zeros(m, np.uint16)
+            oracle.scaling_decompress(stream, dec, m, width, 16, strategy, BF16)
+            want[rows] = dec.reshape(-1, 256)
+    final = oracle.superchunk_add_mean_copy(want.reshape(-1), tot_bits, n, BF16)
+    for r in range(W):
+        assert (to_bits(outs[r].cpu()) == final).all(), r
+    exact = torch.stack([v.double() for v in vecs]).sum(0) / W
+    err = float((outs[0].cpu().double() - exact).pow(2).sum() / exact.pow(2).sum())
+    assert err < 0.02, err
