@@ -22,7 +22,8 @@ import torch
 
 from . import bitrate, capi
 from .compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
-from .dynamiq_pipeline import dynamic_bitrate_allreduce, dynamic_bitrate_allreduce_grouped
+from .dynamiq_pipeline import (dynamic_bitrate_allreduce, dynamic_bitrate_allreduce_grouped,
+                               dynamic_bitrate_allreduce_single_pass)
 from .ring_sim import ring_allreduce, split_chunks
 
 HBM_PEAK = 8000.0  # GB/s
@@ -327,6 +328,53 @@ def config4(dev, limit=None):
                   achieved_bits_with_scales=bits / elems + OV, nmse=num / den, output_checksum=check,
                   ms_per_25MB_bucket=round(gpu_ms / len(timed), 4),
                   pipeline_GBps_of_bf16_input=round(2.0 * sum(m for _, m in timed) / (gpu_ms * 1e-3) / 1e9, 1))
+        # everything on the device, one launch for the three widths; eager, then captured once and replayed
+        strategy = 2 if name == "aee" else 3
+        for graphed in (False, True):
+            work, graph, src, out = {}, None, None, None
+            num = den = 0.0
+            bits = elems = 0
+            check = 0
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            times = []
+            for b in _llama_buckets(dev, limit=limit):
+                x = b.to(torch.bfloat16)
+                if graphed and src is None:
+                    src, out = torch.empty_like(x), [torch.empty_like(x)]
+                    src.copy_(x)
+                    dynamic_bitrate_allreduce_single_pass([src], u, strategy=strategy, seed=3, out=out, work=work)
+                    torch.cuda.synchronize()
+                    side = torch.cuda.Stream()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.stream(side):
+                        with torch.cuda.graph(graph, stream=side):
+                            _, _, counts = dynamic_bitrate_allreduce_single_pass([src], u, strategy=strategy, seed=3, out=out,
+                                                                                 work=work, stream=side.cuda_stream)
+                if graphed and x.numel() == src.numel():
+                    src.copy_(x)
+                    s.record()
+                    graph.replay()
+                    e.record()
+                    outs = out
+                else:
+                    s.record()
+                    outs, _, counts = dynamic_bitrate_allreduce_single_pass([x], u, strategy=strategy, seed=3,
+                                                                            work=None if graphed else work)
+                    e.record()
+                e.synchronize()
+                times.append((s.elapsed_time(e), x.numel()))
+                num += float(((outs[0].double() - b.double()) ** 2).sum())
+                den += float((b.double() ** 2).sum())
+                c = counts.tolist()
+                bits += 8 * c[0] + 4 * c[1] + 2 * c[2]
+                elems += sum(c[:3])
+                check ^= int(outs[0].view(torch.int16).to(torch.int64).sum()) & 0xFFFFFFFF
+            timed = times[3:] if len(times) > 3 else times
+            gpu_ms = sum(t for t, _ in timed)
+            _emit(config=4, method=name, pipeline="single_pass+graph" if graphed else "single_pass", buckets=len(times),
+                  elements=elems * 256, u=u, achieved_avg_code_bits=bits / elems, achieved_bits_with_scales=bits / elems + OV,
+                  nmse=num / den, output_checksum=check, ms_per_25MB_bucket=round(gpu_ms / len(timed), 4),
+                  pipeline_GBps_of_bf16_input=round(2.0 * sum(m for _, m in timed) / (gpu_ms * 1e-3) / 1e9, 1))
 
 
 def config5(dev, n=1 << 30):
@@ -412,7 +460,7 @@ def kernels(dev, n=6553600):
     line("superchunk_mean_center", lambda: capi.superchunk_mean_center(src, res, stats, n, 8), 4 * n + 4 * nsc, elements="bf16")
     line("superchunk_add_mean_copy", lambda: capi.superchunk_add_mean_copy(res, out, stats, n), 4 * n + 2 * nsc, elements="bf16")
     order = torch.empty(nsc, dtype=torch.int32, device=dev)
-    work = torch.empty(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
     qbits = torch.empty(nsc, dtype=torch.int64, device=dev)
     u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)
     line("group_plan_stats", lambda: capi.group_plan_stats(stats, u, qbits, order, work), 4 * nsc + 12 * nsc, superchunks=nsc)

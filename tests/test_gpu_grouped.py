@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("nsc", [1, 5, 1023, 1024, 1025, 25600, 300001])
+@pytest.mark.parametrize("nsc", [1, 5, 1023, 1024, 1025, 4096, 4097, 25600, 65535, 65536, 65537, 300001])
 def test_group_plan_matches_nonzero(capi, nsc):
     g = torch.Generator().manual_seed(nsc)
     q = torch.tensor([2, 4, 8, 16])[torch.randint(0, 4 if nsc > 5 else 3, (nsc,), generator=g)].to(DEV)
@@ -22,12 +22,16 @@ def test_group_plan_matches_nonzero(capi, nsc):
         q[:] = 8            # a single group
     order = torch.full((nsc,), -1, dtype=torch.int32, device=DEV)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
-    capi.group_plan(q, order, work)
-    counts = work[:4].tolist()
-    want = [torch.nonzero(q == w).view(-1) for w in (8, 4, 2)]
-    assert counts[:3] == [w.numel() for w in want] and counts[3] == int((q == 16).sum())
-    got = order[:sum(counts[:3])].cpu()
-    assert torch.equal(got, torch.cat(want).cpu().to(torch.int32))
+    for rep in range(3):        # the same work buffer serves call after call
+        if rep:
+            q = q.roll(rep * 37 + 1)
+            order.fill_(-1)
+        capi.group_plan(q, order, work)
+        counts = work[:4].tolist()
+        want = [torch.nonzero(q == w).view(-1) for w in (8, 4, 2)]
+        assert counts[:3] == [w.numel() for w in want] and counts[3] == int((q == 16).sum())
+        got = order[:sum(counts[:3])].cpu()
+        assert torch.equal(got, torch.cat(want).cpu().to(torch.int32))
 
 
 def test_group_plan_stats_all_bf16_norms(capi, oracle):

@@ -109,6 +109,21 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 1, 0, 1, S), "strategy")
     err(L.dq_scaling_dec_comp_rows(P, P, P, P, P, 0, 4, 1, 0, 2, S), "n must be positive")
     err(L.dq_scaling_decompress_rows(P, P, P, P, 2560, 10, 4, 1, 0, 2, S, 1), "stats cannot be combined")
+    Z = ctypes.c_uint64(0)
+    err(L.dq_mixed_compress(P, N, 1, 0, P, P, 0, 0, N, P, P, Z, Z, 100, 1, 0, 2, S), "world")           # ring_world 0
+    err(L.dq_mixed_compress(P, N, 1, 0, P, P, 3, 3, N, P, P, Z, Z, 100, 1, 0, 2, S), "world")           # chunk outside the ring
+    err(L.dq_mixed_compress(P, N, 1, 0, P, P, 0, 1, N, P, P, Z, Z, 100, 0, 0, 2, S), "unsupported element dtype")
+    err(L.dq_mixed_compress(P, N, 1, 0, P, P, 0, 1, N, P, P, Z, Z, 100, 1, 0, 0, S), "strategy")
+    err(L.dq_mixed_compress(P, N, 1, 0, P, N, 0, 1, N, P, P, Z, Z, 100, 1, 0, 2, S), "null pointer")
+    err(L.dq_mixed_compress(P, P, 1, 25700, P, P, 0, 1, N, P, P, Z, Z, 100, 1, 0, 2, S), "256 * nsc")   # n beyond the plan
+    err(L.dq_mixed_compress(P, P, 0, 100, P, P, 0, 1, N, P, P, Z, Z, 100, 1, 0, 2, S), "world")         # centring by 0 ranks
+    err(L.dq_mixed_decompress(P, P, P, P, 0, 1, N, 0, 100, 1, 0, 2, S), "n_limit")
+    err(L.dq_mixed_decompress(P, P, P, P, 0, 1, N, 100, 0, 1, 0, 2, S), "n must be positive")
+    err(L.dq_superchunk_stats(P, P, N, 0, 1, 1, 0, S), "n must be positive")
+    err(L.dq_superchunk_stats(P, N, N, 100, 1, 1, 0, S), "null pointer")
+    err(L.dq_superchunk_stats(P, P, N, 100, 0, 1, 0, S), "world")
+    assert L.dq_mixed_required_bytes(25600, 1) == (25600 + 3) * 274 and L.dq_mixed_required_bytes(25600, 8) == (3200 + 3) * 274
+    assert L.dq_mixed_required_bytes(0, 1) == 0
     err(L.dq_eden_quantize(P, 100, P, P, 4, P, P, P, 10, 0, S), "multiple of 32")
     err(L.dq_eden_quantize(P, 8192, P, P, 4, P, P, P, 1, 0, S), "work buffer is too small")
     err(L.dq_eden_dequantize(P, 64, P, 9, P, 0, S), "nbits")
