@@ -240,10 +240,24 @@ def config3(dev, n=124439808, W=8):
         e.record()
         e.synchronize()
         same = all(torch.equal(outs[0], v) for v in outs[1:])
-        _emit(config=3, world=W, elements_per_rank=n, nbits="dynamic{2,4,8}", method=name, u=u,
+        _emit(config=3, world=W, elements_per_rank=n, nbits="dynamic{2,4,8}", method=name, pipeline="grouped", u=u,
               avg_code_bits=float(qbits.float().mean()), nmse_vs_fp64_mean=_nmse(exact / W, outs[0]),
               ranks_identical=same, pipeline_total_ms=round(s.elapsed_time(e), 3))
         del outs, comps
+        # the same all-reduce with one codec launch per ring step for the three widths and no residual buffers
+        work = {}
+        strategy = 2 if name == "aee" else 3
+        for timed in (False, True):             # the first call allocates the stream buffers
+            s.record()
+            outs, _, counts = dynamic_bitrate_allreduce_single_pass(grads, u, strategy=strategy, seed=7, work=work)
+            e.record()
+            e.synchronize()
+        c = counts.tolist()
+        same = all(torch.equal(outs[0], v) for v in outs[1:])
+        _emit(config=3, world=W, elements_per_rank=n, nbits="dynamic{2,4,8}", method=name, pipeline="single_pass", u=u,
+              avg_code_bits=(8 * c[0] + 4 * c[1] + 2 * c[2]) / max(1, sum(c[:3])), nmse_vs_fp64_mean=_nmse(exact / W, outs[0]),
+              ranks_identical=same, pipeline_total_ms=round(s.elapsed_time(e), 3))
+        del outs, work
 
 
 LLAMA3_8B = [("embed", 128256 * 4096)] + [
