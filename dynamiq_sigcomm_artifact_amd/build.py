@@ -27,6 +27,7 @@ HIP_SOURCES = [
     "dq_scaling_tile16.hip",
     "dq_grouping.hip",
     "dq_scaling_mixed.hip",
+    "dq_rht_scaling.hip",
     "dq_superchunk.hip",
     "dq_hadamard.hip",
     "dq_packing.hip",

@@ -25,7 +25,7 @@ EXPORTS = [
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
-    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag",
+    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
     "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_thc_quantize", "dq_thc_dequantize",
 ]
@@ -97,6 +97,12 @@ def lib():
         L.dq_hadamard.argtypes = [vp, i64, i32, vp, i32]
         L.dq_rht_blocked.restype = i32
         L.dq_rht_blocked.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp]
+        L.dq_rht_scaling_compress.restype = i32
+        L.dq_rht_scaling_compress.argtypes = [vp, vp, i32, vp, vp, i32, i64, i64, f32, i32, i32, i32, u64, u64, vp]
+        L.dq_scaling_decompress_irht.restype = i32
+        L.dq_scaling_decompress_irht.argtypes = [vp, vp, i32, vp, i64, i64, f32, i32, i32, i32, vp]
+        L.dq_pack_signs.restype = i32
+        L.dq_pack_signs.argtypes = [vp, vp, i64, i32, vp]
         L.dq_rand_diag.restype = i32
         L.dq_rand_diag.argtypes = [vp, i64, i64, i32, vp]
         L.dq_bins_to_bits.restype = i32
@@ -292,6 +298,39 @@ def hadamard(vec, stream=None):
 def rht_blocked(vec, sign, block, scale, inverse=False, stream=None):
     _check(lib().dq_rht_blocked(vec.data_ptr(), 0 if sign is None else sign.data_ptr(), vec.numel(), block, float(scale),
                                 1 if inverse else 0, _dev(vec), _stream(stream)))
+
+
+def _packed(sign):
+    return 1 if sign is not None and sign.dtype == torch.int32 else 0
+
+
+def pack_signs(sign, stream=None):
+    """float32 +-1 vector -> int32 [ceil(n / 32)], bit e % 32 of word e / 32 set where sign[e] < 0"""
+    bits = torch.empty((sign.numel() + 31) // 32, dtype=torch.int32, device=sign.device)
+    _check(lib().dq_pack_signs(sign.data_ptr(), bits.data_ptr(), sign.numel(), _dev(sign), _stream(stream)))
+    return bits
+
+
+def rht_scaling_compress(src, sign, dst, block, scale, nbits, strategy, rand_pool=None, seed=0, step=0, stream=None):
+    """rht_blocked (forward) + scaling_compress of the rotated fp32 vector in one launch; src is not modified.
+    sign: None, float32 +-1 values, or the int32 bit vector of pack_signs.
+    rand_pool: float32 or bfloat16 [n], or None for the in-kernel rounding stream keyed by (seed, step, chunk)"""
+    if src.dtype != torch.float32:
+        raise RuntimeError("rht_scaling_compress: src must be float32")
+    code = 0
+    if rand_pool is not None:
+        code = dtype_code(rand_pool)
+    _check(lib().dq_rht_scaling_compress(src.data_ptr(), _ptr(sign), _packed(sign), dst.data_ptr(), _ptr(rand_pool), code, src.numel(),
+                                         block, float(scale), nbits, _dev(src), strategy, int(seed), int(step),
+                                         _stream(stream)))
+
+
+def scaling_decompress_irht(src, sign, dst, block, scale, nbits, strategy, stream=None):
+    """scaling_decompress into float32 + rht_blocked (inverse) in one launch"""
+    if dst.dtype != torch.float32:
+        raise RuntimeError("scaling_decompress_irht: dst must be float32")
+    _check(lib().dq_scaling_decompress_irht(src.data_ptr(), _ptr(sign), _packed(sign), dst.data_ptr(), dst.numel(), block, float(scale),
+                                            nbits, _dev(dst), strategy, _stream(stream)))
 
 
 def rand_diag(out, seed, stream=None):

@@ -511,6 +511,50 @@ int dq_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, floa
     return finish(dq::launch_rht_blocked(vec, sign, n, block, scale, inverse, static_cast<hipStream_t>(stream)));
 }
 
+static int check_rht_scaling(int64_t n, int64_t block, int nbits, int strategy)
+{
+    if (!(block > 0) || (block & (block - 1)) != 0) return fail(DQ_ERR_POW2, "block");
+    if (block > 32768) return fail(DQ_ERR_SIZE, "block must not exceed 32768 (one workgroup holds a whole transform block)");
+    if (!(n > 0) || n % block != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of block");
+    if (n % 256 != 0) return fail(DQ_ERR_N_SUPER);
+    if (nbits < 2 || nbits > 8) return fail(DQ_ERR_NBITS);
+    if (strategy != 2 && strategy != 3) return fail(DQ_ERR_STRATEGY);
+    return DQ_OK;
+}
+
+int dq_rht_scaling_compress(const float *src, const void *sign, int sign_packed, uint8_t *dst, const void *rand_pool, int rand_dtype,
+                            int64_t n, int64_t block, float scale, int nbits, int device, int strategy, uint64_t seed,
+                            uint64_t step, dq_stream_t stream)
+{
+    int rc = check_rht_scaling(n, block, nbits, strategy);
+    if (rc) return rc;
+    if (rand_pool && rand_dtype != DQ_F32 && rand_dtype != DQ_BF16) return fail(DQ_ERR_DTYPE);
+    if (!src || !dst) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_rht_compress(src, sign, sign_packed ? 1 : 0, dst, rand_pool, rand_pool ? rand_dtype : 3, n, block, scale, nbits,
+                                          strategy == 3, mee_params(nbits), seed, step, static_cast<hipStream_t>(stream)));
+}
+
+int dq_scaling_decompress_irht(const uint8_t *src, const void *sign, int sign_packed, float *dst, int64_t n, int64_t block, float scale,
+                               int nbits, int device, int strategy, dq_stream_t stream)
+{
+    int rc = check_rht_scaling(n, block, nbits, strategy);
+    if (rc) return rc;
+    if (!src || !dst) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_irht_decompress(src, sign, sign_packed ? 1 : 0, dst, n, block, scale, nbits, strategy == 3, mee_params(nbits),
+                                             static_cast<hipStream_t>(stream)));
+}
+
+int dq_pack_signs(const float *sign, uint32_t *bits, int64_t n, int device, dq_stream_t stream)
+{
+    if (!(n > 0)) return fail(DQ_ERR_N);
+    if (!sign || !bits) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_pack_signs(sign, bits, n, static_cast<hipStream_t>(stream)));
+}
+
 int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t stream)
 {
     if (!(size > 0)) return fail(DQ_ERR_N);

@@ -18,42 +18,10 @@
 // Inside the tile the stages are done four at a time (radix 16) on registers;
 // the LDS index is padded by one float per 16 (i + i/16), which keeps every
 // access pattern used here free of bank conflicts.
-#include "dq_device.cuh"
+#include "dq_fwht.cuh"
 #include "dq_launch.h"
 
 namespace dq {
-
-__device__ __forceinline__ int pad_idx(int i) { return i + (i >> 4); }
-
-template <int M> __device__ __forceinline__ void butterflies(float (&v)[1 << M])
-{
-#pragma unroll
-    for (int h = 1; h < (1 << M); h <<= 1) {
-#pragma unroll
-        for (int i = 0; i < (1 << M); i++) {
-            if ((i & h) == 0) {
-                float a = v[i], b = v[i + h];
-                v[i] = a + b;
-                v[i + h] = a - b;
-            }
-        }
-    }
-}
-
-// stages for index bits [p, p+M) of the tile
-template <int M> __device__ __forceinline__ void lds_pass(float *lds, int p, int ntuples, int tid, int nthreads)
-{
-    for (int u = tid; u < ntuples; u += nthreads) {
-        const int lo = u & ((1 << p) - 1);
-        const int base = ((u >> p) << (p + M)) | lo;
-        float v[1 << M];
-#pragma unroll
-        for (int j = 0; j < (1 << M); j++) v[j] = lds[pad_idx(base + (j << p))];
-        butterflies<M>(v);
-#pragma unroll
-        for (int j = 0; j < (1 << M); j++) lds[pad_idx(base + (j << p))] = v[j];
-    }
-}
 
 struct FwhtArgs {
     float *x;
@@ -119,17 +87,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
     __syncthreads();
 
     // butterfly stages, four index bits at a time
-    for (int p = a.b0; p < a.b1; p += 4) {
-        const int m = min(4, a.b1 - p);
-        const int ntuples = tile >> m;
-        switch (m) {
-        case 4: lds_pass<4>(lds, p, ntuples, tid, nthreads); break;
-        case 3: lds_pass<3>(lds, p, ntuples, tid, nthreads); break;
-        case 2: lds_pass<2>(lds, p, ntuples, tid, nthreads); break;
-        default: lds_pass<1>(lds, p, ntuples, tid, nthreads); break;
-        }
-        __syncthreads();
-    }
+    fwht_lds_stages(lds, a.kt, a.b0, a.b1, tid, nthreads);
 
     // store (coalesced), optional scale then sign flip
     if (a.vec) {
@@ -196,6 +154,7 @@ static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, fl
     if (kb <= kMaxTileBits) {
         // single pass; small blocks share a tile
         int kt = kb < kPrefTileBits ? kPrefTileBits : kb;
+        while (kt > kb && kt > 10 && (n >> kt) < 512) kt--; // short vectors: two workgroups per CU before larger tiles
         while (kt > kb && ((int64_t)1 << kt) > n) kt--;
         a.kt = kt; a.b0 = 0; a.b1 = kb; a.cbits = kt; a.sbits = kt;
         a.apply_scale = apply_scale; a.sign_mode = sign_fwd | sign_inv;
@@ -260,6 +219,22 @@ __global__ __launch_bounds__(256) void rand_diag_kernel(float *__restrict__ out,
         const int64_t idx = (int64_t)k * s8 + j;
         if (idx < size) out[idx] = ((r >> (4 * k)) & 15u) >= 8u ? 1.0f : -1.0f;
     }
+}
+
+// one bit per element of a +-1 vector, set where the value is negative; bit e % 32 of word e / 32
+__global__ __launch_bounds__(256) void pack_signs_kernel(const float *__restrict__ sign, uint32_t *__restrict__ bits, int64_t n)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool neg = e < n && sign[e] < 0.0f;
+    const uint64_t m = __builtin_amdgcn_ballot_w64(neg);
+    const int lane = threadIdx.x & 63;
+    if ((lane & 31) == 0 && e < n) bits[e >> 5] = (uint32_t)(m >> lane);
+}
+
+hipError_t launch_pack_signs(const float *sign, uint32_t *bits, int64_t n, hipStream_t stream)
+{
+    hipLaunchKernelGGL(pack_signs_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, sign, bits, n);
+    return hipGetLastError();
 }
 
 hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream)

@@ -126,6 +126,40 @@ __device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int6
     v.set(t);
 }
 
+// Quantise the wave's chunks (lane = chunk, 16 values in v, 16 uniform values in r; lanes of rows at or beyond
+// rows_here hold zeros) and stream the run of rows_here records to gout.  win_out: Rec<NBITS>::WIN bytes of LDS,
+// 16-byte aligned, owned by this wave.
+template <int NBITS, bool MEE, class RV, class RR>
+__device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const MeeArg<NBITS, MEE> &mp, uint8_t *gout,
+                                                 int rows_here, uint8_t *win_out)
+{
+    typedef Rec<NBITS> RC;
+    const int lane = threadIdx.x & 63;
+    const int row = lane >> 4, j = lane & 15;
+    const bool active = row < rows_here;
+    const int total = rows_here * RC::REC;
+
+    uint32_t w[RC::WORDS], q, ub;
+    const uint32_t amax = v.absmax_bits();
+    const bool lane_fast = amax <= kFastMaxBits && r.unit_interval();
+    if (__builtin_amdgcn_ballot_w64(!lane_fast) == 0)
+        chunk_encode_fast<NBITS, MEE>(v, r, amax, mp, w, q, ub);
+    else
+        chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
+
+    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
+    if (active) {
+        uint8_t *rec = win_out + mis + row * RC::REC;
+        chunk_write<NBITS>(rec + j * RC::CB, w, q);
+        if (j == 0) {
+            rec[16 * RC::CB] = (uint8_t)ub;
+            rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+        }
+    }
+    wave_lds_sync();
+    window_flush(win_out, gout, mis, total, lane);
+}
+
 // compress (FUSED = false) or decode-accumulate-recompress (FUSED = true) of tile `tile` of a run of nsc
 // records.  Record k of the packed streams (and row k of rnd) belongs to superchunk rows[k] of src
 // (to superchunk k when rows is null).  win_out / win_in: Rec<NBITS>::WIN bytes of LDS each, 16-byte
@@ -183,26 +217,7 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
         }
     }
 
-    uint32_t w[RC::WORDS], q, ub;
-    const uint32_t amax = v.absmax_bits();
-    const bool lane_fast = amax <= kFastMaxBits && r.unit_interval();
-    if (__builtin_amdgcn_ballot_w64(!lane_fast) == 0)
-        chunk_encode_fast<NBITS, MEE>(v, r, amax, mp, w, q, ub);
-    else
-        chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
-
-    uint8_t *gout = dst + sc0 * RC::REC;
-    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
-    if (active) {
-        uint8_t *rec = win_out + mis + row * RC::REC;
-        chunk_write<NBITS>(rec + j * RC::CB, w, q);
-        if (j == 0) {
-            rec[16 * RC::CB] = (uint8_t)ub;
-            rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
-        }
-    }
-    wave_lds_sync();
-    window_flush(win_out, gout, mis, total, lane);
+    encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, rows_here, win_out);
 }
 
 // Tile `tile` of a run of nsc records: record k decodes into superchunk rows[k] of dst (superchunk k when

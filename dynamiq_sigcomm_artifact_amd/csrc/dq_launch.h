@@ -88,6 +88,16 @@ hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t 
                               int inverse, hipStream_t stream);
 hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream);
 
+// blocked randomized Hadamard transform fused with the hierarchical chunk-16 quantiser (dq_rht_scaling.hip);
+// rand_kind: DQ_F32 or DQ_BF16 pool, or 3 for the in-kernel stream (rnd ignored)
+hipError_t launch_pack_signs(const float *sign, uint32_t *bits, int64_t n, hipStream_t stream);
+// sign: fp32 +-1 values, or with sign_bits one bit per element (launch_pack_signs); may be null
+hipError_t launch_rht_compress(const float *src, const void *sign, int sign_bits, uint8_t *dst, const void *rnd, int rand_kind,
+                               int64_t n, int64_t block, float scale, int nbits, bool mee, const MeeParams &mp,
+                               uint64_t seed, uint64_t step, hipStream_t stream);
+hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign_bits, float *dst, int64_t n, int64_t block,
+                                  float scale, int nbits, bool mee, const MeeParams &mp, hipStream_t stream);
+
 // EDEN Lloyd-Max quantiser + packer, THC uniform quantiser (dq_eden.hip)
 int64_t eden_work_doubles(int64_t n);
 hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,

@@ -131,6 +131,79 @@ torch::Tensor rht_blocked(torch::Tensor vec, c10::optional<torch::Tensor> sign, 
     return vec;
 }
 
+// sign for the fused transform + quantiser calls: float32 +-1 values or the int32 bit vector of pack_signs
+static const void *sign_arg(const c10::optional<torch::Tensor> &sign, const torch::Tensor &vec, int64_t n, int *packed)
+{
+    *packed = 0;
+    if (!sign.has_value()) return nullptr;
+    TORCH_CHECK(sign->device() == vec.device(), "sign must be on the same device as the vector");
+    TORCH_CHECK(sign->is_contiguous(), "sign must be contiguous");
+    if (sign->dtype() == torch::kInt32) {
+        TORCH_CHECK(sign->numel() >= (n + 31) / 32, "packed sign has fewer than n bits");
+        *packed = 1;
+    } else {
+        TORCH_CHECK(sign->dtype() == torch::kFloat32, "sign must be torch.float32 (+-1 values) or torch.int32 (packed bits)");
+        TORCH_CHECK(sign->numel() >= n, "sign has fewer elements than the vector");
+    }
+    return sign->data_ptr();
+}
+
+torch::Tensor pack_signs(torch::Tensor sign, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(sign.device().type() == torch::kCUDA && sign.dtype() == torch::kFloat32 && sign.is_contiguous(),
+                "sign must be a contiguous torch.float32 CUDA tensor");
+    TORCH_CHECK(sign.numel() > 0, "sign must not be empty");
+    auto bits = torch::empty({(sign.numel() + 31) / 32}, sign.options().dtype(torch::kInt32));
+    check_status(dq_pack_signs(sign.data_ptr<float>(), reinterpret_cast<uint32_t *>(bits.data_ptr<int32_t>()), sign.numel(),
+                               sign.device().index(), as_stream(stream_p)),
+                 "pack_signs");
+    return bits;
+}
+
+void rht_scaling_compress(torch::Tensor src, c10::optional<torch::Tensor> sign, torch::Tensor dst, int64_t block, double scale,
+                          int nbits, c10::optional<torch::Tensor> rand_pool, uint64_t seed = 0, uint64_t step = 0,
+                          uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA && src.dtype() == torch::kFloat32 && src.is_contiguous(),
+                "input must be a contiguous torch.float32 CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA && dst.dtype() == torch::kUInt8 && dst.is_contiguous(),
+                "output must be a contiguous torch.uint8 CUDA tensor");
+    const int64_t n = src.numel();
+    TORCH_CHECK(n > 0 && n % 256 == 0, "the element count must be a positive multiple of 256");
+    TORCH_CHECK(dst.numel() >= dq_scaling_required_bytes(n, nbits, 16, strategy), "output buffer is too small");
+    int packed = 0;
+    const void *sp = sign_arg(sign, src, n, &packed);
+    const void *rp = nullptr;
+    int rcode = DQ_F32;
+    if (rand_pool.has_value()) {
+        TORCH_CHECK(rand_pool->device() == src.device() && rand_pool->is_contiguous(), "rand_pool must be a contiguous tensor on the input's device");
+        TORCH_CHECK(rand_pool->dtype() == torch::kFloat32 || rand_pool->dtype() == torch::kBFloat16, "rand_pool must be torch.float32 or torch.bfloat16");
+        TORCH_CHECK(rand_pool->numel() >= n, "rand_pool has fewer elements than the input");
+        rcode = dq_dtype_of(rand_pool->scalar_type());
+        rp = rand_pool->data_ptr();
+    }
+    check_status(dq_rht_scaling_compress(src.data_ptr<float>(), sp, packed, dst.data_ptr<uint8_t>(), rp, rcode, n, block,
+                                         (float)scale, nbits, src.device().index(), strategy, seed, step, as_stream(stream_p)),
+                 "rht_scaling_compress");
+}
+
+void scaling_decompress_irht(torch::Tensor src, c10::optional<torch::Tensor> sign, torch::Tensor dst, int64_t block, double scale,
+                             int nbits, uint64_t stream_p = 0, int strategy = 2)
+{
+    TORCH_CHECK(src.device().type() == torch::kCUDA && src.dtype() == torch::kUInt8 && src.is_contiguous(),
+                "input must be a contiguous torch.uint8 CUDA tensor");
+    TORCH_CHECK(dst.device().type() == torch::kCUDA && dst.dtype() == torch::kFloat32 && dst.is_contiguous(),
+                "output must be a contiguous torch.float32 CUDA tensor");
+    const int64_t n = dst.numel();
+    TORCH_CHECK(n > 0 && n % 256 == 0, "the element count must be a positive multiple of 256");
+    TORCH_CHECK(src.numel() >= dq_scaling_required_bytes(n, nbits, 16, strategy), "input buffer is too small");
+    int packed = 0;
+    const void *sp = sign_arg(sign, dst, n, &packed);
+    check_status(dq_scaling_decompress_irht(src.data_ptr<uint8_t>(), sp, packed, dst.data_ptr<float>(), n, block, (float)scale,
+                                            nbits, dst.device().index(), strategy, as_stream(stream_p)),
+                 "scaling_decompress_irht");
+}
+
 torch::Tensor rand_diag(int64_t size, int64_t seed, torch::Device device, uint64_t stream_p = 0)
 {
     TORCH_CHECK(device.type() == torch::kCUDA, "device must be a CUDA device");
@@ -751,6 +824,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("scaling_dec_comp_ex", &scaling_dec_comp_ex, "scaling decompress and compress (also float32 buffers, 2..8-bit codes)", py::arg("recv"), py::arg("inp"), py::arg("send"), py::arg("rand_pool"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
     modul.def("scaling_required_bytes", &scaling_required_bytes, "packed size in bytes", py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("strategy"));
     modul.def("rht_blocked", &rht_blocked, "in-place blocked randomized Hadamard transform", py::arg("vec"), py::arg("sign"), py::arg("block"), py::arg("scale"), py::arg("inverse") = false, py::arg("stream_p") = 0);
+    modul.def("pack_signs", &pack_signs, "+-1 float32 vector -> int32 bit vector (bit set where negative)", py::arg("sign"), py::arg("stream_p") = 0);
+    modul.def("rht_scaling_compress", &rht_scaling_compress, "blocked randomized Hadamard transform + hierarchical chunk-16 compress in one launch (the rotated vector never reaches memory)", py::arg("src"), py::arg("sign"), py::arg("dst"), py::arg("block"), py::arg("scale"), py::arg("nbits"), py::arg("rand_pool") = py::none(), py::arg("seed") = 0, py::arg("step") = 0, py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("scaling_decompress_irht", &scaling_decompress_irht, "hierarchical chunk-16 decompress + inverse blocked randomized Hadamard transform in one launch", py::arg("src"), py::arg("sign"), py::arg("dst"), py::arg("block"), py::arg("scale"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("rand_diag", &rand_diag, "EDEN's seeded +-1 diagonal", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
     modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width; returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);

@@ -79,6 +79,7 @@ def config1(dev):
     rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
     sign = torch.empty(n, device=dev)
     capi.rand_diag(sign, 0)
+    sign_bits = capi.pack_signs(sign)
     for kb in (10, 11, 12, 13, 14, 15, 20):
         B = 1 << kb
         scale = 1.0 / math.sqrt(B)
@@ -95,8 +96,27 @@ def config1(dev):
             capi.scaling_compress(x, packed2, rand, n, nbits, 16, 2)
             capi.scaling_decompress(packed2, plain, n, nbits, 16, 2)
             t_rht = _time_us(lambda: capi.rht_blocked(y, sign, B, scale, False))
-            _emit(config=1, block=B, nbits=nbits, nmse_rht=_nmse(x, z), nmse_no_rht=_nmse(x, plain),
-                  rht_us=round(t_rht, 2), rht_GBps=round(8.0 * n / t_rht / 1e3, 1))
+            line = dict(config=1, block=B, nbits=nbits, nmse_rht=_nmse(x, z), nmse_no_rht=_nmse(x, plain),
+                        rht_us=round(t_rht, 2), rht_GBps=round(8.0 * n / t_rht / 1e3, 1))
+            if kb <= 15:
+                # the same round trip with the transform fused into the codec: same bytes, two launches instead of four
+                fused = torch.zeros_like(packed)
+                capi.rht_scaling_compress(x, sign_bits, fused, B, scale, nbits, 2, rand_pool=rand)
+                zf = torch.empty_like(x)
+                capi.scaling_decompress_irht(fused, sign_bits, zf, B, scale, nbits, 2)
+                t4 = _time_us(lambda: (capi.rht_blocked(y, sign, B, scale, False),
+                                       capi.scaling_compress(y, packed, rand, n, nbits, 16, 2),
+                                       capi.scaling_decompress(packed, z, n, nbits, 16, 2),
+                                       capi.rht_blocked(z, sign, B, scale, True)))
+                t2 = _time_us(lambda: (capi.rht_scaling_compress(x, sign_bits, fused, B, scale, nbits, 2, rand_pool=rand),
+                                       capi.scaling_decompress_irht(fused, sign_bits, zf, B, scale, nbits, 2)))
+                y2 = x.clone()
+                capi.rht_blocked(y2, sign, B, scale, False)
+                capi.scaling_compress(y2, packed, rand, n, nbits, 16, 2)
+                line.update(fused_bytes_equal=bool(torch.equal(fused, packed)), nmse_fused=_nmse(x, zf),
+                            roundtrip_4_launches_us=round(t4, 2), roundtrip_fused_us=round(t2, 2),
+                            roundtrip_fused_GBps_fp32_in=round(4.0 * n / t2 / 1e3, 1))
+            _emit(**line)
     # the reference-legal path for this configuration: EDEN (whole-vector rotation, Lloyd-Max bins, bit planes)
     from .eden import Eden
     eden = Eden(device=dev)
@@ -418,6 +438,32 @@ def config5(dev, n=1 << 30):
         t = _time_us(lambda: capi.rht_blocked(x, sign, B, 1.0, False), 2, 5)
         _emit(config=5, op="rht_blocked", block=B, us=round(t, 1), GBps=round(12.0 * n / t / 1e3, 1),
               frac_hbm=round(12.0 * n / t / 1e3 / HBM_PEAK, 4))
+    # the transform fused with the quantiser: the rotated vector never reaches memory (the in-place transforms
+    # above have changed x: draw it again)
+    x = torch.randn(n, generator=g, device=dev) * 1e-3
+    rand = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty_like(x)
+    sign_bits = capi.pack_signs(sign)
+    for kb, nbits in ((10, 4), (13, 2), (13, 4), (13, 5), (13, 8), (15, 4)):
+        B = 1 << kb
+        sc = 1.0 / math.sqrt(B)
+        packed = torch.zeros(capi.required_bytes(n, nbits, 16, 2), dtype=torch.uint8, device=dev)
+        tp = _time_us(lambda: capi.rht_scaling_compress(x, sign, packed, B, sc, nbits, 2, rand_pool=rand), 2, 5)
+        tx = _time_us(lambda: capi.rht_scaling_compress(x, sign, packed, B, sc, nbits, 2, seed=1, step=0), 2, 5)
+        td = _time_us(lambda: capi.scaling_decompress_irht(packed, sign, out, B, sc, nbits, 2), 2, 5)
+        tb = _time_us(lambda: capi.rht_scaling_compress(x, sign_bits, packed, B, sc, nbits, 2, seed=1, step=0), 2, 5)
+        tdb = _time_us(lambda: capi.scaling_decompress_irht(packed, sign_bits, out, B, sc, nbits, 2), 2, 5)
+        pb = (nbits + OV) / 8
+        _emit(config=5, op="rht+quantise fused", block=B, nbits=nbits, nmse=_nmse(x, out),
+              compress_pool_us=round(tp, 1), compress_philox_us=round(tx, 1), decompress_us=round(td, 1),
+              compress_pool_frac_hbm=round((4 + 4 + 2 + pb) * n / tp / 1e3 / HBM_PEAK, 4),
+              compress_philox_frac_hbm=round((4 + 4 + pb) * n / tx / 1e3 / HBM_PEAK, 4),
+              decompress_frac_hbm=round((4 + 4 + pb) * n / td / 1e3 / HBM_PEAK, 4),
+              packed_signs_compress_philox_us=round(tb, 1), packed_signs_decompress_us=round(tdb, 1),
+              packed_signs_compress_frac_hbm=round((4 + 0.125 + pb) * n / tb / 1e3 / HBM_PEAK, 4),
+              packed_signs_decompress_frac_hbm=round((4 + 0.125 + pb) * n / tdb / 1e3 / HBM_PEAK, 4),
+              roundtrip_GBps_fp32_in=round(4.0 * n / (tb + tdb) / 1e3, 1))
+        del packed
     t = _time_us(lambda: capi.hadamard(x), 1, 3)
     _emit(config=5, op="hadamard_whole_vector", n=n, us=round(t, 1))
 

@@ -311,6 +311,28 @@ int dq_hadamard(float *vec, int64_t n, int device, dq_stream_t stream, int depth
  * sign may be NULL (all +1).  n must be a multiple of block. */
 int dq_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale,
                    int inverse, int device, dq_stream_t stream);
+/* Extension: dq_rht_blocked (forward) followed by dq_scaling_compress of the
+ * rotated vector, without the rotated vector ever reaching memory -- a
+ * workgroup keeps whole transform blocks in LDS and quantises them there.  src
+ * (fp32 [n]) is not modified; dst receives the hierarchical chunk-16 records
+ * (strategy 2 or 3, nbits 2..8), byte for byte those of the two calls.
+ * block = 2^k <= 32768; n a multiple of block and of 256.  sign: NULL, fp32
+ * +-1 values [n] (sign_packed = 0), or one bit per element as written by
+ * dq_pack_signs (sign_packed = 1: 4 bytes less traffic per element).
+ * rand_pool: fp32 or bf16 [n] (rand_dtype DQ_F32 / DQ_BF16), or NULL for the
+ * in-kernel Philox stream of dq_scaling_compress_philox keyed by (seed, step,
+ * chunk). */
+int dq_rht_scaling_compress(const float *src, const void *sign, int sign_packed, uint8_t *dst,
+                            const void *rand_pool, int rand_dtype, int64_t n, int64_t block,
+                            float scale, int nbits, int device, int strategy, uint64_t seed,
+                            uint64_t step, dq_stream_t stream);
+/* the way back: dq_scaling_decompress into fp32 followed by dq_rht_blocked
+ * (inverse), the decoded vector staying in LDS. */
+int dq_scaling_decompress_irht(const uint8_t *src, const void *sign, int sign_packed, float *dst,
+                               int64_t n, int64_t block, float scale, int nbits, int device,
+                               int strategy, dq_stream_t stream);
+/* bits: uint32 [ceil(n / 32)]; bit e % 32 of word e / 32 is set where sign[e] < 0 */
+int dq_pack_signs(const float *sign, uint32_t *bits, int64_t n, int device, dq_stream_t stream);
 /* srrcomp.py:61-106 (SRRCompUtils.randDiag, torchRNG=False) computed on the
  * device: out[size] of +-1.0f. */
 int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t stream);

@@ -1,0 +1,140 @@
+"""The transform fused with the quantiser (dq_rht_scaling_compress, dq_scaling_decompress_irht) against the two-call
+sequences it replaces -- rht_blocked + scaling_compress, scaling_decompress + inverse rht_blocked -- byte for byte /
+bit for bit, and one case straight against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import F32, to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(n, generator=g) * 1e-3).to(DEV)
+    sign = (torch.randint(0, 2, (n,), generator=g).float() * 2 - 1).to(DEV)
+    return g, x, sign
+
+
+@pytest.mark.parametrize("block", [2, 64, 256, 1024, 4096, 8192, 16384, 32768])
+@pytest.mark.parametrize("nbits,strategy", [(2, 2), (4, 2), (5, 3), (8, 3), (8, 2)])
+def test_fused_equals_two_calls(capi, block, nbits, strategy):
+    # a vector that is not a whole number of 8192-element tiles, and at least two transform blocks
+    n = max(3 * 8192 + 2048 + 256, 2 * block)
+    n = (n + block - 1) // block * block
+    n = (n + 255) // 256 * 256
+    assert n % block == 0
+    g, x, sign = _case(n, block + nbits)
+    scale = 1.0 / np.sqrt(block)
+    nb = capi.required_bytes(n, nbits, 16, strategy)
+    for pool_dt in (torch.float32, torch.bfloat16, None):
+        rot = x.clone()
+        capi.rht_blocked(rot, sign, block, scale, False)
+        want = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+        if pool_dt is None:
+            capi.scaling_compress_philox(rot, want, n, nbits, 16, strategy, 11, 3)
+            pool = None
+        else:
+            pool = torch.rand(n, generator=g).to(pool_dt).to(DEV)
+            capi.scaling_compress(rot, want, pool, n, nbits, 16, strategy)
+        x_before = x.clone()
+        got = torch.full((nb + 32,), 0x5A, dtype=torch.uint8, device=DEV)
+        capi.rht_scaling_compress(x, sign, got, block, scale, nbits, strategy, rand_pool=pool, seed=11, step=3)
+        assert torch.equal(x, x_before)
+        assert torch.equal(got[:nb], want), (block, nbits, strategy, pool_dt)
+        assert bool((got[nb:] == 0x5A).all())
+    # the signs as one bit per element: same bytes (the last `want` is the in-kernel random stream's)
+    bits = capi.pack_signs(sign)
+    got = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+    capi.rht_scaling_compress(x, bits, got, block, scale, nbits, strategy, seed=11, step=3)
+    assert torch.equal(got, want)
+    # the way back
+    dec = torch.empty(n, dtype=torch.float32, device=DEV)
+    capi.scaling_decompress(want, dec, n, nbits, 16, strategy)
+    capi.rht_blocked(dec, sign, block, scale, True)
+    back = torch.full((n + 8,), 7.0, dtype=torch.float32, device=DEV)
+    capi.scaling_decompress_irht(want, sign, back[:n], block, scale, nbits, strategy)
+    assert torch.equal(back[:n].view(torch.int32), dec.view(torch.int32))
+    assert bool((back[n:] == 7.0).all())
+    back2 = torch.empty(n, dtype=torch.float32, device=DEV)
+    capi.scaling_decompress_irht(want, bits, back2, block, scale, nbits, strategy)
+    assert torch.equal(back2.view(torch.int32), dec.view(torch.int32))
+    err = float((back[:n] - x).pow(2).sum() / x.pow(2).sum())
+    assert err < {2: 1.0, 4: 0.05, 5: 0.02, 8: 2e-3}[nbits]
+
+
+@pytest.mark.parametrize("n,block", [(256, 256), (256, 16), (512, 512), (768, 256), (1280, 256), (2048, 1024)])
+def test_small_vectors_no_sign_unaligned(capi, n, block):
+    g, x, _ = _case(n, n + block)
+    pool = torch.rand(n, generator=g).to(DEV)
+    nb = capi.required_bytes(n, 4, 16, 2)
+    rot = x.clone()
+    capi.rht_blocked(rot, None, block, 0.5, False)
+    want = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(rot, want, pool, n, 4, 16, 2)
+    # source, pool and stream at addresses that are only element / byte aligned
+    xs = torch.zeros(n + 8, device=DEV)[1:1 + n].copy_(x)
+    ps = torch.zeros(n + 8, device=DEV)[3:3 + n].copy_(pool)
+    got = torch.zeros(nb + 16, dtype=torch.uint8, device=DEV)[7:7 + nb]
+    capi.rht_scaling_compress(xs, None, got, block, 0.5, 4, 2, rand_pool=ps)
+    assert torch.equal(got, want)
+    dec = torch.empty(n, device=DEV)
+    capi.scaling_decompress(want, dec, n, 4, 16, 2)
+    capi.rht_blocked(dec, None, block, 0.5, True)
+    back = torch.zeros(n + 8, device=DEV)[1:1 + n]
+    capi.scaling_decompress_irht(got, None, back, block, 0.5, 4, 2)
+    assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
+
+
+@pytest.mark.parametrize("n", [1, 31, 32, 33, 64, 255, 1000, 100003])
+def test_pack_signs(capi, n):
+    g = torch.Generator().manual_seed(n)
+    sign = (torch.randint(0, 2, (n,), generator=g).float() * 2 - 1)
+    bits = capi.pack_signs(sign.to(DEV)).cpu().numpy().view(np.uint32)
+    want = np.packbits((sign.numpy() < 0).astype(np.uint8), bitorder="little")
+    want = np.concatenate([want, np.zeros(-want.size % 4, np.uint8)]).view(np.uint32)
+    mask = np.full(want.size, 0xFFFFFFFF, np.uint32)
+    if n % 32:
+        mask[-1] = (1 << (n % 32)) - 1
+    assert ((bits & mask) == want).all()
+
+
+def test_fused_against_oracle(capi, oracle):
+    n, block, nbits, strategy = 8192 + 4096, 4096, 5, 3
+    g, x, sign = _case(n, 99)
+    pool = torch.rand(n, generator=g)
+    scale = np.float32(1.0 / np.sqrt(block))
+    got = torch.zeros(capi.required_bytes(n, nbits, 16, strategy), dtype=torch.uint8, device=DEV)
+    capi.rht_scaling_compress(x, sign, got, block, float(scale), nbits, strategy, rand_pool=pool.to(DEV))
+    rot = oracle.rht_blocked(x.cpu().numpy(), sign.cpu().numpy(), block, scale)
+    want = oracle.scaling_compress(rot, pool.numpy(), n, nbits, 16, strategy, F32)
+    assert (got.cpu().numpy() == want).all()
+    dec = np.zeros(n, np.float32)
+    oracle.scaling_decompress(want, dec, n, nbits, 16, strategy, F32)
+    back_o = oracle.rht_blocked(dec, sign.cpu().numpy(), block, scale, inverse=True)
+    back = torch.empty(n, device=DEV)
+    capi.scaling_decompress_irht(got, sign, back, block, float(scale), nbits, strategy)
+    assert (back.cpu().numpy().view(np.uint32) == back_o.view(np.uint32)).all()
+
+
+def test_fused_full_size_properties(capi):
+    """2^26 elements, block 2^15 (the largest tile): round trip error and the same bytes as the two calls on a slice"""
+    n, block, nbits = 1 << 26, 1 << 15, 4
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(n, generator=g, device=DEV) * 1e-3
+    sign = torch.empty(n, device=DEV)
+    capi.rand_diag(sign, 5)
+    scale = 1.0 / np.sqrt(block)
+    enc = torch.zeros(capi.required_bytes(n, nbits, 16, 2), dtype=torch.uint8, device=DEV)
+    capi.rht_scaling_compress(x, sign, enc, block, scale, nbits, 2, seed=1, step=2)
+    back = torch.empty_like(x)
+    capi.scaling_decompress_irht(enc, sign, back, block, scale, nbits, 2)
+    err = float((back - x).pow(2).sum() / x.pow(2).sum())
+    assert 0.005 < err < 0.03, err
+    rot = x.clone()
+    capi.rht_blocked(rot, sign, block, scale, False)
+    want = torch.zeros_like(enc)
+    capi.scaling_compress_philox(rot, want, n, nbits, 16, 2, 1, 2)
+    assert torch.equal(enc, want)

@@ -81,6 +81,7 @@ def test_argument_errors_are_reported_before_any_device_work():
         assert rc != 0
         assert text in L.dq_last_error().decode(), (L.dq_last_error().decode(), text)
 
+    Z = ctypes.c_uint64(0)
     err(L.dq_scaling_compress(P, P, P, 0, 4, 16, 1, 0, 2, S), "n must be positive")
     err(L.dq_scaling_compress(P, P, P, 256, 9, 16, 1, 0, 2, S), "nbits")
     err(L.dq_scaling_compress(P, P, P, 256, 4, 16, 7, 0, 2, S), "unsupported element dtype")
@@ -99,6 +100,18 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_rht_blocked(P, P, 1024, 48, ctypes.c_float(1.0), 0, 0, S), "block")
     err(L.dq_rht_blocked(P, P, 1000, 64, ctypes.c_float(1.0), 0, 0, S), "multiple of block")
     err(L.dq_rand_diag(P, 0, 1, 0, S), "n must be positive")
+    F1 = ctypes.c_float(1.0)
+    err(L.dq_rht_scaling_compress(P, P, 0, P, P, 2, 1024, 48, F1, 4, 0, 2, Z, Z, S), "power of 2")
+    err(L.dq_rht_scaling_compress(P, P, 0, P, P, 2, 1 << 17, 1 << 16, F1, 4, 0, 2, Z, Z, S), "32768")
+    err(L.dq_rht_scaling_compress(P, P, 0, P, P, 2, 1000, 8, F1, 4, 0, 2, Z, Z, S), "superchunk")          # n % 256
+    err(L.dq_rht_scaling_compress(P, P, 0, P, P, 2, 1024, 64, F1, 9, 0, 2, Z, Z, S), "nbits")
+    err(L.dq_rht_scaling_compress(P, P, 0, P, P, 2, 1024, 64, F1, 4, 0, 1, Z, Z, S), "strategy")
+    err(L.dq_rht_scaling_compress(P, P, 0, P, P, 0, 1024, 64, F1, 4, 0, 2, Z, Z, S), "unsupported element dtype")   # binary16 pool
+    err(L.dq_rht_scaling_compress(N, P, 0, P, P, 2, 1024, 64, F1, 4, 0, 2, Z, Z, S), "null pointer")
+    err(L.dq_scaling_decompress_irht(P, P, 1, N, 1024, 64, F1, 4, 0, 2, S), "null pointer")
+    err(L.dq_scaling_decompress_irht(P, P, 1, P, 1024, 96, F1, 4, 0, 2, S), "power of 2")
+    err(L.dq_pack_signs(P, N, 100, 0, S), "null pointer")
+    err(L.dq_pack_signs(P, P, 0, 0, S), "n must be positive")
     err(L.dq_bins_to_bits(P, 48, P, 6, 4, 0, S), "multiple of 32")
     err(L.dq_bits_to_bins(P, 64, P, 9, 4, 0, S), "narr")
     err(L.dq_quantization(N, 16, 0, ctypes.c_float(1.0), ctypes.c_float(1.0), 1, S), "null pointer")
@@ -109,7 +122,6 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 1, 0, 1, S), "strategy")
     err(L.dq_scaling_dec_comp_rows(P, P, P, P, P, 0, 4, 1, 0, 2, S), "n must be positive")
     err(L.dq_scaling_decompress_rows(P, P, P, P, 2560, 10, 4, 1, 0, 2, S, 1), "stats cannot be combined")
-    Z = ctypes.c_uint64(0)
     err(L.dq_mixed_compress(P, N, 1, 0, P, P, 0, 0, N, P, P, Z, Z, 100, 1, 0, 2, S), "world")           # ring_world 0
     err(L.dq_mixed_compress(P, N, 1, 0, P, P, 3, 3, N, P, P, Z, Z, 100, 1, 0, 2, S), "world")           # chunk outside the ring
     err(L.dq_mixed_compress(P, N, 1, 0, P, P, 0, 1, N, P, P, Z, Z, 100, 0, 0, 2, S), "unsupported element dtype")
