@@ -292,4 +292,23 @@ struct WorldDiv {
     __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
 };
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// LDS accesses of one wave execute in order; the fence only stops the compiler
+// from moving them across the hand-over between lanes
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// floor(log2(v)) for v >= 1
+inline int ilog2(int64_t v)
+{
+    int k = 0;
+    while (((int64_t)1 << (k + 1)) <= v) k++;
+    return k;
+}
+
 } // namespace dq

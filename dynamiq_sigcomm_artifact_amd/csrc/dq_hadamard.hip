@@ -115,13 +115,6 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
     }
 }
 
-static inline int ilog2(int64_t v)
-{
-    int k = 0;
-    while (((int64_t)1 << (k + 1)) <= v) k++;
-    return k;
-}
-
 static hipError_t launch_tile(const FwhtArgs &a, int64_t ntiles, hipStream_t stream)
 {
     const int tile = 1 << a.kt;

@@ -226,13 +226,6 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
     }
 }
 
-inline int ilog2(int64_t v)
-{
-    int k = 0;
-    while (((int64_t)1 << (k + 1)) <= v) k++;
-    return k;
-}
-
 constexpr int kPrefTileBits = 13; // 32 KiB tiles: eight waves, one run each, several workgroups per CU
 
 struct Geometry {
@@ -293,17 +286,6 @@ hipError_t run_decompress(const uint8_t *src, const void *sign, int sign_bits, f
     return hipGetLastError();
 }
 
-#define DQ_RHT_NBITS_MEE(FN, PRE, ...)                                                                     \
-    switch (nbits) {                                                                                      \
-    case 2: return mee ? FN<PRE, 2, true>(__VA_ARGS__) : FN<PRE, 2, false>(__VA_ARGS__);                  \
-    case 3: return mee ? FN<PRE, 3, true>(__VA_ARGS__) : FN<PRE, 3, false>(__VA_ARGS__);                  \
-    case 4: return mee ? FN<PRE, 4, true>(__VA_ARGS__) : FN<PRE, 4, false>(__VA_ARGS__);                  \
-    case 5: return mee ? FN<PRE, 5, true>(__VA_ARGS__) : FN<PRE, 5, false>(__VA_ARGS__);                  \
-    case 6: return mee ? FN<PRE, 6, true>(__VA_ARGS__) : FN<PRE, 6, false>(__VA_ARGS__);                  \
-    case 7: return mee ? FN<PRE, 7, true>(__VA_ARGS__) : FN<PRE, 7, false>(__VA_ARGS__);                  \
-    default: return mee ? FN<PRE, 8, true>(__VA_ARGS__) : FN<PRE, 8, false>(__VA_ARGS__);                 \
-    }
-
 } // namespace
 
 // rand_kind: DQ_F32 or DQ_BF16 pool, or DQ_PHILOX (rnd ignored)
@@ -313,18 +295,18 @@ hipError_t launch_rht_compress(const float *src, const void *sign, int sign_bits
 {
     const RandKey key{seed, step};
     if (rand_kind == DQ_PHILOX) {
-        DQ_RHT_NBITS_MEE(run_compress, DQ_PHILOX, src, sign, sign_bits, dst, nullptr, n, block, scale, mp, key, stream)
+        DQ_NBITS_MEE(run_compress, DQ_PHILOX, src, sign, sign_bits, dst, nullptr, n, block, scale, mp, key, stream)
     } else if (rand_kind == DQ_BF16) {
-        DQ_RHT_NBITS_MEE(run_compress, DQ_BF16, src, sign, sign_bits, dst, rnd, n, block, scale, mp, key, stream)
+        DQ_NBITS_MEE(run_compress, DQ_BF16, src, sign, sign_bits, dst, rnd, n, block, scale, mp, key, stream)
     } else {
-        DQ_RHT_NBITS_MEE(run_compress, DQ_F32, src, sign, sign_bits, dst, rnd, n, block, scale, mp, key, stream)
+        DQ_NBITS_MEE(run_compress, DQ_F32, src, sign, sign_bits, dst, rnd, n, block, scale, mp, key, stream)
     }
 }
 
 hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign_bits, float *dst, int64_t n, int64_t block, float scale,
                                   int nbits, bool mee, const MeeParams &mp, hipStream_t stream)
 {
-    DQ_RHT_NBITS_MEE(run_decompress, 0, src, sign, sign_bits, dst, n, block, scale, mp, stream)
+    DQ_NBITS_MEE(run_decompress, 0, src, sign, sign_bits, dst, n, block, scale, mp, stream)
 }
 
 } // namespace dq

@@ -107,18 +107,6 @@ static hipError_t run_decompress(const uint8_t *src, void *dst, const int32_t *r
     return hipGetLastError();
 }
 
-// FN<dtype..., NBITS, MEE>(args) for the runtime (nbits, mee)
-#define DQ_NBITS_MEE(FN, PRE, ...)                                                                        \
-    switch (nbits) {                                                                                      \
-    case 2: return mee ? FN<PRE, 2, true>(__VA_ARGS__) : FN<PRE, 2, false>(__VA_ARGS__);                  \
-    case 3: return mee ? FN<PRE, 3, true>(__VA_ARGS__) : FN<PRE, 3, false>(__VA_ARGS__);                  \
-    case 4: return mee ? FN<PRE, 4, true>(__VA_ARGS__) : FN<PRE, 4, false>(__VA_ARGS__);                  \
-    case 5: return mee ? FN<PRE, 5, true>(__VA_ARGS__) : FN<PRE, 5, false>(__VA_ARGS__);                  \
-    case 6: return mee ? FN<PRE, 6, true>(__VA_ARGS__) : FN<PRE, 6, false>(__VA_ARGS__);                  \
-    case 7: return mee ? FN<PRE, 7, true>(__VA_ARGS__) : FN<PRE, 7, false>(__VA_ARGS__);                  \
-    default: return mee ? FN<PRE, 8, true>(__VA_ARGS__) : FN<PRE, 8, false>(__VA_ARGS__);                 \
-    }
-
 #define DQ_COMMA ,
 
 static hipError_t dispatch_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd,

@@ -26,16 +26,6 @@ template <int CTRL> __device__ __forceinline__ float dpp_shift(float v)
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// LDS accesses of one wave execute in order; the fence only stops the compiler from moving them
-__device__ __forceinline__ void wave_lds_sync()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 template <int DT>
 __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__restrict__ src, void *__restrict__ residual,
                                                              uint32_t *__restrict__ stats, float *__restrict__ mean_out,

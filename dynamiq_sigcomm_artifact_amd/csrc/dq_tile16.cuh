@@ -201,8 +201,6 @@ template <> struct Raw16<DQ_PHILOX> {
 
 // ---- record windows --------------------------------------------------------------------
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
 // the (up to two) aligned 128-bit pieces of a packed run this lane moves
 struct WinRegs {
     u32x4 a, b;
@@ -244,15 +242,6 @@ __device__ __forceinline__ void window_flush(const uint8_t *win, uint8_t *g, int
     for (int v = lane; v < (body >> 4); v += 64) gv[v] = wv[v];
     const int tl = lane - 32; // lanes 32.. store the tail so head and tail overlap in time
     if (tl >= 0 && tl < tail) g[head + body + tl] = win[mis + head + body + tl];
-}
-
-// LDS accesses of one wave execute in order; the fence only stops the compiler
-// from moving them across the hand-over between lanes
-__device__ __forceinline__ void wave_lds_sync()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // ---- per-chunk code words -----------------------------------------------------------------
