@@ -409,6 +409,58 @@ def config4(dev, limit=None):
                   elements=elems * 256, u=u, achieved_avg_code_bits=bits / elems, achieved_bits_with_scales=bits / elems + OV,
                   nmse=num / den, output_checksum=check, ms_per_25MB_bucket=round(gpu_ms / len(timed), 4),
                   pipeline_GBps_of_bf16_input=round(2.0 * sum(m for _, m in timed) / (gpu_ms * 1e-3) / 1e9, 1))
+    config4_streams(dev, u)
+
+
+def config4_streams(dev, u, nbuckets=48, rounds=8):
+    """Back-to-back buckets with no host work between them.  The launches of `nbuckets` buckets are captured into one
+    graph per stream (each stream takes every k-th bucket; every capture is an ordinary single-stream one) and the
+    graphs are replayed side by side: with several streams the small launches of a bucket -- statistics, plan -- overlap
+    the codec launches of its neighbours."""
+    xs = [b.to(torch.bfloat16).clone() for b in _llama_buckets(dev, limit=nbuckets)]
+    keep = []                                   # graphs and streams stay alive until the function returns
+    for nstreams in (1, 2, 3, 4):
+        streams = [torch.cuda.Stream() for _ in range(nstreams)]
+        graphs = []
+        for k, st in enumerate(streams):
+            work, out = {}, [torch.empty_like(xs[0])]
+
+            def share():
+                for x in xs[k::nstreams]:
+                    dynamic_bitrate_allreduce_single_pass([x], u, strategy=2, seed=3, out=out, work=work)
+
+            with torch.cuda.stream(st):
+                share()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(st):
+                with torch.cuda.graph(g, stream=st):
+                    share()
+            graphs.append(g)
+            keep.append((g, st, work, out))
+        main = torch.cuda.current_stream()
+
+        def replay_all():
+            for g, st in zip(graphs, streams):
+                st.wait_stream(main)
+                with torch.cuda.stream(st):
+                    g.replay()
+            for st in streams:
+                main.wait_stream(st)
+
+        replay_all()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(rounds):
+            replay_all()
+        e.record()
+        e.synchronize()
+        per = s.elapsed_time(e) / (rounds * len(xs))
+        _emit(config=4, method="aee", pipeline="single_pass, %d buckets replayed as graphs" % len(xs), streams=nstreams,
+              rounds=rounds, ms_per_25MB_bucket=round(per, 4),
+              pipeline_GBps_of_bf16_input=round(2.0 * xs[0].numel() / (per * 1e-3) / 1e9, 1))
+    torch.cuda.synchronize()
 
 
 def config5(dev, n=1 << 30):
