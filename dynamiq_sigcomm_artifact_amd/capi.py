@@ -27,7 +27,7 @@ EXPORTS = [
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
-    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_thc_quantize", "dq_thc_dequantize",
+    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
 ]
 
 _lib = None
@@ -119,6 +119,10 @@ def lib():
         L.dq_thc_quantize.argtypes = [vp, vp, vp, i64, vp, vp, i32, i32, vp]
         L.dq_thc_dequantize.restype = i32
         L.dq_thc_dequantize.argtypes = [vp, vp, i64, vp, vp, i32, vp]
+        L.dq_thc_rht_quantize.restype = i32
+        L.dq_thc_rht_quantize.argtypes = [vp, vp, vp, vp, i64, i64, f32, vp, vp, i32, i32, vp]
+        L.dq_thc_dequantize_irht.restype = i32
+        L.dq_thc_dequantize_irht.argtypes = [vp, vp, vp, i64, i64, f32, vp, vp, i32, vp]
         L.dq_quantization.restype = i32
         L.dq_quantization.argtypes = [vp, i64, i32, f32, f32, u64, vp]
         _lib = L
@@ -398,3 +402,28 @@ def thc_dequantize(levels_in, out, step, lo, stream=None):
         raise RuntimeError("thc_dequantize: out is too small")
     _check(lib().dq_thc_dequantize(levels_in.data_ptr(), out.data_ptr(), n, step.data_ptr(), lo.data_ptr(), _dev(out),
                                    _stream(stream)))
+
+
+def thc_rht_quantize(work, sign, uniform, levels_out, block, scale, lo, delta, levels, stream=None):
+    """rht_blocked (forward) + thc_quantize in the transform's own passes; `work` holds the vector on entry and
+    intermediate values on return"""
+    if work.dtype != torch.float32 or uniform.dtype != torch.float32 or levels_out.dtype != torch.bfloat16 \
+            or lo.dtype != torch.float32 or delta.dtype != torch.float32:
+        raise RuntimeError("thc_rht_quantize: work, uniform, lo, delta must be float32 and the output bfloat16")
+    n = work.numel()
+    if uniform.numel() < n or levels_out.numel() < n or (sign is not None and sign.numel() < n):
+        raise RuntimeError("thc_rht_quantize: a buffer is too small")
+    _check(lib().dq_thc_rht_quantize(work.data_ptr(), _ptr(sign), uniform.data_ptr(), levels_out.data_ptr(), n, block,
+                                     float(scale), lo.data_ptr(), delta.data_ptr(), levels, _dev(work), _stream(stream)))
+
+
+def thc_dequantize_irht(levels_in, sign, out, block, scale, step, lo, stream=None):
+    """thc_dequantize + rht_blocked (inverse) in the transform's own passes"""
+    if levels_in.dtype != torch.bfloat16 or out.dtype != torch.float32 or step.dtype != torch.float32 \
+            or lo.dtype != torch.float32:
+        raise RuntimeError("thc_dequantize_irht: levels must be bfloat16, out, step, lo float32")
+    n = out.numel()
+    if levels_in.numel() < n or (sign is not None and sign.numel() < n):
+        raise RuntimeError("thc_dequantize_irht: a buffer is too small")
+    _check(lib().dq_thc_dequantize_irht(levels_in.data_ptr(), _ptr(sign), out.data_ptr(), n, block, float(scale),
+                                        step.data_ptr(), lo.data_ptr(), _dev(out), _stream(stream)))

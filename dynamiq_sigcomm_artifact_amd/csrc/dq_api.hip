@@ -627,6 +627,36 @@ int dq_thc_quantize(const float *rotated, const float *uniform, void *levels_bf1
     return finish(dq::launch_thc_quantize(rotated, uniform, levels_bf16, n, lo, delta, levels, static_cast<hipStream_t>(stream)));
 }
 
+static int check_thc_rht(int64_t n, int64_t block)
+{
+    if (!(block > 0) || (block & (block - 1)) != 0) return fail(DQ_ERR_POW2, "block");
+    if (!(n > 0) || n % block != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of block");
+    return DQ_OK;
+}
+
+int dq_thc_rht_quantize(float *work, const float *sign, const float *uniform, void *levels_bf16, int64_t n, int64_t block,
+                        float scale, const float *lo, const float *delta, int levels, int device, dq_stream_t stream)
+{
+    int rc = check_thc_rht(n, block);
+    if (rc) return rc;
+    if (levels < 2 || levels > 256) return fail(DQ_ERR_SIZE, "levels must be in [2, 256]");
+    if (!work || !uniform || !levels_bf16 || !lo || !delta) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_thc_rht_quantize(work, sign, uniform, levels_bf16, n, block, scale, lo, delta, levels,
+                                              static_cast<hipStream_t>(stream)));
+}
+
+int dq_thc_dequantize_irht(const void *levels_bf16, const float *sign, float *out, int64_t n, int64_t block, float scale,
+                           const float *step, const float *lo, int device, dq_stream_t stream)
+{
+    int rc = check_thc_rht(n, block);
+    if (rc) return rc;
+    if (!levels_bf16 || !out || !step || !lo) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_thc_dequantize_irht(levels_bf16, sign, out, n, block, scale, step, lo,
+                                                 static_cast<hipStream_t>(stream)));
+}
+
 int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const float *step, const float *lo, int device,
                       dq_stream_t stream)
 {

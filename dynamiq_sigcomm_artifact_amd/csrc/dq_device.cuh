@@ -292,6 +292,19 @@ struct WorldDiv {
     __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
 };
 
+// THC's uniform stochastic quantiser (testbed_evaluation/new_comm_hooks/thc_hooks.py:161-166):
+// x = clamp((v - lo) / delta, 0, levels - 1); level = floor(x) + (u < x - floor(x))
+__device__ __forceinline__ float thc_level(float v, float u, float lo, float delta, float top)
+{
+    float x = (v - lo) / delta;
+    // torch.clamp_ keeps NaN
+    if (x < 0.0f) x = 0.0f;
+    if (x > top) x = top;
+    const float fl = __builtin_floorf(x);
+    const float prob = x - fl;
+    return fl + ((u < prob) ? 1.0f : 0.0f);
+}
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // LDS accesses of one wave execute in order; the fence only stops the compiler

@@ -189,18 +189,6 @@ __global__ __launch_bounds__(256) void eden_dequantize_kernel(const uint32_t *__
 
 // ---- THC ------------------------------------------------------------------------------------------
 
-// x = clamp((v - lo) / delta, 0, levels - 1); level = floor(x) + (u < x - floor(x))
-__device__ __forceinline__ float thc_level(float v, float u, float lo, float delta, float top)
-{
-    float x = (v - lo) / delta;
-    // torch.clamp_ keeps NaN
-    if (x < 0.0f) x = 0.0f;
-    if (x > top) x = top;
-    const float fl = __builtin_floorf(x);
-    const float prob = x - fl;
-    return fl + ((u < prob) ? 1.0f : 0.0f);
-}
-
 // levels stored as bf16; VEC: four elements per thread through 16-byte loads and one 8-byte store
 template <bool VEC>
 __global__ __launch_bounds__(256) void thc_quantize_kernel(const float *__restrict__ rotated, const float *__restrict__ uniform,

@@ -35,6 +35,12 @@ struct FwhtArgs {
     int apply_scale;
     int sign_mode;     // 0 none, 1 multiply on load, 2 multiply on store
     int vec;           // 16-byte accesses allowed
+    // THC's quantiser folded into the two ends of a transform (all null / unused otherwise):
+    const uint16_t *in_levels; // the pass loads float(level) * *in_step + *in_lo instead of x
+    const float *in_step, *in_lo;
+    uint16_t *out_levels;      // the pass stores thc_level(value, uniform) as bf16 instead of the value
+    const float *uniform, *out_lo, *out_delta;
+    float out_top;
 };
 
 __global__ void fwht_tile_kernel(FwhtArgs a)
@@ -64,7 +70,15 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (g < a.n) {
-                v = *reinterpret_cast<const float4 *>(a.x + g);
+                if (a.in_levels) {
+                    const uint2 l = *reinterpret_cast<const uint2 *>(a.in_levels + g);
+                    const float step = *a.in_step, lo = *a.in_lo;
+                    const float p0 = bf16_bits_to_f32(l.x & 0xffffu) * step, p1 = bf16_bits_to_f32(l.x >> 16) * step;
+                    const float p2 = bf16_bits_to_f32(l.y & 0xffffu) * step, p3 = bf16_bits_to_f32(l.y >> 16) * step;
+                    v = make_float4(p0 + lo, p1 + lo, p2 + lo, p3 + lo);
+                } else {
+                    v = *reinterpret_cast<const float4 *>(a.x + g);
+                }
                 if (a.sign_mode == 1) {
                     const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
                     v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
@@ -78,7 +92,12 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
             float v = 0.0f;
             if (g < a.n) {
-                v = a.x[g];
+                if (a.in_levels) {
+                    const float prod = bf16_bits_to_f32(a.in_levels[g]) * *a.in_step;
+                    v = prod + *a.in_lo;
+                } else {
+                    v = a.x[g];
+                }
                 if (a.sign_mode == 1) v *= a.sign[g];
             }
             lds[pad_idx(i)] = v;
@@ -101,7 +120,16 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
                 const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
                 v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
             }
-            *reinterpret_cast<float4 *>(a.x + g) = v;
+            if (a.out_levels) {
+                const float4 u = *reinterpret_cast<const float4 *>(a.uniform + g);
+                const float lo = *a.out_lo, delta = *a.out_delta;
+                uint2 o;
+                o.x = f32x2_to_bf16x2(thc_level(v.x, u.x, lo, delta, a.out_top), thc_level(v.y, u.y, lo, delta, a.out_top));
+                o.y = f32x2_to_bf16x2(thc_level(v.z, u.z, lo, delta, a.out_top), thc_level(v.w, u.w, lo, delta, a.out_top));
+                *reinterpret_cast<uint2 *>(a.out_levels + g) = o;
+            } else {
+                *reinterpret_cast<float4 *>(a.x + g) = v;
+            }
         }
     } else {
         for (int i = tid; i < tile; i += nthreads) {
@@ -110,7 +138,10 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             float v = lds[pad_idx(i)];
             if (a.apply_scale) v *= a.scale;
             if (a.sign_mode == 2) v *= a.sign[g];
-            a.x[g] = v;
+            if (a.out_levels)
+                a.out_levels[g] = (uint16_t)f32_to_bf16_bits(thc_level(v, a.uniform[g], *a.out_lo, *a.out_delta, a.out_top));
+            else
+                a.x[g] = v;
         }
     }
 }
@@ -135,13 +166,28 @@ constexpr int kPrefTileBits = 13; // 32 KiB tiles keep several workgroups per CU
 constexpr int kStridedCols = 5;   // 32 consecutive floats (128 B) per row of a strided tile
 
 // transform index bits [0, kb) of every aligned block of 2^kb elements of x[0..n)
+// THC's quantiser at the ends of a transform: `in` replaces the load of the first pass, `out` the store of the last
+struct ThcEnds {
+    const uint16_t *in_levels = nullptr;
+    const float *in_step = nullptr, *in_lo = nullptr;
+    uint16_t *out_levels = nullptr;
+    const float *uniform = nullptr, *out_lo = nullptr, *out_delta = nullptr;
+    float out_top = 0.0f;
+};
+
 static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, float scale, int apply_scale,
-                              int inverse, hipStream_t stream)
+                              int inverse, hipStream_t stream, const ThcEnds &thc = ThcEnds())
 {
     const bool vec16 = (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-                       (sign == nullptr || (reinterpret_cast<uintptr_t>(sign) & 15) == 0);
+                       (sign == nullptr || (reinterpret_cast<uintptr_t>(sign) & 15) == 0) &&
+                       (reinterpret_cast<uintptr_t>(thc.in_levels) & 7) == 0 &&
+                       (reinterpret_cast<uintptr_t>(thc.out_levels) & 7) == 0 &&
+                       (reinterpret_cast<uintptr_t>(thc.uniform) & 15) == 0;
     FwhtArgs a;
     a.x = x; a.sign = sign; a.n = n; a.scale = scale;
+    a.in_levels = nullptr; a.in_step = thc.in_step; a.in_lo = thc.in_lo;
+    a.out_levels = nullptr; a.uniform = thc.uniform; a.out_lo = thc.out_lo; a.out_delta = thc.out_delta;
+    a.out_top = thc.out_top;
     const int sign_fwd = (sign && !inverse) ? 1 : 0, sign_inv = (sign && inverse) ? 2 : 0;
 
     if (kb <= kMaxTileBits) {
@@ -152,6 +198,8 @@ static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, fl
         a.kt = kt; a.b0 = 0; a.b1 = kb; a.cbits = kt; a.sbits = kt;
         a.apply_scale = apply_scale; a.sign_mode = sign_fwd | sign_inv;
         a.vec = vec16 && kt >= 2 && (n & 3) == 0;
+        a.in_levels = thc.in_levels;
+        a.out_levels = thc.out_levels;
         const int64_t ntiles = (n + ((int64_t)1 << kt) - 1) >> kt;
         return launch_tile(a, ntiles, stream);
     }
@@ -160,8 +208,10 @@ static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, fl
     int kt = kPrefTileBits;
     a.kt = kt; a.b0 = 0; a.b1 = kt; a.cbits = kt; a.sbits = kt;
     a.apply_scale = 0; a.sign_mode = sign_fwd; a.vec = vec16;
+    a.in_levels = thc.in_levels;
     hipError_t e = launch_tile(a, n >> kt, stream);
     if (e != hipSuccess) return e;
+    a.in_levels = nullptr;
     int s = kt;
     const int max_rows = kMaxTileBits - kStridedCols;
     while (s < kb) {
@@ -174,6 +224,7 @@ static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, fl
         const bool last = (s + r == kb);
         a.apply_scale = last ? apply_scale : 0;
         a.sign_mode = last ? sign_inv : 0;
+        a.out_levels = last ? thc.out_levels : nullptr;
         a.vec = vec16;
         e = launch_tile(a, n >> a.kt, stream);
         if (e != hipSuccess) return e;
@@ -191,6 +242,27 @@ hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t 
                               hipStream_t stream)
 {
     return fwht_blocks(vec, sign, n, ilog2(block), scale, 1, inverse, stream);
+}
+
+// rotate (forward) and quantise: vec is read and left holding intermediate values
+hipError_t launch_thc_rht_quantize(float *vec, const float *sign, const float *uniform, void *levels_out, int64_t n,
+                                   int64_t block, float scale, const float *lo, const float *delta, int levels,
+                                   hipStream_t stream)
+{
+    ThcEnds thc;
+    thc.out_levels = static_cast<uint16_t *>(levels_out);
+    thc.uniform = uniform; thc.out_lo = lo; thc.out_delta = delta; thc.out_top = (float)(levels - 1);
+    return fwht_blocks(vec, sign, n, ilog2(block), scale, 1, 0, stream, thc);
+}
+
+// dequantise and rotate back into out
+hipError_t launch_thc_dequantize_irht(const void *levels_in, const float *sign, float *out, int64_t n, int64_t block,
+                                      float scale, const float *step, const float *lo, hipStream_t stream)
+{
+    ThcEnds thc;
+    thc.in_levels = static_cast<const uint16_t *>(levels_in);
+    thc.in_step = step; thc.in_lo = lo;
+    return fwht_blocks(out, sign, n, ilog2(block), scale, 1, 1, stream, thc);
 }
 
 // ---- randDiag -----------------------------------------------------------------------

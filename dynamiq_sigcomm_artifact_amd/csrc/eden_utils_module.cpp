@@ -793,6 +793,48 @@ void thc_dequantize(torch::Tensor levels, torch::Tensor out, torch::Tensor step,
                  "thc_dequantize");
 }
 
+static const float *thc_sign_arg(const c10::optional<torch::Tensor> &sign, int64_t n)
+{
+    if (!sign.has_value()) return nullptr;
+    check_f32_cuda(*sign, "sign");
+    TORCH_CHECK(sign->numel() >= n, "sign has fewer elements than the vector");
+    return sign->data_ptr<float>();
+}
+
+void thc_rht_quantize(torch::Tensor work, c10::optional<torch::Tensor> sign, torch::Tensor uniform, torch::Tensor levels_out,
+                      int64_t block, double scale, torch::Tensor lo, torch::Tensor delta, int levels, uint64_t stream_p = 0)
+{
+    check_f32_cuda(work, "work");
+    check_f32_cuda(uniform, "uniform");
+    check_f32_cuda(lo, "lo");
+    check_f32_cuda(delta, "delta");
+    TORCH_CHECK(levels_out.device().type() == torch::kCUDA && levels_out.dtype() == torch::kBFloat16 && levels_out.is_contiguous(),
+                "levels_out must be a contiguous torch.bfloat16 CUDA tensor");
+    const int64_t n = work.numel();
+    TORCH_CHECK(uniform.numel() >= n && levels_out.numel() >= n, "uniform or levels_out has fewer elements than work");
+    TORCH_CHECK(lo.numel() == 1 && delta.numel() == 1, "lo and delta must hold one value");
+    check_status(dq_thc_rht_quantize(work.data_ptr<float>(), thc_sign_arg(sign, n), uniform.data_ptr<float>(), levels_out.data_ptr(), n,
+                                     block, (float)scale, lo.data_ptr<float>(), delta.data_ptr<float>(), levels,
+                                     work.device().index(), as_stream(stream_p)),
+                 "thc_rht_quantize");
+}
+
+void thc_dequantize_irht(torch::Tensor levels, c10::optional<torch::Tensor> sign, torch::Tensor out, int64_t block, double scale,
+                         torch::Tensor step, torch::Tensor lo, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(levels.device().type() == torch::kCUDA && levels.dtype() == torch::kBFloat16 && levels.is_contiguous(),
+                "levels must be a contiguous torch.bfloat16 CUDA tensor");
+    check_f32_cuda(out, "out");
+    check_f32_cuda(step, "step");
+    check_f32_cuda(lo, "lo");
+    const int64_t n = out.numel();
+    TORCH_CHECK(levels.numel() >= n, "levels has fewer elements than out");
+    TORCH_CHECK(step.numel() == 1 && lo.numel() == 1, "step and lo must hold one value");
+    check_status(dq_thc_dequantize_irht(levels.data_ptr(), thc_sign_arg(sign, n), out.data_ptr<float>(), n, block, (float)scale,
+                                        step.data_ptr<float>(), lo.data_ptr<float>(), out.device().index(), as_stream(stream_p)),
+                 "thc_dequantize_irht");
+}
+
 void init_lookup_table() { check_status(dq_init_lookup_table(), "init_lookup_table"); }
 
 std::string abi_version() { return dq_version(); }
@@ -845,5 +887,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("eden_dequantize", &eden_dequantize, "EDEN: centroids of the packed bins", py::arg("packed"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
     modul.def("thc_quantize", &thc_quantize, "THC: uniform stochastic quantiser of the rotated vector, bfloat16 levels", py::arg("rotated"), py::arg("uniform"), py::arg("lo"), py::arg("delta"), py::arg("levels"), py::arg("stream_p") = 0);
     modul.def("thc_dequantize", &thc_dequantize, "THC: out = float(levels) * step + lo", py::arg("levels"), py::arg("out"), py::arg("step"), py::arg("lo"), py::arg("stream_p") = 0);
+    modul.def("thc_rht_quantize", &thc_rht_quantize, "THC: blocked randomized Hadamard transform whose last pass stores the quantiser's levels (work is scratch afterwards)", py::arg("work"), py::arg("sign"), py::arg("uniform"), py::arg("levels_out"), py::arg("block"), py::arg("scale"), py::arg("lo"), py::arg("delta"), py::arg("levels"), py::arg("stream_p") = 0);
+    modul.def("thc_dequantize_irht", &thc_dequantize_irht, "THC: inverse transform whose first pass loads float(levels) * step + lo", py::arg("levels"), py::arg("sign"), py::arg("out"), py::arg("block"), py::arg("scale"), py::arg("step"), py::arg("lo"), py::arg("stream_p") = 0);
     modul.def("abi_version", &abi_version, "version string of libdynamiq_eden.so");
 }

@@ -156,6 +156,8 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         work["recv"] = [torch.zeros(cap, dtype=torch.uint8, device=dev) for _ in range(W if W > 1 else 0)]
     stats, mean, order, plan = work["stats"], work["mean"], work["order"], work["plan"]
     send, recv = work["send"], work["recv"]
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream     # looked up once per bucket, not once per launch
     for r in range(W):
         capi.superchunk_stats(rank_vecs[r], stats[r], mean[r], n, W, stream=stream)
     if W == 1:

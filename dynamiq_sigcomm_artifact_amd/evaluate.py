@@ -613,6 +613,27 @@ def kernels(dev, n=6553600):
     lo, delta = torch.tensor([-4.0], device=dev), torch.tensor([8.0 / 63], device=dev)
     line("thc_quantize", lambda: capi.thc_quantize(y, uni, lev, lo, delta, 64), 10 * d, n=d)
     line("thc_dequantize", lambda: capi.thc_dequantize(lev, y, delta, lo), 6 * d, n=d)
+    # THC end to end on the padded bucket: rotation and quantiser as separate calls and folded into the transform's passes
+    inv = 1.0 / math.sqrt(d)
+    line("thc: rht_blocked + thc_quantize", lambda: (capi.rht_blocked(y, sign, d, inv, False),
+                                                      capi.thc_quantize(y, uni, lev, lo, delta, 64)), 30 * d, n=d, launches=3)
+    line("thc_rht_quantize (folded)", lambda: capi.thc_rht_quantize(y, sign, uni, lev, d, inv, lo, delta, 64), 22 * d, n=d,
+         launches=2)
+    line("thc: thc_dequantize + inverse rht_blocked", lambda: (capi.thc_dequantize(lev, y, delta, lo),
+                                                                capi.rht_blocked(y, sign, d, inv, True)), 26 * d, n=d, launches=3)
+    line("thc_dequantize_irht (folded)", lambda: capi.thc_dequantize_irht(lev, sign, y, d, inv, delta, lo), 18 * d, n=d,
+         launches=2)
+    # the transform folded into the hierarchical codec (blocks of 2^13, 4-bit)
+    x32 = torch.randn(d, generator=g, device=dev) * 1e-3
+    sign_bits = capi.pack_signs(sign)
+    pk = torch.zeros(capi.required_bytes(d, 4, 16, 2), dtype=torch.uint8, device=dev)
+    pb = (4 + OV) / 8
+    line("rht_scaling_compress (packed signs, in-kernel rounding stream)",
+         lambda: capi.rht_scaling_compress(x32, sign_bits, pk, 8192, 1.0 / math.sqrt(8192), 4, 2, seed=1, step=0),
+         (4 + 0.125 + pb) * d, n=d, block=8192, nbits=4)
+    line("scaling_decompress_irht (packed signs)",
+         lambda: capi.scaling_decompress_irht(pk, sign_bits, x32, 8192, 1.0 / math.sqrt(8192), 4, 2),
+         (4 + 0.125 + pb) * d, n=d, block=8192, nbits=4)
     bins = torch.randint(0, 32, (d,), generator=g, device=dev, dtype=torch.int32)
     arr = torch.empty(d // 32 * 5, dtype=torch.int32, device=dev)
     line("EdenBinsToBits", lambda: capi.bins_to_bits(bins, arr, 5), 4 * d + d // 32 * 5 * 4, n=d, nbits=5)

@@ -4,11 +4,12 @@
 
 Same constructor parameters, same ``compress(tensor, name, max_norm)`` /
 ``decompress(tensor, name, max_norm=None)``; the element-wise chains of the reference
-become three launches each way:
+become the passes of one transform each way:
 
-  compress    rht (diagonal, Hadamard, 1/sqrt(d) in one pass for d <= 2^15) -> thc_quantize
-              (sub, div, clamp, floor, Bernoulli add, bf16 cast in one pass)
-  decompress  thc_dequantize (cast, mul, add) -> inverse rht
+  compress    thc_rht_quantize: diagonal and Hadamard, with 1/sqrt(d) and the quantiser (sub, div, clamp, floor,
+              Bernoulli add, bf16 cast) in the store of the last pass -- one pass in all for d <= 2^15
+  decompress  thc_dequantize_irht: the dequantiser (cast, mul, add) in the load of the first pass of the inverse
+              transform
 
 The Bernoulli draws come from ``torch.rand`` on the sender generator (the reference calls
 ``bernoulli_`` on the same generator; the two consume torch's stream differently, so the
@@ -132,14 +133,15 @@ class OldINCACudaHadamardCompressor:
         work[:orig_size].copy_(tensor.float())
         if dim > orig_size:
             work[orig_size:].zero_()
-        rotated = self.hadamards[name].rht(work)
         min_coordinate, delta = self._coordinate_range(max_norm, dim)
         if uniform is None:
             uniform = self._work_buffer(name, tag="uniform")
             uniform.uniform_(0.0, 1.0, generator=self.sender_prng)
         out = torch.empty(dim, dtype=torch.bfloat16, device=self.device)
-        capi.thc_quantize(rotated, uniform, out, min_coordinate.float().reshape(1), delta.float().reshape(1),
-                          self.quantization_levels)
+        # rotation and quantiser in the transform's own passes: the rotated vector is never stored
+        h = self.hadamards[name]
+        capi.thc_rht_quantize(work, h.random_diagonal, uniform, out, dim, h.inv_sqrt, min_coordinate.float().reshape(1),
+                              delta.float().reshape(1), self.quantization_levels)
         return out
 
     def decompress(self, tensor, name, max_norm=None):
@@ -149,6 +151,7 @@ class OldINCACudaHadamardCompressor:
         orig_size = self.original_size[name]
         min_coordinate, delta = self._coordinate_range(max_norm, dim)
         work = self._work_buffer(name)
-        capi.thc_dequantize(tensor, work, (delta / self.nclients).float().reshape(1), min_coordinate.float().reshape(1))
-        restored = self.hadamards[name].irht(work)
-        return restored[:orig_size]
+        h = self.hadamards[name]
+        capi.thc_dequantize_irht(tensor, h.random_diagonal, work, dim, h.inv_sqrt,
+                                 (delta / self.nclients).float().reshape(1), min_coordinate.float().reshape(1))
+        return work[:orig_size]

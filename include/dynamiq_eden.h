@@ -287,6 +287,21 @@ int dq_thc_quantize(const float *rotated, const float *uniform, void *levels_bf1
 int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const float *step,
                       const float *lo, int device, dq_stream_t stream);
 
+/* thc_hooks.py:95-100 + :161-166 in one call: the forward transform of
+ * dq_rht_blocked (sign flip, FWHT per block of `block` = 2^k, scale) whose last
+ * pass stores dq_thc_quantize's levels instead of the rotated values.  work
+ * (fp32 [n]) is the vector on entry and holds intermediate values on return
+ * (the reference's work buffer is scratch as well, thc_hooks.py:152-158). */
+int dq_thc_rht_quantize(float *work, const float *sign, const float *uniform, void *levels_bf16,
+                        int64_t n, int64_t block, float scale, const float *lo, const float *delta,
+                        int levels, int device, dq_stream_t stream);
+
+/* thc_hooks.py:176-181: dq_thc_dequantize folded into the first pass of the
+ * inverse transform of dq_rht_blocked; the result lands in out (fp32 [n]). */
+int dq_thc_dequantize_irht(const void *levels_bf16, const float *sign, float *out, int64_t n,
+                           int64_t block, float scale, const float *step, const float *lo,
+                           int device, dq_stream_t stream);
+
 /* ---- superchunk mean-centring ---------------------------------------- */
 
 /* csrc/cuda_hadamard.h:23-24 (superchunk_mean_center_with_cuda).  residual

@@ -212,3 +212,48 @@ def test_binding_functions(eden_utils, capi):
         eden_utils.eden_quantize(x[:100].contiguous(), bnd, cen, nbits)
     with pytest.raises(RuntimeError, match="boundaries must hold"):
         eden_utils.eden_quantize(x, bnd[:5].contiguous(), cen, nbits)
+
+
+@pytest.mark.parametrize("n,block", [(64, 64), (1024, 1024), (1024, 64), (1 << 15, 1 << 15), (1 << 16, 1 << 16),
+                                     (1 << 20, 1 << 20), (1 << 22, 1 << 22), (1 << 18, 1 << 12), (3 << 14, 1 << 14)])
+def test_thc_quantiser_folded_into_the_transform(capi, n, block):
+    """dq_thc_rht_quantize == rht_blocked + thc_quantize and dq_thc_dequantize_irht == thc_dequantize + inverse
+    rht_blocked, bit for bit, for single-pass and multi-pass transforms"""
+    g = torch.Generator().manual_seed(n + block)
+    x = (torch.randn(n, generator=g) * 1e-2).to(DEV)
+    sign = (torch.randint(0, 2, (n,), generator=g).float() * 2 - 1).to(DEV)
+    uni = torch.rand(n, generator=g).to(DEV)
+    scale = float(np.float32(1.0) / np.float32(np.sqrt(block)))
+    norm = float(x.norm())
+    T, levels = 2.5, 31
+    hi = T * norm / np.sqrt(n)
+    lo = torch.tensor([-hi], dtype=torch.float32, device=DEV)
+    delta = torch.tensor([2 * hi / (levels - 1) + 1e-23], dtype=torch.float32, device=DEV)
+    rot = x.clone()
+    capi.rht_blocked(rot, sign, block, scale, False)
+    want = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    capi.thc_quantize(rot, uni, want, lo, delta, levels)
+    work = x.clone()
+    got = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    capi.thc_rht_quantize(work, sign, uni, got, block, scale, lo, delta, levels)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert int(want.float().max()) <= levels - 1 and float(want.float().std()) > 1.0       # the quantiser did something
+    # the way back, as after a direct sum over 4 ranks
+    summed = (want.float() * 4).to(torch.bfloat16)
+    step = delta / 4
+    dec = torch.empty(n, device=DEV)
+    capi.thc_dequantize(summed, dec, step, lo)
+    capi.rht_blocked(dec, sign, block, scale, True)
+    back = torch.full((n,), 7.0, device=DEV)
+    capi.thc_dequantize_irht(summed, sign, back, block, scale, step, lo)
+    assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
+    # buffers that are only element-aligned take the scalar paths
+    if n <= 1 << 16:
+        w2 = torch.zeros(n + 4, device=DEV)[1:1 + n].copy_(x)
+        u2 = torch.zeros(n + 4, device=DEV)[3:3 + n].copy_(uni)
+        g2 = torch.zeros(n + 4, dtype=torch.bfloat16, device=DEV)[1:1 + n]
+        capi.thc_rht_quantize(w2, sign, u2, g2, block, scale, lo, delta, levels)
+        assert torch.equal(g2.view(torch.int16), want.view(torch.int16))
+        b2 = torch.zeros(n + 4, device=DEV)[1:1 + n]
+        capi.thc_dequantize_irht(g2 * 4, sign, b2, block, scale, step, lo)
+        assert torch.equal(b2.view(torch.int32), dec.view(torch.int32))

@@ -141,6 +141,12 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_eden_dequantize(P, 64, P, 9, P, 0, S), "nbits")
     err(L.dq_eden_dequantize(P, 64, P, 4, ctypes.c_void_p(0x1004), 0, S), "16-byte aligned")
     err(L.dq_thc_quantize(P, P, P, 64, P, P, 1, 0, S), "levels")
+    err(L.dq_thc_rht_quantize(P, P, P, P, 96, 48, F1, P, P, 31, 0, S), "power of 2")
+    err(L.dq_thc_rht_quantize(P, P, P, P, 100, 64, F1, P, P, 31, 0, S), "multiple of block")
+    err(L.dq_thc_rht_quantize(P, P, P, P, 64, 64, F1, P, P, 1, 0, S), "levels")
+    err(L.dq_thc_rht_quantize(P, P, N, P, 64, 64, F1, P, P, 31, 0, S), "null pointer")
+    err(L.dq_thc_dequantize_irht(P, P, N, 64, 64, F1, P, P, 0, S), "null pointer")
+    err(L.dq_thc_dequantize_irht(P, P, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
     assert capi.group_plan_work_ints(25600) == 4 + 4 * 25 and capi.eden_work_doubles(8192) == 2
     # a good call clears the message
