@@ -200,11 +200,12 @@ def group_plan_work_ints(nsc):
 
 
 def group_plan(qbits, order, work, stream=None):
-    """qbits int64 [nsc] -> order int32 [nsc] (8-bit rows, then 4-bit, then 2-bit), work[0:3] = counts"""
+    """qbits int64 [nsc] -> order int32 [3 * nsc]: the 8-bit rows from entry 0, the 4-bit rows from nsc, the 2-bit rows
+    from 2 * nsc (group_rows() slices them); work[0:3] = counts"""
     if qbits.dtype != torch.int64 or order.dtype != torch.int32 or work.dtype != torch.int32:
         raise RuntimeError("group_plan: qbits must be int64, order and work int32")
-    if order.numel() < qbits.numel():
-        raise RuntimeError("group_plan: order has fewer entries than qbits")
+    if order.numel() < 3 * qbits.numel():
+        raise RuntimeError("group_plan: order has fewer than 3 * nsc entries")
     _check(lib().dq_group_plan(qbits.data_ptr(), qbits.numel(), order.data_ptr(), work.data_ptr(), work.numel(),
                                _dev(qbits), _stream(stream)))
 
@@ -213,12 +214,18 @@ def _ptr(t):
     return 0 if t is None else t.data_ptr()
 
 
+def group_rows(order, nsc, width, count):
+    """the row list of one width in a planned `order` (a view)"""
+    base = {8: 0, 4: 1, 2: 2}[width] * nsc
+    return order[base:base + count]
+
+
 def group_plan_stats(stats, u, qbits_out, order, work, stream=None):
     """stats bf16 [nsc, 2] (mean, reduced sum of squares), offset u -> qbits_out (int64 or None), order, work"""
     if stats.dtype != torch.bfloat16 or order.dtype != torch.int32 or work.dtype != torch.int32:
         raise RuntimeError("group_plan_stats: stats must be bfloat16, order and work int32")
     nsc = stats.numel() // 2
-    if order.numel() < nsc or (qbits_out is not None and (qbits_out.dtype != torch.int64 or qbits_out.numel() < nsc)):
+    if order.numel() < 3 * nsc or (qbits_out is not None and (qbits_out.dtype != torch.int64 or qbits_out.numel() < nsc)):
         raise RuntimeError("group_plan_stats: order / qbits_out too small or of the wrong dtype")
     _check(lib().dq_group_plan_stats(stats.data_ptr(), float(u), nsc, _ptr(qbits_out), order.data_ptr(), work.data_ptr(),
                                      work.numel(), _dev(stats), _stream(stream)))

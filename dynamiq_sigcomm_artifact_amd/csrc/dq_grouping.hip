@@ -1,13 +1,25 @@
 // Stable partition of the superchunks of a bucket by their bit width: what three
 // torch.nonzero(qbits == w) calls produce in the reference
-// (testbed_evaluation/new_comm_hooks/comm_hooks.py:964-966), as two launches and no
-// host synchronisation.
+// (testbed_evaluation/new_comm_hooks/comm_hooks.py:964-966), without host synchronisation.
 //
-//   order[0 .. n8)            indices i with qbits[i] == 8, ascending
-//   order[n8 .. n8+n4)        indices with qbits[i] == 4, ascending
-//   order[n8+n4 .. n8+n4+n2)  indices with qbits[i] == 2, ascending
+//   order[0 .. n8)                 indices i with qbits[i] == 8, ascending
+//   order[nsc .. nsc + n4)         indices with qbits[i] == 4, ascending
+//   order[2 nsc .. 2 nsc + n2)     indices with qbits[i] == 2, ascending
 //   work[0..2] = n8, n4, n2;  work[3] = superchunks of any other width (in no group)
-//   work[4 + 4*b + w]         per-tile counts (tile b = superchunks [1024 b, 1024 b + 1024))
+//   work[8 ...]                    per-tile counts of the two-launch path (tile b = superchunks
+//                                  [1024 b, 1024 b + 1024))
+//
+// Every group has a region of its own, so where an index goes depends only on the superchunks before it.
+// Buckets of up to 65536 superchunks (64 tiles) take ONE launch: the workgroup of tile b counts the
+// classes of all tiles before it itself (at most 63 K superchunks, eight coalesced loads in flight per
+// thread: cheaper than a second launch, and nothing waits on another workgroup), scans its own tile and places it; the
+// workgroup of the last tile also writes the group sizes.  What makes the recount cheap is that the width
+// is a monotone step function of the bf16 norm pattern (every operation of the rule is monotone, and
+// neighbouring bf16 values are 2^-8 apart, far more than the error of the log2 polynomial): two waves
+// first find the two patterns at which the width becomes 4 and 8 by a 64-way search with the exact rule,
+// and a superchunk is then classified by two integer compares.
+// Longer vectors take two launches: count per tile, then every tile sums the counts of the tiles before it
+// and places its indices.
 #include "dq_launch.h"
 
 namespace dq {
@@ -39,20 +51,141 @@ __device__ __forceinline__ int64_t qbits_of_norm(uint32_t norm_bits, float u)
     return (int64_t)1 << z;
 }
 
-// where the widths come from: an int64 array, or the norm column of the interleaved bf16 stats
+constexpr int kMaxPattern = 0x7f80; // +infinity: the patterns 0 .. 0x7f80 are the non-negative norms in ascending order
+
+// where the widths come from: an int64 array, or the norm column of the interleaved bf16 stats.
+//   operator()(i)           the width of superchunk i by the rule itself (two-launch path)
+//   prepare / load / cls    the one-launch path: prepare() fills thr[2] (no barrier inside), load() only
+//                           loads, cls() turns a loaded value into the class 0 (8 bits) .. 3 (no group)
 struct WidthsFromArray {
     const int64_t *qbits;
+    typedef int64_t Raw;
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
+    bool word_aligned() const { return true; }
+    __device__ __forceinline__ void prepare(int *, int, int) const {}
+    __device__ __forceinline__ Raw load(int i) const { return qbits[i]; }
+    __device__ __forceinline__ int cls(Raw q, const int *) const { return width_class(q); }
 };
+
 struct WidthsFromStats {
     const uint16_t *stats;
     float u;
+    typedef uint32_t Raw; // a (mean, norm) pair: the norm pattern is the high half
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits_of_norm(stats[2 * i + 1], u); }
+    // index of the first of 64 probes lo + step * (l + 1) (clamped to kMaxPattern) whose width is >= target; 64 if none
+    __device__ __forceinline__ int first_probe(int lo, int step, int lane, int64_t target) const
+    {
+        const int p = min(lo + step * (lane + 1), kMaxPattern);
+        const uint64_t hit = __builtin_amdgcn_ballot_w64(qbits_of_norm((uint32_t)p, u) >= target);
+        return hit ? __builtin_ctzll(hit) : 64;
+    }
+    // wave 0 finds thr[0] = the smallest pattern of width >= 4, wave 1 thr[1] = that of width 8
+    // (kMaxPattern + 1 when no pattern reaches it)
+    __device__ __forceinline__ void prepare(int *thr, int wave, int lane) const
+    {
+        if (wave > 1) return;
+        const int64_t target = wave == 0 ? 4 : 8;
+        int t = kMaxPattern + 1;
+        const int a = first_probe(-1, 512, lane, target);
+        if (a < 64) {
+            const int lo = -1 + 512 * a;
+            const int b = first_probe(lo, 8, lane, target);
+            const int lo2 = lo + 8 * b;
+            t = lo2 + 1 + first_probe(lo2, 1, lane, target);
+        }
+        if (lane == 0) thr[wave] = t;
+    }
+    bool word_aligned() const { return (reinterpret_cast<uintptr_t>(stats) & 3) == 0; } // load() reads pairs as one word
+    __device__ __forceinline__ Raw load(int i) const { return reinterpret_cast<const uint32_t *>(stats)[i]; }
+    __device__ __forceinline__ int cls(Raw pair, const int *thr) const
+    {
+        const uint32_t r = pair >> 16;
+        if (r <= (uint32_t)kMaxPattern) return (int)r >= thr[1] ? 0 : ((int)r >= thr[0] ? 1 : 2);
+        return width_class(qbits_of_norm(r, u)); // negative or NaN norms: the rule itself
+    }
 };
 
 // three 21-bit counters in one word
 __device__ __forceinline__ uint64_t one_of(int cls) { return cls < 3 ? (uint64_t)1 << (21 * cls) : 0; }
 __device__ __forceinline__ int field(uint64_t p, int cls) { return (int)((p >> (21 * cls)) & 0x1fffff); }
+
+// ---- one launch (up to 64 tiles) ----------------------------------------------------------------------
+
+constexpr int kOneThreads = kTile; // one superchunk per thread while placing
+constexpr int kOneMaxTiles = 64;
+constexpr int kOneBatch = 8;       // loads in flight per thread while recounting the tiles before
+
+template <class W>
+__global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t *__restrict__ qbits_out, int nsc,
+                                                              int32_t *__restrict__ order, int32_t *__restrict__ work)
+{
+    __shared__ int thr[2];
+    __shared__ uint64_t before_sum[kOneThreads / 64], scan_sum[kOneThreads / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nbefore = (int)blockIdx.x * kTile; // superchunks of the tiles before this one
+    const int own = nbefore + (int)threadIdx.x;
+
+    // this tile's load and the first batch of the recount are in flight while the thresholds are searched
+    typename W::Raw own_raw = typename W::Raw();
+    if (own < nsc) own_raw = widths.load(own);
+    uint64_t mine = 0;
+    bool ready = false;
+    for (int i0 = 0; i0 < nbefore; i0 += kOneBatch * kOneThreads) {
+        typename W::Raw raw[kOneBatch];
+#pragma unroll
+        for (int j = 0; j < kOneBatch; j++) {
+            const int i = i0 + j * kOneThreads + (int)threadIdx.x;
+            if (i < nbefore) raw[j] = widths.load(i);
+        }
+        if (!ready) {
+            widths.prepare(thr, wave, lane);
+            __syncthreads();
+            ready = true;
+        }
+#pragma unroll
+        for (int j = 0; j < kOneBatch; j++) {
+            const int i = i0 + j * kOneThreads + (int)threadIdx.x;
+            if (i < nbefore) mine += one_of(widths.cls(raw[j], thr));
+        }
+    }
+    if (!ready) {
+        widths.prepare(thr, wave, lane);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mine += __shfl_xor(mine, d, 64);
+
+    // this tile: class of the thread's superchunk, inclusive scan over the wave
+    const int c = own < nsc ? widths.cls(own_raw, thr) : 3;
+    if (qbits_out && own < nsc) qbits_out[own] = c == 0 ? 8 : (c == 1 ? 4 : (c == 2 ? 2 : (int64_t)widths(own)));
+    const uint64_t cnt = one_of(c);
+    uint64_t incl = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint64_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 0) before_sum[wave] = mine;
+    if (lane == 63) scan_sum[wave] = incl;
+    __syncthreads();
+    uint64_t before = 0, excl = incl - cnt, tile_all = 0;
+#pragma unroll
+    for (int k = 0; k < kOneThreads / 64; k++) {
+        before += before_sum[k];
+        if (k < wave) excl += scan_sum[k];
+        tile_all += scan_sum[k];
+    }
+    if (c < 3) order[(int64_t)c * nsc + field(before, c) + field(excl, c)] = own;
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        const uint64_t all = before + tile_all;
+        work[0] = field(all, 0);
+        work[1] = field(all, 1);
+        work[2] = field(all, 2);
+        work[3] = nsc - field(all, 0) - field(all, 1) - field(all, 2);
+    }
+}
+
+// ---- two launches (any length) ------------------------------------------------------------------------
 
 template <class W>
 __global__ __launch_bounds__(kThreads) void plan_count_kernel(W widths, int64_t nsc, int32_t *__restrict__ work)
@@ -71,7 +204,7 @@ __global__ __launch_bounds__(kThreads) void plan_count_kernel(W widths, int64_t 
         if (c[w]) atomicAdd(&cnt[w], c[w]);
     }
     __syncthreads();
-    if (threadIdx.x < 4) work[4 + 4 * blockIdx.x + threadIdx.x] = cnt[threadIdx.x];
+    if (threadIdx.x < 4) work[8 + 4 * blockIdx.x + threadIdx.x] = cnt[threadIdx.x];
 }
 
 template <class W>
@@ -91,7 +224,7 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
         for (int tile = threadIdx.x; tile < ntiles; tile += kThreads) {
 #pragma unroll
             for (int w = 0; w < 4; w++) {
-                const int c = work[4 + 4 * tile + w];
+                const int c = work[8 + 4 * tile + w];
                 t[w] += c;
                 if (tile < (int)blockIdx.x) b[w] += c;
             }
@@ -131,10 +264,9 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
     uint64_t excl = incl - mine;
     for (int w = 0; w < wave; w++) excl += wave_sum[w];
 
-    const int group_base[3] = {0, total[0], total[0] + total[1]};
-    int pos[3];
+    int64_t pos[3];
 #pragma unroll
-    for (int w = 0; w < 3; w++) pos[w] = group_base[w] + before[w] + field(excl, w);
+    for (int w = 0; w < 3; w++) pos[w] = (int64_t)w * nsc + before[w] + field(excl, w);
 #pragma unroll
     for (int k = 0; k < kPer; k++) {
 #pragma unroll
@@ -146,12 +278,17 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
 
 } // namespace
 
-int64_t group_plan_work_ints(int64_t nsc) { return 4 + 4 * ((nsc + kTile - 1) / kTile); }
+int64_t group_plan_work_ints(int64_t nsc) { return 8 + 4 * ((nsc + kTile - 1) / kTile); }
 
 template <class W>
 static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *order, int32_t *work, hipStream_t stream)
 {
     const int ntiles = (int)((nsc + kTile - 1) / kTile);
+    if (ntiles <= kOneMaxTiles && widths.word_aligned()) {
+        hipLaunchKernelGGL(plan_one_kernel<W>, dim3(ntiles), dim3(kOneThreads), 0, stream, widths, qbits_out, (int)nsc, order,
+                           work);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(plan_count_kernel<W>, dim3(ntiles), dim3(kThreads), 0, stream, widths, nsc, work);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

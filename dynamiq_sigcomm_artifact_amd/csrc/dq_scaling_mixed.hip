@@ -14,8 +14,9 @@
 // The record formats are those of the single-width kernels, so each of the three runs is byte for byte
 // what dq_scaling_compress_rows writes for the same superchunks and random values.
 //
-// Rounding randomness: row k of rand_pool (256 values) belongs to position k of `order`; the in-kernel
-// stream is keyed by the chunk's index in the source vector.
+// Rounding randomness: row k of rand_pool (256 values) belongs to the k-th superchunk of the concatenation
+// 8-bit group | 4-bit group | 2-bit group; the in-kernel stream is keyed by the chunk's index in the source
+// vector.
 #include "dq_hier16_tiles.cuh"
 #include "dq_launch.h"
 
@@ -24,16 +25,18 @@ namespace dq {
 namespace {
 
 struct MixedPlan {
-    const int32_t *order;  // superchunk indices, grouped 8 | 4 | 2
+    const int32_t *order;  // superchunk indices: the 8-bit group from entry 0, the 4-bit group from nsc, the 2-bit group from 2 nsc
     const int32_t *counts; // n8, n4, n2
     int chunk, world;
+    int nsc;               // the counts are clamped so that their sum cannot exceed it
 };
 
 struct Segment {
     int cls;          // 0: 8-bit, 1: 4-bit, 2: 2-bit, 3: nothing to do
     int tile;         // tile inside the run
     int cnt;          // records in the run
-    int64_t pos0;     // position in `order` of the run's first record
+    int64_t row0;     // entry of `order` holding the run's first superchunk
+    int64_t pos0;     // rank of that superchunk in the concatenation 8 | 4 | 2 (row of the random pool)
     int64_t byte_off; // where the run starts in the packed stream
 };
 
@@ -41,18 +44,18 @@ __device__ __forceinline__ Segment locate(const MixedPlan &p, int block)
 {
     constexpr int kRec[3] = {Rec<8>::REC, Rec<4>::REC, Rec<2>::REC};
     Segment s;
-    s.cls = 3; s.tile = 0; s.cnt = 0; s.pos0 = 0; s.byte_off = 0;
+    s.cls = 3; s.tile = 0; s.cnt = 0; s.row0 = 0; s.pos0 = 0; s.byte_off = 0;
     int64_t pos = 0, off = 0;
     int t = block;
 #pragma unroll
     for (int g = 0; g < 3; g++) {
-        const int n = p.counts[g];
+        const int n = min(max(p.counts[g], 0), p.nsc - (int)pos); // a corrupt count cannot lead outside a region or the pool
         const int per = (n + p.world - 1) / p.world;
         const int begin = (int)min((int64_t)per * p.chunk, (int64_t)n);
         const int cnt = min(per, n - begin);
         const int tiles = (cnt + kRowsPerWave - 1) / kRowsPerWave;
         if (s.cls == 3 && t < tiles) {
-            s.cls = g; s.tile = t; s.cnt = cnt; s.pos0 = pos + begin; s.byte_off = off;
+            s.cls = g; s.tile = t; s.cnt = cnt; s.row0 = (int64_t)g * p.nsc + begin; s.pos0 = pos + begin; s.byte_off = off;
         }
         t -= tiles;
         pos += n;
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restri
 
     const Segment s = locate(plan, blockIdx.x);
     if (s.cls == 3) return;
-    const int32_t *rows = plan.order + s.pos0;
+    const int32_t *rows = plan.order + s.row0;
     const void *r = RDT == DQ_PHILOX ? nullptr : static_cast<const char *>(rnd) + s.pos0 * 256 * RESZ;
     const uint8_t *in = FUSED ? recv + s.byte_off : nullptr;
     uint8_t *out = dst + s.byte_off;
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(64) void mixed_decompress_kernel(const uint8_t *__r
 
     const Segment s = locate(plan, blockIdx.x);
     if (s.cls == 3) return;
-    const int32_t *rows = plan.order + s.pos0;
+    const int32_t *rows = plan.order + s.row0;
     const uint8_t *in = src + s.byte_off;
     switch (s.cls) {
     case 0:
@@ -162,7 +165,7 @@ hipError_t launch_mixed_compress(const void *src, const float *center_mean, int 
                                  const uint8_t *recv, uint8_t *dst, const void *rnd, const RandKey *philox, int64_t nsc,
                                  int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
 {
-    const MixedPlan plan{order, counts, ring_chunk, ring_world};
+    const MixedPlan plan{order, counts, ring_chunk, ring_world, (int)nsc};
     Center ctr;
     ctr.mean = center_mean;
     ctr.n_valid = n_valid;
@@ -189,7 +192,7 @@ hipError_t launch_mixed_decompress(const uint8_t *src, void *dst, const int32_t 
                                    int ring_chunk, int ring_world, const void *stats, int64_t limit, int64_t nsc,
                                    int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
 {
-    const MixedPlan plan{order, counts, ring_chunk, ring_world};
+    const MixedPlan plan{order, counts, ring_chunk, ring_world, (int)nsc};
     const uint16_t *st = static_cast<const uint16_t *>(stats);
     if ((dtype & 0xf) == DQ_BF16)
         return mee ? run_decompress<DQ_BF16, true>(src, dst, plan, nsc, st, limit, mp, stream)

@@ -352,7 +352,7 @@ torch::Tensor group_plan(torch::Tensor qbits, torch::Tensor order, uint64_t stre
     TORCH_CHECK(qbits.is_contiguous() && order.is_contiguous(), "qbits and order must be contiguous");
     const int64_t nsc = qbits.numel();
     TORCH_CHECK(nsc > 0, "qbits must not be empty");
-    TORCH_CHECK(order.numel() >= nsc, "order has fewer entries than qbits");
+    TORCH_CHECK(order.numel() >= 3 * nsc, "order has fewer than 3 * nsc entries");
     auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
     check_status(dq_group_plan(qbits.data_ptr<int64_t>(), nsc, order.data_ptr<int32_t>(), work.data_ptr<int32_t>(),
                                work.numel(), qbits.device().index(), as_stream(stream_p)),
@@ -370,7 +370,7 @@ torch::Tensor group_plan_stats(torch::Tensor stats, double u, torch::Tensor orde
     TORCH_CHECK(stats.is_contiguous() && order.is_contiguous(), "stats and order must be contiguous");
     const int64_t nsc = stats.numel() / 2;
     TORCH_CHECK(nsc > 0 && stats.numel() == 2 * nsc, "stats must hold (mean, norm) pairs");
-    TORCH_CHECK(order.numel() >= nsc, "order has fewer entries than superchunks");
+    TORCH_CHECK(order.numel() >= 3 * nsc, "order has fewer than 3 * nsc entries");
     int64_t *qptr = nullptr;
     if (qbits_out.has_value()) {
         TORCH_CHECK(qbits_out->device().type() == torch::kCUDA && qbits_out->dtype() == torch::kInt64 &&
@@ -467,7 +467,7 @@ static void check_plan_tensors(const torch::Tensor &order, const torch::Tensor &
     TORCH_CHECK(order.device().type() == torch::kCUDA && counts.device().type() == torch::kCUDA, "order and counts must be CUDA tensors");
     TORCH_CHECK(order.dtype() == torch::kInt32 && counts.dtype() == torch::kInt32, "order and counts must be torch.int32");
     TORCH_CHECK(order.is_contiguous() && counts.is_contiguous(), "order and counts must be contiguous");
-    TORCH_CHECK(order.numel() >= nsc, "order has fewer entries than superchunks");
+    TORCH_CHECK(order.numel() >= 3 * nsc, "order has fewer than 3 * nsc entries");
     TORCH_CHECK(counts.numel() >= 3, "counts must hold the three group sizes");
 }
 
@@ -871,7 +871,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("scaling_decompress_irht", &scaling_decompress_irht, "hierarchical chunk-16 decompress + inverse blocked randomized Hadamard transform in one launch", py::arg("src"), py::arg("sign"), py::arg("dst"), py::arg("block"), py::arg("scale"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("rand_diag", &rand_diag, "EDEN's seeded +-1 diagonal", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
-    modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width; returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
+    modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width into the three regions of order (8-bit rows from 0, 4-bit from nsc, 2-bit from 2 nsc); returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
     modul.def("group_plan_stats", &group_plan_stats, "bit widths from the reduced bf16 norms and the offset u, and the partition by width, in one call; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
     modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);

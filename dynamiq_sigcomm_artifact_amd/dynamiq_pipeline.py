@@ -84,7 +84,7 @@ def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=
         work["key"] = key
         work["residuals"] = [torch.empty(nsc * SUPERCHUNK, dtype=dt, device=dev) for _ in range(W)]
         work["stats"] = [torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev) for _ in range(W)]
-        work["order"] = torch.empty(nsc, dtype=torch.int32, device=dev)
+        work["order"] = torch.empty(3 * nsc, dtype=torch.int32, device=dev)
     residuals, stats, order = work["residuals"], work["stats"], work["order"]
     stream = torch.cuda.current_stream().cuda_stream
     for r in range(W):
@@ -103,12 +103,10 @@ def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=
     assert counts[3] == 0, "bit widths outside {2, 4, 8}"
 
     outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
-    start = 0
-    for q, cnt in zip((8, 4, 2), counts[:3]):
+    for g, (q, cnt) in enumerate(zip((8, 4, 2), counts[:3])):
         if cnt == 0:
             continue
-        rows = order[start:start + cnt]
-        start += cnt
+        rows = order[g * nsc:g * nsc + cnt]          # every width has a region of nsc entries
         comps = compressors[q]
         if W == 1:
             c = comps[0]
@@ -150,7 +148,7 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         work["stats"] = [torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev) for _ in range(W)]
         work["mean"] = [torch.empty(nsc, dtype=torch.float32, device=dev) for _ in range(W)]
         work["total"] = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
-        work["order"] = torch.empty(nsc, dtype=torch.int32, device=dev)
+        work["order"] = torch.empty(3 * nsc, dtype=torch.int32, device=dev)
         work["plan"] = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
         work["send"] = [torch.zeros(cap, dtype=torch.uint8, device=dev) for _ in range(W)]
         work["recv"] = [torch.zeros(cap, dtype=torch.uint8, device=dev) for _ in range(W if W > 1 else 0)]

@@ -571,7 +571,7 @@ def kernels(dev, n=6553600):
     stats = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
     line("superchunk_mean_center", lambda: capi.superchunk_mean_center(src, res, stats, n, 8), 4 * n + 4 * nsc, elements="bf16")
     line("superchunk_add_mean_copy", lambda: capi.superchunk_add_mean_copy(res, out, stats, n), 4 * n + 2 * nsc, elements="bf16")
-    order = torch.empty(nsc, dtype=torch.int32, device=dev)
+    order = torch.empty(3 * nsc, dtype=torch.int32, device=dev)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
     qbits = torch.empty(nsc, dtype=torch.int64, device=dev)
     u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)

@@ -149,11 +149,13 @@ int dq_philox_uniform(void *out, int64_t n, int dtype, int device, uint64_t seed
 int64_t dq_group_plan_work_ints(int64_t nsc);
 
 /* comm_hooks.py:964-966.  qbits: int64 [nsc] on the device (the output of
- * _dynamic_bitrate_qbits, :48-66).  order: int32 [nsc]; on return
- * order[0..n8) lists, ascending, the superchunks with qbits == 8, then n4 with
- * 4, then n2 with 2 (torch.nonzero order).  work[0..2] = n8, n4, n2 and
- * work[3] = superchunks of any other width (they appear in no group); the rest
- * of work is scratch.  Two launches on `stream`, no host synchronisation. */
+ * _dynamic_bitrate_qbits, :48-66).  order: int32 [3 * nsc], one region of nsc
+ * entries per width; on return order[0..n8) lists, ascending, the superchunks
+ * with qbits == 8, order[nsc..nsc+n4) those with 4 and order[2*nsc..2*nsc+n2)
+ * those with 2 (torch.nonzero order); the rest of order is not written.
+ * work[0..2] = n8, n4, n2 and work[3] = superchunks of any other width (they
+ * appear in no group); the rest of work is scratch.  One launch on `stream`
+ * for nsc <= 65536, two beyond; no host synchronisation. */
 int dq_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work,
                   int64_t work_ints, int device, dq_stream_t stream);
 
@@ -212,8 +214,9 @@ int dq_scaling_decompress_rows(const uint8_t *src, void *dst, const int32_t *row
  * ring_chunk = 0 addresses whole groups.
  *
  * Rounding randomness: rand_pool != NULL -> row k (256 values, element type of
- * src, or bf16 with DQ_RAND_BF16) belongs to position k of `order`, so the
- * pool holds >= 256 * nsc values; rand_pool == NULL -> the in-kernel Philox
+ * src, or bf16 with DQ_RAND_BF16) belongs to the k-th superchunk of the
+ * concatenation 8-bit group | 4-bit group | 2-bit group, so the pool holds
+ * >= 256 * nsc values; rand_pool == NULL -> the in-kernel Philox
  * stream of dq_scaling_compress_philox, keyed by (seed, step, index of the
  * chunk in src).
  *

@@ -20,7 +20,7 @@ def test_group_plan_matches_nonzero(capi, nsc):
     q = torch.tensor([2, 4, 8, 16])[torch.randint(0, 4 if nsc > 5 else 3, (nsc,), generator=g)].to(DEV)
     if nsc == 1023:
         q[:] = 8            # a single group
-    order = torch.full((nsc,), -1, dtype=torch.int32, device=DEV)
+    order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
     for rep in range(3):        # the same work buffer serves call after call
         if rep:
@@ -30,8 +30,10 @@ def test_group_plan_matches_nonzero(capi, nsc):
         counts = work[:4].tolist()
         want = [torch.nonzero(q == w).view(-1) for w in (8, 4, 2)]
         assert counts[:3] == [w.numel() for w in want] and counts[3] == int((q == 16).sum())
-        got = order[:sum(counts[:3])].cpu()
-        assert torch.equal(got, torch.cat(want).cpu().to(torch.int32))
+        for g in range(3):      # one region of nsc entries per width; nothing written beyond a group
+            region = order[g * nsc:(g + 1) * nsc].cpu()
+            assert torch.equal(region[:counts[g]], want[g].cpu().to(torch.int32))
+            assert bool((region[counts[g]:] == -1).all())
 
 
 def test_group_plan_stats_all_bf16_norms(capi, oracle):
@@ -44,7 +46,7 @@ def test_group_plan_stats_all_bf16_norms(capi, oracle):
     stats = torch.zeros(nsc, 2, dtype=torch.bfloat16)
     stats[:, 1] = norms
     stats_d = stats.to(DEV)
-    order = torch.empty(nsc, dtype=torch.int32, device=DEV)
+    order = torch.empty(3 * nsc, dtype=torch.int32, device=DEV)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
     qout = torch.empty(nsc, dtype=torch.int64, device=DEV)
     finite = torch.isfinite(norms.float())
@@ -55,8 +57,10 @@ def test_group_plan_stats_all_bf16_norms(capi, oracle):
         assert (got == want).all(), (u, np.nonzero(got != want)[0][:10], got[got != want][:10], want[got != want][:10])
         counts = work[:4].tolist()
         assert counts == [int((want == 8).sum()), int((want == 4).sum()), int((want == 2).sum()), 0]
-        idx = np.concatenate([np.nonzero(want == w)[0] for w in (8, 4, 2)])
-        assert (order.cpu().numpy() == idx).all()
+        order_h = order.cpu().numpy()
+        for g, w in enumerate((8, 4, 2)):
+            idx = np.nonzero(want == w)[0]
+            assert (order_h[g * nsc:g * nsc + idx.size] == idx).all()
         t = bitrate.dynamic_bitrate_qbits(stats_d[:, 1], u).cpu()
         assert int((t[finite] != qout.cpu()[finite]).sum()) == 0, u
 
@@ -176,3 +180,29 @@ def test_grouped_pipeline_equals_reference_sequence(eden_utils, W, method):
     ref = torch.stack([v.double() for v in vecs]).mean(0)
     nmse = float(((b_out[0].double() - ref) ** 2).sum() / (ref ** 2).sum())
     assert nmse < 0.2
+
+
+@pytest.mark.parametrize("nsc,shift", [(70000, 0), (4099, 1), (65536, 1)])
+def test_group_plan_stats_two_launch_paths(capi, oracle, nsc, shift):
+    """more than 64 tiles, and a stats buffer that is only 2-byte aligned, take the two-launch path: same result"""
+    g = torch.Generator().manual_seed(nsc)
+    norms = torch.exp(torch.randn(nsc, generator=g) * 6.0).to(torch.bfloat16)
+    buf = torch.zeros(2 * nsc + 2, dtype=torch.bfloat16)
+    stats = buf[shift:shift + 2 * nsc].view(nsc, 2)
+    stats[:, 1] = norms
+    stats_d = buf.to(DEV)[shift:shift + 2 * nsc].view(nsc, 2)
+    assert stats_d.data_ptr() % 4 == 2 * shift
+    order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    qout = torch.empty(nsc, dtype=torch.int64, device=DEV)
+    u = 7.1
+    capi.group_plan_stats(stats_d, u, qout, order, work)
+    want = oracle.dynamic_bitrate_qbits(to_bits(norms), u)
+    assert (qout.cpu().numpy() == want).all()
+    counts = work[:4].tolist()
+    assert counts == [int((want == 8).sum()), int((want == 4).sum()), int((want == 2).sum()), 0] and min(counts[:3]) > 0
+    order_h = order.cpu().numpy()
+    for gi, w in enumerate((8, 4, 2)):
+        idx = np.nonzero(want == w)[0]
+        assert (order_h[gi * nsc:gi * nsc + idx.size] == idx).all()
+        assert (order_h[gi * nsc + idx.size:(gi + 1) * nsc] == -1).all()

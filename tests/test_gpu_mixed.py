@@ -20,20 +20,21 @@ def make_plan(capi, nsc, seed, weights=(1, 1, 1)):
     g = torch.Generator().manual_seed(seed)
     w = torch.tensor(weights, dtype=torch.float)
     q = torch.tensor([8, 4, 2])[torch.multinomial(w, nsc, replacement=True, generator=g)].to(DEV)
-    order = torch.full((nsc,), -1, dtype=torch.int32, device=DEV)
+    order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
     capi.group_plan(q, order, work)
     return q, order, work
 
 
-def segments(counts, chunk, world):
-    """(width, position of the run in `order`, records, byte offset) of ring chunk `chunk`, and the stream size"""
+def segments(counts, chunk, world, nsc):
+    """(width, entry of `order` where the run's rows start, row of the random pool of its first record, records, byte
+    offset) of ring chunk `chunk`, and the stream size"""
     out, pos, off = [], 0, 0
-    for q, n in zip((8, 4, 2), counts):
+    for g, (q, n) in enumerate(zip((8, 4, 2), counts)):
         per = -(-n // world)
         begin = min(per * chunk, n)
         cnt = min(per, n - begin)
-        out.append((q, pos + begin, cnt, off))
+        out.append((q, g * nsc + begin, pos + begin, cnt, off))
         pos += n
         off += cnt * REC[q]
     return out, off
@@ -57,7 +58,7 @@ def test_mixed_matches_per_group_calls(capi, dt, strategy, nsc, world, weights):
     out = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
     out_ref = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
     for chunk in range(world):
-        segs, total = segments(counts, chunk, world)
+        segs, total = segments(counts, chunk, world, nsc)
         assert total <= cap
         enc = torch.full((cap + 16,), 0xAB, dtype=torch.uint8, device=DEV)
         send = torch.full((cap + 16,), 0xCD, dtype=torch.uint8, device=DEV)
@@ -69,10 +70,10 @@ def test_mixed_matches_per_group_calls(capi, dt, strategy, nsc, world, weights):
         capi.mixed_decompress(send, out, order, work, nsc, strategy, stats=stats, n_limit=n_valid, ring_chunk=chunk,
                               ring_world=world)
         assert bool((enc[total:] == 0xAB).all()) and bool((send[total:] == 0xCD).all())    # nothing past the stream
-        for width, pos, cnt, off in segs:
+        for width, row0, pos, cnt, off in segs:
             if cnt == 0:
                 continue
-            rows = order[pos:pos + cnt]
+            rows = order[row0:row0 + cnt]
             rnd = pool[pos * 256:(pos + cnt) * 256]
             nb = cnt * REC[width]
             e = torch.zeros(nb, dtype=torch.uint8, device=DEV)
@@ -103,10 +104,10 @@ def test_mixed_philox_matches_oracle(capi, oracle, dt, odt, strategy):
         uni = (uni.view(np.uint32) >> 16).astype(np.uint16)     # k/256 is exact in bf16
     src_h = to_bits(full.cpu())
     ord_h = order.cpu().numpy()
-    segs, total = segments(counts, 0, 1)
+    segs, total = segments(counts, 0, 1, nsc)
     got = enc.cpu().numpy()
-    for width, pos, cnt, off in segs:
-        rows = ord_h[pos:pos + cnt]
+    for width, row0, pos, cnt, off in segs:
+        rows = ord_h[row0:row0 + cnt]
         gs = src_h.reshape(-1, 256)[rows].reshape(-1).copy()
         gu = uni.reshape(-1, 256)[rows].reshape(-1).copy()
         want = oracle.scaling_compress(gs, gu, cnt * 256, width, 16, strategy, odt)
@@ -193,7 +194,7 @@ def test_mixed_pipeline_replays_as_graph(capi):
     src = torch.empty(n, dtype=torch.bfloat16, device=DEV)
     stats = torch.zeros(nsc, 2, dtype=torch.bfloat16, device=DEV)
     mean = torch.zeros(nsc, dtype=torch.float32, device=DEV)
-    order = torch.zeros(nsc, dtype=torch.int32, device=DEV)
+    order = torch.zeros(3 * nsc, dtype=torch.int32, device=DEV)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
     enc = torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=DEV)
     out = torch.zeros(n, dtype=torch.bfloat16, device=DEV)

@@ -148,7 +148,7 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_thc_dequantize_irht(P, P, N, 64, 64, F1, P, P, 0, S), "null pointer")
     err(L.dq_thc_dequantize_irht(P, P, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
-    assert capi.group_plan_work_ints(25600) == 4 + 4 * 25 and capi.eden_work_doubles(8192) == 2
+    assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 and capi.eden_work_doubles(8192) == 2
     # a good call clears the message
     assert L.dq_scaling_check_common(256, 4, 16, 2, 1) == 0 and L.dq_last_error().decode() == ""
     assert L.dq_status_string(16).decode() == "kernel launch failed"
