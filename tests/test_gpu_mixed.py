@@ -296,3 +296,44 @@ def test_single_pass_pipeline_matches_oracle(capi, oracle, W, strategy):
     exact = torch.stack([v.double() for v in vecs]).sum(0) / W
     err = float((outs[0].cpu().double() - exact).pow(2).sum() / exact.pow(2).sum())
     assert err < 0.02, err
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_mixed_special_values(capi, dt, strategy):
+    """NaN, infinities, huge, tiny and all-zero superchunks take the guarded path of a wave: the folded calls still equal
+    mean_center + the per-width calls, and the random pool may hold values outside [0, 1]"""
+    nsc, n = 97, 97 * 256 - 13
+    g = torch.Generator().manual_seed(7 + strategy)
+    x = torch.randn(n, generator=g) * 1e-2
+    x[5] = float("nan"); x[300] = float("inf"); x[301] = float("-inf"); x[1000] = 3e38; x[1001] = -1e-40
+    x[256 * 10:256 * 12] = 0.0
+    x[256 * 20:256 * 21] = 1e30
+    x[256 * 30:256 * 31] = 1e-38
+    src = x.to(dt).to(DEV)
+    pool = torch.rand(nsc * 256, generator=g)
+    pool[77] = 1.5; pool[78] = -0.25; pool[79] = float("nan")
+    pool = pool.to(dt).to(DEV)
+    q, order, work = make_plan(capi, nsc, 5)
+    counts = work[:3].tolist()
+    stats = torch.zeros(nsc, 2, dtype=torch.bfloat16, device=DEV)
+    mean = torch.zeros(nsc, device=DEV)
+    capi.superchunk_stats(src, stats, mean, n, 3)
+    residual = torch.zeros(nsc * 256, dtype=dt, device=DEV)
+    stats2 = torch.zeros_like(stats)
+    capi.superchunk_mean_center(src, residual, stats2, n, 3)
+    assert torch.equal(bits_t(stats), bits_t(stats2))
+    cap = capi.mixed_required_bytes(nsc, 1)
+    enc = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+    capi.mixed_compress(src, order, work, enc, nsc, strategy, rand_pool=pool, center_mean=mean, center_world=3, n=n)
+    out = torch.full((n,), 7.0, dtype=dt, device=DEV)
+    capi.mixed_decompress(enc, out, order, work, nsc, strategy, stats=stats, n_limit=n)
+    out_ref = torch.full((n,), 7.0, dtype=dt, device=DEV)
+    segs, total = segments(counts, 0, 1, nsc)
+    for width, row0, pos, cnt, off in segs:
+        rows = order[row0:row0 + cnt]
+        e = torch.zeros(cnt * REC[width], dtype=torch.uint8, device=DEV)
+        capi.scaling_compress_rows(residual, rows, e, pool[pos * 256:(pos + cnt) * 256], cnt, width, strategy)
+        assert torch.equal(enc[off:off + e.numel()], e), width
+        capi.scaling_decompress_rows(e, out_ref, rows, stats, n, cnt, width, strategy)
+    assert torch.equal(bits_t(out), bits_t(out_ref))

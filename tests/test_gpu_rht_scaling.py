@@ -138,3 +138,29 @@ def test_fused_full_size_properties(capi):
     want = torch.zeros_like(enc)
     capi.scaling_compress_philox(rot, want, n, nbits, 16, 2, 1, 2)
     assert torch.equal(enc, want)
+
+
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_fused_special_values(capi, strategy):
+    """non-finite and extreme inputs spread over whole transform blocks by the butterflies: still the two-call bytes"""
+    n, block, nbits = 8192 * 3, 1024, 4
+    g, x, sign = _case(n, 5)
+    x[3] = float("inf"); x[1024 + 7] = float("nan"); x[2048:3072] = 0.0; x[4096] = 3e38; x[4097] = 3e38
+    x[5120:6144] = 1e-40
+    pool = torch.rand(n, generator=g).to(DEV)
+    pool[9000] = 2.0
+    scale = 1.0 / 32
+    rot = x.clone()
+    capi.rht_blocked(rot, sign, block, scale, False)
+    nb = capi.required_bytes(n, nbits, 16, strategy)
+    want = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+    capi.scaling_compress(rot, want, pool, n, nbits, 16, strategy)
+    got = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+    capi.rht_scaling_compress(x, capi.pack_signs(sign), got, block, scale, nbits, strategy, rand_pool=pool)
+    assert torch.equal(got, want)
+    dec = torch.empty(n, device=DEV)
+    capi.scaling_decompress(want, dec, n, nbits, 16, strategy)
+    capi.rht_blocked(dec, sign, block, scale, True)
+    back = torch.empty(n, device=DEV)
+    capi.scaling_decompress_irht(got, sign, back, block, scale, nbits, strategy)
+    assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
