@@ -4,9 +4,9 @@
 A step = scaling_compress followed by scaling_decompress of one 25 MB DDP
 bucket (6,553,600 fp32 gradient elements, Student-t(3) * 1e-3 with 0.1 % of the
 entries multiplied by 100), hierarchical AEE (strategy 2), chunk 16, 4-bit
-codes, bf16 random pool -- the second configuration of BASELINE.json.  Inputs
-are resident in HBM before the timed region; the calls go through the C ABI of
-libdynamiq_eden.so on torch's current stream.
+codes, bf16 random pool -- the 25 MB bucket configuration the headline metric
+is quoted on.  Inputs are resident in HBM before the timed region; the calls go
+through the C ABI of libdynamiq_eden.so on torch's current stream.
 
 Prints ONE JSON line (see the fields below).  `value` is fp32 gradient bytes
 (4 * N) per second of compress+decompress.  `roofline` prices the dominant
