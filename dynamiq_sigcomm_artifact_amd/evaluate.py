@@ -158,8 +158,17 @@ def config2(dev):
                       roundtrip_GBps_of_fp32_input=round(4.0 * n / (tc + td) / 1e3, 1),
                       compress_frac_hbm=round((sb + 2 + pb) * n / tc / 1e3 / HBM_PEAK, 4),
                       decompress_frac_hbm=round((sb + pb) * n / td / 1e3 / HBM_PEAK, 4))
+    # the flat quantiser (strategy 0) next to the same quantiser written as torch CPU ops: two independent
+    # implementations of one formula, different random draws
     for nbits in (4, 8):
-        _cpu_torch_line(x32, nbits)
+        packed = torch.zeros(capi.required_bytes(n, nbits, 16, 0), dtype=torch.uint8, device=dev)
+        out = torch.empty_like(x32)
+        capi.scaling_compress(x32, packed, rand, n, nbits, 16, 0)
+        capi.scaling_decompress(packed, out, n, nbits, 16, 0)
+        cpu_nmse = _cpu_torch_line(x32, nbits)
+        gpu_nmse = _nmse(x32, out)
+        _emit(config=2, source="fp32", strategy=0, nbits=nbits, nmse=gpu_nmse, nmse_cpu_torch=cpu_nmse,
+              nmse_ratio=round(gpu_nmse / cpu_nmse, 4))
 
 
 def _torch_cpu_roundtrip(x, rand, nbits, chunk=16):
@@ -191,9 +200,11 @@ def _cpu_torch_line(x32, nbits):
         out = _torch_cpu_roundtrip(xc, rc, nbits)
         ts.append(time.perf_counter() - t0)
     ts.sort()
+    nmse = _nmse(xc, out)
     _emit(config=2, path="cpu torch op sequence (csrc/logic.py:225-296)", nbits=nbits, threads=threads,
           roundtrip_ms=round(ts[2] * 1e3, 2), roundtrip_GBps_of_fp32_input=round(4.0 * xc.numel() / ts[2] / 1e9, 3),
-          nmse=_nmse(xc, out))
+          nmse=nmse)
+    return nmse
 
 
 def _params(d, W, r):
