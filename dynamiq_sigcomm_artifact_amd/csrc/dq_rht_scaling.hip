@@ -226,6 +226,140 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
     }
 }
 
+// ---- blocks of 2^15: the tile in two halves -----------------------------------------------------------
+//
+// A 2^15 tile with its padding needs 139 KB of LDS: one workgroup per CU, whose load, butterfly and
+// quantise phases cannot overlap with a neighbour's.  Here thread t owns chunk t of both halves of the
+// block: the stages of strides 1..8 run on registers, the stages of strides 16 .. 2^13 run in LDS one half
+// after the other (70 KB: two workgroups per CU), and the last stage (stride 2^14) pairs the thread's own
+// two chunks in registers.  The record windows (and the MEE table of the inverse kernel) share the LDS with
+// the tile: they are used only before the first half enters it or after the second has left.  Both kernels
+// ask for eight waves per SIMD (64 registers): two resident workgroups are worth more than the few values
+// the forward kernel then spills (measured 1.55 against 1.69 ms at 2^30 elements).
+constexpr int kSplitBits = 15, kHalfBits = 14, kSplitThreads = 1024;
+
+// stages of strides 16 .. 2^13 of the half block whose chunk t the thread holds in v (in and out)
+__device__ __forceinline__ void half_block_stages(float (&v)[16], float *lds, int tid)
+{
+    float *mine = lds + tid * 17;
+#pragma unroll
+    for (int i = 0; i < 16; i++) mine[i] = v[i];
+    fwht_lds_stages_after4(lds, kHalfBits, kHalfBits, tid, kSplitThreads);
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[i] = mine[i];
+    __syncthreads(); // the half has left the LDS
+}
+
+template <int RDT, int NBITS, bool MEE>
+__global__ __launch_bounds__(kSplitThreads, 8) void rht_compress_split_kernel(const float *__restrict__ x, uint8_t *__restrict__ dst,
+                                                                          const void *__restrict__ rnd, RhtTileArgs a,
+                                                                          int rvec, RandKey key, MeeArg<NBITS, MEE> mp)
+{
+    typedef Rec<NBITS> RC;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t origin = (int64_t)blockIdx.x << kSplitBits;
+    float va[16], vb[16];
+    load_chunk(va, x, a, origin + tid * 16);
+    load_chunk(vb, x, a, origin + (1 << kHalfBits) + tid * 16);
+    butterflies<4>(va);
+    butterflies<4>(vb);
+    half_block_stages(va, lds, tid);
+    half_block_stages(vb, lds, tid);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float p = va[i], q = vb[i];
+        va[i] = p + q;
+        vb[i] = p - q;
+    }
+    // quantise: the wave's 64 chunks of a half are 4 superchunks, one run of records
+    uint8_t *win_out = reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int64_t sc0 = (origin >> 8) + h * 64 + wave * kRowsPerWave;
+        Raw16<DQ_F32> v;
+        Raw16<RDT> r;
+        if constexpr (RDT == DQ_PHILOX)
+            r.generate(key, sc0 * 16 + lane);
+        else
+            r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
+#pragma unroll
+        for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint((h ? vb[i] : va[i]) * a.scale);
+        encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, kRowsPerWave, win_out);
+        wave_lds_sync(); // the window is reused for the other half
+    }
+}
+
+template <int NBITS, bool MEE>
+__global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel(const uint8_t *__restrict__ src,
+                                                                             float *__restrict__ x, RhtTileArgs a,
+                                                                             MeeArg<NBITS, MEE> mp)
+{
+    typedef Rec<NBITS> RC;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = lane >> 4, j = lane & 15;
+    const int64_t origin = (int64_t)blockIdx.x << kSplitBits;
+    uint8_t *win_in = reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN;
+    float *table = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds) + (kSplitThreads / 64) * RC::WIN);
+    if (MEE) {
+        for (int k = tid; k < (1 << NBITS); k += kSplitThreads) table[k] = f16_bits_to_f32(mp.table[k]);
+        __syncthreads();
+    }
+    float va[16], vb[16];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int64_t sc0 = (origin >> 8) + h * 64 + wave * kRowsPerWave;
+        const int total = kRowsPerWave * RC::REC;
+        const uint8_t *g = src + sc0 * RC::REC;
+        const WinRegs wr = window_fetch(g, total, lane);
+        const int mis = window_commit(win_in, wr, g, total, lane);
+        wave_lds_sync();
+        const uint8_t *rec = win_in + mis + row * RC::REC;
+        uint32_t cw[RC::WORDS], cq;
+        chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+        const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+        float t[16];
+        chunk_decode<NBITS, MEE, false>(cw, cq, ub, table, t);
+#pragma unroll
+        for (int i = 0; i < 16; i++) (h ? vb[i] : va[i]) = t[i];
+        wave_lds_sync(); // the window is reused for the other half
+    }
+    __syncthreads(); // windows and table are done with: the tile takes the LDS
+    butterflies<4>(va);
+    butterflies<4>(vb);
+    half_block_stages(va, lds, tid);
+    half_block_stages(vb, lds, tid);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float p = va[i], q = vb[i];
+        va[i] = p + q;
+        vb[i] = p - q;
+    }
+    // store one half after the other through the LDS, so that every store instruction covers 1 KiB contiguously
+    float *mine = lds + tid * 17;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) mine[i] = h ? vb[i] : va[i];
+        __syncthreads();
+        const int64_t half_origin = origin + ((int64_t)h << kHalfBits);
+        if (a.vec) {
+            for (int i = tid * 4; i < (1 << kHalfBits); i += kSplitThreads * 4) {
+                const int q = pad_idx(i);
+                float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
+                v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale;
+                flip4(v, a, half_origin + i);
+                *reinterpret_cast<float4 *>(x + half_origin + i) = v;
+            }
+        } else {
+            for (int i = tid; i < (1 << kHalfBits); i += kSplitThreads)
+                x[half_origin + i] = flip1(lds[pad_idx(i)] * a.scale, a, half_origin + i);
+        }
+        __syncthreads();
+    }
+}
+
 constexpr int kPrefTileBits = 13; // 32 KiB tiles: eight waves, one run each, several workgroups per CU
 
 struct Geometry {
@@ -263,6 +397,15 @@ hipError_t run_compress(const float *src, const void *sign, int sign_bits, uint8
                         float scale, const MeeParams &mp, RandKey key, hipStream_t stream)
 {
     const Geometry g = geometry(src, sign, sign_bits, n, block, scale);
+    if (g.a.kb == kSplitBits) {
+        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float);
+        auto split = rht_compress_split_kernel<RDT, NBITS, MEE>;
+        hipError_t es = allow_lds(split, half_lds);
+        if (es != hipSuccess) return es;
+        hipLaunchKernelGGL(split, dim3((unsigned)(n >> kSplitBits)), dim3(kSplitThreads), half_lds, stream, src, dst, rnd, g.a,
+                           aligned16(rnd) ? 1 : 0, key, make_arg<NBITS, MEE>(mp));
+        return hipGetLastError();
+    }
     const size_t lds = g.lds_floats * sizeof(float) + (size_t)(g.threads / 64) * Rec<NBITS>::WIN;
     auto kernel = rht_compress_kernel<RDT, NBITS, MEE>;
     hipError_t e = allow_lds(kernel, lds);
@@ -277,6 +420,15 @@ hipError_t run_decompress(const uint8_t *src, const void *sign, int sign_bits, f
                           const MeeParams &mp, hipStream_t stream)
 {
     const Geometry g = geometry(dst, sign, sign_bits, n, block, scale);
+    if (g.a.kb == kSplitBits) {
+        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float);
+        auto split = irht_decompress_split_kernel<NBITS, MEE>;
+        hipError_t es = allow_lds(split, half_lds);
+        if (es != hipSuccess) return es;
+        hipLaunchKernelGGL(split, dim3((unsigned)(n >> kSplitBits)), dim3(kSplitThreads), half_lds, stream, src, dst, g.a,
+                           make_arg<NBITS, MEE>(mp));
+        return hipGetLastError();
+    }
     const size_t lds = g.lds_floats * sizeof(float) + (size_t)(g.threads / 64) * Rec<NBITS>::WIN +
                        (MEE ? (sizeof(float) << NBITS) : 0);
     auto kernel = irht_decompress_kernel<NBITS, MEE>;
