@@ -15,6 +15,8 @@
 // of the hier16 kernels (dq_hier16_tiles.cuh).  Numerics of the quantiser: csrc/cuda_hierarchical_mee.cu:203-505;
 // of the transform: csrc/cuda_hadamard.cu:66-157,534-605 with the sign flip and 1/sqrt(block) of
 // testbed_evaluation/new_comm_hooks/thc_hooks.py:95-107 folded in.
+#include <algorithm>
+
 #include "dq_fwht.cuh"
 #include "dq_hier16_tiles.cuh"
 #include "dq_launch.h"
@@ -123,32 +125,33 @@ __global__ void rht_compress_kernel(const float *__restrict__ x, uint8_t *__rest
     }
     fwht_lds_stages_after4(lds, a.kt, a.kb, tid, nthreads);
 
-    // quantise: a wave takes runs of 64 chunks (4 superchunks, one contiguous run of records)
-    const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
-    uint8_t *win_out = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(a.kt)) + wave * RC::WIN;
+    // quantise: the tile holds one run of 64 chunks (4 superchunks, one contiguous run of records) per wave.
+    // Every wave first takes its chunks into registers; after the barrier the tile is dead and the record
+    // windows reuse its LDS.
+    const int lane = tid & 63, wave = tid >> 6;
     const int64_t nsc_total = a.n >> 8, sc_origin = origin >> 8;
     const int tile_sc = max(1, tile >> 8);
-    for (int run = wave; run * kRowsPerWave < tile_sc; run += nwaves) {
-        const int64_t sc0 = sc_origin + run * kRowsPerWave;
-        if (sc0 >= nsc_total) break;
-        const int rows_here = (int)min((int64_t)min(kRowsPerWave, tile_sc - run * kRowsPerWave), nsc_total - sc0);
-        Raw16<DQ_F32> v;
-        Raw16<RDT> r;
-        if ((lane >> 4) < rows_here) {
-            if constexpr (RDT == DQ_PHILOX)
-                r.generate(key, sc0 * 16 + lane);
-            else
-                r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
-            const float *mine = lds + (run * 64 + lane) * 17; // pad_idx(16 c + i) = 17 c + i
+    const int64_t sc0 = sc_origin + wave * kRowsPerWave;
+    const int rows_here = (wave * kRowsPerWave < tile_sc && sc0 < nsc_total)
+                              ? (int)min((int64_t)min(kRowsPerWave, tile_sc - wave * kRowsPerWave), nsc_total - sc0)
+                              : 0;
+    Raw16<DQ_F32> v;
+    Raw16<RDT> r;
+    if ((lane >> 4) < rows_here) {
+        if constexpr (RDT == DQ_PHILOX)
+            r.generate(key, sc0 * 16 + lane);
+        else
+            r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
+        const float *mine = lds + (wave * 64 + lane) * 17; // pad_idx(16 c + i) = 17 c + i
 #pragma unroll
-            for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint(mine[i] * a.scale);
-        } else {
-            v.zero();
-            r.zero();
-        }
-        encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, rows_here, win_out);
-        wave_lds_sync(); // the window is reused by this wave's next run
+        for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint(mine[i] * a.scale);
+    } else {
+        v.zero();
+        r.zero();
     }
+    __syncthreads();
+    if (rows_here > 0)
+        encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, rows_here, reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN);
 }
 
 template <int NBITS, bool MEE>
@@ -161,7 +164,8 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
     const int tile = 1 << a.kt;
     const int64_t origin = (int64_t)blockIdx.x << a.kt;
     const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
-    uint8_t *windows = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(a.kt));
+    // the record windows and the MEE table use the tile's LDS before the tile itself does
+    uint8_t *windows = reinterpret_cast<uint8_t *>(lds);
     uint8_t *win_in = windows + wave * RC::WIN;
     float *table = reinterpret_cast<float *>(windows + nwaves * RC::WIN);
     if (MEE) {
@@ -169,34 +173,34 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
         __syncthreads();
     }
 
-    // decode the tile's records into LDS, one lane per chunk; chunks beyond n become zeros
+    // decode the wave's run of records into registers, one lane per chunk; chunks beyond n become zeros
     const int64_t nsc_total = a.n >> 8, sc_origin = origin >> 8;
     const int tile_sc = max(1, tile >> 8);
-    for (int run = wave; run * kRowsPerWave < tile_sc; run += nwaves) {
-        const int64_t sc0 = sc_origin + run * kRowsPerWave;
-        const int rows_here = sc0 < nsc_total
-                                  ? (int)min((int64_t)min(kRowsPerWave, tile_sc - run * kRowsPerWave), nsc_total - sc0)
-                                  : 0;
-        const int row = lane >> 4, j = lane & 15;
-        float t[16];
+    const int64_t sc0 = sc_origin + wave * kRowsPerWave;
+    const int rows_here = (wave * kRowsPerWave < tile_sc && sc0 < nsc_total)
+                              ? (int)min((int64_t)min(kRowsPerWave, tile_sc - wave * kRowsPerWave), nsc_total - sc0)
+                              : 0;
+    const int row = lane >> 4, j = lane & 15;
+    float t[16];
 #pragma unroll
-        for (int i = 0; i < 16; i++) t[i] = 0.0f;
-        if (rows_here > 0) {
-            const int total = rows_here * RC::REC;
-            const uint8_t *g = src + sc0 * RC::REC;
-            const WinRegs wr = window_fetch(g, total, lane);
-            const int mis = window_commit(win_in, wr, g, total, lane);
-            wave_lds_sync();
-            if (row < rows_here) {
-                const uint8_t *rec = win_in + mis + row * RC::REC;
-                uint32_t cw[RC::WORDS], cq;
-                chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
-                const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
-                chunk_decode<NBITS, MEE, false>(cw, cq, ub, table, t);
-            }
-            wave_lds_sync(); // the window is reused by this wave's next run
+    for (int i = 0; i < 16; i++) t[i] = 0.0f;
+    if (rows_here > 0) {
+        const int total = rows_here * RC::REC;
+        const uint8_t *g = src + sc0 * RC::REC;
+        const WinRegs wr = window_fetch(g, total, lane);
+        const int mis = window_commit(win_in, wr, g, total, lane);
+        wave_lds_sync();
+        if (row < rows_here) {
+            const uint8_t *rec = win_in + mis + row * RC::REC;
+            uint32_t cw[RC::WORDS], cq;
+            chunk_read<NBITS>(rec + j * RC::CB, cw, cq);
+            const uint32_t ub = (uint32_t)rec[16 * RC::CB] | ((uint32_t)rec[16 * RC::CB + 1] << 8);
+            chunk_decode<NBITS, MEE, false>(cw, cq, ub, table, t);
         }
-        const int c = run * 64 + lane;
+    }
+    __syncthreads(); // windows and table are done with: the tile takes the LDS
+    {
+        const int c = wave * 64 + lane;
         if (c * 16 < tile) {
             chunk_stages(t, a.kb);
             float *mine = lds + c * 17;
@@ -406,7 +410,9 @@ hipError_t run_compress(const float *src, const void *sign, int sign_bits, uint8
                            aligned16(rnd) ? 1 : 0, key, make_arg<NBITS, MEE>(mp));
         return hipGetLastError();
     }
-    const size_t lds = g.lds_floats * sizeof(float) + (size_t)(g.threads / 64) * Rec<NBITS>::WIN;
+    if (g.a.kt >= kSplitBits) return hipErrorInvalidValue; // one run of records per wave needs tiles of at most 2^14
+    const size_t windows = (size_t)(g.threads / 64) * Rec<NBITS>::WIN;
+    const size_t lds = std::max(g.lds_floats * sizeof(float), windows);
     auto kernel = rht_compress_kernel<RDT, NBITS, MEE>;
     hipError_t e = allow_lds(kernel, lds);
     if (e != hipSuccess) return e;
@@ -429,8 +435,9 @@ hipError_t run_decompress(const uint8_t *src, const void *sign, int sign_bits, f
                            make_arg<NBITS, MEE>(mp));
         return hipGetLastError();
     }
-    const size_t lds = g.lds_floats * sizeof(float) + (size_t)(g.threads / 64) * Rec<NBITS>::WIN +
-                       (MEE ? (sizeof(float) << NBITS) : 0);
+    if (g.a.kt >= kSplitBits) return hipErrorInvalidValue;
+    const size_t windows = (size_t)(g.threads / 64) * Rec<NBITS>::WIN + (MEE ? (sizeof(float) << NBITS) : 0);
+    const size_t lds = std::max(g.lds_floats * sizeof(float), windows);
     auto kernel = irht_decompress_kernel<NBITS, MEE>;
     hipError_t e = allow_lds(kernel, lds);
     if (e != hipSuccess) return e;
