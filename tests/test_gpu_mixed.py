@@ -337,3 +337,56 @@ def test_mixed_special_values(capi, dt, strategy):
         assert torch.equal(enc[off:off + e.numel()], e), width
         capi.scaling_decompress_rows(e, out_ref, rows, stats, n, cnt, width, strategy)
     assert torch.equal(bits_t(out), bits_t(out_ref))
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_mixed_random_shapes(capi, block):
+    """seeded random plans, ring splits, element types, random sources and alignments: the one-launch calls against
+    the per-width calls on every run of every ring chunk"""
+    rng = np.random.default_rng(1000 + block)
+    for case in range(12):
+        nsc = int(rng.choice([1, 3, 4, 5, 63, 64, 65, 257, 1023, 1500, 4097]))
+        world = int(rng.choice([1, 2, 3, 5, 8]))
+        weights = tuple(float(w) for w in rng.choice([0.0, 0.2, 1.0, 3.0], size=3))
+        if sum(weights) == 0:
+            weights = (1.0, 1.0, 1.0)
+        dt = [torch.bfloat16, torch.float32][int(rng.integers(2))]
+        strategy = int(rng.choice([2, 3]))
+        use_philox = bool(rng.integers(2))
+        seed = int(rng.integers(1 << 30))
+        q, order, work = make_plan(capi, nsc, seed, weights)
+        counts = work[:3].tolist()
+        g = torch.Generator().manual_seed(seed)
+        shift = int(rng.integers(0, 4)) * (8 if dt == torch.bfloat16 else 4) + int(rng.integers(2))   # element offset of the view
+        full = torch.zeros(nsc * 256 + 64, dtype=dt, device=DEV)[shift:shift + nsc * 256]
+        full.copy_((torch.randn(nsc * 256, generator=g) * float(10.0 ** rng.uniform(-6, 2))).to(dt))
+        peer = (torch.randn(nsc * 256, generator=g) * 1e-2).to(dt).to(DEV)
+        pool_dt = dt if (dt == torch.bfloat16 or rng.integers(2)) else torch.bfloat16
+        pool = torch.rand(nsc * 256, generator=g).to(pool_dt).to(DEV)
+        cap = capi.mixed_required_bytes(nsc, world)
+        off0 = int(rng.integers(0, 16))
+        tag = (block, case, nsc, world, weights, dt, strategy, use_philox, shift, off0)
+        for chunk in range(world):
+            enc = torch.zeros(cap + 32, dtype=torch.uint8, device=DEV)[off0:off0 + cap]
+            send = torch.zeros(cap + 32, dtype=torch.uint8, device=DEV)[off0:off0 + cap]
+            kw = dict(seed=seed, step=chunk) if use_philox else dict(rand_pool=pool)
+            capi.mixed_compress(full, order, work, enc, nsc, strategy, ring_chunk=chunk, ring_world=world, **kw)
+            capi.mixed_compress(peer, order, work, send, nsc, strategy, recv=enc, ring_chunk=chunk, ring_world=world, **kw)
+            segs, total = segments(counts, chunk, world, nsc)
+            for width, row0, pos, cnt, off in segs:
+                if cnt == 0:
+                    continue
+                rows = order[row0:row0 + cnt]
+                nb = cnt * REC[width]
+                if use_philox:
+                    uni = torch.empty(nsc * 256, dtype=dt, device=DEV)
+                    capi.philox_uniform(uni, seed, chunk)
+                    rnd = uni.view(-1, 256)[rows.long()].reshape(-1).contiguous()
+                else:
+                    rnd = pool[pos * 256:(pos + cnt) * 256]
+                e = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+                s = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+                capi.scaling_compress_rows(full, rows, e, rnd, cnt, width, strategy)
+                capi.scaling_dec_comp_rows(e, peer, rows, s, rnd, cnt, width, strategy)
+                assert torch.equal(enc[off:off + nb], e), tag + (chunk, width)
+                assert torch.equal(send[off:off + nb], s), tag + (chunk, width)
