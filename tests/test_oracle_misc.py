@@ -84,6 +84,30 @@ def test_mean_center_closed_forms(oracle, dt):
     assert (res == want_res).all()
 
 
+def test_superchunk_stats_means(oracle):
+    """the statistics-only variant: same stats as mean_center, and the unrounded binary32 means it reports are the ones
+    the residual is formed with (numpy pairwise halving in float32; the ragged last superchunk divides by its length)"""
+    g = torch.Generator().manual_seed(9)
+    n, W = 256 * 3 + 50, 3
+    x = (torch.randn(n, generator=g) * 1e-2 + 0.03).to(torch.bfloat16)
+    res, stats = oracle.superchunk_mean_center(to_bits(x), n, W, BF16)
+    stats2, means = oracle.superchunk_stats(to_bits(x), n, W, BF16)
+    assert (stats == stats2).all() and means.dtype == np.float32 and means.size == 4
+    v = (bits_to_f32(to_bits(x), BF16) / np.float32(W)).astype(np.float32)
+    for b in range(4):
+        blk = np.zeros(256, np.float32)
+        valid = min(256, n - 256 * b)
+        blk[:valid] = v[256 * b:256 * b + valid]
+        s = blk.copy()
+        while s.size > 1:
+            h = s.size // 2
+            s = (s[:h] + s[h:]).astype(np.float32)
+        mean = np.float32(s[0] / np.float32(valid))
+        assert means[b] == mean
+        want = to_bits(torch.from_numpy((blk[:valid] - mean).astype(np.float32)).to(torch.bfloat16))
+        assert (res[256 * b:256 * b + valid] == want).all()
+
+
 def test_add_mean_restores_input(oracle):
     g = torch.Generator().manual_seed(4)
     n, W = 256 * 5 + 77, 8
