@@ -588,6 +588,20 @@ def kernels(dev, n=6553600):
     u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)
     line("group_plan_stats", lambda: capi.group_plan_stats(stats, u, qbits, order, work), 4 * nsc + 12 * nsc, superchunks=nsc)
     line("group_plan", lambda: capi.group_plan(qbits, order, work), 8 * nsc + 4 * nsc, superchunks=nsc)
+    # statistics without the residual, then the three widths of the plan in one launch (centring folded into the load,
+    # rounding stream drawn in the kernel) and back (mean added on the store)
+    mean32 = torch.empty(nsc, dtype=torch.float32, device=dev)
+    line("superchunk_stats", lambda: capi.superchunk_stats(src, stats, mean32, n, 8), 2 * n + 8 * nsc, elements="bf16")
+    capi.group_plan_stats(stats, u, None, order, work)
+    counts = work[:3]
+    n8, n4, n2 = (int(c) for c in counts.tolist())
+    stream_bytes = 274 * n8 + 146 * n4 + 82 * n2
+    mixed = torch.zeros(capi.mixed_required_bytes(nsc), dtype=torch.uint8, device=dev)
+    line("mixed_compress (centred load)",
+         lambda: capi.mixed_compress(src, order, counts, mixed, nsc, 2, seed=1, step=0, center_mean=mean32, center_world=8, n=n),
+         2 * n + 4 * nsc + 4 * nsc + stream_bytes, elements="bf16", groups=[n8, n4, n2])
+    line("mixed_decompress (+mean)", lambda: capi.mixed_decompress(mixed, out, order, counts, nsc, 2, stats=stats),
+         2 * n + 4 * nsc + 4 * nsc + stream_bytes, elements="bf16", groups=[n8, n4, n2])
     rows = torch.arange(0, nsc, 2, dtype=torch.int32, device=dev)
     nr = rows.numel()
     nb = capi.required_bytes(nr * 256, 4, 16, 2)
