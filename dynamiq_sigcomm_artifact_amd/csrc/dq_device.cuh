@@ -316,6 +316,17 @@ __device__ __forceinline__ void wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Transposes an 8 x 8 bit matrix held in a 64-bit word: bit 8 i + j becomes bit 8 j + i.  With byte i = the bin
+// of element i, byte p of the result holds bit p of the eight bins, element 0 in its lowest bit.
+__device__ __forceinline__ uint64_t transpose8x8(uint64_t x)
+{
+    uint64_t t;
+    t = 0x0f0f0f0f00000000ull & (x ^ (x << 28)); x ^= t ^ (t >> 28);
+    t = 0x3333000033330000ull & (x ^ (x << 14)); x ^= t ^ (t >> 14);
+    t = 0x5500550055005500ull & (x ^ (x << 7));  x ^= t ^ (t >> 7);
+    return x;
+}
+
 // floor(log2(v)) for v >= 1
 inline int ilog2(int64_t v)
 {

@@ -9,7 +9,7 @@
 //   norm    one workgroup folds work[] the same way -> sumsq (double); norm = sqrtf((float)sumsq)
 //   bins    x = (v * (float)sqrt(n)) / norm; bin = number of boundaries < x (torch.bucketize, right=False);
 //           bit plane p of 32 consecutive bins -> packed[p * n/32 + w]; the products centroid[bin] * v are
-//           summed in double with the tile scheme above -> work[b]
+//           summed in double, thread t adding elements 16 t + k of the tile (k ascending), then halved -> work[b]
 //   scale   dot = fold(work[]); scale = (norm * norm) / (float)dot
 // The sums are in double with a fixed association, so the result does not depend on the launch geometry
 // and the CPU restatement reproduces it bit for bit.
@@ -79,6 +79,10 @@ __global__ __launch_bounds__(kEdenThreads) void eden_norm_kernel(const double *_
     }
 }
 
+// Every thread owns sixteen consecutive elements (four 16-byte loads), so that it builds its half word of every
+// bit plane in registers.  The boundaries sit in LDS in breadth-first order of the search tree (node 1 = the
+// middle boundary, children of node i at 2 i and 2 i + 1): the lanes of a wave read one level of the tree at a
+// time, consecutive words, where the sorted layout puts a whole level into a few banks.
 template <int NBITS>
 __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__restrict__ vec, int64_t n,
                                                                 const float *__restrict__ boundaries,
@@ -88,11 +92,14 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
 {
     constexpr int L = 1 << NBITS;
     __shared__ double lds[kEdenThreads];
-    __shared__ float bnd[L], cen[L];
-    __shared__ uint32_t planes[NBITS][kEdenTile / 32]; // the tile's 128 words of every bit plane
+    __shared__ float tree[L], cen[L];
     for (int k = threadIdx.x; k < L; k += kEdenThreads) {
-        bnd[k] = k < L - 1 ? boundaries[k] : 0.0f;
         cen[k] = centroids[k];
+        if (k < L - 1) {
+            // sorted position k = (2 r + 1) 2^(NBITS - 1 - level) - 1 is node 2^level + r
+            const int tz = __builtin_ctz(k + 1);
+            tree[(1 << (NBITS - 1 - tz)) + ((k + 1) >> (tz + 1))] = boundaries[k];
+        }
     }
     __syncthreads();
     const float norm = result[3];
@@ -100,51 +107,56 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
     const bool ordinary = nb >= 0x0d800000u && nb <= 0x71800000u; // uniform over the grid
     const double yn = ordinary ? recip_f64(norm) : 0.0;
     const int64_t words = n >> 5;
-    const int64_t base = (int64_t)blockIdx.x * kEdenTile;
-    const int lane = threadIdx.x & 63;
-    // all sixteen elements of the thread walk the boundary table in lockstep: sixteen independent LDS reads
-    // per search step instead of one dependent chain per element
+    const int64_t first = (int64_t)blockIdx.x * kEdenTile + (int64_t)threadIdx.x * kEdenPerThread;
+    // n is a multiple of 32: the sixteen elements are all inside the vector or all outside
+    const bool in = first < n;
     float v[kEdenPerThread], x[kEdenPerThread];
-    int bin[kEdenPerThread];
+    int node[kEdenPerThread];
+    if (in) {
+        if ((reinterpret_cast<uintptr_t>(vec) & 15) == 0) { // uniform over the grid
 #pragma unroll
-    for (int k = 0; k < kEdenPerThread; k++) {
-        const int64_t i = base + threadIdx.x + (int64_t)kEdenThreads * k;
-        v[k] = i < n ? vec[i] : 0.0f;
+            for (int q = 0; q < kEdenPerThread / 4; q++) {
+                const float4 f = *reinterpret_cast<const float4 *>(vec + first + 4 * q);
+                v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < kEdenPerThread; k++) v[k] = vec[first + k];
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kEdenPerThread; k++) v[k] = 0.0f;
     }
 #pragma unroll
     for (int k = 0; k < kEdenPerThread; k++) {
         const float scaled = v[k] * sqrt_n;
         x[k] = ordinary ? div_by(scaled, yn) : scaled / norm;
-        bin[k] = 0;
+        node[k] = 1;
     }
+    // the sixteen searches advance level by level: sixteen independent LDS reads per level
 #pragma unroll
-    for (int step = L >> 1; step > 0; step >>= 1) {
+    for (int level = 0; level < NBITS; level++) {
 #pragma unroll
-        for (int k = 0; k < kEdenPerThread; k++) {
-            if (bnd[bin[k] + step - 1] < x[k]) bin[k] += step;
-        }
+        for (int k = 0; k < kEdenPerThread; k++) node[k] = 2 * node[k] + (tree[node[k]] < x[k] ? 1 : 0);
     }
     double acc = 0.0;
+    uint32_t four[kEdenPerThread / 4];
+#pragma unroll
+    for (int q = 0; q < kEdenPerThread / 4; q++) four[q] = 0;
 #pragma unroll
     for (int k = 0; k < kEdenPerThread; k++) {
-        const int64_t i = base + threadIdx.x + (int64_t)kEdenThreads * k;
-        const bool in = i < n;
-        if (in) acc += (double)cen[bin[k]] * (double)v[k];
-        const int w = (threadIdx.x >> 5) + 8 * k; // word of the tile
-#pragma unroll
-        for (int p = 0; p < NBITS; p++) {
-            const uint64_t m = __ballot(in && ((bin[k] >> p) & 1));
-            if ((lane & 31) == 0) planes[p][w] = (uint32_t)(m >> (lane & 32));
-        }
+        const int bin = node[k] - L;
+        if (in) acc += (double)cen[bin] * (double)v[k];
+        four[k >> 2] |= (uint32_t)bin << (8 * (k & 3));
     }
-    __syncthreads();
-    // 512 contiguous bytes per plane and tile
-    if (threadIdx.x < kEdenTile / 32) {
-        const int64_t w = (base >> 5) + threadIdx.x;
-        if (w < words) {
+    if (in) {
+        const uint64_t lo8 = transpose8x8((uint64_t)four[0] | ((uint64_t)four[1] << 32));
+        const uint64_t hi8 = transpose8x8((uint64_t)four[2] | ((uint64_t)four[3] << 32));
+        // plane p, word (first >> 5), half (first >> 4) & 1
+        uint16_t *half = reinterpret_cast<uint16_t *>(packed) + (first >> 4);
 #pragma unroll
-            for (int p = 0; p < NBITS; p++) packed[(int64_t)p * words + w] = planes[p][threadIdx.x];
-        }
+        for (int p = 0; p < NBITS; p++)
+            half[(int64_t)p * words * 2] = (uint16_t)(((lo8 >> (8 * p)) & 0xffu) | (((hi8 >> (8 * p)) & 0xffu) << 8));
     }
     const double total = fold256(acc, lds);
     if (threadIdx.x == 0) work[blockIdx.x] = total;

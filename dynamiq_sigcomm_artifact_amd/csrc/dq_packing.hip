@@ -1,24 +1,45 @@
 // EDEN bit-plane packing (csrc/cuda_packing.cu:11-29,76-95) and the THC-style
 // in-place stochastic rounding (csrc/cuda_hadamard.cu:607-627).
 //
-// Packing on wave64: one lane per bin, one 64-bit ballot per bit plane, whose
-// halves are the two consecutive 32-bin words of that plane.
 #include "dq_device.cuh"
 #include "dq_launch.h"
 
 namespace dq {
 
+// sixteen consecutive bins per thread, i.e. half a word of every bit plane: the bins' bytes go through two
+// 8 x 8 bit transposes (one per eight bins), after which byte j of a result is plane 8 s + j of those bins
+template <bool VEC>
 __global__ __launch_bounds__(256) void bins_to_bits_kernel(const int32_t *__restrict__ bins, int64_t nbins,
                                                            uint32_t *__restrict__ arr, int nbits)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t first = g * 16;
+    if (first >= nbins) return; // nbins is a multiple of 32
     const int64_t words = nbins >> 5;
-    const int lane = threadIdx.x & 63;
-    const uint32_t b = (i < nbins) ? (uint32_t)bins[i] : 0u;
-    const int64_t w = i >> 5;
-    for (int p = 0; p < nbits; p++) {
-        const uint64_t m = __ballot((b >> p) & 1u);
-        if ((lane & 31) == 0 && w < words) arr[(int64_t)p * words + w] = (uint32_t)(m >> (lane & 32));
+    uint32_t b[16];
+    if (VEC) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int4 v = *reinterpret_cast<const int4 *>(bins + first + 4 * q);
+            b[4 * q] = (uint32_t)v.x; b[4 * q + 1] = (uint32_t)v.y; b[4 * q + 2] = (uint32_t)v.z; b[4 * q + 3] = (uint32_t)v.w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) b[k] = (uint32_t)bins[first + k];
+    }
+    uint16_t *half = reinterpret_cast<uint16_t *>(arr) + g;
+    for (int s = 0; 8 * s < nbits; s++) {
+        uint64_t lo = 0, hi = 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            lo |= (uint64_t)((b[k] >> (8 * s)) & 0xffu) << (8 * k);
+            hi |= (uint64_t)((b[8 + k] >> (8 * s)) & 0xffu) << (8 * k);
+        }
+        lo = transpose8x8(lo);
+        hi = transpose8x8(hi);
+        const int planes = min(8, nbits - 8 * s);
+        for (int j = 0; j < planes; j++)
+            half[(int64_t)(8 * s + j) * words * 2] = (uint16_t)(((lo >> (8 * j)) & 0xffu) | (((hi >> (8 * j)) & 0xffu) << 8));
     }
 }
 
@@ -42,7 +63,11 @@ __global__ __launch_bounds__(256) void bits_to_bins_kernel(int32_t *__restrict__
 
 hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits, hipStream_t stream)
 {
-    hipLaunchKernelGGL(bins_to_bits_kernel, dim3((unsigned)((nbins + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
+    const dim3 grid((unsigned)((nbins / 16 + 255) / 256)), block(256);
+    if ((reinterpret_cast<uintptr_t>(bins) & 15) == 0)
+        hipLaunchKernelGGL(bins_to_bits_kernel<true>, grid, block, 0, stream, bins, nbins, arr, nbits);
+    else
+        hipLaunchKernelGGL(bins_to_bits_kernel<false>, grid, block, 0, stream, bins, nbins, arr, nbits);
     return hipGetLastError();
 }
 

@@ -864,7 +864,8 @@ static double halve256(double *lane)
     return lane[0];
 }
 
-static double tiled_sum(int64_t n, dqo_term_fn term, void *ctx)
+/* consecutive == 0: lane l of a tile adds elements l + 256 k; otherwise elements 16 l + k (k ascending either way) */
+static double tiled_sum(int64_t n, dqo_term_fn term, void *ctx, int consecutive)
 {
     const int64_t tiles = (n + 4095) / 4096;
     double *tile_sum = (double *)malloc((size_t)tiles * sizeof(double));
@@ -873,7 +874,7 @@ static double tiled_sum(int64_t n, dqo_term_fn term, void *ctx)
         for (int l = 0; l < 256; l++) {
             double acc = 0.0;
             for (int k = 0; k < 16; k++) {
-                int64_t i = b * 4096 + l + 256 * k;
+                int64_t i = b * 4096 + (consecutive ? 16 * l + k : l + 256 * k);
                 if (i < n) acc += term(i, ctx);
             }
             lane[l] = acc;
@@ -905,7 +906,7 @@ void dqo_eden_quantize(const float *vec, int64_t n, const float *boundaries, con
 {
     const int nb = (1 << nbits) - 1;
     struct eden_ctx ctx = {vec, centroids, bins};
-    const float sumsq = (float)tiled_sum(n, term_sq, &ctx);
+    const float sumsq = (float)tiled_sum(n, term_sq, &ctx, 0);
     const float norm = sqrtf(sumsq);
     const float sqrt_n = (float)sqrt((double)n);
     for (int64_t i = 0; i < n; i++) {
@@ -914,7 +915,7 @@ void dqo_eden_quantize(const float *vec, int64_t n, const float *boundaries, con
         while (b < nb && boundaries[b] < x) b++;
         bins[i] = b;
     }
-    const float dot = (float)tiled_sum(n, term_dot, &ctx);
+    const float dot = (float)tiled_sum(n, term_dot, &ctx, 1);
     result[0] = sumsq;
     result[1] = dot;
     result[2] = (norm * norm) / dot;

@@ -180,6 +180,19 @@ def test_bit_plane_packing(capi, oracle, eden_utils, nbits, nbins):
     assert torch.equal(back.cpu(), bins)
 
 
+@pytest.mark.parametrize("nbits", [3, 8, 9, 12, 17, 32])
+def test_bit_plane_packing_wide_and_misaligned(capi, oracle, nbits):
+    """planes beyond the first eight, bins with bits above nbits set (ignored), a source that is not 16-byte aligned"""
+    nbins = 32 * 77
+    g = torch.Generator().manual_seed(nbits)
+    store = torch.randint(-2 ** 31, 2 ** 31 - 1, (nbins + 3,), generator=g, dtype=torch.int32).to(DEV)
+    for off in (0, 1, 3):
+        bins = store[off:off + nbins]
+        arr = torch.zeros(nbins // 32 * nbits, dtype=torch.int32, device=DEV)
+        capi.bins_to_bits(bins, arr, nbits)
+        _eq("bins_to_bits", arr.cpu().numpy().view(np.uint32), oracle.bins_to_bits(bins.cpu().numpy(), nbits))
+
+
 def test_quantization_compression(eden_utils):
     """values land on floor/ceil of t = clamp(v/div, +-max), unbiased in the mean"""
     n = 1 << 20
