@@ -127,28 +127,39 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
 #pragma unroll
         for (int k = 0; k < kEdenPerThread; k++) v[k] = 0.0f;
     }
+    if (ordinary) {
 #pragma unroll
-    for (int k = 0; k < kEdenPerThread; k++) {
-        const float scaled = v[k] * sqrt_n;
-        x[k] = ordinary ? div_by(scaled, yn) : scaled / norm;
-        node[k] = 1;
+        for (int k = 0; k < kEdenPerThread; k++) x[k] = div_by(v[k] * sqrt_n, yn);
+    } else {
+#pragma unroll
+        for (int k = 0; k < kEdenPerThread; k++) x[k] = (v[k] * sqrt_n) / norm;
     }
-    // the sixteen searches advance level by level: sixteen independent LDS reads per level
+    // the sixteen searches advance level by level: sixteen independent LDS reads per level; node[] holds the
+    // node's byte offset into the table
+#pragma unroll
+    for (int k = 0; k < kEdenPerThread; k++) node[k] = 4;
 #pragma unroll
     for (int level = 0; level < NBITS; level++) {
 #pragma unroll
-        for (int k = 0; k < kEdenPerThread; k++) node[k] = 2 * node[k] + (tree[node[k]] < x[k] ? 1 : 0);
+        for (int k = 0; k < kEdenPerThread; k++) {
+            const float b = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(tree) + node[k]);
+            node[k] = 2 * node[k] + (b < x[k] ? 4 : 0);
+        }
     }
+    // the product of two floats is exact in double, so the fused multiply-add rounds like multiply, then add;
+    // threads past the end hold zeros and drop their sum below
     double acc = 0.0;
     uint32_t four[kEdenPerThread / 4];
 #pragma unroll
     for (int q = 0; q < kEdenPerThread / 4; q++) four[q] = 0;
 #pragma unroll
     for (int k = 0; k < kEdenPerThread; k++) {
-        const int bin = node[k] - L;
-        if (in) acc += (double)cen[bin] * (double)v[k];
-        four[k >> 2] |= (uint32_t)bin << (8 * (k & 3));
+        const uint32_t off = (uint32_t)(node[k] - 4 * L); // 4 * bin
+        const float c = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(cen) + off);
+        acc = __builtin_fma((double)c, (double)v[k], acc);
+        four[k >> 2] |= (k & 3) ? off << (8 * (k & 3) - 2) : off >> 2;
     }
+    if (!in) acc = 0.0;
     if (in) {
         const uint64_t lo8 = transpose8x8((uint64_t)four[0] | ((uint64_t)four[1] << 32));
         const uint64_t hi8 = transpose8x8((uint64_t)four[2] | ((uint64_t)four[3] << 32));
