@@ -316,6 +316,26 @@ __device__ __forceinline__ void wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// 16-byte slot s of a wave's output tile lives at LDS slot s ^ ((s >> 3) & 7): both
+// the per-lane writes (slots S*lane + j) and the lane-contiguous reads (slots
+// 64*k + lane) then touch eight distinct bank groups per eight lanes
+__device__ __forceinline__ int swz(int s) { return s ^ ((s >> 3) & 7); }
+
+// A wave holds 64 x 16 words, sixteen consecutive ones per lane; they leave as contiguous 16-byte pieces, lane
+// after lane.  tile: the wave's 256 LDS slots; dst: where the wave's first word goes (16-byte aligned);
+// valid_slots: how many of the 256 pieces lie inside the destination.  Every lane of the wave must call.
+__device__ __forceinline__ void store_wave_words16(uint4 *tile, const uint32_t (&w)[16], uint4 *dst, int lane, int valid_slots)
+{
+#pragma unroll
+    for (int j = 0; j < 4; j++) tile[swz(4 * lane + j)] = make_uint4(w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]);
+    wave_lds_sync();
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int s = 64 * k + lane;
+        if (s < valid_slots) dst[s] = tile[swz(s)];
+    }
+}
+
 // Transposes an 8 x 8 bit matrix held in a 64-bit word: bit 8 i + j becomes bit 8 j + i.  With byte i = the bin
 // of element i, byte p of the result holds bit p of the eight bins, element 0 in its lowest bit.
 __device__ __forceinline__ uint64_t transpose8x8(uint64_t x)

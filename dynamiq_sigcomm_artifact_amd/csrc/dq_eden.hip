@@ -187,27 +187,42 @@ __global__ __launch_bounds__(kEdenThreads) void eden_scale_kernel(const double *
     }
 }
 
-// four consecutive elements per thread: they share the 32-bin word of every bit plane
+// sixteen consecutive elements per thread: its half word of every bit plane, transposed back into sixteen bins;
+// the centroids leave through a per-wave LDS tile so that the lanes store contiguous 16-byte pieces
 template <int NBITS>
 __global__ __launch_bounds__(256) void eden_dequantize_kernel(const uint32_t *__restrict__ packed, int64_t n,
                                                               const float *__restrict__ centroids, float *__restrict__ out)
 {
     constexpr int L = 1 << NBITS;
     __shared__ float cen[L];
+    __shared__ __attribute__((aligned(16))) uint4 tiles[4][256];
     for (int k = threadIdx.x; k < L; k += 256) cen[k] = centroids[k];
     __syncthreads();
-    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= n) return;
-    const int64_t words = n >> 5, w = i >> 5;
-    const int t = (int)(i & 31);
-    uint32_t bins[4] = {0, 0, 0, 0};
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t first = g * 16, wave_first = (g - lane) * 16;
+    if (wave_first >= n) return; // the whole wave
+    const int64_t words = n >> 5;
+    uint64_t lo = 0, hi = 0;
+    if (first < n) { // n is a multiple of 32
+        const uint16_t *half = reinterpret_cast<const uint16_t *>(packed) + g;
 #pragma unroll
-    for (int p = 0; p < NBITS; p++) {
-        const uint32_t word = packed[(int64_t)p * words + w] >> t;
-#pragma unroll
-        for (int k = 0; k < 4; k++) bins[k] |= ((word >> k) & 1u) << p;
+        for (int p = 0; p < NBITS; p++) {
+            const uint32_t h = half[(int64_t)p * words * 2];
+            lo |= (uint64_t)(h & 0xffu) << (8 * p);
+            hi |= (uint64_t)(h >> 8) << (8 * p);
+        }
     }
-    *reinterpret_cast<float4 *>(out + i) = make_float4(cen[bins[0]], cen[bins[1]], cen[bins[2]], cen[bins[3]]);
+    lo = transpose8x8(lo);
+    hi = transpose8x8(hi);
+    uint32_t w[16];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        w[k] = __float_as_uint(cen[(lo >> (8 * k)) & 0xffu]);
+        w[8 + k] = __float_as_uint(cen[(hi >> (8 * k)) & 0xffu]);
+    }
+    store_wave_words16(tiles[wave], w, reinterpret_cast<uint4 *>(out + wave_first), lane,
+                       (int)min((int64_t)256, (n - wave_first) >> 2));
 }
 
 // ---- THC ------------------------------------------------------------------------------------------
@@ -293,9 +308,8 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
 hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits, float *out,
                                   hipStream_t stream)
 {
-    // n is a multiple of 32, so groups of four never straddle a word; out comes from an allocator (16-byte aligned)
-    // or at a multiple-of-32 element offset into one
-    dim3 grid((unsigned)((n / 4 + 255) / 256)), block(256);
+    // n is a multiple of 32 and out 16-byte aligned: a thread's sixteen elements are half a word of every plane
+    dim3 grid((unsigned)((n / 16 + 255) / 256)), block(256);
     switch (nbits) {
 #define DQ_EDEN_CASE(B)                                                                                      \
     case B: hipLaunchKernelGGL(eden_dequantize_kernel<B>, grid, block, 0, stream, packed, n, centroids, out); break;

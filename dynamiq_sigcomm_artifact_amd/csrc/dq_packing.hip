@@ -43,22 +43,42 @@ __global__ __launch_bounds__(256) void bins_to_bits_kernel(const int32_t *__rest
     }
 }
 
-// four consecutive bins per thread: they share the word of every bit plane
+// the inverse: sixteen consecutive bins per thread from its half word of every plane (the transpose is its own
+// inverse); the bins leave through a per-wave LDS tile so that the lanes store contiguous 16-byte pieces
 __global__ __launch_bounds__(256) void bits_to_bins_kernel(int32_t *__restrict__ bins, int64_t nbins,
                                                            const uint32_t *__restrict__ arr, int nbits)
 {
-    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= nbins) return;
+    __shared__ __attribute__((aligned(16))) uint4 tiles[4][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t first = g * 16, wave_first = (g - lane) * 16;
     const int64_t words = nbins >> 5;
-    const int64_t w = i >> 5;
-    const int t = (int)(i & 31);
-    int32_t v[4] = {0, 0, 0, 0};
-    for (int p = 0; p < nbits; p++) {
-        const uint32_t word = arr[(int64_t)p * words + w] >> t;
+    const bool in = first < nbins; // nbins is a multiple of 32
+    uint32_t b[16];
 #pragma unroll
-        for (int k = 0; k < 4; k++) v[k] += (int32_t)((word >> k) & 1u) << p;
+    for (int k = 0; k < 16; k++) b[k] = 0;
+    if (in) {
+        const uint16_t *half = reinterpret_cast<const uint16_t *>(arr) + g;
+        for (int s = 0; 8 * s < nbits; s++) {
+            uint64_t lo = 0, hi = 0;
+            const int planes = min(8, nbits - 8 * s);
+            for (int j = 0; j < planes; j++) {
+                const uint32_t h = half[(int64_t)(8 * s + j) * words * 2];
+                lo |= (uint64_t)(h & 0xffu) << (8 * j);
+                hi |= (uint64_t)(h >> 8) << (8 * j);
+            }
+            lo = transpose8x8(lo);
+            hi = transpose8x8(hi);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                b[k] |= (uint32_t)((lo >> (8 * k)) & 0xffu) << (8 * s);
+                b[8 + k] |= (uint32_t)((hi >> (8 * k)) & 0xffu) << (8 * s);
+            }
+        }
     }
-    *reinterpret_cast<int4 *>(bins + i) = make_int4(v[0], v[1], v[2], v[3]);
+    if (wave_first >= nbins) return; // the whole wave
+    store_wave_words16(tiles[wave], b, reinterpret_cast<uint4 *>(bins + wave_first), lane,
+                       (int)min((int64_t)256, (nbins - wave_first) >> 2));
 }
 
 hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int nbits, hipStream_t stream)
@@ -73,8 +93,8 @@ hipError_t launch_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr
 
 hipError_t launch_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr, int nbits, hipStream_t stream)
 {
-    // nbins is a multiple of 32 and bins a whole tensor: groups of four are 16-byte aligned
-    hipLaunchKernelGGL(bits_to_bins_kernel, dim3((unsigned)((nbins / 4 + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
+    // nbins is a multiple of 32 and bins 16-byte aligned: so is every group of sixteen
+    hipLaunchKernelGGL(bits_to_bins_kernel, dim3((unsigned)((nbins / 16 + 255) / 256)), dim3(256), 0, stream, bins, nbins, arr, nbits);
     return hipGetLastError();
 }
 

@@ -320,11 +320,6 @@ __device__ __forceinline__ float log2_det_ge1(float x)
     return (float)k + r;
 }
 
-// 16-byte slot s of a wave's output tile lives at LDS slot s ^ ((s >> 3) & 7): both
-// the per-lane writes (slots S*lane + j) and the lane-contiguous reads (slots
-// 64*k + lane) then touch eight distinct bank groups per eight lanes
-__device__ __forceinline__ int swz(int s) { return s ^ ((s >> 3) & 7); }
-
 template <int NBITS, bool MEE> static MeeArg<NBITS, MEE> make_arg(const MeeParams &mp)
 {
     MeeArg<NBITS, MEE> a;
