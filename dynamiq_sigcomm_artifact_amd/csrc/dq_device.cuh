@@ -347,6 +347,8 @@ __device__ __forceinline__ uint64_t transpose8x8(uint64_t x)
     return x;
 }
 
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 // floor(log2(v)) for v >= 1
 inline int ilog2(int64_t v)
 {

@@ -5,7 +5,11 @@
 // row, so the superchunk maximum is a row reduction without LDS or barriers.
 //
 // These kernels are the catch-all behind the C ABI: they also serve buffers
-// whose alignment rules out the vectorised chunk-16 kernels.  Numerics follow
+// whose alignment rules out the vectorised chunk-16 kernels.  For chunks of 8
+// and 32 elements in 16-byte aligned buffers the chunk size is a template
+// argument (CT): the thread's chunk then comes in through 16-byte loads and
+// stays in registers for both passes, and decoded chunks leave through a
+// swizzled per-wave LDS tile as lane-contiguous 16-byte stores.  Numerics follow
 // csrc/cuda_hadamard.cu:768-861,941-1234 (flat) and
 // csrc/cuda_hierarchical_mee.cu:698-1294 (hierarchical) of the reference.
 #include "dq_device.cuh"
@@ -52,26 +56,95 @@ __device__ __forceinline__ float row16_hmax(float v)
     return v;
 }
 
+// ---- a chunk of a compile-time size in registers ---------------------------------
+
+template <int DT> __device__ __forceinline__ float elem_from_bits(uint32_t b)
+{
+    return DT == DQ_F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+template <int DT> __device__ __forceinline__ uint32_t elem_to_bits(float v)
+{
+    return DT == DQ_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v);
+}
+
+// 16-byte pieces of a chunk of CT elements
+template <int DT, int CT> struct ChunkShape {
+    static constexpr int kBytes = CT * (int)sizeof(typename ElemIO<DT>::storage);
+    static constexpr int kSlots = kBytes / 16;
+};
+
+// the chunk starts on a 16-byte boundary
+template <int DT, int CT>
+__device__ __forceinline__ void load_chunk(const void *p, int64_t base, float (&v)[CT])
+{
+    constexpr int S = ChunkShape<DT, CT>::kSlots;
+    const uint4 *q = reinterpret_cast<const uint4 *>(static_cast<const char *>(p) + base * (ChunkShape<DT, CT>::kBytes / CT));
+#pragma unroll
+    for (int j = 0; j < S; j++) {
+        const uint4 w = q[j];
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            if (DT == DQ_F32) {
+                v[4 * j + k] = __uint_as_float(ww[k]);
+            } else {
+                v[8 * j + 2 * k] = elem_from_bits<DT>(ww[k] & 0xffffu);
+                v[8 * j + 2 * k + 1] = elem_from_bits<DT>(ww[k] >> 16);
+            }
+        }
+    }
+}
+
+// A wave's chunks, S 16-byte pieces per lane, leave as lane-contiguous pieces (see swz()).  tile: 64 S slots of
+// LDS owned by the wave; dst: where the wave's first piece goes; valid: pieces inside the destination.
+template <int S>
+__device__ __forceinline__ void store_wave_slots(uint4 *tile, const uint4 (&slot)[S], uint4 *dst, int lane, int valid)
+{
+#pragma unroll
+    for (int j = 0; j < S; j++) tile[swz(S * lane + j)] = slot[j];
+    wave_lds_sync();
+#pragma unroll
+    for (int k = 0; k < S; k++) {
+        const int s = 64 * k + lane;
+        if (s < valid) dst[s] = tile[swz(s)];
+    }
+}
+
 // ---- compress ----------------------------------------------------------------
 
-template <int DT, int RDT, bool HIER, bool MEE>
+// CT: the chunk size when it is 8 or 32 and src and rnd are 16-byte aligned, else 0
+template <int DT, int RDT, bool HIER, bool MEE, int CT>
 __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
     const void *__restrict__ src, uint8_t *__restrict__ dst, const void *__restrict__ rnd,
-    int64_t nchunks, int nbits, int C, MeeParams mp)
+    int64_t nchunks, int nbits, int Crt, MeeParams mp)
 {
     typedef ElemIO<DT> IO;
+    constexpr int kUnroll = CT ? CT : 1;
+    const int C = CT ? CT : Crt;
     const int64_t chunk = (int64_t)blockIdx.x * kGenericBlock + threadIdx.x;
     const bool active = chunk < nchunks; // hierarchical: whole 16-lane rows are active or not
     const int R = (1 << (nbits - 1)) - 1;
     const int PB = (C * nbits) >> 3;
     const int64_t base = chunk * C;
 
+    float ev[CT ? CT : 1], rv[CT ? CT : 1];
+    if (CT) {
+        if (active) {
+            load_chunk<DT, (CT ? CT : 1)>(src, base, ev);
+            load_chunk<RDT, (CT ? CT : 1)>(rnd, base, rv);
+        } else {
+#pragma unroll
+            for (int i = 0; i < (CT ? CT : 1); i++) ev[i] = rv[i] = 0.0f;
+        }
+    }
+
     // pass 1: chunk absmax
     float a = 0.0f;
     if (active) {
-        a = __builtin_fabsf(IO::load(src, base));
+        a = __builtin_fabsf(CT ? ev[0] : IO::load(src, base));
+#pragma unroll kUnroll
         for (int i = 1; i < C; i++) {
-            float v = __builtin_fabsf(IO::load(src, base + i));
+            float v = __builtin_fabsf(CT ? ev[CT ? i : 0] : IO::load(src, base + i));
             a = (DT == DQ_F16) ? h_max(a, v) : __builtin_fmaxf(a, v);
         }
     }
@@ -142,9 +215,10 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
 
     // pass 2: codes
     BytePacker pk(cb);
+#pragma unroll kUnroll
     for (int i = 0; i < C; i++) {
-        float v = IO::load(src, base + i);
-        float r = ElemIO<RDT>::load(rnd, base + i);
+        float v = CT ? ev[CT ? i : 0] : IO::load(src, base + i);
+        float r = CT ? rv[CT ? i : 0] : ElemIO<RDT>::load(rnd, base + i);
         int sv;
         if (DT == DQ_F16) {
             float x = h_div(v, d);
@@ -165,46 +239,87 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
 
 // ---- decompress ----------------------------------------------------------------
 
-template <int DT, bool HIER, bool MEE, bool ADD>
+// CT: the chunk size when it is 8 or 32 and dst is 16-byte aligned, else 0
+template <int DT, bool HIER, bool MEE, bool ADD, int CT>
 __global__ __launch_bounds__(kGenericBlock) void generic_decompress_kernel(
-    const uint8_t *__restrict__ src, void *__restrict__ dst, int64_t nchunks, int nbits, int C,
+    const uint8_t *__restrict__ src, void *__restrict__ dst, int64_t nchunks, int nbits, int Crt,
     MeeParams mp)
 {
     typedef ElemIO<DT> IO;
+    constexpr int CR = CT ? CT : 1;
+    constexpr int S = ChunkShape<DT, CR>::kSlots;
+    __shared__ __attribute__((aligned(16))) uint4 tiles[(CT && S > 1) ? kGenericBlock / 64 : 1][(CT && S > 1) ? 64 * S : 1];
+    const int C = CT ? CT : Crt;
     const int64_t chunk = (int64_t)blockIdx.x * kGenericBlock + threadIdx.x;
-    if (chunk >= nchunks) return;
+    const bool active = chunk < nchunks;
+    if (!CT && !active) return;
+    const int lane = threadIdx.x & 63;
+    if (CT && chunk - lane >= nchunks) return; // the whole wave
     const int R = (1 << (nbits - 1)) - 1;
     const int PB = (C * nbits) >> 3;
     const int64_t base = chunk * C;
 
-    const uint8_t *cb;
-    float sc;
-    if (HIER) {
-        const int CB = PB + 1;
-        const int64_t rec = (chunk >> 4) * (16 * CB + 2);
-        cb = src + rec + (chunk & 15) * CB;
-        uint32_t ub = (uint32_t)src[rec + 16 * CB] | ((uint32_t)src[rec + 16 * CB + 1] << 8);
-        if (DT == DQ_F16)
-            sc = h_mul((float)cb[PB], f16_bits_to_f32(ub));
-        else
-            sc = nonneg_scale((float)cb[PB] * nonneg_scale(bf16_bits_to_f32(ub)));
-    } else {
-        cb = src + chunk * (PB + 2);
-        uint32_t sb = (uint32_t)cb[PB] | ((uint32_t)cb[PB + 1] << 8);
-        sc = (DT == DQ_F16) ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb);
-    }
-
-    for (int i = 0; i < C; i++) {
-        int code = chunk_code(cb, i, nbits);
-        float lev = MEE ? f16_bits_to_f32(mp.table[code]) : (float)(code - R);
-        float v;
-        if (DT == DQ_F16) {
-            v = h_mul(lev, sc);
-            if (ADD) v = h_add(IO::load(dst, base + i), v);
+    float out[CR];
+#pragma unroll
+    for (int i = 0; i < CR; i++) out[i] = 0.0f;
+    if (active) {
+        const uint8_t *cb;
+        float sc;
+        if (HIER) {
+            const int CB = PB + 1;
+            const int64_t rec = (chunk >> 4) * (16 * CB + 2);
+            cb = src + rec + (chunk & 15) * CB;
+            uint32_t ub = (uint32_t)src[rec + 16 * CB] | ((uint32_t)src[rec + 16 * CB + 1] << 8);
+            if (DT == DQ_F16)
+                sc = h_mul((float)cb[PB], f16_bits_to_f32(ub));
+            else
+                sc = nonneg_scale((float)cb[PB] * nonneg_scale(bf16_bits_to_f32(ub)));
         } else {
-            v = ADD ? __builtin_fmaf(lev, sc, IO::load(dst, base + i)) : lev * sc;
+            cb = src + chunk * (PB + 2);
+            uint32_t sb = (uint32_t)cb[PB] | ((uint32_t)cb[PB + 1] << 8);
+            sc = (DT == DQ_F16) ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb);
         }
-        IO::store(dst, base + i, v);
+        float old[CR];
+        if (CT && ADD) load_chunk<DT, CR>(dst, base, old);
+
+#pragma unroll CR
+        for (int i = 0; i < C; i++) {
+            int code = chunk_code(cb, i, nbits);
+            float lev = MEE ? f16_bits_to_f32(mp.table[code]) : (float)(code - R);
+            float v;
+            if (DT == DQ_F16) {
+                v = h_mul(lev, sc);
+                if (ADD) v = h_add(CT ? old[CT ? i : 0] : IO::load(dst, base + i), v);
+            } else {
+                v = ADD ? __builtin_fmaf(lev, sc, CT ? old[CT ? i : 0] : IO::load(dst, base + i)) : lev * sc;
+            }
+            if (CT)
+                out[CT ? i : 0] = v;
+            else
+                IO::store(dst, base + i, v);
+        }
+    }
+    if constexpr (CT != 0) {
+        uint4 slot[S];
+#pragma unroll
+        for (int j = 0; j < S; j++) {
+            uint32_t w[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if (DT == DQ_F32)
+                    w[k] = __float_as_uint(out[4 * j + k]);
+                else
+                    w[k] = elem_to_bits<DT>(out[8 * j + 2 * k]) | (elem_to_bits<DT>(out[8 * j + 2 * k + 1]) << 16);
+            }
+            slot[j] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+        uint4 *wave_dst = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + (chunk - lane) * ChunkShape<DT, CR>::kBytes);
+        if constexpr (S == 1) {
+            if (active) wave_dst[lane] = slot[0];
+        } else {
+            const int valid = (int)min((int64_t)64, nchunks - (chunk - lane)) * S;
+            store_wave_slots<S>(tiles[threadIdx.x >> 6], slot, wave_dst, lane, valid);
+        }
     }
 }
 
@@ -216,12 +331,20 @@ static hipError_t launch_compress_t(const void *src, uint8_t *dst, const void *r
 {
     int64_t nchunks = n / C;
     unsigned grid = (unsigned)((nchunks + kGenericBlock - 1) / kGenericBlock);
-    if (DT == DQ_F32 && rand_bf16)
-        hipLaunchKernelGGL((generic_compress_kernel<DT, DQ_BF16, HIER, MEE>), dim3(grid), dim3(kGenericBlock), 0,
-                           stream, src, dst, rnd, nchunks, nbits, C, mp);
-    else
-        hipLaunchKernelGGL((generic_compress_kernel<DT, DT, HIER, MEE>), dim3(grid), dim3(kGenericBlock), 0,
-                           stream, src, dst, rnd, nchunks, nbits, C, mp);
+    const int ct = (aligned16(src) && aligned16(rnd) && (C == 8 || C == 32)) ? C : 0;
+#define DQ_GENERIC_COMPRESS(RDT, CT)                                                                                    \
+    hipLaunchKernelGGL((generic_compress_kernel<DT, RDT, HIER, MEE, CT>), dim3(grid), dim3(kGenericBlock), 0, stream, src, \
+                       dst, rnd, nchunks, nbits, C, mp)
+    if (DT == DQ_F32 && rand_bf16) {
+        if (ct == 32) DQ_GENERIC_COMPRESS(DQ_BF16, 32);
+        else if (ct == 8) DQ_GENERIC_COMPRESS(DQ_BF16, 8);
+        else DQ_GENERIC_COMPRESS(DQ_BF16, 0);
+    } else {
+        if (ct == 32) DQ_GENERIC_COMPRESS(DT, 32);
+        else if (ct == 8) DQ_GENERIC_COMPRESS(DT, 8);
+        else DQ_GENERIC_COMPRESS(DT, 0);
+    }
+#undef DQ_GENERIC_COMPRESS
     return hipGetLastError();
 }
 
@@ -231,12 +354,20 @@ static hipError_t launch_decompress_t(const uint8_t *src, void *dst, int64_t n, 
 {
     int64_t nchunks = n / C;
     unsigned grid = (unsigned)((nchunks + kGenericBlock - 1) / kGenericBlock);
-    if (add)
-        hipLaunchKernelGGL((generic_decompress_kernel<DT, HIER, MEE, true>), dim3(grid),
-                           dim3(kGenericBlock), 0, stream, src, dst, nchunks, nbits, C, mp);
-    else
-        hipLaunchKernelGGL((generic_decompress_kernel<DT, HIER, MEE, false>), dim3(grid),
-                           dim3(kGenericBlock), 0, stream, src, dst, nchunks, nbits, C, mp);
+    const int ct = (aligned16(dst) && (C == 8 || C == 32)) ? C : 0;
+#define DQ_GENERIC_DECOMPRESS(ADD, CT)                                                                                    \
+    hipLaunchKernelGGL((generic_decompress_kernel<DT, HIER, MEE, ADD, CT>), dim3(grid), dim3(kGenericBlock), 0, stream, src, \
+                       dst, nchunks, nbits, C, mp)
+    if (add) {
+        if (ct == 32) DQ_GENERIC_DECOMPRESS(true, 32);
+        else if (ct == 8) DQ_GENERIC_DECOMPRESS(true, 8);
+        else DQ_GENERIC_DECOMPRESS(true, 0);
+    } else {
+        if (ct == 32) DQ_GENERIC_DECOMPRESS(false, 32);
+        else if (ct == 8) DQ_GENERIC_DECOMPRESS(false, 8);
+        else DQ_GENERIC_DECOMPRESS(false, 0);
+    }
+#undef DQ_GENERIC_DECOMPRESS
     return hipGetLastError();
 }
 

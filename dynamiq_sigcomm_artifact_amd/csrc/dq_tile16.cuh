@@ -329,6 +329,5 @@ template <int NBITS, bool MEE> static MeeArg<NBITS, MEE> make_arg(const MeeParam
     return a;
 }
 
-static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 } // namespace dq

@@ -98,6 +98,35 @@ def test_functional_sweep(capi, oracle, dt, C, nbits, strategy):
               make_rand(n, 3000 + nbits * 19 + C + strategy, tdt), tag)
 
 
+@pytest.mark.parametrize("dt", [F16, BF16, F32])
+@pytest.mark.parametrize("C", [8, 32])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+def test_chunks_of_8_and_32_in_aligned_buffers(capi, oracle, dt, C, strategy):
+    """chunk sizes 8 and 32 in 16-byte aligned buffers (the kernels that keep the chunk in registers): chunk counts
+    that end inside a wave, inside a workgroup and past one, every width the chunk size allows, canaries around the
+    decoded vector"""
+    tdt = TORCH_DT[dt]
+    for nbits in (2, 3, 4, 5, 8):
+        if (C * nbits) % 8:
+            continue
+        for nchunks in (16, 48, 208, 256 + 80, 1024 + 16):
+            n = C * nchunks
+            g = torch.Generator().manual_seed(C * 1000 + nbits * 10 + strategy + nchunks)
+            src = (torch.randn(n, generator=g) * 0.02).to(tdt)
+            src[5] = float("inf") if nchunks == 48 else src[5]
+            rnd = torch.rand(n, generator=g).to(tdt)
+            tag = "dt=%d C=%d b=%d s=%d chunks=%d" % (dt, C, nbits, strategy, nchunks)
+            enc_o = _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src, rnd, tag)
+            # the decoded vector inside a larger buffer, 16-byte aligned at both ends
+            pad = 16
+            buf = torch.full((n + 2 * pad,), 3.0, dtype=tdt, device=DEV)
+            capi.scaling_decompress(torch.from_numpy(enc_o).to(DEV), buf[pad:pad + n], n, nbits, C, strategy)
+            got = buf.float().cpu()
+            assert bool((got[:pad] == 3).all()) and bool((got[pad + n:] == 3).all()), tag + " wrote outside the vector"
+            inp = (torch.randn(n, generator=g) * 0.01).to(tdt)
+            _dec_comp(capi, oracle, dt, n, nbits, C, strategy, src, inp, rnd, torch.rand(n, generator=g).to(tdt), tag)
+
+
 @pytest.mark.parametrize("dt", [BF16, F32])
 @pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [2, 3])
