@@ -12,8 +12,10 @@
 // swizzled per-wave LDS tile as lane-contiguous 16-byte stores.  Numerics follow
 // csrc/cuda_hadamard.cu:768-861,941-1234 (flat) and
 // csrc/cuda_hierarchical_mee.cu:698-1294 (hierarchical) of the reference.
-#include "dq_device.cuh"
+#include <type_traits>
+
 #include "dq_launch.h"
+#include "dq_tile16.cuh"
 
 namespace dq {
 
@@ -109,6 +111,10 @@ __device__ __forceinline__ void store_wave_slots(uint4 *tile, const uint4 (&slot
         if (s < valid) dst[s] = tile[swz(s)];
     }
 }
+
+// LDS bytes for the packed run of a wave's 64 chunks of CT elements at up to 8 bits (flat: 64 (CT + 2),
+// hierarchical: 4 (16 (CT + 1) + 2)), its 16-byte phase and the rounding up to whole 16-byte pieces
+template <int CT> struct WindowBytes { static constexpr int value = CT ? 64 * CT + 160 : 16; };
 
 // ---- compress ----------------------------------------------------------------
 
@@ -213,28 +219,36 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
     }
     if (!active) return;
 
-    // pass 2: codes
+    // pass 2: codes.  v / d is the correctly rounded quotient either way: with the chunk in registers and d an
+    // ordinary number it is the product with 1/d in double (see div_by), otherwise the IEEE division
     BytePacker pk(cb);
+    const auto codes = [&](auto fast) {
+        const double yd = decltype(fast)::value ? recip_f64(d) : 0.0;
 #pragma unroll kUnroll
-    for (int i = 0; i < C; i++) {
-        float v = CT ? ev[CT ? i : 0] : IO::load(src, base + i);
-        float r = CT ? rv[CT ? i : 0] : ElemIO<RDT>::load(rnd, base + i);
-        int sv;
-        if (DT == DQ_F16) {
-            float x = h_div(v, d);
-            if (MEE) x = mee_inverse_half(x, mp.c, mp.l2b);
-            sv = sr_half(x, r);
-        } else if (HIER) {
-            float x = v / d;
-            if (MEE) x = mee_inverse_guarded(x, mp.c, mp.l2b);
-            sv = sr_guarded(x, r);
-        } else {
-            float x = v / d;
-            if (MEE) x = mee_inverse_plain(x, mp.c, mp.l2b);
-            sv = sr_plain(x, r);
+        for (int i = 0; i < C; i++) {
+            float v = CT ? ev[CT ? i : 0] : IO::load(src, base + i);
+            float r = CT ? rv[CT ? i : 0] : ElemIO<RDT>::load(rnd, base + i);
+            float x = decltype(fast)::value ? div_by(v, yd) : v / d;
+            int sv;
+            if (DT == DQ_F16) {
+                x = rh(x);
+                if (MEE) x = mee_inverse_half(x, mp.c, mp.l2b);
+                sv = sr_half(x, r);
+            } else if (HIER) {
+                if (MEE) x = mee_inverse_guarded(x, mp.c, mp.l2b);
+                sv = sr_guarded(x, r);
+            } else {
+                if (MEE) x = mee_inverse_plain(x, mp.c, mp.l2b);
+                sv = sr_plain(x, r);
+            }
+            pk.put(clamp_code(sv, R), nbits);
         }
-        pk.put(clamp_code(sv, R), nbits);
-    }
+    };
+    const uint32_t db = __float_as_uint(d);
+    if (CT && db >= 0x0d800000u && db <= 0x71800000u) // a normal number in [2^-100, 2^100]
+        codes(std::true_type{});
+    else
+        codes(std::false_type{});
 }
 
 // ---- decompress ----------------------------------------------------------------
@@ -254,10 +268,30 @@ __global__ __launch_bounds__(kGenericBlock) void generic_decompress_kernel(
     const bool active = chunk < nchunks;
     if (!CT && !active) return;
     const int lane = threadIdx.x & 63;
-    if (CT && chunk - lane >= nchunks) return; // the whole wave
+    const int64_t wave_first = chunk - lane;
+    if (CT && wave_first >= nchunks) return; // the whole wave
     const int R = (1 << (nbits - 1)) - 1;
     const int PB = (C * nbits) >> 3;
     const int64_t base = chunk * C;
+
+    // CT: the wave's packed run comes in as 16-byte pieces into an LDS window (byte k of the run at win[mis + k])
+    __shared__ __attribute__((aligned(16))) uint8_t wins[CT ? kGenericBlock / 64 : 1][WindowBytes<CT>::value];
+    const int64_t run_start = !CT ? 0 : HIER ? (wave_first >> 4) * (16 * (PB + 1) + 2) : wave_first * (PB + 2);
+    const uint8_t *ibase;
+    if constexpr (CT != 0) {
+        const uint8_t *g = src + run_start;
+        const int mis = (int)(reinterpret_cast<uintptr_t>(g) & 15);
+        const int nact = (int)min((int64_t)64, nchunks - wave_first);
+        const int total = HIER ? (nact >> 4) * (16 * (PB + 1) + 2) : nact * (PB + 2);
+        const int nvec = (mis + total + 15) >> 4;
+        const u32x4 *ga = reinterpret_cast<const u32x4 *>(g - mis);
+        u32x4 *wv = reinterpret_cast<u32x4 *>(wins[threadIdx.x >> 6]);
+        for (int v = lane; v < nvec; v += 64) wv[v] = ga[v];
+        wave_lds_sync();
+        ibase = wins[threadIdx.x >> 6] + mis;
+    } else {
+        ibase = src;
+    }
 
     float out[CR];
 #pragma unroll
@@ -267,15 +301,15 @@ __global__ __launch_bounds__(kGenericBlock) void generic_decompress_kernel(
         float sc;
         if (HIER) {
             const int CB = PB + 1;
-            const int64_t rec = (chunk >> 4) * (16 * CB + 2);
-            cb = src + rec + (chunk & 15) * CB;
-            uint32_t ub = (uint32_t)src[rec + 16 * CB] | ((uint32_t)src[rec + 16 * CB + 1] << 8);
+            const int64_t rec = (chunk >> 4) * (16 * CB + 2) - run_start;
+            cb = ibase + rec + (chunk & 15) * CB;
+            uint32_t ub = (uint32_t)ibase[rec + 16 * CB] | ((uint32_t)ibase[rec + 16 * CB + 1] << 8);
             if (DT == DQ_F16)
                 sc = h_mul((float)cb[PB], f16_bits_to_f32(ub));
             else
                 sc = nonneg_scale((float)cb[PB] * nonneg_scale(bf16_bits_to_f32(ub)));
         } else {
-            cb = src + chunk * (PB + 2);
+            cb = ibase + (chunk * (PB + 2) - run_start);
             uint32_t sb = (uint32_t)cb[PB] | ((uint32_t)cb[PB + 1] << 8);
             sc = (DT == DQ_F16) ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb);
         }
@@ -313,11 +347,11 @@ __global__ __launch_bounds__(kGenericBlock) void generic_decompress_kernel(
             }
             slot[j] = make_uint4(w[0], w[1], w[2], w[3]);
         }
-        uint4 *wave_dst = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + (chunk - lane) * ChunkShape<DT, CR>::kBytes);
+        uint4 *wave_dst = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + wave_first * ChunkShape<DT, CR>::kBytes);
         if constexpr (S == 1) {
             if (active) wave_dst[lane] = slot[0];
         } else {
-            const int valid = (int)min((int64_t)64, nchunks - (chunk - lane)) * S;
+            const int valid = (int)min((int64_t)64, nchunks - wave_first) * S;
             store_wave_slots<S>(tiles[threadIdx.x >> 6], slot, wave_dst, lane, valid);
         }
     }

@@ -113,7 +113,13 @@ def test_chunks_of_8_and_32_in_aligned_buffers(capi, oracle, dt, C, strategy):
             n = C * nchunks
             g = torch.Generator().manual_seed(C * 1000 + nbits * 10 + strategy + nchunks)
             src = (torch.randn(n, generator=g) * 0.02).to(tdt)
-            src[5] = float("inf") if nchunks == 48 else src[5]
+            if nchunks == 48:
+                src[5] = float("inf")
+            if nchunks == 208:                      # NaN, -inf, a zero chunk, a chunk of tiny values, one of huge ones
+                src[7], src[C + 3] = float("nan"), float("-inf")
+                src[2 * C:3 * C] = 0.0
+                src[3 * C:4 * C] = (torch.randn(C, generator=g) * 1e-30).to(tdt)
+                src[4 * C:5 * C] = (torch.randn(C, generator=g) * (6e4 if dt == F16 else 1e30)).to(tdt)
             rnd = torch.rand(n, generator=g).to(tdt)
             tag = "dt=%d C=%d b=%d s=%d chunks=%d" % (dt, C, nbits, strategy, nchunks)
             enc_o = _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src, rnd, tag)
