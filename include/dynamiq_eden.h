@@ -264,10 +264,12 @@ int64_t dq_eden_work_doubles(int64_t n);
  *   packed  = bit planes of the bins, uint32 [n / 32 * nbits]
  *   result  = float32 [4] on the device: sum of squares, <centroids[bin], vec>,
  *             scale = ||vec||^2 / <centroids[bin], vec>, ||vec||
- * Sums are accumulated in double in a fixed order (4096-element tiles, stride
- * 256 inside a tile, halving trees), so the result is independent of the launch
- * shape; torch's own reduction order is not specified, hence `scale` agrees with
- * the reference to rounding error, not bit for bit. */
+ * Sums are accumulated in double in a fixed order (4096-element tiles, 256
+ * partial sums per tile -- of elements t + 256 k for the sum of squares, of
+ * elements 16 t + k for the dot product, k ascending -- then halving trees), so
+ * the result is independent of the launch shape; torch's own reduction order is
+ * not specified, hence `scale` agrees with the reference to rounding error, not
+ * bit for bit. */
 int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,
                      int nbits, uint32_t *packed, float *result, double *work,
                      int64_t work_doubles, int device, dq_stream_t stream);
