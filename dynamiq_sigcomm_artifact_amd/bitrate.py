@@ -102,3 +102,38 @@ def dynamic_bitrate_adjust_u(norms_list, prev_u, target_avg_bits):
             return u, avg, delta
         step *= 0.5
     return best.triple()
+
+
+class NormHistogram(object):
+    """The two searches above without a pass over the norms per probe: the norm patterns of every bucket are counted
+    into a device histogram (``add``, one small launch per bucket, after the statistics all-reduce), and one launch runs
+    the whole search on the counts.  Same (u, average, delta) as the functions above on the same norms; one read-back
+    per search instead of one per probe."""
+
+    def __init__(self, device):
+        from . import capi
+        self._capi = capi
+        self.hist = torch.zeros(capi.bitrate_hist_ints(), dtype=torch.int32, device=device)
+        self.result = torch.zeros(4, dtype=torch.float64, device=device)
+        self.count = 0
+
+    def add(self, stats, stream=None):
+        """stats: bf16 [nsc, 2] as written by superchunk_mean_center / superchunk_stats"""
+        self._capi.norm_histogram(stats, self.hist, stream)
+        self.count += stats.numel() // 2
+
+    def _search(self, mode, prev_u, target_avg_bits, stream):
+        self._capi.bitrate_search(self.hist, mode, prev_u, target_avg_bits, self.result, stream)
+        self.count = 0                      # the kernel leaves the histogram zeroed
+        if hasattr(stream, "synchronize"):
+            stream.synchronize()            # tolist() below only waits for torch's current stream
+        u, avg, delta, _ = self.result.tolist()
+        return u, avg, delta
+
+    def binary_search_u(self, target_avg_bits, stream=None):
+        """comm_hooks.py:94-114 on the norms added since the last search"""
+        return self._search(0, DYNAMIC_BITRATE_U_MAX, target_avg_bits, stream)
+
+    def adjust_u(self, prev_u, target_avg_bits, stream=None):
+        """comm_hooks.py:117-139 on the norms added since the last search"""
+        return self._search(1, prev_u, target_avg_bits, stream)

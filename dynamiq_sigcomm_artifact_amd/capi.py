@@ -22,6 +22,7 @@ EXPORTS = [
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
     "dq_scaling_compress_philox", "dq_scaling_dec_comp_philox", "dq_philox_uniform",
     "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
+    "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
@@ -75,6 +76,12 @@ def lib():
         L.dq_group_plan.argtypes = [vp, i64, vp, vp, i64, i32, vp]
         L.dq_group_plan_stats.restype = i32
         L.dq_group_plan_stats.argtypes = [vp, c.c_double, i64, vp, vp, vp, i64, i32, vp]
+        L.dq_bitrate_hist_ints.restype = i64
+        L.dq_bitrate_hist_ints.argtypes = []
+        L.dq_norm_histogram.restype = i32
+        L.dq_norm_histogram.argtypes = [vp, i64, vp, i64, i32, vp]
+        L.dq_bitrate_search.restype = i32
+        L.dq_bitrate_search.argtypes = [vp, i64, i32, c.c_double, c.c_double, vp, i32, vp]
         L.dq_scaling_compress_rows.restype = i32
         L.dq_scaling_compress_rows.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_scaling_dec_comp_rows.restype = i32
@@ -229,6 +236,27 @@ def group_plan_stats(stats, u, qbits_out, order, work, stream=None):
         raise RuntimeError("group_plan_stats: order / qbits_out too small or of the wrong dtype")
     _check(lib().dq_group_plan_stats(stats.data_ptr(), float(u), nsc, _ptr(qbits_out), order.data_ptr(), work.data_ptr(),
                                      work.numel(), _dev(stats), _stream(stream)))
+
+
+def bitrate_hist_ints():
+    return int(lib().dq_bitrate_hist_ints())
+
+
+def norm_histogram(stats, hist, stream=None):
+    """adds the norm patterns of stats (bf16 [nsc, 2]: mean, reduced sum of squares) to hist (int32 [bitrate_hist_ints()])"""
+    if stats.dtype != torch.bfloat16 or hist.dtype != torch.int32:
+        raise RuntimeError("norm_histogram: stats must be bfloat16 and hist int32")
+    _check(lib().dq_norm_histogram(stats.data_ptr(), stats.numel() // 2, hist.data_ptr(), hist.numel(), _dev(stats),
+                                   _stream(stream)))
+
+
+def bitrate_search(hist, mode, prev_u, target_avg_bits, result, stream=None):
+    """mode 0: bisection, 1: correction from prev_u; result float64 [4] = u, average width, target - average, probes;
+    hist comes back zeroed"""
+    if hist.dtype != torch.int32 or result.dtype != torch.float64 or result.numel() < 4:
+        raise RuntimeError("bitrate_search: hist must be int32 and result float64 [4]")
+    _check(lib().dq_bitrate_search(hist.data_ptr(), hist.numel(), int(mode), float(prev_u), float(target_avg_bits),
+                                   result.data_ptr(), _dev(hist), _stream(stream)))
 
 
 def scaling_compress_rows(src, rows, dst, rand_pool, nrows, nbits, strategy, stream=None):

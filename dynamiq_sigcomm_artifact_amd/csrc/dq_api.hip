@@ -311,6 +311,30 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
     return finish(dq::launch_group_plan_stats(stats, (float)u, nsc, qbits_out, order, work, static_cast<hipStream_t>(stream)));
 }
 
+int64_t dq_bitrate_hist_ints(void) { return dq::bitrate_hist_ints(); }
+
+int dq_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, int64_t hist_ints, int device, dq_stream_t stream)
+{
+    if (!(nsc > 0) || nsc > (int64_t)0x7fffffff) return fail(DQ_ERR_N, "nsc must be in [1, 2^31)");
+    if (!stats || !hist) return fail(DQ_ERR_NULL);
+    if (hist_ints < dq::bitrate_hist_ints()) return fail(DQ_ERR_SIZE, "hist buffer is too small");
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_norm_histogram(stats, nsc, hist, static_cast<hipStream_t>(stream)));
+}
+
+int dq_bitrate_search(uint32_t *hist, int64_t hist_ints, int mode, double prev_u, double target_avg_bits, double *result,
+                      int device, dq_stream_t stream)
+{
+    if (mode != 0 && mode != 1) return fail(DQ_ERR_SIZE, "mode must be 0 (bisection) or 1 (correction from prev_u)");
+    if (!hist || !result) return fail(DQ_ERR_NULL);
+    if (hist_ints < dq::bitrate_hist_ints()) return fail(DQ_ERR_SIZE, "hist buffer is too small");
+    if (prev_u != prev_u || target_avg_bits != target_avg_bits) return fail(DQ_ERR_SIZE, "prev_u and target_avg_bits must be numbers");
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_bitrate_search(hist, mode, prev_u, target_avg_bits, result, static_cast<hipStream_t>(stream)));
+}
+
 static int check_rows(int64_t nrows, int nbits, int dtype, int strategy, bool rand)
 {
     if (!(nrows > 0) || nrows > (int64_t)0x7fffffff) return DQ_ERR_N;

@@ -1,0 +1,189 @@
+// The search for the offset u of the dynamic bit-width rule
+// (testbed_evaluation/new_comm_hooks/comm_hooks.py:73-139) without a pass over the norms per probe.
+//
+// The reference evaluates the average width at every probe of u with ten torch ops and a reduction over the
+// norm tensors of all buckets, and reads the sum back to the host each time (up to 33 probes per search).
+// The width of a superchunk depends on its norm only through the bf16 pattern, and as a function of the
+// pattern it is a step function with two steps.  So:
+//   norm_histogram_kernel   counts the norm patterns of a bucket's statistics into a histogram (one pass per
+//                           bucket, accumulated over the buckets of a training step);
+//   bitrate_search_kernel   one workgroup: turns the histogram into suffix counts, then runs the reference's
+//                           whole bisection (or its incremental correction) in double, each probe being two
+//                           threshold searches over the patterns and two look-ups.
+// The result (u, average width, target - average) equals what the torch ops of the reference give for the same
+// norms: the counts are exact integers and the arithmetic of the search is the same IEEE double arithmetic.
+#include "dq_bitwidth.cuh"
+#include "dq_launch.h"
+
+namespace dq {
+
+namespace {
+
+constexpr int kNanBin = kMaxPattern + 1;       // NaN norms: 2 bits whatever u is
+constexpr int kSearchThreads = 1024;
+constexpr int kBinsPerThread = 32;             // 1024 x 32 = 32768 >= kNanBin + 1
+
+// negative norms (and -0) are clamped to the same epsilon as +0: bin 0
+__device__ __forceinline__ int bin_of(uint32_t pattern)
+{
+    if (pattern <= (uint32_t)kMaxPattern) return (int)pattern;
+    return (pattern & 0x7fffu) > (uint32_t)kMaxPattern ? kNanBin : 0;
+}
+
+// A workgroup counts rounds of up to 8192 norms in LDS -- 16-bit counters, two per word, so the whole range of
+// patterns fits into 64 KB -- and adds the non-zero counters to the histogram in memory after each round: a few
+// hundred atomics per round instead of one per norm, most of which would hit the same few hundred words.
+constexpr int kHistThreads = 1024;
+constexpr int kHistRound = 8192;               // norms per round (a 16-bit counter holds up to 65535)
+constexpr int kHistWords = 16384;              // 32768 counters
+
+__global__ __launch_bounds__(kHistThreads) void norm_histogram_kernel(const uint16_t *__restrict__ stats, int64_t nsc,
+                                                                     uint32_t *__restrict__ hist)
+{
+    __shared__ uint32_t local[kHistWords];
+    const int t = threadIdx.x;
+    for (int64_t round0 = (int64_t)blockIdx.x * kHistRound; round0 < nsc; round0 += (int64_t)gridDim.x * kHistRound) {
+        for (int w = t; w < kHistWords; w += kHistThreads) local[w] = 0u;
+        __syncthreads();
+        const int64_t end = min(round0 + kHistRound, nsc);
+        for (int64_t i = round0 + t; i < end; i += kHistThreads) {
+            const int bin = bin_of(stats[2 * i + 1]);
+            atomicAdd(&local[bin >> 1], 1u << (16 * (bin & 1)));
+        }
+        __syncthreads();
+        for (int w = t; w < kHistWords; w += kHistThreads) {
+            const uint32_t pair = local[w];
+            if (pair & 0xffffu) atomicAdd(&hist[2 * w], pair & 0xffffu);
+            if (pair >> 16) atomicAdd(&hist[2 * w + 1], pair >> 16);
+        }
+        __syncthreads();
+    }
+}
+
+struct Probe {
+    double avg, delta;
+};
+
+// out[0..2] = u, average width, target - average; out[3] = number of probes.  hist: pattern counts in, zeros out.
+__global__ __launch_bounds__(kSearchThreads) void bitrate_search_kernel(uint32_t *__restrict__ hist, int mode, double prev_u,
+                                                                       double target, double *__restrict__ out)
+{
+    __shared__ uint32_t part[kSearchThreads];
+    __shared__ int thr[2];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+    // suffix counts in place: hist[p] = number of norms whose pattern is >= p, p = 0 .. kMaxPattern
+    uint32_t v[kBinsPerThread];
+    uint32_t own = 0;
+#pragma unroll
+    for (int k = 0; k < kBinsPerThread; k++) {
+        const int p = kBinsPerThread * t + k;
+        v[k] = p <= kMaxPattern ? hist[p] : 0u;
+        own += v[k];
+    }
+    part[t] = own;
+    __syncthreads();
+    for (int off = 1; off < kSearchThreads; off <<= 1) {
+        const uint32_t x = t + off < kSearchThreads ? part[t + off] : 0u;
+        __syncthreads();
+        part[t] += x;
+        __syncthreads();
+    }
+    uint32_t run = part[t] - own; // the bins of the threads above
+#pragma unroll
+    for (int k = kBinsPerThread - 1; k >= 0; k--) {
+        const int p = kBinsPerThread * t + k;
+        run += v[k];
+        if (p <= kMaxPattern) hist[p] = run;
+    }
+    __syncthreads();
+    const uint64_t total = (uint64_t)hist[0] + hist[kNanBin];
+
+    int probes = 0;
+    // every thread evaluates the same doubles, so the control flow below is uniform without a broadcast
+    const auto probe = [&](double u) {
+        width_thresholds((float)u, thr, wave, lane);
+        __syncthreads();
+        const int t4 = thr[0], t8 = thr[1];
+        const uint64_t n4 = t4 <= kMaxPattern ? hist[t4] : 0u, n8 = t8 <= kMaxPattern ? hist[t8] : 0u;
+        __syncthreads();
+        probes++;
+        Probe r;
+        r.avg = total ? (double)(2 * total + 2 * n4 + 4 * n8) / (double)total : 0.0;
+        r.delta = target - r.avg;
+        return r;
+    };
+    const double u_min = -10.0, u_max = 60.0, tol = 0.1;
+    double res_u, res_avg, res_delta;
+    if (mode == 0) {
+        // comm_hooks.py:94-114
+        double low = u_min, high = u_max;
+        Probe r = probe(high);
+        double best_u = high, best_avg = r.avg, best_delta = r.delta;
+        bool done = false;
+        for (int it = 0; it < 32 && !done; it++) {
+            const double mid = (low + high) * 0.5;
+            r = probe(mid);
+            if (__builtin_fabs(r.delta) < __builtin_fabs(best_delta)) {
+                best_u = mid; best_avg = r.avg; best_delta = r.delta;
+            }
+            if (__builtin_fabs(r.delta) <= tol) {
+                best_u = mid; best_avg = r.avg; best_delta = r.delta;
+                done = true;
+            } else if (r.delta > 0) {
+                low = mid;
+            } else {
+                high = mid;
+            }
+        }
+        res_u = best_u; res_avg = best_avg; res_delta = best_delta;
+    } else {
+        // comm_hooks.py:117-139
+        const double start = __builtin_fmax(u_min, __builtin_fmin(u_max, prev_u));
+        Probe r = probe(start);
+        res_u = start; res_avg = r.avg; res_delta = r.delta;
+        if (!(__builtin_fabs(r.delta) <= tol)) {
+            const double old_delta = r.delta;
+            double step = old_delta;
+            bool done = false;
+            for (int it = 0; it < 32 && !done; it++) {
+                const double cand = __builtin_fmax(u_min, __builtin_fmin(u_max, start + step));
+                r = probe(cand);
+                if (__builtin_fabs(r.delta) < __builtin_fabs(res_delta)) {
+                    res_u = cand; res_avg = r.avg; res_delta = r.delta;
+                }
+                if (__builtin_fabs(r.delta) <= tol || old_delta * r.delta >= 0) {
+                    res_u = cand; res_avg = r.avg; res_delta = r.delta;
+                    done = true;
+                }
+                step *= 0.5;
+            }
+        }
+    }
+    if (t == 0) {
+        out[0] = res_u; out[1] = res_avg; out[2] = res_delta; out[3] = (double)probes;
+    }
+    // ready for the next accumulation
+#pragma unroll
+    for (int k = 0; k < kBinsPerThread; k++) hist[kBinsPerThread * t + k] = 0u;
+}
+
+} // namespace
+
+int64_t bitrate_hist_ints() { return (int64_t)kSearchThreads * kBinsPerThread; }
+
+hipError_t launch_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, hipStream_t stream)
+{
+    const unsigned grid = (unsigned)std::min<int64_t>((nsc + kHistRound - 1) / kHistRound, 1024);
+    hipLaunchKernelGGL(norm_histogram_kernel, dim3(grid), dim3(kHistThreads), 0, stream, static_cast<const uint16_t *>(stats), nsc,
+                       hist);
+    return hipGetLastError();
+}
+
+hipError_t launch_bitrate_search(uint32_t *hist, int mode, double prev_u, double target, double *out, hipStream_t stream)
+{
+    hipLaunchKernelGGL(bitrate_search_kernel, dim3(1), dim3(kSearchThreads), 0, stream, hist, mode, prev_u, target, out);
+    return hipGetLastError();
+}
+
+} // namespace dq

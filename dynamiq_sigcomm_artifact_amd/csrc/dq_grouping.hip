@@ -20,6 +20,7 @@
 // and a superchunk is then classified by two integer compares.
 // Longer vectors take two launches: count per tile, then every tile sums the counts of the tiles before it
 // and places its indices.
+#include "dq_bitwidth.cuh"
 #include "dq_launch.h"
 
 namespace dq {
@@ -31,27 +32,6 @@ constexpr int kThreads = 256;
 constexpr int kPer = kTile / kThreads;
 
 __device__ __forceinline__ int width_class(int64_t q) { return q == 8 ? 0 : q == 4 ? 1 : q == 2 ? 2 : 3; }
-
-__device__ __forceinline__ float round_bf16(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
-
-// testbed_evaluation/new_comm_hooks/comm_hooks.py:64-70 on a bf16 norm: every torch op computes in
-// binary32 and rounds its result to bf16
-__device__ __forceinline__ int64_t qbits_of_norm(uint32_t norm_bits, float u)
-{
-    const float eps = 1e-20f;
-    float x = bf16_bits_to_f32(norm_bits);
-    x = (x != x) ? x : round_bf16(x > eps ? x : eps);
-    x = round_bf16(log2_det(x));
-    x = round_bf16(x * (float)(4.0 / (512.0 / 17.0)));
-    x = round_bf16(x + u);
-    x = (x != x) ? x : round_bf16(x > eps ? x : eps);
-    x = round_bf16(log2_det(x));
-    x = __builtin_floorf(x);
-    int z = (x != x) ? 1 : (x < 1.0f ? 1 : (x > 3.0f ? 3 : (int)x));
-    return (int64_t)1 << z;
-}
-
-constexpr int kMaxPattern = 0x7f80; // +infinity: the patterns 0 .. 0x7f80 are the non-negative norms in ascending order
 
 // where the widths come from: an int64 array, or the norm column of the interleaved bf16 stats.
 //   operator()(i)           the width of superchunk i by the rule itself (two-launch path)
@@ -72,29 +52,7 @@ struct WidthsFromStats {
     float u;
     typedef uint32_t Raw; // a (mean, norm) pair: the norm pattern is the high half
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits_of_norm(stats[2 * i + 1], u); }
-    // index of the first of 64 probes lo + step * (l + 1) (clamped to kMaxPattern) whose width is >= target; 64 if none
-    __device__ __forceinline__ int first_probe(int lo, int step, int lane, int64_t target) const
-    {
-        const int p = min(lo + step * (lane + 1), kMaxPattern);
-        const uint64_t hit = __builtin_amdgcn_ballot_w64(qbits_of_norm((uint32_t)p, u) >= target);
-        return hit ? __builtin_ctzll(hit) : 64;
-    }
-    // wave 0 finds thr[0] = the smallest pattern of width >= 4, wave 1 thr[1] = that of width 8
-    // (kMaxPattern + 1 when no pattern reaches it)
-    __device__ __forceinline__ void prepare(int *thr, int wave, int lane) const
-    {
-        if (wave > 1) return;
-        const int64_t target = wave == 0 ? 4 : 8;
-        int t = kMaxPattern + 1;
-        const int a = first_probe(-1, 512, lane, target);
-        if (a < 64) {
-            const int lo = -1 + 512 * a;
-            const int b = first_probe(lo, 8, lane, target);
-            const int lo2 = lo + 8 * b;
-            t = lo2 + 1 + first_probe(lo2, 1, lane, target);
-        }
-        if (lane == 0) thr[wave] = t;
-    }
+    __device__ __forceinline__ void prepare(int *thr, int wave, int lane) const { width_thresholds(u, thr, wave, lane); }
     bool word_aligned() const { return (reinterpret_cast<uintptr_t>(stats) & 3) == 0; } // load() reads pairs as one word
     __device__ __forceinline__ Raw load(int i) const { return reinterpret_cast<const uint32_t *>(stats)[i]; }
     __device__ __forceinline__ int cls(Raw pair, const int *thr) const

@@ -385,6 +385,35 @@ torch::Tensor group_plan_stats(torch::Tensor stats, double u, torch::Tensor orde
     return work.slice(0, 0, 4);
 }
 
+int64_t bitrate_hist_ints() { return dq_bitrate_hist_ints(); }
+
+void norm_histogram(torch::Tensor stats, torch::Tensor hist, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(stats.device().type() == torch::kCUDA && hist.device().type() == torch::kCUDA, "stats and hist must be CUDA tensors");
+    TORCH_CHECK(stats.dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+    TORCH_CHECK(hist.dtype() == torch::kInt32, "hist must be torch.int32");
+    TORCH_CHECK(stats.is_contiguous() && hist.is_contiguous(), "stats and hist must be contiguous");
+    const int64_t nsc = stats.numel() / 2;
+    TORCH_CHECK(nsc > 0 && stats.numel() == 2 * nsc, "stats must hold (mean, norm) pairs");
+    TORCH_CHECK(hist.numel() >= dq_bitrate_hist_ints(), "hist has fewer than bitrate_hist_ints() entries");
+    check_status(dq_norm_histogram(stats.data_ptr(), nsc, reinterpret_cast<uint32_t *>(hist.data_ptr<int32_t>()), hist.numel(),
+                                   stats.device().index(), as_stream(stream_p)),
+                 "norm_histogram");
+}
+
+torch::Tensor bitrate_search(torch::Tensor hist, int mode, double prev_u, double target_avg_bits, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(hist.device().type() == torch::kCUDA, "hist must be a CUDA tensor");
+    TORCH_CHECK(hist.dtype() == torch::kInt32 && hist.is_contiguous(), "hist must be a contiguous torch.int32 tensor");
+    TORCH_CHECK(hist.numel() >= dq_bitrate_hist_ints(), "hist has fewer than bitrate_hist_ints() entries");
+    TORCH_CHECK(mode == 0 || mode == 1, "mode must be 0 (bisection) or 1 (correction from prev_u)");
+    auto result = torch::empty({4}, hist.options().dtype(torch::kFloat64));
+    check_status(dq_bitrate_search(reinterpret_cast<uint32_t *>(hist.data_ptr<int32_t>()), hist.numel(), mode, prev_u,
+                                   target_avg_bits, result.data_ptr<double>(), hist.device().index(), as_stream(stream_p)),
+                 "bitrate_search");
+    return result;
+}
+
 void scaling_compress_rows(torch::Tensor src, torch::Tensor rows, torch::Tensor dst, torch::Tensor rand_pool, int64_t nrows,
                            int nbits, uint64_t stream_p = 0, int strategy = 2)
 {
@@ -873,6 +902,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
     modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width into the three regions of order (8-bit rows from 0, 4-bit from nsc, 2-bit from 2 nsc); returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
     modul.def("group_plan_stats", &group_plan_stats, "bit widths from the reduced bf16 norms and the offset u, and the partition by width, in one call; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
+    modul.def("bitrate_hist_ints", &bitrate_hist_ints, "int32 entries of the norm-pattern histogram");
+    modul.def("norm_histogram", &norm_histogram, "adds the bf16 norm patterns of a bucket's statistics to the histogram", py::arg("stats"), py::arg("hist"), py::arg("stream_p") = 0);
+    modul.def("bitrate_search", &bitrate_search, "the reference's search for the offset u (mode 0: bisection, 1: correction from prev_u) on the histogram, one launch; returns float64 [4] = u, average width, target - average, probes and leaves hist zeroed", py::arg("hist"), py::arg("mode"), py::arg("prev_u"), py::arg("target_avg_bits"), py::arg("stream_p") = 0);
     modul.def("scaling_compress_rows", &scaling_compress_rows, "compress the superchunks rows[k] of src into consecutive records", py::arg("src"), py::arg("rows"), py::arg("dst"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_dec_comp_rows", &scaling_dec_comp_rows, "fused ring step over the superchunks rows[k] of inp", py::arg("recv"), py::arg("inp"), py::arg("rows"), py::arg("send"), py::arg("rand_pool"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_decompress_rows", &scaling_decompress_rows, "decode consecutive records into the superchunks rows[k] of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("rows"), py::arg("stats"), py::arg("n_limit"), py::arg("nrows"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);

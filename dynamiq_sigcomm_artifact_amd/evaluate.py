@@ -321,6 +321,52 @@ def _llama_buckets(dev, bucket=6553600, limit=None):
         yield buf[:fill // 256 * 256]
 
 
+def _offset_search_lines(dev, norms_list, target, u_ref):
+    """the once-per-step search for u over the norms of every bucket: the reference's torch op sequence (one pass over
+    all norms and one read-back per probe) against the histogram of norm patterns (one small launch per bucket while the
+    step runs, one launch and one read-back for the search)"""
+    import time
+    stats = []
+    for t in norms_list:
+        st = torch.zeros((t.numel(), 2), dtype=torch.bfloat16, device=dev)
+        st[:, 1] = t
+        stats.append(st)
+    hist = bitrate.NormHistogram(dev)
+
+    def wall(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            out = fn()
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return best * 1e3, out
+
+    def hist_search(mode, prev):
+        for st in stats:
+            hist.add(st)
+        return hist.binary_search_u(target) if mode == 0 else hist.adjust_u(prev, target)
+
+    nsc = sum(t.numel() for t in norms_list)
+    for name, ref_fn, mode, prev in (
+            ("bisection (first compressed step)", lambda: bitrate.dynamic_bitrate_binary_search_u(norms_list, target), 0, 0.0),
+            ("correction from u + 1.5 (later steps)", lambda: bitrate.dynamic_bitrate_adjust_u(norms_list, u_ref + 1.5, target),
+             1, u_ref + 1.5)):
+        ms_ref, want = wall(ref_fn)
+        ms_hist, got = wall(lambda: hist_search(mode, prev))
+        _emit(config=4, pipeline="offset search: " + name, buckets=len(norms_list), superchunks=nsc,
+              torch_op_sequence_ms=round(ms_ref, 3), histogram_ms=round(ms_hist, 3), probes=int(hist.result[3]),
+              same_result=bool(tuple(want) == tuple(got)), u=got[0])
+    add_us = _time_us(lambda: hist.add(stats[0]))
+    hist.hist.zero_()
+    # an empty histogram never meets the tolerance: all 33 probes, the longest the search launch can take
+    search_us = _time_us(lambda: capi.bitrate_search(hist.hist, 0, 0.0, target, hist.result))
+    _emit(config=4, pipeline="offset search: device time", histogram_add_us_per_bucket=round(add_us, 2),
+          search_launch_us_33_probes=round(search_us, 2))
+
+
 def config4(dev, limit=None):
     target = 5.0 - bitrate.DYNAMIC_BITRATE_HEADROOM
     from .compressors import superchunk_mean_center
@@ -334,6 +380,7 @@ def config4(dev, limit=None):
         superchunk_mean_center(x, res, st, n, 1, 256)
         norms_list.append(st[:, 1].clone())
     u, avg_bits, delta = bitrate.dynamic_bitrate_binary_search_u(norms_list, target)
+    _offset_search_lines(dev, norms_list, target, u)
     # pass 2: quantise, with the reference's op sequence and with the gather/scatter folded into the kernels
     # an untimed pass of the op sequence first: its index_select / nonzero results have a different size in every
     # bucket, and the first pass pays the allocator for each of them

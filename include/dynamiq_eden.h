@@ -168,6 +168,32 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
                         int32_t *order, int32_t *work, int64_t work_ints, int device,
                         dq_stream_t stream);
 
+/* ---- the offset u of the bit-width rule (comm_hooks.py:73-139) -----------
+ *
+ * The reference probes the average width at up to 33 values of u per search,
+ * each probe being ten torch ops and a reduction over the norms of every bucket
+ * with a read-back.  The width depends on a norm only through its bf16 pattern,
+ * so the library counts the patterns once and searches on the counts. */
+
+/* number of uint32 the `hist` argument below must hold (zeroed before the first
+ * dq_norm_histogram of a training step) */
+int64_t dq_bitrate_hist_ints(void);
+
+/* adds the norm patterns stats[2 * i + 1], i < nsc (the reduced sums of squares
+ * written by dq_superchunk_mean_center / dq_superchunk_stats, after the
+ * all-reduce) to hist; call once per bucket.  At most 2^32 - 1 norms in all. */
+int dq_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, int64_t hist_ints,
+                      int device, dq_stream_t stream);
+
+/* mode 0: _dynamic_bitrate_binary_search_u (comm_hooks.py:94-114); mode 1:
+ * _dynamic_bitrate_adjust_u from prev_u (:117-139).  One launch, the whole
+ * search on the device.  result: float64 [4] on the device = u, the average
+ * width at u, target_avg_bits minus that average, the number of probes; the
+ * first three are what the reference's function returns for the same norms.
+ * hist is consumed: on return it is all zero, ready for the next step. */
+int dq_bitrate_search(uint32_t *hist, int64_t hist_ints, int mode, double prev_u,
+                      double target_avg_bits, double *result, int device, dq_stream_t stream);
+
 /* comm_hooks.py:1001 + scaling_compress: dst record k (and rand_pool row k,
  * 256 elements) encodes superchunk rows[k] of src.  rows: int32 [nrows] on the
  * device, every entry in [0, src superchunks).  rows == NULL means rows[k] = k. */

@@ -341,3 +341,59 @@ def dynamic_bitrate_qbits(norms_bf16, u, stride=1):
     q = np.zeros(count, np.int64)
     lib().dqo_dynamic_bitrate_qbits(_p(norms_bf16), stride, count, float(u), _p(q))
     return q
+
+
+# ---- the search for the offset u (comm_hooks.py:48-139) -----------------------------------------------
+# Plain Python around dqo_dynamic_bitrate_qbits: at most 33 evaluations, each one pass of the C rule over the
+# norms.  Pinned by the same search written with the reference's own torch ops on the CPU (the package's
+# bitrate module) -- see tests/test_oracle_misc.py.
+
+BITRATE_U_MIN, BITRATE_U_MAX, BITRATE_TOL, BITRATE_MAX_ITERS = -10.0, 60.0, 0.1, 32
+
+
+def dynamic_bitrate_avg_delta(norms_list, u, target):
+    """comm_hooks.py:73-91; norms_list: arrays of bf16 bit patterns"""
+    bits = chunks = 0
+    for norms in norms_list:
+        if norms.size:
+            bits += int(dynamic_bitrate_qbits(np.ascontiguousarray(norms), u).sum())
+            chunks += norms.size
+    avg = float(bits) / chunks if chunks else 0.0
+    return avg, target - avg
+
+
+def dynamic_bitrate_binary_search_u(norms_list, target):
+    """comm_hooks.py:94-114"""
+    low, high = BITRATE_U_MIN, BITRATE_U_MAX
+    best = (high,) + dynamic_bitrate_avg_delta(norms_list, high, target)
+    for _ in range(BITRATE_MAX_ITERS):
+        mid = (low + high) * 0.5
+        avg, delta = dynamic_bitrate_avg_delta(norms_list, mid, target)
+        if abs(delta) < abs(best[2]):
+            best = (mid, avg, delta)
+        if abs(delta) <= BITRATE_TOL:
+            return mid, avg, delta
+        if delta > 0:
+            low = mid
+        else:
+            high = mid
+    return best
+
+
+def dynamic_bitrate_adjust_u(norms_list, prev_u, target):
+    """comm_hooks.py:117-139"""
+    prev_u = max(BITRATE_U_MIN, min(BITRATE_U_MAX, float(prev_u)))
+    old_avg, old_delta = dynamic_bitrate_avg_delta(norms_list, prev_u, target)
+    if abs(old_delta) <= BITRATE_TOL:
+        return prev_u, old_avg, old_delta
+    step = old_delta
+    best = (prev_u, old_avg, old_delta)
+    for _ in range(BITRATE_MAX_ITERS):
+        cand = max(BITRATE_U_MIN, min(BITRATE_U_MAX, prev_u + step))
+        avg, delta = dynamic_bitrate_avg_delta(norms_list, cand, target)
+        if abs(delta) < abs(best[2]):
+            best = (cand, avg, delta)
+        if abs(delta) <= BITRATE_TOL or old_delta * delta >= 0:
+            return cand, avg, delta
+        step *= 0.5
+    return best

@@ -1,0 +1,114 @@
+"""The search for the offset u on a histogram of the norm patterns (dq_norm_histogram, dq_bitrate_search) against the
+oracle's restatement of comm_hooks.py:73-139 over the norms themselves, and against the reference's torch op sequence
+run on the device.  Every result is compared with ==: counts are integers and the search runs in IEEE double."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MAXP = 0x7f80
+
+
+def _stats(norms):
+    """bf16 [nsc, 2] statistics with the given norm column"""
+    st = torch.zeros((norms.numel(), 2), dtype=torch.bfloat16, device=DEV)
+    st[:, 1] = norms.to(DEV)
+    st[:, 0] = 0.25
+    return st
+
+
+def _norm_sets():
+    g = torch.Generator().manual_seed(3)
+    sets = {
+        "lognormal": [torch.exp(torch.randn(25600, generator=g) * 3 - 8).to(torch.bfloat16)],
+        "three buckets": [torch.exp(torch.randn(n, generator=g) * s - 6).to(torch.bfloat16)
+                          for n, s in ((5000, 5.0), (1, 1.0), (70001, 0.5))],
+        "narrow": [(torch.rand(4096, generator=g) * 1e-4 + 2e-4).to(torch.bfloat16)],
+        "one value": [torch.full((300,), 1.0).to(torch.bfloat16)],
+    }
+    special = torch.exp(torch.randn(2000, generator=g) * 4 - 5).to(torch.bfloat16)
+    special[::7] = 0.0
+    special[1::97] = float("nan")
+    special[2::131] = -1.0
+    special[3::211] = -0.0
+    sets["zeros, NaN, negative"] = [special]
+    return sets
+
+
+def test_norm_histogram_counts(capi):
+    norms = _norm_sets()["zeros, NaN, negative"][0].clone()
+    norms[5] = float("inf")
+    norms[6] = float("-inf")
+    hist = torch.zeros(capi.bitrate_hist_ints(), dtype=torch.int32, device=DEV)
+    capi.norm_histogram(_stats(norms), hist)
+    capi.norm_histogram(_stats(norms[:100]), hist)          # accumulates
+    pat = np.concatenate([to_bits(norms), to_bits(norms[:100])]).astype(np.int64)
+    nan = (pat & 0x7fff) > MAXP
+    bins = np.where(nan, MAXP + 1, np.where(pat > MAXP, 0, pat))
+    want = np.bincount(bins, minlength=hist.numel())
+    assert (hist.cpu().numpy() == want).all()
+    assert want[MAXP] == 2 and want[MAXP + 1] > 0           # +inf (in both calls), NaN
+
+
+@pytest.mark.parametrize("name", list(_norm_sets().keys()))
+def test_search_equals_the_oracle_on_the_norms(capi, oracle, name):
+    from dynamiq_sigcomm_artifact_amd.bitrate import NormHistogram
+    norms_list = _norm_sets()[name]
+    bits_list = [to_bits(t) for t in norms_list]
+    h = NormHistogram(DEV)
+    for target in (1.375, 2.375, 3.375, 4.375, 5.375, 7.375, 9.0):
+        for t in norms_list:
+            h.add(_stats(t))
+        assert h.count == sum(t.numel() for t in norms_list)
+        got = h.binary_search_u(target)
+        want = oracle.dynamic_bitrate_binary_search_u(bits_list, target)
+        assert got == tuple(want), (name, target, got, want)
+        assert int(h.hist.abs().sum()) == 0 and h.count == 0          # consumed
+        for prev in (want[0], want[0] + 6.0, want[0] - 3.5, 60.0, -10.0, 100.0, -50.0):
+            for t in norms_list:
+                h.add(_stats(t))
+            got = h.adjust_u(prev, target)
+            want2 = oracle.dynamic_bitrate_adjust_u(bits_list, prev, target)
+            assert got == tuple(want2), (name, target, prev, got, want2)
+
+
+def test_search_equals_the_torch_op_sequence_on_the_device():
+    """the reference's own functions as mirrored in bitrate.py, on device tensors (the scalar u enters the add in
+    binary32 there, as in the reference's CUDA run)"""
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    g = torch.Generator().manual_seed(9)
+    norms_list = [torch.exp(torch.randn(n, generator=g) * 4 - 7).to(torch.bfloat16).to(DEV) for n in (30000, 777)]
+    h = B.NormHistogram(DEV)
+    for target in (2.375, 4.375, 6.375):
+        for t in norms_list:
+            h.add(_stats(t))
+        got = h.binary_search_u(target)
+        want = B.dynamic_bitrate_binary_search_u(norms_list, target)
+        assert got == tuple(want), (target, got, want)
+        for prev in (want[0] + 5.0, want[0] - 2.0):
+            for t in norms_list:
+                h.add(_stats(t))
+            assert h.adjust_u(prev, target) == tuple(B.dynamic_bitrate_adjust_u(norms_list, prev, target))
+
+
+def test_closed_forms_and_the_empty_histogram():
+    """all norms 1.0: log2 = 0, so the width is 2 below u = 4, 4 below 8 (bf16(u) = 7.96875 already rounds to 8 bits), 8
+    from there on, and the bisection can be followed by hand"""
+    from dynamiq_sigcomm_artifact_amd.bitrate import NormHistogram
+    h = NormHistogram(DEV)
+    ones = _stats(torch.ones(1000).to(torch.bfloat16))
+    h.add(ones)
+    assert h.binary_search_u(4.0) == (7.5, 4.0, 0.0)              # probes 60, 25, 7.5
+    h.add(ones)
+    assert h.binary_search_u(3.0) == (7.5, 4.0, -1.0)             # unreachable: the first probe at distance 1 is kept
+    h.add(ones)
+    assert h.adjust_u(60.0, 4.0) == (56.0, 8.0, -4.0)             # one step of the deficit, same sign: returned
+    h.add(ones)
+    assert h.adjust_u(7.0, 4.0) == (7.0, 4.0, 0.0)
+    assert float(h.result[3]) == 1.0                              # one probe
+    # nothing added: the average is 0.0 everywhere, the starting candidate stays the best
+    assert h.binary_search_u(4.375) == (60.0, 0.0, 4.375)
+    assert float(h.result[3]) == 33.0

@@ -66,6 +66,28 @@ def test_plan_and_mixed_bindings(capi, eden_utils):
         eu.mixed_compress(src, order_a, counts, torch.zeros(16, dtype=torch.uint8, device=DEV), nsc, seed=1)
 
 
+def test_offset_search_bindings(capi, eden_utils):
+    eu = eden_utils
+    g = torch.Generator().manual_seed(4)
+    stats = torch.zeros(5000, 2, dtype=torch.bfloat16, device=DEV)
+    stats[:, 1] = torch.exp(torch.randn(5000, generator=g) * 4 - 6).to(torch.bfloat16).to(DEV)
+    assert eu.bitrate_hist_ints() == capi.bitrate_hist_ints()
+    ha = torch.zeros(capi.bitrate_hist_ints(), dtype=torch.int32, device=DEV)
+    hb = torch.zeros_like(ha)
+    for mode, prev in ((0, 60.0), (1, 3.0)):
+        capi.norm_histogram(stats, ha)
+        eu.norm_histogram(stats, hb)
+        assert torch.equal(ha, hb) and int(ha.sum()) == 5000
+        ra = torch.zeros(4, dtype=torch.float64, device=DEV)
+        capi.bitrate_search(ha, mode, prev, 4.375, ra)
+        rb = eu.bitrate_search(hb, mode, prev, 4.375)
+        assert ra.tolist() == rb.tolist() and int(hb.abs().sum()) == 0
+    with pytest.raises(RuntimeError, match="bitrate_hist_ints"):
+        eu.norm_histogram(stats, torch.zeros(100, dtype=torch.int32, device=DEV))
+    with pytest.raises(RuntimeError, match="mode must be"):
+        eu.bitrate_search(hb, 2, 0.0, 4.0)
+
+
 def test_transform_bindings(capi, eden_utils):
     eu = eden_utils
     n, block, nbits = 8192 * 2, 2048, 5

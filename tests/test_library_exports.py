@@ -118,6 +118,13 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_group_plan(P, 0, P, P, 100, 0, S), "nsc")
     err(L.dq_group_plan(P, 5000, P, P, 8, 0, S), "work buffer is too small")
     err(L.dq_group_plan_stats(N, ctypes.c_double(1.0), 100, N, P, P, 100, 0, S), "null pointer")
+    err(L.dq_norm_histogram(P, 100, P, 100, 0, S), "hist buffer is too small")
+    err(L.dq_norm_histogram(N, 100, P, 32768, 0, S), "null pointer")
+    err(L.dq_norm_histogram(P, 0, P, 32768, 0, S), "nsc must be in")
+    err(L.dq_bitrate_search(P, 32768, 2, ctypes.c_double(0.0), ctypes.c_double(4.0), P, 0, S), "mode must be 0")
+    err(L.dq_bitrate_search(P, 100, 0, ctypes.c_double(0.0), ctypes.c_double(4.0), P, 0, S), "hist buffer is too small")
+    err(L.dq_bitrate_search(P, 32768, 1, ctypes.c_double(float("nan")), ctypes.c_double(4.0), P, 0, S), "must be numbers")
+    err(L.dq_bitrate_search(P, 32768, 0, ctypes.c_double(0.0), ctypes.c_double(4.0), N, 0, S), "null pointer")
     err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 0, 0, 2, S), "unsupported element dtype")        # binary16 has no row-list kernels
     err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 1, 0, 1, S), "strategy")
     err(L.dq_scaling_dec_comp_rows(P, P, P, P, P, 0, 4, 1, 0, 2, S), "n must be positive")
@@ -148,7 +155,7 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_thc_dequantize_irht(P, P, N, 64, 64, F1, P, P, 0, S), "null pointer")
     err(L.dq_thc_dequantize_irht(P, P, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
-    assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 and capi.eden_work_doubles(8192) == 2
+    assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 and capi.eden_work_doubles(8192) == 2 and capi.bitrate_hist_ints() == 32768
     # a good call clears the message
     assert L.dq_scaling_check_common(256, 4, 16, 2, 1) == 0 and L.dq_last_error().decode() == ""
     assert L.dq_status_string(16).decode() == "kernel launch failed"

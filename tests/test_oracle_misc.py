@@ -241,6 +241,42 @@ def test_dynamic_bitrate_rule(oracle):
     assert [int(_torch_qbits(torch.tensor([1.0]).to(torch.bfloat16), u)[0]) for u in us] == [2, 4, 4, 8, 8]
 
 
+def test_offset_search_closed_forms_and_torch_sequence(oracle, monkeypatch):
+    """the oracle's two searches for u: cases that can be followed by hand, and the package's torch restatement of
+    comm_hooks.py:94-139 run on the CPU with the scalar add done in binary32 (what the device kernel of torch does;
+    torch's CPU kernel rounds the scalar u to bf16 first, which is not what the reference's GPU run computes)"""
+    ones = [to_bits(torch.ones(1000).to(torch.bfloat16))]
+    # all norms 1.0: width 2 below u = 4, 4 up to bf16(u) = 7.9375, 8 from 7.96875 on.  Probes 60, 25, 7.5:
+    assert oracle.dynamic_bitrate_binary_search_u(ones, 4.0) == (7.5, 4.0, 0.0)
+    # 3 bits cannot be met: the first probe at distance 1 (u = 7.5) stays the best of 33
+    assert oracle.dynamic_bitrate_binary_search_u(ones, 3.0) == (7.5, 4.0, -1.0)
+    assert oracle.dynamic_bitrate_adjust_u(ones, 60.0, 4.0) == (56.0, 8.0, -4.0)     # deficit keeps its sign: returned
+    assert oracle.dynamic_bitrate_adjust_u(ones, 7.0, 4.0) == (7.0, 4.0, 0.0)
+    assert oracle.dynamic_bitrate_adjust_u(ones, 100.0, 8.0) == (60.0, 8.0, 0.0)     # prev_u is clipped to [-10, 60]
+    assert oracle.dynamic_bitrate_binary_search_u([], 4.375) == (60.0, 0.0, 4.375)
+
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+
+    def qbits_binary32_scalar(norms, u):
+        eps = 1e-20
+        ln = torch.log2(torch.clamp(norms, min=eps)).mul(B.DYNAMIC_BITRATE_NORM_SCALE)
+        score = (ln.float() + torch.tensor(float(u), dtype=torch.float32)).to(norms.dtype)
+        z = torch.floor(torch.log2(torch.clamp(score, min=eps))).to(torch.int64).clamp_(1, 3)
+        return torch.bitwise_left_shift(torch.ones_like(z), z)
+
+    monkeypatch.setattr(B, "dynamic_bitrate_qbits", qbits_binary32_scalar)
+    g = torch.Generator().manual_seed(0)
+    for trial in range(4):
+        norms = [torch.exp(torch.randn(5000 + 17 * trial, generator=g) * (1 + trial) - 6 - trial).to(torch.bfloat16)
+                 for _ in range(3)]
+        nb = [to_bits(t) for t in norms]
+        for target in (1.375, 3.375, 4.375, 7.375):
+            a = B.dynamic_bitrate_binary_search_u(norms, target)
+            assert a == tuple(oracle.dynamic_bitrate_binary_search_u(nb, target))
+            for prev in (a[0], a[0] + 6, a[0] - 3, 60.0, -10.0):
+                assert B.dynamic_bitrate_adjust_u(norms, prev, target) == tuple(oracle.dynamic_bitrate_adjust_u(nb, prev, target))
+
+
 def test_bit_width_rule_non_finite_norms(oracle):
     """the device conversion to int64 saturates: +inf norms land in the 8-bit group, NaN norms in the 2-bit group"""
     import numpy as np
