@@ -218,6 +218,17 @@ def _torch_qbits(norms, u):
     return torch.bitwise_left_shift(torch.ones_like(z), z)
 
 
+def _torch_qbits_binary32_scalar(norms, u):
+    """the same sequence with the scalar add done the way torch's device kernel does it: in binary32, rounded to the
+    tensor's dtype afterwards"""
+    eps = 1e-20
+    ln = torch.log2(torch.clamp(norms, min=eps)).mul(4.0 / (512.0 / 17.0))
+    score = (ln.float() + torch.tensor(float(u), dtype=torch.float32)).to(norms.dtype)
+    z = torch.floor(torch.log2(torch.clamp(score, min=eps))).to(torch.int64)
+    z.clamp_(1, 3)
+    return torch.bitwise_left_shift(torch.ones_like(z), z)
+
+
 def test_dynamic_bitrate_rule(oracle):
     g = torch.Generator().manual_seed(6)
     norms = torch.exp(torch.randn(20000, generator=g) * 6 - 8).to(torch.bfloat16)
@@ -231,8 +242,16 @@ def test_dynamic_bitrate_rule(oracle):
         if prev is not None:
             assert (q >= prev).all()                                   # monotone in u
         prev = q
-        tq = _torch_qbits(norms, float(u)).numpy()
-        assert (q != tq).mean() < 1e-3                                  # log2 ulps at bf16 ties only
+        # torch's CPU kernel rounds the scalar u to bf16 before the add, its device kernel (what the reference runs, and
+        # what the rule restates) adds it in binary32: the plain CPU sequence differs on a few norms per offset ...
+        assert (q != _torch_qbits(norms, float(u)).numpy()).mean() < 1e-3
+        # ... and with the add done in binary32 it agrees on every one
+        assert (q == _torch_qbits_binary32_scalar(norms, float(u)).numpy()).all()
+    # every finite non-negative bf16 norm, offsets off the bf16 grid
+    pat = np.arange(0, 0x7f80, dtype=np.uint16)
+    every = torch.from_numpy(pat.view(np.int16)).view(torch.bfloat16)
+    for u in np.random.default_rng(0).uniform(-10, 60, 60):
+        assert (oracle.dynamic_bitrate_qbits(pat, float(u)) == _torch_qbits_binary32_scalar(every, float(u)).numpy()).all()
     # norm 1 -> log2 = 0 -> score = bf16(u): 2 bits below 4, 4 bits in [4, 8), 8 bits from 8 on;
     # bf16(7.97) = 7.96875 has log2 = 2.9943, which ROUNDS to 3.0 in bf16 and therefore already gets 8 bits
     one = to_bits(torch.tensor([1.0]).to(torch.bfloat16))
@@ -257,14 +276,7 @@ def test_offset_search_closed_forms_and_torch_sequence(oracle, monkeypatch):
 
     from dynamiq_sigcomm_artifact_amd import bitrate as B
 
-    def qbits_binary32_scalar(norms, u):
-        eps = 1e-20
-        ln = torch.log2(torch.clamp(norms, min=eps)).mul(B.DYNAMIC_BITRATE_NORM_SCALE)
-        score = (ln.float() + torch.tensor(float(u), dtype=torch.float32)).to(norms.dtype)
-        z = torch.floor(torch.log2(torch.clamp(score, min=eps))).to(torch.int64).clamp_(1, 3)
-        return torch.bitwise_left_shift(torch.ones_like(z), z)
-
-    monkeypatch.setattr(B, "dynamic_bitrate_qbits", qbits_binary32_scalar)
+    monkeypatch.setattr(B, "dynamic_bitrate_qbits", _torch_qbits_binary32_scalar)
     g = torch.Generator().manual_seed(0)
     for trial in range(4):
         norms = [torch.exp(torch.randn(5000 + 17 * trial, generator=g) * (1 + trial) - 6 - trial).to(torch.bfloat16)
