@@ -635,6 +635,13 @@ def kernels(dev, n=6553600):
     u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)
     line("group_plan_stats", lambda: capi.group_plan_stats(stats, u, qbits, order, work), 4 * nsc + 12 * nsc, superchunks=nsc)
     line("group_plan", lambda: capi.group_plan(qbits, order, work), 8 * nsc + 4 * nsc, superchunks=nsc)
+    # the search for u: the norm patterns of the bucket into the histogram; the whole bisection on an empty histogram
+    # (never meets the tolerance: all 33 probes)
+    hist = torch.zeros(capi.bitrate_hist_ints(), dtype=torch.int32, device=dev)
+    found = torch.zeros(4, dtype=torch.float64, device=dev)
+    line("norm_histogram", lambda: capi.norm_histogram(stats, hist), 4 * nsc, superchunks=nsc)
+    hist.zero_()
+    line("bitrate_search", lambda: capi.bitrate_search(hist, 0, 0.0, 4.375, found), 8 * hist.numel(), probes=33)
     # statistics without the residual, then the three widths of the plan in one launch (centring folded into the load,
     # rounding stream drawn in the kernel) and back (mean added on the store)
     mean32 = torch.empty(nsc, dtype=torch.float32, device=dev)
