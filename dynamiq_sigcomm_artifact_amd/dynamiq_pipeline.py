@@ -121,7 +121,8 @@ def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=
     return outs, total, qbits
 
 
-def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=None, work=None, stream=None):
+def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=None, work=None, stream=None,
+                                          norm_histogram=None):
     """The same all-reduce with every stage kept on the device: no residual buffers (the centring is folded
     into the codec's loads), no group tensors, no per-width launches and no read-back of the group sizes --
     a fixed sequence of launches per bucket (statistics, plan, and one codec launch per ring step for all
@@ -131,6 +132,9 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
     mixed_decompress.  The bit widths follow the device rule of group_plan_stats; the rounding randomness is
     the in-kernel stream keyed by (seed + rank, ring step, index of the chunk in the vector), so results are
     reproducible but not those of dynamic_bitrate_allreduce, whose random values come from the pool.
+
+    norm_histogram: a bitrate.NormHistogram that collects the reduced norms of the step's buckets for the search of
+    the next step's u (comm_hooks.py:962, 904-931) -- one more small launch per bucket.
 
     Returns (result tensors per rank, reduced stats, device int32 tensor [n8, n4, n2, other])."""
     from . import capi
@@ -166,6 +170,8 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         for r in range(1, W):
             total.add_(stats[r])
     capi.group_plan_stats(total, float(u), None, order, plan, stream=stream)
+    if norm_histogram is not None:
+        norm_histogram.add(total, stream=stream)
     outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
 
     def encode(r, chunk, step, received=None):

@@ -112,3 +112,21 @@ def test_closed_forms_and_the_empty_histogram():
     # nothing added: the average is 0.0 everywhere, the starting candidate stays the best
     assert h.binary_search_u(4.375) == (60.0, 0.0, 4.375)
     assert float(h.result[3]) == 33.0
+
+
+def test_pipeline_feeds_the_histogram(oracle):
+    """a step of three buckets through the single-pass all-reduce with the histogram attached: the u for the next step
+    equals the oracle's search over the reduced norms of the three buckets"""
+    from dynamiq_sigcomm_artifact_amd.bitrate import NormHistogram
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import dynamic_bitrate_allreduce_single_pass
+    g = torch.Generator().manual_seed(21)
+    h = NormHistogram(DEV)
+    reduced = []
+    for nsc, W in ((40, 2), (7, 1), (130, 3)):
+        scales = torch.exp(torch.randn(nsc, 1, generator=g) * 4.0) * 1e-3
+        vecs = [(torch.randn(nsc, 256, generator=g) * scales).reshape(-1).to(torch.bfloat16).to(DEV) for _ in range(W)]
+        _, total, _ = dynamic_bitrate_allreduce_single_pass(vecs, 7.0, norm_histogram=h)
+        reduced.append(to_bits(total[:, 1].contiguous()))
+    assert h.count == 177
+    got = h.adjust_u(7.0, 4.375)
+    assert got == tuple(oracle.dynamic_bitrate_adjust_u(reduced, 7.0, 4.375))
