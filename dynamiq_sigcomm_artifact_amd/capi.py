@@ -22,7 +22,7 @@ EXPORTS = [
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
     "dq_scaling_compress_philox", "dq_scaling_dec_comp_philox", "dq_philox_uniform",
     "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
-    "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
+    "dq_group_plan_stats_dev_u", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
@@ -76,6 +76,8 @@ def lib():
         L.dq_group_plan.argtypes = [vp, i64, vp, vp, i64, i32, vp]
         L.dq_group_plan_stats.restype = i32
         L.dq_group_plan_stats.argtypes = [vp, c.c_double, i64, vp, vp, vp, i64, i32, vp]
+        L.dq_group_plan_stats_dev_u.restype = i32
+        L.dq_group_plan_stats_dev_u.argtypes = [vp, vp, i64, vp, vp, vp, i64, i32, vp]
         L.dq_bitrate_hist_ints.restype = i64
         L.dq_bitrate_hist_ints.argtypes = []
         L.dq_norm_histogram.restype = i32
@@ -228,12 +230,20 @@ def group_rows(order, nsc, width, count):
 
 
 def group_plan_stats(stats, u, qbits_out, order, work, stream=None):
-    """stats bf16 [nsc, 2] (mean, reduced sum of squares), offset u -> qbits_out (int64 or None), order, work"""
+    """stats bf16 [nsc, 2] (mean, reduced sum of squares), offset u (a number, or a float64 device tensor read when the
+    kernels run) -> qbits_out (int64 or None), order, work"""
     if stats.dtype != torch.bfloat16 or order.dtype != torch.int32 or work.dtype != torch.int32:
         raise RuntimeError("group_plan_stats: stats must be bfloat16, order and work int32")
     nsc = stats.numel() // 2
     if order.numel() < 3 * nsc or (qbits_out is not None and (qbits_out.dtype != torch.int64 or qbits_out.numel() < nsc)):
         raise RuntimeError("group_plan_stats: order / qbits_out too small or of the wrong dtype")
+    if isinstance(u, torch.Tensor):
+        # the offset stays on the device (one float64, e.g. the first entry of bitrate_search's result)
+        if u.dtype != torch.float64 or u.numel() < 1 or u.device != stats.device:
+            raise RuntimeError("group_plan_stats: a tensor u must be float64 on the device of stats")
+        _check(lib().dq_group_plan_stats_dev_u(stats.data_ptr(), u.data_ptr(), nsc, _ptr(qbits_out), order.data_ptr(),
+                                               work.data_ptr(), work.numel(), _dev(stats), _stream(stream)))
+        return
     _check(lib().dq_group_plan_stats(stats.data_ptr(), float(u), nsc, _ptr(qbits_out), order.data_ptr(), work.data_ptr(),
                                      work.numel(), _dev(stats), _stream(stream)))
 

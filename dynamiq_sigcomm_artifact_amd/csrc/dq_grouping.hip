@@ -42,6 +42,7 @@ struct WidthsFromArray {
     typedef int64_t Raw;
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
     bool word_aligned() const { return true; }
+    __device__ __forceinline__ void resolve() {}
     __device__ __forceinline__ void prepare(int *, int, int) const {}
     __device__ __forceinline__ Raw load(int i) const { return qbits[i]; }
     __device__ __forceinline__ int cls(Raw q, const int *) const { return width_class(q); }
@@ -50,7 +51,12 @@ struct WidthsFromArray {
 struct WidthsFromStats {
     const uint16_t *stats;
     float u;
+    const double *u_dev;  // when set, the offset is read from device memory (the search for u leaves it there)
     typedef uint32_t Raw; // a (mean, norm) pair: the norm pattern is the high half
+    __device__ __forceinline__ void resolve()
+    {
+        if (u_dev) u = (float)*u_dev;
+    }
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits_of_norm(stats[2 * i + 1], u); }
     __device__ __forceinline__ void prepare(int *thr, int wave, int lane) const { width_thresholds(u, thr, wave, lane); }
     bool word_aligned() const { return (reinterpret_cast<uintptr_t>(stats) & 3) == 0; } // load() reads pairs as one word
@@ -79,6 +85,7 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
 {
     __shared__ int thr[2];
     __shared__ uint64_t before_sum[kOneThreads / 64], scan_sum[kOneThreads / 64];
+    widths.resolve();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nbefore = (int)blockIdx.x * kTile; // superchunks of the tiles before this one
     const int own = nbefore + (int)threadIdx.x;
@@ -149,6 +156,7 @@ template <class W>
 __global__ __launch_bounds__(kThreads) void plan_count_kernel(W widths, int64_t nsc, int32_t *__restrict__ work)
 {
     __shared__ int cnt[4];
+    widths.resolve();
     if (threadIdx.x < 4) cnt[threadIdx.x] = 0;
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kTile + threadIdx.x * kPer;
@@ -172,6 +180,7 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
 {
     __shared__ int before[4], total[4];
     __shared__ uint64_t wave_sum[kThreads / 64];
+    widths.resolve();
     if (threadIdx.x < 4) {
         before[threadIdx.x] = 0;
         total[threadIdx.x] = 0;
@@ -259,10 +268,11 @@ hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, 
     return run_plan(WidthsFromArray{qbits}, nullptr, nsc, order, work, stream);
 }
 
-hipError_t launch_group_plan_stats(const void *stats, float u, int64_t nsc, int64_t *qbits_out, int32_t *order,
-                                   int32_t *work, hipStream_t stream)
+// u_dev != nullptr: the offset is *u_dev at the time the kernels run, u is ignored
+hipError_t launch_group_plan_stats(const void *stats, float u, const double *u_dev, int64_t nsc, int64_t *qbits_out,
+                                   int32_t *order, int32_t *work, hipStream_t stream)
 {
-    return run_plan(WidthsFromStats{static_cast<const uint16_t *>(stats), u}, qbits_out, nsc, order, work, stream);
+    return run_plan(WidthsFromStats{static_cast<const uint16_t *>(stats), u, u_dev}, qbits_out, nsc, order, work, stream);
 }
 
 } // namespace dq

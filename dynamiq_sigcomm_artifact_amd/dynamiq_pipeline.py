@@ -133,6 +133,8 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
     the in-kernel stream keyed by (seed + rank, ring step, index of the chunk in the vector), so results are
     reproducible but not those of dynamic_bitrate_allreduce, whose random values come from the pool.
 
+    u: the offset of the width rule, a number or a float64 device tensor (e.g. result[0:1] of the offset search: then
+    nothing of the step is read back).
     norm_histogram: a bitrate.NormHistogram that collects the reduced norms of the step's buckets for the search of
     the next step's u (comm_hooks.py:962, 904-931) -- one more small launch per bucket.
 
@@ -169,7 +171,7 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         total.copy_(stats[0])
         for r in range(1, W):
             total.add_(stats[r])
-    capi.group_plan_stats(total, float(u), None, order, plan, stream=stream)
+    capi.group_plan_stats(total, u if isinstance(u, torch.Tensor) else float(u), None, order, plan, stream=stream)
     if norm_histogram is not None:
         norm_histogram.add(total, stream=stream)
     outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]

@@ -130,3 +130,28 @@ def test_pipeline_feeds_the_histogram(oracle):
     assert h.count == 177
     got = h.adjust_u(7.0, 4.375)
     assert got == tuple(oracle.dynamic_bitrate_adjust_u(reduced, 7.0, 4.375))
+
+
+@pytest.mark.parametrize("nsc", [3000, 70000])
+def test_plan_reads_the_offset_from_device_memory(capi, nsc):
+    """search -> plan with nothing read back: the plan kernels (one launch and, beyond 65536 superchunks, two) take u from
+    the search's result tensor and give the widths, counts and order of the call that gets the same u as a number"""
+    from dynamiq_sigcomm_artifact_amd.bitrate import NormHistogram
+    g = torch.Generator().manual_seed(nsc)
+    stats = _stats(torch.exp(torch.randn(nsc, generator=g) * 4 - 6).to(torch.bfloat16))
+    h = NormHistogram(DEV)
+    h.add(stats)
+    capi.bitrate_search(h.hist, 0, 0.0, 4.375, h.result)             # no read-back here
+    order_a = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    order_b = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    work_a = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    work_b = torch.zeros_like(work_a)
+    q_a = torch.zeros(nsc, dtype=torch.int64, device=DEV)
+    q_b = torch.zeros_like(q_a)
+    capi.group_plan_stats(stats, h.result[0:1], q_a, order_a, work_a)
+    u = float(h.result[0])
+    capi.group_plan_stats(stats, u, q_b, order_b, work_b)
+    assert torch.equal(q_a, q_b) and torch.equal(order_a, order_b) and work_a[:4].tolist() == work_b[:4].tolist()
+    assert sorted(work_a[:3].tolist())[1] > 0                        # at least two widths in use
+    with pytest.raises(RuntimeError, match="float64"):
+        capi.group_plan_stats(stats, torch.zeros(1, device=DEV), None, order_a, work_a)
