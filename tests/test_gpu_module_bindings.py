@@ -82,6 +82,16 @@ def test_offset_search_bindings(capi, eden_utils):
         capi.bitrate_search(ha, mode, prev, 4.375, ra)
         rb = eu.bitrate_search(hb, mode, prev, 4.375)
         assert ra.tolist() == rb.tolist() and int(hb.abs().sum()) == 0
+    # the plan with the offset left on the device
+    nsc = 5000
+    order_a = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    order_b = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    capi.group_plan_stats(stats, rb[0:1], None, order_a, work)
+    counts = eu.group_plan_stats_dev_u(stats, rb[0:1], order_b)
+    assert counts.tolist() == work[:4].tolist() and torch.equal(order_a, order_b)
+    with pytest.raises(RuntimeError, match="float64"):
+        eu.group_plan_stats_dev_u(stats, rb[0:1].float(), order_b)
     with pytest.raises(RuntimeError, match="bitrate_hist_ints"):
         eu.norm_histogram(stats, torch.zeros(100, dtype=torch.int32, device=DEV))
     with pytest.raises(RuntimeError, match="mode must be"):
