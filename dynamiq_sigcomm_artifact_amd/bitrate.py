@@ -122,9 +122,16 @@ class NormHistogram(object):
         self._capi.norm_histogram(stats, self.hist, stream)
         self.count += stats.numel() // 2
 
-    def _search(self, mode, prev_u, target_avg_bits, stream):
+    def launch_search(self, mode, prev_u, target_avg_bits, stream=None):
+        """the search as one launch, nothing read back: returns the device tensor float64 [4] = u, average width,
+        target - average, probes (also ``self.result``).  mode 0: bisection; 1: correction from prev_u, a number or a
+        float64 device tensor -- ``self.result[0:1]`` chains the steps of a training run on the device."""
         self._capi.bitrate_search(self.hist, mode, prev_u, target_avg_bits, self.result, stream)
         self.count = 0                      # the kernel leaves the histogram zeroed
+        return self.result
+
+    def _search(self, mode, prev_u, target_avg_bits, stream):
+        self.launch_search(mode, prev_u, target_avg_bits, stream)
         if hasattr(stream, "synchronize"):
             stream.synchronize()            # tolist() below only waits for torch's current stream
         u, avg, delta, _ = self.result.tolist()

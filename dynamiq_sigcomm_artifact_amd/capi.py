@@ -83,7 +83,7 @@ def lib():
         L.dq_norm_histogram.restype = i32
         L.dq_norm_histogram.argtypes = [vp, i64, vp, i64, i32, vp]
         L.dq_bitrate_search.restype = i32
-        L.dq_bitrate_search.argtypes = [vp, i64, i32, c.c_double, c.c_double, vp, i32, vp]
+        L.dq_bitrate_search.argtypes = [vp, i64, i32, c.c_double, vp, c.c_double, vp, i32, vp]
         L.dq_scaling_compress_rows.restype = i32
         L.dq_scaling_compress_rows.argtypes = [vp, vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_scaling_dec_comp_rows.restype = i32
@@ -261,12 +261,17 @@ def norm_histogram(stats, hist, stream=None):
 
 
 def bitrate_search(hist, mode, prev_u, target_avg_bits, result, stream=None):
-    """mode 0: bisection, 1: correction from prev_u; result float64 [4] = u, average width, target - average, probes;
-    hist comes back zeroed"""
+    """mode 0: bisection, 1: correction from prev_u (a number or a float64 device tensor); result float64 [4] = u, average
+    width, target - average, probes; hist comes back zeroed"""
     if hist.dtype != torch.int32 or result.dtype != torch.float64 or result.numel() < 4:
         raise RuntimeError("bitrate_search: hist must be int32 and result float64 [4]")
-    _check(lib().dq_bitrate_search(hist.data_ptr(), hist.numel(), int(mode), float(prev_u), float(target_avg_bits),
-                                   result.data_ptr(), _dev(hist), _stream(stream)))
+    prev_dev = None
+    if isinstance(prev_u, torch.Tensor):        # the starting point stays on the device (it may be result itself)
+        if prev_u.dtype != torch.float64 or prev_u.numel() < 1 or prev_u.device != hist.device:
+            raise RuntimeError("bitrate_search: a tensor prev_u must be float64 on the device of hist")
+        prev_dev, prev_u = prev_u, 0.0
+    _check(lib().dq_bitrate_search(hist.data_ptr(), hist.numel(), int(mode), float(prev_u), _ptr(prev_dev),
+                                   float(target_avg_bits), result.data_ptr(), _dev(hist), _stream(stream)))
 
 
 def scaling_compress_rows(src, rows, dst, rand_pool, nrows, nbits, strategy, stream=None):

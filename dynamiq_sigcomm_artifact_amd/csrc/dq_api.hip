@@ -334,8 +334,8 @@ int dq_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, int64_t hi
     return finish(dq::launch_norm_histogram(stats, nsc, hist, static_cast<hipStream_t>(stream)));
 }
 
-int dq_bitrate_search(uint32_t *hist, int64_t hist_ints, int mode, double prev_u, double target_avg_bits, double *result,
-                      int device, dq_stream_t stream)
+int dq_bitrate_search(uint32_t *hist, int64_t hist_ints, int mode, double prev_u, const double *prev_u_dev,
+                      double target_avg_bits, double *result, int device, dq_stream_t stream)
 {
     if (mode != 0 && mode != 1) return fail(DQ_ERR_SIZE, "mode must be 0 (bisection) or 1 (correction from prev_u)");
     if (!hist || !result) return fail(DQ_ERR_NULL);
@@ -343,7 +343,7 @@ int dq_bitrate_search(uint32_t *hist, int64_t hist_ints, int mode, double prev_u
     if (prev_u != prev_u || target_avg_bits != target_avg_bits) return fail(DQ_ERR_SIZE, "prev_u and target_avg_bits must be numbers");
     int rc;
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_bitrate_search(hist, mode, prev_u, target_avg_bits, result, static_cast<hipStream_t>(stream)));
+    return finish(dq::launch_bitrate_search(hist, mode, prev_u, prev_u_dev, target_avg_bits, result, static_cast<hipStream_t>(stream)));
 }
 
 static int check_rows(int64_t nrows, int nbits, int dtype, int strategy, bool rand)

@@ -65,12 +65,15 @@ struct Probe {
 };
 
 // out[0..2] = u, average width, target - average; out[3] = number of probes.  hist: pattern counts in, zeros out.
+// prev_u_dev != nullptr: the starting point of the correction is *prev_u_dev (it may be out[0] of the previous search)
 __global__ __launch_bounds__(kSearchThreads) void bitrate_search_kernel(uint32_t *__restrict__ hist, int mode, double prev_u,
-                                                                       double target, double *__restrict__ out)
+                                                                       const double *prev_u_dev, double target,
+                                                                       double *out)
 {
     __shared__ uint32_t part[kSearchThreads];
     __shared__ int thr[2];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    if (prev_u_dev) prev_u = *prev_u_dev; // read by every thread long before thread 0 writes out[]
 
     // suffix counts in place: hist[p] = number of norms whose pattern is >= p, p = 0 .. kMaxPattern
     uint32_t v[kBinsPerThread];
@@ -180,9 +183,11 @@ hipError_t launch_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist,
     return hipGetLastError();
 }
 
-hipError_t launch_bitrate_search(uint32_t *hist, int mode, double prev_u, double target, double *out, hipStream_t stream)
+hipError_t launch_bitrate_search(uint32_t *hist, int mode, double prev_u, const double *prev_u_dev, double target, double *out,
+                                 hipStream_t stream)
 {
-    hipLaunchKernelGGL(bitrate_search_kernel, dim3(1), dim3(kSearchThreads), 0, stream, hist, mode, prev_u, target, out);
+    hipLaunchKernelGGL(bitrate_search_kernel, dim3(1), dim3(kSearchThreads), 0, stream, hist, mode, prev_u, prev_u_dev, target,
+                       out);
     return hipGetLastError();
 }
 

@@ -67,7 +67,8 @@ hipError_t launch_group_plan_stats(const void *stats, float u, const double *u_d
 // the offset u of the bit-width rule from a histogram of the norm patterns (dq_bitrate.hip)
 int64_t bitrate_hist_ints();
 hipError_t launch_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, hipStream_t stream);
-hipError_t launch_bitrate_search(uint32_t *hist, int mode, double prev_u, double target, double *out, hipStream_t stream);
+hipError_t launch_bitrate_search(uint32_t *hist, int mode, double prev_u, const double *prev_u_dev, double target, double *out,
+                                 hipStream_t stream);
 
 // all bit-width groups of a planned bucket in one launch (dq_scaling_mixed.hip); mp: the MEE
 // parameters of 8, 4 and 2 bits in this order

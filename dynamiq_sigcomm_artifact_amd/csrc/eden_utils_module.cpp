@@ -435,7 +435,7 @@ torch::Tensor bitrate_search(torch::Tensor hist, int mode, double prev_u, double
     TORCH_CHECK(hist.numel() >= dq_bitrate_hist_ints(), "hist has fewer than bitrate_hist_ints() entries");
     TORCH_CHECK(mode == 0 || mode == 1, "mode must be 0 (bisection) or 1 (correction from prev_u)");
     auto result = torch::empty({4}, hist.options().dtype(torch::kFloat64));
-    check_status(dq_bitrate_search(reinterpret_cast<uint32_t *>(hist.data_ptr<int32_t>()), hist.numel(), mode, prev_u,
+    check_status(dq_bitrate_search(reinterpret_cast<uint32_t *>(hist.data_ptr<int32_t>()), hist.numel(), mode, prev_u, nullptr,
                                    target_avg_bits, result.data_ptr<double>(), hist.device().index(), as_stream(stream_p)),
                  "bitrate_search");
     return result;

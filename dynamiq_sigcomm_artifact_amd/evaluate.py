@@ -477,15 +477,22 @@ def config4_streams(dev, u, nbuckets=48, rounds=8):
     the codec launches of its neighbours."""
     xs = [b.to(torch.bfloat16).clone() for b in _llama_buckets(dev, limit=nbuckets)]
     keep = []                                   # graphs and streams stay alive until the function returns
-    for nstreams in (1, 2, 3, 4):
+    target = 5.0 - bitrate.DYNAMIC_BITRATE_HEADROOM
+    # (streams, closed loop): in the closed loop the plans read u from device memory, every bucket adds its norms to the
+    # histogram and a round ends with the correction of u for the next one -- a whole training step without a read-back
+    for nstreams, closed in ((1, False), (2, False), (3, False), (4, False), (1, True), (2, True)):
         streams = [torch.cuda.Stream() for _ in range(nstreams)]
         graphs = []
+        hist = bitrate.NormHistogram(dev) if closed else None
+        if closed:
+            hist.result[0] = u
         for k, st in enumerate(streams):
             work, out = {}, [torch.empty_like(xs[0])]
 
             def share():
                 for x in xs[k::nstreams]:
-                    dynamic_bitrate_allreduce_single_pass([x], u, strategy=2, seed=3, out=out, work=work)
+                    dynamic_bitrate_allreduce_single_pass([x], hist.result[0:1] if closed else u, strategy=2, seed=3, out=out,
+                                                          work=work, norm_histogram=hist)
 
             with torch.cuda.stream(st):
                 share()
@@ -505,6 +512,8 @@ def config4_streams(dev, u, nbuckets=48, rounds=8):
                     g.replay()
             for st in streams:
                 main.wait_stream(st)
+            if closed:
+                hist.launch_search(1, hist.result[0:1], target)
 
         replay_all()
         torch.cuda.synchronize()
@@ -515,9 +524,13 @@ def config4_streams(dev, u, nbuckets=48, rounds=8):
         e.record()
         e.synchronize()
         per = s.elapsed_time(e) / (rounds * len(xs))
-        _emit(config=4, method="aee", pipeline="single_pass, %d buckets replayed as graphs" % len(xs), streams=nstreams,
-              rounds=rounds, ms_per_25MB_bucket=round(per, 4),
-              pipeline_GBps_of_bf16_input=round(2.0 * xs[0].numel() / (per * 1e-3) / 1e9, 1))
+        name = "single_pass, %d buckets replayed as graphs" % len(xs)
+        extra = {}
+        if closed:
+            name += " + norm histogram + search for the next u (u read from device memory)"
+            extra = dict(u_after_rounds=float(hist.result[0]), probes_last_search=int(hist.result[3]))
+        _emit(config=4, method="aee", pipeline=name, streams=nstreams, rounds=rounds, ms_per_25MB_bucket=round(per, 4),
+              pipeline_GBps_of_bf16_input=round(2.0 * xs[0].numel() / (per * 1e-3) / 1e9, 1), **extra)
     torch.cuda.synchronize()
 
 

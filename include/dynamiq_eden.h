@@ -198,9 +198,13 @@ int dq_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, int64_t hi
  * search on the device.  result: float64 [4] on the device = u, the average
  * width at u, target_avg_bits minus that average, the number of probes; the
  * first three are what the reference's function returns for the same norms.
- * hist is consumed: on return it is all zero, ready for the next step. */
+ * hist is consumed: on return it is all zero, ready for the next step.
+ * prev_u_dev (may be NULL): when set, mode 1 starts from the float64 it points
+ * to on the device instead of prev_u; it may be result itself, so that the u of
+ * one step feeds the correction of the next without leaving the device. */
 int dq_bitrate_search(uint32_t *hist, int64_t hist_ints, int mode, double prev_u,
-                      double target_avg_bits, double *result, int device, dq_stream_t stream);
+                      const double *prev_u_dev, double target_avg_bits, double *result,
+                      int device, dq_stream_t stream);
 
 /* comm_hooks.py:1001 + scaling_compress: dst record k (and rand_pool row k,
  * 256 elements) encodes superchunk rows[k] of src.  rows: int32 [nrows] on the

@@ -155,3 +155,30 @@ def test_plan_reads_the_offset_from_device_memory(capi, nsc):
     assert sorted(work_a[:3].tolist())[1] > 0                        # at least two widths in use
     with pytest.raises(RuntimeError, match="float64"):
         capi.group_plan_stats(stats, torch.zeros(1, device=DEV), None, order_a, work_a)
+
+
+def test_steps_chained_on_the_device(capi, oracle):
+    """four training steps with drifting norms: the correction of every step starts from the u the previous search left
+    in device memory, the plans read it from there, nothing is read back until the end -- and the final triple is the
+    one the oracle's functions give when chained on the host"""
+    from dynamiq_sigcomm_artifact_amd.bitrate import NormHistogram
+    g = torch.Generator().manual_seed(33)
+    h = NormHistogram(DEV)
+    target = 4.375
+    steps = [[torch.exp(torch.randn(n, generator=g) * 3 - 7 + 0.8 * k).to(torch.bfloat16) for n in (9000, 400)] for k in range(4)]
+    want = None
+    for k, norms_list in enumerate(steps):
+        for t in norms_list:
+            h.add(_stats(t))
+        h.launch_search(0 if k == 0 else 1, 0.0 if k == 0 else h.result[0:1], target)
+        bits = [to_bits(t) for t in norms_list]
+        want = (oracle.dynamic_bitrate_binary_search_u(bits, target) if k == 0
+                else oracle.dynamic_bitrate_adjust_u(bits, want[0], target))
+        # a plan of the next step reading u from the device
+        nsc = norms_list[0].numel()
+        order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+        work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+        q = torch.zeros(nsc, dtype=torch.int64, device=DEV)
+        capi.group_plan_stats(_stats(norms_list[0]), h.result[0:1], q, order, work)
+        assert (q.cpu().numpy() == oracle.dynamic_bitrate_qbits(bits[0], want[0])).all()
+    assert tuple(h.result[:3].tolist()) == tuple(want)

@@ -123,10 +123,10 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_norm_histogram(P, 100, P, 100, 0, S), "hist buffer is too small")
     err(L.dq_norm_histogram(N, 100, P, 32768, 0, S), "null pointer")
     err(L.dq_norm_histogram(P, 0, P, 32768, 0, S), "nsc must be in")
-    err(L.dq_bitrate_search(P, 32768, 2, ctypes.c_double(0.0), ctypes.c_double(4.0), P, 0, S), "mode must be 0")
-    err(L.dq_bitrate_search(P, 100, 0, ctypes.c_double(0.0), ctypes.c_double(4.0), P, 0, S), "hist buffer is too small")
-    err(L.dq_bitrate_search(P, 32768, 1, ctypes.c_double(float("nan")), ctypes.c_double(4.0), P, 0, S), "must be numbers")
-    err(L.dq_bitrate_search(P, 32768, 0, ctypes.c_double(0.0), ctypes.c_double(4.0), N, 0, S), "null pointer")
+    err(L.dq_bitrate_search(P, 32768, 2, ctypes.c_double(0.0), N, ctypes.c_double(4.0), P, 0, S), "mode must be 0")
+    err(L.dq_bitrate_search(P, 100, 0, ctypes.c_double(0.0), N, ctypes.c_double(4.0), P, 0, S), "hist buffer is too small")
+    err(L.dq_bitrate_search(P, 32768, 1, ctypes.c_double(float("nan")), N, ctypes.c_double(4.0), P, 0, S), "must be numbers")
+    err(L.dq_bitrate_search(P, 32768, 0, ctypes.c_double(0.0), N, ctypes.c_double(4.0), N, 0, S), "null pointer")
     err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 0, 0, 2, S), "unsupported element dtype")        # binary16 has no row-list kernels
     err(L.dq_scaling_compress_rows(P, P, P, P, 10, 4, 1, 0, 1, S), "strategy")
     err(L.dq_scaling_dec_comp_rows(P, P, P, P, P, 0, 4, 1, 0, 2, S), "n must be positive")
