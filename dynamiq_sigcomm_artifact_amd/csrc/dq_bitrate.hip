@@ -30,11 +30,11 @@ __device__ __forceinline__ int bin_of(uint32_t pattern)
     return (pattern & 0x7fffu) > (uint32_t)kMaxPattern ? kNanBin : 0;
 }
 
-// A workgroup counts rounds of up to 8192 norms in LDS -- 16-bit counters, two per word, so the whole range of
-// patterns fits into 64 KB -- and adds the non-zero counters to the histogram in memory after each round: a few
-// hundred atomics per round instead of one per norm, most of which would hit the same few hundred words.
+// A workgroup counts batches of up to 8192 norms in LDS -- 16-bit counters, two per word, so the whole range of
+// patterns fits into 64 KB -- and adds the non-zero counters to the histogram in memory after each batch: a few
+// hundred atomics per batch instead of one per norm, most of which would hit the same few hundred words.
 constexpr int kHistThreads = 1024;
-constexpr int kHistRound = 8192;               // norms per round (a 16-bit counter holds up to 65535)
+constexpr int kHistBatch = 8192;               // norms per batch (a 16-bit counter holds up to 65535)
 constexpr int kHistWords = 16384;              // 32768 counters
 
 __global__ __launch_bounds__(kHistThreads) void norm_histogram_kernel(const uint16_t *__restrict__ stats, int64_t nsc,
@@ -42,11 +42,11 @@ __global__ __launch_bounds__(kHistThreads) void norm_histogram_kernel(const uint
 {
     __shared__ uint32_t local[kHistWords];
     const int t = threadIdx.x;
-    for (int64_t round0 = (int64_t)blockIdx.x * kHistRound; round0 < nsc; round0 += (int64_t)gridDim.x * kHistRound) {
+    for (int64_t batch0 = (int64_t)blockIdx.x * kHistBatch; batch0 < nsc; batch0 += (int64_t)gridDim.x * kHistBatch) {
         for (int w = t; w < kHistWords; w += kHistThreads) local[w] = 0u;
         __syncthreads();
-        const int64_t end = min(round0 + kHistRound, nsc);
-        for (int64_t i = round0 + t; i < end; i += kHistThreads) {
+        const int64_t end = min(batch0 + kHistBatch, nsc);
+        for (int64_t i = batch0 + t; i < end; i += kHistThreads) {
             const int bin = bin_of(stats[2 * i + 1]);
             atomicAdd(&local[bin >> 1], 1u << (16 * (bin & 1)));
         }
@@ -177,7 +177,7 @@ int64_t bitrate_hist_ints() { return (int64_t)kSearchThreads * kBinsPerThread; }
 
 hipError_t launch_norm_histogram(const void *stats, int64_t nsc, uint32_t *hist, hipStream_t stream)
 {
-    const unsigned grid = (unsigned)std::min<int64_t>((nsc + kHistRound - 1) / kHistRound, 1024);
+    const unsigned grid = (unsigned)std::min<int64_t>((nsc + kHistBatch - 1) / kHistBatch, 1024);
     hipLaunchKernelGGL(norm_histogram_kernel, dim3(grid), dim3(kHistThreads), 0, stream, static_cast<const uint16_t *>(stats), nsc,
                        hist);
     return hipGetLastError();
