@@ -77,7 +77,7 @@ def lib():
         L.dq_group_plan_stats.restype = i32
         L.dq_group_plan_stats.argtypes = [vp, c.c_double, i64, vp, vp, vp, i64, i32, vp]
         L.dq_group_plan_stats_dev_u.restype = i32
-        L.dq_group_plan_stats_dev_u.argtypes = [vp, vp, i64, vp, vp, vp, i64, i32, vp]
+        L.dq_group_plan_stats_dev_u.argtypes = [vp, vp, i64, vp, vp, vp, i64, vp, i64, i32, vp]
         L.dq_bitrate_hist_ints.restype = i64
         L.dq_bitrate_hist_ints.argtypes = []
         L.dq_norm_histogram.restype = i32
@@ -229,9 +229,10 @@ def group_rows(order, nsc, width, count):
     return order[base:base + count]
 
 
-def group_plan_stats(stats, u, qbits_out, order, work, stream=None):
+def group_plan_stats(stats, u, qbits_out, order, work, stream=None, hist=None):
     """stats bf16 [nsc, 2] (mean, reduced sum of squares), offset u (a number, or a float64 device tensor read when the
-    kernels run) -> qbits_out (int64 or None), order, work"""
+    kernels run) -> qbits_out (int64 or None), order, work; hist (int32 [bitrate_hist_ints()] or None) also gets the bucket's
+    norm patterns -- within the same launch when u is a device tensor"""
     if stats.dtype != torch.bfloat16 or order.dtype != torch.int32 or work.dtype != torch.int32:
         raise RuntimeError("group_plan_stats: stats must be bfloat16, order and work int32")
     nsc = stats.numel() // 2
@@ -241,9 +242,14 @@ def group_plan_stats(stats, u, qbits_out, order, work, stream=None):
         # the offset stays on the device (one float64, e.g. the first entry of bitrate_search's result)
         if u.dtype != torch.float64 or u.numel() < 1 or u.device != stats.device:
             raise RuntimeError("group_plan_stats: a tensor u must be float64 on the device of stats")
+        if hist is not None and hist.dtype != torch.int32:
+            raise RuntimeError("group_plan_stats: hist must be int32")
         _check(lib().dq_group_plan_stats_dev_u(stats.data_ptr(), u.data_ptr(), nsc, _ptr(qbits_out), order.data_ptr(),
-                                               work.data_ptr(), work.numel(), _dev(stats), _stream(stream)))
+                                               work.data_ptr(), work.numel(), _ptr(hist), 0 if hist is None else hist.numel(),
+                                               _dev(stats), _stream(stream)))
         return
+    if hist is not None:
+        norm_histogram(stats, hist, stream)
     _check(lib().dq_group_plan_stats(stats.data_ptr(), float(u), nsc, _ptr(qbits_out), order.data_ptr(), work.data_ptr(),
                                      work.numel(), _dev(stats), _stream(stream)))
 

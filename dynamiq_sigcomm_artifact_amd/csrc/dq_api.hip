@@ -308,18 +308,20 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
     if (work_ints < dq::group_plan_work_ints(nsc)) return fail(DQ_ERR_SIZE, "work buffer is too small");
     int rc;
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_group_plan_stats(stats, (float)u, nullptr, nsc, qbits_out, order, work, static_cast<hipStream_t>(stream)));
+    return finish(dq::launch_group_plan_stats(stats, (float)u, nullptr, nsc, qbits_out, order, work, nullptr, static_cast<hipStream_t>(stream)));
 }
 
 int dq_group_plan_stats_dev_u(const void *stats, const double *u_dev, int64_t nsc, int64_t *qbits_out, int32_t *order,
-                              int32_t *work, int64_t work_ints, int device, dq_stream_t stream)
+                              int32_t *work, int64_t work_ints, uint32_t *hist, int64_t hist_ints, int device,
+                              dq_stream_t stream)
 {
     if (!(nsc > 0) || nsc > (int64_t)0x7fffffff) return fail(DQ_ERR_N, "nsc must be in [1, 2^31)");
     if (!stats || !u_dev || !order || !work) return fail(DQ_ERR_NULL);
     if (work_ints < dq::group_plan_work_ints(nsc)) return fail(DQ_ERR_SIZE, "work buffer is too small");
+    if (hist && hist_ints < dq::bitrate_hist_ints()) return fail(DQ_ERR_SIZE, "hist buffer is too small");
     int rc;
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_group_plan_stats(stats, 0.0f, u_dev, nsc, qbits_out, order, work, static_cast<hipStream_t>(stream)));
+    return finish(dq::launch_group_plan_stats(stats, 0.0f, u_dev, nsc, qbits_out, order, work, hist, static_cast<hipStream_t>(stream)));
 }
 
 int64_t dq_bitrate_hist_ints(void) { return dq::bitrate_hist_ints(); }

@@ -19,45 +19,14 @@ namespace dq {
 
 namespace {
 
-constexpr int kNanBin = kMaxPattern + 1;       // NaN norms: 2 bits whatever u is
 constexpr int kSearchThreads = 1024;
 constexpr int kBinsPerThread = 32;             // 1024 x 32 = 32768 >= kNanBin + 1
-
-// negative norms (and -0) are clamped to the same epsilon as +0: bin 0
-__device__ __forceinline__ int bin_of(uint32_t pattern)
-{
-    if (pattern <= (uint32_t)kMaxPattern) return (int)pattern;
-    return (pattern & 0x7fffu) > (uint32_t)kMaxPattern ? kNanBin : 0;
-}
-
-// A workgroup counts batches of up to 8192 norms in LDS -- 16-bit counters, two per word, so the whole range of
-// patterns fits into 64 KB -- and adds the non-zero counters to the histogram in memory after each batch: a few
-// hundred atomics per batch instead of one per norm, most of which would hit the same few hundred words.
-constexpr int kHistThreads = 1024;
-constexpr int kHistBatch = 8192;               // norms per batch (a 16-bit counter holds up to 65535)
-constexpr int kHistWords = 16384;              // 32768 counters
 
 __global__ __launch_bounds__(kHistThreads) void norm_histogram_kernel(const uint16_t *__restrict__ stats, int64_t nsc,
                                                                      uint32_t *__restrict__ hist)
 {
     __shared__ uint32_t local[kHistWords];
-    const int t = threadIdx.x;
-    for (int64_t batch0 = (int64_t)blockIdx.x * kHistBatch; batch0 < nsc; batch0 += (int64_t)gridDim.x * kHistBatch) {
-        for (int w = t; w < kHistWords; w += kHistThreads) local[w] = 0u;
-        __syncthreads();
-        const int64_t end = min(batch0 + kHistBatch, nsc);
-        for (int64_t i = batch0 + t; i < end; i += kHistThreads) {
-            const int bin = bin_of(stats[2 * i + 1]);
-            atomicAdd(&local[bin >> 1], 1u << (16 * (bin & 1)));
-        }
-        __syncthreads();
-        for (int w = t; w < kHistWords; w += kHistThreads) {
-            const uint32_t pair = local[w];
-            if (pair & 0xffffu) atomicAdd(&hist[2 * w], pair & 0xffffu);
-            if (pair >> 16) atomicAdd(&hist[2 * w + 1], pair >> 16);
-        }
-        __syncthreads();
-    }
+    count_norm_patterns(stats, nsc, (int64_t)blockIdx.x * kHistBatch, (int64_t)gridDim.x * kHistBatch, hist, local);
 }
 
 struct Probe {

@@ -55,4 +55,45 @@ __device__ __forceinline__ void width_thresholds(float u, int *thr, int wave, in
     if (lane == 0) thr[wave] = t;
 }
 
+// ---- histogram of the norm patterns (what the search for u works on) ----------------------------------
+
+constexpr int kNanBin = kMaxPattern + 1; // NaN norms: 2 bits whatever u is
+
+// negative norms (and -0) are clamped to the same epsilon as +0: bin 0
+__device__ __forceinline__ int bin_of(uint32_t pattern)
+{
+    if (pattern <= (uint32_t)kMaxPattern) return (int)pattern;
+    return (pattern & 0x7fffu) > (uint32_t)kMaxPattern ? kNanBin : 0;
+}
+
+// A workgroup of kHistThreads threads counts batches of up to 8192 norms in LDS -- 16-bit counters, two per word,
+// so the whole range of patterns fits into 64 KB -- and adds the non-zero counters to the histogram in memory
+// after each batch: a few hundred atomics per batch instead of one per norm, most of which would hit the same
+// few hundred words.  The workgroup takes the batches first, first + stride, ...; local: kHistWords words of LDS.
+constexpr int kHistThreads = 1024;
+constexpr int kHistBatch = 8192; // norms per batch (a 16-bit counter holds up to 65535)
+constexpr int kHistWords = 16384; // 32768 counters
+
+__device__ __forceinline__ void count_norm_patterns(const uint16_t *__restrict__ stats, int64_t nsc, int64_t first,
+                                                    int64_t stride, uint32_t *__restrict__ hist, uint32_t *local)
+{
+    const int t = threadIdx.x;
+    for (int64_t batch0 = first; batch0 < nsc; batch0 += stride) {
+        for (int w = t; w < kHistWords; w += kHistThreads) local[w] = 0u;
+        __syncthreads();
+        const int64_t end = min(batch0 + kHistBatch, nsc);
+        for (int64_t i = batch0 + t; i < end; i += kHistThreads) {
+            const int bin = bin_of(stats[2 * i + 1]);
+            atomicAdd(&local[bin >> 1], 1u << (16 * (bin & 1)));
+        }
+        __syncthreads();
+        for (int w = t; w < kHistWords; w += kHistThreads) {
+            const uint32_t pair = local[w];
+            if (pair & 0xffffu) atomicAdd(&hist[2 * w], pair & 0xffffu);
+            if (pair >> 16) atomicAdd(&hist[2 * w + 1], pair >> 16);
+        }
+        __syncthreads();
+    }
+}
+
 } // namespace dq

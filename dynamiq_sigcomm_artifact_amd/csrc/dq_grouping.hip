@@ -42,6 +42,8 @@ struct WidthsFromArray {
     typedef int64_t Raw;
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
     bool word_aligned() const { return true; }
+    __device__ __forceinline__ const uint16_t *norm_stats() const { return nullptr; }
+    const void *norm_stats_host() const { return nullptr; }
     __device__ __forceinline__ void resolve() {}
     __device__ __forceinline__ void prepare(int *, int, int) const {}
     __device__ __forceinline__ Raw load(int i) const { return qbits[i]; }
@@ -53,6 +55,8 @@ struct WidthsFromStats {
     float u;
     const double *u_dev;  // when set, the offset is read from device memory (the search for u leaves it there)
     typedef uint32_t Raw; // a (mean, norm) pair: the norm pattern is the high half
+    __device__ __forceinline__ const uint16_t *norm_stats() const { return stats; }
+    const void *norm_stats_host() const { return stats; }
     __device__ __forceinline__ void resolve()
     {
         if (u_dev) u = (float)*u_dev;
@@ -79,12 +83,23 @@ constexpr int kOneThreads = kTile; // one superchunk per thread while placing
 constexpr int kOneMaxTiles = 64;
 constexpr int kOneBatch = 8;       // loads in flight per thread while recounting the tiles before
 
-template <class W>
+// HIST: the launch has a few workgroups more than tiles (one per 8192 superchunks); they add the norm patterns of the
+// bucket to `hist` (what the search for the next step's u works on) while the others plan, so the histogram costs no
+// launch of its own.
+template <class W, bool HIST>
 __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t *__restrict__ qbits_out, int nsc,
-                                                              int32_t *__restrict__ order, int32_t *__restrict__ work)
+                                                              int32_t *__restrict__ order, int32_t *__restrict__ work,
+                                                              uint32_t *__restrict__ hist)
 {
+    static_assert(kOneThreads == kHistThreads, "the histogram workgroup has the shape of the others");
+    __shared__ uint32_t local[HIST ? kHistWords : 1];
     __shared__ int thr[2];
     __shared__ uint64_t before_sum[kOneThreads / 64], scan_sum[kOneThreads / 64];
+    if (HIST && (int)blockIdx.x >= (nsc + kTile - 1) / kTile) {
+        const int64_t h = (int)blockIdx.x - (nsc + kTile - 1) / kTile; // one batch each
+        count_norm_patterns(widths.norm_stats(), nsc, h * kHistBatch, (int64_t)gridDim.x * kHistBatch, hist, local);
+        return;
+    }
     widths.resolve();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nbefore = (int)blockIdx.x * kTile; // superchunks of the tiles before this one
@@ -141,7 +156,7 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
         tile_all += scan_sum[k];
     }
     if (c < 3) order[(int64_t)c * nsc + field(before, c) + field(excl, c)] = own;
-    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+    if ((int)blockIdx.x == (nsc + kTile - 1) / kTile - 1 && threadIdx.x == 0) { // the last tile (a histogram workgroup may follow)
         const uint64_t all = before + tile_all;
         work[0] = field(all, 0);
         work[1] = field(all, 1);
@@ -247,14 +262,24 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
 
 int64_t group_plan_work_ints(int64_t nsc) { return 8 + 4 * ((nsc + kTile - 1) / kTile); }
 
+// hist (only with widths from statistics): the bucket's norm patterns are added to it
 template <class W>
-static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *order, int32_t *work, hipStream_t stream)
+static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *order, int32_t *work, uint32_t *hist,
+                           hipStream_t stream)
 {
     const int ntiles = (int)((nsc + kTile - 1) / kTile);
     if (ntiles <= kOneMaxTiles && widths.word_aligned()) {
-        hipLaunchKernelGGL(plan_one_kernel<W>, dim3(ntiles), dim3(kOneThreads), 0, stream, widths, qbits_out, (int)nsc, order,
-                           work);
+        if (hist)
+            hipLaunchKernelGGL((plan_one_kernel<W, true>), dim3(ntiles + (int)((nsc + kHistBatch - 1) / kHistBatch)),
+                               dim3(kOneThreads), 0, stream, widths, qbits_out, (int)nsc, order, work, hist);
+        else
+            hipLaunchKernelGGL((plan_one_kernel<W, false>), dim3(ntiles), dim3(kOneThreads), 0, stream, widths, qbits_out,
+                               (int)nsc, order, work, hist);
         return hipGetLastError();
+    }
+    if (hist) {
+        const hipError_t eh = launch_norm_histogram(widths.norm_stats_host(), nsc, hist, stream);
+        if (eh != hipSuccess) return eh;
     }
     hipLaunchKernelGGL(plan_count_kernel<W>, dim3(ntiles), dim3(kThreads), 0, stream, widths, nsc, work);
     hipError_t e = hipGetLastError();
@@ -265,14 +290,14 @@ static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *o
 
 hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, int32_t *work, hipStream_t stream)
 {
-    return run_plan(WidthsFromArray{qbits}, nullptr, nsc, order, work, stream);
+    return run_plan(WidthsFromArray{qbits}, nullptr, nsc, order, work, nullptr, stream);
 }
 
 // u_dev != nullptr: the offset is *u_dev at the time the kernels run, u is ignored
 hipError_t launch_group_plan_stats(const void *stats, float u, const double *u_dev, int64_t nsc, int64_t *qbits_out,
-                                   int32_t *order, int32_t *work, hipStream_t stream)
+                                   int32_t *order, int32_t *work, uint32_t *hist, hipStream_t stream)
 {
-    return run_plan(WidthsFromStats{static_cast<const uint16_t *>(stats), u, u_dev}, qbits_out, nsc, order, work, stream);
+    return run_plan(WidthsFromStats{static_cast<const uint16_t *>(stats), u, u_dev}, qbits_out, nsc, order, work, hist, stream);
 }
 
 } // namespace dq

@@ -62,7 +62,7 @@ hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, 
                              hipStream_t stream);
 // the same with the widths computed from the norm column of the bf16 stats and the offset u
 hipError_t launch_group_plan_stats(const void *stats, float u, const double *u_dev, int64_t nsc, int64_t *qbits_out,
-                                   int32_t *order, int32_t *work, hipStream_t stream);
+                                   int32_t *order, int32_t *work, uint32_t *hist, hipStream_t stream);
 
 // the offset u of the bit-width rule from a histogram of the norm patterns (dq_bitrate.hip)
 int64_t bitrate_hist_ints();

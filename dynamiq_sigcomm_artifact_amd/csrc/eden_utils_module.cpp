@@ -386,7 +386,8 @@ torch::Tensor group_plan_stats(torch::Tensor stats, double u, torch::Tensor orde
 }
 
 torch::Tensor group_plan_stats_dev_u(torch::Tensor stats, torch::Tensor u, torch::Tensor order,
-                                     c10::optional<torch::Tensor> qbits_out, uint64_t stream_p = 0)
+                                     c10::optional<torch::Tensor> qbits_out, c10::optional<torch::Tensor> hist,
+                                     uint64_t stream_p = 0)
 {
     TORCH_CHECK(stats.device().type() == torch::kCUDA, "stats must be a CUDA tensor");
     TORCH_CHECK(order.device().type() == torch::kCUDA, "order must be a CUDA tensor");
@@ -406,8 +407,18 @@ torch::Tensor group_plan_stats_dev_u(torch::Tensor stats, torch::Tensor u, torch
         qptr = qbits_out->data_ptr<int64_t>();
     }
     auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
+    uint32_t *hptr = nullptr;
+    int64_t hlen = 0;
+    if (hist.has_value()) {
+        TORCH_CHECK(hist->device() == stats.device() && hist->dtype() == torch::kInt32 && hist->is_contiguous() &&
+                        hist->numel() >= dq_bitrate_hist_ints(),
+                    "hist must be a contiguous torch.int32 tensor of bitrate_hist_ints() entries on the device of stats");
+        hptr = reinterpret_cast<uint32_t *>(hist->data_ptr<int32_t>());
+        hlen = hist->numel();
+    }
     check_status(dq_group_plan_stats_dev_u(stats.data_ptr(), u.data_ptr<double>(), nsc, qptr, order.data_ptr<int32_t>(),
-                                           work.data_ptr<int32_t>(), work.numel(), stats.device().index(), as_stream(stream_p)),
+                                           work.data_ptr<int32_t>(), work.numel(), hptr, hlen, stats.device().index(),
+                                           as_stream(stream_p)),
                  "group_plan_stats_dev_u");
     return work.slice(0, 0, 4);
 }
@@ -929,7 +940,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
     modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width into the three regions of order (8-bit rows from 0, 4-bit from nsc, 2-bit from 2 nsc); returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
     modul.def("group_plan_stats", &group_plan_stats, "bit widths from the reduced bf16 norms and the offset u, and the partition by width, in one call; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
-    modul.def("group_plan_stats_dev_u", &group_plan_stats_dev_u, "group_plan_stats with the offset u read from a float64 device tensor when the kernels run", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
+    modul.def("group_plan_stats_dev_u", &group_plan_stats_dev_u, "group_plan_stats with the offset u read from a float64 device tensor when the kernels run; hist also gets the bucket's norm patterns", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("hist") = py::none(), py::arg("stream_p") = 0);
     modul.def("bitrate_hist_ints", &bitrate_hist_ints, "int32 entries of the norm-pattern histogram");
     modul.def("norm_histogram", &norm_histogram, "adds the bf16 norm patterns of a bucket's statistics to the histogram", py::arg("stats"), py::arg("hist"), py::arg("stream_p") = 0);
     modul.def("bitrate_search", &bitrate_search, "the reference's search for the offset u (mode 0: bisection, 1: correction from prev_u) on the histogram, one launch; returns float64 [4] = u, average width, target - average, probes and leaves hist zeroed", py::arg("hist"), py::arg("mode"), py::arg("prev_u"), py::arg("target_avg_bits"), py::arg("stream_p") = 0);

@@ -136,7 +136,7 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
     u: the offset of the width rule, a number or a float64 device tensor (e.g. result[0:1] of the offset search: then
     nothing of the step is read back).
     norm_histogram: a bitrate.NormHistogram that collects the reduced norms of the step's buckets for the search of
-    the next step's u (comm_hooks.py:962, 904-931) -- one more small launch per bucket.
+    the next step's u (comm_hooks.py:962, 904-931).
 
     Returns (result tensors per rank, reduced stats, device int32 tensor [n8, n4, n2, other])."""
     from . import capi
@@ -171,9 +171,11 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         total.copy_(stats[0])
         for r in range(1, W):
             total.add_(stats[r])
-    capi.group_plan_stats(total, u if isinstance(u, torch.Tensor) else float(u), None, order, plan, stream=stream)
+    # with u on the device the histogram is filled by a few more workgroups of the plan launch, otherwise by a launch of its own
+    capi.group_plan_stats(total, u if isinstance(u, torch.Tensor) else float(u), None, order, plan, stream=stream,
+                          hist=None if norm_histogram is None else norm_histogram.hist)
     if norm_histogram is not None:
-        norm_histogram.add(total, stream=stream)
+        norm_histogram.count += nsc
     outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
 
     def encode(r, chunk, step, received=None):

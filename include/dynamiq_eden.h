@@ -170,11 +170,14 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
 
 /* the same with the offset read from device memory when the kernels run
  * (u_dev: one float64, e.g. result[0] of dq_bitrate_search): a training step
- * then needs no read-back of u at all.  No counterpart in the reference, which
- * keeps u on the host. */
+ * then needs no read-back of u at all.  hist (may be NULL; dq_bitrate_hist_ints()
+ * uint32): the bucket's norm patterns are also added to it, as by
+ * dq_norm_histogram, by a few more workgroups of the same launch (for nsc <= 65536).
+ * No counterpart in the reference, which keeps u on the host. */
 int dq_group_plan_stats_dev_u(const void *stats, const double *u_dev, int64_t nsc,
                               int64_t *qbits_out, int32_t *order, int32_t *work,
-                              int64_t work_ints, int device, dq_stream_t stream);
+                              int64_t work_ints, uint32_t *hist, int64_t hist_ints, int device,
+                              dq_stream_t stream);
 
 /* ---- the offset u of the bit-width rule (comm_hooks.py:73-139) -----------
  *

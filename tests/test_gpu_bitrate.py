@@ -182,3 +182,30 @@ def test_steps_chained_on_the_device(capi, oracle):
         capi.group_plan_stats(_stats(norms_list[0]), h.result[0:1], q, order, work)
         assert (q.cpu().numpy() == oracle.dynamic_bitrate_qbits(bits[0], want[0])).all()
     assert tuple(h.result[:3].tolist()) == tuple(want)
+
+
+@pytest.mark.parametrize("nsc", [1, 1000, 25600, 65536, 70000])
+def test_plan_launch_fills_the_histogram(capi, nsc):
+    """the histogram workgroup of the plan launch (and the separate launch beyond 65536 superchunks) counts what
+    norm_histogram counts, and leaves the plan as it is"""
+    g = torch.Generator().manual_seed(nsc)
+    norms = torch.exp(torch.randn(nsc, generator=g) * 4 - 6).to(torch.bfloat16)
+    if nsc > 10:
+        norms[3], norms[5], norms[7] = float("nan"), -1.0, float("inf")
+    stats = _stats(norms)
+    u = torch.tensor([7.3, 0, 0, 0], dtype=torch.float64, device=DEV)
+    want = torch.full((capi.bitrate_hist_ints(),), 5, dtype=torch.int32, device=DEV)      # accumulates on top
+    got = want.clone()
+    capi.norm_histogram(stats, want)
+    order_a = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    order_b = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    work_a = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    work_b = torch.zeros_like(work_a)
+    capi.group_plan_stats(stats, u[0:1], None, order_a, work_a, hist=got)
+    capi.group_plan_stats(stats, 7.3, None, order_b, work_b)
+    assert torch.equal(got, want) and int(got.sum()) == 5 * got.numel() + nsc
+    assert torch.equal(order_a, order_b) and work_a[:4].tolist() == work_b[:4].tolist()
+    # a number for u and a histogram: the same counts through a launch of its own
+    again = torch.full_like(got, 5)
+    capi.group_plan_stats(stats, 7.3, None, order_b, work_b, hist=again)
+    assert torch.equal(again, want)

@@ -118,8 +118,9 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_group_plan(P, 0, P, P, 100, 0, S), "nsc")
     err(L.dq_group_plan(P, 5000, P, P, 8, 0, S), "work buffer is too small")
     err(L.dq_group_plan_stats(N, ctypes.c_double(1.0), 100, N, P, P, 100, 0, S), "null pointer")
-    err(L.dq_group_plan_stats_dev_u(P, N, 100, N, P, P, 100, 0, S), "null pointer")
-    err(L.dq_group_plan_stats_dev_u(P, P, 100, N, P, P, 3, 0, S), "work buffer is too small")
+    err(L.dq_group_plan_stats_dev_u(P, N, 100, N, P, P, 100, N, 0, 0, S), "null pointer")
+    err(L.dq_group_plan_stats_dev_u(P, P, 100, N, P, P, 3, N, 0, 0, S), "work buffer is too small")
+    err(L.dq_group_plan_stats_dev_u(P, P, 100, N, P, P, 100, P, 5, 0, S), "hist buffer is too small")
     err(L.dq_norm_histogram(P, 100, P, 100, 0, S), "hist buffer is too small")
     err(L.dq_norm_histogram(N, 100, P, 32768, 0, S), "null pointer")
     err(L.dq_norm_histogram(P, 0, P, 32768, 0, S), "nsc must be in")
