@@ -90,6 +90,10 @@ def test_offset_search_bindings(capi, eden_utils):
     capi.group_plan_stats(stats, rb[0:1], None, order_a, work)
     counts = eu.group_plan_stats_dev_u(stats, rb[0:1], order_b)
     assert counts.tolist() == work[:4].tolist() and torch.equal(order_a, order_b)
+    capi.norm_histogram(stats, ha)
+    assert eu.group_plan_stats_dev_u(stats, rb[0:1], order_b, None, hb).tolist() == counts.tolist() and torch.equal(ha, hb)
+    ha.zero_()
+    hb.zero_()
     with pytest.raises(RuntimeError, match="float64"):
         eu.group_plan_stats_dev_u(stats, rb[0:1].float(), order_b)
     with pytest.raises(RuntimeError, match="bitrate_hist_ints"):
