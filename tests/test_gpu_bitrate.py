@@ -128,8 +128,20 @@ def test_pipeline_feeds_the_histogram(oracle):
         _, total, _ = dynamic_bitrate_allreduce_single_pass(vecs, 7.0, norm_histogram=h)
         reduced.append(to_bits(total[:, 1].contiguous()))
     assert h.count == 177
+    counted = h.hist.clone()
     got = h.adjust_u(7.0, 4.375)
     assert got == tuple(oracle.dynamic_bitrate_adjust_u(reduced, 7.0, 4.375))
+    # the same step with u in device memory: the plan launches fill the histogram themselves, same counts, same outputs
+    g = torch.Generator().manual_seed(21)
+    u_dev = torch.tensor([7.0], dtype=torch.float64, device=DEV)
+    h2 = NormHistogram(DEV)
+    for nsc, W in ((40, 2), (7, 1), (130, 3)):
+        scales = torch.exp(torch.randn(nsc, 1, generator=g) * 4.0) * 1e-3
+        vecs = [(torch.randn(nsc, 256, generator=g) * scales).reshape(-1).to(torch.bfloat16).to(DEV) for _ in range(W)]
+        outs_a, _, plan_a = dynamic_bitrate_allreduce_single_pass(vecs, u_dev, norm_histogram=h2)
+        outs_b, _, plan_b = dynamic_bitrate_allreduce_single_pass(vecs, 7.0)
+        assert plan_a.tolist() == plan_b.tolist() and all(torch.equal(a, b) for a, b in zip(outs_a, outs_b))
+    assert h2.count == 177 and torch.equal(h2.hist, counted)
 
 
 @pytest.mark.parametrize("nsc", [3000, 70000])
