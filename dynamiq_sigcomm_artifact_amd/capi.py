@@ -105,7 +105,7 @@ def lib():
         L.dq_hadamard.restype = i32
         L.dq_hadamard.argtypes = [vp, i64, i32, vp, i32]
         L.dq_rht_blocked.restype = i32
-        L.dq_rht_blocked.argtypes = [vp, vp, i64, i64, f32, i32, i32, vp]
+        L.dq_rht_blocked.argtypes = [vp, vp, i32, i64, i64, f32, i32, i32, vp]
         L.dq_rht_scaling_compress.restype = i32
         L.dq_rht_scaling_compress.argtypes = [vp, vp, i32, vp, vp, i32, i64, i64, f32, i32, i32, i32, u64, u64, vp]
         L.dq_scaling_decompress_irht.restype = i32
@@ -129,9 +129,9 @@ def lib():
         L.dq_thc_dequantize.restype = i32
         L.dq_thc_dequantize.argtypes = [vp, vp, i64, vp, vp, i32, vp]
         L.dq_thc_rht_quantize.restype = i32
-        L.dq_thc_rht_quantize.argtypes = [vp, vp, vp, vp, i64, i64, f32, vp, vp, i32, i32, vp]
+        L.dq_thc_rht_quantize.argtypes = [vp, vp, i32, vp, vp, i64, i64, f32, vp, vp, i32, i32, vp]
         L.dq_thc_dequantize_irht.restype = i32
-        L.dq_thc_dequantize_irht.argtypes = [vp, vp, vp, i64, i64, f32, vp, vp, i32, vp]
+        L.dq_thc_dequantize_irht.argtypes = [vp, vp, i32, vp, i64, i64, f32, vp, vp, i32, vp]
         L.dq_quantization.restype = i32
         L.dq_quantization.argtypes = [vp, i64, i32, f32, f32, u64, vp]
         _lib = L
@@ -356,12 +356,25 @@ def hadamard(vec, stream=None):
 
 
 def rht_blocked(vec, sign, block, scale, inverse=False, stream=None):
-    _check(lib().dq_rht_blocked(vec.data_ptr(), 0 if sign is None else sign.data_ptr(), vec.numel(), block, float(scale),
+    """sign: None, float32 +-1 values, or the int32 bit vector of pack_signs"""
+    _check_sign(sign, vec.numel(), "rht_blocked")
+    _check(lib().dq_rht_blocked(vec.data_ptr(), _ptr(sign), _packed(sign), vec.numel(), block, float(scale),
                                 1 if inverse else 0, _dev(vec), _stream(stream)))
 
 
 def _packed(sign):
     return 1 if sign is not None and sign.dtype == torch.int32 else 0
+
+
+def _check_sign(sign, n, what):
+    """None, n float32 values or ceil(n / 32) int32 words"""
+    if sign is None:
+        return
+    if sign.dtype == torch.int32:
+        if sign.numel() < (n + 31) // 32:
+            raise RuntimeError(what + ": the packed sign vector is too short")
+    elif sign.dtype != torch.float32 or sign.numel() < n:
+        raise RuntimeError(what + ": sign must be float32 [n] or the int32 bit vector of pack_signs")
 
 
 def pack_signs(sign, stream=None):
@@ -467,9 +480,10 @@ def thc_rht_quantize(work, sign, uniform, levels_out, block, scale, lo, delta, l
             or lo.dtype != torch.float32 or delta.dtype != torch.float32:
         raise RuntimeError("thc_rht_quantize: work, uniform, lo, delta must be float32 and the output bfloat16")
     n = work.numel()
-    if uniform.numel() < n or levels_out.numel() < n or (sign is not None and sign.numel() < n):
+    if uniform.numel() < n or levels_out.numel() < n:
         raise RuntimeError("thc_rht_quantize: a buffer is too small")
-    _check(lib().dq_thc_rht_quantize(work.data_ptr(), _ptr(sign), uniform.data_ptr(), levels_out.data_ptr(), n, block,
+    _check_sign(sign, n, "thc_rht_quantize")
+    _check(lib().dq_thc_rht_quantize(work.data_ptr(), _ptr(sign), _packed(sign), uniform.data_ptr(), levels_out.data_ptr(), n, block,
                                      float(scale), lo.data_ptr(), delta.data_ptr(), levels, _dev(work), _stream(stream)))
 
 
@@ -479,7 +493,8 @@ def thc_dequantize_irht(levels_in, sign, out, block, scale, step, lo, stream=Non
             or lo.dtype != torch.float32:
         raise RuntimeError("thc_dequantize_irht: levels must be bfloat16, out, step, lo float32")
     n = out.numel()
-    if levels_in.numel() < n or (sign is not None and sign.numel() < n):
+    if levels_in.numel() < n:
         raise RuntimeError("thc_dequantize_irht: a buffer is too small")
-    _check(lib().dq_thc_dequantize_irht(levels_in.data_ptr(), _ptr(sign), out.data_ptr(), n, block, float(scale),
+    _check_sign(sign, n, "thc_dequantize_irht")
+    _check(lib().dq_thc_dequantize_irht(levels_in.data_ptr(), _ptr(sign), _packed(sign), out.data_ptr(), n, block, float(scale),
                                         step.data_ptr(), lo.data_ptr(), _dev(out), _stream(stream)))

@@ -537,15 +537,15 @@ int dq_hadamard(float *vec, int64_t n, int device, dq_stream_t stream, int depth
     return finish(dq::launch_hadamard(vec, n, static_cast<hipStream_t>(stream)));
 }
 
-int dq_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale, int inverse, int device,
-                   dq_stream_t stream)
+int dq_rht_blocked(float *vec, const void *sign, int sign_packed, int64_t n, int64_t block, float scale, int inverse,
+                   int device, dq_stream_t stream)
 {
     if (!(block > 0) || (block & (block - 1)) != 0) return fail(DQ_ERR_POW2, "block");
     if (!(n > 0) || n % block != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of block");
     if (!vec) return fail(DQ_ERR_NULL);
     int rc;
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_rht_blocked(vec, sign, n, block, scale, inverse, static_cast<hipStream_t>(stream)));
+    return finish(dq::launch_rht_blocked(vec, sign, sign_packed != 0, n, block, scale, inverse, static_cast<hipStream_t>(stream)));
 }
 
 static int check_rht_scaling(int64_t n, int64_t block, int nbits, int strategy)
@@ -671,26 +671,27 @@ static int check_thc_rht(int64_t n, int64_t block)
     return DQ_OK;
 }
 
-int dq_thc_rht_quantize(float *work, const float *sign, const float *uniform, void *levels_bf16, int64_t n, int64_t block,
-                        float scale, const float *lo, const float *delta, int levels, int device, dq_stream_t stream)
+int dq_thc_rht_quantize(float *work, const void *sign, int sign_packed, const float *uniform, void *levels_bf16, int64_t n,
+                        int64_t block, float scale, const float *lo, const float *delta, int levels, int device,
+                        dq_stream_t stream)
 {
     int rc = check_thc_rht(n, block);
     if (rc) return rc;
     if (levels < 2 || levels > 256) return fail(DQ_ERR_SIZE, "levels must be in [2, 256]");
     if (!work || !uniform || !levels_bf16 || !lo || !delta) return fail(DQ_ERR_NULL);
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_thc_rht_quantize(work, sign, uniform, levels_bf16, n, block, scale, lo, delta, levels,
+    return finish(dq::launch_thc_rht_quantize(work, sign, sign_packed != 0, uniform, levels_bf16, n, block, scale, lo, delta, levels,
                                               static_cast<hipStream_t>(stream)));
 }
 
-int dq_thc_dequantize_irht(const void *levels_bf16, const float *sign, float *out, int64_t n, int64_t block, float scale,
-                           const float *step, const float *lo, int device, dq_stream_t stream)
+int dq_thc_dequantize_irht(const void *levels_bf16, const void *sign, int sign_packed, float *out, int64_t n, int64_t block,
+                           float scale, const float *step, const float *lo, int device, dq_stream_t stream)
 {
     int rc = check_thc_rht(n, block);
     if (rc) return rc;
     if (!levels_bf16 || !out || !step || !lo) return fail(DQ_ERR_NULL);
     if ((rc = select_device(device))) return rc;
-    return finish(dq::launch_thc_dequantize_irht(levels_bf16, sign, out, n, block, scale, step, lo,
+    return finish(dq::launch_thc_dequantize_irht(levels_bf16, sign, sign_packed != 0, out, n, block, scale, step, lo,
                                                  static_cast<hipStream_t>(stream)));
 }
 

@@ -25,7 +25,8 @@ namespace dq {
 
 struct FwhtArgs {
     float *x;
-    const float *sign; // may be null
+    const float *sign;         // +-1 values, or null
+    const uint32_t *sign_bits; // or: one bit per element, set where the sign is negative (dq_pack_signs)
     int64_t n;         // elements in the vector (for bounds of ragged tiles)
     int kt;            // log2 tile elements
     int b0, b1;        // tile-index bits to transform: [b0, b1)
@@ -42,6 +43,28 @@ struct FwhtArgs {
     const float *uniform, *out_lo, *out_delta;
     float out_top;
 };
+
+// the diagonal of +-1 on four consecutive elements from g (a multiple of 4) / on element g: a multiplication by
+// the float value, or a flip of the sign bit where the packed bit is set (the same thing for +-1)
+__device__ __forceinline__ void apply_sign4(const FwhtArgs &a, float4 &v, int64_t g)
+{
+    if (a.sign_bits) {
+        const uint32_t w = a.sign_bits[g >> 5] >> (g & 31);
+        v.x = __uint_as_float(__float_as_uint(v.x) ^ ((w & 1u) << 31));
+        v.y = __uint_as_float(__float_as_uint(v.y) ^ ((w & 2u) << 30));
+        v.z = __uint_as_float(__float_as_uint(v.z) ^ ((w & 4u) << 29));
+        v.w = __uint_as_float(__float_as_uint(v.w) ^ ((w & 8u) << 28));
+    } else {
+        const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
+        v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
+    }
+}
+
+__device__ __forceinline__ float apply_sign1(const FwhtArgs &a, float v, int64_t g)
+{
+    if (a.sign_bits) return __uint_as_float(__float_as_uint(v) ^ (((a.sign_bits[g >> 5] >> (g & 31)) & 1u) << 31));
+    return v * a.sign[g];
+}
 
 __global__ void fwht_tile_kernel(FwhtArgs a)
 {
@@ -79,10 +102,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
                 } else {
                     v = *reinterpret_cast<const float4 *>(a.x + g);
                 }
-                if (a.sign_mode == 1) {
-                    const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
-                    v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
-                }
+                if (a.sign_mode == 1) apply_sign4(a, v, g);
             }
             const int q = pad_idx(i); // i % 4 == 0: the four floats stay inside one padded group of 16
             lds[q] = v.x; lds[q + 1] = v.y; lds[q + 2] = v.z; lds[q + 3] = v.w;
@@ -98,7 +118,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
                 } else {
                     v = a.x[g];
                 }
-                if (a.sign_mode == 1) v *= a.sign[g];
+                if (a.sign_mode == 1) v = apply_sign1(a, v, g);
             }
             lds[pad_idx(i)] = v;
         }
@@ -116,10 +136,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             const int q = pad_idx(i);
             float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
             if (a.apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
-            if (a.sign_mode == 2) {
-                const float4 s = *reinterpret_cast<const float4 *>(a.sign + g);
-                v.x *= s.x; v.y *= s.y; v.z *= s.z; v.w *= s.w;
-            }
+            if (a.sign_mode == 2) apply_sign4(a, v, g);
             if (a.out_levels) {
                 const float4 u = *reinterpret_cast<const float4 *>(a.uniform + g);
                 const float lo = *a.out_lo, delta = *a.out_delta;
@@ -137,7 +154,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             if (g >= a.n) continue;
             float v = lds[pad_idx(i)];
             if (a.apply_scale) v *= a.scale;
-            if (a.sign_mode == 2) v *= a.sign[g];
+            if (a.sign_mode == 2) v = apply_sign1(a, v, g);
             if (a.out_levels)
                 a.out_levels[g] = (uint16_t)f32_to_bf16_bits(thc_level(v, a.uniform[g], *a.out_lo, *a.out_delta, a.out_top));
             else
@@ -175,16 +192,19 @@ struct ThcEnds {
     float out_top = 0.0f;
 };
 
-static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, float scale, int apply_scale,
+// sign: float +-1 values, or (sign_packed) the bit vector of dq_pack_signs; may be null
+static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int64_t n, int kb, float scale, int apply_scale,
                               int inverse, hipStream_t stream, const ThcEnds &thc = ThcEnds())
 {
     const bool vec16 = (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
-                       (sign == nullptr || (reinterpret_cast<uintptr_t>(sign) & 15) == 0) &&
+                       (sign == nullptr || sign_packed || (reinterpret_cast<uintptr_t>(sign) & 15) == 0) &&
                        (reinterpret_cast<uintptr_t>(thc.in_levels) & 7) == 0 &&
                        (reinterpret_cast<uintptr_t>(thc.out_levels) & 7) == 0 &&
                        (reinterpret_cast<uintptr_t>(thc.uniform) & 15) == 0;
     FwhtArgs a;
-    a.x = x; a.sign = sign; a.n = n; a.scale = scale;
+    a.x = x; a.n = n; a.scale = scale;
+    a.sign = sign_packed ? nullptr : static_cast<const float *>(sign);
+    a.sign_bits = sign_packed ? static_cast<const uint32_t *>(sign) : nullptr;
     a.in_levels = nullptr; a.in_step = thc.in_step; a.in_lo = thc.in_lo;
     a.out_levels = nullptr; a.uniform = thc.uniform; a.out_lo = thc.out_lo; a.out_delta = thc.out_delta;
     a.out_top = thc.out_top;
@@ -235,34 +255,34 @@ static hipError_t fwht_blocks(float *x, const float *sign, int64_t n, int kb, fl
 
 hipError_t launch_hadamard(float *vec, int64_t n, hipStream_t stream)
 {
-    return fwht_blocks(vec, nullptr, n, ilog2(n), 1.0f, 0, 0, stream);
+    return fwht_blocks(vec, nullptr, false, n, ilog2(n), 1.0f, 0, 0, stream);
 }
 
-hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale, int inverse,
-                              hipStream_t stream)
+hipError_t launch_rht_blocked(float *vec, const void *sign, bool sign_packed, int64_t n, int64_t block, float scale,
+                              int inverse, hipStream_t stream)
 {
-    return fwht_blocks(vec, sign, n, ilog2(block), scale, 1, inverse, stream);
+    return fwht_blocks(vec, sign, sign_packed, n, ilog2(block), scale, 1, inverse, stream);
 }
 
 // rotate (forward) and quantise: vec is read and left holding intermediate values
-hipError_t launch_thc_rht_quantize(float *vec, const float *sign, const float *uniform, void *levels_out, int64_t n,
-                                   int64_t block, float scale, const float *lo, const float *delta, int levels,
+hipError_t launch_thc_rht_quantize(float *vec, const void *sign, bool sign_packed, const float *uniform, void *levels_out,
+                                   int64_t n, int64_t block, float scale, const float *lo, const float *delta, int levels,
                                    hipStream_t stream)
 {
     ThcEnds thc;
     thc.out_levels = static_cast<uint16_t *>(levels_out);
     thc.uniform = uniform; thc.out_lo = lo; thc.out_delta = delta; thc.out_top = (float)(levels - 1);
-    return fwht_blocks(vec, sign, n, ilog2(block), scale, 1, 0, stream, thc);
+    return fwht_blocks(vec, sign, sign_packed, n, ilog2(block), scale, 1, 0, stream, thc);
 }
 
 // dequantise and rotate back into out
-hipError_t launch_thc_dequantize_irht(const void *levels_in, const float *sign, float *out, int64_t n, int64_t block,
-                                      float scale, const float *step, const float *lo, hipStream_t stream)
+hipError_t launch_thc_dequantize_irht(const void *levels_in, const void *sign, bool sign_packed, float *out, int64_t n,
+                                      int64_t block, float scale, const float *step, const float *lo, hipStream_t stream)
 {
     ThcEnds thc;
     thc.in_levels = static_cast<const uint16_t *>(levels_in);
     thc.in_step = step; thc.in_lo = lo;
-    return fwht_blocks(out, sign, n, ilog2(block), scale, 1, 1, stream, thc);
+    return fwht_blocks(out, sign, sign_packed, n, ilog2(block), scale, 1, 1, stream, thc);
 }
 
 // ---- randDiag -----------------------------------------------------------------------

@@ -90,15 +90,16 @@ hipError_t launch_add_mean_copy(const void *residual, void *dst, const void *sta
 
 // Walsh-Hadamard (dq_hadamard.hip)
 hipError_t launch_hadamard(float *vec, int64_t n, hipStream_t stream);
-hipError_t launch_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale,
+// sign: float +-1 values, or (sign_packed) the bit vector of launch_pack_signs; may be null
+hipError_t launch_rht_blocked(float *vec, const void *sign, bool sign_packed, int64_t n, int64_t block, float scale,
                               int inverse, hipStream_t stream);
 hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream);
 // THC's quantiser folded into the last pass of the forward transform / the first pass of the inverse one
-hipError_t launch_thc_rht_quantize(float *vec, const float *sign, const float *uniform, void *levels_out, int64_t n,
-                                   int64_t block, float scale, const float *lo, const float *delta, int levels,
+hipError_t launch_thc_rht_quantize(float *vec, const void *sign, bool sign_packed, const float *uniform, void *levels_out,
+                                   int64_t n, int64_t block, float scale, const float *lo, const float *delta, int levels,
                                    hipStream_t stream);
-hipError_t launch_thc_dequantize_irht(const void *levels_in, const float *sign, float *out, int64_t n, int64_t block,
-                                      float scale, const float *step, const float *lo, hipStream_t stream);
+hipError_t launch_thc_dequantize_irht(const void *levels_in, const void *sign, bool sign_packed, float *out, int64_t n,
+                                      int64_t block, float scale, const float *step, const float *lo, hipStream_t stream);
 
 // blocked randomized Hadamard transform fused with the hierarchical chunk-16 quantiser (dq_rht_scaling.hip);
 // rand_kind: DQ_F32 or DQ_BF16 pool, or 3 for the in-kernel stream (rnd ignored)

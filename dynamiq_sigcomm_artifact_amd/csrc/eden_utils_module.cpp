@@ -111,21 +111,17 @@ void quantization_compression(torch::Tensor vec, float div_factor, float tensor_
 
 void set_quantization_seed(uint64_t seed) { g_quant_seed.store(seed); }
 
+static const void *sign_arg(const c10::optional<torch::Tensor> &sign, const torch::Tensor &vec, int64_t n, int *packed);
+
 torch::Tensor rht_blocked(torch::Tensor vec, c10::optional<torch::Tensor> sign, int64_t block, double scale, bool inverse,
                           uint64_t stream_p = 0)
 {
     TORCH_CHECK(vec.device().type() == torch::kCUDA, "input must be a CUDA tensor");
     TORCH_CHECK(vec.dtype() == torch::kFloat32, "input must be a torch.float32 CUDA tensor");
     TORCH_CHECK(vec.is_contiguous(), "input must be contiguous");
-    const float *sp = nullptr;
-    if (sign.has_value()) {
-        TORCH_CHECK(sign->device() == vec.device(), "sign must be on the same device as the input");
-        TORCH_CHECK(sign->dtype() == torch::kFloat32, "sign must be torch.float32");
-        TORCH_CHECK(sign->is_contiguous(), "sign must be contiguous");
-        TORCH_CHECK(sign->numel() >= vec.numel(), "sign has fewer elements than the input");
-        sp = sign->data_ptr<float>();
-    }
-    check_status(dq_rht_blocked(vec.data_ptr<float>(), sp, vec.numel(), block, (float)scale, inverse ? 1 : 0,
+    int packed = 0;
+    const void *sp = sign_arg(sign, vec, vec.numel(), &packed);
+    check_status(dq_rht_blocked(vec.data_ptr<float>(), sp, packed, vec.numel(), block, (float)scale, inverse ? 1 : 0,
                                 vec.device().index(), as_stream(stream_p)),
                  "rht_blocked");
     return vec;
@@ -860,14 +856,6 @@ void thc_dequantize(torch::Tensor levels, torch::Tensor out, torch::Tensor step,
                  "thc_dequantize");
 }
 
-static const float *thc_sign_arg(const c10::optional<torch::Tensor> &sign, int64_t n)
-{
-    if (!sign.has_value()) return nullptr;
-    check_f32_cuda(*sign, "sign");
-    TORCH_CHECK(sign->numel() >= n, "sign has fewer elements than the vector");
-    return sign->data_ptr<float>();
-}
-
 void thc_rht_quantize(torch::Tensor work, c10::optional<torch::Tensor> sign, torch::Tensor uniform, torch::Tensor levels_out,
                       int64_t block, double scale, torch::Tensor lo, torch::Tensor delta, int levels, uint64_t stream_p = 0)
 {
@@ -880,7 +868,9 @@ void thc_rht_quantize(torch::Tensor work, c10::optional<torch::Tensor> sign, tor
     const int64_t n = work.numel();
     TORCH_CHECK(uniform.numel() >= n && levels_out.numel() >= n, "uniform or levels_out has fewer elements than work");
     TORCH_CHECK(lo.numel() == 1 && delta.numel() == 1, "lo and delta must hold one value");
-    check_status(dq_thc_rht_quantize(work.data_ptr<float>(), thc_sign_arg(sign, n), uniform.data_ptr<float>(), levels_out.data_ptr(), n,
+    int packed = 0;
+    const void *sp = sign_arg(sign, work, n, &packed);
+    check_status(dq_thc_rht_quantize(work.data_ptr<float>(), sp, packed, uniform.data_ptr<float>(), levels_out.data_ptr(), n,
                                      block, (float)scale, lo.data_ptr<float>(), delta.data_ptr<float>(), levels,
                                      work.device().index(), as_stream(stream_p)),
                  "thc_rht_quantize");
@@ -897,7 +887,9 @@ void thc_dequantize_irht(torch::Tensor levels, c10::optional<torch::Tensor> sign
     const int64_t n = out.numel();
     TORCH_CHECK(levels.numel() >= n, "levels has fewer elements than out");
     TORCH_CHECK(step.numel() == 1 && lo.numel() == 1, "step and lo must hold one value");
-    check_status(dq_thc_dequantize_irht(levels.data_ptr(), thc_sign_arg(sign, n), out.data_ptr<float>(), n, block, (float)scale,
+    int packed = 0;
+    const void *sp = sign_arg(sign, out, n, &packed);
+    check_status(dq_thc_dequantize_irht(levels.data_ptr(), sp, packed, out.data_ptr<float>(), n, block, (float)scale,
                                         step.data_ptr<float>(), lo.data_ptr<float>(), out.device().index(), as_stream(stream_p)),
                  "thc_dequantize_irht");
 }

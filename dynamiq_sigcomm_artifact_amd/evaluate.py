@@ -715,6 +715,15 @@ def kernels(dev, n=6553600):
                                                                 capi.rht_blocked(y, sign, d, inv, True)), 26 * d, n=d, launches=3)
     line("thc_dequantize_irht (folded)", lambda: capi.thc_dequantize_irht(lev, sign, y, d, inv, delta, lo), 18 * d, n=d,
          launches=2)
+    # the same with the diagonal as packed bits
+    sbits = capi.pack_signs(sign)
+    for kb in (10, 15):
+        y.normal_(generator=g)
+        line("rht_blocked (packed signs)", lambda: capi.rht_blocked(y, sbits, 1 << kb, 1.0, False), 8.125 * d, n=d, block=1 << kb)
+    line("thc_rht_quantize (folded, packed signs)", lambda: capi.thc_rht_quantize(y, sbits, uni, lev, d, inv, lo, delta, 64),
+         18.125 * d, n=d, launches=2)
+    line("thc_dequantize_irht (folded, packed signs)", lambda: capi.thc_dequantize_irht(lev, sbits, y, d, inv, delta, lo),
+         14.125 * d, n=d, launches=2)
     # the transform folded into the hierarchical codec (blocks of 2^13, 4-bit)
     x32 = torch.randn(d, generator=g, device=dev) * 1e-3
     sign_bits = capi.pack_signs(sign)

@@ -77,19 +77,21 @@ class EdenHadamardRHT:
         self.random_diagonal = torch.empty(dim, dtype=torch.float32, device=device)
         self.random_diagonal.bernoulli_(0.5, generator=self.generator)
         self.random_diagonal.mul_(2.0).sub_(1.0)
+        # the kernels read the diagonal as one bit per element (1/32 of the traffic, same rotation)
+        self.diagonal_bits = capi.pack_signs(self.random_diagonal)
         # div_(math.sqrt(dim)) with a host scalar is a product with the float32 reciprocal on the device
         self.inv_sqrt = float(np.float32(1.0) / np.float32(math.sqrt(dim)))
 
     def rht(self, vec):
         if vec.numel() != self.dim:
             raise ValueError(f"expected {self.dim} elements, got {vec.numel()}")
-        capi.rht_blocked(vec, self.random_diagonal, self.dim, self.inv_sqrt, False)
+        capi.rht_blocked(vec, self.diagonal_bits, self.dim, self.inv_sqrt, False)
         return vec
 
     def irht(self, vec):
         if vec.numel() != self.dim:
             raise ValueError(f"expected {self.dim} elements, got {vec.numel()}")
-        capi.rht_blocked(vec, self.random_diagonal, self.dim, self.inv_sqrt, True)
+        capi.rht_blocked(vec, self.diagonal_bits, self.dim, self.inv_sqrt, True)
         return vec
 
 
@@ -140,7 +142,7 @@ class OldINCACudaHadamardCompressor:
         out = torch.empty(dim, dtype=torch.bfloat16, device=self.device)
         # rotation and quantiser in the transform's own passes: the rotated vector is never stored
         h = self.hadamards[name]
-        capi.thc_rht_quantize(work, h.random_diagonal, uniform, out, dim, h.inv_sqrt, min_coordinate.float().reshape(1),
+        capi.thc_rht_quantize(work, h.diagonal_bits, uniform, out, dim, h.inv_sqrt, min_coordinate.float().reshape(1),
                               delta.float().reshape(1), self.quantization_levels)
         return out
 
@@ -152,6 +154,6 @@ class OldINCACudaHadamardCompressor:
         min_coordinate, delta = self._coordinate_range(max_norm, dim)
         work = self._work_buffer(name)
         h = self.hadamards[name]
-        capi.thc_dequantize_irht(tensor, h.random_diagonal, work, dim, h.inv_sqrt,
+        capi.thc_dequantize_irht(tensor, h.diagonal_bits, work, dim, h.inv_sqrt,
                                  (delta / self.nclients).float().reshape(1), min_coordinate.float().reshape(1))
         return work[:orig_size]

@@ -338,15 +338,15 @@ int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const floa
  * pass stores dq_thc_quantize's levels instead of the rotated values.  work
  * (fp32 [n]) is the vector on entry and holds intermediate values on return
  * (the reference's work buffer is scratch as well, thc_hooks.py:152-158). */
-int dq_thc_rht_quantize(float *work, const float *sign, const float *uniform, void *levels_bf16,
-                        int64_t n, int64_t block, float scale, const float *lo, const float *delta,
-                        int levels, int device, dq_stream_t stream);
+int dq_thc_rht_quantize(float *work, const void *sign, int sign_packed, const float *uniform,
+                        void *levels_bf16, int64_t n, int64_t block, float scale, const float *lo,
+                        const float *delta, int levels, int device, dq_stream_t stream);
 
 /* thc_hooks.py:176-181: dq_thc_dequantize folded into the first pass of the
  * inverse transform of dq_rht_blocked; the result lands in out (fp32 [n]). */
-int dq_thc_dequantize_irht(const void *levels_bf16, const float *sign, float *out, int64_t n,
-                           int64_t block, float scale, const float *step, const float *lo,
-                           int device, dq_stream_t stream);
+int dq_thc_dequantize_irht(const void *levels_bf16, const void *sign, int sign_packed, float *out,
+                           int64_t n, int64_t block, float scale, const float *step,
+                           const float *lo, int device, dq_stream_t stream);
 
 /* ---- superchunk mean-centring ---------------------------------------- */
 
@@ -369,9 +369,12 @@ int dq_hadamard(float *vec, int64_t n, int device, dq_stream_t stream, int depth
 /* Extension (no reference entry point; fuses thc_hooks.py:95-107 /
  * srrcomp.py:317-319): per block of `block` = 2^k floats, in place,
  *   forward: y = FWHT(sign .* x) * scale,   inverse: y = sign .* (FWHT(x) * scale).
- * sign may be NULL (all +1).  n must be a multiple of block. */
-int dq_rht_blocked(float *vec, const float *sign, int64_t n, int64_t block, float scale,
-                   int inverse, int device, dq_stream_t stream);
+ * sign: fp32 [n] of +-1 values, or (sign_packed != 0) the bit vector written by
+ * dq_pack_signs -- 1/32 of the traffic, same result; NULL means all +1.
+ * n must be a multiple of block.  dq_thc_rht_quantize / dq_thc_dequantize_irht
+ * take sign the same way. */
+int dq_rht_blocked(float *vec, const void *sign, int sign_packed, int64_t n, int64_t block,
+                   float scale, int inverse, int device, dq_stream_t stream);
 /* Extension: dq_rht_blocked (forward) followed by dq_scaling_compress of the
  * rotated vector, without the rotated vector ever reaching memory -- a
  * workgroup keeps whole transform blocks in LDS and quantises them there.  src

@@ -247,8 +247,28 @@ def test_thc_quantiser_folded_into_the_transform(capi, n, block):
     back = torch.full((n,), 7.0, device=DEV)
     capi.thc_dequantize_irht(summed, sign, back, block, scale, step, lo)
     assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
+    # the diagonal as packed bits: the same levels, the same vector back, the same rotation
+    bits = capi.pack_signs(sign)
+    work.copy_(x)
+    got.zero_()
+    capi.thc_rht_quantize(work, bits, uni, got, block, scale, lo, delta, levels)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    back.fill_(7.0)
+    capi.thc_dequantize_irht(summed, bits, back, block, scale, step, lo)
+    assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
+    rot2 = x.clone()
+    capi.rht_blocked(rot2, bits, block, scale, False)
+    assert torch.equal(rot2.view(torch.int32), rot.view(torch.int32))
+    capi.rht_blocked(rot2, bits, block, scale, True)
+    capi.rht_blocked(rot, sign, block, scale, True)
+    assert torch.equal(rot2.view(torch.int32), rot.view(torch.int32))
     # buffers that are only element-aligned take the scalar paths
     if n <= 1 << 16:
+        r3 = torch.zeros(n + 4, device=DEV)[1:1 + n].copy_(x)
+        r4 = r3.clone()
+        capi.rht_blocked(r3, bits, block, scale, False)
+        capi.rht_blocked(r4, sign, block, scale, False)
+        assert torch.equal(r3.view(torch.int32), r4.view(torch.int32))
         w2 = torch.zeros(n + 4, device=DEV)[1:1 + n].copy_(x)
         u2 = torch.zeros(n + 4, device=DEV)[3:3 + n].copy_(uni)
         g2 = torch.zeros(n + 4, dtype=torch.bfloat16, device=DEV)[1:1 + n]

@@ -97,8 +97,8 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_superchunk_mean_center(P, P, P, 256, 2, 128, 1, 0, S), "superchunk_size must be 256")
     err(L.dq_superchunk_add_mean_copy(P, P, N, 256, 256, 1, 0, S), "null pointer")
     err(L.dq_hadamard(P, 1000, 0, S, 0), "power of 2")
-    err(L.dq_rht_blocked(P, P, 1024, 48, ctypes.c_float(1.0), 0, 0, S), "block")
-    err(L.dq_rht_blocked(P, P, 1000, 64, ctypes.c_float(1.0), 0, 0, S), "multiple of block")
+    err(L.dq_rht_blocked(P, P, 0, 1024, 48, ctypes.c_float(1.0), 0, 0, S), "block")
+    err(L.dq_rht_blocked(P, P, 1, 1000, 64, ctypes.c_float(1.0), 0, 0, S), "multiple of block")
     err(L.dq_rand_diag(P, 0, 1, 0, S), "n must be positive")
     F1 = ctypes.c_float(1.0)
     err(L.dq_rht_scaling_compress(P, P, 0, P, P, 2, 1024, 48, F1, 4, 0, 2, Z, Z, S), "power of 2")
@@ -151,12 +151,12 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_eden_dequantize(P, 64, P, 9, P, 0, S), "nbits")
     err(L.dq_eden_dequantize(P, 64, P, 4, ctypes.c_void_p(0x1004), 0, S), "16-byte aligned")
     err(L.dq_thc_quantize(P, P, P, 64, P, P, 1, 0, S), "levels")
-    err(L.dq_thc_rht_quantize(P, P, P, P, 96, 48, F1, P, P, 31, 0, S), "power of 2")
-    err(L.dq_thc_rht_quantize(P, P, P, P, 100, 64, F1, P, P, 31, 0, S), "multiple of block")
-    err(L.dq_thc_rht_quantize(P, P, P, P, 64, 64, F1, P, P, 1, 0, S), "levels")
-    err(L.dq_thc_rht_quantize(P, P, N, P, 64, 64, F1, P, P, 31, 0, S), "null pointer")
-    err(L.dq_thc_dequantize_irht(P, P, N, 64, 64, F1, P, P, 0, S), "null pointer")
-    err(L.dq_thc_dequantize_irht(P, P, P, 0, 64, F1, P, P, 0, S), "multiple of block")
+    err(L.dq_thc_rht_quantize(P, P, 0, P, P, 96, 48, F1, P, P, 31, 0, S), "power of 2")
+    err(L.dq_thc_rht_quantize(P, P, 1, P, P, 100, 64, F1, P, P, 31, 0, S), "multiple of block")
+    err(L.dq_thc_rht_quantize(P, P, 0, P, P, 64, 64, F1, P, P, 1, 0, S), "levels")
+    err(L.dq_thc_rht_quantize(P, P, 0, N, P, 64, 64, F1, P, P, 31, 0, S), "null pointer")
+    err(L.dq_thc_dequantize_irht(P, P, 0, N, 64, 64, F1, P, P, 0, S), "null pointer")
+    err(L.dq_thc_dequantize_irht(P, P, 1, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
     assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 and capi.eden_work_doubles(8192) == 2 and capi.bitrate_hist_ints() == 32768
     # a good call clears the message
