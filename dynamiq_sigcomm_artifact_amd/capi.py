@@ -26,7 +26,7 @@ EXPORTS = [
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
-    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
+    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
     "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
 ]
@@ -114,6 +114,8 @@ def lib():
         L.dq_pack_signs.argtypes = [vp, vp, i64, i32, vp]
         L.dq_rand_diag.restype = i32
         L.dq_rand_diag.argtypes = [vp, i64, i64, i32, vp]
+        L.dq_rand_diag_bits.restype = i32
+        L.dq_rand_diag_bits.argtypes = [vp, i64, i64, i32, vp]
         L.dq_bins_to_bits.restype = i32
         L.dq_bins_to_bits.argtypes = [vp, i64, vp, i64, i32, i32, vp]
         L.dq_bits_to_bins.restype = i32
@@ -408,6 +410,13 @@ def scaling_decompress_irht(src, sign, dst, block, scale, nbits, strategy, strea
 
 def rand_diag(out, seed, stream=None):
     _check(lib().dq_rand_diag(out.data_ptr(), out.numel(), seed, _dev(out), _stream(stream)))
+
+
+def rand_diag_bits(bits, size, seed, stream=None):
+    """the diagonal of rand_diag(size, seed) as the int32 bit vector of pack_signs; size a multiple of 256"""
+    if bits.dtype != torch.int32 or bits.numel() < size // 32:
+        raise RuntimeError("rand_diag_bits: bits must be int32 [size / 32]")
+    _check(lib().dq_rand_diag_bits(bits.data_ptr(), size, seed, _dev(bits), _stream(stream)))
 
 
 def bins_to_bits(bins, arr, nbits, stream=None):

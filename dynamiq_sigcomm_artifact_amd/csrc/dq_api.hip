@@ -601,6 +601,15 @@ int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t
     return finish(dq::launch_rand_diag(out, size, seed, static_cast<hipStream_t>(stream)));
 }
 
+int dq_rand_diag_bits(uint32_t *bits, int64_t size, int64_t seed, int device, dq_stream_t stream)
+{
+    if (!(size > 0) || size % 256 != 0) return fail(DQ_ERR_SIZE, "size must be a positive multiple of 256");
+    if (!bits) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_rand_diag_bits(bits, size, seed, static_cast<hipStream_t>(stream)));
+}
+
 int dq_bins_to_bits(const int32_t *bins, int64_t nbins, uint32_t *arr, int64_t narr, int nbits, int device,
                     dq_stream_t stream)
 {

@@ -287,10 +287,9 @@ hipError_t launch_thc_dequantize_irht(const void *levels_in, const void *sign, b
 
 // ---- randDiag -----------------------------------------------------------------------
 
-__global__ __launch_bounds__(256) void rand_diag_kernel(float *__restrict__ out, int64_t size, int64_t s8, uint64_t ss)
+// the 32 random bits of column j: nibble k decides element k * s8 + j (+1 where the nibble is >= 8)
+__device__ __forceinline__ uint64_t rand_diag_word(int64_t j, uint64_t ss)
 {
-    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (j >= s8) return;
     const uint64_t M = 0xffffffffull;
     uint64_t r = (uint64_t)j + ss;
     r = (1103515245ull * r + 12345ull + ss) & M;
@@ -298,11 +297,33 @@ __global__ __launch_bounds__(256) void rand_diag_kernel(float *__restrict__ out,
     r += 0x9e3779b9ull; // the carry into bit 32 is kept
     r = ((r ^ (r >> 16)) * 0x85ebca6bull) & M;
     r = ((r ^ (r >> 13)) * 0xc2b2ae35ull) & M;
-    r = (r ^ (r >> 16)) & M;
+    return (r ^ (r >> 16)) & M;
+}
+
+__global__ __launch_bounds__(256) void rand_diag_kernel(float *__restrict__ out, int64_t size, int64_t s8, uint64_t ss)
+{
+    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (j >= s8) return;
+    const uint64_t r = rand_diag_word(j, ss);
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const int64_t idx = (int64_t)k * s8 + j;
         if (idx < size) out[idx] = ((r >> (4 * k)) & 15u) >= 8u ? 1.0f : -1.0f;
+    }
+}
+
+// The same diagonal as the bit vector of pack_signs (bit set where the value is -1), for size = 8 s8 with s8 a
+// multiple of 32: a wave holds 64 consecutive columns, and its ballot for nibble k is two whole words of segment k.
+__global__ __launch_bounds__(256) void rand_diag_bits_kernel(uint32_t *__restrict__ bits, int64_t s8, uint64_t ss)
+{
+    const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const uint64_t r = j < s8 ? rand_diag_word(j, ss) : ~0ull; // columns past the end: +1, bit clear
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const uint64_t m = __builtin_amdgcn_ballot_w64(((r >> (4 * k)) & 15u) < 8u);
+        // lanes 0 and 32 store the halves; a half that starts at or past s8 belongs to nobody
+        if ((lane & 31) == 0 && j < s8) bits[((int64_t)k * s8 + j) >> 5] = (uint32_t)(m >> lane);
     }
 }
 
@@ -322,13 +343,27 @@ hipError_t launch_pack_signs(const float *sign, uint32_t *bits, int64_t n, hipSt
     return hipGetLastError();
 }
 
-hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream)
+static uint64_t rand_diag_seed(int64_t seed)
 {
     const uint64_t M = 0xffffffffull;
     uint64_t ss = ((uint64_t)seed * 1664525ull + 1013904223ull) & M;
-    ss = (ss * 8121ull + 28411ull) & M;
+    return (ss * 8121ull + 28411ull) & M;
+}
+
+hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream)
+{
     const int64_t s8 = size / 8 + (size % 8 != 0);
-    hipLaunchKernelGGL(rand_diag_kernel, dim3((unsigned)((s8 + 255) / 256)), dim3(256), 0, stream, out, size, s8, ss);
+    hipLaunchKernelGGL(rand_diag_kernel, dim3((unsigned)((s8 + 255) / 256)), dim3(256), 0, stream, out, size, s8,
+                       rand_diag_seed(seed));
+    return hipGetLastError();
+}
+
+// size: a multiple of 256
+hipError_t launch_rand_diag_bits(uint32_t *bits, int64_t size, int64_t seed, hipStream_t stream)
+{
+    const int64_t s8 = size / 8;
+    hipLaunchKernelGGL(rand_diag_bits_kernel, dim3((unsigned)((s8 + 255) / 256)), dim3(256), 0, stream, bits, s8,
+                       rand_diag_seed(seed));
     return hipGetLastError();
 }
 

@@ -94,6 +94,8 @@ hipError_t launch_hadamard(float *vec, int64_t n, hipStream_t stream);
 hipError_t launch_rht_blocked(float *vec, const void *sign, bool sign_packed, int64_t n, int64_t block, float scale,
                               int inverse, hipStream_t stream);
 hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream);
+// the same diagonal as packed bits (set where the value is -1); size a multiple of 256
+hipError_t launch_rand_diag_bits(uint32_t *bits, int64_t size, int64_t seed, hipStream_t stream);
 // THC's quantiser folded into the last pass of the forward transform / the first pass of the inverse one
 hipError_t launch_thc_rht_quantize(float *vec, const void *sign, bool sign_packed, const float *uniform, void *levels_out,
                                    int64_t n, int64_t block, float scale, const float *lo, const float *delta, int levels,

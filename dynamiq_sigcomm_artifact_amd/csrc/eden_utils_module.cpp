@@ -144,6 +144,17 @@ static const void *sign_arg(const c10::optional<torch::Tensor> &sign, const torc
     return sign->data_ptr();
 }
 
+torch::Tensor rand_diag_bits(int64_t size, int64_t seed, torch::Device device, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(device.type() == torch::kCUDA, "device must be a CUDA device");
+    TORCH_CHECK(size > 0 && size % 256 == 0, "size must be a positive multiple of 256");
+    auto bits = torch::empty({size / 32}, torch::TensorOptions().dtype(torch::kInt32).device(device));
+    check_status(dq_rand_diag_bits(reinterpret_cast<uint32_t *>(bits.data_ptr<int32_t>()), size, seed, bits.device().index(),
+                                   as_stream(stream_p)),
+                 "rand_diag_bits");
+    return bits;
+}
+
 torch::Tensor pack_signs(torch::Tensor sign, uint64_t stream_p = 0)
 {
     TORCH_CHECK(sign.device().type() == torch::kCUDA && sign.dtype() == torch::kFloat32 && sign.is_contiguous(),
@@ -929,6 +940,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("rht_scaling_compress", &rht_scaling_compress, "blocked randomized Hadamard transform + hierarchical chunk-16 compress in one launch (the rotated vector never reaches memory)", py::arg("src"), py::arg("sign"), py::arg("dst"), py::arg("block"), py::arg("scale"), py::arg("nbits"), py::arg("rand_pool") = py::none(), py::arg("seed") = 0, py::arg("step") = 0, py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("scaling_decompress_irht", &scaling_decompress_irht, "hierarchical chunk-16 decompress + inverse blocked randomized Hadamard transform in one launch", py::arg("src"), py::arg("sign"), py::arg("dst"), py::arg("block"), py::arg("scale"), py::arg("nbits"), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("rand_diag", &rand_diag, "EDEN's seeded +-1 diagonal", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
+    modul.def("rand_diag_bits", &rand_diag_bits, "EDEN's seeded +-1 diagonal as the int32 bit vector of pack_signs (bit set where the value is -1)", py::arg("size"), py::arg("seed"), py::arg("device"), py::arg("stream_p") = 0);
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
     modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width into the three regions of order (8-bit rows from 0, 4-bit from nsc, 2-bit from 2 nsc); returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
     modul.def("group_plan_stats", &group_plan_stats, "bit widths from the reduced bf16 norms and the offset u, and the partition by width, in one call; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);

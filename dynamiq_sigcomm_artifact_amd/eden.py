@@ -98,6 +98,20 @@ class Eden(object):
         # with the float32 reciprocal
         return float(np.float32(1.0) / np.float32(math.sqrt(n)))
 
+    # the diagonal of randDiag (srrcomp.py:61-106): one bit per element where the size allows it (multiples of 256),
+    # the float vector otherwise -- the transform takes either
+    def _diag_buffer(self, n):
+        if n % 256 == 0:
+            return torch.empty(n // 32, dtype=torch.int32, device=self.device)
+        return torch.empty(n, dtype=torch.float32, device=self.device)
+
+    @staticmethod
+    def _rand_diag(diag, n, seed):
+        if diag.dtype == torch.int32:
+            capi.rand_diag_bits(diag, n, seed)
+        else:
+            capi.rand_diag(diag, seed)
+
     # ---- srrcomp.py:293-326 ----
     def _compress_slice(self, vec, vec_type, nbits, num_hadamard, seed):
         orig_dim = n = vec.numel()
@@ -108,9 +122,9 @@ class Eden(object):
             n, vec = padded_dim, padded
         else:
             vec = vec.contiguous().clone()
-        diag = torch.empty(n, device=self.device)
+        diag = self._diag_buffer(n)
         for i in range(num_hadamard):
-            capi.rand_diag(diag, seed + i)
+            self._rand_diag(diag, n, seed + i)
             capi.rht_blocked(vec, diag, n, self._inv_sqrt(n), False)
         centroids, boundaries = self._tables(nbits)
         packed = torch.empty(n // 32 * nbits, dtype=torch.int32, device=self.device)
@@ -130,8 +144,8 @@ class Eden(object):
         centroids, _ = self._tables(nbits)
         vec = torch.empty(n, dtype=torch.float32, device=self.device)
         capi.eden_dequantize(packed_bins.to(torch.int32), n, centroids, nbits, vec)
-        diag = torch.empty(n, device=self.device)
+        diag = self._diag_buffer(n)
         for i in range(num_hadamard):
-            capi.rand_diag(diag, seed + num_hadamard - 1 - i)
+            self._rand_diag(diag, n, seed + num_hadamard - 1 - i)
             capi.rht_blocked(vec, diag, n, self._inv_sqrt(n), True)
         return (scale * vec)[:orig_dim].to(vec_type)

@@ -683,6 +683,8 @@ def kernels(dev, n=6553600):
     y = torch.randn(d, generator=g, device=dev)
     sign = torch.empty(d, device=dev)
     line("rand_diag", lambda: capi.rand_diag(sign, 0), 4 * d, n=d)
+    dbits = torch.empty(d // 32, dtype=torch.int32, device=dev)
+    line("rand_diag_bits", lambda: capi.rand_diag_bits(dbits, d, 0), d // 8, n=d)
     line("Hadamard (whole vector)", lambda: capi.hadamard(y), 16 * d, n=d, passes=2)
     y.normal_(generator=g)
     line("rht_blocked (whole vector, sign + scale)", lambda: capi.rht_blocked(y, sign, d, 1.0, False), 20 * d, n=d, passes=2)

@@ -400,6 +400,10 @@ int dq_pack_signs(const float *sign, uint32_t *bits, int64_t n, int device, dq_s
 /* srrcomp.py:61-106 (SRRCompUtils.randDiag, torchRNG=False) computed on the
  * device: out[size] of +-1.0f. */
 int dq_rand_diag(float *out, int64_t size, int64_t seed, int device, dq_stream_t stream);
+/* the same diagonal written as the bit vector dq_pack_signs would make of it
+ * (uint32 [size / 32], bit set where the value is -1), without the float vector:
+ * size a positive multiple of 256. */
+int dq_rand_diag_bits(uint32_t *bits, int64_t size, int64_t seed, int device, dq_stream_t stream);
 
 /* ---- EDEN bit-plane packing ------------------------------------------ */
 

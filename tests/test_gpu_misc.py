@@ -167,6 +167,20 @@ def test_rand_diag(capi, oracle, size, seed):
     _eq("rand_diag", out.cpu().numpy(), oracle.rand_diag(size, seed))
 
 
+@pytest.mark.parametrize("size", [256, 768, 1024, 256 * 33, 1 << 20, 256 * 4097])
+@pytest.mark.parametrize("seed", [0, 7, 2 ** 31])
+def test_rand_diag_bits(capi, oracle, size, seed):
+    """the diagonal generated as packed bits == the float diagonal of the oracle, packed"""
+    bits = torch.full((size // 32 + 2,), 0x55555555, dtype=torch.int32, device=DEV)
+    capi.rand_diag_bits(bits[:size // 32], size, seed)
+    want = np.packbits(oracle.rand_diag(size, seed) < 0, bitorder="little").view(np.uint32)
+    got = bits.cpu().numpy().view(np.uint32)
+    assert (got[:size // 32] == want).all() and (got[size // 32:] == 0x55555555).all()
+    sign = torch.empty(size, device=DEV)
+    capi.rand_diag(sign, seed)
+    assert torch.equal(capi.pack_signs(sign), bits[:size // 32])
+
+
 @pytest.mark.parametrize("nbits", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("nbins", [32, 64, 96, 1024, 1056, 100000 * 32])
 def test_bit_plane_packing(capi, oracle, eden_utils, nbits, nbins):
