@@ -702,6 +702,20 @@ def kernels(dev, n=6553600):
         out = torch.empty(d, device=dev)
         line("eden_quantize", lambda: capi.eden_quantize(y, bnd, cen, nbits, packed, result, work64), 8 * d + d // 8 * nbits, n=d, nbits=nbits)
         line("eden_dequantize", lambda: capi.eden_dequantize(packed, d, cen, nbits, out), 4 * d + d // 8 * nbits, n=d, nbits=nbits)
+    # EDEN end to end on the padded bucket (srrcomp.py:293-354): fresh diagonal, rotation, quantiser -- with the float
+    # diagonal and with the diagonal as bits
+    cen, bnd = (t.to(dev) for t in normal_centroids_and_boundaries(4))
+    packed = torch.empty(d // 32 * 4, dtype=torch.int32, device=dev)
+    inv_d = 1.0 / math.sqrt(d)
+    line("eden compress: rand_diag + rht_blocked + eden_quantize", lambda: (
+        capi.rand_diag(sign, 1), capi.rht_blocked(y, sign, d, inv_d, False),
+        capi.eden_quantize(y, bnd, cen, 4, packed, result, work64)), 4 * d + 20 * d + 8.5 * d, n=d, nbits=4, launches=7)
+    line("eden compress: rand_diag_bits + rht_blocked + eden_quantize", lambda: (
+        capi.rand_diag_bits(dbits, d, 1), capi.rht_blocked(y, dbits, d, inv_d, False),
+        capi.eden_quantize(y, bnd, cen, 4, packed, result, work64)), 0.125 * d + 16.125 * d + 8.5 * d, n=d, nbits=4, launches=7)
+    line("eden decompress: eden_dequantize + rand_diag_bits + inverse rht_blocked", lambda: (
+        capi.eden_dequantize(packed, d, cen, 4, out), capi.rand_diag_bits(dbits, d, 1),
+        capi.rht_blocked(out, dbits, d, inv_d, True)), 4.5 * d + 0.125 * d + 16.125 * d, n=d, nbits=4, launches=4)
     uni = torch.rand(d, generator=g, device=dev)
     lev = torch.empty(d, dtype=torch.bfloat16, device=dev)
     lo, delta = torch.tensor([-4.0], device=dev), torch.tensor([8.0 / 63], device=dev)
