@@ -138,3 +138,12 @@ def test_transform_bindings(capi, eden_utils):
     eu.thc_dequantize_irht(la, sign, rb, n, 1.0 / math.sqrt(n), delta, lo)
     assert torch.equal(ra, rb)
     assert float((ra - x).pow(2).sum() / x.pow(2).sum()) < 0.05
+    # the diagonal as bits through the module: same levels, same vector back, same rotation; the seeded diagonal as bits
+    eu.thc_rht_quantize(x.clone(), bits_a, uni, lb.zero_(), n, 1.0 / math.sqrt(n), lo, delta, 31)
+    assert torch.equal(bits_t(la), bits_t(lb))
+    eu.thc_dequantize_irht(la, bits_a, rb.zero_(), n, 1.0 / math.sqrt(n), delta, lo)
+    assert torch.equal(ra, rb)
+    assert torch.equal(eu.rht_blocked(x.clone(), bits_a, block, scale, False), eu.rht_blocked(x.clone(), sign, block, scale, False))
+    assert torch.equal(eu.rand_diag_bits(n, 5, x.device), capi.pack_signs(eu.rand_diag(n, 5, x.device)))
+    with pytest.raises(RuntimeError, match="multiple of 256"):
+        eu.rand_diag_bits(100, 5, x.device)
