@@ -667,6 +667,11 @@ def kernels(dev, n=6553600):
     line("mixed_compress (centred load)",
          lambda: capi.mixed_compress(src, order, counts, mixed, nsc, 2, seed=1, step=0, center_mean=mean32, center_world=8, n=n),
          2 * n + 4 * nsc + 4 * nsc + stream_bytes, elements="bf16", groups=[n8, n4, n2])
+    mixed2 = torch.zeros_like(mixed)
+    line("mixed_compress (fused ring step: decode recv, add, centre, encode)",
+         lambda: capi.mixed_compress(src, order, counts, mixed2, nsc, 2, seed=1, step=1, recv=mixed, center_mean=mean32,
+                                     center_world=8, n=n),
+         2 * n + 4 * nsc + 4 * nsc + 2 * stream_bytes, elements="bf16", groups=[n8, n4, n2])
     line("mixed_decompress (+mean)", lambda: capi.mixed_decompress(mixed, out, order, counts, nsc, 2, stats=stats),
          2 * n + 4 * nsc + 4 * nsc + stream_bytes, elements="bf16", groups=[n8, n4, n2])
     rows = torch.arange(0, nsc, 2, dtype=torch.int32, device=dev)
