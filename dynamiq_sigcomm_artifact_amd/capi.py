@@ -28,7 +28,7 @@ EXPORTS = [
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
-    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
+    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_eden_dequantize_irht", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
 ]
 
 _lib = None
@@ -130,6 +130,8 @@ def lib():
         L.dq_thc_quantize.argtypes = [vp, vp, vp, i64, vp, vp, i32, i32, vp]
         L.dq_thc_dequantize.restype = i32
         L.dq_thc_dequantize.argtypes = [vp, vp, i64, vp, vp, i32, vp]
+        L.dq_eden_dequantize_irht.restype = i32
+        L.dq_eden_dequantize_irht.argtypes = [vp, i64, vp, i32, vp, i32, vp, i64, f32, vp, i32, vp]
         L.dq_thc_rht_quantize.restype = i32
         L.dq_thc_rht_quantize.argtypes = [vp, vp, i32, vp, vp, i64, i64, f32, vp, vp, i32, i32, vp]
         L.dq_thc_dequantize_irht.restype = i32
@@ -480,6 +482,20 @@ def thc_dequantize(levels_in, out, step, lo, stream=None):
         raise RuntimeError("thc_dequantize: out is too small")
     _check(lib().dq_thc_dequantize(levels_in.data_ptr(), out.data_ptr(), n, step.data_ptr(), lo.data_ptr(), _dev(out),
                                    _stream(stream)))
+
+
+def eden_dequantize_irht(packed, n, centroids, nbits, sign, out, block, scale, post_scale=None, stream=None):
+    """eden_dequantize + rht_blocked (inverse) in the transform's own passes; post_scale: a float32 device scalar that
+    multiplies the result (EDEN's scale), or None"""
+    if packed.dtype != torch.int32 or centroids.dtype != torch.float32 or out.dtype != torch.float32:
+        raise RuntimeError("eden_dequantize_irht: packed must be int32, centroids and out float32")
+    if packed.numel() < n // 32 * nbits or centroids.numel() < (1 << nbits) or out.numel() < n:
+        raise RuntimeError("eden_dequantize_irht: a buffer is too small")
+    if post_scale is not None and (post_scale.dtype != torch.float32 or post_scale.device != out.device):
+        raise RuntimeError("eden_dequantize_irht: post_scale must be a float32 tensor on the device of out")
+    _check_sign(sign, n, "eden_dequantize_irht")
+    _check(lib().dq_eden_dequantize_irht(packed.data_ptr(), n, centroids.data_ptr(), nbits, _ptr(sign), _packed(sign),
+                                         out.data_ptr(), block, float(scale), _ptr(post_scale), _dev(out), _stream(stream)))
 
 
 def thc_rht_quantize(work, sign, uniform, levels_out, block, scale, lo, delta, levels, stream=None):

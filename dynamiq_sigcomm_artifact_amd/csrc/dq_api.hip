@@ -704,6 +704,21 @@ int dq_thc_dequantize_irht(const void *levels_bf16, const void *sign, int sign_p
                                                  static_cast<hipStream_t>(stream)));
 }
 
+int dq_eden_dequantize_irht(const uint32_t *packed, int64_t n, const float *centroids, int nbits, const void *sign,
+                            int sign_packed, float *out, int64_t block, float scale, const float *post_scale, int device,
+                            dq_stream_t stream)
+{
+    if (nbits < 1 || nbits > 8) return fail(DQ_ERR_NBITS, "nbits must be in [1, 8]");
+    if (!(n > 0) || (n & 31) != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of 32");
+    if (!(block >= 16) || (block & (block - 1)) != 0) return fail(DQ_ERR_POW2, "block (at least 16)");
+    if (n % block != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of block");
+    if (!packed || !centroids || !out) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_eden_dequantize_irht(packed, centroids, nbits, sign, sign_packed != 0, out, n, block, scale,
+                                                  post_scale, static_cast<hipStream_t>(stream)));
+}
+
 int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const float *step, const float *lo, int device,
                       dq_stream_t stream)
 {

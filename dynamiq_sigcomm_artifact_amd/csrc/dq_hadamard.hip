@@ -42,6 +42,12 @@ struct FwhtArgs {
     uint16_t *out_levels;      // the pass stores thc_level(value, uniform) as bf16 instead of the value
     const float *uniform, *out_lo, *out_delta;
     float out_top;
+    // EDEN's dequantiser folded into the ends of an inverse transform (null / unused otherwise):
+    const uint32_t *in_planes; // the pass loads centroids[bin] from the bit planes of the bins instead of x
+    const float *in_centroids; // 2^in_nbits values
+    int64_t in_words;          // words per plane (n / 32)
+    int in_nbits;
+    const float *post_scale;   // the last pass multiplies by *post_scale after scale and sign
 };
 
 // the diagonal of +-1 on four consecutive elements from g (a multiple of 4) / on element g: a multiplication by
@@ -88,7 +94,33 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
     }
 
     // load (coalesced), optional sign flip
-    if (a.vec) {
+    if (a.in_planes) {
+        // sixteen consecutive bins per thread from its half word of every plane (two 8 x 8 bit transposes), their
+        // centroids into one padded group of the tile; the centroid table sits behind the tile
+        float *cen = lds + tile + tile / 16 + 1;
+        for (int k = tid; k < (1 << a.in_nbits); k += nthreads) cen[k] = a.in_centroids[k];
+        __syncthreads();
+        for (int i = tid * 16; i < tile; i += nthreads * 16) {
+            const int64_t g = origin + i; // the first pass works on contiguous tiles
+            uint64_t lo8 = 0, hi8 = 0;
+            if (g < a.n) {
+                const uint16_t *half = reinterpret_cast<const uint16_t *>(a.in_planes) + (g >> 4);
+                for (int p = 0; p < a.in_nbits; p++) {
+                    const uint32_t h = half[(int64_t)p * a.in_words * 2];
+                    lo8 |= (uint64_t)(h & 0xffu) << (8 * p);
+                    hi8 |= (uint64_t)(h >> 8) << (8 * p);
+                }
+                lo8 = transpose8x8(lo8);
+                hi8 = transpose8x8(hi8);
+            }
+            const int q = pad_idx(i);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                lds[q + k] = g < a.n ? cen[(lo8 >> (8 * k)) & 0xffu] : 0.0f;
+                lds[q + 8 + k] = g < a.n ? cen[(hi8 >> (8 * k)) & 0xffu] : 0.0f;
+            }
+        }
+    } else if (a.vec) {
         for (int i = tid * 4; i < tile; i += nthreads * 4) {
             const int64_t g = origin + ((int64_t)(i >> a.cbits) << a.sbits) + (i & cmask);
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -137,6 +169,10 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
             if (a.apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
             if (a.sign_mode == 2) apply_sign4(a, v, g);
+            if (a.post_scale) {
+                const float ps = *a.post_scale;
+                v.x *= ps; v.y *= ps; v.z *= ps; v.w *= ps;
+            }
             if (a.out_levels) {
                 const float4 u = *reinterpret_cast<const float4 *>(a.uniform + g);
                 const float lo = *a.out_lo, delta = *a.out_delta;
@@ -155,6 +191,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
             float v = lds[pad_idx(i)];
             if (a.apply_scale) v *= a.scale;
             if (a.sign_mode == 2) v = apply_sign1(a, v, g);
+            if (a.post_scale) v *= *a.post_scale;
             if (a.out_levels)
                 a.out_levels[g] = (uint16_t)f32_to_bf16_bits(thc_level(v, a.uniform[g], *a.out_lo, *a.out_delta, a.out_top));
             else
@@ -168,7 +205,7 @@ static hipError_t launch_tile(const FwhtArgs &a, int64_t ntiles, hipStream_t str
     const int tile = 1 << a.kt;
     int threads = tile / 16;
     threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
-    const size_t lds_bytes = (size_t)(tile + tile / 16 + 1) * sizeof(float);
+    const size_t lds_bytes = (size_t)(tile + tile / 16 + 1 + (a.in_planes ? 256 : 0)) * sizeof(float);
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(fwht_tile_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -190,6 +227,11 @@ struct ThcEnds {
     uint16_t *out_levels = nullptr;
     const float *uniform = nullptr, *out_lo = nullptr, *out_delta = nullptr;
     float out_top = 0.0f;
+    // EDEN: `in_planes` replaces the load of the first pass, `post_scale` multiplies the store of the last
+    const uint32_t *in_planes = nullptr;
+    const float *in_centroids = nullptr;
+    int in_nbits = 0;
+    const float *post_scale = nullptr;
 };
 
 // sign: float +-1 values, or (sign_packed) the bit vector of dq_pack_signs; may be null
@@ -206,6 +248,8 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.sign = sign_packed ? nullptr : static_cast<const float *>(sign);
     a.sign_bits = sign_packed ? static_cast<const uint32_t *>(sign) : nullptr;
     a.in_levels = nullptr; a.in_step = thc.in_step; a.in_lo = thc.in_lo;
+    a.in_planes = nullptr; a.in_centroids = thc.in_centroids; a.in_words = n >> 5; a.in_nbits = thc.in_nbits;
+    a.post_scale = nullptr;
     a.out_levels = nullptr; a.uniform = thc.uniform; a.out_lo = thc.out_lo; a.out_delta = thc.out_delta;
     a.out_top = thc.out_top;
     const int sign_fwd = (sign && !inverse) ? 1 : 0, sign_inv = (sign && inverse) ? 2 : 0;
@@ -220,6 +264,8 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
         a.vec = vec16 && kt >= 2 && (n & 3) == 0;
         a.in_levels = thc.in_levels;
         a.out_levels = thc.out_levels;
+        a.in_planes = thc.in_planes;
+        a.post_scale = thc.post_scale;
         const int64_t ntiles = (n + ((int64_t)1 << kt) - 1) >> kt;
         return launch_tile(a, ntiles, stream);
     }
@@ -229,9 +275,11 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.kt = kt; a.b0 = 0; a.b1 = kt; a.cbits = kt; a.sbits = kt;
     a.apply_scale = 0; a.sign_mode = sign_fwd; a.vec = vec16;
     a.in_levels = thc.in_levels;
+    a.in_planes = thc.in_planes;
     hipError_t e = launch_tile(a, n >> kt, stream);
     if (e != hipSuccess) return e;
     a.in_levels = nullptr;
+    a.in_planes = nullptr;
     int s = kt;
     const int max_rows = kMaxTileBits - kStridedCols;
     while (s < kb) {
@@ -245,6 +293,7 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
         a.apply_scale = last ? apply_scale : 0;
         a.sign_mode = last ? sign_inv : 0;
         a.out_levels = last ? thc.out_levels : nullptr;
+        a.post_scale = last ? thc.post_scale : nullptr;
         a.vec = vec16;
         e = launch_tile(a, n >> a.kt, stream);
         if (e != hipSuccess) return e;
@@ -283,6 +332,20 @@ hipError_t launch_thc_dequantize_irht(const void *levels_in, const void *sign, b
     thc.in_levels = static_cast<const uint16_t *>(levels_in);
     thc.in_step = step; thc.in_lo = lo;
     return fwht_blocks(out, sign, sign_packed, n, ilog2(block), scale, 1, 1, stream, thc);
+}
+
+// EDEN: centroids of the packed bins, rotated back (inverse transform over the whole vector or per block) and,
+// with post_scale, multiplied by EDEN's scale -- the dequantised vector never reaches memory
+hipError_t launch_eden_dequantize_irht(const uint32_t *packed, const float *centroids, int nbits, const void *sign,
+                                       bool sign_packed, float *out, int64_t n, int64_t block, float scale,
+                                       const float *post_scale, hipStream_t stream)
+{
+    ThcEnds ends;
+    ends.in_planes = packed;
+    ends.in_centroids = centroids;
+    ends.in_nbits = nbits;
+    ends.post_scale = post_scale;
+    return fwht_blocks(out, sign, sign_packed, n, ilog2(block), scale, 1, 1, stream, ends);
 }
 
 // ---- randDiag -----------------------------------------------------------------------

@@ -93,6 +93,11 @@ hipError_t launch_hadamard(float *vec, int64_t n, hipStream_t stream);
 // sign: float +-1 values, or (sign_packed) the bit vector of launch_pack_signs; may be null
 hipError_t launch_rht_blocked(float *vec, const void *sign, bool sign_packed, int64_t n, int64_t block, float scale,
                               int inverse, hipStream_t stream);
+// EDEN's dequantiser folded into the first pass of the inverse transform, EDEN's scale (device scalar, may be null)
+// into the last
+hipError_t launch_eden_dequantize_irht(const uint32_t *packed, const float *centroids, int nbits, const void *sign,
+                                       bool sign_packed, float *out, int64_t n, int64_t block, float scale,
+                                       const float *post_scale, hipStream_t stream);
 hipError_t launch_rand_diag(float *out, int64_t size, int64_t seed, hipStream_t stream);
 // the same diagonal as packed bits (set where the value is -1); size a multiple of 256
 hipError_t launch_rand_diag_bits(uint32_t *bits, int64_t size, int64_t seed, hipStream_t stream);

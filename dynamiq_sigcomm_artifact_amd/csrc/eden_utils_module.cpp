@@ -835,6 +835,32 @@ torch::Tensor eden_dequantize(torch::Tensor packed, torch::Tensor centroids, int
     return out;
 }
 
+torch::Tensor eden_dequantize_irht(torch::Tensor packed, torch::Tensor centroids, int nbits, c10::optional<torch::Tensor> sign,
+                                   int64_t block, double scale, c10::optional<torch::Tensor> post_scale, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(packed.device().type() == torch::kCUDA && packed.dtype() == torch::kInt32 && packed.is_contiguous(),
+                "packed must be a contiguous torch.int32 CUDA tensor");
+    check_f32_cuda(centroids, "centroids");
+    TORCH_CHECK(nbits >= 1 && nbits <= 8, "nbits must be in [1, 8]");
+    TORCH_CHECK(packed.numel() > 0 && packed.numel() % nbits == 0, "packed size must be a multiple of nbits");
+    TORCH_CHECK(centroids.numel() == (1 << nbits), "centroids must hold 2^nbits values");
+    const int64_t n = packed.numel() / nbits * 32;
+    auto out = torch::empty({n}, centroids.options());
+    int sign_packed = 0;
+    const void *sp = sign_arg(sign, out, n, &sign_packed);
+    const float *ps = nullptr;
+    if (post_scale.has_value()) {
+        check_f32_cuda(*post_scale, "post_scale");
+        TORCH_CHECK(post_scale->numel() == 1, "post_scale must hold one value");
+        ps = post_scale->data_ptr<float>();
+    }
+    check_status(dq_eden_dequantize_irht(reinterpret_cast<const uint32_t *>(packed.data_ptr<int32_t>()), n, centroids.data_ptr<float>(),
+                                         nbits, sp, sign_packed, out.data_ptr<float>(), block, (float)scale, ps,
+                                         packed.device().index(), as_stream(stream_p)),
+                 "eden_dequantize_irht");
+    return out;
+}
+
 torch::Tensor thc_quantize(torch::Tensor rotated, torch::Tensor uniform, torch::Tensor lo, torch::Tensor delta, int levels,
                            uint64_t stream_p = 0)
 {
@@ -960,6 +986,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("philox_uniform", &philox_uniform, "the uniform values of that stream written out as a tensor", py::arg("out"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0);
     modul.def("eden_quantize", &eden_quantize, "EDEN: normalise, bucketize against the Lloyd-Max boundaries, pack bit planes, scale; returns [packed, result]", py::arg("vec"), py::arg("boundaries"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
     modul.def("eden_dequantize", &eden_dequantize, "EDEN: centroids of the packed bins", py::arg("packed"), py::arg("centroids"), py::arg("nbits"), py::arg("stream_p") = 0);
+    modul.def("eden_dequantize_irht", &eden_dequantize_irht, "EDEN: centroids of the packed bins rotated back (inverse blocked transform) and multiplied by post_scale, without the dequantised vector reaching memory", py::arg("packed"), py::arg("centroids"), py::arg("nbits"), py::arg("sign"), py::arg("block"), py::arg("scale"), py::arg("post_scale") = py::none(), py::arg("stream_p") = 0);
     modul.def("thc_quantize", &thc_quantize, "THC: uniform stochastic quantiser of the rotated vector, bfloat16 levels", py::arg("rotated"), py::arg("uniform"), py::arg("lo"), py::arg("delta"), py::arg("levels"), py::arg("stream_p") = 0);
     modul.def("thc_dequantize", &thc_dequantize, "THC: out = float(levels) * step + lo", py::arg("levels"), py::arg("out"), py::arg("step"), py::arg("lo"), py::arg("stream_p") = 0);
     modul.def("thc_rht_quantize", &thc_rht_quantize, "THC: blocked randomized Hadamard transform whose last pass stores the quantiser's levels (work is scratch afterwards)", py::arg("work"), py::arg("sign"), py::arg("uniform"), py::arg("levels_out"), py::arg("block"), py::arg("scale"), py::arg("lo"), py::arg("delta"), py::arg("levels"), py::arg("stream_p") = 0);

@@ -143,9 +143,23 @@ class Eden(object):
         n = packed_bins.numel() // nbits * 32
         centroids, _ = self._tables(nbits)
         vec = torch.empty(n, dtype=torch.float32, device=self.device)
-        capi.eden_dequantize(packed_bins.to(torch.int32), n, centroids, nbits, vec)
+        if num_hadamard == 0:
+            capi.eden_dequantize(packed_bins.to(torch.int32), n, centroids, nbits, vec)
+            return (scale * vec)[:orig_dim].to(vec_type)
+        # the dequantiser rides on the first pass of the first rotation, the product with the scale on the last pass of
+        # the last one: same bits as eden_dequantize, the rotations and `scale * vec`
+        scale32 = scale.reshape(1).to(device=self.device, dtype=torch.float32) if isinstance(scale, torch.Tensor) else \
+            torch.tensor([scale], dtype=torch.float32, device=self.device)
         diag = self._diag_buffer(n)
         for i in range(num_hadamard):
             self._rand_diag(diag, n, seed + num_hadamard - 1 - i)
-            capi.rht_blocked(vec, diag, n, self._inv_sqrt(n), True)
-        return (scale * vec)[:orig_dim].to(vec_type)
+            last = scale32 if i == num_hadamard - 1 else None
+            if i == 0:
+                capi.eden_dequantize_irht(packed_bins.to(torch.int32), n, centroids, nbits, diag, vec, n, self._inv_sqrt(n),
+                                          post_scale=last)
+            elif last is None:
+                capi.rht_blocked(vec, diag, n, self._inv_sqrt(n), True)
+            else:
+                capi.rht_blocked(vec, diag, n, self._inv_sqrt(n), True)
+                vec = scale32 * vec
+        return vec[:orig_dim].to(vec_type)

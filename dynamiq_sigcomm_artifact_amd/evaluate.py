@@ -721,6 +721,10 @@ def kernels(dev, n=6553600):
     line("eden decompress: eden_dequantize + rand_diag_bits + inverse rht_blocked", lambda: (
         capi.eden_dequantize(packed, d, cen, 4, out), capi.rand_diag_bits(dbits, d, 1),
         capi.rht_blocked(out, dbits, d, inv_d, True)), 4.5 * d + 0.125 * d + 16.125 * d, n=d, nbits=4, launches=4)
+    line("eden decompress: rand_diag_bits + eden_dequantize_irht (folded, scale included)", lambda: (
+        capi.rand_diag_bits(dbits, d, 1),
+        capi.eden_dequantize_irht(packed, d, cen, 4, dbits, out, d, inv_d, post_scale=result[2:3])),
+        0.125 * d + 0.5 * d + 0.125 * d + 12 * d, n=d, nbits=4, launches=3)
     uni = torch.rand(d, generator=g, device=dev)
     lev = torch.empty(d, dtype=torch.bfloat16, device=dev)
     lo, delta = torch.tensor([-4.0], device=dev), torch.tensor([8.0 / 63], device=dev)

@@ -329,6 +329,18 @@ int dq_thc_quantize(const float *rotated, const float *uniform, void *levels_bf1
                     const float *lo, const float *delta, int levels, int device,
                     dq_stream_t stream);
 
+/* srrcomp.py:343-354 in one call per rotation: dq_eden_dequantize folded into
+ * the first pass of the inverse transform of dq_rht_blocked (sign, sign_packed,
+ * block, scale as there; block >= 16), so that the dequantised vector never
+ * reaches memory; out (fp32 [n]) receives the rotated vector.  post_scale (a
+ * float32 on the device, e.g. result + 2 of dq_eden_quantize; may be NULL)
+ * multiplies every element last, which is the reference's `scale * vec`.
+ * Same bits as dq_eden_dequantize, dq_rht_blocked(inverse) and the product. */
+int dq_eden_dequantize_irht(const uint32_t *packed, int64_t n, const float *centroids, int nbits,
+                            const void *sign, int sign_packed, float *out, int64_t block,
+                            float scale, const float *post_scale, int device,
+                            dq_stream_t stream);
+
 /* thc_hooks.py:176-178: out = float(levels) * *step + *lo (two roundings). */
 int dq_thc_dequantize(const void *levels_bf16, float *out, int64_t n, const float *step,
                       const float *lo, int device, dq_stream_t stream);

@@ -277,3 +277,33 @@ def test_thc_quantiser_folded_into_the_transform(capi, n, block):
         b2 = torch.zeros(n + 4, device=DEV)[1:1 + n]
         capi.thc_dequantize_irht(g2 * 4, sign, b2, block, scale, step, lo)
         assert torch.equal(b2.view(torch.int32), dec.view(torch.int32))
+
+
+@pytest.mark.parametrize("nbits", [1, 3, 4, 8])
+@pytest.mark.parametrize("n,block", [(32, 32), (96, 32), (1024, 1024), (4096 * 3, 4096), (1 << 15, 1 << 15), (1 << 16, 1 << 16),
+                                     (1 << 20, 1 << 20), (1 << 22, 1 << 22), (1 << 18, 1 << 12)])
+def test_eden_dequantiser_folded_into_the_inverse_transform(capi, nbits, n, block):
+    """dq_eden_dequantize_irht == eden_dequantize, inverse rht_blocked, product with the scale -- bit for bit, single-pass
+    and multi-pass transforms, float and packed diagonals, with and without the scale"""
+    g = torch.Generator().manual_seed(n + nbits)
+    cen, _ = _tables(nbits)
+    bins = torch.randint(0, 1 << nbits, (n,), generator=g, dtype=torch.int32).to(DEV)
+    packed = torch.empty(n // 32 * nbits, dtype=torch.int32, device=DEV)
+    capi.bins_to_bits(bins, packed, nbits)
+    sign = (torch.randint(0, 2, (n,), generator=g).float() * 2 - 1).to(DEV)
+    scale = float(np.float32(1.0) / np.float32(np.sqrt(block)))
+    eden_scale = torch.tensor([0.00123], dtype=torch.float32, device=DEV)
+    want = torch.empty(n, device=DEV)
+    capi.eden_dequantize(packed, n, cen, nbits, want)
+    capi.rht_blocked(want, sign, block, scale, True)
+    for sg in (sign, capi.pack_signs(sign), None):
+        ref = want
+        if sg is None:
+            ref = torch.empty(n, device=DEV)
+            capi.eden_dequantize(packed, n, cen, nbits, ref)
+            capi.rht_blocked(ref, None, block, scale, True)
+        got = torch.full((n + 8,), 7.0, device=DEV)
+        capi.eden_dequantize_irht(packed, n, cen, nbits, sg, got[:n], block, scale)
+        assert torch.equal(got[:n].view(torch.int32), ref.view(torch.int32)) and bool((got[n:] == 7.0).all())
+        capi.eden_dequantize_irht(packed, n, cen, nbits, sg, got[:n], block, scale, post_scale=eden_scale)
+        assert torch.equal(got[:n].view(torch.int32), (eden_scale * ref).view(torch.int32)) and bool((got[n:] == 7.0).all())

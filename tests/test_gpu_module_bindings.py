@@ -145,5 +145,13 @@ def test_transform_bindings(capi, eden_utils):
     assert torch.equal(ra, rb)
     assert torch.equal(eu.rht_blocked(x.clone(), bits_a, block, scale, False), eu.rht_blocked(x.clone(), sign, block, scale, False))
     assert torch.equal(eu.rand_diag_bits(n, 5, x.device), capi.pack_signs(eu.rand_diag(n, 5, x.device)))
+    # EDEN's dequantiser folded into the inverse rotation
+    from dynamiq_sigcomm_artifact_amd.eden import normal_centroids_and_boundaries
+    cen = normal_centroids_and_boundaries(4)[0].to(DEV)
+    pk = torch.randint(-2 ** 31, 2 ** 31 - 1, (n // 32 * 4,), generator=g, dtype=torch.int32).to(DEV)
+    es = torch.tensor([0.5], device=DEV)
+    oa = torch.empty(n, device=DEV)
+    capi.eden_dequantize_irht(pk, n, cen, 4, bits_a, oa, n, 1.0 / math.sqrt(n), post_scale=es)
+    assert torch.equal(oa, eu.eden_dequantize_irht(pk, cen, 4, bits_a, n, 1.0 / math.sqrt(n), es))
     with pytest.raises(RuntimeError, match="multiple of 256"):
         eu.rand_diag_bits(100, 5, x.device)

@@ -158,6 +158,10 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_thc_rht_quantize(P, P, 0, P, P, 64, 64, F1, P, P, 1, 0, S), "levels")
     err(L.dq_thc_rht_quantize(P, P, 0, N, P, 64, 64, F1, P, P, 31, 0, S), "null pointer")
     err(L.dq_thc_dequantize_irht(P, P, 0, N, 64, 64, F1, P, P, 0, S), "null pointer")
+    err(L.dq_eden_dequantize_irht(P, 64, P, 9, P, 0, P, 64, F1, N, 0, S), "nbits must be in")
+    err(L.dq_eden_dequantize_irht(P, 48, P, 4, P, 0, P, 16, F1, N, 0, S), "multiple of 32")
+    err(L.dq_eden_dequantize_irht(P, 64, P, 4, P, 0, P, 8, F1, N, 0, S), "block")
+    err(L.dq_eden_dequantize_irht(P, 64, P, 4, P, 0, N, 64, F1, N, 0, S), "null pointer")
     err(L.dq_thc_dequantize_irht(P, P, 1, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
     assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 and capi.eden_work_doubles(8192) == 2 and capi.bitrate_hist_ints() == 32768
