@@ -303,3 +303,62 @@ def test_hip_graph_replay(capi):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(send, want_send) and torch.equal(out, want_out), k
+
+
+def test_offset_search_on_the_whole_gradient_set():
+    """config 4's size: the norm patterns of 29,315,072 superchunks in one histogram call and bucket by bucket, against
+    torch.bincount of the same bins; the search on it against the reference's torch op sequence on the device"""
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    from dynamiq_sigcomm_artifact_amd import capi
+    nsc = 29315072
+    g = torch.Generator(device=DEV).manual_seed(4)
+    stats = torch.zeros((nsc, 2), dtype=torch.bfloat16, device=DEV)
+    stats[:, 1] = torch.exp(torch.randn(nsc, generator=g, device=DEV) * 3.0 - 9.0).to(torch.bfloat16)
+    stats[::100003, 1] = float("nan")
+    stats[5::70001, 1] = 0.0
+    pat = stats[:, 1].contiguous().view(torch.int16).to(torch.int64) & 0xffff
+    bins = torch.where((pat & 0x7fff) > 0x7f80, torch.full_like(pat, 0x7f81), torch.where(pat > 0x7f80, torch.zeros_like(pat), pat))
+    want = torch.bincount(bins, minlength=capi.bitrate_hist_ints()).to(torch.int32)
+    h = B.NormHistogram(DEV)
+    h.add(stats)
+    assert torch.equal(h.hist, want)
+    h.hist.zero_()
+    for k in range(0, nsc, 25600 * 64):                      # in pieces, as the buckets of a step would arrive
+        h.add(stats[k:k + 25600 * 64])
+    assert torch.equal(h.hist, want)
+    norms = stats[:, 1].contiguous()
+    finite = norms[~torch.isnan(norms)]                      # the op sequence on NaN norms is the device's int conversion
+    got = h.binary_search_u(4.375)
+    nan_count = int(torch.isnan(norms).sum())
+    # the reference's sequence over the finite norms plus 2 bits for every NaN norm
+    def avg(u):
+        return (float(B.dynamic_bitrate_qbits(finite, u).sum().item()) + 2.0 * nan_count) / nsc
+    assert abs(got[1] - avg(got[0])) == 0.0 and abs((4.375 - got[1]) - got[2]) == 0.0
+    assert abs(got[2]) <= B.DYNAMIC_BITRATE_TOL
+
+
+def test_eden_at_the_padded_bucket_size(capi, oracle):
+    """d = 2^23: the quantiser against the oracle, the folded dequantiser + inverse rotation against the separate calls"""
+    n, nbits = 1 << 23, 4
+    gold = np.load(__import__("os").path.join(__import__("os").path.dirname(__file__), "golden", "eden_golden.npz"))
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(n, generator=g) * 2e-3
+    cen = torch.from_numpy(gold["centroids_%d" % nbits]).to(DEV)
+    bnd = torch.from_numpy(gold["boundaries_%d" % nbits]).to(DEV)
+    packed = torch.empty(n // 32 * nbits, dtype=torch.int32, device=DEV)
+    result = torch.zeros(4, device=DEV)
+    work = torch.zeros(capi.eden_work_doubles(n), dtype=torch.float64, device=DEV)
+    capi.eden_quantize(x.to(DEV), bnd, cen, nbits, packed, result, work)
+    bins_o, res_o = oracle.eden_quantize(x.numpy(), gold["boundaries_%d" % nbits], gold["centroids_%d" % nbits], nbits)
+    assert (result.cpu().numpy().view(np.uint32) == res_o.view(np.uint32)).all()
+    assert (packed.cpu().numpy().view(np.uint32) == oracle.bins_to_bits(bins_o, nbits)).all()
+    bits = torch.empty(n // 32, dtype=torch.int32, device=DEV)
+    capi.rand_diag_bits(bits, n, 3)
+    inv = float(np.float32(1.0) / np.float32(np.sqrt(n)))
+    want = torch.empty(n, device=DEV)
+    capi.eden_dequantize(packed, n, cen, nbits, want)
+    capi.rht_blocked(want, bits, n, inv, True)
+    want = result[2:3] * want
+    got = torch.empty(n, device=DEV)
+    capi.eden_dequantize_irht(packed, n, cen, nbits, bits, got, n, inv, post_scale=result[2:3])
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
