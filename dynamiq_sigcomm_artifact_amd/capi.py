@@ -28,7 +28,7 @@ EXPORTS = [
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
-    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_dequantize", "dq_eden_dequantize_irht", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
+    "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_quantize_static_max_n", "dq_eden_quantize_static", "dq_eden_dequantize", "dq_eden_dequantize_irht", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
 ]
 
 _lib = None
@@ -124,6 +124,10 @@ def lib():
         L.dq_eden_work_doubles.argtypes = [i64]
         L.dq_eden_quantize.restype = i32
         L.dq_eden_quantize.argtypes = [vp, i64, vp, vp, i32, vp, vp, vp, i64, i32, vp]
+        L.dq_eden_quantize_static_max_n.restype = i64
+        L.dq_eden_quantize_static_max_n.argtypes = []
+        L.dq_eden_quantize_static.restype = i32
+        L.dq_eden_quantize_static.argtypes = [vp, i64, vp, vp, i32, vp, vp, i32, vp]
         L.dq_eden_dequantize.restype = i32
         L.dq_eden_dequantize.argtypes = [vp, i64, vp, i32, vp, i32, vp]
         L.dq_thc_quantize.restype = i32
@@ -451,6 +455,22 @@ def eden_quantize(vec, boundaries, centroids, nbits, packed, result, work, strea
         raise RuntimeError("eden_quantize: a buffer is too small")
     _check(lib().dq_eden_quantize(vec.data_ptr(), n, boundaries.data_ptr(), centroids.data_ptr(), nbits, packed.data_ptr(),
                                   result.data_ptr(), work.data_ptr(), work.numel(), _dev(vec), _stream(stream)))
+
+
+def eden_quantize_static(vec, boundaries, centroids, nbits, packed, result, stream=None, n=None):
+    """eden_quantize with the partial sums in the library's static device array: nothing is allocated.
+    Calls that overlap on one GPU race on that array."""
+    for t, name in ((vec, "vec"), (boundaries, "boundaries"), (centroids, "centroids"), (result, "result")):
+        if t.dtype != torch.float32:
+            raise RuntimeError("eden_quantize_static: %s must be float32" % name)
+    if packed.dtype != torch.int32:
+        raise RuntimeError("eden_quantize_static: packed must be int32")
+    n = vec.numel() if n is None else int(n)
+    if boundaries.numel() < (1 << nbits) - 1 or centroids.numel() < (1 << nbits) or result.numel() < 4 \
+            or packed.numel() < n // 32 * nbits or vec.numel() < n:
+        raise RuntimeError("eden_quantize_static: a buffer is too small")
+    _check(lib().dq_eden_quantize_static(vec.data_ptr(), n, boundaries.data_ptr(), centroids.data_ptr(), nbits,
+                                         packed.data_ptr(), result.data_ptr(), _dev(vec), _stream(stream)))
 
 
 def eden_dequantize(packed, n, centroids, nbits, out, stream=None):

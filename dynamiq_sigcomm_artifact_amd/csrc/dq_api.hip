@@ -650,6 +650,22 @@ int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const
                                            static_cast<hipStream_t>(stream)));
 }
 
+int64_t dq_eden_quantize_static_max_n(void) { return dq::eden_static_max_n(); }
+
+int dq_eden_quantize_static(const float *vec, int64_t n, const float *boundaries, const float *centroids, int nbits,
+                            uint32_t *packed, float *result, int device, dq_stream_t stream)
+{
+    if (!(n > 0) || (n & 31) != 0) return fail(DQ_ERR_SIZE, "n must be a positive multiple of 32");
+    if (n > dq::eden_static_max_n())
+        return fail(DQ_ERR_SIZE, "n exceeds the static scratch array (dq_eden_quantize_static_max_n); use dq_eden_quantize");
+    if (nbits < 1 || nbits > 8) return fail(DQ_ERR_NBITS, "nbits must be in [1, 8]");
+    if (!vec || !boundaries || !centroids || !packed || !result) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_eden_quantize_static(vec, n, boundaries, centroids, nbits, packed, result, device,
+                                                  static_cast<hipStream_t>(stream)));
+}
+
 int dq_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits, float *out, int device,
                        dq_stream_t stream)
 {

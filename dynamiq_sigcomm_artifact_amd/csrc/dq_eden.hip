@@ -13,6 +13,8 @@
 //   scale   dot = fold(work[]); scale = (norm * norm) / (float)dot
 // The sums are in double with a fixed association, so the result does not depend on the launch geometry
 // and the CPU restatement reproduces it bit for bit.
+#include <mutex>
+
 #include "dq_launch.h"
 #include "dq_tile16.cuh"
 
@@ -303,6 +305,46 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
     }
     hipLaunchKernelGGL(eden_scale_kernel, dim3(1), block, 0, stream, work, tiles, result);
     return hipGetLastError();
+}
+
+} // namespace dq
+
+// ---- EDEN quantise without any allocation ------------------------------------------------------
+// The per-tile partial sums of launch_eden_quantize live in this array instead of a caller's buffer.
+// Every device the library runs on holds its own copy for the life of the process (512 KiB).  The
+// array's name is only a host-side handle: its device address comes from hipGetSymbolAddress, once
+// per device, and that pointer is what the kernels receive.
+static constexpr int64_t kEdenStaticMaxTiles = 65536; // 2^28 elements of 4096-element tiles
+static __device__ __align__(256) double eden_static_scratch[kEdenStaticMaxTiles];
+
+namespace dq {
+
+int64_t eden_static_max_n() { return kEdenStaticMaxTiles * (int64_t)kEdenTile; }
+
+hipError_t launch_eden_quantize_static(const float *vec, int64_t n, const float *boundaries, const float *centroids,
+                                       int nbits, uint32_t *packed, float *result, int device, hipStream_t stream)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static double *scratch_of[kMaxDevices]; // device address of eden_static_scratch, per device
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    if (eden_tiles(n) > kEdenStaticMaxTiles) return hipErrorInvalidValue;
+    double *scratch;
+    {
+        std::lock_guard<std::mutex> g(lock);
+        if (!scratch_of[device]) {
+            // the caller has made `device` current
+            void *p = nullptr;
+            const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(eden_static_scratch));
+            if (e != hipSuccess) return e;
+            if (!p) return hipErrorInvalidSymbol;
+            scratch_of[device] = static_cast<double *>(p);
+        }
+        scratch = scratch_of[device];
+    }
+    // every word of scratch that a kernel reads has been written by an earlier kernel of this same
+    // call (sumsq -> norm, bins -> scale), so nothing has to be cleared between calls
+    return launch_eden_quantize(vec, n, boundaries, centroids, nbits, packed, result, scratch, stream);
 }
 
 hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits, float *out,

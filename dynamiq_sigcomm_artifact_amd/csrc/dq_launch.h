@@ -123,6 +123,12 @@ int64_t eden_work_doubles(int64_t n);
 hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,
                                 int nbits, uint32_t *packed, float *result, double *work,
                                 hipStream_t stream);
+// the same launches with the partial sums in the library's own static device array (no allocation anywhere);
+// `device` must be current
+int64_t eden_static_max_n();
+hipError_t launch_eden_quantize_static(const float *vec, int64_t n, const float *boundaries, const float *centroids,
+                                       int nbits, uint32_t *packed, float *result, int device,
+                                       hipStream_t stream);
 hipError_t launch_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits,
                                   float *out, hipStream_t stream);
 hipError_t launch_thc_quantize(const float *rotated, const float *uniform, void *out, int64_t n,

@@ -315,6 +315,21 @@ int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const
                      int nbits, uint32_t *packed, float *result, double *work,
                      int64_t work_doubles, int device, dq_stream_t stream);
 
+/* No counterpart in the reference.  dq_eden_quantize for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the same launches and the same results, with
+ * the per-tile partial sums in a static device array inside the library
+ * (512 KiB per GPU, held until the process ends) instead of a caller's `work`.
+ * Neither this call nor anything it runs allocates or frees memory.
+ * n is limited to dq_eden_quantize_static_max_n() = 2^28 elements; a larger n
+ * is refused with DQ_ERR_SIZE.  All calls on one GPU share the array: calls
+ * that may overlap on one GPU (two streams, two threads) race -- serialise them
+ * or use dq_eden_quantize with separate work buffers. */
+int64_t dq_eden_quantize_static_max_n(void);
+int dq_eden_quantize_static(const float *vec, int64_t n, const float *boundaries,
+                            const float *centroids, int nbits, uint32_t *packed, float *result,
+                            int device, dq_stream_t stream);
+
 /* srrcomp.py:343-345: out_i = centroids[bin_i] from the bit planes.  out must be
  * 16-byte aligned. */
 int dq_eden_dequantize(const uint32_t *packed, int64_t n, const float *centroids, int nbits,
