@@ -104,6 +104,61 @@ def dynamic_bitrate_adjust_u(norms_list, prev_u, target_avg_bits):
     return best.triple()
 
 
+# ---- fixed-proportion allocation (the non-dynamic P2P_dynamiQ hook) -------------------------------------
+
+def fixed_proportion_thresholds(aggregation_method):
+    """comm_hooks.py:842-856: the fractions of a bucket's superchunks that get 8, 4 and 2 bits, chosen by the
+    "<n>bit" token of the method name ("4bit" + "fixed": every superchunk 4 bits; no token: the 5-bit mix)"""
+    name = aggregation_method
+    if "4bit" in name:
+        return {4: 1, 8: 0, 2: 0} if "fixed" in name else {8: 0.05, 4: 0.6, 2: 0.35}
+    if "3bit" in name:
+        return {8: 1 / 40, 4: 13 / 40, 2: 26 / 40}
+    if "6bit" in name:
+        return {8: 0.55, 4: 0.35, 2: 0.1}
+    if "7bit" in name:
+        return {8: 0.75, 4: 0.22, 2: 0.03}
+    return {8: 0.35, 4: 0.45, 2: 0.2}
+
+
+def fixed_proportion_counts(num_superchunks, thresholds):
+    """comm_hooks.py:713-716: (superchunks at 8 bits, at 4 bits, at 2 bits); the products are truncated, and the
+    2-bit share gives way when the two together exceed the bucket"""
+    top = int(num_superchunks * thresholds[8])
+    bottom = int(num_superchunks * thresholds[2])
+    if top + bottom > num_superchunks:
+        bottom = max(0, num_superchunks - top)
+    return top, num_superchunks - top - bottom, bottom
+
+
+def fixed_proportion_groups(norms, thresholds):
+    """comm_hooks.py:710-721 as the reference's torch ops: the superchunks in descending order of their reduced
+    squared norm (stable: equal norms keep index order; NaN sorts above every number), the first `top` at 8 bits, the
+    last `bottom` at 2, the rest at 4.  Returns three int64 index tensors **in sorted order** -- the order in which the
+    hook gathers the group tensor, hence the order of the records and of the rounding-randomness rows."""
+    norms = norms.float()
+    top, _, bottom = fixed_proportion_counts(norms.numel(), thresholds)
+    order = torch.argsort(norms, descending=True, stable=True)
+    n = norms.numel()
+    return order[:top], order[top:n - bottom], order[n - bottom:] if bottom > 0 else order[:0]
+
+
+def fixed_proportion_plan(stats, thresholds, order=None, work=None, stream=None):
+    """The same three lists from the interleaved bf16 (mean, norm) statistics by one launch, without a sort and
+    without a read-back: ``order`` int32 [3 * nsc] (the 8-bit list at 0, the 4-bit list at nsc, the 2-bit list at
+    2 * nsc, each in sorted order) and ``work[0..2]`` = the three counts, i.e. what the row-list and mixed codec
+    kernels take.  Returns (order, work, (n8, n4, n2))."""
+    from . import capi
+    nsc = stats.numel() // 2
+    n8, n4, n2 = fixed_proportion_counts(nsc, thresholds)
+    if order is None:
+        order = torch.empty(3 * nsc, dtype=torch.int32, device=stats.device)
+    if work is None:
+        work = torch.empty(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=stats.device)
+    capi.group_plan_sorted(stats, n8, n2, order, work, stream)
+    return order, work, (n8, n4, n2)
+
+
 class NormHistogram(object):
     """The two searches above without a pass over the norms per probe: the norm patterns of every bucket are counted
     into a device histogram (``add``, one small launch per bucket, after the statistics all-reduce), and one launch runs

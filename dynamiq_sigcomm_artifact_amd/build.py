@@ -68,12 +68,22 @@ def _run(cmd, what):
     return time.time() - t0
 
 
-def build_kernels(verbose=True, jobs=6):
+def _newest_header():
+    return max(os.path.getmtime(os.path.join(CSRC, f)) for f in os.listdir(CSRC) if f.endswith((".cuh", ".h")))
+
+
+def build_kernels(verbose=True, jobs=6, only_changed=False):
+    """only_changed: keep an object file that is newer than its source and every header (for edit-compile loops;
+    the default recompiles everything)"""
     os.makedirs(OBJ_DIR, exist_ok=True)
     hipcc = _hipcc()
+    headers = _newest_header() if only_changed else 0.0
 
     def one(src):
         obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        if only_changed and os.path.exists(obj) and \
+                os.path.getmtime(obj) > max(headers, os.path.getmtime(os.path.join(CSRC, src))):
+            return obj
         dt = _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj], "hipcc " + src)
         if verbose:
             print("  hipcc %-28s %.1fs" % (src, dt))
@@ -122,6 +132,6 @@ def build_all(verbose=True):
 if __name__ == "__main__":
     only = sys.argv[1] if len(sys.argv) > 1 else "all"
     if only in ("all", "kernels"):
-        build_kernels()
+        build_kernels(only_changed="--changed" in sys.argv)
     if only in ("all", "ext"):
         build_extension()

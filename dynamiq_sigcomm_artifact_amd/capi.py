@@ -6,6 +6,7 @@ device index and a stream handle straight to ``libdynamiq_eden.so`` and raises
 library must be present; there is no fallback path.
 """
 import ctypes
+import threading
 import os
 
 import torch
@@ -22,7 +23,7 @@ EXPORTS = [
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
     "dq_scaling_compress_philox", "dq_scaling_dec_comp_philox", "dq_philox_uniform",
     "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
-    "dq_group_plan_stats_dev_u", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
+    "dq_group_plan_stats_dev_u", "dq_group_plan_sorted", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
@@ -76,6 +77,8 @@ def lib():
         L.dq_group_plan.argtypes = [vp, i64, vp, vp, i64, i32, vp]
         L.dq_group_plan_stats.restype = i32
         L.dq_group_plan_stats.argtypes = [vp, c.c_double, i64, vp, vp, vp, i64, i32, vp]
+        L.dq_group_plan_sorted.restype = i32
+        L.dq_group_plan_sorted.argtypes = [vp, i64, i64, i64, vp, vp, vp, i64, i32, vp]
         L.dq_group_plan_stats_dev_u.restype = i32
         L.dq_group_plan_stats_dev_u.argtypes = [vp, vp, i64, vp, vp, vp, i64, vp, i64, i32, vp]
         L.dq_bitrate_hist_ints.restype = i64
@@ -171,14 +174,55 @@ def _check(rc):
         raise RuntimeError(lib().dq_last_error().decode())
 
 
-def _stream(stream):
-    if stream is None:
-        stream = torch.cuda.current_stream().cuda_stream
-    return ctypes.c_void_p(int(stream))
+# The kernels dereference whatever address they are given: a host pointer, a strided view or a buffer of another
+# GPU is a memory fault on the device, not an error code.  Every tensor whose address goes into the library passes
+# through _p / _ptr / _dev, which refuse anything but contiguous device tensors and note the device; _call refuses a
+# mix of devices before the library is entered.
+_seen = threading.local()
+
+
+def _note(t):
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError("a tensor argument is required, got %s" % type(t).__name__)
+    if not t.is_cuda:
+        raise RuntimeError("tensor arguments must live on the GPU (got a %s tensor)" % t.device.type)
+    if not t.is_contiguous():
+        raise RuntimeError("tensor arguments must be contiguous")
+    devices = getattr(_seen, "devices", None)
+    if devices is None:
+        devices = _seen.devices = set()
+    devices.add(t.device.index)
+
+
+def _p(t):
+    _note(t)
+    return t.data_ptr()
+
+
+def _ptr(t):
+    return 0 if t is None else _p(t)
 
 
 def _dev(t):
-    return t.device.index if t.device.index is not None else torch.cuda.current_device()
+    _note(t)
+    return t.device.index
+
+
+def _call(fn, *args):
+    devices = getattr(_seen, "devices", None) or set()
+    _seen.devices = set()
+    if len(devices) > 1:
+        raise RuntimeError("tensor arguments live on different devices: %s" % sorted(devices))
+    _check(fn(*args))
+
+
+def _stream(stream):
+    """a raw stream handle (int), a torch.cuda.Stream, or None for torch's current stream"""
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    elif hasattr(stream, "cuda_stream"):
+        stream = stream.cuda_stream
+    return ctypes.c_void_p(int(stream))
 
 
 def required_bytes(n, nbits, chunk_size, strategy):
@@ -186,30 +230,30 @@ def required_bytes(n, nbits, chunk_size, strategy):
 
 
 def check_common(n, nbits, chunk_size, strategy, strict=True):
-    _check(lib().dq_scaling_check_common(n, nbits, chunk_size, strategy, 1 if strict else 0))
+    _call(lib().dq_scaling_check_common, n, nbits, chunk_size, strategy, 1 if strict else 0)
 
 
 def mee_lookup_table(nbits):
     import numpy as np
     table = np.zeros(256, np.uint16)
     params = np.zeros(4, np.uint16)
-    _check(lib().dq_mee_lookup_table(nbits, table.ctypes.data_as(ctypes.c_void_p), params.ctypes.data_as(ctypes.c_void_p)))
+    _call(lib().dq_mee_lookup_table, nbits, table.ctypes.data_as(ctypes.c_void_p), params.ctypes.data_as(ctypes.c_void_p))
     return table, params
 
 
 def scaling_compress(src, dst, rand_pool, n, nbits, chunk_size, strategy, stream=None):
-    _check(lib().dq_scaling_compress(src.data_ptr(), dst.data_ptr(), rand_pool.data_ptr(), n, nbits, chunk_size,
-                                     _pair_code(src, rand_pool), _dev(src), strategy, _stream(stream)))
+    _call(lib().dq_scaling_compress, _p(src), _p(dst), _p(rand_pool), n, nbits, chunk_size,
+                                     _pair_code(src, rand_pool), _dev(src), strategy, _stream(stream))
 
 
 def scaling_decompress(src, dst, n, nbits, chunk_size, strategy, add=False, stream=None):
-    _check(lib().dq_scaling_decompress(src.data_ptr(), dst.data_ptr(), n, nbits, chunk_size, dtype_code(dst), _dev(dst),
-                                       strategy, _stream(stream), 1 if add else 0))
+    _call(lib().dq_scaling_decompress, _p(src), _p(dst), n, nbits, chunk_size, dtype_code(dst), _dev(dst),
+                                       strategy, _stream(stream), 1 if add else 0)
 
 
 def scaling_dec_comp(recv, inp, send, rand_pool, n, nbits, chunk_size, strategy, stream=None):
-    _check(lib().dq_scaling_dec_comp(recv.data_ptr(), inp.data_ptr(), send.data_ptr(), rand_pool.data_ptr(), n, nbits,
-                                     chunk_size, _pair_code(inp, rand_pool), _dev(inp), strategy, _stream(stream)))
+    _call(lib().dq_scaling_dec_comp, _p(recv), _p(inp), _p(send), _p(rand_pool), n, nbits,
+                                     chunk_size, _pair_code(inp, rand_pool), _dev(inp), strategy, _stream(stream))
 
 
 def group_plan_work_ints(nsc):
@@ -223,18 +267,26 @@ def group_plan(qbits, order, work, stream=None):
         raise RuntimeError("group_plan: qbits must be int64, order and work int32")
     if order.numel() < 3 * qbits.numel():
         raise RuntimeError("group_plan: order has fewer than 3 * nsc entries")
-    _check(lib().dq_group_plan(qbits.data_ptr(), qbits.numel(), order.data_ptr(), work.data_ptr(), work.numel(),
-                               _dev(qbits), _stream(stream)))
-
-
-def _ptr(t):
-    return 0 if t is None else t.data_ptr()
+    _call(lib().dq_group_plan, _p(qbits), qbits.numel(), _p(order), _p(work), work.numel(),
+                               _dev(qbits), _stream(stream))
 
 
 def group_rows(order, nsc, width, count):
     """the row list of one width in a planned `order` (a view)"""
     base = {8: 0, 4: 1, 2: 2}[width] * nsc
     return order[base:base + count]
+
+
+def group_plan_sorted(stats, top_count, bottom_count, order, work, stream=None, qbits_out=None):
+    """fixed-proportion groups (comm_hooks.py:710-721): order / work[0:3] as group_plan writes them, every list in
+    the order of the stable descending sort of the norms stats[:, 1]"""
+    if stats.dtype != torch.bfloat16 or order.dtype != torch.int32 or work.dtype != torch.int32:
+        raise RuntimeError("group_plan_sorted: stats must be bfloat16, order and work int32")
+    nsc = stats.numel() // 2
+    if order.numel() < 3 * nsc or (qbits_out is not None and (qbits_out.dtype != torch.int64 or qbits_out.numel() < nsc)):
+        raise RuntimeError("group_plan_sorted: order / qbits_out too small or of the wrong dtype")
+    _call(lib().dq_group_plan_sorted, _p(stats), nsc, int(top_count), int(bottom_count), _ptr(qbits_out),
+                                      _p(order), _p(work), work.numel(), _dev(stats), _stream(stream))
 
 
 def group_plan_stats(stats, u, qbits_out, order, work, stream=None, hist=None):
@@ -252,14 +304,14 @@ def group_plan_stats(stats, u, qbits_out, order, work, stream=None, hist=None):
             raise RuntimeError("group_plan_stats: a tensor u must be float64 on the device of stats")
         if hist is not None and hist.dtype != torch.int32:
             raise RuntimeError("group_plan_stats: hist must be int32")
-        _check(lib().dq_group_plan_stats_dev_u(stats.data_ptr(), u.data_ptr(), nsc, _ptr(qbits_out), order.data_ptr(),
-                                               work.data_ptr(), work.numel(), _ptr(hist), 0 if hist is None else hist.numel(),
-                                               _dev(stats), _stream(stream)))
+        _call(lib().dq_group_plan_stats_dev_u, _p(stats), _p(u), nsc, _ptr(qbits_out), _p(order),
+                                               _p(work), work.numel(), _ptr(hist), 0 if hist is None else hist.numel(),
+                                               _dev(stats), _stream(stream))
         return
     if hist is not None:
         norm_histogram(stats, hist, stream)
-    _check(lib().dq_group_plan_stats(stats.data_ptr(), float(u), nsc, _ptr(qbits_out), order.data_ptr(), work.data_ptr(),
-                                     work.numel(), _dev(stats), _stream(stream)))
+    _call(lib().dq_group_plan_stats, _p(stats), float(u), nsc, _ptr(qbits_out), _p(order), _p(work),
+                                     work.numel(), _dev(stats), _stream(stream))
 
 
 def bitrate_hist_ints():
@@ -270,8 +322,8 @@ def norm_histogram(stats, hist, stream=None):
     """adds the norm patterns of stats (bf16 [nsc, 2]: mean, reduced sum of squares) to hist (int32 [bitrate_hist_ints()])"""
     if stats.dtype != torch.bfloat16 or hist.dtype != torch.int32:
         raise RuntimeError("norm_histogram: stats must be bfloat16 and hist int32")
-    _check(lib().dq_norm_histogram(stats.data_ptr(), stats.numel() // 2, hist.data_ptr(), hist.numel(), _dev(stats),
-                                   _stream(stream)))
+    _call(lib().dq_norm_histogram, _p(stats), stats.numel() // 2, _p(hist), hist.numel(), _dev(stats),
+                                   _stream(stream))
 
 
 def bitrate_search(hist, mode, prev_u, target_avg_bits, result, stream=None):
@@ -284,25 +336,25 @@ def bitrate_search(hist, mode, prev_u, target_avg_bits, result, stream=None):
         if prev_u.dtype != torch.float64 or prev_u.numel() < 1 or prev_u.device != hist.device:
             raise RuntimeError("bitrate_search: a tensor prev_u must be float64 on the device of hist")
         prev_dev, prev_u = prev_u, 0.0
-    _check(lib().dq_bitrate_search(hist.data_ptr(), hist.numel(), int(mode), float(prev_u), _ptr(prev_dev),
-                                   float(target_avg_bits), result.data_ptr(), _dev(hist), _stream(stream)))
+    _call(lib().dq_bitrate_search, _p(hist), hist.numel(), int(mode), float(prev_u), _ptr(prev_dev),
+                                   float(target_avg_bits), _p(result), _dev(hist), _stream(stream))
 
 
 def scaling_compress_rows(src, rows, dst, rand_pool, nrows, nbits, strategy, stream=None):
-    _check(lib().dq_scaling_compress_rows(src.data_ptr(), _ptr(rows), dst.data_ptr(), rand_pool.data_ptr(), nrows, nbits,
-                                          _pair_code(src, rand_pool), _dev(src), strategy, _stream(stream)))
+    _call(lib().dq_scaling_compress_rows, _p(src), _ptr(rows), _p(dst), _p(rand_pool), nrows, nbits,
+                                          _pair_code(src, rand_pool), _dev(src), strategy, _stream(stream))
 
 
 def scaling_dec_comp_rows(recv, inp, rows, send, rand_pool, nrows, nbits, strategy, stream=None):
-    _check(lib().dq_scaling_dec_comp_rows(recv.data_ptr(), inp.data_ptr(), _ptr(rows), send.data_ptr(),
-                                          rand_pool.data_ptr(), nrows, nbits, _pair_code(inp, rand_pool), _dev(inp),
-                                          strategy, _stream(stream)))
+    _call(lib().dq_scaling_dec_comp_rows, _p(recv), _p(inp), _ptr(rows), _p(send),
+                                          _p(rand_pool), nrows, nbits, _pair_code(inp, rand_pool), _dev(inp),
+                                          strategy, _stream(stream))
 
 
 def scaling_decompress_rows(src, dst, rows, stats, n_limit, nrows, nbits, strategy, add=False, stream=None):
-    _check(lib().dq_scaling_decompress_rows(src.data_ptr(), dst.data_ptr(), _ptr(rows), _ptr(stats), n_limit, nrows,
+    _call(lib().dq_scaling_decompress_rows, _p(src), _p(dst), _ptr(rows), _ptr(stats), n_limit, nrows,
                                             nbits, dtype_code(dst), _dev(dst), strategy, _stream(stream),
-                                            1 if add else 0))
+                                            1 if add else 0)
 
 
 def mixed_required_bytes(nsc, ring_world=1):
@@ -314,60 +366,60 @@ def mixed_compress(src, order, counts, dst, nsc, strategy, rand_pool=None, seed=
     """all three bit-width groups of the plan (order, counts = work[0:3] of group_plan*) in one launch; recv makes it
     the ring's fused step; center_mean (float32 per superchunk, from superchunk_stats) centres src on load"""
     code = dtype_code(src) if rand_pool is None else _pair_code(src, rand_pool)
-    _check(lib().dq_mixed_compress(src.data_ptr(), _ptr(center_mean), center_world, n, order.data_ptr(), counts.data_ptr(),
-                                   ring_chunk, ring_world, _ptr(recv), dst.data_ptr(), _ptr(rand_pool), int(seed), int(step),
-                                   nsc, code, _dev(src), strategy, _stream(stream)))
+    _call(lib().dq_mixed_compress, _p(src), _ptr(center_mean), center_world, n, _p(order), _p(counts),
+                                   ring_chunk, ring_world, _ptr(recv), _p(dst), _ptr(rand_pool), int(seed), int(step),
+                                   nsc, code, _dev(src), strategy, _stream(stream))
 
 
 def mixed_decompress(src, dst, order, counts, nsc, strategy, stats=None, n_limit=None, ring_chunk=0, ring_world=1,
                      stream=None):
-    _check(lib().dq_mixed_decompress(src.data_ptr(), dst.data_ptr(), order.data_ptr(), counts.data_ptr(), ring_chunk,
+    _call(lib().dq_mixed_decompress, _p(src), _p(dst), _p(order), _p(counts), ring_chunk,
                                      ring_world, _ptr(stats), nsc * 256 if n_limit is None else n_limit, nsc,
-                                     dtype_code(dst), _dev(dst), strategy, _stream(stream)))
+                                     dtype_code(dst), _dev(dst), strategy, _stream(stream))
 
 
 def superchunk_stats(src, stats, mean, n, world_size, stream=None):
     """the statistics of superchunk_mean_center without the residual; mean (float32 [nsc] or None) gets the unrounded means"""
-    _check(lib().dq_superchunk_stats(src.data_ptr(), stats.data_ptr(), _ptr(mean), n, world_size, dtype_code(src), _dev(src),
-                                     _stream(stream)))
+    _call(lib().dq_superchunk_stats, _p(src), _p(stats), _ptr(mean), n, world_size, dtype_code(src), _dev(src),
+                                     _stream(stream))
 
 
 def scaling_compress_philox(src, dst, n, nbits, chunk_size, strategy, seed, step, stream=None):
     """scaling_compress with the uniform values drawn in the kernel (Philox keyed by seed, counter = chunk, step)"""
-    _check(lib().dq_scaling_compress_philox(src.data_ptr(), dst.data_ptr(), n, nbits, chunk_size, dtype_code(src), _dev(src),
-                                            strategy, int(seed), int(step), _stream(stream)))
+    _call(lib().dq_scaling_compress_philox, _p(src), _p(dst), n, nbits, chunk_size, dtype_code(src), _dev(src),
+                                            strategy, int(seed), int(step), _stream(stream))
 
 
 def scaling_dec_comp_philox(recv, inp, send, n, nbits, chunk_size, strategy, seed, step, stream=None):
-    _check(lib().dq_scaling_dec_comp_philox(recv.data_ptr(), inp.data_ptr(), send.data_ptr(), n, nbits, chunk_size,
-                                            dtype_code(inp), _dev(inp), strategy, int(seed), int(step), _stream(stream)))
+    _call(lib().dq_scaling_dec_comp_philox, _p(recv), _p(inp), _p(send), n, nbits, chunk_size,
+                                            dtype_code(inp), _dev(inp), strategy, int(seed), int(step), _stream(stream))
 
 
 def philox_uniform(out, seed, step, stream=None):
     """the uniform values of that stream as a tensor (any of the three element types)"""
-    _check(lib().dq_philox_uniform(out.data_ptr(), out.numel(), dtype_code(out), _dev(out), int(seed), int(step),
-                                   _stream(stream)))
+    _call(lib().dq_philox_uniform, _p(out), out.numel(), dtype_code(out), _dev(out), int(seed), int(step),
+                                   _stream(stream))
 
 
 def superchunk_mean_center(src, residual, stats, n, world_size, superchunk_size=256, stream=None):
-    _check(lib().dq_superchunk_mean_center(src.data_ptr(), residual.data_ptr(), stats.data_ptr(), n, world_size,
-                                           superchunk_size, dtype_code(src), _dev(src), _stream(stream)))
+    _call(lib().dq_superchunk_mean_center, _p(src), _p(residual), _p(stats), n, world_size,
+                                           superchunk_size, dtype_code(src), _dev(src), _stream(stream))
 
 
 def superchunk_add_mean_copy(residual, dst, stats, n, superchunk_size=256, stream=None):
-    _check(lib().dq_superchunk_add_mean_copy(residual.data_ptr(), dst.data_ptr(), stats.data_ptr(), n, superchunk_size,
-                                             dtype_code(residual), _dev(residual), _stream(stream)))
+    _call(lib().dq_superchunk_add_mean_copy, _p(residual), _p(dst), _p(stats), n, superchunk_size,
+                                             dtype_code(residual), _dev(residual), _stream(stream))
 
 
 def hadamard(vec, stream=None):
-    _check(lib().dq_hadamard(vec.data_ptr(), vec.numel(), _dev(vec), _stream(stream), 0))
+    _call(lib().dq_hadamard, _p(vec), vec.numel(), _dev(vec), _stream(stream), 0)
 
 
 def rht_blocked(vec, sign, block, scale, inverse=False, stream=None):
     """sign: None, float32 +-1 values, or the int32 bit vector of pack_signs"""
     _check_sign(sign, vec.numel(), "rht_blocked")
-    _check(lib().dq_rht_blocked(vec.data_ptr(), _ptr(sign), _packed(sign), vec.numel(), block, float(scale),
-                                1 if inverse else 0, _dev(vec), _stream(stream)))
+    _call(lib().dq_rht_blocked, _p(vec), _ptr(sign), _packed(sign), vec.numel(), block, float(scale),
+                                1 if inverse else 0, _dev(vec), _stream(stream))
 
 
 def _packed(sign):
@@ -388,7 +440,7 @@ def _check_sign(sign, n, what):
 def pack_signs(sign, stream=None):
     """float32 +-1 vector -> int32 [ceil(n / 32)], bit e % 32 of word e / 32 set where sign[e] < 0"""
     bits = torch.empty((sign.numel() + 31) // 32, dtype=torch.int32, device=sign.device)
-    _check(lib().dq_pack_signs(sign.data_ptr(), bits.data_ptr(), sign.numel(), _dev(sign), _stream(stream)))
+    _call(lib().dq_pack_signs, _p(sign), _p(bits), sign.numel(), _dev(sign), _stream(stream))
     return bits
 
 
@@ -401,41 +453,41 @@ def rht_scaling_compress(src, sign, dst, block, scale, nbits, strategy, rand_poo
     code = 0
     if rand_pool is not None:
         code = dtype_code(rand_pool)
-    _check(lib().dq_rht_scaling_compress(src.data_ptr(), _ptr(sign), _packed(sign), dst.data_ptr(), _ptr(rand_pool), code, src.numel(),
+    _call(lib().dq_rht_scaling_compress, _p(src), _ptr(sign), _packed(sign), _p(dst), _ptr(rand_pool), code, src.numel(),
                                          block, float(scale), nbits, _dev(src), strategy, int(seed), int(step),
-                                         _stream(stream)))
+                                         _stream(stream))
 
 
 def scaling_decompress_irht(src, sign, dst, block, scale, nbits, strategy, stream=None):
     """scaling_decompress into float32 + rht_blocked (inverse) in one launch"""
     if dst.dtype != torch.float32:
         raise RuntimeError("scaling_decompress_irht: dst must be float32")
-    _check(lib().dq_scaling_decompress_irht(src.data_ptr(), _ptr(sign), _packed(sign), dst.data_ptr(), dst.numel(), block, float(scale),
-                                            nbits, _dev(dst), strategy, _stream(stream)))
+    _call(lib().dq_scaling_decompress_irht, _p(src), _ptr(sign), _packed(sign), _p(dst), dst.numel(), block, float(scale),
+                                            nbits, _dev(dst), strategy, _stream(stream))
 
 
 def rand_diag(out, seed, stream=None):
-    _check(lib().dq_rand_diag(out.data_ptr(), out.numel(), seed, _dev(out), _stream(stream)))
+    _call(lib().dq_rand_diag, _p(out), out.numel(), seed, _dev(out), _stream(stream))
 
 
 def rand_diag_bits(bits, size, seed, stream=None):
     """the diagonal of rand_diag(size, seed) as the int32 bit vector of pack_signs; size a multiple of 256"""
     if bits.dtype != torch.int32 or bits.numel() < size // 32:
         raise RuntimeError("rand_diag_bits: bits must be int32 [size / 32]")
-    _check(lib().dq_rand_diag_bits(bits.data_ptr(), size, seed, _dev(bits), _stream(stream)))
+    _call(lib().dq_rand_diag_bits, _p(bits), size, seed, _dev(bits), _stream(stream))
 
 
 def bins_to_bits(bins, arr, nbits, stream=None):
-    _check(lib().dq_bins_to_bits(bins.data_ptr(), bins.numel(), arr.data_ptr(), arr.numel(), nbits, _dev(bins), _stream(stream)))
+    _call(lib().dq_bins_to_bits, _p(bins), bins.numel(), _p(arr), arr.numel(), nbits, _dev(bins), _stream(stream))
 
 
 def bits_to_bins(bins, arr, nbits, stream=None):
-    _check(lib().dq_bits_to_bins(bins.data_ptr(), bins.numel(), arr.data_ptr(), arr.numel(), nbits, _dev(bins), _stream(stream)))
+    _call(lib().dq_bits_to_bins, _p(bins), bins.numel(), _p(arr), arr.numel(), nbits, _dev(bins), _stream(stream))
 
 
 def quantization(vec, div_factor, tensor_max, seed, stream=None):
-    _check(lib().dq_quantization(vec.data_ptr(), vec.numel(), _dev(vec), float(div_factor), float(tensor_max), int(seed),
-                                 _stream(stream)))
+    _call(lib().dq_quantization, _p(vec), vec.numel(), _dev(vec), float(div_factor), float(tensor_max), int(seed),
+                                 _stream(stream))
 
 
 def eden_work_doubles(n):
@@ -453,8 +505,8 @@ def eden_quantize(vec, boundaries, centroids, nbits, packed, result, work, strea
     if boundaries.numel() < (1 << nbits) - 1 or centroids.numel() < (1 << nbits) or result.numel() < 4 \
             or packed.numel() < n // 32 * nbits:
         raise RuntimeError("eden_quantize: a buffer is too small")
-    _check(lib().dq_eden_quantize(vec.data_ptr(), n, boundaries.data_ptr(), centroids.data_ptr(), nbits, packed.data_ptr(),
-                                  result.data_ptr(), work.data_ptr(), work.numel(), _dev(vec), _stream(stream)))
+    _call(lib().dq_eden_quantize, _p(vec), n, _p(boundaries), _p(centroids), nbits, _p(packed),
+                                  _p(result), _p(work), work.numel(), _dev(vec), _stream(stream))
 
 
 def eden_quantize_static(vec, boundaries, centroids, nbits, packed, result, stream=None, n=None):
@@ -469,8 +521,8 @@ def eden_quantize_static(vec, boundaries, centroids, nbits, packed, result, stre
     if boundaries.numel() < (1 << nbits) - 1 or centroids.numel() < (1 << nbits) or result.numel() < 4 \
             or packed.numel() < n // 32 * nbits or vec.numel() < n:
         raise RuntimeError("eden_quantize_static: a buffer is too small")
-    _check(lib().dq_eden_quantize_static(vec.data_ptr(), n, boundaries.data_ptr(), centroids.data_ptr(), nbits,
-                                         packed.data_ptr(), result.data_ptr(), _dev(vec), _stream(stream)))
+    _call(lib().dq_eden_quantize_static, _p(vec), n, _p(boundaries), _p(centroids), nbits,
+                                         _p(packed), _p(result), _dev(vec), _stream(stream))
 
 
 def eden_dequantize(packed, n, centroids, nbits, out, stream=None):
@@ -478,8 +530,8 @@ def eden_dequantize(packed, n, centroids, nbits, out, stream=None):
         raise RuntimeError("eden_dequantize: packed must be int32, centroids and out float32")
     if packed.numel() < n // 32 * nbits or out.numel() < n or centroids.numel() < (1 << nbits):
         raise RuntimeError("eden_dequantize: a buffer is too small")
-    _check(lib().dq_eden_dequantize(packed.data_ptr(), n, centroids.data_ptr(), nbits, out.data_ptr(), _dev(out),
-                                    _stream(stream)))
+    _call(lib().dq_eden_dequantize, _p(packed), n, _p(centroids), nbits, _p(out), _dev(out),
+                                    _stream(stream))
 
 
 def thc_quantize(rotated, uniform, levels_out, lo, delta, levels, stream=None):
@@ -489,8 +541,8 @@ def thc_quantize(rotated, uniform, levels_out, lo, delta, levels, stream=None):
     n = rotated.numel()
     if uniform.numel() < n or levels_out.numel() < n:
         raise RuntimeError("thc_quantize: a buffer is too small")
-    _check(lib().dq_thc_quantize(rotated.data_ptr(), uniform.data_ptr(), levels_out.data_ptr(), n, lo.data_ptr(),
-                                 delta.data_ptr(), levels, _dev(rotated), _stream(stream)))
+    _call(lib().dq_thc_quantize, _p(rotated), _p(uniform), _p(levels_out), n, _p(lo),
+                                 _p(delta), levels, _dev(rotated), _stream(stream))
 
 
 def thc_dequantize(levels_in, out, step, lo, stream=None):
@@ -500,8 +552,8 @@ def thc_dequantize(levels_in, out, step, lo, stream=None):
     n = levels_in.numel()
     if out.numel() < n:
         raise RuntimeError("thc_dequantize: out is too small")
-    _check(lib().dq_thc_dequantize(levels_in.data_ptr(), out.data_ptr(), n, step.data_ptr(), lo.data_ptr(), _dev(out),
-                                   _stream(stream)))
+    _call(lib().dq_thc_dequantize, _p(levels_in), _p(out), n, _p(step), _p(lo), _dev(out),
+                                   _stream(stream))
 
 
 def eden_dequantize_irht(packed, n, centroids, nbits, sign, out, block, scale, post_scale=None, stream=None):
@@ -514,8 +566,8 @@ def eden_dequantize_irht(packed, n, centroids, nbits, sign, out, block, scale, p
     if post_scale is not None and (post_scale.dtype != torch.float32 or post_scale.device != out.device):
         raise RuntimeError("eden_dequantize_irht: post_scale must be a float32 tensor on the device of out")
     _check_sign(sign, n, "eden_dequantize_irht")
-    _check(lib().dq_eden_dequantize_irht(packed.data_ptr(), n, centroids.data_ptr(), nbits, _ptr(sign), _packed(sign),
-                                         out.data_ptr(), block, float(scale), _ptr(post_scale), _dev(out), _stream(stream)))
+    _call(lib().dq_eden_dequantize_irht, _p(packed), n, _p(centroids), nbits, _ptr(sign), _packed(sign),
+                                         _p(out), block, float(scale), _ptr(post_scale), _dev(out), _stream(stream))
 
 
 def thc_rht_quantize(work, sign, uniform, levels_out, block, scale, lo, delta, levels, stream=None):
@@ -528,8 +580,8 @@ def thc_rht_quantize(work, sign, uniform, levels_out, block, scale, lo, delta, l
     if uniform.numel() < n or levels_out.numel() < n:
         raise RuntimeError("thc_rht_quantize: a buffer is too small")
     _check_sign(sign, n, "thc_rht_quantize")
-    _check(lib().dq_thc_rht_quantize(work.data_ptr(), _ptr(sign), _packed(sign), uniform.data_ptr(), levels_out.data_ptr(), n, block,
-                                     float(scale), lo.data_ptr(), delta.data_ptr(), levels, _dev(work), _stream(stream)))
+    _call(lib().dq_thc_rht_quantize, _p(work), _ptr(sign), _packed(sign), _p(uniform), _p(levels_out), n, block,
+                                     float(scale), _p(lo), _p(delta), levels, _dev(work), _stream(stream))
 
 
 def thc_dequantize_irht(levels_in, sign, out, block, scale, step, lo, stream=None):
@@ -541,5 +593,5 @@ def thc_dequantize_irht(levels_in, sign, out, block, scale, step, lo, stream=Non
     if levels_in.numel() < n:
         raise RuntimeError("thc_dequantize_irht: a buffer is too small")
     _check_sign(sign, n, "thc_dequantize_irht")
-    _check(lib().dq_thc_dequantize_irht(levels_in.data_ptr(), _ptr(sign), _packed(sign), out.data_ptr(), n, block, float(scale),
-                                        step.data_ptr(), lo.data_ptr(), _dev(out), _stream(stream)))
+    _call(lib().dq_thc_dequantize_irht, _p(levels_in), _ptr(sign), _packed(sign), _p(out), n, block, float(scale),
+                                        _p(step), _p(lo), _dev(out), _stream(stream))

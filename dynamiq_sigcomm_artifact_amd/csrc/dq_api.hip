@@ -311,6 +311,22 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
     return finish(dq::launch_group_plan_stats(stats, (float)u, nullptr, nsc, qbits_out, order, work, nullptr, static_cast<hipStream_t>(stream)));
 }
 
+int dq_group_plan_sorted(const void *stats, int64_t nsc, int64_t top_count, int64_t bottom_count, int64_t *qbits_out,
+                         int32_t *order, int32_t *work, int64_t work_ints, int device, dq_stream_t stream)
+{
+    if (!(nsc > 0)) return fail(DQ_ERR_N);
+    if (nsc > 65535) return fail(DQ_ERR_SIZE, "dq_group_plan_sorted handles buckets of up to 65535 superchunks");
+    if (top_count < 0 || bottom_count < 0 || top_count + bottom_count > nsc)
+        return fail(DQ_ERR_SIZE, "top_count and bottom_count must be non-negative and sum to at most nsc");
+    if (!stats || !order || !work) return fail(DQ_ERR_NULL);
+    if (reinterpret_cast<uintptr_t>(stats) & 3) return fail(DQ_ERR_SIZE, "stats must be 4-byte aligned");
+    if (work_ints < 4) return fail(DQ_ERR_SIZE, "work buffer is too small");
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_group_plan_sorted(stats, nsc, top_count, bottom_count, qbits_out, order, work,
+                                               static_cast<hipStream_t>(stream)));
+}
+
 int dq_group_plan_stats_dev_u(const void *stats, const double *u_dev, int64_t nsc, int64_t *qbits_out, int32_t *order,
                               int32_t *work, int64_t work_ints, uint32_t *hist, int64_t hist_ints, int device,
                               dq_stream_t stream)

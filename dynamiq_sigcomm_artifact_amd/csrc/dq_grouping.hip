@@ -258,7 +258,170 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
     }
 }
 
+// ---- fixed-proportion groups: the stable descending sort of the norms in one launch -------------------
+//
+// testbed_evaluation/new_comm_hooks/comm_hooks.py:710-721: sorted = argsort(norms, descending, stable); the first
+// `top` entries of sorted are the 8-bit group, the last `bottom` the 2-bit group, the rest the 4-bit group, each **in
+// sorted order**.  The norms are bf16 values, so the sort key has 16 bits and the position of superchunk i is
+//     G(key_i) + E(i),   G = superchunks with a key that sorts earlier,   E = superchunks j < i with the same key
+// -- a counting sort.  As in plan_one_kernel no workgroup waits for another: the workgroup of tile b (256
+// superchunks) counts the keys of the whole bucket itself, in an LDS histogram of 65536 16-bit counters (128 KB),
+// in two steps: first the superchunks before its tile (the counter of key_i is then the part of E(i) that lies in
+// earlier tiles), then the rest; an in-place exclusive scan of the histogram gives G.  The part of E inside the tile
+// comes from comparing the tile's keys with each other.  nsc <= 65535, so no counter overflows.
+//
+// Sort key (ascending key = descending norm, as torch.sort orders floats): NaN (either sign) first, then +inf ...
+// +0 = -0 ... -inf.
+constexpr int kSortThreads = 1024;
+constexpr int kSortTile = 256;
+constexpr int kSortWords = 32768; // 65536 16-bit counters
+constexpr int kSortBatch = 8;
+
+__device__ __forceinline__ uint32_t descending_key(uint32_t pattern)
+{
+    const uint32_t mag = pattern & 0x7fffu;
+    if (mag > (uint32_t)kMaxPattern) return 0u;             // NaN
+    if (pattern & 0x8000u) return 0x7fffu + mag;            // -0 -> 0x7fff (the key of +0), -inf -> 0xff7f
+    return 0x7fffu - mag;                                   // +inf -> 0x7f, +0 -> 0x7fff
+}
+
+__device__ __forceinline__ void count_keys(const uint32_t *__restrict__ pairs, int begin, int end, uint32_t *hist)
+{
+    for (int i0 = begin; i0 < end; i0 += kSortBatch * kSortThreads) {
+        uint32_t raw[kSortBatch];
+#pragma unroll
+        for (int j = 0; j < kSortBatch; j++) {
+            const int i = i0 + j * kSortThreads + (int)threadIdx.x;
+            if (i < end) raw[j] = pairs[i];
+        }
+#pragma unroll
+        for (int j = 0; j < kSortBatch; j++) {
+            const int i = i0 + j * kSortThreads + (int)threadIdx.x;
+            if (i < end) {
+                const uint32_t k = descending_key(raw[j] >> 16);
+                atomicAdd(&hist[k >> 1], 1u << (16 * (k & 1)));
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kSortThreads) void sorted_plan_kernel(const uint32_t *__restrict__ pairs, int nsc, int top,
+                                                                  int bottom, int64_t *__restrict__ qbits_out,
+                                                                  int32_t *__restrict__ order, int32_t *__restrict__ work)
+{
+    __shared__ __align__(16) uint32_t hist[kSortWords];
+    __shared__ __align__(16) uint16_t tile_key[kSortTile];
+    __shared__ int part_rank[kSortThreads / kSortTile][kSortTile];
+    __shared__ uint32_t wave_sum[kSortThreads / 64];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int nbefore = (int)blockIdx.x * kSortTile;
+    const int e = t & (kSortTile - 1), part = t / kSortTile; // element of the tile, quarter of its predecessors
+    const int own = nbefore + e;
+    const int valid = min(kSortTile, nsc - nbefore);
+
+    uint32_t key = 0;
+    if (e < valid) key = descending_key(pairs[own] >> 16);
+    if (part == 0) tile_key[e] = (uint16_t)key;
+    {
+        uint4 *h4 = reinterpret_cast<uint4 *>(hist);
+        for (int w = t; w < kSortWords / 4; w += kSortThreads) h4[w] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    __syncthreads();
+
+    // superchunks of the tile with the same key and a smaller index: quarter `part` of the candidates
+    {
+        int r = 0;
+        const int j0 = part * (kSortTile / 4);
+        const uint4 *k4 = reinterpret_cast<const uint4 *>(tile_key + j0);
+#pragma unroll
+        for (int q = 0; q < kSortTile / 4 / 8; q++) {
+            const uint4 v = k4[q]; // the same address in every lane: a broadcast
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int h = 0; h < 8; h++) {
+                const int j = j0 + 8 * q + h;
+                const uint32_t kj = (w[h >> 1] >> (16 * (h & 1))) & 0xffffu;
+                r += (kj == key && j < e) ? 1 : 0;
+            }
+        }
+        part_rank[part][e] = r;
+    }
+    count_keys(pairs, 0, nbefore, hist);
+    __syncthreads();
+    int same_before = 0;
+    if (part == 0 && e < valid) {
+        same_before = (int)((hist[key >> 1] >> (16 * (key & 1))) & 0xffffu);
+#pragma unroll
+        for (int q = 0; q < kSortThreads / kSortTile; q++) same_before += part_rank[q][e];
+    }
+    __syncthreads();
+    count_keys(pairs, nbefore, nsc, hist);
+    __syncthreads();
+
+    // exclusive scan of the 65536 counters in place: thread t owns counters [64 t, 64 t + 64)
+    {
+        uint4 *mine = reinterpret_cast<uint4 *>(hist + 32 * t);
+        uint4 v[8];
+        uint32_t sum = 0;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            v[q] = mine[q];
+            const uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+            for (int h = 0; h < 4; h++) sum += (w[h] & 0xffffu) + (w[h] >> 16);
+        }
+        uint32_t incl = sum;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) wave_sum[wave] = incl;
+        __syncthreads();
+        uint32_t run = incl - sum;
+        for (int k = 0; k < wave; k++) run += wave_sum[k];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+            for (int h = 0; h < 4; h++) {
+                const uint32_t lo = w[h] & 0xffffu, hi = w[h] >> 16;
+                w[h] = (run & 0xffffu) | ((run + lo) << 16); // an exclusive prefix is at most nsc - 1 < 65536
+                run += lo + hi;
+            }
+            mine[q] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+    __syncthreads();
+
+    if (part == 0 && e < valid) {
+        const int pos = (int)((hist[key >> 1] >> (16 * (key & 1))) & 0xffffu) + same_before;
+        const int mid_end = nsc - bottom;
+        int region, at;
+        if (pos < top) region = 0, at = pos;
+        else if (pos < mid_end) region = 1, at = pos - top;
+        else region = 2, at = pos - mid_end;
+        order[(int64_t)region * nsc + at] = own;
+        if (qbits_out) qbits_out[own] = region == 0 ? 8 : (region == 1 ? 4 : 2);
+    }
+    if (blockIdx.x == 0 && t == 0) {
+        work[0] = top;
+        work[1] = nsc - top - bottom;
+        work[2] = bottom;
+        work[3] = 0;
+    }
+}
+
 } // namespace
+
+hipError_t launch_group_plan_sorted(const void *stats, int64_t nsc, int64_t top, int64_t bottom, int64_t *qbits_out,
+                                    int32_t *order, int32_t *work, hipStream_t stream)
+{
+    const int ntiles = (int)((nsc + kSortTile - 1) / kSortTile);
+    hipLaunchKernelGGL(sorted_plan_kernel, dim3(ntiles), dim3(kSortThreads), 0, stream,
+                       static_cast<const uint32_t *>(stats), (int)nsc, (int)top, (int)bottom, qbits_out, order, work);
+    return hipGetLastError();
+}
 
 int64_t group_plan_work_ints(int64_t nsc) { return 8 + 4 * ((nsc + kTile - 1) / kTile); }
 

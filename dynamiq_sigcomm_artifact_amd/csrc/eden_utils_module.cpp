@@ -392,6 +392,31 @@ torch::Tensor group_plan_stats(torch::Tensor stats, double u, torch::Tensor orde
     return work.slice(0, 0, 4);
 }
 
+torch::Tensor group_plan_sorted(torch::Tensor stats, int64_t top_count, int64_t bottom_count, torch::Tensor order,
+                                c10::optional<torch::Tensor> qbits_out, uint64_t stream_p = 0)
+{
+    TORCH_CHECK(stats.device().type() == torch::kCUDA, "stats must be a CUDA tensor");
+    TORCH_CHECK(order.device().type() == torch::kCUDA, "order must be a CUDA tensor");
+    TORCH_CHECK(stats.dtype() == torch::kBFloat16, "stats must be torch.bfloat16");
+    TORCH_CHECK(order.dtype() == torch::kInt32, "order must be torch.int32");
+    TORCH_CHECK(stats.is_contiguous() && order.is_contiguous(), "stats and order must be contiguous");
+    const int64_t nsc = stats.numel() / 2;
+    TORCH_CHECK(nsc > 0 && stats.numel() == 2 * nsc, "stats must hold (mean, norm) pairs");
+    TORCH_CHECK(order.numel() >= 3 * nsc, "order has fewer than 3 * nsc entries");
+    int64_t *qptr = nullptr;
+    if (qbits_out.has_value()) {
+        TORCH_CHECK(qbits_out->device().type() == torch::kCUDA && qbits_out->dtype() == torch::kInt64 &&
+                        qbits_out->is_contiguous() && qbits_out->numel() >= nsc,
+                    "qbits_out must be a contiguous torch.int64 CUDA tensor with one entry per superchunk");
+        qptr = qbits_out->data_ptr<int64_t>();
+    }
+    auto work = torch::empty({4}, order.options());
+    check_status(dq_group_plan_sorted(stats.data_ptr(), nsc, top_count, bottom_count, qptr, order.data_ptr<int32_t>(),
+                                      work.data_ptr<int32_t>(), work.numel(), stats.device().index(), as_stream(stream_p)),
+                 "group_plan_sorted");
+    return work;
+}
+
 torch::Tensor group_plan_stats_dev_u(torch::Tensor stats, torch::Tensor u, torch::Tensor order,
                                      c10::optional<torch::Tensor> qbits_out, c10::optional<torch::Tensor> hist,
                                      uint64_t stream_p = 0)
@@ -970,6 +995,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("set_quantization_seed", &set_quantization_seed, "seed of quantization_compression's random stream", py::arg("seed"));
     modul.def("group_plan", &group_plan, "stable partition of superchunk indices by bit width into the three regions of order (8-bit rows from 0, 4-bit from nsc, 2-bit from 2 nsc); returns int32 [4] = counts of 8/4/2/other", py::arg("qbits"), py::arg("order"), py::arg("stream_p") = 0);
     modul.def("group_plan_stats", &group_plan_stats, "bit widths from the reduced bf16 norms and the offset u, and the partition by width, in one call; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
+    modul.def("group_plan_sorted", &group_plan_sorted, "fixed-proportion groups: the first top_count superchunks of the stable descending sort of the norms in the 8-bit region of order, the last bottom_count in the 2-bit region, the rest in the 4-bit region, each in sorted order; returns int32 [4] = counts of 8/4/2/other", py::arg("stats"), py::arg("top_count"), py::arg("bottom_count"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("stream_p") = 0);
     modul.def("group_plan_stats_dev_u", &group_plan_stats_dev_u, "group_plan_stats with the offset u read from a float64 device tensor when the kernels run; hist also gets the bucket's norm patterns", py::arg("stats"), py::arg("u"), py::arg("order"), py::arg("qbits_out") = py::none(), py::arg("hist") = py::none(), py::arg("stream_p") = 0);
     modul.def("bitrate_hist_ints", &bitrate_hist_ints, "int32 entries of the norm-pattern histogram");
     modul.def("norm_histogram", &norm_histogram, "adds the bf16 norm patterns of a bucket's statistics to the histogram", py::arg("stats"), py::arg("hist"), py::arg("stream_p") = 0);

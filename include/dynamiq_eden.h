@@ -168,6 +168,25 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
                         int32_t *order, int32_t *work, int64_t work_ints, int device,
                         dq_stream_t stream);
 
+/* comm_hooks.py:710-721, the fixed-proportion allocation of the non-dynamic
+ * P2P_dynamiQ hook: sorted = argsort(norms, descending=True, stable=True) over
+ * the reduced sums of squares stats[2 * i + 1]; its first top_count entries are
+ * the 8-bit group, its last bottom_count entries the 2-bit group, the rest the
+ * 4-bit group (the caller derives the two counts from the method's fractions,
+ * :713-716, :842-856).  order / work as written by dq_group_plan, except that
+ * every list is in **sorted order** (descending norm, equal norms by ascending
+ * index, NaN before every number, -0 == +0: torch's documented order and what
+ * its CPU sort does; torch's radix sort on a device orders NaNs by payload and
+ * puts a NaN with the sign bit set behind -inf, patterns that sums of squares
+ * computed on a device do not take), which is the order in which the hook
+ * gathers a group and pairs it with rand_pool rows.  qbits_out: int64
+ * [nsc] or NULL.  One launch, no sort passes (the key is a 16-bit pattern:
+ * counting sort in LDS), no host synchronisation.  nsc <= 65535 (DQ_ERR_SIZE
+ * beyond); stats 4-byte aligned. */
+int dq_group_plan_sorted(const void *stats, int64_t nsc, int64_t top_count, int64_t bottom_count,
+                         int64_t *qbits_out, int32_t *order, int32_t *work, int64_t work_ints,
+                         int device, dq_stream_t stream);
+
 /* the same with the offset read from device memory when the kernels run
  * (u_dev: one float64, e.g. result[0] of dq_bitrate_search): a training step
  * then needs no read-back of u at all.  hist (may be NULL; dq_bitrate_hist_ints()

@@ -343,6 +343,35 @@ def dynamic_bitrate_qbits(norms_bf16, u, stride=1):
     return q
 
 
+def argsort_descending_stable(norms_bf16, stride=1):
+    """comm_hooks.py:718 on bf16 bit patterns: int64 order"""
+    _chk(norms_bf16, np.uint16, "norms")
+    count = (norms_bf16.size + stride - 1) // stride
+    order = np.zeros(count, np.int64)
+    f = lib().dqo_argsort_descending_stable
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]
+    f(_p(norms_bf16), stride, count, _p(order))
+    return order
+
+
+def fixed_proportion_groups(norms_bf16, top_count, bottom_count, stride=1):
+    """comm_hooks.py:718-721: the 8-, 4- and 2-bit index lists, each in sorted order"""
+    order = argsort_descending_stable(norms_bf16, stride)
+    n = order.size
+    return order[:top_count], order[top_count:n - bottom_count], order[n - bottom_count:]
+
+
+def quantization(vec, div_factor, tensor_max, seed):
+    """cuda_hadamard.cu:607-627 on a float32 array (returns a new array)"""
+    out = np.ascontiguousarray(vec, np.float32).copy()
+    f = lib().dqo_quantization
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_float, ctypes.c_uint64]
+    f(_p(out), out.size, float(div_factor), float(tensor_max), int(seed))
+    return out
+
+
 # ---- the search for the offset u (comm_hooks.py:48-139) -----------------------------------------------
 # Plain Python around dqo_dynamic_bitrate_qbits: at most 33 evaluations, each one pass of the C rule over the
 # norms.  Pinned by the same search written with the reference's own torch ops on the CPU (the package's

@@ -977,3 +977,74 @@ void dqo_dynamic_bitrate_qbits(const uint16_t *norms_bf16, int64_t stride, int64
         qbits[i] = (int64_t)1 << z;
     }
 }
+
+/* ------------------------------------------------------------------------ */
+/* fixed-proportion groups                                                   */
+/* ------------------------------------------------------------------------ */
+
+/* torch.sort's order on floats, descending: NaN above every number, then the usual >; equal values
+ * (including -0 and +0) are ties */
+static int sorts_before(float a, float b)
+{
+    const int an = a != a, bn = b != b;
+    if (an || bn) return an && !bn;
+    return a > b;
+}
+
+/* testbed_evaluation/new_comm_hooks/comm_hooks.py:718: torch.argsort(norms, descending=True, stable=True)
+ * on the bf16 norms widened to float, as a bottom-up merge sort on the comparison itself (ties keep the
+ * left run's element first = ascending index). */
+void dqo_argsort_descending_stable(const uint16_t *norms_bf16, int64_t stride, int64_t count, int64_t *order)
+{
+    if (count <= 0) return;
+    int64_t *a = order, *b = (int64_t *)malloc(sizeof(int64_t) * (size_t)count);
+    for (int64_t i = 0; i < count; i++) a[i] = i;
+    for (int64_t width = 1; width < count; width *= 2) {
+        for (int64_t lo = 0; lo < count; lo += 2 * width) {
+            const int64_t mid = lo + width < count ? lo + width : count;
+            const int64_t hi = lo + 2 * width < count ? lo + 2 * width : count;
+            int64_t l = lo, r = mid, k = lo;
+            while (l < mid && r < hi) {
+                const float vl = dqo_bf16_to_f32(norms_bf16[a[l] * stride]);
+                const float vr = dqo_bf16_to_f32(norms_bf16[a[r] * stride]);
+                b[k++] = sorts_before(vr, vl) ? a[r++] : a[l++];
+            }
+            while (l < mid) b[k++] = a[l++];
+            while (r < hi) b[k++] = a[r++];
+        }
+        int64_t *t = a; a = b; b = t;
+    }
+    if (a != order) {
+        memcpy(order, a, sizeof(int64_t) * (size_t)count);
+        free(a);
+    } else {
+        free(b);
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* quantization_compression                                                  */
+/* ------------------------------------------------------------------------ */
+
+/* csrc/cuda_hadamard.cu:607-627: t = clamp(v / div_factor, +-tensor_max); v = floor(t) + (u < t - floor(t)).
+ * The reference draws u from curand states that it never initialises (:669-686), so its stream is
+ * undefined ("parity unpinned"); the library defines u for element e as the top 24 bits of word e % 4 of
+ * the Philox4x32-10 block with key = seed and counter = (e / 4, 0), times 2^-24. */
+void dqo_quantization(float *vec, int64_t n, float div_factor, float tensor_max, uint64_t seed)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    for (int64_t g = 0; g * 4 < n; g++) {
+        const uint32_t ctr[4] = {(uint32_t)g, (uint32_t)((uint64_t)g >> 32), 0u, 0u};
+        uint32_t w[4];
+        dqo_philox4x32_10(ctr, key, w);
+        for (int k = 0; k < 4 && g * 4 + k < n; k++) {
+            float t = vec[g * 4 + k] / div_factor;
+            t = t < tensor_max ? t : tensor_max;
+            t = t > -tensor_max ? t : -tensor_max;
+            const float fl = floorf(t);
+            const float prob = t - fl;
+            const float u = (float)(w[k] >> 8) * 5.9604644775390625e-08f;
+            vec[g * 4 + k] = fl + (u < prob ? 1.0f : 0.0f);
+        }
+    }
+}

@@ -156,6 +156,15 @@ void dqo_thc_dequantize(const uint16_t *levels_bf16, float *out, int64_t n, floa
 void dqo_dynamic_bitrate_qbits(const uint16_t *norms_bf16, int64_t stride, int64_t count,
                                double u, int64_t *qbits);
 
+/* testbed_evaluation/new_comm_hooks/comm_hooks.py:718: torch.argsort(norms, descending=True,
+ * stable=True) of bf16 norms (NaN first, ties by ascending index); order: int64 [count]. */
+void dqo_argsort_descending_stable(const uint16_t *norms_bf16, int64_t stride, int64_t count,
+                                   int64_t *order);
+
+/* csrc/cuda_hadamard.cu:607-627 with the library's Philox stream in place of the reference's
+ * uninitialised curand states ("parity unpinned" for the stream, the arithmetic is the reference's). */
+void dqo_quantization(float *vec, int64_t n, float div_factor, float tensor_max, uint64_t seed);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,152 @@
+"""dq_group_plan_sorted (the fixed-proportion allocation of comm_hooks.py:710-721 as one launch) against
+torch.argsort(descending=True, stable=True) on the device and against the oracle; the groups feed the row-list
+codec, whose bytes are compared with the gather -> codec sequence the hook runs."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import to_bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+EXOTIC = "NaN of either sign, -0"
+
+
+def _stats(norms):
+    st = torch.zeros((norms.numel(), 2), dtype=torch.bfloat16, device=DEV)
+    st[:, 1] = norms.to(DEV)
+    st[:, 0] = 0.25
+    return st
+
+
+def _norm_sets():
+    g = torch.Generator().manual_seed(21)
+    sets = {
+        "bucket 25600 lognormal": torch.exp(torch.randn(25600, generator=g) * 3 - 8),
+        "tie-heavy 25600 (12 values)": torch.exp2(torch.randint(-6, 6, (25600,), generator=g).float()),
+        "all equal 4097": torch.full((4097,), 0.125),
+        "all zero 25600": torch.zeros(25600),
+        "one": torch.tensor([3.0]),
+        "255": torch.exp(torch.randn(255, generator=g)),
+        "256": torch.exp(torch.randn(256, generator=g)),
+        "257": torch.exp(torch.randn(257, generator=g)),
+        "65535 narrow": torch.rand(65535, generator=g) * 1e-4 + 2e-4,
+    }
+    sp = torch.exp(torch.randn(30011, generator=g) * 4 - 5)
+    sp[::7] = 0.0
+    sp[3::11] = -0.0
+    sp[1::97] = float("nan")
+    sp[2::131] = -1.0
+    sp[5::173] = float("inf")
+    sp[6::191] = float("-inf")
+    sets["zeros, NaN, infinities, negatives"] = sp
+    sets = {k: v.to(torch.bfloat16) for k, v in sets.items()}
+    # torch documents NaN as the greatest value and equal values as ties; its CPU sort and its small device sort behave
+    # so.  Its large device sort is a radix sort on the bit pattern: NaNs order by payload, a NaN with the sign bit set
+    # (what the CPU's float -> bf16 conversion writes: 0xffff) goes behind -inf, and -0 may be told from +0.  The library
+    # follows the documented order.  The comparison with torch on the device therefore uses one NaN pattern (0x7fc0,
+    # what device arithmetic produces) and +0 only; NaNs of either sign and payload and -0 are compared with the oracle
+    # (EXOTIC), which is pinned by torch's CPU sort.
+    bits = sets["zeros, NaN, infinities, negatives"].view(torch.int16)
+    exotic = bits.clone()
+    bits[1::97] = 0x7fc0
+    bits[3::11] = 0
+    exotic[1::97] = torch.tensor(0xffff - 0x10000, dtype=torch.int16)
+    exotic[98::194] = 0x7fff
+    exotic[1::291] = 0x7fc0
+    sets[EXOTIC] = exotic.view(torch.bfloat16)
+    return sets
+
+
+@pytest.mark.parametrize("name", sorted(_norm_sets()))
+@pytest.mark.parametrize("method", ["x_5bit", "x_3bit", "x_4bit_fixed", "x_7bit"])
+def test_sorted_plan_matches_argsort(capi, oracle, name, method):
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    norms = _norm_sets()[name]
+    nsc = norms.numel()
+    st = _stats(norms)
+    thr = B.fixed_proportion_thresholds(method)
+    top, mid, bottom = B.fixed_proportion_counts(nsc, thr)
+    order = torch.full((3 * nsc,), -7, dtype=torch.int32, device=DEV)
+    work = torch.full((capi.group_plan_work_ints(nsc),), -7, dtype=torch.int32, device=DEV)
+    qb = torch.zeros(nsc, dtype=torch.int64, device=DEV)
+    capi.group_plan_sorted(st, top, bottom, order, work, qbits_out=qb)
+    o = order.cpu().numpy()
+    assert work[:4].tolist() == [top, mid, bottom, 0]
+    # the reference's own ops on the device (comm_hooks.py:710-721)
+    g8, g4, g2 = B.fixed_proportion_groups(st[:, 1], thr)
+    # and the oracle
+    o8, o4, o2 = oracle.fixed_proportion_groups(to_bits(st.reshape(-1))[1:], top, bottom, stride=2)
+    for base, cnt, g, og in ((0, top, g8, o8), (nsc, mid, g4, o4), (2 * nsc, bottom, g2, o2)):
+        assert (o[base:base + cnt] == og).all(), (name, method, base)
+        if name != EXOTIC:
+            assert (o[base:base + cnt] == g.cpu().numpy()).all(), (name, method, base)
+        assert (o[base + cnt:base + nsc] == -7).all()                      # nothing written beyond a list
+    want_q = np.zeros(nsc, np.int64)
+    want_q[o8], want_q[o4], want_q[o2] = 8, 4, 2
+    assert (qb.cpu().numpy() == want_q).all()
+
+
+def test_sorted_plan_wrapper_and_module(capi, eden_utils):
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    g = torch.Generator().manual_seed(5)
+    st = _stats(torch.exp(torch.randn(1000, generator=g)).to(torch.bfloat16))
+    thr = B.fixed_proportion_thresholds("dynamiQ_mee_5bit")
+    order, work, counts = B.fixed_proportion_plan(st, thr)
+    assert counts == (350, 450, 200) and work[:3].tolist() == [350, 450, 200]
+    order2 = torch.zeros_like(order)
+    w2 = eden_utils.group_plan_sorted(st, 350, 200, order2)
+    assert w2.tolist() == [350, 450, 200, 0]
+    for base, cnt in ((0, 350), (1000, 450), (2000, 200)):
+        assert torch.equal(order[base:base + cnt], order2[base:base + cnt])
+    srt = torch.argsort(st[:, 1].float(), descending=True, stable=True)
+    assert torch.equal(order[:350].long(), srt[:350])
+
+
+def test_sorted_plan_validation(capi):
+    st = _stats(torch.ones(70000).to(torch.bfloat16))
+    order = torch.zeros(3 * 70000, dtype=torch.int32, device=DEV)
+    work = torch.zeros(64, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="65535"):
+        capi.group_plan_sorted(st, 10, 10, order, work)
+    with pytest.raises(RuntimeError, match="top_count"):
+        capi.group_plan_sorted(st[:100], 60, 60, order, work)
+    with pytest.raises(RuntimeError, match="4-byte aligned"):
+        capi.group_plan_sorted(st.reshape(-1)[1:201].reshape(100, 2), 10, 10, order, work)
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_groups_feed_the_row_codec(capi, oracle, strategy):
+    """one bucket end to end as the fixed-proportion hook runs it (one rank): groups in sorted order -> index_select ->
+    compress (rand rows paired with the position in the group) -> decompress -> index_copy_, against the row-list
+    kernels fed by the device plan"""
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    nsc = 1200
+    g = torch.Generator().manual_seed(8)
+    scale = torch.exp(torch.randn(nsc, 1, generator=g) * 2 - 4)
+    x = (torch.randn(nsc, 256, generator=g) * scale).to(torch.bfloat16).to(DEV)
+    st = _stats((x.float() ** 2).sum(1).to(torch.bfloat16))
+    thr = B.fixed_proportion_thresholds("m_5bit")
+    order, work, counts = B.fixed_proportion_plan(st, thr)
+    groups = B.fixed_proportion_groups(st[:, 1], thr)
+    out = torch.zeros_like(x)
+    want = torch.zeros_like(x)
+    for width, base, cnt, idx in ((8, 0, counts[0], groups[0]), (4, nsc, counts[1], groups[1]), (2, 2 * nsc, counts[2], groups[2])):
+        rand = torch.rand(cnt * 256, generator=g).to(torch.bfloat16).to(DEV)
+        nbytes = capi.required_bytes(cnt * 256, width, 16, strategy)
+        # the hook's sequence, through the oracle
+        gathered = torch.index_select(x, 0, idx).reshape(-1)
+        packed_o = oracle.scaling_compress(to_bits(gathered), to_bits(rand), cnt * 256, width, 16, strategy, 1)
+        dec = np.zeros(cnt * 256, np.uint16)
+        oracle.scaling_decompress(packed_o, dec, cnt * 256, width, 16, strategy, 1)
+        want.index_copy_(0, idx, torch.from_numpy(dec.view(np.int16)).view(torch.bfloat16).reshape(cnt, 256).to(DEV))
+        # the library: no gather, rows from the plan
+        rows = order[base:base + cnt]
+        packed = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+        capi.scaling_compress_rows(x.reshape(-1), rows, packed, rand, cnt, width, strategy)
+        assert (packed.cpu().numpy() == packed_o[:nbytes]).all(), width
+        capi.scaling_decompress_rows(packed, out.reshape(-1), rows, None, nsc * 256, cnt, width, strategy)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))

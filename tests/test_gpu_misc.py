@@ -224,3 +224,28 @@ def test_quantization_compression(eden_utils):
     q3 = v.clone()
     eden_utils.quantization_compression(q3, 0.5, 10.0)
     assert not torch.equal(q, q3)
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 1021, 1 << 16])
+def test_quantization_matches_oracle(capi, oracle, n):
+    """dq_quantization against the oracle's restatement of cuda_hadamard.cu:607-627 on the same Philox stream"""
+    g = torch.Generator().manual_seed(n)
+    v = torch.rand(n, generator=g) * 30.0 - 15.0
+    if n > 8:
+        v[:8] = torch.tensor([0.0, 1.0, -1.0, 2.5, -2.5, 1e9, -1e9, float("inf")])
+    for div, tmax, seed in ((0.5, 10.0, 123), (0.37, 100.0, 0xFEDCBA9876543210), (3.0, 0.5, 0)):
+        q = v.clone().to(DEV)
+        capi.quantization(q, div, tmax, seed)
+        want = oracle.quantization(v.numpy(), div, tmax, seed)
+        assert (q.cpu().numpy().view(np.uint32) == want.view(np.uint32)).all(), (n, div)
+
+
+def test_quantization_compression_module_stream(eden_utils, oracle):
+    """the module function draws seed, seed + golden ratio, ... from set_quantization_seed"""
+    v = torch.rand(4096) * 12.0 - 6.0
+    eden_utils.set_quantization_seed(123)
+    for k in range(2):
+        q = v.clone().to(DEV)
+        eden_utils.quantization_compression(q, 0.5, 10.0)
+        want = oracle.quantization(v.numpy(), 0.5, 10.0, (123 + k * 0x9E3779B97F4A7C15) & (2 ** 64 - 1))
+        assert (q.cpu().numpy() == want).all()

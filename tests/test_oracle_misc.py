@@ -318,3 +318,32 @@ def test_philox_known_answers(oracle):
         want = (np.frombuffer(w.astype("<u4").tobytes(), np.uint8) | 1).astype(np.float32) / 256
         got = u[16 * chunk: 16 * chunk + 16]
         assert (got == want[:got.size]).all()
+
+
+# ---- quantization_compression (cuda_hadamard.cu:607-627) ------------------------------------------------
+
+def test_quantization_oracle_closed_forms(oracle):
+    """integers stay, values land on floor or floor + 1 of the clamped quotient, the direction is decided by the
+    Philox word the documentation names (re-derived here from the known-answer-pinned block function)"""
+    n, seed = 1003, 0x1234567890ABCDEF
+    rng = np.random.default_rng(5)
+    v = (rng.random(n, dtype=np.float32) * 30.0 - 15.0).astype(np.float32)
+    v[:8] = [0.0, 1.0, -1.0, 2.5, -2.5, 1e9, -1e9, 0.5]
+    div, tmax = np.float32(0.5), np.float32(10.0)
+    got = oracle.quantization(v, div, tmax, seed)
+    t = np.clip((v / div).astype(np.float32), -tmax, tmax)
+    fl = np.floor(t)
+    u = np.zeros(n, np.float32)
+    for g in range((n + 3) // 4):
+        w = oracle.philox4x32_10([g & 0xffffffff, g >> 32, 0, 0], [seed & 0xffffffff, seed >> 32])
+        for k in range(min(4, n - 4 * g)):
+            u[4 * g + k] = np.float32(int(w[k]) >> 8) * np.float32(2.0 ** -24)
+    want = fl + (u < (t - fl)).astype(np.float32)
+    assert (got == want).all()
+    assert got[0] == 0.0 and got[1] == 2.0 and got[2] == -2.0 and got[3] == 5.0 and got[4] == -5.0
+    assert got[5] == 10.0 and got[6] == -10.0 and got[7] == 1.0            # clamped, and exact quotients never move
+    # unbiased: the mean rounding error vanishes
+    big = (rng.random(1 << 18, dtype=np.float32) * 8.0 - 4.0).astype(np.float32)
+    q = oracle.quantization(big, np.float32(0.37), np.float32(100.0), 7)
+    assert abs(float((q - big / np.float32(0.37)).mean())) < 5e-3
+    assert not (oracle.quantization(big, 0.37, 100.0, 8) == q).all()
