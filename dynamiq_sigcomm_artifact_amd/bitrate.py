@@ -187,8 +187,8 @@ class NormHistogram(object):
 
     def _search(self, mode, prev_u, target_avg_bits, stream):
         self.launch_search(mode, prev_u, target_avg_bits, stream)
-        if hasattr(stream, "synchronize"):
-            stream.synchronize()            # tolist() below only waits for torch's current stream
+        # tolist() only waits for torch's current stream: wait for the one the search ran on
+        self._capi.torch_stream(stream, self.result.device).synchronize()
         u, avg, delta, _ = self.result.tolist()
         return u, avg, delta
 

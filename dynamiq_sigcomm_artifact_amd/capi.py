@@ -225,6 +225,18 @@ def _stream(stream):
     return ctypes.c_void_p(int(stream))
 
 
+def torch_stream(stream, device=None):
+    """the torch.cuda.Stream object for what the wrappers accept as `stream` (None, a raw handle, a torch stream), so
+    that torch ops, waits and read-backs can be put on the stream the kernels run on"""
+    if stream is None:
+        return torch.cuda.current_stream(device)
+    if hasattr(stream, "cuda_stream"):
+        return stream
+    if int(stream) == 0:
+        return torch.cuda.default_stream(device)
+    return torch.cuda.ExternalStream(int(stream), device=device)
+
+
 def required_bytes(n, nbits, chunk_size, strategy):
     return int(lib().dq_scaling_required_bytes(n, nbits, chunk_size, strategy))
 

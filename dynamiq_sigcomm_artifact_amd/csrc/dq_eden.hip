@@ -7,7 +7,7 @@
 //   sumsq   tile b = elements [4096 b, 4096 b + 4096): thread t adds v^2 of elements t + 256 k (k ascending)
 //           in double, the 256 sums are halved (stride 128 .. 1) -> work[b]
 //   norm    one workgroup folds work[] the same way -> sumsq (double); norm = sqrtf((float)sumsq)
-//   bins    x = (v * (float)sqrt(n)) / norm; bin = number of boundaries < x (torch.bucketize, right=False);
+//   bins    x = (v * (float)sqrt(n)) / norm; bin = number of boundaries b with !(b >= x) (torch.bucketize, right=False: NaN -> last bin);
 //           bit plane p of 32 consecutive bins -> packed[p * n/32 + w]; the products centroid[bin] * v are
 //           summed in double, thread t adding elements 16 t + k of the tile (k ascending), then halved -> work[b]
 //   scale   dot = fold(work[]); scale = (norm * norm) / (float)dot
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
 #pragma unroll
         for (int k = 0; k < kEdenPerThread; k++) {
             const float b = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(tree) + node[k]);
-            node[k] = 2 * node[k] + (b < x[k] ? 4 : 0);
+            node[k] = 2 * node[k] + (!(b >= x[k]) ? 4 : 0); // torch's lower bound: a NaN goes right at every level
         }
     }
     // the product of two floats is exact in double, so the fused multiply-add rounds like multiply, then add;

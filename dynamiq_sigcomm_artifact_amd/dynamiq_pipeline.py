@@ -160,17 +160,20 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         work["recv"] = [torch.zeros(cap, dtype=torch.uint8, device=dev) for _ in range(W if W > 1 else 0)]
     stats, mean, order, plan = work["stats"], work["mean"], work["order"], work["plan"]
     send, recv = work["send"], work["recv"]
-    if stream is None:
-        stream = torch.cuda.current_stream().cuda_stream     # looked up once per bucket, not once per launch
+    # one stream for the kernels and for the torch ops between them (the statistics sum, the exchange copies):
+    # resolved once per bucket, not once per launch
+    torch_stream = capi.torch_stream(stream, dev)
+    stream = torch_stream.cuda_stream
     for r in range(W):
         capi.superchunk_stats(rank_vecs[r], stats[r], mean[r], n, W, stream=stream)
     if W == 1:
         total = stats[0]
     else:
         total = work["total"]
-        total.copy_(stats[0])
-        for r in range(1, W):
-            total.add_(stats[r])
+        with torch.cuda.stream(torch_stream):
+            total.copy_(stats[0])
+            for r in range(1, W):
+                total.add_(stats[r])
     # with u on the device the histogram is filled by a few more workgroups of the plan launch, otherwise by a launch of its own
     capi.group_plan_stats(total, u if isinstance(u, torch.Tensor) else float(u), None, order, plan, stream=stream,
                           hist=None if norm_histogram is None else norm_histogram.hist)
@@ -192,8 +195,9 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         return outs, total, plan[:4]
 
     def exchange(src_bufs, dst_bufs):
-        for r in range(W):
-            dst_bufs[(r + 1) % W].copy_(src_bufs[r])
+        with torch.cuda.stream(torch_stream):
+            for r in range(W):
+                dst_bufs[(r + 1) % W].copy_(src_bufs[r])
 
     # reduce-scatter: W - 1 steps, then the owner's step; all-gather of the owners' streams
     for step in range(W - 1):

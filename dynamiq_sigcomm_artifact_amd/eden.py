@@ -71,7 +71,7 @@ class Eden(object):
     # ---- srrcomp.py:251-291 ----
     def compress(self, vec, nbits, seed):
         vec_type = vec.dtype
-        vec = vec.to(torch.float32).clone()
+        vec = vec.to(self.device, torch.float32).clone()        # the kernels only take buffers of self.device
 
         def low_po2(n):
             return 2 ** int(np.log2(n)) if n else 0
@@ -144,7 +144,7 @@ class Eden(object):
         centroids, _ = self._tables(nbits)
         vec = torch.empty(n, dtype=torch.float32, device=self.device)
         if num_hadamard == 0:
-            capi.eden_dequantize(packed_bins.to(torch.int32), n, centroids, nbits, vec)
+            capi.eden_dequantize(packed_bins.to(self.device, torch.int32), n, centroids, nbits, vec)
             return (scale * vec)[:orig_dim].to(vec_type)
         # the dequantiser rides on the first pass of the first rotation, the product with the scale on the last pass of
         # the last one: same bits as eden_dequantize, the rotations and `scale * vec`
@@ -155,7 +155,7 @@ class Eden(object):
             self._rand_diag(diag, n, seed + num_hadamard - 1 - i)
             last = scale32 if i == num_hadamard - 1 else None
             if i == 0:
-                capi.eden_dequantize_irht(packed_bins.to(torch.int32), n, centroids, nbits, diag, vec, n, self._inv_sqrt(n),
+                capi.eden_dequantize_irht(packed_bins.to(self.device, torch.int32), n, centroids, nbits, diag, vec, n, self._inv_sqrt(n),
                                           post_scale=last)
             elif last is None:
                 capi.rht_blocked(vec, diag, n, self._inv_sqrt(n), True)

@@ -320,7 +320,8 @@ int64_t dq_eden_work_doubles(int64_t n);
  * vec: float32 [n], n a positive multiple of 32 (the caller pads, :300-309).
  * boundaries: float32 [2^nbits - 1] ascending, centroids: float32 [2^nbits]
  * (Eden.boundaries[nbits], Eden.centroids[nbits]); nbits 1..8.
- *   bin_i   = #{ boundaries < (vec_i * (float)sqrt(n)) / ||vec|| }   (torch.bucketize, right=False)
+ *   bin_i   = #{ b in boundaries : !(b >= x_i) },  x_i = (vec_i * (float)sqrt(n)) / ||vec||
+ *             (torch.bucketize, right=False; a NaN x_i -- an all-zero vec -- lands in the last bin)
  *   packed  = bit planes of the bins, uint32 [n / 32 * nbits]
  *   result  = float32 [4] on the device: sum of squares, <centroids[bin], vec>,
  *             scale = ||vec||^2 / <centroids[bin], vec>, ||vec||

@@ -899,7 +899,8 @@ static double term_dot(int64_t i, void *c)
 }
 
 /* srrcomp.py:356-361: bins = bucketize(vec * sqrt(n) / ||vec||, boundaries) with right=False, i.e. the
- * number of boundaries strictly below the value; scale = ||vec||^2 / <centroids[bins], vec>.
+ * number of boundaries strictly below the value (a NaN value, 0/0 of an all-zero slice, lands in the last bin as in
+ * torch's lower-bound search); scale = ||vec||^2 / <centroids[bins], vec>.
  * result = {sum of squares, dot, scale, norm}. */
 void dqo_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids, int nbits,
                        int32_t *bins, float *result)
@@ -912,7 +913,7 @@ void dqo_eden_quantize(const float *vec, int64_t n, const float *boundaries, con
     for (int64_t i = 0; i < n; i++) {
         const float x = (vec[i] * sqrt_n) / norm;
         int b = 0;
-        while (b < nb && boundaries[b] < x) b++;
+        while (b < nb && !(boundaries[b] >= x)) b++; /* torch's lower bound: NaN passes every boundary */
         bins[i] = b;
     }
     const float dot = (float)tiled_sum(n, term_dot, &ctx, 1);

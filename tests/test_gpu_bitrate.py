@@ -221,3 +221,30 @@ def test_plan_launch_fills_the_histogram(capi, nsc):
     again = torch.full_like(got, 5)
     capi.group_plan_stats(stats, 7.3, None, order_b, work_b, hist=again)
     assert torch.equal(again, want)
+
+
+def test_search_and_pipeline_on_a_side_stream(capi):
+    """the search's read-back waits for the stream it was launched on, and the pipeline puts its torch ops (statistics
+    sum, exchange copies) on the stream of its kernels: a side stream given as a torch stream or as a raw handle gives
+    the results of the current stream"""
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import dynamic_bitrate_allreduce_single_pass
+    g = torch.Generator().manual_seed(17)
+    norms = torch.exp(torch.randn(25600, generator=g) * 3 - 8).to(torch.bfloat16)
+    st = _stats(norms)
+    h = B.NormHistogram(DEV)
+    h.add(st)
+    want = h.binary_search_u(4.375)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for s in (side, side.cuda_stream):
+        h.add(st, stream=s)
+        assert h.binary_search_u(4.375, stream=s) == want
+    vecs = [(torch.randn(256 * 300 + 17, generator=g) * 1e-2).to(torch.bfloat16).to(DEV) for _ in range(3)]
+    ref, total, counts = dynamic_bitrate_allreduce_single_pass(vecs, want[0], seed=3)
+    torch.cuda.synchronize()
+    outs, total2, counts2 = dynamic_bitrate_allreduce_single_pass(vecs, want[0], seed=3, stream=side)
+    side.synchronize()
+    assert counts.tolist() == counts2.tolist()
+    for a, b in zip(ref, outs):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))

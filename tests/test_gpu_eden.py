@@ -40,7 +40,7 @@ def test_eden_quantize_bit_exact(capi, oracle, nbits, n):
 
 
 def test_eden_quantize_degenerate_norms(capi, oracle):
-    """all zeros (0/0 -> NaN compares false with every boundary: bin 0) and a norm outside the fast-division range"""
+    """all zeros (0/0 -> NaN: torch.bucketize's lower bound sends it to the last bin) and a norm outside the fast-division range"""
     cen, bnd = _tables(4)
     for x in (torch.zeros(64), torch.full((64,), 1e-30), torch.full((64,), 3e18) * torch.randn(64).sign()):
         packed = torch.zeros(8, dtype=torch.int32, device=DEV)

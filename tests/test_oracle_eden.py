@@ -131,3 +131,17 @@ def test_thc_oracle_closed_forms(oracle):
     assert abs(lev.mean() - 17.3) < 0.01
     back = oracle.thc_dequantize(oracle.thc_quantize(v[:4], u0[:4], lo, delta, levels), np.float32(delta), np.float32(lo))
     assert np.allclose(back, [-1, -1, 1, 1], atol=1e-6)
+
+
+def test_nan_goes_to_the_last_bin_like_torch_bucketize(oracle):
+    """an all-zero slice: 0/0 = NaN for every element; torch.bucketize(right=False) is a lower-bound search whose
+    comparison `!(boundary >= x)` holds for NaN at every step, so every bin is the last one"""
+    import torch
+    bnd = np.array([-1.0, 0.0, 1.0], np.float32)
+    cen = np.array([-1.5, -0.5, 0.5, 1.5], np.float32)
+    bins, res = oracle.eden_quantize(np.zeros(64, np.float32), bnd, cen, 2)
+    want = torch.bucketize(torch.full((64,), float("nan")), torch.from_numpy(bnd)).numpy()
+    assert (bins == want).all() and (bins == 3).all()
+    x = np.array([-2.0, -1.0, -0.5, 0.0, 0.5, 1.0, 2.0, np.nan] * 4, np.float32)
+    got = np.array([sum(1 for b in bnd if not (b >= v)) for v in x])
+    assert (got == torch.bucketize(torch.from_numpy(x), torch.from_numpy(bnd)).numpy()).all()
