@@ -253,6 +253,18 @@ template <int NBITS> __device__ __forceinline__ void words_put(uint32_t (&w)[Rec
     if ((bit & 31) + NBITS > 32) w[(bit >> 5) + 1] |= code >> (32 - (bit & 31));
 }
 
+// replaces the code of element i
+template <int NBITS> __device__ __forceinline__ void words_set(uint32_t (&w)[Rec<NBITS>::WORDS], int i, uint32_t code)
+{
+    constexpr uint32_t kMask = (1u << NBITS) - 1u;
+    const int bit = i * NBITS;
+    w[bit >> 5] = (w[bit >> 5] & ~(kMask << (bit & 31))) | (code << (bit & 31));
+    if ((bit & 31) + NBITS > 32) {
+        const int done = 32 - (bit & 31);
+        w[(bit >> 5) + 1] = (w[(bit >> 5) + 1] & ~(kMask >> done)) | (code >> done);
+    }
+}
+
 template <int NBITS> __device__ __forceinline__ uint32_t words_get(const uint32_t (&w)[Rec<NBITS>::WORDS], int i)
 {
     const int bit = i * NBITS;
