@@ -179,6 +179,43 @@ def test_special_values(capi, oracle, dt, strategy):
         _roundtrip_nan_safe(capi, oracle, dt, n, nbits, 16, strategy, src, rnd, "special b=%d" % nbits)
 
 
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_random_values_on_the_rounding_boundary(capi, oracle, nbits, strategy):
+    """The kernels decide most codes from a cheap estimate of the coordinate and redo an element with the reference's
+    exact chain when coordinate - random value comes close to an integer.  Here every random value is the fractional
+    part of its element's coordinate (to float32 accuracy, and one or two float32 steps beside it), so every element
+    sits on that boundary: bytes must still be the oracle's."""
+    from helpers import unpack_stream
+    nsc = 40
+    n = nsc * 256
+    g = torch.Generator().manual_seed(900 + 10 * nbits + strategy)
+    scale = torch.exp(torch.randn(nsc, 1, generator=g) * 2.0 - 6.0)
+    src = (torch.randn(nsc, 256, generator=g) * scale).reshape(-1)
+    src[5::97] = 0.0
+    # the quantisation steps the oracle uses: from the records of a first pass with any random values
+    enc = oracle.scaling_compress(src.numpy(), np.full(n, 0.5, np.float32), n, nbits, 16, strategy, F32)
+    _, (q, unit) = unpack_stream(enc, n, nbits, 16, strategy)
+    step = q.astype(np.float64).repeat(16) * bits_to_f32(unit, BF16).astype(np.float64).repeat(256)
+    x = src.numpy().astype(np.float64) / step
+    if strategy == 3:
+        _, params = capi.mee_lookup_table(nbits)
+        c, l2b = (float(v) for v in params[[1, 3]].view(np.float16).astype(np.float64))
+        x = np.sign(x) * np.log2(np.abs(x) / c + 1.0) / l2b
+    frac = (x - np.floor(x)).astype(np.float32)
+    for shift in (0, 1, -1, 2, -2):
+        rnd = frac.copy()
+        for _ in range(abs(shift)):
+            rnd = np.nextafter(rnd, np.float32(2.0 if shift > 0 else -1.0))
+        rnd = np.clip(rnd, 0.0, 1.0).astype(np.float32)
+        tag = "boundary b=%d s=%d shift=%d" % (nbits, strategy, shift)
+        _roundtrip(capi, oracle, F32, n, nbits, 16, strategy, src, torch.from_numpy(rnd), tag)
+        # the fused ring step sees the same situation through its accumulated input
+        if shift == 0:
+            inp = torch.zeros(n)
+            _dec_comp(capi, oracle, F32, n, nbits, 16, strategy, src, inp, torch.from_numpy(rnd), torch.from_numpy(rnd), tag)
+
+
 def _wide_source(n, tdt, seed):
     """random magnitudes over the whole exponent range of the type, plus zeros, infinities, NaN and
     values the type cannot hold without rounding to the extremes"""

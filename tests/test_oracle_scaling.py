@@ -37,46 +37,83 @@ def test_check_common(oracle, args, code):
 
 # ---- special cases with known answers ---------------------------------------------------
 
-@pytest.mark.parametrize("nbits", [2, 4, 8])
-def test_all_zero_superchunk(oracle, nbits):
+def _elems(values, dt):
+    """float values -> the oracle's storage for element type dt"""
+    return bf16_of(values) if dt == BF16 else np.asarray(values, np.float32)
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+def test_all_zero_superchunk(oracle, nbits, dt):
     n, R = 256, (1 << (nbits - 1)) - 1
-    src = np.zeros(n, np.uint16)
-    rnd = bf16_of(np.linspace(0, 0.99, n))
-    enc = oracle.scaling_compress(src, rnd, n, nbits, 16, 2, BF16)
+    src = _elems(np.zeros(n), dt)
+    rnd = _elems(np.linspace(0, 0.99, n), dt)
+    enc = oracle.scaling_compress(src, rnd, n, nbits, 16, 2, dt)
     codes, (q, unit) = unpack_stream(enc, n, nbits, 16, 2)
     assert (codes == R).all()                      # ceil(0 - r) = 0 for r < 1
     assert (q == 255).all()                        # all chunk scales equal the maximum
     want_unit = bf16_of([np.float32(np.float32(0.0) / np.float32(R) + np.float32(1e-7)) / np.float32(255.0)])
     assert unit[0] == want_unit[0]
     # r == 1.0 exactly (bf16-rounded torch.rand can produce it): floor - 1
-    rnd1 = bf16_of(np.ones(n))
-    codes1, _ = unpack_stream(oracle.scaling_compress(src, rnd1, n, nbits, 16, 2, BF16), n, nbits, 16, 2)
+    rnd1 = _elems(np.ones(n), dt)
+    codes1, _ = unpack_stream(oracle.scaling_compress(src, rnd1, n, nbits, 16, 2, dt), n, nbits, 16, 2)
     assert (codes1 == max(R - 1, 0)).all()
-    # flat layout stores bf16(1e-7) as the scale
-    encf = oracle.scaling_compress(src, rnd, n, nbits, 16, 0, BF16)
-    _, (scale, _) = unpack_stream(encf, n, nbits, 16, 0)
-    assert (scale == bf16_of([1e-7])[0]).all()
+    # MEE: the same codes (the lattice coordinate of 0 is 0), unit from the lattice maximum instead of R
+    codes_m, (q_m, unit_m) = unpack_stream(oracle.scaling_compress(src, rnd, n, nbits, 16, 3, dt), n, nbits, 16, 3)
+    assert (codes_m == R).all() and (q_m == 255).all() and unit_m[0] == want_unit[0]
+    # flat layout stores T(1e-7) as the scale: 2 bytes of bf16, or the first two... only for 2-byte types
+    if dt == BF16:
+        encf = oracle.scaling_compress(src, rnd, n, nbits, 16, 0, dt)
+        _, (scale, _) = unpack_stream(encf, n, nbits, 16, 0)
+        assert (scale == bf16_of([1e-7])[0]).all()
 
 
-@pytest.mark.parametrize("nbits", [2, 4, 8])
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [0, 2])
-def test_single_extreme_element(oracle, nbits, strategy):
+def test_single_extreme_element(oracle, nbits, strategy, dt):
     """one +-max element in an otherwise zero superchunk -> code 2R / 0 there, R elsewhere"""
+    if dt == F32 and strategy == 0:
+        pytest.skip("the flat layout with float32 elements stores a 4-byte scale: covered by the tile16 tests")
     n, R = 256, (1 << (nbits - 1)) - 1
     for pos, sign in ((0, 1.0), (37, -1.0), (255, 1.0)):
         v = np.zeros(n, np.float32)
         v[pos] = sign * 0.5
-        enc = oracle.scaling_compress(bf16_of(v), bf16_of(np.full(n, 0.5)), n, nbits, 16, strategy, BF16)
+        enc = oracle.scaling_compress(_elems(v, dt), _elems(np.full(n, 0.5), dt), n, nbits, 16, strategy, dt)
         codes, _ = unpack_stream(enc, n, nbits, 16, strategy)
         want = np.full(n, R)
         # |x| = 0.5/scale is just below R (scale carries +1e-7 and is rounded up); rand 0.5 decides
         want[pos] = codes[pos]
         assert (codes == want).all()
         assert codes[pos] in ((2 * R, 2 * R - 1) if sign > 0 else (0, 1))
-        dec = np.zeros(n, np.uint16)
-        oracle.scaling_decompress(enc, dec, n, nbits, 16, strategy, BF16)
-        d = bits_to_f32(dec, BF16)
+        dec = np.zeros(n, np.uint16 if dt == BF16 else np.float32)
+        oracle.scaling_decompress(enc, dec, n, nbits, 16, strategy, dt)
+        d = bits_to_f32(dec, dt)
         assert (np.delete(d, pos) == 0).all() and abs(d[pos] - v[pos]) <= 0.5 / max(R, 1) * 1.02
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+def test_rounding_direction_hierarchical(oracle, nbits, dt):
+    """hierarchical layout, every width and both element types: with the chunk maximum R * 2^-10 in every chunk the
+    quantisation step is just above 2^-10, so k * 2^-10 sits just below the integer k; rand 0 rounds every non-zero
+    value up, rand 1 floors, and an exact zero gives 0 / -1"""
+    n, R = 256, (1 << (nbits - 1)) - 1
+    base = np.zeros((16, 16), np.float32)
+    base[:, 0] = R / 1024.0
+    ks = (np.arange(1, 16) % (R + 1)).astype(np.float32)            # integers 0 .. R
+    base[:, 1:] = ks / 1024.0
+    base[::2, 1:] *= -1.0
+    base = base.reshape(-1)
+    c0, (q, unit) = unpack_stream(oracle.scaling_compress(_elems(base, dt), _elems(np.zeros(n), dt), n, nbits, 16, 2, dt), n, nbits, 16, 2)
+    c1, _ = unpack_stream(oracle.scaling_compress(_elems(base, dt), _elems(np.ones(n), dt), n, nbits, 16, 2, dt), n, nbits, 16, 2)
+    step = q.astype(np.float32).repeat(16) * bits_to_f32(unit, BF16).repeat(256)
+    assert (step > 2.0 ** -10).all() and (step < 2.0 ** -10 * 1.02).all()
+    x = (bits_to_f32(_elems(base, dt), dt).astype(np.float64) / step.astype(np.float64))
+    up = np.where(base == 0, 0, np.ceil(x))
+    down = np.where(base == 0, -1, np.floor(x))
+    assert (c0 - R == np.clip(up, -R, R)).all()
+    assert (c1 - R == np.clip(down, -R, R)).all()
 
 
 def test_rounding_direction_at_rand_extremes(oracle):
