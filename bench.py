@@ -9,13 +9,19 @@ is quoted on.  Inputs are resident in HBM before the timed region; the calls go
 through the C ABI of libdynamiq_eden.so on torch's current stream.
 
 Prints ONE JSON line (see the fields below).  `value` is fp32 gradient bytes
-(4 * N) per second of compress+decompress.  `roofline` prices the dominant
-kernel (compress) at its algorithmic bytes (4 + 2 + (q + 0.5625) / 8 per
-element) against the 8 TB/s HBM peak, with the kernel's average launch duration
-measured here with HIP events on the launch stream.  `cpu_baseline` times the
-scalar C oracle (a port of the reference algorithm) on the host, on one core;
-`cpu_torch_path` times the same round trip written as torch CPU tensor ops (the
-shape of the reference's own torch implementation) on torch's thread pool.
+(4 * N) per second of compress+decompress with ONE bucket's buffers replayed
+(69 MB: after the warm-up they sit partly in the 256 MB Infinity Cache);
+`value_cold` is the same step walking a ring of distinct bucket sets whose
+footprint exceeds 512 MB, so that every launch streams from and to HBM.
+`roofline` prices the dominant kernel (compress) at its algorithmic bytes
+(4 + 2 + (q + 0.5625) / 8 per element) against the 8 TB/s HBM peak, with the
+kernel's average launch duration measured here with HIP events on the launch
+stream (the timed launches are replayed from a HIP graph so that the host's
+per-call cost is not part of the figure; `eager_ms_per_step` has it): `frac` for the replayed bucket, `frac_cold` for the ring of buckets.
+`cpu_baseline` times the reference's CPU-runnable path for this workload -- the
+hierarchical chunk quantiser as a torch op sequence (cpu_baselines.py) -- on all
+host cores; `cpu_scalar_port` is the scalar C oracle on one core and
+`cpu_rht_path` EDEN's torch round trip (srrcomp.py:293-353) on 2^20 elements.
 """
 import argparse
 import json
@@ -55,6 +61,30 @@ def make_bucket(n, seed, device):
 
 
 def event_ms(fn, iters):
+    """average device time of one fn() in ms: `iters` calls recorded into one HIP graph on a side stream and replayed
+    between two events on that stream, so that the host's per-call cost (a few microseconds through ctypes, about
+    the duration of these kernels) cannot sit between the launches"""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(iters):
+                fn()
+        graph.replay()
+        side.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record(side)
+        graph.replay()
+        end.record(side)
+        end.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    return start.elapsed_time(end) / iters
+
+
+def eager_ms(fn, iters):
+    """the same with one host call per launch (what a Python caller sees)"""
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     start.record()
@@ -76,7 +106,10 @@ def main():
     ap.add_argument("--src", choices=["fp32", "bf16"], default="fp32")
     ap.add_argument("--rand", choices=["pool", "philox"], default="pool",
                     help="pool: the reference's rand_pool tensor (default); philox: uniform values drawn in the kernel")
-    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the cpu_baseline leg (0 = skip)")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of each cpu_baseline leg (0 = skip)")
+    ap.add_argument("--cold-sets", type=int, default=-1,
+                    help="distinct bucket sets (source, random pool, packed, output) the cold leg walks; default: as many "
+                         "as make up 640 MB, at least 10; 0 or 1 = skip the cold leg")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle parity check of a sample")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain elementwise fp32 copy kernel (out = -in) of the same element count, "
@@ -125,8 +158,10 @@ def main():
     torch.cuda.synchronize()
 
     # ---- timed region: exactly `steps` steps between two synchronisations ----
-    t0 = time.perf_counter()
     ms_per_step = event_ms(step, args.steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eager_ms_per_step = eager_ms(step, args.steps)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     value = 4.0 * n / (ms_per_step * 1e-3) / 1e9
@@ -139,6 +174,63 @@ def main():
     dec_bytes = (sbytes + (nbits + OVERHEAD_BITS) / 8.0) * n
     comp_gbs = comp_bytes / (comp_ms * 1e-3) / 1e9
     dec_gbs = dec_bytes / (dec_ms * 1e-3) / 1e9
+
+    # ---- the same step over a ring of distinct buckets (> 512 MB): no launch finds its operands in a cache ----
+    cold = None
+    set_bytes = src.numel() * src.element_size() + rand.numel() * 2 + packed.numel() + out.numel() * out.element_size()
+    if args.cold_sets < 0:
+        args.cold_sets = max(10, -(-640000000 // set_bytes))
+    if args.cold_sets > 1:
+        sets = [(src, rand, packed, out)]
+        for k in range(1, args.cold_sets):
+            xk = make_bucket(n, k, dev)
+            gk = torch.Generator(device=dev)
+            gk.manual_seed(1000 + k)
+            sets.append((xk if args.src == "fp32" else xk.to(torch.bfloat16),
+                         torch.rand(n, generator=gk, device=dev).to(torch.bfloat16), torch.zeros_like(packed),
+                         torch.empty_like(out)))
+        pos = [0]
+
+        def nxt():
+            pos[0] = (pos[0] + 1) % len(sets)
+            return sets[pos[0]]
+
+        def compress_cold():
+            s_, r_, p_, _ = nxt()
+            if args.rand == "philox":
+                capi.scaling_compress_philox(s_, p_, n, nbits, C, strategy, 2026, 0)
+            else:
+                capi.scaling_compress(s_, p_, r_, n, nbits, C, strategy)
+
+        def decompress_cold():
+            _, _, p_, o_ = nxt()
+            capi.scaling_decompress(p_, o_, n, nbits, C, strategy)
+
+        def step_cold():
+            s_, r_, p_, o_ = nxt()
+            if args.rand == "philox":
+                capi.scaling_compress_philox(s_, p_, n, nbits, C, strategy, 2026, 0)
+            else:
+                capi.scaling_compress(s_, p_, r_, n, nbits, C, strategy)
+            capi.scaling_decompress(p_, o_, n, nbits, C, strategy)
+
+        for _ in range(len(sets)):
+            step_cold()
+        torch.cuda.synchronize()
+        step_cold_ms = event_ms(step_cold, args.steps)
+        comp_cold_ms = event_ms(compress_cold, args.steps)
+        dec_cold_ms = event_ms(decompress_cold, args.steps)
+        cold = {
+            "sets": len(sets),
+            "footprint_MB": round(set_bytes * len(sets) / 1e6, 1),
+            "ms_per_step": round(step_cold_ms, 5),
+            "value": round(4.0 * n / (step_cold_ms * 1e-3) / 1e9, 2),
+            "compress_ms": round(comp_cold_ms, 5),
+            "decompress_ms": round(dec_cold_ms, 5),
+            "compress_GBps": round(comp_bytes / (comp_cold_ms * 1e-3) / 1e9, 1),
+            "decompress_GBps": round(dec_bytes / (dec_cold_ms * 1e-3) / 1e9, 1),
+        }
+        del sets[1:]
 
     if args.pmc_calibration:
         cal_src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
@@ -153,7 +245,7 @@ def main():
 
     # ---- parity of a sample against the oracle (the checker, not the product) ----
     bit_exact = None
-    cpu = None
+    cpu_scalar = None
     if not args.no_check or args.cpu_seconds > 0:
         import oracle as O
         odt = O.F32 if args.src == "fp32" else O.BF16
@@ -180,13 +272,13 @@ def main():
         if args.cpu_seconds > 0:
             reps, spent = 0, 0.0
             dec_o = np.zeros(m, src_h.dtype)
-            while spent < args.cpu_seconds and reps < 64:
+            while spent < args.cpu_seconds / 2 and reps < 64:
                 t1 = time.perf_counter()
                 enc_o = O.scaling_compress(src_h, rand_h, m, nbits, C, strategy, odt)
                 O.scaling_decompress(enc_o, dec_o, m, nbits, C, strategy, odt)
                 spent += time.perf_counter() - t1
                 reps += 1
-            cpu = {
+            cpu_scalar = {
                 "value": round(4.0 * m * reps / spent / 1e9, 4),
                 "unit": "GB/s",
                 "cores": 1,
@@ -195,24 +287,41 @@ def main():
                           % (m, reps),
             }
 
-    # ---- the same round trip as a torch op sequence on the host cores (shape of the reference's own torch
-    #      implementation, csrc/logic.py:225-296); a second reported baseline beside the scalar port ----
-    cpu_torch = None
-    if args.cpu_seconds > 0 and nbits in (4, 8) and args.src == "fp32":
-        from dynamiq_sigcomm_artifact_amd.evaluate import _torch_cpu_roundtrip
-        xc, rc = src.cpu(), torch.rand(n)
-        _torch_cpu_roundtrip(xc, rc, nbits)
-        ts = []
-        while len(ts) < 9 and sum(ts) < args.cpu_seconds:
-            t1 = time.perf_counter()
-            _torch_cpu_roundtrip(xc, rc, nbits)
-            ts.append(time.perf_counter() - t1)
-        ts.sort()
-        cpu_torch = {
-            "value": round(4.0 * n / ts[len(ts) // 2] / 1e9, 3),
+    # ---- the reference's CPU-runnable path for this workload on all host cores: the hierarchical chunk quantiser as a
+    #      torch op sequence of the shape of the reference's own torch implementation (csrc/logic.py:225-296) ----
+    cpu = None
+    cpu_rht = None
+    if args.cpu_seconds > 0:
+        import cpu_baselines as CB
+        xc, rc = x32.cpu(), torch.rand(n)
+        if strategy == 2:
+            sec, reps = CB.median_seconds(lambda: CB.hier_roundtrip(xc, rc, nbits), args.cpu_seconds)
+            cpu = {
+                "value": round(4.0 * n / sec / 1e9, 3),
+                "unit": "GB/s",
+                "cores": torch.get_num_threads(),
+                "kind": "port",
+                "sample": "the whole bucket (%d fp32 elements), median of %d compress+decompress round trips of the "
+                          "hierarchical chunk-16 quantiser as torch CPU ops (output equal to the oracle's, tests/test_cpu_baselines.py)"
+                          % (n, reps),
+            }
+        else:
+            cpu = cpu_scalar
+        # EDEN's rotate -> Lloyd-Max quantise -> bit planes -> back (srrcomp.py:293-353), the CPU path of the 2^20 configuration
+        from dynamiq_sigcomm_artifact_amd.eden import normal_centroids_and_boundaries
+        d1 = 1 << 20
+        cen, bnd = normal_centroids_and_boundaries(4)
+        cen, bnd = cen.float(), bnd.float()
+        g1 = torch.Generator().manual_seed(0)
+        x1 = torch.randn(d1, generator=g1) * 1e-3
+        sec, reps = CB.median_seconds(lambda: CB.rht_roundtrip(x1.clone(), 4, 0, cen, bnd), args.cpu_seconds / 2, max_reps=5)
+        cpu_rht = {
+            "value": round(4.0 * d1 / sec / 1e9, 4),
             "unit": "GB/s",
             "cores": torch.get_num_threads(),
-            "sample": "the whole bucket, median of %d round trips of the flat chunk-16 quantiser as torch CPU ops" % len(ts),
+            "kind": "port",
+            "sample": "2^20 fp32 N(0, 1e-3^2), median of %d EDEN compress+decompress round trips at 4 bits as torch CPU ops "
+                      "(randDiag, Hadamard / sqrt(n), bucketize, EdenBinsToBits and back)" % reps,
         }
 
     result = {
@@ -247,9 +356,14 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(comp_gbs / HBM_PEAK_GBS, 4),
+            "frac_is": "one bucket's buffers replayed (69 MB working set: cache-assisted, part of the traffic is served by "
+                       "the 256 MB Infinity Cache); frac_cold is the HBM-only figure",
+            "frac_cold": round(cold["compress_GBps"] / HBM_PEAK_GBS, 4) if cold else None,
+            "achieved_cold": cold["compress_GBps"] if cold else None,
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.src, nbits, strategy, n)) if args.rand == "pool" else None,
             "algorithmic_bytes_per_launch": int(comp_bytes),
             "avg_launch_ms": round(comp_ms, 5),
+            "avg_launch_ms_cold": cold["compress_ms"] if cold else None,
         },
         "kernels": {
             "compress": {"ms": round(comp_ms, 5), "algorithmic_GBps": round(comp_gbs, 1), "frac_hbm": round(comp_gbs / HBM_PEAK_GBS, 4)},
@@ -258,9 +372,13 @@ def main():
         "frac_hbm_roundtrip": round((comp_bytes + dec_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "nmse": nmse,
         "bit_exact_vs_oracle": bit_exact,
+        "eager_ms_per_step": round(eager_ms_per_step, 5),
         "host_wall_ms_per_step": round(wall_ms, 5),
+        "value_cold": cold["value"] if cold else None,
+        "cold": cold,
         "cpu_baseline": cpu,
-        "cpu_torch_path": cpu_torch,
+        "cpu_scalar_port": cpu_scalar,
+        "cpu_rht_path": cpu_rht,
     }
     print(json.dumps(result))
 

@@ -181,21 +181,25 @@ def _check(rc):
 _seen = threading.local()
 
 
-def _note(t):
+def _refuse(t):
     if not isinstance(t, torch.Tensor):
         raise RuntimeError("a tensor argument is required, got %s" % type(t).__name__)
     if not t.is_cuda:
         raise RuntimeError("tensor arguments must live on the GPU (got a %s tensor)" % t.device.type)
-    if not t.is_contiguous():
-        raise RuntimeError("tensor arguments must be contiguous")
-    devices = getattr(_seen, "devices", None)
-    if devices is None:
-        devices = _seen.devices = set()
-    devices.add(t.device.index)
+    raise RuntimeError("tensor arguments must be contiguous")
 
 
 def _p(t):
-    _note(t)
+    try:
+        ok = t.is_cuda and t.is_contiguous()
+    except AttributeError:
+        ok = False
+    if not ok:
+        _refuse(t)
+    try:
+        _seen.devices.append(t.device.index)
+    except AttributeError:
+        _seen.devices = [t.device.index]
     return t.data_ptr()
 
 
@@ -204,15 +208,18 @@ def _ptr(t):
 
 
 def _dev(t):
-    _note(t)
+    _p(t)
     return t.device.index
 
 
 def _call(fn, *args):
-    devices = getattr(_seen, "devices", None) or set()
-    _seen.devices = set()
-    if len(devices) > 1:
-        raise RuntimeError("tensor arguments live on different devices: %s" % sorted(devices))
+    devices = getattr(_seen, "devices", None)
+    if devices:
+        first = devices[0]
+        mixed = any(d != first for d in devices)
+        del devices[:]
+        if mixed:
+            raise RuntimeError("tensor arguments live on different devices")
     _check(fn(*args))
 
 

@@ -1,6 +1,8 @@
+#!/usr/bin/env python3
 """Runs the synthetic workloads of the build's baseline configurations on one GPU
 and prints one JSON line per measurement (NMSE, GB/s, fraction of the 8 TB/s HBM
-peak).  ``python -m dynamiq_sigcomm_artifact_amd.evaluate --config 1|2|3|4|5``.
+peak).  ``python evaluate.py --config 1|2|3|4|5``.  A measurement tool beside
+``bench.py``; the library does not import it.
 
   1  2^20 fp32 N(0,1e-3^2): blocked randomized Hadamard + quantise + pack and back
   2  25 MB bucket, Student-t with outliers: 4/8-bit round trips, fp32 and bf16
@@ -8,6 +10,9 @@ peak).  ``python -m dynamiq_sigcomm_artifact_amd.evaluate --config 1|2|3|4|5``.
   4  Llama-3-8B shaped gradient set in 25 MB buckets: dynamic {2,4,8}-bit allocation
   5  2^30 fp32: compress / decompress / fused sweep, and the blocked transform
 ``--kernels`` times every entry point of the library on one 25 MB bucket.
+``--reference-benchmark`` prints the table of the reference's own microbenchmark
+(cuda_kernels/tests/benchmark_scaling_quantization.py:60-112: bf16, chunk 16, 268,435,456 elements,
+2/4/8 bits x strategy 2/3, eager launches through the eden_utils module) with the fraction of the HBM peak.
 
 Timings: 10 warm-up launches, then 50 launches replayed from a HIP graph between two
 events (cuda_kernels/tests/benchmark_scaling_quantization.py:41-57 times eager launches;
@@ -16,15 +21,23 @@ the graph keeps the host's per-call cost out of the figure).
 import argparse
 import json
 import math
+import os
+import sys
 import types
 
 import torch
 
-from . import bitrate, capi
-from .compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
-from .dynamiq_pipeline import (dynamic_bitrate_allreduce, dynamic_bitrate_allreduce_grouped,
-                               dynamic_bitrate_allreduce_single_pass)
-from .ring_sim import ring_allreduce, split_chunks
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import cpu_baselines                                                                       # noqa: E402
+from dynamiq_sigcomm_artifact_amd import bitrate, capi                                     # noqa: E402
+from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern   # noqa: E402
+from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import (dynamic_bitrate_allreduce,     # noqa: E402
+                                                           dynamic_bitrate_allreduce_grouped,
+                                                           dynamic_bitrate_allreduce_single_pass)
+from dynamiq_sigcomm_artifact_amd.ring_sim import ring_allreduce, split_chunks             # noqa: E402
 
 HBM_PEAK = 8000.0  # GB/s
 OV = 0.5625        # scale overhead, bits per element
@@ -118,7 +131,7 @@ def config1(dev):
                             roundtrip_fused_GBps_fp32_in=round(4.0 * n / t2 / 1e3, 1))
             _emit(**line)
     # the reference-legal path for this configuration: EDEN (whole-vector rotation, Lloyd-Max bins, bit planes)
-    from .eden import Eden
+    from dynamiq_sigcomm_artifact_amd.eden import Eden
     eden = Eden(device=dev)
     for nbits in (4, 5, 8):
         data = eden.compress(x, nbits, 0)
@@ -171,20 +184,7 @@ def config2(dev):
               nmse_ratio=round(gpu_nmse / cpu_nmse, 4))
 
 
-def _torch_cpu_roundtrip(x, rand, nbits, chunk=16):
-    """the chunk-scaling quantiser as a torch op sequence of the shape the reference's own torch implementation has
-    (csrc/logic.py:225-296: abs, row max, div, add 1e-7, div, floor, stochastic carry from the random tensor, nibble pack;
-    unpack, mul), here on CPU tensors"""
-    rng = (1 << (nbits - 1)) - 1
-    v = x.view(-1, chunk).clone()
-    scale = v.abs().max(dim=1, keepdim=True)[0].div_(rng).add_(1e-7)
-    v.div_(scale)
-    fl = torch.floor(v)
-    codes = fl.add_(rand.view(-1, chunk) < v.sub_(fl)).clamp_(-rng, rng).add_(rng).to(torch.uint8)
-    if nbits == 4:
-        packed = codes[:, 0::2] | (codes[:, 1::2] << 4)
-        codes = torch.stack((packed & 15, packed >> 4), dim=2).reshape(-1, chunk)
-    return codes.float().sub_(rng).mul_(scale).reshape(-1)
+_torch_cpu_roundtrip = cpu_baselines.flat_roundtrip
 
 
 def _cpu_torch_line(x32, nbits):
@@ -251,7 +251,7 @@ def config3(dev, n=124439808, W=8):
             del vecs, comps
     # "5 bits" as the dynamic {2, 4, 8} mix (target 5 - 0.625 code bits): mean-centre, allocate, one grouped ring per width
     target = 5.0 - bitrate.DYNAMIC_BITRATE_HEADROOM
-    from .compressors import superchunk_mean_center
+    from dynamiq_sigcomm_artifact_amd.compressors import superchunk_mean_center
     nsc = npad // 256
     norms = torch.zeros(nsc, dtype=torch.bfloat16, device=dev)
     res = torch.empty(npad, dtype=torch.bfloat16, device=dev)
@@ -369,7 +369,7 @@ def _offset_search_lines(dev, norms_list, target, u_ref):
 
 def config4(dev, limit=None):
     target = 5.0 - bitrate.DYNAMIC_BITRATE_HEADROOM
-    from .compressors import superchunk_mean_center
+    from dynamiq_sigcomm_artifact_amd.compressors import superchunk_mean_center
     # pass 1: norms of every superchunk -> u
     norms_list = []
     for b in _llama_buckets(dev, limit=limit):
@@ -697,7 +697,7 @@ def kernels(dev, n=6553600):
         y.normal_(generator=g)
         line("rht_blocked", lambda: capi.rht_blocked(y, sign, 1 << kb, 1.0, False), 12 * d, n=d, block=1 << kb)
     # consumers of the rotated vector
-    from .eden import normal_centroids_and_boundaries
+    from dynamiq_sigcomm_artifact_amd.eden import normal_centroids_and_boundaries
     y.normal_(generator=g)
     for nbits in (4, 8):
         cen, bnd = (t.to(dev) for t in normal_centroids_and_boundaries(nbits))
@@ -767,10 +767,70 @@ def kernels(dev, n=6553600):
     line("quantization_compression", lambda: capi.quantization(y, 0.5, 15.0, 1), 8 * d, n=d)
 
 
+def reference_benchmark(dev, n=16 * 16 * 65536 * 16):
+    """cuda_kernels/tests/benchmark_scaling_quantization.py:60-112 on this GPU, through the drop-in module: the same
+    inputs (:31-39), the same eager timing loops (:41-57; 10 warm-up + 50 launches, 5 + 25 for the two ring-step
+    variants), the same CSV columns, plus the fraction of the 8 TB/s HBM peak each time amounts to for the
+    algorithmic bytes of the call (2 + 2 + (q + 0.5625) / 8 per element for compress, ...)."""
+    import dynamiq_sigcomm_artifact_amd as pkg
+    eden_utils = pkg.load_eden_utils()
+    torch.manual_seed(2026)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def time_ms(fn, warmup=10, iters=50):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / iters
+
+    print("device=%s" % torch.cuda.get_device_name(0), flush=True)
+    print("dtype,chunk_size,nbits,strategy,compress_ms,decompress_ms,split_dec_comp_ms,fused_dec_comp_ms,"
+          "frac_hbm_compress,frac_hbm_decompress,frac_hbm_split,frac_hbm_fused", flush=True)
+    chunk_size, dtype = 16, torch.bfloat16
+    idx = torch.arange(n, dtype=torch.float32, device=dev)
+    values = torch.sin(idx * 0.017) * 1.7 + torch.cos(idx * 0.0071) * 0.3
+    values += (idx.remainder(7) - 3.0) * 0.013
+    src = values.to(dtype).contiguous()
+    del idx, values
+    inp_template = (src.float() * -0.25).to(dtype).contiguous()
+    rand_pool = torch.rand(n, dtype=torch.float32, device=dev).to(dtype).contiguous()
+    for nbits in (2, 4, 8):
+        for strategy in (2, 3):
+            encoded = torch.zeros(capi.required_bytes(n, nbits, chunk_size, strategy), dtype=torch.uint8, device=dev)
+            send = torch.zeros_like(encoded)
+            send_split = torch.zeros_like(encoded)
+            decoded = torch.empty_like(src)
+            inp = inp_template.clone()
+            inp_split = inp_template.clone()
+            eden_utils.scaling_compress(src, encoded, rand_pool, n, nbits, chunk_size, stream, strategy)
+            torch.cuda.synchronize()
+            c_ms = time_ms(lambda: eden_utils.scaling_compress(src, encoded, rand_pool, n, nbits, chunk_size, stream, strategy))
+            d_ms = time_ms(lambda: eden_utils.scaling_decompress(encoded, decoded, n, nbits, chunk_size, stream, strategy))
+            s_ms = time_ms(lambda: (eden_utils.scaling_decompress_add(encoded, inp_split, n, nbits, chunk_size, stream, strategy),
+                                    eden_utils.scaling_compress(inp_split, send_split, rand_pool, n, nbits, chunk_size, stream, strategy)),
+                           warmup=5, iters=25)
+            f_ms = time_ms(lambda: eden_utils.scaling_dec_comp(encoded, inp, send, rand_pool, n, nbits, chunk_size, stream, strategy),
+                           warmup=5, iters=25)
+            pk = (nbits + OV) / 8.0
+            frac = lambda bytes_per_elem, ms: bytes_per_elem * n / (ms * 1e-3) / 1e9 / HBM_PEAK
+            print("%s,%d,%d,%d,%.4f,%.4f,%.4f,%.4f,%.3f,%.3f,%.3f,%.3f"
+                  % (dtype, chunk_size, nbits, strategy, c_ms, d_ms, s_ms, f_ms, frac(4 + pk, c_ms), frac(2 + pk, d_ms),
+                     frac((pk + 4) + (4 + pk), s_ms), frac(4 + 2 * pk, f_ms)), flush=True)
+            del encoded, send, send_split, decoded, inp, inp_split
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--kernels", action="store_true", help="time every entry point of the library on a 25 MB bucket")
+    ap.add_argument("--reference-benchmark", action="store_true",
+                    help="the table of cuda_kernels/tests/benchmark_scaling_quantization.py with the fraction of the HBM peak")
     ap.add_argument("--limit", type=int, default=None, help="config 4: number of 25 MB buckets to process")
     ap.add_argument("--n", type=int, default=None, help="configs 3 and 5: element count override")
     args = ap.parse_args()
@@ -781,8 +841,11 @@ def main():
     if args.kernels:
         kernels(dev, **({"n": args.n} if args.n else {}))
         return
+    if args.reference_benchmark:
+        reference_benchmark(dev, **({"n": args.n} if args.n else {}))
+        return
     if args.config is None:
-        raise SystemExit("give --config N or --kernels")
+        raise SystemExit("give --config N, --kernels or --reference-benchmark")
     if args.config == 1:
         config1(dev)
     elif args.config == 2:
