@@ -767,6 +767,32 @@ def kernels(dev, n=6553600):
     line("quantization_compression", lambda: capi.quantization(y, 0.5, 15.0, 1), 8 * d, n=d)
 
 
+def quantiser_sizes(dev, nbits=4):
+    """the production quantiser (bf16, chunk 16, hierarchical) at the three sizes that matter: one 25 MB bucket, one ring
+    chunk of the 8 x 124,439,808 configuration, and 2^28 elements (beyond every cache): compress, decompress and the
+    fused ring step for AEE and MEE, graph-replayed"""
+    for n in (6553600, 15555072, 1 << 28):
+        g = torch.Generator(device=dev).manual_seed(n & 0xffff)
+        src = (torch.randn(n, generator=g, device=dev) * 1e-3).to(torch.bfloat16)
+        inp = (torch.randn(n, generator=g, device=dev) * 1e-3).to(torch.bfloat16)
+        rnd = torch.rand(n, generator=g, device=dev).to(torch.bfloat16)
+        out = torch.empty_like(src)
+        pk = (nbits + OV) / 8.0
+        iters = 10 if n > (1 << 27) else 50
+        for strategy, name in ((2, "aee"), (3, "mee")):
+            enc = torch.zeros(capi.required_bytes(n, nbits, 16, strategy), dtype=torch.uint8, device=dev)
+            send = torch.zeros_like(enc)
+            capi.scaling_compress(src, enc, rnd, n, nbits, 16, strategy)
+            for op, fn, bpe in (("compress", lambda: capi.scaling_compress(src, enc, rnd, n, nbits, 16, strategy), 4 + pk),
+                                ("decompress", lambda: capi.scaling_decompress(enc, out, n, nbits, 16, strategy), 2 + pk),
+                                ("dec_comp", lambda: capi.scaling_dec_comp(enc, inp, send, rnd, n, nbits, 16, strategy), 4 + 2 * pk)):
+                t = _time_us(fn, 5, iters)
+                _emit(sizes=True, op=op, method=name, n=n, nbits=nbits, us=round(t, 2), GBps_algorithmic=round(bpe * n / t / 1e3, 1),
+                      frac_hbm=round(bpe * n / t / 1e3 / HBM_PEAK, 4))
+            del enc, send
+        del src, inp, rnd, out
+
+
 def reference_benchmark(dev, n=16 * 16 * 65536 * 16):
     """cuda_kernels/tests/benchmark_scaling_quantization.py:60-112 on this GPU, through the drop-in module: the same
     inputs (:31-39), the same eager timing loops (:41-57; 10 warm-up + 50 launches, 5 + 25 for the two ring-step
@@ -829,6 +855,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--kernels", action="store_true", help="time every entry point of the library on a 25 MB bucket")
+    ap.add_argument("--quantiser-sizes", action="store_true",
+                    help="compress / decompress / fused step of the production quantiser (bf16, 4-bit, AEE and MEE) at 25 MB, at "
+                         "the ring-chunk size of the 8-rank configuration and at 2^28 elements")
     ap.add_argument("--reference-benchmark", action="store_true",
                     help="the table of cuda_kernels/tests/benchmark_scaling_quantization.py with the fraction of the HBM peak")
     ap.add_argument("--limit", type=int, default=None, help="config 4: number of 25 MB buckets to process")
@@ -841,11 +870,14 @@ def main():
     if args.kernels:
         kernels(dev, **({"n": args.n} if args.n else {}))
         return
+    if args.quantiser_sizes:
+        quantiser_sizes(dev)
+        return
     if args.reference_benchmark:
         reference_benchmark(dev, **({"n": args.n} if args.n else {}))
         return
     if args.config is None:
-        raise SystemExit("give --config N, --kernels or --reference-benchmark")
+        raise SystemExit("give --config N, --kernels, --quantiser-sizes or --reference-benchmark")
     if args.config == 1:
         config1(dev)
     elif args.config == 2:
