@@ -56,37 +56,6 @@ __device__ __forceinline__ void chunk_encode_guarded(const RV &v, const RR &r, c
     }
 }
 
-// One element of the fast quantiser, every operation as the reference orders them (three correctly rounded
-// divisions and the deterministic log2 for MEE): the signed code before clamping.
-template <bool MEE, class ARG>
-__device__ __forceinline__ int exact_code_fast(float vi, float ri, double yd, const ARG &mp)
-{
-    float x = div_by(vi, yd);
-    if (MEE) {
-        const float arg = div_by(__builtin_fabsf(x), mp.inv_c) + 1.0f;
-        const float lat = div_by(log2_det_ge1(arg), mp.inv_l2b);
-        x = __builtin_copysignf(lat, x);
-    }
-    const float fl = __builtin_floorf(x);
-    const float c = __builtin_ceilf((x - fl) - ri);
-    return (int)(fl + c); // |fl| <= R + 1 and c in {-1, 0, 1}: exact
-}
-
-// The code of an element is ceil(L - r) for the coordinate L the exact chain computes -- v / d (AEE) or
-// +-log2(|v / d| / c + 1) / log2(base) (MEE) -- because floor(L) + ceil(frac(L) - r) is that integer.  A cheap
-// estimate of L - r gives the same code unless it comes within kDelta of an integer; such elements (one in a few
-// thousand) are redone with the exact chain, so the bytes are those of the exact chain throughout.
-//   AEE: estimate fma(v, rcp(d), -r); the hardware reciprocal is good to 1 ulp, so the distance to the exact
-//        v / d - r is below (R + 1) (2^-23 + 2^-24) + ulp(R + 1) / 2 < 0.27 (R + 1) 2^-20.
-//   MEE: estimate fma(v_log_f32(fma(|v rcp(d)|, 1 / c, 1)), +-1 / log2(base), -r), v_log_f32 being good to 1 ulp;
-//        estimate and exact chain both approximate log2(|v| / (d c) + 1) / log2(base), their distance is bounded by
-//        (1.44 * 5e-7 + 2.7 ulp(log)) / log2(base) + 2 ulp(R): < 6.5e-5 for 6..8 bits (log2(base) = 0.0286, log < 4)
-//        and < 1.1e-5 below (log2(base) >= 0.09, log < 1.5); measured over 4e9 random operands per width: 1.5e-5
-//        and 4.8e-6.
-template <int NBITS, bool MEE> struct EstimateGuard {
-    static constexpr float kDelta = MEE ? (NBITS >= 6 ? 0x1p-12f : 0x1p-14f) : (float)(1 << (NBITS - 1)) * 0x1p-20f;
-};
-
 // the same quantiser for a wave whose elements are all finite and <= 2^100 in
 // magnitude (amax_bits is the integer-order maximum of |v|) and whose random
 // values all lie in [0, 1]: none of the guards can fire
@@ -111,38 +80,7 @@ __device__ __forceinline__ void chunk_encode_fast(const RV &v, const RR &r, uint
     const float d = (float)qi * unit; // exact: 8 x 8 significant bits
 #pragma unroll
     for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
-    const float rd = __builtin_amdgcn_rcpf(d);
-    const float rc = MEE ? (float)mp.inv_c : 0.0f, rl2b = MEE ? (float)mp.inv_l2b : 0.0f;
-    constexpr float kDelta = EstimateGuard<NBITS, MEE>::kDelta;
-    bool doubt[16], any = false;
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const float vi = v.get(i);
-        float t;
-        if (MEE) {
-            const float est = __builtin_amdgcn_logf(__builtin_fmaf(__builtin_fabsf(vi * rd), rc, 1.0f));
-            t = __builtin_fmaf(est, __builtin_copysignf(rl2b, vi), -r.get(i));
-        } else {
-            t = __builtin_fmaf(vi, rd, -r.get(i));
-        }
-        const float c = __builtin_ceilf(t);
-        doubt[i] = __builtin_fabsf((c - t) - 0.5f) > 0.5f - kDelta;
-        any |= doubt[i];
-        const int sv = (int)c; // |t| < 2^20: exact
-        words_put<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
-    }
-    if (__builtin_amdgcn_ballot_w64(any) != 0) {
-        const double yd = recip_f64(d);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            // a zero element has L = 0 on both routes whatever its random value is
-            const bool redo = doubt[i] && (__float_as_uint(v.get(i)) << 1) != 0;
-            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
-                const int sv = exact_code_fast<MEE>(v.get(i), r.get(i), yd, mp);
-                if (redo) words_set<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
-            }
-        }
-    }
+    estimate_codes<NBITS, MEE>(v, r, d, mp, w);
 }
 
 constexpr uint32_t kFastMaxBits = 0x71800000u; // 2^100

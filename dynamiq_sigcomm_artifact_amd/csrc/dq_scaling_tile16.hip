@@ -111,10 +111,18 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
     }
 
     const bool fast = __builtin_amdgcn_ballot_w64(!ordinary_scale(d)) == 0;
-    const double yd = fast ? recip_f64(d) : 0.0;
     uint32_t w[Rec<NBITS>::WORDS];
 #pragma unroll
     for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = 0;
+    // binary32 arithmetic, ordinary scales (so every element is finite and at most (R + 1) d) and random values in
+    // [0, 1]: the codes come from the estimate with its exact redo near the rounding boundaries
+    bool estimated = false;
+    if constexpr (DT != DQ_F16) {
+        estimated = fast && __builtin_amdgcn_ballot_w64(!r.unit_interval()) == 0;
+        if (estimated) estimate_codes<NBITS, MEE>(v, r, d, mp, w);
+    }
+    const double yd = fast && !estimated ? recip_f64(d) : 0.0;
+    if (!estimated) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const float e = v.get(i);
@@ -147,6 +155,7 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
             sv = sr_plain(x, r.get(i));
         }
         words_put<NBITS>(w, i, (uint32_t)clamp_code(sv, R));
+    }
     }
 
     uint8_t *gout = dst + G::stream_offset(c0);
