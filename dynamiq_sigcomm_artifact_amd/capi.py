@@ -27,7 +27,7 @@ EXPORTS = [
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
-    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_scaling_decompress_irht", "dq_pack_signs",
+    "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_rht_scaling_compress_mfma16", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
     "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_quantize_static_max_n", "dq_eden_quantize_static", "dq_eden_dequantize", "dq_eden_dequantize_irht", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
 ]
@@ -111,6 +111,8 @@ def lib():
         L.dq_rht_blocked.argtypes = [vp, vp, i32, i64, i64, f32, i32, i32, vp]
         L.dq_rht_scaling_compress.restype = i32
         L.dq_rht_scaling_compress.argtypes = [vp, vp, i32, vp, vp, i32, i64, i64, f32, i32, i32, i32, u64, u64, vp]
+        L.dq_rht_scaling_compress_mfma16.restype = i32
+        L.dq_rht_scaling_compress_mfma16.argtypes = [vp, vp, i32, vp, i64, i64, f32, i32, u64, u64, vp]
         L.dq_scaling_decompress_irht.restype = i32
         L.dq_scaling_decompress_irht.argtypes = [vp, vp, i32, vp, i64, i64, f32, i32, i32, i32, vp]
         L.dq_pack_signs.restype = i32
@@ -475,6 +477,16 @@ def rht_scaling_compress(src, sign, dst, block, scale, nbits, strategy, rand_poo
     _call(lib().dq_rht_scaling_compress, _p(src), _ptr(sign), _packed(sign), _p(dst), _ptr(rand_pool), code, src.numel(),
                                          block, float(scale), nbits, _dev(src), strategy, int(seed), int(step),
                                          _stream(stream))
+
+
+def rht_scaling_compress_mfma16(src, sign, dst, block, scale, seed=0, step=0, stream=None):
+    """measurement variant of rht_scaling_compress (4-bit AEE, in-kernel rounding stream): the first four stages of the
+    transform on the matrix cores; agrees with the default to rounding error only"""
+    if src.dtype != torch.float32:
+        raise RuntimeError("rht_scaling_compress_mfma16: src must be float32")
+    _check_sign(sign, src.numel(), "rht_scaling_compress_mfma16")
+    _call(lib().dq_rht_scaling_compress_mfma16, _p(src), _ptr(sign), _packed(sign), _p(dst), src.numel(), block, float(scale),
+          _dev(src), int(seed), int(step), _stream(stream))
 
 
 def scaling_decompress_irht(src, sign, dst, block, scale, nbits, strategy, stream=None):

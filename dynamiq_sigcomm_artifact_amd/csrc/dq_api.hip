@@ -588,6 +588,22 @@ int dq_rht_scaling_compress(const float *src, const void *sign, int sign_packed,
                                           strategy == 3, mee_params(nbits), seed, step, static_cast<hipStream_t>(stream)));
 }
 
+int dq_rht_scaling_compress_mfma16(const float *src, const void *sign, int sign_packed, uint8_t *dst, int64_t n, int64_t block,
+                                   float scale, int device, uint64_t seed, uint64_t step, dq_stream_t stream)
+{
+    int rc = check_rht_scaling(n, block, 4, 2);
+    if (rc) return rc;
+    if (!src || !dst) return fail(DQ_ERR_NULL);
+    if (block < 16 || block > 16384) return fail(DQ_ERR_SIZE, "the matrix-core variant takes blocks of 16 .. 16384");
+    if ((reinterpret_cast<uintptr_t>(src) & 15) || (sign && !sign_packed && (reinterpret_cast<uintptr_t>(sign) & 15)))
+        return fail(DQ_ERR_SIZE, "the matrix-core variant needs 16-byte aligned vectors");
+    if ((rc = select_device(device))) return rc;
+    const hipError_t e = dq::launch_rht_compress_mfma16(src, sign, sign_packed ? 1 : 0, dst, n, block, scale, mee_params(4), seed, step,
+                                                        static_cast<hipStream_t>(stream));
+    if (e == hipErrorInvalidValue) return fail(DQ_ERR_SIZE, "the matrix-core variant needs n to be a multiple of its tile (8192 elements or the block)");
+    return finish(e);
+}
+
 int dq_scaling_decompress_irht(const uint8_t *src, const void *sign, int sign_packed, float *dst, int64_t n, int64_t block, float scale,
                                int nbits, int device, int strategy, dq_stream_t stream)
 {

@@ -118,6 +118,8 @@ hipError_t launch_pack_signs(const float *sign, uint32_t *bits, int64_t n, hipSt
 hipError_t launch_rht_compress(const float *src, const void *sign, int sign_bits, uint8_t *dst, const void *rnd, int rand_kind,
                                int64_t n, int64_t block, float scale, int nbits, bool mee, const MeeParams &mp,
                                uint64_t seed, uint64_t step, hipStream_t stream);
+hipError_t launch_rht_compress_mfma16(const float *src, const void *sign, int sign_bits, uint8_t *dst, int64_t n, int64_t block,
+                                      float scale, const MeeParams &mp, uint64_t seed, uint64_t step, hipStream_t stream);
 hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign_bits, float *dst, int64_t n, int64_t block,
                                   float scale, int nbits, bool mee, const MeeParams &mp, hipStream_t stream);
 

@@ -102,8 +102,39 @@ __host__ __device__ inline int padded_tile_floats(int kt)
     return (tile + tile / 16 + 1 + 3) & ~3;
 }
 
-template <int RDT, int NBITS, bool MEE>
-__global__ void rht_compress_kernel(const float *__restrict__ x, uint8_t *__restrict__ dst, const void *__restrict__ rnd,
+// The stages of strides 1..8 of 64 chunks as one matrix product on the matrix cores: Y = X H16, X the wave's 64 x 16
+// block of chunks, H16[i][j] = (-1)^popcount(i & j).  v_mfma_f32_16x16x4_f32 takes a 16 x 4 slice of X (lane l: row
+// l % 16, column l / 16 of the slice) against a 4 x 16 slice of H16 (lane l: row l / 16, column l % 16) and leaves a
+// 16 x 16 block of Y with lane l holding rows 4 (l / 16) .. + 3 of column l % 16.  With slice j made of the columns
+// 4 (l / 16) + j of X, a lane's four slice operands are one aligned float4 of its row.  The sums of a product are not
+// formed in the butterfly order, so the last bits differ from the stage-by-stage transform (the reference's own
+// tolerance for the transform is 1e-5 relative): a measurement variant, not the default.
+typedef float mfma_f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void chunk_stages_mfma16(const float *__restrict__ x, const RhtTileArgs &a, int64_t origin, int chunk0,
+                                                    int lane, float *lds)
+{
+    const int m = lane & 15, kk = lane >> 4;
+    float h[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) h[j] = (__builtin_popcount((4 * kk + j) & m) & 1) ? -1.0f : 1.0f;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        const int64_t g = origin + (int64_t)(chunk0 + 16 * b + m) * 16 + 4 * kk;
+        float4 q = *reinterpret_cast<const float4 *>(x + g);
+        flip4(q, a, g);
+        mfma_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(q.x, h[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(q.y, h[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(q.z, h[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(q.w, h[3], acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) lds[(chunk0 + 16 * b + 4 * kk + i) * 17 + m] = acc[i];
+    }
+}
+
+template <int RDT, int NBITS, bool MEE, bool MFMA16 = false>
+__global__ __attribute__((amdgpu_waves_per_eu(8, 8))) void rht_compress_kernel(const float *__restrict__ x, uint8_t *__restrict__ dst, const void *__restrict__ rnd,
                                     RhtTileArgs a, int rvec, RandKey key, MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
@@ -115,6 +146,10 @@ __global__ void rht_compress_kernel(const float *__restrict__ x, uint8_t *__rest
     // every lane loads chunks of 16 consecutive floats (64 bytes, as the quantiser's own kernels do), flips the
     // signs and does the stages of strides 1..8 on its registers; elements beyond n (a ragged last tile) are zero
     const int nchunks = tile >> 4;
+    if constexpr (MFMA16) {
+        // whole tiles, 16-byte aligned, blocks of at least 16 (checked by the launcher)
+        for (int c0 = (tid >> 6) * 64; c0 < nchunks; c0 += nthreads) chunk_stages_mfma16(x, a, origin, c0, tid & 63, lds);
+    } else {
     for (int c = tid; c < nchunks; c += nthreads) {
         float v[16];
         load_chunk(v, x, a, origin + c * 16);
@@ -122,6 +157,7 @@ __global__ void rht_compress_kernel(const float *__restrict__ x, uint8_t *__rest
         float *mine = lds + c * 17; // pad_idx(16 c + i) = 17 c + i
 #pragma unroll
         for (int i = 0; i < 16; i++) mine[i] = v[i];
+    }
     }
     fwht_lds_stages_after4(lds, a.kt, a.kb, tid, nthreads);
 
@@ -460,6 +496,23 @@ hipError_t launch_rht_compress(const float *src, const void *sign, int sign_bits
     } else {
         DQ_NBITS_MEE(run_compress, DQ_F32, src, sign, sign_bits, dst, rnd, n, block, scale, mp, key, stream)
     }
+}
+
+// the 4-bit AEE kernel with the in-kernel rounding stream and the first four stages on the matrix cores (measurement variant)
+hipError_t launch_rht_compress_mfma16(const float *src, const void *sign, int sign_bits, uint8_t *dst, int64_t n, int64_t block,
+                                      float scale, const MeeParams &mp, uint64_t seed, uint64_t step, hipStream_t stream)
+{
+    const Geometry g = geometry(src, sign, sign_bits, n, block, scale);
+    if (g.a.kb < 4 || g.a.kb >= kSplitBits || g.a.kt >= kSplitBits || g.a.kt < 10 || !g.a.vec || (n & ((1 << g.a.kt) - 1)) != 0 || (g.threads & 63) != 0)
+        return hipErrorInvalidValue;
+    const size_t windows = (size_t)(g.threads / 64) * Rec<4>::WIN;
+    const size_t lds = std::max(g.lds_floats * sizeof(float), windows);
+    auto kernel = rht_compress_kernel<DQ_PHILOX, 4, false, true>;
+    hipError_t e = allow_lds(kernel, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3(g.grid), dim3(g.threads), lds, stream, src, dst, nullptr, g.a, 0, RandKey{seed, step},
+                       make_arg<4, false>(mp));
+    return hipGetLastError();
 }
 
 hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign_bits, float *dst, int64_t n, int64_t block, float scale,

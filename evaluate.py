@@ -793,6 +793,34 @@ def quantiser_sizes(dev, nbits=4):
         del src, inp, rnd, out
 
 
+def mfma_experiment(dev, n=1 << 28, block=8192):
+    """the transform fused with the quantiser (4-bit AEE, packed signs, in-kernel rounding stream), its first four stages
+    as add / subtract butterflies (the library's kernel) and as a product with the +-1 matrix on the matrix cores"""
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn(n, generator=g, device=dev) * 1e-3
+    sign = torch.empty(n // 32, dtype=torch.int32, device=dev)
+    capi.rand_diag_bits(sign, n, 1)
+    scale = 1.0 / math.sqrt(block)
+    nbytes = capi.required_bytes(n, 4, 16, 2)
+    a, b = (torch.zeros(nbytes, dtype=torch.uint8, device=dev) for _ in range(2))
+    bytes_per = (4 + 0.125 + (4 + OV) / 8) * n
+    variants = (("butterflies (VALU)", lambda: capi.rht_scaling_compress(x, sign, a, block, scale, 4, 2, seed=3, step=1)),
+                ("H16 on the matrix cores (v_mfma_f32_16x16x4_f32)",
+                 lambda: capi.rht_scaling_compress_mfma16(x, sign, b, block, scale, seed=3, step=1)))
+    times = {name: [] for name, _ in variants}
+    for _ in range(5):                      # alternating, so that clock and box drift hit both alike
+        for name, fn in variants:
+            times[name].append(_time_us(fn, 3, 10))
+    for name, _ in variants:
+        ts = sorted(times[name])
+        _emit(mfma_experiment=True, first_four_stages=name, n=n, block=block, us_median=round(ts[2], 1), us_min=round(ts[0], 1),
+              us_max=round(ts[-1], 1), frac_hbm_median=round(bytes_per / ts[2] / 1e3 / HBM_PEAK, 4))
+    out_a, out_b = torch.empty_like(x), torch.empty_like(x)
+    capi.scaling_decompress_irht(a, sign, out_a, block, scale, 4, 2)
+    capi.scaling_decompress_irht(b, sign, out_b, block, scale, 4, 2)
+    _emit(mfma_experiment=True, bytes_differing=float((a != b).float().mean()), nmse_butterflies=_nmse(x, out_a), nmse_matrix_cores=_nmse(x, out_b))
+
+
 def reference_benchmark(dev, n=16 * 16 * 65536 * 16):
     """cuda_kernels/tests/benchmark_scaling_quantization.py:60-112 on this GPU, through the drop-in module: the same
     inputs (:31-39), the same eager timing loops (:41-57; 10 warm-up + 50 launches, 5 + 25 for the two ring-step
@@ -858,6 +886,8 @@ def main():
     ap.add_argument("--quantiser-sizes", action="store_true",
                     help="compress / decompress / fused step of the production quantiser (bf16, 4-bit, AEE and MEE) at 25 MB, at "
                          "the ring-chunk size of the 8-rank configuration and at 2^28 elements")
+    ap.add_argument("--mfma-experiment", action="store_true",
+                    help="the transform fused with the quantiser (blocks of 8192) with its first four stages as butterflies and on the matrix cores")
     ap.add_argument("--reference-benchmark", action="store_true",
                     help="the table of cuda_kernels/tests/benchmark_scaling_quantization.py with the fraction of the HBM peak")
     ap.add_argument("--limit", type=int, default=None, help="config 4: number of 25 MB buckets to process")
@@ -872,6 +902,9 @@ def main():
         return
     if args.quantiser_sizes:
         quantiser_sizes(dev)
+        return
+    if args.mfma_experiment:
+        mfma_experiment(dev, **({"n": args.n} if args.n else {}))
         return
     if args.reference_benchmark:
         reference_benchmark(dev, **({"n": args.n} if args.n else {}))

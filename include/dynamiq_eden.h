@@ -437,6 +437,20 @@ int dq_rht_scaling_compress(const float *src, const void *sign, int sign_packed,
                             const void *rand_pool, int rand_dtype, int64_t n, int64_t block,
                             float scale, int nbits, int device, int strategy, uint64_t seed,
                             uint64_t step, dq_stream_t stream);
+/* Measurement variant, no counterpart in the reference: dq_rht_scaling_compress
+ * for 4-bit AEE codes with the in-kernel rounding stream, the transform's first
+ * four stages (H16 on 16 consecutive elements) computed as a product with the
+ * +-1 matrix on the matrix cores (v_mfma_f32_16x16x4_f32) instead of add /
+ * subtract butterflies.  A product sums in another order than the butterflies,
+ * so the rotated values agree with dq_rht_blocked to rounding error (1e-5
+ * relative, the reference's tolerance for its transform) and a small share of
+ * the codes differ by one step; it is also slower (16 multiply-adds per element
+ * on the matrix pipe against 4 additions).  Kept to answer that question with a
+ * number; use dq_rht_scaling_compress.  block 16 .. 16384, 16-byte aligned
+ * buffers, n a multiple of the kernel's tile. */
+int dq_rht_scaling_compress_mfma16(const float *src, const void *sign, int sign_packed, uint8_t *dst,
+                                   int64_t n, int64_t block, float scale, int device,
+                                   uint64_t seed, uint64_t step, dq_stream_t stream);
 /* the way back: dq_scaling_decompress into fp32 followed by dq_rht_blocked
  * (inverse), the decoded vector staying in LDS. */
 int dq_scaling_decompress_irht(const uint8_t *src, const void *sign, int sign_packed, float *dst,

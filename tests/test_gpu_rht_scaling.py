@@ -1,6 +1,8 @@
 """The transform fused with the quantiser (dq_rht_scaling_compress, dq_scaling_decompress_irht) against the two-call
 sequences it replaces -- rht_blocked + scaling_compress, scaling_decompress + inverse rht_blocked -- byte for byte /
 bit for bit, and one case straight against the oracle."""
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -164,3 +166,30 @@ def test_fused_special_values(capi, strategy):
     back = torch.empty(n, device=DEV)
     capi.scaling_decompress_irht(got, sign, back, block, scale, nbits, strategy)
     assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
+
+
+@pytest.mark.parametrize("block", [16, 1024, 8192, 16384])
+def test_matrix_core_variant_agrees_to_rounding_error(capi, block):
+    """dq_rht_scaling_compress_mfma16 forms the first four stages as a matrix product: another summation order, so
+    the records agree with the butterfly kernel's except for codes whose value sat on a rounding boundary"""
+    n = 1 << 18
+    g = torch.Generator().manual_seed(block)
+    x = (torch.randn(n, generator=g) * 1e-3).to(DEV)
+    sign = torch.empty(n // 32, dtype=torch.int32, device=DEV)
+    capi.rand_diag_bits(sign, n, 7)
+    scale = 1.0 / math.sqrt(block)
+    nbytes = capi.required_bytes(n, 4, 16, 2)
+    a = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    b = torch.zeros(nbytes + 16, dtype=torch.uint8, device=DEV)
+    capi.rht_scaling_compress(x, sign, a, block, scale, 4, 2, seed=11, step=2)
+    capi.rht_scaling_compress_mfma16(x, sign, b, block, scale, seed=11, step=2)
+    assert bool((b[nbytes:] == 0).all())
+    differing = float((a != b[:nbytes]).float().mean())
+    assert differing < 2e-3, differing
+    out_a, out_b = torch.empty_like(x), torch.empty_like(x)
+    capi.scaling_decompress_irht(a, sign, out_a, block, scale, 4, 2)
+    capi.scaling_decompress_irht(b[:nbytes].clone(), sign, out_b, block, scale, 4, 2)
+    nm = lambda y: float(((y - x).double() ** 2).sum() / (x.double() ** 2).sum())
+    assert abs(nm(out_a) - nm(out_b)) < 0.01 * nm(out_a)
+    with pytest.raises(RuntimeError):
+        capi.rht_scaling_compress_mfma16(x, sign, b, 8, 1.0)
