@@ -44,7 +44,7 @@ OVERHEAD_BITS = 0.5625  # hierarchical scale bytes per element, in bits
 # the --pmc-calibration copy kernel: FETCH_SIZE x 1.999, WRITE_SIZE x 1.000.
 # key: (source dtype, nbits, strategy, elements)
 MEASURED_TRAFFIC_BYTES = {
-    ("fp32", 4, 2, 6553600): int((25600.0 / 12806.6 * 19240.6 + 1.0 * 3800.0) * 1024),
+    ("fp32", 4, 2, 6553600): int((25600.0 / 12806.9 * 19253.6 + 1.0 * 3800.0) * 1024),
 }
 
 
