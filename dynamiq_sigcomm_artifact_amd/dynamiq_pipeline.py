@@ -121,6 +121,84 @@ def dynamic_bitrate_allreduce_grouped(rank_vecs, u, compressors, out=None, work=
     return outs, total, qbits
 
 
+def fixed_proportion_allreduce(rank_vecs, thresholds, compressors, out=None, fixed_4bit_only=False):
+    """One bucket partition of the non-dynamic hook, ``P2P_dynamiQ_hook``'s ``compress_and_reduce_and_decompress``
+    (comm_hooks.py:682-786), as the reference's op sequence: mean-centre, reduce the statistics, sort the norms
+    (stable, descending), gather the first / middle / last share as the 8- / 4- / 2-bit groups **in sorted order**, one
+    compressed ring per group, scatter back, add the means.  ``fixed_4bit_only`` is the "fixed" method: only the 4-bit
+    group (everything, thresholds {4: 1, 8: 0, 2: 0}) is communicated (:768-772)."""
+    W = len(rank_vecs)
+    n = rank_vecs[0].numel()
+    nsc = (n + SUPERCHUNK - 1) // SUPERCHUNK
+    dev, dt = rank_vecs[0].device, rank_vecs[0].dtype
+    residuals = [torch.empty(nsc * SUPERCHUNK, dtype=dt, device=dev) for _ in range(W)]
+    stats = [torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev) for _ in range(W)]
+    for r in range(W):
+        superchunk_mean_center(rank_vecs[r], residuals[r], stats[r], n, W, SUPERCHUNK)
+    total = stats[0].clone()
+    for r in range(1, W):
+        total.add_(stats[r])
+    groups_idx = bitrate.fixed_proportion_groups(total[:, 1], thresholds)
+    res2d = [res.view(-1, SUPERCHUNK) for res in residuals]
+    for q, idx in zip((8, 4, 2), groups_idx):
+        if idx.numel() == 0 or (fixed_4bit_only and q != 4):
+            continue
+        groups = [torch.index_select(res2d[r], 0, idx).reshape(-1) for r in range(W)]
+        comps = compressors[q]
+        if W == 1:
+            c = comps[0]
+            send = c.create_tensor(groups[0], torch.uint8)
+            c.compression(groups[0], send)
+            c.decompression(send, groups[0])
+        else:
+            ring_allreduce(groups, comps, align=SUPERCHUNK)
+        for r in range(W):
+            res2d[r].index_copy_(0, idx, groups[r].view(-1, SUPERCHUNK))
+    outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
+    for r in range(W):
+        superchunk_add_mean_copy(residuals[r], outs[r], total, n, SUPERCHUNK)
+    return outs, total, groups_idx
+
+
+def fixed_proportion_allreduce_grouped(rank_vecs, thresholds, compressors, out=None, fixed_4bit_only=False):
+    """The same all-reduce, bit for bit, with the sort, the slices, the gathers, the scatters and the final mean add
+    replaced by one launch of the device plan (group_plan_sorted) and the row-list codec calls; the group sizes follow
+    from the fractions on the host, so nothing is read back."""
+    eu = load_eden_utils()
+    W = len(rank_vecs)
+    n = rank_vecs[0].numel()
+    nsc = (n + SUPERCHUNK - 1) // SUPERCHUNK
+    dev, dt = rank_vecs[0].device, rank_vecs[0].dtype
+    residuals = [torch.empty(nsc * SUPERCHUNK, dtype=dt, device=dev) for _ in range(W)]
+    stats = [torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev) for _ in range(W)]
+    for r in range(W):
+        superchunk_mean_center(rank_vecs[r], residuals[r], stats[r], n, W, SUPERCHUNK)
+    total = stats[0] if W == 1 else stats[0].clone()
+    for r in range(1, W):
+        total.add_(stats[r])
+    counts = bitrate.fixed_proportion_counts(nsc, thresholds)
+    order = torch.empty(3 * nsc, dtype=torch.int32, device=dev)
+    eu.group_plan_sorted(total, counts[0], counts[2], order, None, torch.cuda.current_stream().cuda_stream)
+    outs = out if out is not None else [torch.empty(n, dtype=dt, device=dev) for _ in range(W)]
+    if fixed_4bit_only:
+        # the groups that are not communicated keep their local residual: copy it through first
+        for r in range(W):
+            superchunk_add_mean_copy(residuals[r], outs[r], total, n, SUPERCHUNK)
+    for g, (q, cnt) in enumerate(zip((8, 4, 2), counts)):
+        if cnt == 0 or (fixed_4bit_only and q != 4):
+            continue
+        rows = order[g * nsc:g * nsc + cnt]
+        comps = compressors[q]
+        if W == 1:
+            c = comps[0]
+            send = torch.empty(c.compressed_numel(cnt * SUPERCHUNK), dtype=torch.uint8, device=dev)
+            c.compression_rows(residuals[0], rows, send)
+            c.decompression_rows(send, outs[0], rows, total, n)
+        else:
+            ring_allreduce_rows(residuals, rows, comps, outs, total, n)
+    return outs, total, order, counts
+
+
 def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=None, work=None, stream=None,
                                           norm_histogram=None):
     """The same all-reduce with every stage kept on the device: no residual buffers (the centring is folded

@@ -150,3 +150,40 @@ def test_groups_feed_the_row_codec(capi, oracle, strategy):
         assert (packed.cpu().numpy() == packed_o[:nbytes]).all(), width
         capi.scaling_decompress_rows(packed, out.reshape(-1), rows, None, nsc * 256, cnt, width, strategy)
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("W", [1, 2, 3])
+@pytest.mark.parametrize("method,cls", [("dynamiQ_aee_5bit", "aee"), ("dynamiQ_mee_3bit", "mee"), ("dynamiQ_mee_4bit_fixed", "mee")])
+def test_fixed_proportion_allreduce_device_plan_equals_op_sequence(capi, W, method, cls):
+    """the whole partition of the non-dynamic hook: sort / slice / index_select / ring / index_copy_ / add-mean as the
+    reference runs it against one plan launch + row-list codec calls; same random rows, so the outputs are bit-equal"""
+    import types
+    from dynamiq_sigcomm_artifact_amd import bitrate as B
+    from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import fixed_proportion_allreduce, fixed_proportion_allreduce_grouped
+    K = Aee_Dynamic_Range_GPU_kern if cls == "aee" else Mee_Dynamic_Range_GPU_kern
+    n = 256 * 700 + 77                       # a ragged tail
+    g = torch.Generator().manual_seed(31 + W)
+    scale = torch.exp(torch.randn((n + 255) // 256, generator=g) * 2 - 5).repeat_interleave(256)[:n]
+    vecs = [(torch.randn(n, generator=g) * scale + 1e-3).to(torch.bfloat16).to(DEV) for _ in range(W)]
+    thr = B.fixed_proportion_thresholds(method)
+    fixed = "fixed" in method
+
+    def comps():
+        gen = torch.Generator(device=DEV).manual_seed(5)
+        params = lambda r: {"d": {(0, 0): n + 256}, "world_size": W, "rank": r, "args": types.SimpleNamespace(aggregation_method=method)}
+        return {q: [K(q, 16, params(r), generator=gen) for r in range(W)] for q in (8, 4, 2)}
+
+    ref, total, idx = fixed_proportion_allreduce([v.clone() for v in vecs], thr, comps(), fixed_4bit_only=fixed)
+    out, total2, order, counts = fixed_proportion_allreduce_grouped([v.clone() for v in vecs], thr, comps(), fixed_4bit_only=fixed)
+    assert torch.equal(total.view(torch.int16), total2.view(torch.int16))
+    nsc = (n + 255) // 256
+    for gi, (cnt, ix) in enumerate(zip(counts, idx)):
+        assert torch.equal(order[gi * nsc:gi * nsc + cnt].long(), ix)
+    for a, b in zip(ref, out):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    for r in range(1, W):
+        assert torch.equal(out[0], out[r])
+    exact = sum(v.double() for v in vecs) / W
+    nmse = float(((out[0].double() - exact) ** 2).sum() / (exact ** 2).sum())
+    assert nmse < 0.2
