@@ -265,7 +265,7 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
 // sorted order**.  The norms are bf16 values, so the sort key has 16 bits and the position of superchunk i is
 //     G(key_i) + E(i),   G = superchunks with a key that sorts earlier,   E = superchunks j < i with the same key
 // -- a counting sort.  As in plan_one_kernel no workgroup waits for another: the workgroup of tile b (256
-// superchunks) counts the keys of the whole bucket itself, in an LDS histogram of 65536 16-bit counters (128 KB),
+// superchunks) counts the keys of the whole bucket itself, in an LDS histogram (128 KB, 144 KB with its padding),
 // in two steps: first the superchunks before its tile (the counter of key_i is then the part of E(i) that lies in
 // earlier tiles), then the rest; an in-place exclusive scan of the histogram gives G.  The part of E inside the tile
 // comes from comparing the tile's keys with each other.  nsc <= 65535, so no counter overflows.
@@ -274,10 +274,25 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
 // +0 = -0 ... -inf.
 constexpr int kSortThreads = 1024;
 constexpr int kSortTile = 256;
-constexpr int kSortWords = 32768; // 65536 16-bit counters
-constexpr int kSortBatch = 8;
+constexpr int kSortWords = 32768;                          // words of the histogram
+constexpr int kSortLdsWords = kSortWords + kSortWords / 8; // stored with 4 words of padding after every 32
+constexpr int kSortBatch = 32;                             // loads in flight per thread: 32768 superchunks in one round trip
 
-__device__ __forceinline__ uint32_t descending_key(uint32_t pattern)
+// Word w of the histogram lives at w + 4 (w / 32): in the scan thread t owns the 32 words [32 t, 32 t + 32), and with a
+// lane stride of 36 words instead of 32 the 16-byte accesses of neighbouring lanes fall into different banks (unpadded,
+// all lanes of a wave hit the same four banks).
+__device__ __forceinline__ int hist_slot(uint32_t word) { return (int)(word + ((word >> 5) << 2)); }
+
+// Two layouts.  Sums of squares are not negative, so normally every pattern is one of 0 .. 0x7f80 or a NaN: then a key
+// takes 15 bits, NaN -> 0, +inf -> 1, ..., +0 -> 0x7f81, and every counter has a word of its own (narrow).  A bucket that
+// holds a negative pattern (-0 included) takes the general key, 16 bits, with two 16-bit counters per word (wide); its
+// counting and its scan cost about twice the narrow ones.
+__device__ __forceinline__ uint32_t narrow_key(uint32_t pattern)
+{
+    return pattern <= (uint32_t)kMaxPattern ? (uint32_t)kMaxPattern + 1u - pattern : 0u; // NaN (sign bit clear) -> 0
+}
+
+__device__ __forceinline__ uint32_t wide_key(uint32_t pattern)
 {
     const uint32_t mag = pattern & 0x7fffu;
     if (mag > (uint32_t)kMaxPattern) return 0u;             // NaN
@@ -285,117 +300,144 @@ __device__ __forceinline__ uint32_t descending_key(uint32_t pattern)
     return 0x7fffu - mag;                                   // +inf -> 0x7f, +0 -> 0x7fff
 }
 
-__device__ __forceinline__ void count_keys(const uint32_t *__restrict__ pairs, int begin, int end, uint32_t *hist)
+template <bool WIDE> __device__ __forceinline__ uint32_t sort_key(uint32_t pattern) { return WIDE ? wide_key(pattern) : narrow_key(pattern); }
+
+template <bool WIDE> __device__ __forceinline__ void count_one(uint32_t *hist, uint32_t pattern)
 {
-    for (int i0 = begin; i0 < end; i0 += kSortBatch * kSortThreads) {
+    const uint32_t k = sort_key<WIDE>(pattern);
+    if (WIDE)
+        atomicAdd(&hist[hist_slot(k >> 1)], 1u << (16 * (k & 1)));
+    else
+        atomicAdd(&hist[hist_slot(k)], 1u);
+}
+
+template <bool WIDE> __device__ __forceinline__ int counter_of(const uint32_t *hist, uint32_t k)
+{
+    return WIDE ? (int)((hist[hist_slot(k >> 1)] >> (16 * (k & 1))) & 0xffffu) : (int)hist[hist_slot(k)];
+}
+
+// adds the keys of the superchunks [begin, end) to the histogram; cached: the (mean, norm) pairs of the first
+// kSortBatch * kSortThreads superchunks, already in registers (pair j of thread t = superchunk j * kSortThreads + t)
+template <bool WIDE>
+__device__ __forceinline__ void count_keys(const uint32_t *__restrict__ pairs, int begin, int end, uint32_t *hist,
+                                           const uint32_t (&cached)[kSortBatch])
+{
+#pragma unroll
+    for (int j = 0; j < kSortBatch; j++) {
+        const int i = j * kSortThreads + (int)threadIdx.x;
+        if (i >= begin && i < end) count_one<WIDE>(hist, cached[j] >> 16);
+    }
+    for (int i0 = max(begin, kSortBatch * kSortThreads) / (kSortBatch * kSortThreads) * (kSortBatch * kSortThreads); i0 < end;
+         i0 += kSortBatch * kSortThreads) {
         uint32_t raw[kSortBatch];
 #pragma unroll
         for (int j = 0; j < kSortBatch; j++) {
             const int i = i0 + j * kSortThreads + (int)threadIdx.x;
-            if (i < end) raw[j] = pairs[i];
+            if (i >= begin && i < end) raw[j] = pairs[i];
         }
 #pragma unroll
         for (int j = 0; j < kSortBatch; j++) {
             const int i = i0 + j * kSortThreads + (int)threadIdx.x;
-            if (i < end) {
-                const uint32_t k = descending_key(raw[j] >> 16);
-                atomicAdd(&hist[k >> 1], 1u << (16 * (k & 1)));
-            }
+            if (i >= begin && i < end) count_one<WIDE>(hist, raw[j] >> 16);
         }
     }
 }
 
-__global__ __launch_bounds__(kSortThreads) void sorted_plan_kernel(const uint32_t *__restrict__ pairs, int nsc, int top,
-                                                                  int bottom, int64_t *__restrict__ qbits_out,
-                                                                  int32_t *__restrict__ order, int32_t *__restrict__ work)
+// exclusive scan of the counters in place; thread t owns the words [32 t, 32 t + 32)
+template <bool WIDE> __device__ __forceinline__ void scan_counters(uint32_t *hist, uint32_t *wave_sum)
 {
-    __shared__ __align__(16) uint32_t hist[kSortWords];
-    __shared__ __align__(16) uint16_t tile_key[kSortTile];
-    __shared__ int part_rank[kSortThreads / kSortTile][kSortTile];
-    __shared__ uint32_t wave_sum[kSortThreads / 64];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    uint4 *mine = reinterpret_cast<uint4 *>(hist + 36 * t); // hist_slot(32 t)
+    uint4 v[8];
+    uint32_t sum = 0;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        v[q] = mine[q];
+        const uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+        for (int h = 0; h < 4; h++) sum += WIDE ? (w[h] & 0xffffu) + (w[h] >> 16) : w[h];
+    }
+    uint32_t incl = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum;
+    for (int k = 0; k < wave; k++) run += wave_sum[k];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+        for (int h = 0; h < 4; h++) {
+            if (WIDE) {
+                const uint32_t lo = w[h] & 0xffffu, hi = w[h] >> 16;
+                w[h] = (run & 0xffffu) | ((run + lo) << 16); // an exclusive prefix is at most nsc - 1 < 65536
+                run += lo + hi;
+            } else {
+                const uint32_t c = w[h];
+                w[h] = run;
+                run += c;
+            }
+        }
+        mine[q] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+template <bool WIDE>
+__device__ __forceinline__ void sorted_plan_body(const uint32_t *__restrict__ pairs, int nsc, int top, int bottom,
+                                                 int64_t *__restrict__ qbits_out, int32_t *__restrict__ order,
+                                                 const uint32_t (&cached)[kSortBatch], uint32_t own_pattern, uint32_t *hist,
+                                                 uint16_t *tile_key, int (*part_rank)[kSortTile], uint32_t *wave_sum)
+{
+    const int t = threadIdx.x;
     const int nbefore = (int)blockIdx.x * kSortTile;
     const int e = t & (kSortTile - 1), part = t / kSortTile; // element of the tile, quarter of its predecessors
     const int own = nbefore + e;
     const int valid = min(kSortTile, nsc - nbefore);
-
-    uint32_t key = 0;
-    if (e < valid) key = descending_key(pairs[own] >> 16);
+    const uint32_t key = e < valid ? sort_key<WIDE>(own_pattern) : 0u;
     if (part == 0) tile_key[e] = (uint16_t)key;
-    {
-        uint4 *h4 = reinterpret_cast<uint4 *>(hist);
-        for (int w = t; w < kSortWords / 4; w += kSortThreads) h4[w] = make_uint4(0u, 0u, 0u, 0u);
-    }
-    __syncthreads();
+    __syncthreads(); // the zeroed histogram and the tile's keys are in place
 
-    // superchunks of the tile with the same key and a smaller index: quarter `part` of the candidates
+    // superchunks of the tile with the same key and a smaller index: quarter `part` of the candidates (the quarters
+    // behind the element's own hold none)
     {
         int r = 0;
         const int j0 = part * (kSortTile / 4);
-        const uint4 *k4 = reinterpret_cast<const uint4 *>(tile_key + j0);
+        if (j0 <= e) {
+            const uint4 *k4 = reinterpret_cast<const uint4 *>(tile_key + j0);
 #pragma unroll
-        for (int q = 0; q < kSortTile / 4 / 8; q++) {
-            const uint4 v = k4[q]; // the same address in every lane: a broadcast
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            for (int q = 0; q < kSortTile / 4 / 8; q++) {
+                const uint4 v = k4[q]; // the same address in every lane: a broadcast
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int h = 0; h < 8; h++) {
-                const int j = j0 + 8 * q + h;
-                const uint32_t kj = (w[h >> 1] >> (16 * (h & 1))) & 0xffffu;
-                r += (kj == key && j < e) ? 1 : 0;
+                for (int h = 0; h < 8; h++) {
+                    const int j = j0 + 8 * q + h;
+                    const uint32_t kj = (w[h >> 1] >> (16 * (h & 1))) & 0xffffu;
+                    r += (kj == key && j < e) ? 1 : 0;
+                }
             }
         }
         part_rank[part][e] = r;
     }
-    count_keys(pairs, 0, nbefore, hist);
+    count_keys<WIDE>(pairs, 0, nbefore, hist, cached);
     __syncthreads();
     int same_before = 0;
     if (part == 0 && e < valid) {
-        same_before = (int)((hist[key >> 1] >> (16 * (key & 1))) & 0xffffu);
+        same_before = counter_of<WIDE>(hist, key);
 #pragma unroll
         for (int q = 0; q < kSortThreads / kSortTile; q++) same_before += part_rank[q][e];
     }
     __syncthreads();
-    count_keys(pairs, nbefore, nsc, hist);
+    count_keys<WIDE>(pairs, nbefore, nsc, hist, cached);
     __syncthreads();
-
-    // exclusive scan of the 65536 counters in place: thread t owns counters [64 t, 64 t + 64)
-    {
-        uint4 *mine = reinterpret_cast<uint4 *>(hist + 32 * t);
-        uint4 v[8];
-        uint32_t sum = 0;
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            v[q] = mine[q];
-            const uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
-#pragma unroll
-            for (int h = 0; h < 4; h++) sum += (w[h] & 0xffffu) + (w[h] >> 16);
-        }
-        uint32_t incl = sum;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t up = __shfl_up(incl, d, 64);
-            if (lane >= d) incl += up;
-        }
-        if (lane == 63) wave_sum[wave] = incl;
-        __syncthreads();
-        uint32_t run = incl - sum;
-        for (int k = 0; k < wave; k++) run += wave_sum[k];
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
-#pragma unroll
-            for (int h = 0; h < 4; h++) {
-                const uint32_t lo = w[h] & 0xffffu, hi = w[h] >> 16;
-                w[h] = (run & 0xffffu) | ((run + lo) << 16); // an exclusive prefix is at most nsc - 1 < 65536
-                run += lo + hi;
-            }
-            mine[q] = make_uint4(w[0], w[1], w[2], w[3]);
-        }
-    }
+    scan_counters<WIDE>(hist, wave_sum);
     __syncthreads();
 
     if (part == 0 && e < valid) {
-        const int pos = (int)((hist[key >> 1] >> (16 * (key & 1))) & 0xffffu) + same_before;
+        const int pos = counter_of<WIDE>(hist, key) + same_before;
         const int mid_end = nsc - bottom;
         int region, at;
         if (pos < top) region = 0, at = pos;
@@ -404,6 +446,47 @@ __global__ __launch_bounds__(kSortThreads) void sorted_plan_kernel(const uint32_
         order[(int64_t)region * nsc + at] = own;
         if (qbits_out) qbits_out[own] = region == 0 ? 8 : (region == 1 ? 4 : 2);
     }
+}
+
+__global__ __launch_bounds__(kSortThreads) void sorted_plan_kernel(const uint32_t *__restrict__ pairs, int nsc, int top,
+                                                                  int bottom, int64_t *__restrict__ qbits_out,
+                                                                  int32_t *__restrict__ order, int32_t *__restrict__ work)
+{
+    __shared__ __align__(16) uint32_t hist[kSortLdsWords];
+    __shared__ __align__(16) uint16_t tile_key[kSortTile];
+    __shared__ int part_rank[kSortThreads / kSortTile][kSortTile];
+    __shared__ uint32_t wave_sum[kSortThreads / 64];
+    __shared__ int any_negative;
+    const int t = threadIdx.x;
+    if (t == 0) any_negative = 0;
+    // the first kSortBatch * kSortThreads pairs stay in registers for all three passes over them
+    uint32_t cached[kSortBatch];
+#pragma unroll
+    for (int j = 0; j < kSortBatch; j++) {
+        const int i = j * kSortThreads + t;
+        cached[j] = i < nsc ? pairs[i] : 0u;
+    }
+    const int own = (int)blockIdx.x * kSortTile + (t & (kSortTile - 1));
+    const uint32_t own_pattern = own < nsc ? pairs[own] >> 16 : 0u;
+    {
+        uint4 *h4 = reinterpret_cast<uint4 *>(hist);
+        for (int w = t; w < kSortLdsWords / 4; w += kSortThreads) h4[w] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    __syncthreads();
+    // any pattern with the sign bit set that is not a NaN (a NaN is key 0 in both layouts)
+    bool negative = false;
+#pragma unroll
+    for (int j = 0; j < kSortBatch; j++) negative |= (cached[j] >> 31) != 0 && (cached[j] & 0x7fff0000u) <= ((uint32_t)kMaxPattern << 16);
+    for (int i = kSortBatch * kSortThreads + t; i < nsc; i += kSortThreads) {
+        const uint32_t p = pairs[i];
+        negative |= (p >> 31) != 0 && (p & 0x7fff0000u) <= ((uint32_t)kMaxPattern << 16);
+    }
+    if (__builtin_amdgcn_ballot_w64(negative) != 0 && (t & 63) == 0) any_negative = 1;
+    __syncthreads();
+    if (any_negative)
+        sorted_plan_body<true>(pairs, nsc, top, bottom, qbits_out, order, cached, own_pattern, hist, tile_key, part_rank, wave_sum);
+    else
+        sorted_plan_body<false>(pairs, nsc, top, bottom, qbits_out, order, cached, own_pattern, hist, tile_key, part_rank, wave_sum);
     if (blockIdx.x == 0 && t == 0) {
         work[0] = top;
         work[1] = nsc - top - bottom;
