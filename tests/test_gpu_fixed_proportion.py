@@ -33,6 +33,8 @@ def _norm_sets():
         "256": torch.exp(torch.randn(256, generator=g)),
         "257": torch.exp(torch.randn(257, generator=g)),
         "65535 narrow": torch.rand(65535, generator=g) * 1e-4 + 2e-4,
+        # more than one round of loads per thread with keys of either sign (the two-counters-per-word layout)
+        "40001 of either sign": torch.randn(40001, generator=g) * torch.exp(torch.randn(40001, generator=g)),
     }
     sp = torch.exp(torch.randn(30011, generator=g) * 4 - 5)
     sp[::7] = 0.0
