@@ -97,6 +97,67 @@ __device__ __forceinline__ void load_chunk(const void *p, int64_t base, float (&
     }
 }
 
+// The same chunk kept as loaded (two 16-bit elements per register) and widened at each use: half the registers of
+// the float array for fp16 / bf16, which decides how many waves fit on a SIMD when a lane holds 32 elements and
+// their 32 random values
+template <int DT, int CT> struct PackedChunk {
+    static constexpr int kWords = ChunkShape<DT, CT>::kBytes / 4;
+    uint32_t w[kWords];
+    __device__ __forceinline__ void load(const void *p, int64_t base)
+    {
+        const uint4 *q = reinterpret_cast<const uint4 *>(static_cast<const char *>(p) + base * (ChunkShape<DT, CT>::kBytes / CT));
+#pragma unroll
+        for (int j = 0; j < kWords / 4; j++) {
+            const uint4 v = q[j];
+            w[4 * j] = v.x; w[4 * j + 1] = v.y; w[4 * j + 2] = v.z; w[4 * j + 3] = v.w;
+        }
+    }
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int j = 0; j < kWords; j++) w[j] = 0u;
+    }
+    __device__ __forceinline__ float get(int i) const
+    {
+        if (DT == DQ_F32) return __uint_as_float(w[i]);
+        return elem_from_bits<DT>((w[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+    }
+    // bfloat16 / binary32 only.  The binary32 bit pattern of max |element| in integer order (a NaN sorts above infinity)
+    __device__ __forceinline__ uint32_t absmax_bits() const
+    {
+        if (DT == DQ_F32) {
+            uint32_t m = w[0] & 0x7fffffffu;
+#pragma unroll
+            for (int k = 1; k < kWords; k++) m = max(m, w[k] & 0x7fffffffu);
+            return m;
+        }
+        uint32_t m = w[0] & 0x7fff7fffu;
+#pragma unroll
+        for (int k = 1; k < kWords; k++) m = pk_max_u16(m, w[k] & 0x7fff7fffu);
+        return max(m << 16, m & 0xffff0000u);
+    }
+    // every element in [+0, 1]
+    __device__ __forceinline__ bool unit_interval() const
+    {
+        uint32_t m = w[0];
+#pragma unroll
+        for (int k = 1; k < kWords; k++) m = DT == DQ_F32 ? max(m, w[k]) : pk_max_u16(m, w[k]);
+        return DT == DQ_F32 ? m <= 0x3f800000u : max(m & 0xffffu, m >> 16) <= 0x3f80u;
+    }
+};
+
+// elements [OFF, OFF + 16) of a chunk as the 16-element operand of estimate_codes(); positions at and beyond the
+// chunk's end read as `pad`
+template <class CHUNK, int OFF, int CT> struct Sixteen {
+    const CHUNK &c;
+    float pad;
+    __device__ __forceinline__ float get(int i) const { return OFF + i < CT ? c.get(OFF + i < CT ? OFF + i : 0) : pad; }
+};
+
+struct MeeReciprocals {
+    double inv_c, inv_l2b;
+};
+
 // A wave's chunks, S 16-byte pieces per lane, leave as lane-contiguous pieces (see swz()).  tile: 64 S slots of
 // LDS owned by the wave; dst: where the wave's first piece goes; valid: pieces inside the destination.
 template <int S>
@@ -118,12 +179,14 @@ template <int CT> struct WindowBytes { static constexpr int value = CT ? 64 * CT
 
 // ---- compress ----------------------------------------------------------------
 
-// CT: the chunk size when it is 8 or 32 and src and rnd are 16-byte aligned, else 0
-template <int DT, int RDT, bool HIER, bool MEE, int CT>
+// CT: the chunk size when it is 8 or 32 and src and rnd are 16-byte aligned, else 0.  NB: the code width when it is
+// 2, 4 or 8 and CT is not 0 (the packing loop then unrolls into constant shifts), else 0
+template <int DT, int RDT, bool HIER, bool MEE, int CT, int NB>
 __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
     const void *__restrict__ src, uint8_t *__restrict__ dst, const void *__restrict__ rnd,
-    int64_t nchunks, int nbits, int Crt, MeeParams mp)
+    int64_t nchunks, int nbits_rt, int Crt, MeeParams mp)
 {
+    const int nbits = NB ? NB : nbits_rt;
     typedef ElemIO<DT> IO;
     constexpr int kUnroll = CT ? CT : 1;
     const int C = CT ? CT : Crt;
@@ -133,24 +196,25 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
     const int PB = (C * nbits) >> 3;
     const int64_t base = chunk * C;
 
-    float ev[CT ? CT : 1], rv[CT ? CT : 1];
+    PackedChunk<DT, (CT ? CT : 8)> ev;
+    PackedChunk<RDT, (CT ? CT : 8)> rv;
     if (CT) {
         if (active) {
-            load_chunk<DT, (CT ? CT : 1)>(src, base, ev);
-            load_chunk<RDT, (CT ? CT : 1)>(rnd, base, rv);
+            ev.load(src, base);
+            rv.load(rnd, base);
         } else {
-#pragma unroll
-            for (int i = 0; i < (CT ? CT : 1); i++) ev[i] = rv[i] = 0.0f;
+            ev.zero();
+            rv.zero();
         }
     }
 
     // pass 1: chunk absmax
     float a = 0.0f;
     if (active) {
-        a = __builtin_fabsf(CT ? ev[0] : IO::load(src, base));
+        a = __builtin_fabsf(CT ? ev.get(0) : IO::load(src, base));
 #pragma unroll kUnroll
         for (int i = 1; i < C; i++) {
-            float v = __builtin_fabsf(CT ? ev[CT ? i : 0] : IO::load(src, base + i));
+            float v = __builtin_fabsf(CT ? ev.get(CT ? i : 0) : IO::load(src, base + i));
             a = (DT == DQ_F16) ? h_max(a, v) : __builtin_fmaxf(a, v);
         }
     }
@@ -226,8 +290,8 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
         const double yd = decltype(fast)::value ? recip_f64(d) : 0.0;
 #pragma unroll kUnroll
         for (int i = 0; i < C; i++) {
-            float v = CT ? ev[CT ? i : 0] : IO::load(src, base + i);
-            float r = CT ? rv[CT ? i : 0] : ElemIO<RDT>::load(rnd, base + i);
+            float v = CT ? ev.get(CT ? i : 0) : IO::load(src, base + i);
+            float r = CT ? rv.get(CT ? i : 0) : ElemIO<RDT>::load(rnd, base + i);
             float x = decltype(fast)::value ? div_by(v, yd) : v / d;
             int sv;
             if (DT == DQ_F16) {
@@ -245,7 +309,36 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
         }
     };
     const uint32_t db = __float_as_uint(d);
-    if (CT && db >= 0x0d800000u && db <= 0x71800000u) // a normal number in [2^-100, 2^100]
+    const bool ordinary = db >= 0x0d800000u && db <= 0x71800000u; // a normal number in [2^-100, 2^100]
+    if constexpr (CT != 0 && NB != 0 && DT != DQ_F16) {
+        // binary32 arithmetic: when every lane of the wave has an ordinary scale, finite elements (so |v| <= (R + 1) d)
+        // and random values in [0, 1], the codes come from the estimate with its exact redo near the rounding
+        // boundaries, sixteen elements at a time (dq_tile16.cuh)
+        const bool lane_ok = ordinary && ev.absmax_bits() <= 0x71800000u && rv.unit_interval();
+        if (__builtin_amdgcn_ballot_w64(!lane_ok) == 0) {
+            MeeReciprocals rc;
+            rc.inv_c = MEE ? recip_f64(mp.c) : 0.0;
+            rc.inv_l2b = MEE ? recip_f64(mp.l2b) : 0.0;
+            constexpr int kGroup = CT < 16 ? CT : 16; // elements per call
+            constexpr int kGroupBytes = kGroup * NB / 8;
+            auto group = [&](auto off) {
+                constexpr int OFF = decltype(off)::value;
+                uint32_t w[Rec<NB>::WORDS];
+#pragma unroll
+                for (int k = 0; k < Rec<NB>::WORDS; k++) w[k] = 0;
+                // padding: v = 0 with r = 1/2 is never in doubt
+                const Sixteen<decltype(ev), OFF, CT> v16{ev, 0.0f};
+                const Sixteen<decltype(rv), OFF, CT> r16{rv, 0.5f};
+                estimate_codes<NB, MEE>(v16, r16, d, rc, w);
+#pragma unroll
+                for (int k = 0; k < kGroupBytes; k++) cb[OFF * NB / 8 + k] = (uint8_t)(w[k >> 2] >> (8 * (k & 3)));
+            };
+            group(std::integral_constant<int, 0>{});
+            if constexpr (CT > 16) group(std::integral_constant<int, 16>{});
+            return;
+        }
+    }
+    if (CT && ordinary)
         codes(std::true_type{});
     else
         codes(std::false_type{});
@@ -253,12 +346,13 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
 
 // ---- decompress ----------------------------------------------------------------
 
-// CT: the chunk size when it is 8 or 32 and dst is 16-byte aligned, else 0
-template <int DT, bool HIER, bool MEE, bool ADD, int CT>
+// CT: the chunk size when it is 8 or 32 and dst is 16-byte aligned, else 0; NB as in generic_compress_kernel
+template <int DT, bool HIER, bool MEE, bool ADD, int CT, int NB>
 __global__ __launch_bounds__(kGenericBlock) void generic_decompress_kernel(
-    const uint8_t *__restrict__ src, void *__restrict__ dst, int64_t nchunks, int nbits, int Crt,
+    const uint8_t *__restrict__ src, void *__restrict__ dst, int64_t nchunks, int nbits_rt, int Crt,
     MeeParams mp)
 {
+    const int nbits = NB ? NB : nbits_rt;
     typedef ElemIO<DT> IO;
     constexpr int CR = CT ? CT : 1;
     constexpr int S = ChunkShape<DT, CR>::kSlots;
@@ -366,9 +460,16 @@ static hipError_t launch_compress_t(const void *src, uint8_t *dst, const void *r
     int64_t nchunks = n / C;
     unsigned grid = (unsigned)((nchunks + kGenericBlock - 1) / kGenericBlock);
     const int ct = (aligned16(src) && aligned16(rnd) && (C == 8 || C == 32)) ? C : 0;
-#define DQ_GENERIC_COMPRESS(RDT, CT)                                                                                    \
-    hipLaunchKernelGGL((generic_compress_kernel<DT, RDT, HIER, MEE, CT>), dim3(grid), dim3(kGenericBlock), 0, stream, src, \
+#define DQ_GENERIC_COMPRESS_NB(RDT, CT, NB)                                                                                 \
+    hipLaunchKernelGGL((generic_compress_kernel<DT, RDT, HIER, MEE, CT, NB>), dim3(grid), dim3(kGenericBlock), 0, stream, src, \
                        dst, rnd, nchunks, nbits, C, mp)
+#define DQ_GENERIC_COMPRESS(RDT, CT)                                  \
+    do {                                                              \
+        if (CT != 0 && nbits == 2) DQ_GENERIC_COMPRESS_NB(RDT, CT, (CT ? 2 : 0));      \
+        else if (CT != 0 && nbits == 4) DQ_GENERIC_COMPRESS_NB(RDT, CT, (CT ? 4 : 0)); \
+        else if (CT != 0 && nbits == 8) DQ_GENERIC_COMPRESS_NB(RDT, CT, (CT ? 8 : 0)); \
+        else DQ_GENERIC_COMPRESS_NB(RDT, CT, 0);                      \
+    } while (0)
     if (DT == DQ_F32 && rand_bf16) {
         if (ct == 32) DQ_GENERIC_COMPRESS(DQ_BF16, 32);
         else if (ct == 8) DQ_GENERIC_COMPRESS(DQ_BF16, 8);
@@ -379,6 +480,7 @@ static hipError_t launch_compress_t(const void *src, uint8_t *dst, const void *r
         else DQ_GENERIC_COMPRESS(DT, 0);
     }
 #undef DQ_GENERIC_COMPRESS
+#undef DQ_GENERIC_COMPRESS_NB
     return hipGetLastError();
 }
 
@@ -389,9 +491,16 @@ static hipError_t launch_decompress_t(const uint8_t *src, void *dst, int64_t n, 
     int64_t nchunks = n / C;
     unsigned grid = (unsigned)((nchunks + kGenericBlock - 1) / kGenericBlock);
     const int ct = (aligned16(dst) && (C == 8 || C == 32)) ? C : 0;
-#define DQ_GENERIC_DECOMPRESS(ADD, CT)                                                                                    \
-    hipLaunchKernelGGL((generic_decompress_kernel<DT, HIER, MEE, ADD, CT>), dim3(grid), dim3(kGenericBlock), 0, stream, src, \
+#define DQ_GENERIC_DECOMPRESS_NB(ADD, CT, NB)                                                                                 \
+    hipLaunchKernelGGL((generic_decompress_kernel<DT, HIER, MEE, ADD, CT, NB>), dim3(grid), dim3(kGenericBlock), 0, stream, src, \
                        dst, nchunks, nbits, C, mp)
+#define DQ_GENERIC_DECOMPRESS(ADD, CT)                                \
+    do {                                                              \
+        if (CT != 0 && nbits == 2) DQ_GENERIC_DECOMPRESS_NB(ADD, CT, (CT ? 2 : 0));      \
+        else if (CT != 0 && nbits == 4) DQ_GENERIC_DECOMPRESS_NB(ADD, CT, (CT ? 4 : 0)); \
+        else if (CT != 0 && nbits == 8) DQ_GENERIC_DECOMPRESS_NB(ADD, CT, (CT ? 8 : 0)); \
+        else DQ_GENERIC_DECOMPRESS_NB(ADD, CT, 0);                    \
+    } while (0)
     if (add) {
         if (ct == 32) DQ_GENERIC_DECOMPRESS(true, 32);
         else if (ct == 8) DQ_GENERIC_DECOMPRESS(true, 8);
@@ -402,6 +511,7 @@ static hipError_t launch_decompress_t(const uint8_t *src, void *dst, int64_t n, 
         else DQ_GENERIC_DECOMPRESS(false, 0);
     }
 #undef DQ_GENERIC_DECOMPRESS
+#undef DQ_GENERIC_DECOMPRESS_NB
     return hipGetLastError();
 }
 

@@ -181,22 +181,25 @@ def test_special_values(capi, oracle, dt, strategy):
 
 @pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [2, 3])
-def test_random_values_on_the_rounding_boundary(capi, oracle, nbits, strategy):
+@pytest.mark.parametrize("C", [16, 8, 32])
+def test_random_values_on_the_rounding_boundary(capi, oracle, nbits, strategy, C):
     """The kernels decide most codes from a cheap estimate of the coordinate and redo an element with the reference's
     exact chain when coordinate - random value comes close to an integer.  Here every random value is the fractional
     part of its element's coordinate (to float32 accuracy, and one or two float32 steps beside it), so every element
     sits on that boundary: bytes must still be the oracle's."""
     from helpers import unpack_stream
+    if (C * nbits) % 8:
+        pytest.skip("the code bytes of a chunk must be whole")
     nsc = 40
-    n = nsc * 256
+    n = nsc * 16 * C
     g = torch.Generator().manual_seed(900 + 10 * nbits + strategy)
     scale = torch.exp(torch.randn(nsc, 1, generator=g) * 2.0 - 6.0)
-    src = (torch.randn(nsc, 256, generator=g) * scale).reshape(-1)
+    src = (torch.randn(nsc, 16 * C, generator=g) * scale).reshape(-1)
     src[5::97] = 0.0
     # the quantisation steps the oracle uses: from the records of a first pass with any random values
-    enc = oracle.scaling_compress(src.numpy(), np.full(n, 0.5, np.float32), n, nbits, 16, strategy, F32)
-    _, (q, unit) = unpack_stream(enc, n, nbits, 16, strategy)
-    step = q.astype(np.float64).repeat(16) * bits_to_f32(unit, BF16).astype(np.float64).repeat(256)
+    enc = oracle.scaling_compress(src.numpy(), np.full(n, 0.5, np.float32), n, nbits, C, strategy, F32)
+    _, (q, unit) = unpack_stream(enc, n, nbits, C, strategy)
+    step = q.astype(np.float64).repeat(C) * bits_to_f32(unit, BF16).astype(np.float64).repeat(16 * C)
     x = src.numpy().astype(np.float64) / step
     if strategy == 3:
         _, params = capi.mee_lookup_table(nbits)
@@ -208,12 +211,12 @@ def test_random_values_on_the_rounding_boundary(capi, oracle, nbits, strategy):
         for _ in range(abs(shift)):
             rnd = np.nextafter(rnd, np.float32(2.0 if shift > 0 else -1.0))
         rnd = np.clip(rnd, 0.0, 1.0).astype(np.float32)
-        tag = "boundary b=%d s=%d shift=%d" % (nbits, strategy, shift)
-        _roundtrip(capi, oracle, F32, n, nbits, 16, strategy, src, torch.from_numpy(rnd), tag)
+        tag = "boundary C=%d b=%d s=%d shift=%d" % (C, nbits, strategy, shift)
+        _roundtrip(capi, oracle, F32, n, nbits, C, strategy, src, torch.from_numpy(rnd), tag)
         # the fused ring step sees the same situation through its accumulated input
         if shift == 0:
             inp = torch.zeros(n)
-            _dec_comp(capi, oracle, F32, n, nbits, 16, strategy, src, inp, torch.from_numpy(rnd), torch.from_numpy(rnd), tag)
+            _dec_comp(capi, oracle, F32, n, nbits, C, strategy, src, inp, torch.from_numpy(rnd), torch.from_numpy(rnd), tag)
 
 
 def _wide_source(n, tdt, seed):
