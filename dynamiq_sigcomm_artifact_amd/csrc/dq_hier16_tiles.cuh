@@ -95,14 +95,12 @@ struct Center {
     WorldDiv wd;
 };
 
+// v holds the chunk's 16 elements as loaded when `whole` (the chunk lies inside [0, n_valid)), else they are read here
 template <int DT>
-__device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int64_t e0, const Center &ctr, int64_t sc_src,
-                                             bool vec)
+__device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int64_t e0, const Center &ctr, float mean, bool whole)
 {
     float t[16];
-    const float mean = ctr.mean[sc_src];
-    if (e0 + 16 <= ctr.n_valid) {
-        v.load(src, e0, vec);
+    if (whole) {
 #pragma unroll
         for (int i = 0; i < 16; i++) t[i] = ctr.wd(v.get(i)) - mean;
     } else {
@@ -167,29 +165,37 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
     const bool active = row < rows_here;
     const int total = rows_here * RC::REC;
 
-    // all global loads of the tile are issued before anything waits on them
-    Raw16<DT> v;
-    Raw16<RDT> r;
-    if (active) {
-        if constexpr (RDT != DQ_PHILOX) r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
-        const int64_t sc_src = rows ? (int64_t)rows[sc0 + row] : sc0 + row;
-        if constexpr (RDT == DQ_PHILOX) r.generate(key, sc_src * 16 + j); // keyed by the chunk's place in the source vector
-        if (ctr.mean)
-            center_chunk<DT>(v, src, (sc_src * 16 + j) * 16, ctr, sc_src, vec & 1);
-        else
-            v.load(src, (sc_src * 16 + j) * 16, vec & 1);
-    } else {
-        v.zero();
-        r.zero();
-    }
+    // all global loads of the tile are issued before anything waits on them: the received records and the level
+    // table first (they do not depend on the row list), then the row index, the random values, the mean and the chunk
     WinRegs wr;
     if (FUSED) wr = window_fetch(recv + sc0 * RC::REC, total, lane);
-    if (MEE && FUSED) {
-        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
+    TableRegs<NBITS> tr;
+    if (MEE && FUSED) tr = table_fetch<NBITS>(mp, lane);
+    Raw16<DT> v;
+    Raw16<RDT> r;
+    v.zero();
+    r.zero();
+    int64_t sc_src = sc0 + row, e0 = 0;
+    float mean = 0.0f;
+    bool whole = true;
+    if (active) {
+        if constexpr (RDT != DQ_PHILOX) r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
+        if (rows) sc_src = rows[sc0 + row];
+        e0 = (sc_src * 16 + j) * 16;
+        if (ctr.mean) {
+            mean = ctr.mean[sc_src];
+            whole = e0 + 16 <= ctr.n_valid;
+        }
+        if (whole) v.load(src, e0, vec & 1);
+    }
+    if (active) {
+        if constexpr (RDT == DQ_PHILOX) r.generate(key, sc_src * 16 + j); // keyed by the chunk's place in the source vector
+        if (ctr.mean) center_chunk<DT>(v, src, e0, ctr, mean, whole);
     }
 
     if (FUSED) {
         const int mis_in = window_commit(win_in, wr, recv + sc0 * RC::REC, total, lane);
+        if (MEE) table_commit<NBITS>(table, tr, lane);
         wave_lds_sync();
         if (active) {
             const uint8_t *rec = win_in + mis_in + row * RC::REC;
@@ -247,13 +253,13 @@ __device__ __forceinline__ void decompress_tile(const uint8_t *__restrict__ src,
     }
     Raw16<DT> acc;
     if (ADD && active) acc.load(dst, d_own * 256 + j * 16, vec);
-    float mean = 0.0f;
-    if (stats && active) mean = bf16_bits_to_f32(stats[2 * d_own]);
-    if (MEE) {
-        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
-    }
+    uint32_t mean_bits = 0; // widened where it is used, so that nothing waits for this load here
+    if (stats && active) mean_bits = stats[2 * d_own];
+    TableRegs<NBITS> tr;
+    if (MEE) tr = table_fetch<NBITS>(mp, lane);
 
     const int mis_in = window_commit(win_in, wr, src + sc0 * RC::REC, total, lane);
+    if (MEE) table_commit<NBITS>(table, tr, lane);
     wave_lds_sync();
     Raw16<DT> out;
     if (active) {
@@ -269,6 +275,7 @@ __device__ __forceinline__ void decompress_tile(const uint8_t *__restrict__ src,
         chunk_decode<NBITS, MEE, ADD>(cw, cq, ub, table, t);
         out.set(t);
         if (stats) {
+            const float mean = bf16_bits_to_f32(mean_bits);
 #pragma unroll
             for (int i = 0; i < 16; i++) t[i] = out.get(i) + mean;
             out.set(t);

@@ -196,10 +196,10 @@ __global__ __launch_bounds__(64) void tile16_decompress_kernel(const uint8_t *__
     const WinRegs wr = window_fetch(gin, total, lane);
     Raw16<DT> acc;
     if (ADD && active) acc.load(dst, e0 + lane * 16, vec);
-    if (MEE) {
-        for (int k = lane; k < (1 << NBITS); k += 64) table[k] = f16_bits_to_f32(mp.table[k]);
-    }
+    TableRegs<NBITS> tr;
+    if (MEE) tr = table_fetch<NBITS>(mp, lane);
     const int mis_in = window_commit(win_in, wr, gin, total, lane);
+    if (MEE) table_commit<NBITS>(table, tr, lane);
     wave_lds_sync();
 
     Raw16<DT> out;

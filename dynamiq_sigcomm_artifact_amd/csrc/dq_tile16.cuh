@@ -199,6 +199,41 @@ template <> struct Raw16<DQ_PHILOX> {
     __device__ __forceinline__ bool unit_interval() const { return true; }
 };
 
+// ---- the MEE level table on its way into LDS -------------------------------------------------------
+//
+// The table comes with the kernel arguments as 2^NBITS binary16 patterns.  A lane fetches its pairs of entries with the
+// other loads of its tile (one or two 4-byte loads, no wait in between) and converts and stores them as floats once the
+// tile's own data has arrived.
+template <int NBITS> struct TableRegs {
+    static constexpr int kPairs = (1 << NBITS) / 2;
+    static constexpr int kPerLane = (kPairs + 63) / 64;
+    uint32_t pair[kPerLane];
+};
+
+template <int NBITS, class ARG> __device__ __forceinline__ TableRegs<NBITS> table_fetch(const ARG &mp, int lane)
+{
+    TableRegs<NBITS> t;
+    const uint32_t *pairs = reinterpret_cast<const uint32_t *>(mp.table); // 4-byte aligned inside the argument block
+#pragma unroll
+    for (int j = 0; j < TableRegs<NBITS>::kPerLane; j++) {
+        const int k = lane + 64 * j;
+        t.pair[j] = k < TableRegs<NBITS>::kPairs ? pairs[k] : 0u;
+    }
+    return t;
+}
+
+template <int NBITS> __device__ __forceinline__ void table_commit(float *table, const TableRegs<NBITS> &t, int lane)
+{
+#pragma unroll
+    for (int j = 0; j < TableRegs<NBITS>::kPerLane; j++) {
+        const int k = lane + 64 * j;
+        if (k < TableRegs<NBITS>::kPairs) {
+            table[2 * k] = f16_bits_to_f32(t.pair[j] & 0xffffu);
+            table[2 * k + 1] = f16_bits_to_f32(t.pair[j] >> 16);
+        }
+    }
+}
+
 // ---- record windows --------------------------------------------------------------------
 
 // the (up to two) aligned 128-bit pieces of a packed run this lane moves
