@@ -47,9 +47,11 @@ __device__ __forceinline__ Segment locate(const MixedPlan &p, int block)
     s.cls = 3; s.tile = 0; s.cnt = 0; s.row0 = 0; s.pos0 = 0; s.byte_off = 0;
     int64_t pos = 0, off = 0;
     int t = block;
+    // the three loads leave together, ahead of the arithmetic (taken one by one inside the loop, each waited for its own)
+    const int counts[3] = {p.counts[0], p.counts[1], p.counts[2]};
 #pragma unroll
     for (int g = 0; g < 3; g++) {
-        const int n = min(max(p.counts[g], 0), p.nsc - (int)pos); // a corrupt count cannot lead outside a region or the pool
+        const int n = min(max(counts[g], 0), p.nsc - (int)pos); // a corrupt count cannot lead outside a region or the pool
         const int per = (n + p.world - 1) / p.world;
         const int begin = (int)min((int64_t)per * p.chunk, (int64_t)n);
         const int cnt = min(per, n - begin);
