@@ -1,8 +1,8 @@
 // Fast Walsh-Hadamard transform (unnormalised, Sylvester order) and the blocked
 // randomized transform built on it.
 //
-// One kernel does everything: a workgroup owns a tile of 2^kt floats in LDS and
-// applies the butterfly stages of a contiguous range of index bits to it.
+// A pass: a workgroup owns a tile of 2^kt floats in LDS and applies the butterfly
+// stages of a contiguous range of index bits to it.
 //   * contiguous pass: the tile is 2^kt consecutive floats and the stages are
 //     strides 1 .. 2^(kt-1) (or fewer when the transform block is smaller than
 //     the tile, so several small blocks share one tile);
@@ -15,9 +15,13 @@
 // which is the order of csrc/cuda_hadamard.cu:66-157,205-274,534-605, so the
 // result is bit-identical to a plain stage-by-stage FWHT.
 //
-// Inside the tile the stages are done four at a time (radix 16) on registers;
-// the LDS index is padded by one float per 16 (i + i/16), which keeps every
-// access pattern used here free of bank conflicts.
+// This file plans the passes.  The kernel here, fwht_tile_kernel, does the stages of
+// a tile four at a time (radix 16) between LDS and registers and can take a quantiser
+// at either end (THC's levels, EDEN's bit planes); plain passes of at least 1024
+// elements go to the kernels of dq_rht_scaling.hip, which do the first four stages
+// on the registers a lane loads into and need fewer LDS passes.  The LDS index is
+// padded by one float per 16 (i + i/16), which keeps every access pattern used
+// here free of bank conflicts.
 #include "dq_fwht.cuh"
 #include "dq_launch.h"
 
@@ -253,6 +257,9 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.out_levels = nullptr; a.uniform = thc.uniform; a.out_lo = thc.out_lo; a.out_delta = thc.out_delta;
     a.out_top = thc.out_top;
     const int sign_fwd = (sign && !inverse) ? 1 : 0, sign_inv = (sign && inverse) ? 2 : 0;
+    // without a quantiser folded into its ends a contiguous pass runs as the chunk-first kernel of dq_rht_scaling.hip
+    const bool plain_in = !thc.in_levels && !thc.in_planes;
+    const bool plain = plain_in && !thc.out_levels && !thc.post_scale;
 
     if (kb <= kMaxTileBits) {
         // single pass; small blocks share a tile
@@ -267,6 +274,8 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
         a.in_planes = thc.in_planes;
         a.post_scale = thc.post_scale;
         const int64_t ntiles = (n + ((int64_t)1 << kt) - 1) >> kt;
+        if (plain && kt >= 10)
+            return launch_rht_tile(x, sign, sign_packed ? 1 : 0, n, kt, kb, scale, apply_scale, sign_fwd | sign_inv, a.vec, stream);
         return launch_tile(a, ntiles, stream);
     }
 
@@ -276,7 +285,8 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.apply_scale = 0; a.sign_mode = sign_fwd; a.vec = vec16;
     a.in_levels = thc.in_levels;
     a.in_planes = thc.in_planes;
-    hipError_t e = launch_tile(a, n >> kt, stream);
+    hipError_t e = plain_in ? launch_rht_tile(x, sign, sign_packed ? 1 : 0, n, kt, kt, scale, 0, sign_fwd, a.vec, stream)
+                            : launch_tile(a, n >> kt, stream);
     if (e != hipSuccess) return e;
     a.in_levels = nullptr;
     a.in_planes = nullptr;
@@ -295,7 +305,10 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
         a.out_levels = last ? thc.out_levels : nullptr;
         a.post_scale = last ? thc.post_scale : nullptr;
         a.vec = vec16;
-        e = launch_tile(a, n >> a.kt, stream);
+        if (r >= 4 && !a.out_levels && !a.post_scale && (n & (((int64_t)1 << (s + r)) - 1)) == 0)
+            e = launch_rht_strided(x, sign, sign_packed ? 1 : 0, n, r, s, scale, a.apply_scale, a.sign_mode, a.vec, stream);
+        else
+            e = launch_tile(a, n >> a.kt, stream);
         if (e != hipSuccess) return e;
         s += r;
     }

@@ -122,6 +122,10 @@ hipError_t launch_rht_compress_mfma16(const float *src, const void *sign, int si
                                       float scale, const MeeParams &mp, uint64_t seed, uint64_t step, hipStream_t stream);
 hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign_bits, float *dst, int64_t n, int64_t block,
                                   float scale, int nbits, bool mee, const MeeParams &mp, hipStream_t stream);
+hipError_t launch_rht_tile(float *x, const void *sign, int sign_bits, int64_t n, int kt, int kb, float scale, int apply_scale,
+                           int sign_mode, int vec, hipStream_t stream);
+hipError_t launch_rht_strided(float *x, const void *sign, int sign_bits, int64_t n, int rbits, int sbits, float scale,
+                              int apply_scale, int sign_mode, int vec, hipStream_t stream);
 
 // EDEN Lloyd-Max quantiser + packer, THC uniform quantiser (dq_eden.hip)
 int64_t eden_work_doubles(int64_t n);

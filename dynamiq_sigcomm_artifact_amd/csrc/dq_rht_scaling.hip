@@ -266,6 +266,138 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
     }
 }
 
+// The transform alone (dq_rht_blocked, the first pass of a long dq_hadamard) with the structure of the two kernels
+// above: a lane loads its chunk of 16 consecutive floats, does the stages of strides 1..8 on its registers, the rest
+// runs as LDS passes of up to five stages, and the tile leaves as coalesced 16-byte stores with the scale and (inverse
+// direction) the sign flip.  Against the all-in-LDS kernel of dq_hadamard.hip: two or three LDS passes instead of four,
+// and a thread's loads issued together.  In place: a workgroup reads and writes only its own tile.
+// sign_mode: 0 no flip, 1 flip on load, 2 flip on store
+__global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_mode, int apply_scale)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int tile = 1 << a.kt;
+    const int64_t origin = (int64_t)blockIdx.x << a.kt;
+    RhtTileArgs in = a;
+    if (sign_mode != 1) in.sign = nullptr;
+    const int nchunks = tile >> 4;
+    if (nchunks == 2 * nthreads) {
+        // 2^15 tiles: both chunks of a thread are loaded before either is used
+        float v[16], w[16];
+        load_chunk(v, x, in, origin + tid * 16);
+        load_chunk(w, x, in, origin + (tid + nthreads) * 16);
+        chunk_stages(v, a.kb);
+        chunk_stages(w, a.kb);
+        float *mine = lds + tid * 17, *other = lds + (tid + nthreads) * 17;
+#pragma unroll
+        for (int i = 0; i < 16; i++) mine[i] = v[i];
+#pragma unroll
+        for (int i = 0; i < 16; i++) other[i] = w[i];
+    } else {
+        for (int c = tid; c < nchunks; c += nthreads) {
+            float v[16];
+            load_chunk(v, x, in, origin + c * 16);
+            chunk_stages(v, a.kb);
+            float *mine = lds + c * 17; // pad_idx(16 c + i) = 17 c + i
+#pragma unroll
+            for (int i = 0; i < 16; i++) mine[i] = v[i];
+        }
+    }
+    fwht_lds_stages_after4(lds, a.kt, a.kb, tid, nthreads);
+    const float scale = apply_scale ? a.scale : 1.0f;
+    if (a.vec) {
+        for (int i = tid * 4; i < tile; i += nthreads * 4) {
+            const int64_t g = origin + i;
+            if (g >= a.n) continue;
+            const int q = pad_idx(i);
+            float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
+            if (apply_scale) { v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale; }
+            if (sign_mode == 2) flip4(v, a, g);
+            *reinterpret_cast<float4 *>(x + g) = v;
+        }
+    } else {
+        for (int i = tid; i < tile; i += nthreads) {
+            const int64_t g = origin + i;
+            if (g >= a.n) continue;
+            float v = lds[pad_idx(i)];
+            if (apply_scale) v *= scale;
+            x[g] = sign_mode == 2 ? flip1(v, a, g) : v;
+        }
+    }
+}
+
+// A later pass of a transform longer than one tile: index bits [sbits, sbits + rbits) of the vector.  A tile is
+// 2^rbits rows of 32 consecutive floats (128 bytes), row stride 2^sbits elements; in LDS it is row-major, so row bit b
+// is tile bit b + 5.  A thread owns column tid % 32 of sixteen consecutive rows: it loads them (every load instruction of
+// a wave covers two whole 128-byte row segments), does the four lowest row stages on its registers and leaves the other
+// rbits - 4 (at most 6) to one or two LDS passes.  sign_mode: 0, or 2 = flip on store (the last pass of an inverse).
+__global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbits, int sbits, int sign_mode, int apply_scale)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int tile = 1 << (rbits + 5);
+    const int64_t mids = (int64_t)1 << (sbits - 5);
+    const int64_t hi = blockIdx.x / mids, mid = blockIdx.x % mids;
+    const int64_t origin = (hi << (sbits + rbits)) + (mid << 5);
+    const int col = tid & 31;
+    const int groups = tile >> 9; // groups of sixteen rows
+    if (groups == 2 * (nthreads >> 5)) {
+        // 1024 rows: both groups of a thread are loaded before either is used
+        const int r0 = (tid >> 5) * 16, r1 = r0 + (nthreads >> 5) * 16;
+        float v[16], w[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = x[origin + ((int64_t)(r0 + j) << sbits) + col];
+#pragma unroll
+        for (int j = 0; j < 16; j++) w[j] = x[origin + ((int64_t)(r1 + j) << sbits) + col];
+        butterflies<4>(v);
+        butterflies<4>(w);
+#pragma unroll
+        for (int j = 0; j < 16; j++) lds[pad_idx((r0 + j) * 32 + col)] = v[j];
+#pragma unroll
+        for (int j = 0; j < 16; j++) lds[pad_idx((r1 + j) * 32 + col)] = w[j];
+    } else {
+        for (int grp = tid >> 5; grp < groups; grp += nthreads >> 5) {
+            float v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = x[origin + ((int64_t)(grp * 16 + j) << sbits) + col];
+            butterflies<4>(v);
+#pragma unroll
+            for (int j = 0; j < 16; j++) lds[pad_idx((grp * 16 + j) * 32 + col)] = v[j];
+        }
+    }
+    __syncthreads();
+#define DQ_PASS(P, M)                                     \
+    lds_pass<P, M>(lds, tile >> M, tid, nthreads);        \
+    __syncthreads();
+    switch (rbits - 4) {
+    case 1: DQ_PASS(9, 1) break;
+    case 2: DQ_PASS(9, 2) break;
+    case 3: DQ_PASS(9, 3) break;
+    case 4: DQ_PASS(9, 4) break;
+    case 5: DQ_PASS(9, 5) break;
+    case 6: DQ_PASS(9, 3) DQ_PASS(12, 3) break;
+    default: break;
+    }
+#undef DQ_PASS
+    if (a.vec) {
+        for (int i = tid * 4; i < tile; i += nthreads * 4) {
+            const int64_t g = origin + ((int64_t)(i >> 5) << sbits) + (i & 31);
+            const int q = pad_idx(i);
+            float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
+            if (apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
+            if (sign_mode == 2) flip4(v, a, g);
+            *reinterpret_cast<float4 *>(x + g) = v;
+        }
+    } else {
+        for (int i = tid; i < tile; i += nthreads) {
+            const int64_t g = origin + ((int64_t)(i >> 5) << sbits) + (i & 31);
+            float v = lds[pad_idx(i)];
+            if (apply_scale) v *= a.scale;
+            x[g] = sign_mode == 2 ? flip1(v, a, g) : v;
+        }
+    }
+}
+
 // ---- blocks of 2^15: the tile in two halves -----------------------------------------------------------
 //
 // A 2^15 tile with its padding needs 139 KB of LDS: one workgroup per CU, whose load, butterfly and
@@ -400,6 +532,55 @@ __global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel
     }
 }
 
+// the transform alone on blocks of 2^15, the tile in two halves as above
+__global__ __launch_bounds__(kSplitThreads, 8) void rht_tile_split_kernel(float *__restrict__ x, RhtTileArgs a, int sign_mode,
+                                                                      int apply_scale)
+{
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int tid = threadIdx.x;
+    const int64_t origin = (int64_t)blockIdx.x << kSplitBits;
+    RhtTileArgs in = a;
+    if (sign_mode != 1) in.sign = nullptr;
+    float va[16], vb[16];
+    load_chunk(va, x, in, origin + tid * 16);
+    load_chunk(vb, x, in, origin + (1 << kHalfBits) + tid * 16);
+    butterflies<4>(va);
+    butterflies<4>(vb);
+    half_block_stages(va, lds, tid);
+    half_block_stages(vb, lds, tid);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const float p = va[i], q = vb[i];
+        va[i] = p + q;
+        vb[i] = p - q;
+    }
+    // store one half after the other through the LDS, so that every store instruction covers 1 KiB contiguously
+    float *mine = lds + tid * 17;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) mine[i] = h ? vb[i] : va[i];
+        __syncthreads();
+        const int64_t half_origin = origin + ((int64_t)h << kHalfBits);
+        if (a.vec) {
+            for (int i = tid * 4; i < (1 << kHalfBits); i += kSplitThreads * 4) {
+                const int q = pad_idx(i);
+                float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
+                if (apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
+                if (sign_mode == 2) flip4(v, a, half_origin + i);
+                *reinterpret_cast<float4 *>(x + half_origin + i) = v;
+            }
+        } else {
+            for (int i = tid; i < (1 << kHalfBits); i += kSplitThreads) {
+                float v = lds[pad_idx(i)];
+                if (apply_scale) v *= a.scale;
+                x[half_origin + i] = sign_mode == 2 ? flip1(v, a, half_origin + i) : v;
+            }
+        }
+        __syncthreads();
+    }
+}
+
 constexpr int kPrefTileBits = 13; // 32 KiB tiles: eight waves, one run each, several workgroups per CU
 
 struct Geometry {
@@ -519,6 +700,50 @@ hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign
                                   int nbits, bool mee, const MeeParams &mp, hipStream_t stream)
 {
     DQ_NBITS_MEE(run_decompress, 0, src, sign, sign_bits, dst, n, block, scale, mp, stream)
+}
+
+// stages [0, kb) of every aligned block of 2^kb elements, tiles of 2^kt contiguous elements (10 <= kt <= 15, kb <= kt);
+// vec: 16-byte accesses to x (and to a float sign vector) are allowed
+hipError_t launch_rht_tile(float *x, const void *sign, int sign_bits, int64_t n, int kt, int kb, float scale, int apply_scale,
+                           int sign_mode, int vec, hipStream_t stream)
+{
+    if (kt < 10 || kt > 15 || kb > kt || kb < 0) return hipErrorInvalidValue;
+    RhtTileArgs a;
+    a.sign = sign; a.sign_bits = sign_bits; a.n = n; a.kt = kt; a.kb = kb; a.scale = scale; a.vec = vec;
+    const int tile = 1 << kt;
+    if (kt == kSplitBits && kb == kSplitBits && (n & (tile - 1)) == 0) {
+        // whole blocks of 2^15: half the LDS, two workgroups per CU
+        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float);
+        hipError_t es = allow_lds(rht_tile_split_kernel, half_lds);
+        if (es != hipSuccess) return es;
+        hipLaunchKernelGGL(rht_tile_split_kernel, dim3((unsigned)(n >> kSplitBits)), dim3(kSplitThreads), half_lds, stream, x, a,
+                           sign ? sign_mode : 0, apply_scale);
+        return hipGetLastError();
+    }
+    const unsigned threads = (unsigned)std::min(1024, tile / 16);
+    const size_t lds = (size_t)padded_tile_floats(kt) * sizeof(float);
+    hipError_t e = allow_lds(rht_tile_kernel, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(rht_tile_kernel, dim3((unsigned)((n + tile - 1) >> kt)), dim3(threads), lds, stream, x, a,
+                       sign ? sign_mode : 0, apply_scale);
+    return hipGetLastError();
+}
+
+// stages of the index bits [sbits, sbits + rbits) of x[0 .. n), n a multiple of 2^(sbits + rbits); 4 <= rbits <= 10, sbits >= 5
+hipError_t launch_rht_strided(float *x, const void *sign, int sign_bits, int64_t n, int rbits, int sbits, float scale,
+                              int apply_scale, int sign_mode, int vec, hipStream_t stream)
+{
+    if (rbits < 4 || rbits > 10 || sbits < 5 || (n & (((int64_t)1 << (sbits + rbits)) - 1)) != 0) return hipErrorInvalidValue;
+    RhtTileArgs a;
+    a.sign = sign; a.sign_bits = sign_bits; a.n = n; a.kt = rbits + 5; a.kb = 0; a.scale = scale; a.vec = vec;
+    const int tile = 1 << (rbits + 5);
+    const unsigned threads = (unsigned)std::min(1024, tile / 16);
+    const size_t lds = (size_t)padded_tile_floats(rbits + 5) * sizeof(float);
+    hipError_t e = allow_lds(rht_strided_kernel, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(rht_strided_kernel, dim3((unsigned)(n >> (rbits + 5))), dim3(threads), lds, stream, x, a, rbits, sbits,
+                       sign ? sign_mode : 0, apply_scale);
+    return hipGetLastError();
 }
 
 } // namespace dq

@@ -77,7 +77,7 @@ def test_superchunk_constant_block(capi):
     assert stats.float().tolist() == [c / W, 256 * (c / W) ** 2] * 2
 
 
-@pytest.mark.parametrize("k", [0, 1, 2, 3, 5, 8, 10, 12, 13, 14, 15, 16, 18, 20, 22])
+@pytest.mark.parametrize("k", [0, 1, 2, 3, 5, 8, 10, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24])
 def test_hadamard_whole_vector(capi, oracle, k):
     n = 1 << k
     g = torch.Generator().manual_seed(k)
@@ -129,11 +129,11 @@ def test_hadamard_module_functions(eden_utils, oracle):
         eden_utils.Hadamard(torch.zeros(16, device=DEV, dtype=torch.bfloat16))
 
 
-@pytest.mark.parametrize("kb", [4, 10, 11, 12, 13, 14, 15, 17])
+@pytest.mark.parametrize("kb", [2, 4, 8, 10, 11, 12, 13, 14, 15, 16, 17, 20, 23])
 @pytest.mark.parametrize("inverse", [False, True])
 def test_rht_blocked(capi, oracle, kb, inverse):
     block = 1 << kb
-    nblocks = 3 if kb <= 15 else 2
+    nblocks = 3 if kb <= 15 else (2 if kb < 23 else 1)
     n = block * nblocks
     g = torch.Generator().manual_seed(kb)
     x = torch.randn(n, generator=g) * 1e-3
