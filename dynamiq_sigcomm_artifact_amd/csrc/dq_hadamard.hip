@@ -15,11 +15,13 @@
 // which is the order of csrc/cuda_hadamard.cu:66-157,205-274,534-605, so the
 // result is bit-identical to a plain stage-by-stage FWHT.
 //
-// This file plans the passes.  The kernel here, fwht_tile_kernel, does the stages of
-// a tile four at a time (radix 16) between LDS and registers and can take a quantiser
-// at either end (THC's levels, EDEN's bit planes); plain passes of at least 1024
-// elements go to the kernels of dq_rht_scaling.hip, which do the first four stages
-// on the registers a lane loads into and need fewer LDS passes.  The LDS index is
+// This file plans the passes.  Passes of at least 1024 elements go to the kernels of
+// dq_rht_scaling.hip, which do the first four stages on the registers a lane loads
+// into and need fewer LDS passes; the kernel here, fwht_tile_kernel, does the stages
+// of a tile four at a time (radix 16) between LDS and registers and serves what is
+// left: small tiles, strided passes over fewer than four bits, buffers without
+// 16-byte alignment.  Either kind can take a quantiser at the ends of the transform
+// (THC's levels, EDEN's bit planes and scale).  The LDS index is
 // padded by one float per 16 (i + i/16), which keeps every access pattern used
 // here free of bank conflicts.
 #include "dq_fwht.cuh"
@@ -223,20 +225,8 @@ constexpr int kMaxTileBits = 15; // 2^15 floats = 128 KiB (+ padding) of the 160
 constexpr int kPrefTileBits = 13; // 32 KiB tiles keep several workgroups per CU in flight
 constexpr int kStridedCols = 5;   // 32 consecutive floats (128 B) per row of a strided tile
 
-// transform index bits [0, kb) of every aligned block of 2^kb elements of x[0..n)
-// THC's quantiser at the ends of a transform: `in` replaces the load of the first pass, `out` the store of the last
-struct ThcEnds {
-    const uint16_t *in_levels = nullptr;
-    const float *in_step = nullptr, *in_lo = nullptr;
-    uint16_t *out_levels = nullptr;
-    const float *uniform = nullptr, *out_lo = nullptr, *out_delta = nullptr;
-    float out_top = 0.0f;
-    // EDEN: `in_planes` replaces the load of the first pass, `post_scale` multiplies the store of the last
-    const uint32_t *in_planes = nullptr;
-    const float *in_centroids = nullptr;
-    int in_nbits = 0;
-    const float *post_scale = nullptr;
-};
+// transform index bits [0, kb) of every aligned block of 2^kb elements of x[0..n); `thc`: quantisers at the ends
+typedef TransformEnds ThcEnds;
 
 // sign: float +-1 values, or (sign_packed) the bit vector of dq_pack_signs; may be null
 static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int64_t n, int kb, float scale, int apply_scale,
@@ -257,9 +247,13 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.out_levels = nullptr; a.uniform = thc.uniform; a.out_lo = thc.out_lo; a.out_delta = thc.out_delta;
     a.out_top = thc.out_top;
     const int sign_fwd = (sign && !inverse) ? 1 : 0, sign_inv = (sign && inverse) ? 2 : 0;
-    // without a quantiser folded into its ends a contiguous pass runs as the chunk-first kernel of dq_rht_scaling.hip
-    const bool plain_in = !thc.in_levels && !thc.in_planes;
-    const bool plain = plain_in && !thc.out_levels && !thc.post_scale;
+    // Passes of at least 1024 elements run as the chunk-first kernels of dq_rht_scaling.hip; a quantiser at an end needs
+    // the 16-byte paths there
+    const bool plain = !thc.in_levels && !thc.in_planes && !thc.out_levels && !thc.post_scale;
+    const bool ends_ok = plain || (vec16 && (n & 31) == 0 && (reinterpret_cast<uintptr_t>(thc.in_levels) & 15) == 0);
+    TransformEnds first = thc, last = thc, none;
+    first.out_levels = nullptr; first.post_scale = nullptr;
+    last.in_levels = nullptr; last.in_planes = nullptr;
 
     if (kb <= kMaxTileBits) {
         // single pass; small blocks share a tile
@@ -274,8 +268,9 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
         a.in_planes = thc.in_planes;
         a.post_scale = thc.post_scale;
         const int64_t ntiles = (n + ((int64_t)1 << kt) - 1) >> kt;
-        if (plain && kt >= 10)
-            return launch_rht_tile(x, sign, sign_packed ? 1 : 0, n, kt, kb, scale, apply_scale, sign_fwd | sign_inv, a.vec, stream);
+        if (ends_ok && kt >= 10)
+            return launch_rht_tile(x, sign, sign_packed ? 1 : 0, n, kt, kb, scale, apply_scale, sign_fwd | sign_inv, a.vec, thc,
+                                   stream);
         return launch_tile(a, ntiles, stream);
     }
 
@@ -285,8 +280,8 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.apply_scale = 0; a.sign_mode = sign_fwd; a.vec = vec16;
     a.in_levels = thc.in_levels;
     a.in_planes = thc.in_planes;
-    hipError_t e = plain_in ? launch_rht_tile(x, sign, sign_packed ? 1 : 0, n, kt, kt, scale, 0, sign_fwd, a.vec, stream)
-                            : launch_tile(a, n >> kt, stream);
+    hipError_t e = ends_ok ? launch_rht_tile(x, sign, sign_packed ? 1 : 0, n, kt, kt, scale, 0, sign_fwd, a.vec, first, stream)
+                           : launch_tile(a, n >> kt, stream);
     if (e != hipSuccess) return e;
     a.in_levels = nullptr;
     a.in_planes = nullptr;
@@ -299,14 +294,15 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
         const int r = (rem + passes - 1) / passes;
         a.kt = r + kStridedCols; a.b0 = kStridedCols; a.b1 = kStridedCols + r;
         a.cbits = kStridedCols; a.sbits = s;
-        const bool last = (s + r == kb);
-        a.apply_scale = last ? apply_scale : 0;
-        a.sign_mode = last ? sign_inv : 0;
-        a.out_levels = last ? thc.out_levels : nullptr;
-        a.post_scale = last ? thc.post_scale : nullptr;
+        const bool last_pass = (s + r == kb);
+        a.apply_scale = last_pass ? apply_scale : 0;
+        a.sign_mode = last_pass ? sign_inv : 0;
+        a.out_levels = last_pass ? thc.out_levels : nullptr;
+        a.post_scale = last_pass ? thc.post_scale : nullptr;
         a.vec = vec16;
-        if (r >= 4 && !a.out_levels && !a.post_scale && (n & (((int64_t)1 << (s + r)) - 1)) == 0)
-            e = launch_rht_strided(x, sign, sign_packed ? 1 : 0, n, r, s, scale, a.apply_scale, a.sign_mode, a.vec, stream);
+        if (r >= 4 && ends_ok && (n & (((int64_t)1 << (s + r)) - 1)) == 0)
+            e = launch_rht_strided(x, sign, sign_packed ? 1 : 0, n, r, s, scale, a.apply_scale, a.sign_mode, a.vec,
+                                   last_pass ? last : none, stream);
         else
             e = launch_tile(a, n >> a.kt, stream);
         if (e != hipSuccess) return e;

@@ -122,10 +122,27 @@ hipError_t launch_rht_compress_mfma16(const float *src, const void *sign, int si
                                       float scale, const MeeParams &mp, uint64_t seed, uint64_t step, hipStream_t stream);
 hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign_bits, float *dst, int64_t n, int64_t block,
                                   float scale, int nbits, bool mee, const MeeParams &mp, hipStream_t stream);
+// Quantisers folded into the two ends of a transform (all null: the plain transform).  `in_*` replace the load of the
+// first pass, `out_*` / `post_scale` act on the store of the last one.
+struct TransformEnds {
+    // THC: the pass loads float(level) * *in_step + *in_lo instead of x
+    const uint16_t *in_levels = nullptr;
+    const float *in_step = nullptr, *in_lo = nullptr;
+    // THC: the pass stores thc_level(value, uniform) as bf16 instead of the value
+    uint16_t *out_levels = nullptr;
+    const float *uniform = nullptr, *out_lo = nullptr, *out_delta = nullptr;
+    float out_top = 0.0f;
+    // EDEN: the pass loads centroids[bin] from the bit planes of the bins; the last pass multiplies by *post_scale
+    const uint32_t *in_planes = nullptr;
+    const float *in_centroids = nullptr;
+    int in_nbits = 0;
+    const float *post_scale = nullptr;
+};
+
 hipError_t launch_rht_tile(float *x, const void *sign, int sign_bits, int64_t n, int kt, int kb, float scale, int apply_scale,
-                           int sign_mode, int vec, hipStream_t stream);
+                           int sign_mode, int vec, const TransformEnds &ends, hipStream_t stream);
 hipError_t launch_rht_strided(float *x, const void *sign, int sign_bits, int64_t n, int rbits, int sbits, float scale,
-                              int apply_scale, int sign_mode, int vec, hipStream_t stream);
+                              int apply_scale, int sign_mode, int vec, const TransformEnds &ends, hipStream_t stream);
 
 // EDEN Lloyd-Max quantiser + packer, THC uniform quantiser (dq_eden.hip)
 int64_t eden_work_doubles(int64_t n);

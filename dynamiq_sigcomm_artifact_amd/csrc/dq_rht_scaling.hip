@@ -266,13 +266,102 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
     }
 }
 
+// ---- quantisers folded into the ends of the plain transform (TransformEnds) ------------------------------------
+
+// the sign flip of a chunk that is already in registers (g a multiple of 16; 16-byte accesses to a float sign vector)
+__device__ __forceinline__ void flip16(float (&v)[16], const RhtTileArgs &a, int64_t g)
+{
+    if (!a.sign) return;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float4 q = make_float4(v[4 * k], v[4 * k + 1], v[4 * k + 2], v[4 * k + 3]);
+        flip4(q, a, g + 4 * k);
+        v[4 * k] = q.x; v[4 * k + 1] = q.y; v[4 * k + 2] = q.z; v[4 * k + 3] = q.w;
+    }
+}
+
+// The chunk at g (a multiple of 16; n is a multiple of 32, so the chunk is inside the vector or outside) as the first
+// pass sees it: the floats of x, or THC's levels times step plus lo (thc_hooks.py:176-178: two roundings), or the
+// centroids of EDEN's bins, read from the bit planes (srrcomp.py:343-354); then the sign flip of a forward transform.
+// cen: the centroid table in LDS.
+template <bool ENDS>
+__device__ __forceinline__ void fetch_chunk(float (&v)[16], const float *__restrict__ x, const RhtTileArgs &in,
+                                            const TransformEnds &e, const float *cen, int64_t g)
+{
+    if (!ENDS || (!e.in_levels && !e.in_planes)) {
+        load_chunk(v, x, in, g);
+        return;
+    }
+    if (g >= in.n) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) v[i] = 0.0f;
+        return;
+    }
+    if (e.in_levels) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(e.in_levels + g);
+        const uint4 l0 = p[0], l1 = p[1];
+        const uint32_t w[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+        const float step = *e.in_step, lo = *e.in_lo;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float p0 = bf16_bits_to_f32(w[k] & 0xffffu) * step, p1 = bf16_bits_to_f32(w[k] >> 16) * step;
+            v[2 * k] = p0 + lo;
+            v[2 * k + 1] = p1 + lo;
+        }
+    } else {
+        // sixteen consecutive bins from the thread's half word of every plane (two 8 x 8 bit transposes)
+        const uint16_t *half = reinterpret_cast<const uint16_t *>(e.in_planes) + (g >> 4);
+        const int64_t words = in.n >> 5;
+        uint64_t lo8 = 0, hi8 = 0;
+        for (int p = 0; p < e.in_nbits; p++) {
+            const uint32_t h = half[(int64_t)p * words * 2];
+            lo8 |= (uint64_t)(h & 0xffu) << (8 * p);
+            hi8 |= (uint64_t)(h >> 8) << (8 * p);
+        }
+        lo8 = transpose8x8(lo8);
+        hi8 = transpose8x8(hi8);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = cen[(lo8 >> (8 * k)) & 0xffu];
+            v[8 + k] = cen[(hi8 >> (8 * k)) & 0xffu];
+        }
+    }
+    flip16(v, in, g);
+}
+
+// four consecutive elements of the last pass on their way out: scale, sign flip of an inverse transform, EDEN's scale,
+// then the float store or THC's quantiser (thc_hooks.py:161-166) and a bf16 store
+template <bool ENDS>
+__device__ __forceinline__ void store4(float *__restrict__ x, float4 v, const RhtTileArgs &a, const TransformEnds &e, int sign_mode,
+                                       int apply_scale, int64_t g)
+{
+    if (apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
+    if (sign_mode == 2) flip4(v, a, g);
+    if (ENDS && e.post_scale) {
+        const float ps = *e.post_scale;
+        v.x *= ps; v.y *= ps; v.z *= ps; v.w *= ps;
+    }
+    if (ENDS && e.out_levels) {
+        const float4 u = *reinterpret_cast<const float4 *>(e.uniform + g);
+        const float lo = *e.out_lo, delta = *e.out_delta;
+        uint2 o;
+        o.x = f32x2_to_bf16x2(thc_level(v.x, u.x, lo, delta, e.out_top), thc_level(v.y, u.y, lo, delta, e.out_top));
+        o.y = f32x2_to_bf16x2(thc_level(v.z, u.z, lo, delta, e.out_top), thc_level(v.w, u.w, lo, delta, e.out_top));
+        *reinterpret_cast<uint2 *>(e.out_levels + g) = o;
+    } else {
+        *reinterpret_cast<float4 *>(x + g) = v;
+    }
+}
+
 // The transform alone (dq_rht_blocked, the first pass of a long dq_hadamard) with the structure of the two kernels
 // above: a lane loads its chunk of 16 consecutive floats, does the stages of strides 1..8 on its registers, the rest
 // runs as LDS passes of up to five stages, and the tile leaves as coalesced 16-byte stores with the scale and (inverse
 // direction) the sign flip.  Against the all-in-LDS kernel of dq_hadamard.hip: two or three LDS passes instead of four,
 // and a thread's loads issued together.  In place: a workgroup reads and writes only its own tile.
 // sign_mode: 0 no flip, 1 flip on load, 2 flip on store
-__global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_mode, int apply_scale)
+// ENDS: a quantiser may sit at either end (TransformEnds; 16-byte accesses only: a.vec is set)
+template <bool ENDS>
+__global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_mode, int apply_scale, TransformEnds e)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -280,12 +369,17 @@ __global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_m
     const int64_t origin = (int64_t)blockIdx.x << a.kt;
     RhtTileArgs in = a;
     if (sign_mode != 1) in.sign = nullptr;
+    const float *cen = lds + padded_tile_floats(a.kt); // EDEN's centroids sit behind the tile
+    if (ENDS && e.in_planes) {
+        for (int k = tid; k < (1 << e.in_nbits); k += nthreads) lds[padded_tile_floats(a.kt) + k] = e.in_centroids[k];
+        __syncthreads();
+    }
     const int nchunks = tile >> 4;
     if (nchunks == 2 * nthreads) {
         // 2^15 tiles: both chunks of a thread are loaded before either is used
         float v[16], w[16];
-        load_chunk(v, x, in, origin + tid * 16);
-        load_chunk(w, x, in, origin + (tid + nthreads) * 16);
+        fetch_chunk<ENDS>(v, x, in, e, cen, origin + tid * 16);
+        fetch_chunk<ENDS>(w, x, in, e, cen, origin + (tid + nthreads) * 16);
         chunk_stages(v, a.kb);
         chunk_stages(w, a.kb);
         float *mine = lds + tid * 17, *other = lds + (tid + nthreads) * 17;
@@ -296,7 +390,7 @@ __global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_m
     } else {
         for (int c = tid; c < nchunks; c += nthreads) {
             float v[16];
-            load_chunk(v, x, in, origin + c * 16);
+            fetch_chunk<ENDS>(v, x, in, e, cen, origin + c * 16);
             chunk_stages(v, a.kb);
             float *mine = lds + c * 17; // pad_idx(16 c + i) = 17 c + i
 #pragma unroll
@@ -304,23 +398,19 @@ __global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_m
         }
     }
     fwht_lds_stages_after4(lds, a.kt, a.kb, tid, nthreads);
-    const float scale = apply_scale ? a.scale : 1.0f;
     if (a.vec) {
         for (int i = tid * 4; i < tile; i += nthreads * 4) {
             const int64_t g = origin + i;
             if (g >= a.n) continue;
             const int q = pad_idx(i);
-            float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
-            if (apply_scale) { v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale; }
-            if (sign_mode == 2) flip4(v, a, g);
-            *reinterpret_cast<float4 *>(x + g) = v;
+            store4<ENDS>(x, make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]), a, e, sign_mode, apply_scale, g);
         }
     } else {
         for (int i = tid; i < tile; i += nthreads) {
             const int64_t g = origin + i;
             if (g >= a.n) continue;
             float v = lds[pad_idx(i)];
-            if (apply_scale) v *= scale;
+            if (apply_scale) v *= a.scale;
             x[g] = sign_mode == 2 ? flip1(v, a, g) : v;
         }
     }
@@ -331,7 +421,9 @@ __global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_m
 // is tile bit b + 5.  A thread owns column tid % 32 of sixteen consecutive rows: it loads them (every load instruction of
 // a wave covers two whole 128-byte row segments), does the four lowest row stages on its registers and leaves the other
 // rbits - 4 (at most 6) to one or two LDS passes.  sign_mode: 0, or 2 = flip on store (the last pass of an inverse).
-__global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbits, int sbits, int sign_mode, int apply_scale)
+template <bool ENDS>
+__global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbits, int sbits, int sign_mode, int apply_scale,
+                                   TransformEnds e)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -383,10 +475,7 @@ __global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbi
         for (int i = tid * 4; i < tile; i += nthreads * 4) {
             const int64_t g = origin + ((int64_t)(i >> 5) << sbits) + (i & 31);
             const int q = pad_idx(i);
-            float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
-            if (apply_scale) { v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale; }
-            if (sign_mode == 2) flip4(v, a, g);
-            *reinterpret_cast<float4 *>(x + g) = v;
+            store4<ENDS>(x, make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]), a, e, sign_mode, apply_scale, g);
         }
     } else {
         for (int i = tid; i < tile; i += nthreads) {
@@ -703,15 +792,18 @@ hipError_t launch_irht_decompress(const uint8_t *src, const void *sign, int sign
 }
 
 // stages [0, kb) of every aligned block of 2^kb elements, tiles of 2^kt contiguous elements (10 <= kt <= 15, kb <= kt);
-// vec: 16-byte accesses to x (and to a float sign vector) are allowed
+// vec: 16-byte accesses to x (and to a float sign vector) are allowed; ends: needs vec, n a multiple of 32 and 16-byte
+// aligned levels
 hipError_t launch_rht_tile(float *x, const void *sign, int sign_bits, int64_t n, int kt, int kb, float scale, int apply_scale,
-                           int sign_mode, int vec, hipStream_t stream)
+                           int sign_mode, int vec, const TransformEnds &ends, hipStream_t stream)
 {
     if (kt < 10 || kt > 15 || kb > kt || kb < 0) return hipErrorInvalidValue;
+    const bool plain = !ends.in_levels && !ends.in_planes && !ends.out_levels && !ends.post_scale;
+    if (!plain && (!vec || (n & 31) != 0)) return hipErrorInvalidValue;
     RhtTileArgs a;
     a.sign = sign; a.sign_bits = sign_bits; a.n = n; a.kt = kt; a.kb = kb; a.scale = scale; a.vec = vec;
     const int tile = 1 << kt;
-    if (kt == kSplitBits && kb == kSplitBits && (n & (tile - 1)) == 0) {
+    if (plain && kt == kSplitBits && kb == kSplitBits && (n & (tile - 1)) == 0) {
         // whole blocks of 2^15: half the LDS, two workgroups per CU
         const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float);
         hipError_t es = allow_lds(rht_tile_split_kernel, half_lds);
@@ -721,28 +813,44 @@ hipError_t launch_rht_tile(float *x, const void *sign, int sign_bits, int64_t n,
         return hipGetLastError();
     }
     const unsigned threads = (unsigned)std::min(1024, tile / 16);
-    const size_t lds = (size_t)padded_tile_floats(kt) * sizeof(float);
-    hipError_t e = allow_lds(rht_tile_kernel, lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(rht_tile_kernel, dim3((unsigned)((n + tile - 1) >> kt)), dim3(threads), lds, stream, x, a,
-                       sign ? sign_mode : 0, apply_scale);
+    const size_t lds = ((size_t)padded_tile_floats(kt) + (ends.in_planes ? 256 : 0)) * sizeof(float);
+    const dim3 grid((unsigned)((n + tile - 1) >> kt));
+    if (plain) {
+        hipError_t e = allow_lds(rht_tile_kernel<false>, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(rht_tile_kernel<false>, grid, dim3(threads), lds, stream, x, a, sign ? sign_mode : 0, apply_scale, ends);
+    } else {
+        hipError_t e = allow_lds(rht_tile_kernel<true>, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(rht_tile_kernel<true>, grid, dim3(threads), lds, stream, x, a, sign ? sign_mode : 0, apply_scale, ends);
+    }
     return hipGetLastError();
 }
 
 // stages of the index bits [sbits, sbits + rbits) of x[0 .. n), n a multiple of 2^(sbits + rbits); 4 <= rbits <= 10, sbits >= 5
 hipError_t launch_rht_strided(float *x, const void *sign, int sign_bits, int64_t n, int rbits, int sbits, float scale,
-                              int apply_scale, int sign_mode, int vec, hipStream_t stream)
+                              int apply_scale, int sign_mode, int vec, const TransformEnds &ends, hipStream_t stream)
 {
     if (rbits < 4 || rbits > 10 || sbits < 5 || (n & (((int64_t)1 << (sbits + rbits)) - 1)) != 0) return hipErrorInvalidValue;
+    const bool plain = !ends.out_levels && !ends.post_scale;
+    if (!plain && !vec) return hipErrorInvalidValue;
     RhtTileArgs a;
     a.sign = sign; a.sign_bits = sign_bits; a.n = n; a.kt = rbits + 5; a.kb = 0; a.scale = scale; a.vec = vec;
     const int tile = 1 << (rbits + 5);
     const unsigned threads = (unsigned)std::min(1024, tile / 16);
     const size_t lds = (size_t)padded_tile_floats(rbits + 5) * sizeof(float);
-    hipError_t e = allow_lds(rht_strided_kernel, lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(rht_strided_kernel, dim3((unsigned)(n >> (rbits + 5))), dim3(threads), lds, stream, x, a, rbits, sbits,
-                       sign ? sign_mode : 0, apply_scale);
+    const dim3 grid((unsigned)(n >> (rbits + 5)));
+    if (plain) {
+        hipError_t e = allow_lds(rht_strided_kernel<false>, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(rht_strided_kernel<false>, grid, dim3(threads), lds, stream, x, a, rbits, sbits, sign ? sign_mode : 0,
+                           apply_scale, ends);
+    } else {
+        hipError_t e = allow_lds(rht_strided_kernel<true>, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(rht_strided_kernel<true>, grid, dim3(threads), lds, stream, x, a, rbits, sbits, sign ? sign_mode : 0,
+                           apply_scale, ends);
+    }
     return hipGetLastError();
 }
 
