@@ -648,6 +648,9 @@ def kernels(dev, n=6553600):
     u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)
     line("group_plan_stats", lambda: capi.group_plan_stats(stats, u, qbits, order, work), 4 * nsc + 12 * nsc, superchunks=nsc)
     line("group_plan", lambda: capi.group_plan(qbits, order, work), 8 * nsc + 4 * nsc, superchunks=nsc)
+    # the fixed-proportion allocation: stable descending sort of the norms, top 35 % / bottom 20 % (x_5bit)
+    line("group_plan_sorted", lambda: capi.group_plan_sorted(stats, int(nsc * 0.35), int(nsc * 0.2), order, work), 4 * nsc + 4 * nsc,
+         superchunks=nsc)
     # the search for u: the norm patterns of the bucket into the histogram; the whole bisection on an empty histogram
     # (never meets the tolerance: all 33 probes)
     hist = torch.zeros(capi.bitrate_hist_ints(), dtype=torch.int32, device=dev)
