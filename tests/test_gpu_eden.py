@@ -215,7 +215,7 @@ def test_binding_functions(eden_utils, capi):
 
 
 @pytest.mark.parametrize("n,block", [(64, 64), (1024, 1024), (1024, 64), (1 << 15, 1 << 15), (1 << 16, 1 << 16),
-                                     (1 << 20, 1 << 20), (1 << 22, 1 << 22), (1 << 18, 1 << 12), (3 << 14, 1 << 14)])
+                                     (1 << 17, 1 << 17), (1 << 20, 1 << 20), (1 << 22, 1 << 22), (1 << 23, 1 << 23), (1 << 18, 1 << 12), (3 << 14, 1 << 14)])
 def test_thc_quantiser_folded_into_the_transform(capi, n, block):
     """dq_thc_rht_quantize == rht_blocked + thc_quantize and dq_thc_dequantize_irht == thc_dequantize + inverse
     rht_blocked, bit for bit, for single-pass and multi-pass transforms"""
@@ -281,7 +281,7 @@ def test_thc_quantiser_folded_into_the_transform(capi, n, block):
 
 @pytest.mark.parametrize("nbits", [1, 3, 4, 8])
 @pytest.mark.parametrize("n,block", [(32, 32), (96, 32), (1024, 1024), (4096 * 3, 4096), (1 << 15, 1 << 15), (1 << 16, 1 << 16),
-                                     (1 << 20, 1 << 20), (1 << 22, 1 << 22), (1 << 18, 1 << 12)])
+                                     (1 << 17, 1 << 17), (1 << 20, 1 << 20), (1 << 22, 1 << 22), (1 << 23, 1 << 23), (1 << 18, 1 << 12)])
 def test_eden_dequantiser_folded_into_the_inverse_transform(capi, nbits, n, block):
     """dq_eden_dequantize_irht == eden_dequantize, inverse rht_blocked, product with the scale -- bit for bit, single-pass
     and multi-pass transforms, float and packed diagonals, with and without the scale"""
