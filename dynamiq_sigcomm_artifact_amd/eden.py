@@ -1,5 +1,5 @@
-"""EDEN on the library's kernels -- the host-side mirror of ``srrcomp.Eden``
-(cuda_kernels/src/srrcomp/srrcomp.py:170-447): the same slicing rule, the same
+"""EDEN on the library's kernels -- the host-side mirror of ``srrcomp.Eden`` and of the ``SRRCompUtils`` it inherits
+(cuda_kernels/src/srrcomp/srrcomp.py:13-447): the same slicing rule, the same
 ``compress`` / ``decompress`` signatures and the same per-slice dictionaries, with
 
   * randDiag + Hadamard + 1/sqrt(n) in one launch per rotation (``rht_blocked``),
@@ -51,8 +51,57 @@ def normal_centroids_and_boundaries(nbits):
     return c, (c[:-1] + c[1:]) / 2
 
 
-class Eden(object):
+class SRRCompUtils(object):
+    """The helpers ``srrcomp.Eden`` inherits (srrcomp.py:13-167) on the library's kernels: ``randDiag``, ``Hadamard``,
+    ``EdenBinsToBits`` / ``EdenBitsToBins`` and the ``utils`` table the reference looks its implementations up in.
+    Only device tensors are served (the build has no CPU path): the 'cpu' entries of ``utils`` raise."""
+
+    def __init__(self, gpuacctype="cuda"):
+        if gpuacctype not in ("cuda", "torch"):
+            raise Exception("Illegal gpuacctype {}, use 'cuda' or 'torch'.".format(gpuacctype))
+        self.gpuacctype = gpuacctype                  # both values select the kernels here
+        from . import load_eden_utils
+        eu = load_eden_utils()
+        gpu = {"Hadamard": eu.Hadamard, "BinsToBits": eu.EdenBinsToBits, "BitsToBins": eu.EdenBitsToBins}
+        self.utils = {"gpu": gpu, "cpu": {name: self._device_only for name in gpu}}
+
+    @staticmethod
+    def _device_only(*args, **kwargs):
+        raise RuntimeError("this build serves device tensors only: move the vector to the GPU")
+
+    def randDiag(self, size, device, seed, torchRNG=False):
+        """+-1 floats (srrcomp.py:61-106); with torchRNG torch's own Bernoulli stream, as there"""
+        if torchRNG:
+            prng = torch.Generator(device=device)
+            prng.manual_seed(seed)
+            half = torch.full((size,), 0.5, device=device)
+            return 2 * torch.bernoulli(half, generator=prng) - 1
+        out = torch.empty(size, dtype=torch.float32, device=device)
+        if size:
+            capi.rand_diag(out, seed)
+        return out
+
+    def Hadamard(self, vec):
+        """unnormalised transform of a power-of-two vector, in place like srrcomp.py:108-122; returns the flat view"""
+        d = vec.numel()
+        if d & (d - 1) != 0:
+            raise Exception("input numel must be a power of 2")
+        flat = vec.view(-1)
+        capi.hadamard(flat)
+        return flat
+
+    def EdenBinsToBits(self, bins, nbits):
+        """bit plane p of 32 consecutive bins -> bits[p * n/32 + w] (srrcomp.py:124-145); int32 like eden_utils"""
+        return self.utils["gpu"]["BinsToBits"](bins.to(torch.int32).contiguous(), nbits)
+
+    def EdenBitsToBins(self, bits, nbits):
+        """the inverse (srrcomp.py:147-167); int32 bins like eden_utils (the torch version there returns floats)"""
+        return self.utils["gpu"]["BitsToBins"](bits.to(torch.int32).contiguous(), nbits)
+
+
+class Eden(SRRCompUtils):
     def __init__(self, gpuacctype="cuda", max_padding_overhead=0.1, centroids=None, boundaries=None, device="cuda"):
+        super().__init__(gpuacctype)
         self.max_padding_overhead = max_padding_overhead
         self.device = torch.device(device)
         self.centroids = dict(centroids) if centroids is not None else {}
@@ -133,6 +182,21 @@ class Eden(object):
         capi.eden_quantize(vec, boundaries, centroids, nbits, packed, result, work)
         return {"packed_bins": packed, "vec_type": vec_type, "nbits": nbits, "scale": result[2], "orig_dim": orig_dim,
                 "num_hadamard": num_hadamard, "seed": seed}
+
+    # ---- srrcomp.py:356-361 ----
+    def _quantize(self, vec, nbits):
+        """(bins, scale) of a rotated vector: bins int64 like torch.bucketize's, scale a 0-d tensor.  One call of the
+        quantiser kernels (the bit planes it also writes are unpacked again here); ``compress`` does not go this way."""
+        n = vec.numel()
+        if n == 0 or n % 32:
+            raise RuntimeError("_quantize: the kernels take a positive multiple of 32 elements")
+        vec = vec.to(self.device, torch.float32).contiguous()
+        centroids, boundaries = self._tables(nbits)
+        packed = torch.empty(n // 32 * nbits, dtype=torch.int32, device=self.device)
+        result = torch.empty(4, dtype=torch.float32, device=self.device)
+        work = torch.empty(capi.eden_work_doubles(n), dtype=torch.float64, device=self.device)
+        capi.eden_quantize(vec, boundaries, centroids, nbits, packed, result, work)
+        return self.EdenBitsToBins(packed, nbits).to(torch.int64), result[2]
 
     # ---- srrcomp.py:328-354 ----
     def decompress(self, data):

@@ -307,3 +307,47 @@ def test_eden_dequantiser_folded_into_the_inverse_transform(capi, nbits, n, bloc
         assert torch.equal(got[:n].view(torch.int32), ref.view(torch.int32)) and bool((got[n:] == 7.0).all())
         capi.eden_dequantize_irht(packed, n, cen, nbits, sg, got[:n], block, scale, post_scale=eden_scale)
         assert torch.equal(got[:n].view(torch.int32), (eden_scale * ref).view(torch.int32)) and bool((got[n:] == 7.0).all())
+
+
+def test_srrcomp_utils_surface(capi, oracle):
+    """the helpers srrcomp.Eden inherits from SRRCompUtils (srrcomp.py:13-167) and its _quantize (:356-361), as methods
+    of the drop-in class: each equals the oracle's function or the entry point it wraps"""
+    from dynamiq_sigcomm_artifact_amd.eden import Eden, SRRCompUtils
+    eden = Eden(device=DEV)
+    assert isinstance(eden, SRRCompUtils) and set(eden.utils) == {"cpu", "gpu"}
+    assert set(eden.utils["gpu"]) == {"Hadamard", "BinsToBits", "BitsToBins"}
+    with pytest.raises(Exception, match="Illegal gpuacctype"):
+        SRRCompUtils("opencl")
+    with pytest.raises(RuntimeError, match="device tensors only"):
+        eden.utils["cpu"]["Hadamard"](torch.zeros(8))
+    # randDiag: the integer hash of the reference; with torchRNG torch's own stream of +-1
+    for size, seed in ((1000, 7), (4096, 123456789), (1, 0)):
+        got = eden.randDiag(size, DEV, seed)
+        assert got.dtype == torch.float32 and np.array_equal(got.cpu().numpy(), oracle.rand_diag(size, seed))
+    coins = eden.randDiag(512, DEV, 5, torchRNG=True)
+    assert set(coins.cpu().tolist()) == {-1.0, 1.0} and torch.equal(coins, eden.randDiag(512, DEV, 5, torchRNG=True))
+    # Hadamard: in place, returns the flat view
+    x = torch.randn(1 << 12, generator=torch.Generator().manual_seed(3))
+    x_d = x.to(DEV).view(64, 64)
+    y = eden.Hadamard(x_d)
+    assert y.data_ptr() == x_d.data_ptr() and np.array_equal(y.cpu().numpy(), oracle.fwht(x.numpy()))
+    with pytest.raises(Exception, match="power of 2"):
+        eden.Hadamard(torch.zeros(12, device=DEV))
+    # the packers take the int64 bins of torch.bucketize
+    bins = torch.randint(0, 32, (4096,), generator=torch.Generator().manual_seed(4))
+    bits = eden.EdenBinsToBits(bins.to(DEV), 5)
+    assert bits.dtype == torch.int32 and np.array_equal(bits.cpu().numpy().view(np.uint32), oracle.bins_to_bits(bins.numpy().astype(np.int32), 5).view(np.uint32))
+    assert torch.equal(eden.EdenBitsToBins(bits, 5).cpu(), bins.to(torch.int32))
+    # _quantize: the bins and the scale of eden_quantize
+    n, nbits = 8192, 4
+    v = torch.randn(n, generator=torch.Generator().manual_seed(6)).to(DEV)
+    q_bins, scale = eden._quantize(v, nbits)
+    cen, bnd = eden._tables(nbits)
+    packed = torch.empty(n // 32 * nbits, dtype=torch.int32, device=DEV)
+    result = torch.empty(4, dtype=torch.float32, device=DEV)
+    capi.eden_quantize(v, bnd, cen, nbits, packed, result, torch.empty(capi.eden_work_doubles(n), dtype=torch.float64, device=DEV))
+    assert q_bins.dtype == torch.int64 and torch.equal(eden.EdenBinsToBits(q_bins, nbits), packed)
+    assert float(scale) == float(result[2])
+    # against torch's own ops away from the boundaries: at most a handful of bins differ by the rounding of the quotient
+    ref = torch.bucketize(v * (n ** 0.5) / torch.norm(v, 2), bnd)
+    assert int((ref != q_bins).sum()) <= 2
