@@ -1,4 +1,6 @@
-// Blocked randomized Hadamard transform fused with the hierarchical chunk-16 quantiser.
+// Blocked randomized Hadamard transform fused with the hierarchical chunk-16 quantiser, and -- with the same lane = chunk
+// structure -- the passes of the transform alone (rht_tile_kernel, rht_tile_split_kernel, rht_strided_kernel), with or
+// without THC's / EDEN's quantisers at the ends; dq_hadamard.hip plans which passes a transform takes.
 //
 // rht_blocked followed by scaling_compress moves every element through HBM three times (read, write the
 // rotated vector, read it again); the inverse pair likewise.  Here the rotated tile never leaves the
