@@ -144,8 +144,8 @@ def fixed_proportion_groups(norms, thresholds):
 
 
 def fixed_proportion_plan(stats, thresholds, order=None, work=None, stream=None):
-    """The same three lists from the interleaved bf16 (mean, norm) statistics by one launch, without a sort and
-    without a read-back: ``order`` int32 [3 * nsc] (the 8-bit list at 0, the 4-bit list at nsc, the 2-bit list at
+    """The same three lists from the interleaved bf16 (mean, norm) statistics without a read-back (one launch, no sort
+    passes, up to 65535 superchunks; a radix sort inside ``work`` for longer buckets): ``order`` int32 [3 * nsc] (the 8-bit list at 0, the 4-bit list at nsc, the 2-bit list at
     2 * nsc, each in sorted order) and ``work[0..2]`` = the three counts, i.e. what the row-list and mixed codec
     kernels take.  Returns (order, work, (n8, n4, n2))."""
     from . import capi
@@ -154,7 +154,8 @@ def fixed_proportion_plan(stats, thresholds, order=None, work=None, stream=None)
     if order is None:
         order = torch.empty(3 * nsc, dtype=torch.int32, device=stats.device)
     if work is None:
-        work = torch.empty(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=stats.device)
+        work = torch.empty(max(capi.group_plan_work_ints(nsc), capi.group_plan_sorted_work_ints(nsc)), dtype=torch.int32,
+                           device=stats.device)
     capi.group_plan_sorted(stats, n8, n2, order, work, stream)
     return order, work, (n8, n4, n2)
 

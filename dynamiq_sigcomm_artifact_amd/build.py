@@ -25,7 +25,7 @@ HIP_SOURCES = [
     "dq_scaling_generic.hip",
     "dq_scaling_hier16.hip",
     "dq_scaling_tile16.hip",
-    "dq_grouping.hip", "dq_bitrate.hip",
+    "dq_grouping.hip", "dq_bitrate.hip", "dq_sort.hip",
     "dq_scaling_mixed.hip",
     "dq_rht_scaling.hip",
     "dq_superchunk.hip",

@@ -22,7 +22,7 @@ EXPORTS = [
     "dq_init_lookup_table", "dq_mee_lookup_table",
     "dq_scaling_compress", "dq_scaling_decompress", "dq_scaling_dec_comp",
     "dq_scaling_compress_philox", "dq_scaling_dec_comp_philox", "dq_philox_uniform",
-    "dq_group_plan_work_ints", "dq_group_plan", "dq_group_plan_stats",
+    "dq_group_plan_work_ints", "dq_group_plan_sorted_work_ints", "dq_group_plan", "dq_group_plan_stats",
     "dq_group_plan_stats_dev_u", "dq_group_plan_sorted", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
@@ -73,6 +73,8 @@ def lib():
         L.dq_philox_uniform.argtypes = [vp, i64, i32, i32, u64, u64, vp]
         L.dq_group_plan_work_ints.restype = i64
         L.dq_group_plan_work_ints.argtypes = [i64]
+        L.dq_group_plan_sorted_work_ints.restype = i64
+        L.dq_group_plan_sorted_work_ints.argtypes = [i64]
         L.dq_group_plan.restype = i32
         L.dq_group_plan.argtypes = [vp, i64, vp, vp, i64, i32, vp]
         L.dq_group_plan_stats.restype = i32
@@ -298,9 +300,14 @@ def group_rows(order, nsc, width, count):
     return order[base:base + count]
 
 
+def group_plan_sorted_work_ints(nsc):
+    """int32 entries of the work buffer of group_plan_sorted: 4 up to 65535 superchunks, the radix sort's buffers beyond"""
+    return int(lib().dq_group_plan_sorted_work_ints(nsc))
+
+
 def group_plan_sorted(stats, top_count, bottom_count, order, work, stream=None, qbits_out=None):
     """fixed-proportion groups (comm_hooks.py:710-721): order / work[0:3] as group_plan writes them, every list in
-    the order of the stable descending sort of the norms stats[:, 1]"""
+    the order of the stable descending sort of the norms stats[:, 1]; work: group_plan_sorted_work_ints(nsc) ints"""
     if stats.dtype != torch.bfloat16 or order.dtype != torch.int32 or work.dtype != torch.int32:
         raise RuntimeError("group_plan_sorted: stats must be bfloat16, order and work int32")
     nsc = stats.numel() // 2

@@ -311,18 +311,29 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
     return finish(dq::launch_group_plan_stats(stats, (float)u, nullptr, nsc, qbits_out, order, work, nullptr, static_cast<hipStream_t>(stream)));
 }
 
+// up to here the one-launch counting sort in LDS, beyond it the radix sort in the caller's workspace
+static constexpr int64_t kSortedPlanOneLaunch = 65535;
+
+int64_t dq_group_plan_sorted_work_ints(int64_t nsc)
+{
+    return nsc > kSortedPlanOneLaunch ? dq::group_plan_sorted_large_work_ints(nsc) : 4;
+}
+
 int dq_group_plan_sorted(const void *stats, int64_t nsc, int64_t top_count, int64_t bottom_count, int64_t *qbits_out,
                          int32_t *order, int32_t *work, int64_t work_ints, int device, dq_stream_t stream)
 {
-    if (!(nsc > 0)) return fail(DQ_ERR_N);
-    if (nsc > 65535) return fail(DQ_ERR_SIZE, "dq_group_plan_sorted handles buckets of up to 65535 superchunks");
+    if (!(nsc > 0) || nsc > (int64_t)0x7fffffff) return fail(DQ_ERR_N, "nsc must be in [1, 2^31)");
     if (top_count < 0 || bottom_count < 0 || top_count + bottom_count > nsc)
         return fail(DQ_ERR_SIZE, "top_count and bottom_count must be non-negative and sum to at most nsc");
     if (!stats || !order || !work) return fail(DQ_ERR_NULL);
     if (reinterpret_cast<uintptr_t>(stats) & 3) return fail(DQ_ERR_SIZE, "stats must be 4-byte aligned");
-    if (work_ints < 4) return fail(DQ_ERR_SIZE, "work buffer is too small");
+    if (work_ints < dq_group_plan_sorted_work_ints(nsc))
+        return fail(DQ_ERR_SIZE, "work buffer is too small (dq_group_plan_sorted_work_ints)");
     int rc;
     if ((rc = select_device(device))) return rc;
+    if (nsc > kSortedPlanOneLaunch)
+        return finish(dq::launch_group_plan_sorted_large(stats, nsc, top_count, bottom_count, qbits_out, order, work, work_ints,
+                                                         static_cast<hipStream_t>(stream)));
     return finish(dq::launch_group_plan_sorted(stats, nsc, top_count, bottom_count, qbits_out, order, work,
                                                static_cast<hipStream_t>(stream)));
 }

@@ -64,6 +64,9 @@ hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, 
 // fixed-proportion groups (stable descending sort of the bf16 norms); nsc <= 65535, stats 4-byte aligned
 hipError_t launch_group_plan_sorted(const void *stats, int64_t nsc, int64_t top, int64_t bottom, int64_t *qbits_out,
                                     int32_t *order, int32_t *work, hipStream_t stream);
+int64_t group_plan_sorted_large_work_ints(int64_t nsc);
+hipError_t launch_group_plan_sorted_large(const void *stats, int64_t nsc, int64_t top, int64_t bottom, int64_t *qbits_out,
+                                          int32_t *order, int32_t *work, int64_t work_ints, hipStream_t stream);
 hipError_t launch_group_plan_stats(const void *stats, float u, const double *u_dev, int64_t nsc, int64_t *qbits_out,
                                    int32_t *order, int32_t *work, uint32_t *hist, hipStream_t stream);
 

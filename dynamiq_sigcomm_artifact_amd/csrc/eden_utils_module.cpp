@@ -410,11 +410,11 @@ torch::Tensor group_plan_sorted(torch::Tensor stats, int64_t top_count, int64_t 
                     "qbits_out must be a contiguous torch.int64 CUDA tensor with one entry per superchunk");
         qptr = qbits_out->data_ptr<int64_t>();
     }
-    auto work = torch::empty({4}, order.options());
+    auto work = torch::empty({dq_group_plan_sorted_work_ints(nsc)}, order.options());
     check_status(dq_group_plan_sorted(stats.data_ptr(), nsc, top_count, bottom_count, qptr, order.data_ptr<int32_t>(),
                                       work.data_ptr<int32_t>(), work.numel(), stats.device().index(), as_stream(stream_p)),
                  "group_plan_sorted");
-    return work;
+    return work.slice(0, 0, 4);
 }
 
 torch::Tensor group_plan_stats_dev_u(torch::Tensor stats, torch::Tensor u, torch::Tensor order,

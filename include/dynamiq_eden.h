@@ -180,9 +180,14 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
  * puts a NaN with the sign bit set behind -inf, patterns that sums of squares
  * computed on a device do not take), which is the order in which the hook
  * gathers a group and pairs it with rand_pool rows.  qbits_out: int64
- * [nsc] or NULL.  One launch, no sort passes (the key is a 16-bit pattern:
- * counting sort in LDS), no host synchronisation.  nsc <= 65535 (DQ_ERR_SIZE
- * beyond); stats 4-byte aligned. */
+ * [nsc] or NULL.  No host synchronisation.  Up to 65535 superchunks: one
+ * launch, no sort passes (the key is a 16-bit pattern: counting sort in LDS),
+ * work holds 4 ints.  Longer buckets (the reference's training scripts give
+ * DDP a 4000 MB bucket cap, testbed_evaluation/train_llm_causal.py:416): a
+ * stable radix sort of the 16-bit keys inside `work`, which must then hold
+ * dq_group_plan_sorted_work_ints(nsc) ints (about 12.2 bytes per superchunk).
+ * stats 4-byte aligned. */
+int64_t dq_group_plan_sorted_work_ints(int64_t nsc);
 int dq_group_plan_sorted(const void *stats, int64_t nsc, int64_t top_count, int64_t bottom_count,
                          int64_t *qbits_out, int32_t *order, int32_t *work, int64_t work_ints,
                          int device, dq_stream_t stream);

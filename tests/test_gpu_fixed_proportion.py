@@ -111,7 +111,7 @@ def test_sorted_plan_validation(capi):
     st = _stats(torch.ones(70000).to(torch.bfloat16))
     order = torch.zeros(3 * 70000, dtype=torch.int32, device=DEV)
     work = torch.zeros(64, dtype=torch.int32, device=DEV)
-    with pytest.raises(RuntimeError, match="65535"):
+    with pytest.raises(RuntimeError, match="work buffer is too small"):
         capi.group_plan_sorted(st, 10, 10, order, work)
     with pytest.raises(RuntimeError, match="top_count"):
         capi.group_plan_sorted(st[:100], 60, 60, order, work)
@@ -164,7 +164,8 @@ def test_fixed_proportion_allreduce_device_plan_equals_op_sequence(capi, W, meth
     from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
     from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import fixed_proportion_allreduce, fixed_proportion_allreduce_grouped
     K = Aee_Dynamic_Range_GPU_kern if cls == "aee" else Mee_Dynamic_Range_GPU_kern
-    n = 256 * 700 + 77                       # a ragged tail
+    # a ragged tail; one case beyond the one-launch plan (70,001 superchunks: the radix-sort path)
+    n = 256 * 70000 + 77 if (W == 1 and method == "dynamiQ_aee_5bit") else 256 * 700 + 77
     g = torch.Generator().manual_seed(31 + W)
     scale = torch.exp(torch.randn((n + 255) // 256, generator=g) * 2 - 5).repeat_interleave(256)[:n]
     vecs = [(torch.randn(n, generator=g) * scale + 1e-3).to(torch.bfloat16).to(DEV) for _ in range(W)]
@@ -189,3 +190,41 @@ def test_fixed_proportion_allreduce_device_plan_equals_op_sequence(capi, W, meth
     exact = sum(v.double() for v in vecs) / W
     nmse = float(((out[0].double() - exact) ** 2).sum() / (exact ** 2).sum())
     assert nmse < 0.2
+
+
+@pytest.mark.parametrize("nsc", [65536, 100_003, 1_000_000, 7_812_500])
+@pytest.mark.parametrize("method", ["x_5bit", "x_3bit"])
+def test_sorted_plan_of_a_long_bucket(capi, oracle, nsc, method):
+    """Buckets beyond the one-launch plan (the reference trains with a 4000 MB DDP bucket cap: millions of superchunks)
+    go through the radix sort in the work buffer: the same three lists as the oracle's stable descending sort, NaN first,
+    ties by index; 7,812,500 superchunks = 2 * 10^9 elements."""
+    from dynamiq_sigcomm_artifact_amd import bitrate
+    g = torch.Generator().manual_seed(nsc)
+    norms = torch.exp(torch.randn(nsc, generator=g) * 3 - 8)
+    norms[::1001] = 0.0
+    norms[5::20011] = float("nan")
+    norms[7::30011] = float("inf")
+    if nsc == 100_003:                         # patterns a sum of squares never takes
+        norms[3::997] = -1.5
+        norms[11::4999] = -0.0
+    norms = norms.to(torch.bfloat16)
+    bits = norms.view(torch.int16)
+    bits[5::20011] = 0x7fc0
+    stats = torch.zeros((nsc, 2), dtype=torch.bfloat16)
+    stats[:, 1] = norms
+    stats[:, 0] = 0.25
+    stats_d = stats.to(DEV)
+    thr = bitrate.fixed_proportion_thresholds(method)
+    order, work, (n8, n4, n2) = bitrate.fixed_proportion_plan(stats_d, thr)
+    assert work[:4].tolist() == [n8, n4, n2, 0]
+    want = oracle.argsort_descending_stable(norms.view(torch.int16).numpy().view(np.uint16))
+    o = order.cpu().numpy()
+    assert np.array_equal(o[:n8], want[:n8]), "8-bit list"
+    assert np.array_equal(o[nsc:nsc + n4], want[n8:n8 + n4]), "4-bit list"
+    assert np.array_equal(o[2 * nsc:2 * nsc + n2], want[n8 + n4:]), "2-bit list"
+    # the widths, and a second call into the same buffers
+    qb = torch.zeros(nsc, dtype=torch.int64, device=DEV)
+    capi.group_plan_sorted(stats_d, n8, n2, order, work, qbits_out=qb)
+    q = qb.cpu().numpy()
+    assert (q[want[:n8]] == 8).all() and (q[want[n8:n8 + n4]] == 4).all() and (q[want[n8 + n4:]] == 2).all()
+    assert np.array_equal(order.cpu().numpy()[:n8], want[:n8])

@@ -165,6 +165,10 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_thc_dequantize_irht(P, P, 1, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
     assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 and capi.eden_work_doubles(8192) == 2 and capi.bitrate_hist_ints() == 32768
+    # the sorted plan: four ints up to 65535 superchunks, the radix sort's buffers (about 12.2 bytes per superchunk) beyond
+    assert capi.group_plan_sorted_work_ints(65535) == 4
+    big = capi.group_plan_sorted_work_ints(8_000_000)
+    assert 4 * big >= 12 * 8_000_000 and 4 * big < 13 * 8_000_000
     # a good call clears the message
     assert L.dq_scaling_check_common(256, 4, 16, 2, 1) == 0 and L.dq_last_error().decode() == ""
     assert L.dq_status_string(16).decode() == "kernel launch failed"
