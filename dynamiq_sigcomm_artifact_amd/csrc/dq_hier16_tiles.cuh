@@ -145,6 +145,45 @@ __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const
     window_flush(win_out, gout, mis, total, lane);
 }
 
+// The row list of the tiles a wave works through.  A wave that takes several tiles fetches their entries with one load
+// (lane l holds entry first + l) and hands them out by a lane shuffle: the dependent load in front of a tile's element
+// loads is then paid once per wave instead of once per tile, which is what keeps the row-list kernels from the rate of
+// the plain ones on long buckets.  With a single tile per wave the entries are loaded where they are used, as before.
+struct RowIds {
+    const int32_t *rows; // null: the identity
+    int64_t first;       // entry held by lane 0
+    int32_t held;
+    bool prefetched;
+};
+
+__device__ __forceinline__ RowIds row_ids_plain(const int32_t *rows)
+{
+    RowIds ids;
+    ids.rows = rows; ids.first = 0; ids.held = 0; ids.prefetched = false;
+    return ids;
+}
+
+// entries [first, first + count) of rows (count <= 64, clipped to the list's length nsc)
+__device__ __forceinline__ RowIds row_ids_prefetch(const int32_t *rows, int64_t first, int count, int64_t nsc, int lane)
+{
+    RowIds ids = row_ids_plain(rows);
+    if (rows && count > kRowsPerWave) {
+        ids.first = first;
+        ids.held = (lane < count && first + lane < nsc) ? rows[first + lane] : 0;
+        ids.prefetched = true;
+    }
+    return ids;
+}
+
+// entry k of the list (k the entry itself when there is no list).  Called by every lane of the wave with k inside
+// the list: a prefetched entry comes out of another lane's register.
+__device__ __forceinline__ int64_t row_id(const RowIds &ids, int64_t k)
+{
+    if (!ids.rows) return k;
+    if (ids.prefetched) return (int64_t)__shfl(ids.held, (int)(k - ids.first), 64);
+    return (int64_t)ids.rows[k];
+}
+
 // compress (FUSED = false) or decode-accumulate-recompress (FUSED = true) of tile `tile` of a run of nsc
 // records.  Record k of the packed streams (and row k of rnd) belongs to superchunk rows[k] of src
 // (to superchunk k when rows is null).  win_out / win_in: Rec<NBITS>::WIN bytes of LDS each, 16-byte
@@ -152,7 +191,7 @@ __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const
 template <int DT, int RDT, int NBITS, bool MEE, bool FUSED>
 __device__ __forceinline__ void compress_tile(const void *__restrict__ src, const uint8_t *__restrict__ recv,
                                               uint8_t *__restrict__ dst, const void *__restrict__ rnd,
-                                              const int32_t *__restrict__ rows, int64_t nsc, int64_t tile, int vec,
+                                              const RowIds &rows, int64_t nsc, int64_t tile, int vec,
                                               const RandKey &key, const Center &ctr, const MeeArg<NBITS, MEE> &mp,
                                               uint8_t *win_out, uint8_t *win_in, float *table)
 {
@@ -175,12 +214,12 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
     Raw16<RDT> r;
     v.zero();
     r.zero();
-    int64_t sc_src = sc0 + row, e0 = 0;
+    const int64_t sc_src = row_id(rows, sc0 + min(row, rows_here - 1)); // every lane asks, for an entry of the list
+    int64_t e0 = 0;
     float mean = 0.0f;
     bool whole = true;
     if (active) {
         if constexpr (RDT != DQ_PHILOX) r.load(rnd, (sc0 * 16 + lane) * 16, vec & 2);
-        if (rows) sc_src = rows[sc0 + row];
         e0 = (sc_src * 16 + j) * 16;
         if (ctr.mean) {
             mean = ctr.mean[sc_src];
@@ -220,7 +259,7 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
 // 16-byte slots of LDS; table: 2^NBITS floats of LDS (only when MEE).
 template <int DT, int NBITS, bool MEE, bool ADD>
 __device__ __forceinline__ void decompress_tile(const uint8_t *__restrict__ src, void *__restrict__ dst,
-                                                const int32_t *__restrict__ rows, const uint16_t *__restrict__ stats,
+                                                const RowIds &rows, const uint16_t *__restrict__ stats,
                                                 int64_t limit, int64_t nsc, int64_t tile, int vec,
                                                 const MeeArg<NBITS, MEE> &mp, uint8_t *win_in, uint4 *tile_out, float *table)
 {
@@ -239,18 +278,10 @@ __device__ __forceinline__ void decompress_tile(const uint8_t *__restrict__ src,
 
     const WinRegs wr = window_fetch(src + sc0 * RC::REC, total, lane);
     // destination superchunk of this lane's chunk, and of the slots this lane stores after the transpose
-    int64_t d_own = sc0 + row;
+    const int64_t d_own = row_id(rows, sc0 + min(row, rows_here - 1)); // every lane asks, for an entry of the list
     int64_t d_slot[S];
 #pragma unroll
-    for (int k = 0; k < S; k++) d_slot[k] = sc0 + (64 * k + lane) / (16 * S);
-    if (rows) {
-        if (active) d_own = rows[sc0 + row];
-#pragma unroll
-        for (int k = 0; k < S; k++) {
-            const int rr = (64 * k + lane) / (16 * S);
-            if (rr < rows_here) d_slot[k] = rows[sc0 + rr];
-        }
-    }
+    for (int k = 0; k < S; k++) d_slot[k] = row_id(rows, sc0 + min((64 * k + lane) / (16 * S), rows_here - 1));
     Raw16<DT> acc;
     if (ADD && active) acc.load(dst, d_own * 256 + j * 16, vec);
     uint32_t mean_bits = 0; // widened where it is used, so that nothing waits for this load here

@@ -57,11 +57,16 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     __shared__ __attribute__((aligned(16))) uint8_t win_in[FUSED ? RC::WIN : 16];
     __shared__ float table[(MEE && FUSED) ? (1 << NBITS) : 1];
     const Center none{nullptr, 0, {0.0f, 0.0, 0}};
-    compress_tile<DT, RDT, NBITS, MEE, FUSED>(src, recv, dst, rnd, rows, nsc, blockIdx.x, vec, key, none, mp, win_out, win_in,
-                                              table);
+    compress_tile<DT, RDT, NBITS, MEE, FUSED>(src, recv, dst, rnd, row_ids_plain(rows), nsc, blockIdx.x, vec, key, none, mp, win_out,
+                                              win_in, table);
 }
 
-template <int DT, int NBITS, bool MEE, bool ADD>
+// LONG: the wave takes kTilesPerWaveLong consecutive tiles of a row list and fetches their entries with one load (RowIds).
+// A variant of its own: the loop costs registers (about 50 instead of 20), which the one-tile kernel need not pay.  The
+// encoder has no such variant: looped, it keeps so many scalars alive that they spill into vector registers (over 100).
+constexpr int kTilesPerWaveLong = 4;
+
+template <int DT, int NBITS, bool MEE, bool ADD, bool LONG>
 __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
                                                               const int32_t *__restrict__ rows,
                                                               const uint16_t *__restrict__ stats, int64_t limit,
@@ -70,14 +75,31 @@ __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__
     __shared__ __attribute__((aligned(16))) uint8_t win_in[Rec<NBITS>::WIN];
     __shared__ __attribute__((aligned(16))) uint4 tile_out[64 * Raw16<DT>::kSlots];
     __shared__ float table[MEE ? (1 << NBITS) : 1];
-    decompress_tile<DT, NBITS, MEE, ADD>(src, dst, rows, stats, limit, nsc, blockIdx.x, vec, mp, win_in, tile_out, table);
+    if constexpr (LONG) {
+        const int64_t tile0 = (int64_t)blockIdx.x * kTilesPerWaveLong;
+        const RowIds ids = row_ids_prefetch(rows, tile0 * kRowsPerWave, kTilesPerWaveLong * kRowsPerWave, nsc, threadIdx.x);
+#pragma unroll 1
+        for (int t = 0; t < kTilesPerWaveLong; t++) {
+            decompress_tile<DT, NBITS, MEE, ADD>(src, dst, ids, stats, limit, nsc, tile0 + t, vec, mp, win_in, tile_out, table);
+            wave_lds_sync(); // window, table and output tile are reused by the next tile
+        }
+    } else {
+        decompress_tile<DT, NBITS, MEE, ADD>(src, dst, row_ids_plain(rows), stats, limit, nsc, blockIdx.x, vec, mp, win_in, tile_out,
+                                             table);
+    }
 }
 
 // ---- launchers ------------------------------------------------------------------------------------
 
 
-// one single-wave workgroup per tile of 4 superchunks
-static inline unsigned grid_for(int64_t nsc) { return (unsigned)((nsc + kRowsPerWave - 1) / kRowsPerWave); }
+// one single-wave workgroup per tile of 4 superchunks (per kTilesPerWaveLong tiles in the LONG decoder)
+static inline unsigned grid_for(int64_t nsc, int tiles = 1)
+{
+    const int64_t per = (int64_t)kRowsPerWave * tiles;
+    return (unsigned)((nsc + per - 1) / per);
+}
+
+constexpr int64_t kLongRun = 262144; // superchunks of a row list: 16384 waves of four tiles, two rounds of a full chip
 
 template <int DT, int RDT, int NBITS, bool MEE>
 static hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, const int32_t *rows,
@@ -98,12 +120,19 @@ static hipError_t run_decompress(const uint8_t *src, void *dst, const int32_t *r
                                  int64_t nsc, int add, const MeeParams &mp, hipStream_t stream)
 {
     auto arg = make_arg<NBITS, MEE>(mp);
-    dim3 grid(grid_for(nsc)), block(64);
+    dim3 block(64);
     const int vec = aligned16(dst) ? 1 : 0;
+    if (rows && nsc >= kLongRun && !add) {
+        // a long row list (the decoder of the grouped pipelines on the reference's whole-model buckets)
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false, true>), dim3(grid_for(nsc, kTilesPerWaveLong)), block, 0,
+                           stream, src, dst, rows, stats, limit, nsc, vec, arg);
+        return hipGetLastError();
+    }
+    dim3 grid(grid_for(nsc));
     if (add)
-        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, true>), grid, block, 0, stream, src, dst, rows, stats, limit, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, true, false>), grid, block, 0, stream, src, dst, rows, stats, limit, nsc, vec, arg);
     else
-        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false>), grid, block, 0, stream, src, dst, rows, stats, limit, nsc, vec, arg);
+        hipLaunchKernelGGL((hier16_decompress_kernel<DT, NBITS, MEE, false, false>), grid, block, 0, stream, src, dst, rows, stats, limit, nsc, vec, arg);
     return hipGetLastError();
 }
 

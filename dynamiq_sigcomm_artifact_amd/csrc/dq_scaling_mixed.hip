@@ -24,6 +24,10 @@ namespace dq {
 
 namespace {
 
+// the decoder's waves take one tile of a run, or four in a row when the ring chunk is long
+constexpr int kSpanLong = 4;
+constexpr int64_t kLongChunk = 262144; // superchunks per ring chunk
+
 struct MixedPlan {
     const int32_t *order;  // superchunk indices: the 8-bit group from entry 0, the 4-bit group from nsc, the 2-bit group from 2 nsc
     const int32_t *counts; // n8, n4, n2
@@ -33,14 +37,15 @@ struct MixedPlan {
 
 struct Segment {
     int cls;          // 0: 8-bit, 1: 4-bit, 2: 2-bit, 3: nothing to do
-    int tile;         // tile inside the run
+    int tile;         // first tile inside the run
     int cnt;          // records in the run
     int64_t row0;     // entry of `order` holding the run's first superchunk
     int64_t pos0;     // rank of that superchunk in the concatenation 8 | 4 | 2 (row of the random pool)
     int64_t byte_off; // where the run starts in the packed stream
 };
 
-__device__ __forceinline__ Segment locate(const MixedPlan &p, int block)
+// block -> the run (bit-width group of the ring chunk) it works in and its first tile there; a block takes `span` tiles
+__device__ __forceinline__ Segment locate(const MixedPlan &p, int block, int span)
 {
     constexpr int kRec[3] = {Rec<8>::REC, Rec<4>::REC, Rec<2>::REC};
     Segment s;
@@ -55,9 +60,9 @@ __device__ __forceinline__ Segment locate(const MixedPlan &p, int block)
         const int per = (n + p.world - 1) / p.world;
         const int begin = (int)min((int64_t)per * p.chunk, (int64_t)n);
         const int cnt = min(per, n - begin);
-        const int tiles = (cnt + kRowsPerWave - 1) / kRowsPerWave;
+        const int tiles = ((cnt + kRowsPerWave - 1) / kRowsPerWave + span - 1) / span; // blocks of this run
         if (s.cls == 3 && t < tiles) {
-            s.cls = g; s.tile = t; s.cnt = cnt; s.row0 = (int64_t)g * p.nsc + begin; s.pos0 = pos + begin; s.byte_off = off;
+            s.cls = g; s.tile = t * span; s.cnt = cnt; s.row0 = (int64_t)g * p.nsc + begin; s.pos0 = pos + begin; s.byte_off = off;
         }
         t -= tiles;
         pos += n;
@@ -77,9 +82,9 @@ __global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restri
     __shared__ float table[(MEE && FUSED) ? 256 : 1];
     constexpr int RESZ = RDT == DQ_F32 ? 4 : 2;
 
-    const Segment s = locate(plan, blockIdx.x);
+    const Segment s = locate(plan, blockIdx.x, 1);
     if (s.cls == 3) return;
-    const int32_t *rows = plan.order + s.row0;
+    const RowIds rows = row_ids_plain(plan.order + s.row0);
     const void *r = RDT == DQ_PHILOX ? nullptr : static_cast<const char *>(rnd) + s.pos0 * 256 * RESZ;
     const uint8_t *in = FUSED ? recv + s.byte_off : nullptr;
     uint8_t *out = dst + s.byte_off;
@@ -96,36 +101,48 @@ __global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restri
     }
 }
 
-template <int DT, bool MEE>
+// LONG: a wave takes kSpanLong consecutive tiles of its run and fetches their row-list entries with one load (RowIds);
+// a variant of its own because the loop costs registers (about 50 instead of 20).  The encoder stays with one tile per
+// wave: looped, it keeps so many scalars alive that they spill into vector registers (over 100).
+template <int DT, bool MEE, bool LONG>
 __global__ __launch_bounds__(64) void mixed_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
                                                              MixedPlan plan, const uint16_t *__restrict__ stats,
                                                              int64_t limit, int vec, MeeArg<8, MEE> m8, MeeArg<4, MEE> m4,
                                                              MeeArg<2, MEE> m2)
 {
+    constexpr int span = LONG ? kSpanLong : 1;
     __shared__ __attribute__((aligned(16))) uint8_t win_in[Rec<8>::WIN];
     __shared__ __attribute__((aligned(16))) uint4 tile_out[64 * Raw16<DT>::kSlots];
     __shared__ float table[MEE ? 256 : 1];
 
-    const Segment s = locate(plan, blockIdx.x);
+    const Segment s = locate(plan, blockIdx.x, span);
     if (s.cls == 3) return;
-    const int32_t *rows = plan.order + s.row0;
+    const RowIds rows = LONG ? row_ids_prefetch(plan.order + s.row0, (int64_t)s.tile * kRowsPerWave, span * kRowsPerWave, s.cnt, threadIdx.x)
+                             : row_ids_plain(plan.order + s.row0);
     const uint8_t *in = src + s.byte_off;
-    switch (s.cls) {
-    case 0:
-        decompress_tile<DT, 8, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile, vec, m8, win_in, tile_out, table);
-        break;
-    case 1:
-        decompress_tile<DT, 4, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile, vec, m4, win_in, tile_out, table);
-        break;
-    default:
-        decompress_tile<DT, 2, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile, vec, m2, win_in, tile_out, table);
-        break;
+#define DQ_MIXED_TILES(NBITS, ARG)                                                                                         \
+    _Pragma("unroll 1") for (int t = 0; t < span; t++)                                                                     \
+    {                                                                                                                      \
+        decompress_tile<DT, NBITS, MEE, false>(in, dst, rows, stats, limit, s.cnt, s.tile + t, vec, ARG, win_in, tile_out, \
+                                               table);                                                                     \
+        wave_lds_sync(); /* window, table and output tile are reused by the next tile */                                   \
     }
+    switch (s.cls) {
+    case 0: DQ_MIXED_TILES(8, m8) break;
+    case 1: DQ_MIXED_TILES(4, m4) break;
+    default: DQ_MIXED_TILES(2, m2) break;
+    }
+#undef DQ_MIXED_TILES
 }
 
-// every group rounds its share of a ring chunk up to whole superchunks and its superchunks up to whole
-// tiles: at most nsc / world + 3 records and nsc / (4 world) + 3 tiles
-inline unsigned grid_for(int64_t nsc, int world) { return (unsigned)(nsc / ((int64_t)kRowsPerWave * world) + 4); }
+inline int span_for(int64_t nsc, int world) { return nsc / world >= kLongChunk ? kSpanLong : 1; }
+
+// every group rounds its share of a ring chunk up to whole superchunks, its superchunks up to whole tiles and its tiles
+// up to whole blocks of `span`: at most nsc / world + 3 records and nsc / (4 span world) + 3 blocks
+inline unsigned grid_for(int64_t nsc, int world, int span)
+{
+    return (unsigned)(nsc / ((int64_t)kRowsPerWave * span * world) + 4);
+}
 
 template <int DT, int RDT, bool MEE>
 hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, const void *rnd, const MixedPlan &plan,
@@ -134,7 +151,7 @@ hipError_t run_compress(const void *src, const uint8_t *recv, uint8_t *dst, cons
     const auto m8 = make_arg<8, MEE>(mp[0]);
     const auto m4 = make_arg<4, MEE>(mp[1]);
     const auto m2 = make_arg<2, MEE>(mp[2]);
-    dim3 grid(grid_for(nsc, plan.world)), block(64);
+    dim3 grid(grid_for(nsc, plan.world, 1)), block(64);
     const int vec = (aligned16(src) ? 1 : 0) | (aligned16(rnd) ? 2 : 0);
     if (recv)
         hipLaunchKernelGGL((mixed_compress_kernel<DT, RDT, MEE, true>), grid, block, 0, stream, src, recv, dst, rnd, plan, vec,
@@ -152,8 +169,13 @@ hipError_t run_decompress(const uint8_t *src, void *dst, const MixedPlan &plan, 
     const auto m8 = make_arg<8, MEE>(mp[0]);
     const auto m4 = make_arg<4, MEE>(mp[1]);
     const auto m2 = make_arg<2, MEE>(mp[2]);
-    hipLaunchKernelGGL((mixed_decompress_kernel<DT, MEE>), dim3(grid_for(nsc, plan.world)), dim3(64), 0, stream, src, dst, plan,
-                       stats, limit, aligned16(dst) ? 1 : 0, m8, m4, m2);
+    const int span = span_for(nsc, plan.world);
+    if (span > 1)
+        hipLaunchKernelGGL((mixed_decompress_kernel<DT, MEE, true>), dim3(grid_for(nsc, plan.world, span)), dim3(64), 0, stream, src,
+                           dst, plan, stats, limit, aligned16(dst) ? 1 : 0, m8, m4, m2);
+    else
+        hipLaunchKernelGGL((mixed_decompress_kernel<DT, MEE, false>), dim3(grid_for(nsc, plan.world, 1)), dim3(64), 0, stream, src,
+                           dst, plan, stats, limit, aligned16(dst) ? 1 : 0, m8, m4, m2);
     return hipGetLastError();
 }
 
