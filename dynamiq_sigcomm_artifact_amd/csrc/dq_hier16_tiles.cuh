@@ -116,10 +116,9 @@ __device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int6
 // 16-byte aligned, owned by this wave.
 template <int NBITS, bool MEE, class RV, class RR>
 __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const MeeArg<NBITS, MEE> &mp, uint8_t *gout,
-                                                 int rows_here, uint8_t *win_out)
+                                                 int rows_here, uint8_t *win_out, int lane)
 {
     typedef Rec<NBITS> RC;
-    const int lane = threadIdx.x & 63;
     const int row = lane >> 4, j = lane & 15;
     const bool active = row < rows_here;
     const int total = rows_here * RC::REC;
@@ -193,10 +192,9 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
                                               uint8_t *__restrict__ dst, const void *__restrict__ rnd,
                                               const RowIds &rows, int64_t nsc, int64_t tile, int vec,
                                               const RandKey &key, const Center &ctr, const MeeArg<NBITS, MEE> &mp,
-                                              uint8_t *win_out, uint8_t *win_in, float *table)
+                                              uint8_t *win_out, uint8_t *win_in, float *table, int lane)
 {
     typedef Rec<NBITS> RC;
-    const int lane = threadIdx.x;
     const int row = lane >> 4, j = lane & 15;
     const int64_t sc0 = tile * kRowsPerWave;
     if (sc0 >= nsc) return;
@@ -228,7 +226,10 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
         if (whole) v.load(src, e0, vec & 1);
     }
     if (active) {
-        if constexpr (RDT == DQ_PHILOX) r.generate(key, sc_src * 16 + j); // keyed by the chunk's place in the source vector
+        if constexpr (RDT == DQ_PHILOX) {
+            r.generate(key, sc_src * 16 + j); // keyed by the chunk's place in the source vector
+            if (ctr.mean) r.pin();            // (the centring below is the first to wait for the loads)
+        }
         if (ctr.mean) center_chunk<DT>(v, src, e0, ctr, mean, whole);
     }
 
@@ -249,7 +250,7 @@ __device__ __forceinline__ void compress_tile(const void *__restrict__ src, cons
         }
     }
 
-    encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, rows_here, win_out);
+    encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, rows_here, win_out, lane & 63);
 }
 
 // Tile `tile` of a run of nsc records: record k decodes into superchunk rows[k] of dst (superchunk k when

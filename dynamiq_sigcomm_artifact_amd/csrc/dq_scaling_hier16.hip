@@ -58,12 +58,13 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     __shared__ float table[(MEE && FUSED) ? (1 << NBITS) : 1];
     const Center none{nullptr, 0, {0.0f, 0.0, 0}};
     compress_tile<DT, RDT, NBITS, MEE, FUSED>(src, recv, dst, rnd, row_ids_plain(rows), nsc, blockIdx.x, vec, key, none, mp, win_out,
-                                              win_in, table);
+                                              win_in, table, threadIdx.x);
 }
 
 // LONG: the wave takes kTilesPerWaveLong consecutive tiles of a row list and fetches their entries with one load (RowIds).
 // A variant of its own: the loop costs registers (about 50 instead of 20), which the one-tile kernel need not pay.  The
-// encoder has no such variant: looped, it keeps so many scalars alive that they spill into vector registers (over 100).
+// encoder has no such variant: its time on long buckets goes into arithmetic, not into the wait for the row list, and
+// looped it holds every literal of its tile body in a register of its own (over 100 registers).
 constexpr int kTilesPerWaveLong = 4;
 
 template <int DT, int NBITS, bool MEE, bool ADD, bool LONG>

@@ -88,22 +88,24 @@ __global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restri
     const void *r = RDT == DQ_PHILOX ? nullptr : static_cast<const char *>(rnd) + s.pos0 * 256 * RESZ;
     const uint8_t *in = FUSED ? recv + s.byte_off : nullptr;
     uint8_t *out = dst + s.byte_off;
+    const int lane = threadIdx.x;
     switch (s.cls) {
     case 0:
-        compress_tile<DT, RDT, 8, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m8, win_out, win_in, table);
+        compress_tile<DT, RDT, 8, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m8, win_out, win_in, table, lane);
         break;
     case 1:
-        compress_tile<DT, RDT, 4, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m4, win_out, win_in, table);
+        compress_tile<DT, RDT, 4, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m4, win_out, win_in, table, lane);
         break;
     default:
-        compress_tile<DT, RDT, 2, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m2, win_out, win_in, table);
+        compress_tile<DT, RDT, 2, MEE, FUSED>(src, in, out, r, rows, s.cnt, s.tile, vec, key, ctr, m2, win_out, win_in, table, lane);
         break;
     }
 }
 
 // LONG: a wave takes kSpanLong consecutive tiles of its run and fetches their row-list entries with one load (RowIds);
 // a variant of its own because the loop costs registers (about 50 instead of 20).  The encoder stays with one tile per
-// wave: looped, it keeps so many scalars alive that they spill into vector registers (over 100).
+// wave: its time on long buckets goes into arithmetic (the centring above all), not into the wait for the row list, and
+// looped it holds every literal of its tile body in a register of its own (over 100 registers).
 template <int DT, bool MEE, bool LONG>
 __global__ __launch_bounds__(64) void mixed_decompress_kernel(const uint8_t *__restrict__ src, void *__restrict__ dst,
                                                              MixedPlan plan, const uint16_t *__restrict__ stats,

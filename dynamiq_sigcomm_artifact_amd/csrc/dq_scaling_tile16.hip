@@ -118,7 +118,12 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
     // [0, 1]: the codes come from the estimate with its exact redo near the rounding boundaries
     bool estimated = false;
     if constexpr (DT != DQ_F16) {
-        estimated = fast && __builtin_amdgcn_ballot_w64(!r.unit_interval()) == 0;
+        // the largest-magnitude search above passes over NaN elements (as the reference's does), so the scale says
+        // nothing about them: v * 0 summed over the chunk is NaN exactly when one of them is not finite
+        float finite = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) finite = __builtin_fmaf(v.get(i), 0.0f, finite);
+        estimated = fast && __builtin_amdgcn_ballot_w64(!r.unit_interval() || finite != finite) == 0;
         if (estimated) estimate_codes<NBITS, MEE>(v, r, d, mp, w);
     }
     const double yd = fast && !estimated ? recip_f64(d) : 0.0;

@@ -3,6 +3,7 @@
 // 64 chunks whose packed bytes form one contiguous run of the record stream.
 #pragma once
 
+#include <type_traits>
 #include "dq_device.cuh"
 
 namespace dq {
@@ -188,13 +189,27 @@ template <> struct Raw16<DQ_F16> : Raw16<DQ_BF16> {
 constexpr int DQ_PHILOX = 3;
 
 template <> struct Raw16<DQ_PHILOX> {
-    uint32_t w[4];
-    __device__ __forceinline__ void zero() { w[0] = w[1] = w[2] = w[3] = 0; }
-    __device__ __forceinline__ void generate(const RandKey &key, int64_t chunk) { chunk_uniform_words(key, chunk, w); }
+    uint32_t w[4]; // the generator's words with the lowest bit of every byte set
+    __device__ __forceinline__ void zero() { w[0] = w[1] = w[2] = w[3] = 0x01010101u; }
+    __device__ __forceinline__ void generate(const RandKey &key, int64_t chunk)
+    {
+        chunk_uniform_words(key, chunk, w);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            w[k] |= 0x01010101u;
+            // (the compiler would otherwise push the OR back into every byte's extraction)
+            asm("" : "+v"(w[k]));
+        }
+    }
+    // the generator's arithmetic stays where generate() was called (behind the tile's loads, in front of whatever waits
+    // for them) instead of sinking to the first use of its words
+    __device__ __forceinline__ void pin() const { asm volatile("" ::"v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3])); }
     __device__ __forceinline__ void load(const void *, int64_t, bool) {}
+    // (byte i | 1) as a float: one byte-to-float conversion
+    __device__ __forceinline__ float odd_byte(int i) const { return (float)((w[i >> 2] >> (8 * (i & 3))) & 0xffu); }
     __device__ __forceinline__ float get(int i) const
     {
-        return (float)(((w[i >> 2] >> (8 * (i & 3))) & 0xffu) | 1u) * 0.00390625f;
+        return odd_byte(i) * 0.00390625f;
     }
     __device__ __forceinline__ bool unit_interval() const { return true; }
 };
@@ -383,23 +398,47 @@ __device__ __forceinline__ int exact_code_fast(float vi, float ri, double yd, co
     return (int)(fl + c); // |fl| <= R + 1 and c in {-1, 0, 1}: exact
 }
 
-// The code of an element is ceil(L - r) for the coordinate L the exact chain computes -- v / d (AEE) or
-// +-log2(|v / d| / c + 1) / log2(base) (MEE) -- because floor(L) + ceil(frac(L) - r) is that integer.  A cheap
-// estimate of L - r gives the same code unless it comes within kDelta of an integer; such elements (one in a few
-// thousand) are redone with the exact chain, so the bytes are those of the exact chain throughout.
-//   AEE: estimate fma(v, rcp(d), -r); the hardware reciprocal is good to 1 ulp, so the distance to the exact
-//        v / d - r is below (R + 1) (2^-23 + 2^-24) + ulp(R + 1) / 2 < 0.27 (R + 1) 2^-20.
-//   MEE: estimate fma(v_log_f32(fma(|v rcp(d)|, 1 / c, 1)), +-1 / log2(base), -r), v_log_f32 being good to 1 ulp;
+// The code of an element is clamp(ceil(L - r), -R, R) + R for the coordinate L the exact chain computes -- v / d (AEE)
+// or +-log2(|v / d| / c + 1) / log2(base) (MEE) -- because floor(L) + ceil(frac(L) - r) is that integer; and it is
+// min(floor(L - r + R + 1), 2R) (nothing below zero) as long as L - r is not an integer.  A cheap estimate T of
+// L - r + R + 1 gives the same code unless it comes within kDelta of an integer; such elements (one in a few thousand)
+// are redone with the exact chain, so the bytes are those of the exact chain throughout.
+//   AEE: T = fma(v, rcp(d), (R + 1) - r).  The hardware reciprocal is good to 1 ulp (|v rcp(d) - v / d| < (R + 1) 2^-23),
+//        (R + 1) - r is exact for the in-kernel random bytes and within (R + 1) 2^-26 otherwise, and the fma rounds a
+//        value below 2 (R + 1): its distance to the exact L - r + R + 1 stays below 0.27 (R + 1) 2^-20.
+//   MEE: T = fma(v_log_f32(fma(|v rcp(d)|, 1 / c, 1)), +-1 / log2(base), (R + 1) - r), v_log_f32 being good to 1 ulp;
 //        estimate and exact chain both approximate log2(|v| / (d c) + 1) / log2(base), their distance is bounded by
-//        (1.44 * 5e-7 + 2.7 ulp(log)) / log2(base) + 2 ulp(R): < 6.5e-5 for 6..8 bits (log2(base) = 0.0286, log < 4)
-//        and < 1.1e-5 below (log2(base) >= 0.09, log < 1.5); measured over 4e9 random operands per width: 1.5e-5
-//        and 4.8e-6.
+//        (1.44 * 5e-7 + 2.7 ulp(log)) / log2(base) + 2 ulp(2 R): < 6.9e-5 for 6..8 bits (log2(base) = 0.0286, log < 4)
+//        and < 1.2e-5 below (log2(base) >= 0.09, log < 1.5); measured over 4e9 random operands per width: 1.5e-5
+//        and 4.8e-6 (without the offset in the last fma, which adds at most 3.8e-6 and 1e-6).
 template <int NBITS, bool MEE> struct EstimateGuard {
     static constexpr float kDelta = MEE ? (NBITS >= 6 ? 0x1p-12f : 0x1p-14f) : (float)(1 << (NBITS - 1)) * 0x1p-20f;
 };
 
-// The codes of one chunk against the step d (normal, 2^-100 <= d <= 2^100) for elements that are finite with
-// |v| <= (R + 1) d and random values in [0, 1]: estimate, guard, exact redo.  w must be zeroed.
+// bias - r_i; exact for the in-kernel random bytes ((256 bias - odd byte) / 256 needs 16 bits)
+template <class RR> __device__ __forceinline__ float below(const RR &r, int i, float bias)
+{
+    if constexpr (std::is_same<RR, Raw16<DQ_PHILOX>>::value)
+        return __builtin_fmaf(r.odd_byte(i), -0.00390625f, bias);
+    else
+        return bias - r.get(i);
+}
+
+template <int NBITS, bool MEE, class RV, class RR>
+__device__ __forceinline__ float estimate_coordinate(const RV &v, const RR &r, int i, float rd, float rc, float rl2b)
+{
+    const float vi = v.get(i);
+    const float off = below(r, i, (float)(Rec<NBITS>::R + 1));
+    if (MEE) {
+        const float est = __builtin_amdgcn_logf(__builtin_fmaf(__builtin_fabsf(vi * rd), rc, 1.0f));
+        return __builtin_fmaf(est, __builtin_copysignf(rl2b, vi), off);
+    }
+    return __builtin_fmaf(vi, rd, off);
+}
+
+// The codes of one chunk against the step d (normal, 2^-100 <= d <= 2^100) for elements that are finite (a NaN would
+// pass the guard unnoticed) with |v| <= (R + 1) d and random values in [0, 1]: estimate, guard, exact redo.  w must
+// be zeroed.
 template <int NBITS, bool MEE, class RV, class RR, class ARG>
 __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d, const ARG &mp, uint32_t (&w)[Rec<NBITS>::WORDS])
 {
@@ -410,29 +449,20 @@ __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d
     bool doubt[16], any = false;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-        const float vi = v.get(i);
-        float t;
-        if (MEE) {
-            const float est = __builtin_amdgcn_logf(__builtin_fmaf(__builtin_fabsf(vi * rd), rc, 1.0f));
-            t = __builtin_fmaf(est, __builtin_copysignf(rl2b, vi), -r.get(i));
-        } else {
-            t = __builtin_fmaf(vi, rd, -r.get(i));
-        }
-        const float c = __builtin_ceilf(t);
-        doubt[i] = __builtin_fabsf((c - t) - 0.5f) > 0.5f - kDelta;
+        const float t = estimate_coordinate<NBITS, MEE>(v, r, i, rd, rc, rl2b);
+        doubt[i] = __builtin_fabsf(__builtin_amdgcn_fractf(t) - 0.5f) > 0.5f - kDelta;
         any |= doubt[i];
-        const int sv = (int)c; // |t| < 2^20: exact
-        words_put<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
+        words_put<NBITS>(w, i, (uint32_t)__builtin_amdgcn_fmed3f(t, 0.0f, (float)(2 * R))); // T < 2^20: exact
     }
     if (__builtin_amdgcn_ballot_w64(any) != 0) {
         const double yd = recip_f64(d);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            // a zero element has L = 0 on both routes whatever its random value is
-            const bool redo = doubt[i] && (__float_as_uint(v.get(i)) << 1) != 0;
-            if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+            if (__builtin_amdgcn_ballot_w64(doubt[i]) != 0) {
+                // (among them the zero elements -- padding, sparse input -- whose random value is exactly 0 or 1: their
+                // T is an integer, and the chain's ceil(-r) is 0, or -1 at r = 1)
                 const int sv = exact_code_fast<MEE>(v.get(i), r.get(i), yd, mp);
-                if (redo) words_set<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
+                if (doubt[i]) words_set<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
             }
         }
     }

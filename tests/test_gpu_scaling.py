@@ -179,6 +179,35 @@ def test_special_values(capi, oracle, dt, strategy):
         _roundtrip_nan_safe(capi, oracle, dt, n, nbits, 16, strategy, src, rnd, "special b=%d" % nbits)
 
 
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+@pytest.mark.parametrize("C", [16, 8, 32])
+def test_zero_elements_with_random_values_0_and_1(capi, oracle, dt, strategy, C):
+    """Ordinary magnitudes throughout (so every wave takes the estimate route), many exact zeros of either sign, and
+    random values that are exactly 0 and exactly 1 on zero and non-zero elements alike: coordinate - random value is an
+    integer for those zeros, the case the estimate cannot decide (ceil(-0) = 0, ceil(-1) = -1 in the reference's chain)."""
+    tdt = TORCH_DT[dt]
+    n = 256 * 24
+    g = torch.Generator().manual_seed(77 + strategy)
+    src = torch.randn(n, generator=g) * 1e-2
+    src[torch.rand(n, generator=g) < 0.4] = 0.0
+    src[5::13] = -0.0
+    src[1024:1280] = 0.0            # whole superchunks of zeros
+    src = src.to(tdt)
+    rnd = torch.rand(n, generator=g)
+    rnd[::3] = 0.0
+    rnd[1::5] = 1.0
+    rnd = rnd.to(tdt)
+    for nbits in (2, 4, 5, 8):
+        if (C * nbits) % 8:
+            continue
+        tag = "zeros dt=%d C=%d b=%d s=%d" % (dt, C, nbits, strategy)
+        _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src, rnd, tag)
+        inp = (torch.randn(n, generator=g) * 1e-2)
+        inp[torch.rand(n, generator=g) < 0.5] = 0.0
+        _dec_comp(capi, oracle, dt, n, nbits, C, strategy, src, inp.to(tdt), rnd, rnd.flip(0).contiguous(), tag)
+
+
 @pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [2, 3])
 @pytest.mark.parametrize("C", [16, 8, 32])
