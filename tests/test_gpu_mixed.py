@@ -87,6 +87,46 @@ def test_mixed_matches_per_group_calls(capi, dt, strategy, nsc, world, weights):
     assert bool((out[n_valid:] == 7.0).all())
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("strategy,world", [(2, 1), (3, 2)])
+def test_long_runs_take_the_decoders_of_several_tiles_per_wave(capi, dt, strategy, world):
+    """From 262,144 superchunks per ring chunk (or rows of a list) on, the decoders run as waves of four tiles that fetch
+    their row-list entries with one load.  Their output must be that of the one-tile kernels, which the same records
+    reach here in pieces of 100,000 rows."""
+    nsc = 450_001 * world + 5
+    n_valid = nsc * 256 - 77
+    q, order, work = make_plan(capi, nsc, 11 + world, (1, 6, 2))
+    counts = work[:3].tolist()
+    g = torch.Generator(device=DEV).manual_seed(5 + strategy)
+    full = (torch.randn(nsc * 256, generator=g, device=DEV) * 1e-2).to(dt)
+    stats = torch.randn(nsc, 2, generator=g, device=DEV).mul(1e-2).to(torch.bfloat16)
+    cap = capi.mixed_required_bytes(nsc, world)
+    out = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
+    out_ref = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
+    out_rows = torch.full((n_valid + 300,), 7.0, dtype=dt, device=DEV)
+    long_runs = 0
+    for chunk in range(world):
+        segs, total = segments(counts, chunk, world, nsc)
+        enc = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+        capi.mixed_compress(full, order, work, enc, nsc, strategy, seed=3, step=chunk, ring_chunk=chunk, ring_world=world)
+        capi.mixed_decompress(enc, out, order, work, nsc, strategy, stats=stats, n_limit=n_valid, ring_chunk=chunk,
+                              ring_world=world)
+        for width, row0, pos, cnt, off in segs:
+            rows = order[row0:row0 + cnt]
+            for a in range(0, cnt, 100_000):
+                b = min(cnt, a + 100_000)
+                capi.scaling_decompress_rows(enc[off + a * REC[width]:off + b * REC[width]], out_ref, rows[a:b], stats, n_valid,
+                                             b - a, width, strategy)
+            capi.scaling_decompress_rows(enc[off:off + cnt * REC[width]], out_rows, rows, stats, n_valid, cnt, width, strategy)
+            long_runs += cnt >= 262144
+    assert long_runs >= 1                  # the row-list decoder took its long variant as well
+    assert torch.equal(bits_t(out), bits_t(out_ref))
+    assert torch.equal(bits_t(out_rows), bits_t(out_ref))
+    assert bool((out[n_valid:] == 7.0).all()) and bool((out_rows[n_valid:] == 7.0).all())
+    # and the decoded values are the source to within the 2-bit step of its widest class
+    assert float((out[:n_valid].float() - stats[:, 0].float().repeat_interleave(256)[:n_valid] - full[:n_valid].float()).abs().max()) < 0.1
+
+
 @pytest.mark.parametrize("dt,odt", [(torch.bfloat16, BF16), (torch.float32, F32)])
 @pytest.mark.parametrize("strategy", [2, 3])
 def test_mixed_philox_matches_oracle(capi, oracle, dt, odt, strategy):
