@@ -101,7 +101,7 @@ hipError_t launch_bits_to_bins(int32_t *bins, int64_t nbins, const uint32_t *arr
 // four consecutive elements per thread share one Philox block keyed by
 // (seed, element index / 4); u = top 24 bits * 2^-24 in [0, 1)
 __global__ __launch_bounds__(256) void quantization_kernel(float *__restrict__ vec, int64_t n, float div_factor,
-                                                           float tensor_max, uint32_t k0, uint32_t k1)
+                                                           float tensor_max, uint32_t k0, uint32_t k1, bool vec16)
 {
     const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t i0 = g * 4;
@@ -109,22 +109,34 @@ __global__ __launch_bounds__(256) void quantization_kernel(float *__restrict__ v
     uint32_t c[4] = {(uint32_t)g, (uint32_t)((uint64_t)g >> 32), 0u, 0u};
     philox4x32_10(c, k0, k1);
     const int cnt = (int)min((int64_t)4, n - i0);
-    for (int k = 0; k < cnt; k++) {
-        float t = vec[i0 + k] / div_factor;
+    auto round_one = [&](float x, uint32_t word) {
+        float t = x / div_factor;
         t = t < tensor_max ? t : tensor_max;
         t = t > -tensor_max ? t : -tensor_max;
         const float fl = __builtin_floorf(t);
         const float prob = t - fl;
-        const float u = (float)(c[k] >> 8) * 5.9604644775390625e-08f;
-        vec[i0 + k] = fl + ((u < prob) ? 1.0f : 0.0f);
+        const float u = (float)(word >> 8) * 5.9604644775390625e-08f;
+        return fl + ((u < prob) ? 1.0f : 0.0f);
+    };
+    if (cnt == 4 && vec16) {
+        // the thread's four elements in one 16-byte access each way
+        float4 *p = reinterpret_cast<float4 *>(vec + i0);
+        float4 x = *p;
+        x.x = round_one(x.x, c[0]);
+        x.y = round_one(x.y, c[1]);
+        x.z = round_one(x.z, c[2]);
+        x.w = round_one(x.w, c[3]);
+        *p = x;
+        return;
     }
+    for (int k = 0; k < cnt; k++) vec[i0 + k] = round_one(vec[i0 + k], c[k]);
 }
 
 hipError_t launch_quantization(float *vec, int64_t n, float div_factor, float tensor_max, uint64_t seed, hipStream_t stream)
 {
     const int64_t groups = (n + 3) / 4;
     hipLaunchKernelGGL(quantization_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, vec, n, div_factor,
-                       tensor_max, (uint32_t)seed, (uint32_t)(seed >> 32));
+                       tensor_max, (uint32_t)seed, (uint32_t)(seed >> 32), (reinterpret_cast<uintptr_t>(vec) & 15) == 0);
     return hipGetLastError();
 }
 

@@ -238,6 +238,12 @@ def test_quantization_matches_oracle(capi, oracle, n):
         capi.quantization(q, div, tmax, seed)
         want = oracle.quantization(v.numpy(), div, tmax, seed)
         assert (q.cpu().numpy().view(np.uint32) == want.view(np.uint32)).all(), (n, div)
+        # a view that starts 4 bytes into a buffer (the kernel then leaves its 16-byte accesses)
+        buf = torch.full((n + 3,), 77.0, device=DEV)
+        buf[1:n + 1] = v.to(DEV)
+        capi.quantization(buf[1:n + 1], div, tmax, seed)
+        assert (buf[1:n + 1].cpu().numpy().view(np.uint32) == want.view(np.uint32)).all(), (n, div, "unaligned")
+        assert float(buf[0]) == 77.0 and bool((buf[n + 1:] == 77.0).all())
 
 
 def test_quantization_compression_module_stream(eden_utils, oracle):
