@@ -796,6 +796,50 @@ def quantiser_sizes(dev, nbits=4):
         del src, inp, rnd, out
 
 
+def long_bucket(dev, sizes=(1 << 26, 1 << 28)):
+    """the kernels of the dynamic-bitrate pipeline on buckets of the size the reference trains with
+    (bucket_cap_mb=4000, testbed_evaluation/train_llm_causal.py:416: up to 2 * 10^9 bf16 elements in one bucket):
+    statistics, plan, the three-width codec with centring on load and the mean added on store, and the single-width
+    codec beside them; bf16, target 4.375 bits, in-kernel rounding stream, graph-replayed"""
+    for n in sizes:
+        nsc = n // 256
+        g = torch.Generator(device=dev).manual_seed(3)
+        scale = torch.exp(torch.randn(nsc, 1, generator=g, device=dev) * 1.5 - 7)
+        src = (torch.randn(nsc, 256, generator=g, device=dev) * scale).reshape(-1).to(torch.bfloat16)
+        stats = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
+        mean32 = torch.empty(nsc, dtype=torch.float32, device=dev)
+        iters = 10 if n > (1 << 27) else 30
+        rows = []
+        rows.append(("superchunk_stats", _time_us(lambda: capi.superchunk_stats(src, stats, mean32, n, 8), 3, iters), 2.0 * n))
+        u, _, _ = bitrate.dynamic_bitrate_binary_search_u([stats[:, 1]], 4.375)
+        order = torch.empty(3 * nsc, dtype=torch.int32, device=dev)
+        work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
+        rows.append(("group_plan_stats", _time_us(lambda: capi.group_plan_stats(stats, u, None, order, work), 3, iters), 4.0 * nsc + 4.0 * nsc))
+        counts = work[:3].clone()
+        n8, n4, n2 = (int(c) for c in counts.tolist())
+        sb = 274 * n8 + 146 * n4 + 82 * n2
+        mixed = torch.zeros(capi.mixed_required_bytes(nsc), dtype=torch.uint8, device=dev)
+        mixed2 = torch.zeros_like(mixed)
+        out = torch.empty_like(src)
+        rows.append(("mixed_compress (centred load)", _time_us(
+            lambda: capi.mixed_compress(src, order, counts, mixed, nsc, 2, seed=1, step=0, center_mean=mean32, center_world=8, n=n),
+            3, iters), 2.0 * n + sb))
+        rows.append(("mixed_compress (fused ring step)", _time_us(
+            lambda: capi.mixed_compress(src, order, counts, mixed2, nsc, 2, seed=1, step=1, recv=mixed, center_mean=mean32,
+                                        center_world=8, n=n), 3, iters), 2.0 * n + 2.0 * sb))
+        rows.append(("mixed_decompress (+mean)", _time_us(
+            lambda: capi.mixed_decompress(mixed, out, order, counts, nsc, 2, stats=stats, n_limit=n), 3, iters), 2.0 * n + sb))
+        packed = torch.zeros(capi.required_bytes(n, 4, 16, 2), dtype=torch.uint8, device=dev)
+        rows.append(("scaling_compress_philox (4-bit)", _time_us(
+            lambda: capi.scaling_compress_philox(src, packed, n, 4, 16, 2, 1, 0), 3, iters), 2.0 * n + packed.numel()))
+        rows.append(("scaling_decompress (4-bit)", _time_us(
+            lambda: capi.scaling_decompress(packed, out, n, 4, 16, 2), 3, iters), 2.0 * n + packed.numel()))
+        for name, t, nbytes in rows:
+            _emit(long_bucket=True, kernel=name, elements=n, groups=[n8, n4, n2], us=round(t, 1),
+                  GBps_algorithmic=round(nbytes / t / 1e3, 1), frac_hbm=round(nbytes / t / 1e3 / HBM_PEAK, 4))
+        del src, stats, mean32, order, work, mixed, mixed2, out, packed
+
+
 def mfma_experiment(dev, n=1 << 28, block=8192):
     """the transform fused with the quantiser (4-bit AEE, packed signs, in-kernel rounding stream), its first four stages
     as add / subtract butterflies (the library's kernel) and as a product with the +-1 matrix on the matrix cores"""
@@ -889,6 +933,8 @@ def main():
     ap.add_argument("--quantiser-sizes", action="store_true",
                     help="compress / decompress / fused step of the production quantiser (bf16, 4-bit, AEE and MEE) at 25 MB, at "
                          "the ring-chunk size of the 8-rank configuration and at 2^28 elements")
+    ap.add_argument("--long-bucket", action="store_true",
+                    help="the kernels of the dynamic-bitrate pipeline at 2^26 and 2^28 bf16 elements in one bucket")
     ap.add_argument("--mfma-experiment", action="store_true",
                     help="the transform fused with the quantiser (blocks of 8192) with its first four stages as butterflies and on the matrix cores")
     ap.add_argument("--reference-benchmark", action="store_true",
@@ -905,6 +951,9 @@ def main():
         return
     if args.quantiser_sizes:
         quantiser_sizes(dev)
+        return
+    if args.long_bucket:
+        long_bucket(dev)
         return
     if args.mfma_experiment:
         mfma_experiment(dev, **({"n": args.n} if args.n else {}))
