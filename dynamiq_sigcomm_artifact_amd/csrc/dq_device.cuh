@@ -289,7 +289,11 @@ struct WorldDiv {
     float inv;
     double inv_d;
     int pow2;
+    int fuse16; // world = 2^k with k <= 16
     __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
+    // With fuse16 set, (*this)(v) - mean for a v that came from a 16-bit element is fma(v, inv, -mean): the product with
+    // 2^-k is then exact in binary32 (eight or eleven significant bits, no exponent below the binary32 range for world
+    // sizes up to 2^16), so the fused operation rounds the same number once.
 };
 
 // THC's uniform stochastic quantiser (testbed_evaluation/new_comm_hooks/thc_hooks.py:161-166):

@@ -101,8 +101,17 @@ __device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int6
 {
     float t[16];
     if (whole) {
+        // one branch for the wave on the kind of world size, not one select per element between the two quotients
+        if (DT != DQ_F32 && ctr.wd.fuse16) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) t[i] = ctr.wd(v.get(i)) - mean;
+            for (int i = 0; i < 16; i++) t[i] = __builtin_fmaf(v.get(i), ctr.wd.inv, -mean); // exact: see WorldDiv
+        } else if (ctr.wd.pow2) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = v.get(i) * ctr.wd.inv - mean;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = (float)((double)v.get(i) * ctr.wd.inv_d) - mean;
+        }
     } else {
         // the ragged end of the vector: nothing at or beyond n_valid is read
 #pragma unroll

@@ -67,14 +67,20 @@ __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__rest
     if (row < rows_here) {
 #pragma unroll
         for (int k = 0; k < 16; k++) {
-            float x;
             if (DT == DQ_F32)
-                x = *reinterpret_cast<const float *>(mine + 16 * k * ESZ);
+                v[k] = *reinterpret_cast<const float *>(mine + 16 * k * ESZ);
             else if (DT == DQ_BF16)
-                x = bf16_bits_to_f32(*reinterpret_cast<const uint16_t *>(mine + 16 * k * ESZ));
+                v[k] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t *>(mine + 16 * k * ESZ));
             else
-                x = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(mine + 16 * k * ESZ));
-            v[k] = wd(x);
+                v[k] = f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(mine + 16 * k * ESZ));
+        }
+        // one branch for the wave on the kind of world size, not one select per element between the two quotients
+        if (wd.pow2) {
+#pragma unroll
+            for (int k = 0; k < 16; k++) v[k] = v[k] * wd.inv;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++) v[k] = (float)((double)v[k] * wd.inv_d);
         }
     } else {
 #pragma unroll
@@ -235,6 +241,7 @@ static hipError_t run_mean_center(const void *src, void *residual, void *stats, 
         wd.inv = 1.0f / (float)world_size;
         wd.inv_d = 1.0 / (double)world_size;
         wd.pow2 = (world_size & (world_size - 1)) == 0;
+        wd.fuse16 = wd.pow2 && world_size <= 65536;
         hipLaunchKernelGGL(mean_center_tile_kernel<DT>, dim3((unsigned)((done + 3) / 4)), dim3(64), 0, stream, src, residual,
                            static_cast<uint32_t *>(stats), mean_out, done, wd);
         hipError_t e = hipGetLastError();

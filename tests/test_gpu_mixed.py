@@ -168,6 +168,11 @@ def test_stats_and_centre_on_load(capi, oracle, dt, odt, world, n):
     nsc = (n + 255) // 256
     g = torch.Generator().manual_seed(n + world)
     base = torch.randn(n, generator=g) * 1e-2 + 3e-3
+    if n >= 1024:
+        # superchunks at the bottom of the exponent range: element / world is a denormal binary32 number there, and
+        # the centred value must still be the one of the two-step arithmetic
+        base[256:512] = torch.randn(256, generator=g) * 1e-39
+        base[512:768] = torch.randn(256, generator=g) * 3e-38
     src = torch.full((n + 64,), float("nan"), dtype=dt, device=DEV)     # a NaN beyond n must never be picked up
     src[:n] = base.to(dt)
     stats = torch.zeros(nsc, 2, dtype=torch.bfloat16, device=DEV)
