@@ -127,11 +127,13 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
         if (estimated) estimate_codes<NBITS, MEE>(v, r, d, mp, w);
     }
     const double yd = fast && !estimated ? recip_f64(d) : 0.0;
-    if (!estimated) {
+    // the element-wise chain, compiled once per kind of division: with the choice made per element the compiler
+    // computes both quotients and selects
+    auto chain = [&](auto by_reciprocal) {
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const float e = v.get(i);
-        float x = fast ? div_by(e, yd) : e / d;
+        float x = decltype(by_reciprocal)::value ? div_by(e, yd) : e / d;
         int sv;
         if (DT == DQ_F16) {
             x = rh(x);
@@ -161,6 +163,12 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
         }
         words_put<NBITS>(w, i, (uint32_t)clamp_code(sv, R));
     }
+    };
+    if (!estimated) {
+        if (fast)
+            chain(std::true_type{});
+        else
+            chain(std::false_type{});
     }
 
     uint8_t *gout = dst + G::stream_offset(c0);
