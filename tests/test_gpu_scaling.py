@@ -208,6 +208,39 @@ def test_zero_elements_with_random_values_0_and_1(capi, oracle, dt, strategy, C)
         _dec_comp(capi, oracle, dt, n, nbits, C, strategy, src, inp.to(tdt), rnd, rnd.flip(0).contiguous(), tag)
 
 
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+@pytest.mark.parametrize("C", [16, 8, 32])
+def test_estimate_route_at_the_ends_of_its_range(capi, oracle, dt, strategy, C):
+    """Inputs that keep every wave on the estimate route (finite, ordinary scales, random values in [0, 1]) and sit at the
+    ends of what it handles: magnitudes from 2^-95 to 2^95, chunks whose elements all equal plus or minus the chunk maximum
+    (their coordinate is +-R, or just beyond when the stored scale rounds down: the clamp on either side), and random
+    values 0, 1 and next to them."""
+    tdt = TORCH_DT[dt]
+    nsc = 24
+    n = nsc * 16 * C
+    g = torch.Generator().manual_seed(400 + strategy + C)
+    mags = torch.tensor([2.0 ** -95, 2.0 ** -60, 2.0 ** -20, 1.0, 2.0 ** 20, 2.0 ** 60, 2.0 ** 95, 3.0e-2])
+    src = torch.randn(nsc, 16, C, generator=g)
+    # every third chunk: all elements at +- the same magnitude; the others: one maximum, the rest random below it
+    sign = torch.where(torch.rand(nsc, 16, C, generator=g) < 0.5, -1.0, 1.0)
+    flat = (torch.arange(16).view(1, 16, 1) % 3 == 0)
+    src = torch.where(flat, sign * (1.0 + torch.rand(nsc, 16, 1, generator=g)), src.clamp(-3.0, 3.0) / 3.0)
+    src[:, :, 0] = torch.where(flat[:, :, 0].expand(nsc, 16), src[:, :, 0], sign[:, :, 0] * 1.0)
+    src = (src * mags[torch.arange(nsc) % mags.numel()].view(nsc, 1, 1)).reshape(-1)
+    edge = torch.tensor([0.0, 1.0, 2.0 ** -8, 1.0 - 2.0 ** -8, 2.0 ** -20, 0.5, 0.99609375, 0.00390625])
+    rnd = torch.rand(n, generator=g)
+    pick = torch.rand(n, generator=g) < 0.5
+    rnd = torch.where(pick, edge[torch.randint(0, edge.numel(), (n,), generator=g)], rnd)
+    src, rnd = src.to(tdt), rnd.to(tdt)
+    for nbits in (2, 4, 5, 8):
+        if (C * nbits) % 8:
+            continue
+        tag = "edges dt=%d C=%d b=%d s=%d" % (dt, C, nbits, strategy)
+        _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src, rnd, tag)
+        _dec_comp(capi, oracle, dt, n, nbits, C, strategy, src, (src.float() * -0.5).to(tdt), rnd, rnd.flip(0).contiguous(), tag)
+
+
 @pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [2, 3])
 @pytest.mark.parametrize("C", [16, 8, 32])
