@@ -77,6 +77,27 @@ struct WidthsFromStats {
 __device__ __forceinline__ uint64_t one_of(int cls) { return cls < 3 ? (uint64_t)1 << (21 * cls) : 0; }
 __device__ __forceinline__ int field(uint64_t p, int cls) { return (int)((p >> (21 * cls)) & 0x1fffff); }
 
+// Inclusive scan over the wave's 64 lanes with data-parallel-primitive moves (shifts by 1, 2, 4, 8 inside the rows of
+// sixteen lanes, then lane 15 of a row into the next row, lane 31 into the upper half): a dozen register-to-register
+// instructions where six rounds of cross-lane permutes through the LDS pipeline took about half a microsecond.  The
+// operand packs small counters into one word; no field may overflow into the next one.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint32_t dpp_from(uint32_t x)
+{
+    // lanes without a source, and rows outside ROW_MASK, receive 0
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, ROW_MASK, 0xf, false);
+}
+
+__device__ __forceinline__ uint32_t wave_scan_inclusive(uint32_t x)
+{
+    x += dpp_from<0x111, 0xf>(x); // row_shr:1
+    x += dpp_from<0x112, 0xf>(x); // row_shr:2
+    x += dpp_from<0x114, 0xf>(x); // row_shr:4
+    x += dpp_from<0x118, 0xf>(x); // row_shr:8
+    x += dpp_from<0x142, 0xa>(x); // row_bcast:15 into rows 1 and 3
+    x += dpp_from<0x143, 0xc>(x); // row_bcast:31 into rows 2 and 3
+    return x;
+}
+
 // ---- one launch (up to 64 tiles) ----------------------------------------------------------------------
 
 constexpr int kOneThreads = kTile; // one superchunk per thread while placing
@@ -132,21 +153,22 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
         widths.prepare(thr, wave, lane);
         __syncthreads();
     }
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) mine += __shfl_xor(mine, d, 64);
+    // the wave's total of the recount: a thread has counted at most 63 superchunks, a wave at most 4032 per class, so
+    // two classes share a word (lane 63 of the scan holds the total)
+    const uint32_t mine01 = wave_scan_inclusive((uint32_t)field(mine, 0) | ((uint32_t)field(mine, 1) << 16));
+    const uint32_t mine2 = wave_scan_inclusive((uint32_t)field(mine, 2));
 
-    // this tile: class of the thread's superchunk, inclusive scan over the wave
+    // this tile: class of the thread's superchunk, inclusive scan over the wave (at most 64 per class: a byte each)
     const int c = own < nsc ? widths.cls(own_raw, thr) : 3;
     if (qbits_out && own < nsc) qbits_out[own] = c == 0 ? 8 : (c == 1 ? 4 : (c == 2 ? 2 : (int64_t)widths(own)));
     const uint64_t cnt = one_of(c);
-    uint64_t incl = cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint64_t up = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += up;
+    const uint32_t scanned = wave_scan_inclusive(c < 3 ? 1u << (8 * c) : 0u);
+    const uint64_t incl = (uint64_t)(scanned & 0xffu) | ((uint64_t)((scanned >> 8) & 0xffu) << 21) |
+                          ((uint64_t)((scanned >> 16) & 0xffu) << 42);
+    if (lane == 63) {
+        before_sum[wave] = (uint64_t)(mine01 & 0xffffu) | ((uint64_t)(mine01 >> 16) << 21) | ((uint64_t)mine2 << 42);
+        scan_sum[wave] = incl;
     }
-    if (lane == 0) before_sum[wave] = mine;
-    if (lane == 63) scan_sum[wave] = incl;
     __syncthreads();
     uint64_t before = 0, excl = incl - cnt, tile_all = 0;
 #pragma unroll
