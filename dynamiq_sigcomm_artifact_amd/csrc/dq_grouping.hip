@@ -30,6 +30,7 @@ namespace {
 constexpr int kTile = 1024; // superchunks per workgroup
 constexpr int kThreads = 256;
 constexpr int kPer = kTile / kThreads;
+static_assert(64 * kPer < 1024, "the wave scan of the placing kernel packs three counters of ten bits");
 
 __device__ __forceinline__ int width_class(int64_t q) { return q == 8 ? 0 : q == 4 ? 1 : q == 2 ? 2 : 3; }
 
@@ -257,12 +258,11 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
     }
     // inclusive scan over the wave, then over the waves of the workgroup
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint64_t incl = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint64_t up = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += up;
-    }
+    // (a thread holds at most kPer = 4 superchunks, a wave at most 256 per class: ten bits each)
+    const uint32_t scanned = wave_scan_inclusive((uint32_t)field(mine, 0) | ((uint32_t)field(mine, 1) << 10) |
+                                                 ((uint32_t)field(mine, 2) << 20));
+    const uint64_t incl = (uint64_t)(scanned & 0x3ffu) | ((uint64_t)((scanned >> 10) & 0x3ffu) << 21) |
+                          ((uint64_t)((scanned >> 20) & 0x3ffu) << 42);
     if (lane == 63) wave_sum[wave] = incl;
     __syncthreads();
     uint64_t excl = incl - mine;
@@ -379,12 +379,7 @@ template <bool WIDE> __device__ __forceinline__ void scan_counters(uint32_t *his
 #pragma unroll
         for (int h = 0; h < 4; h++) sum += WIDE ? (w[h] & 0xffffu) + (w[h] >> 16) : w[h];
     }
-    uint32_t incl = sum;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t up = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += up;
-    }
+    const uint32_t incl = wave_scan_inclusive(sum);
     if (lane == 63) wave_sum[wave] = incl;
     __syncthreads();
     uint32_t run = incl - sum;
