@@ -42,11 +42,17 @@ struct WidthsFromArray {
     const int64_t *qbits;
     typedef int64_t Raw;
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
+    __device__ __forceinline__ int64_t width(int64_t i) const { return qbits[i]; }
     bool word_aligned() const { return true; }
     __device__ __forceinline__ const uint16_t *norm_stats() const { return nullptr; }
     const void *norm_stats_host() const { return nullptr; }
     __device__ __forceinline__ void resolve() {}
     __device__ __forceinline__ void prepare(int *, int, int) const {}
+    __device__ __forceinline__ bool known(int (&t)[2]) const // nothing to search for
+    {
+        t[0] = t[1] = 0;
+        return true;
+    }
     __device__ __forceinline__ Raw load(int i) const { return qbits[i]; }
     __device__ __forceinline__ int cls(Raw q, const int *) const { return width_class(q); }
 };
@@ -55,6 +61,7 @@ struct WidthsFromStats {
     const uint16_t *stats;
     float u;
     const double *u_dev;  // when set, the offset is read from device memory (the search for u leaves it there)
+    int thr_host[2];      // the two thresholds of prepare(), found on the host when u is a number (else -1)
     typedef uint32_t Raw; // a (mean, norm) pair: the norm pattern is the high half
     __device__ __forceinline__ const uint16_t *norm_stats() const { return stats; }
     const void *norm_stats_host() const { return stats; }
@@ -63,7 +70,20 @@ struct WidthsFromStats {
         if (u_dev) u = (float)*u_dev;
     }
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits_of_norm(stats[2 * i + 1], u); }
+    // the same by two compares when the host has found the thresholds
+    __device__ __forceinline__ int64_t width(int64_t i) const
+    {
+        const uint32_t r = stats[2 * i + 1];
+        if (thr_host[0] < 0 || r > (uint32_t)kMaxPattern) return qbits_of_norm(r, u);
+        return (int)r >= thr_host[1] ? 8 : ((int)r >= thr_host[0] ? 4 : 2);
+    }
     __device__ __forceinline__ void prepare(int *thr, int wave, int lane) const { width_thresholds(u, thr, wave, lane); }
+    __device__ __forceinline__ bool known(int (&t)[2]) const
+    {
+        t[0] = thr_host[0];
+        t[1] = thr_host[1];
+        return thr_host[0] >= 0;
+    }
     bool word_aligned() const { return (reinterpret_cast<uintptr_t>(stats) & 3) == 0; } // load() reads pairs as one word
     __device__ __forceinline__ Raw load(int i) const { return reinterpret_cast<const uint32_t *>(stats)[i]; }
     __device__ __forceinline__ int cls(Raw pair, const int *thr) const
@@ -131,7 +151,8 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
     typename W::Raw own_raw = typename W::Raw();
     if (own < nsc) own_raw = widths.load(own);
     uint64_t mine = 0;
-    bool ready = false;
+    int t2[2]; // the thresholds: from the kernel arguments, or searched by two waves and handed over through LDS
+    bool ready = widths.known(t2);
     for (int i0 = 0; i0 < nbefore; i0 += kOneBatch * kOneThreads) {
         typename W::Raw raw[kOneBatch];
 #pragma unroll
@@ -142,17 +163,21 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
         if (!ready) {
             widths.prepare(thr, wave, lane);
             __syncthreads();
+            t2[0] = thr[0];
+            t2[1] = thr[1];
             ready = true;
         }
 #pragma unroll
         for (int j = 0; j < kOneBatch; j++) {
             const int i = i0 + j * kOneThreads + (int)threadIdx.x;
-            if (i < nbefore) mine += one_of(widths.cls(raw[j], thr));
+            if (i < nbefore) mine += one_of(widths.cls(raw[j], t2));
         }
     }
     if (!ready) {
         widths.prepare(thr, wave, lane);
         __syncthreads();
+        t2[0] = thr[0];
+        t2[1] = thr[1];
     }
     // the wave's total of the recount: a thread has counted at most 63 superchunks, a wave at most 4032 per class, so
     // two classes share a word (lane 63 of the scan holds the total)
@@ -160,7 +185,7 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
     const uint32_t mine2 = wave_scan_inclusive((uint32_t)field(mine, 2));
 
     // this tile: class of the thread's superchunk, inclusive scan over the wave (at most 64 per class: a byte each)
-    const int c = own < nsc ? widths.cls(own_raw, thr) : 3;
+    const int c = own < nsc ? widths.cls(own_raw, t2) : 3;
     if (qbits_out && own < nsc) qbits_out[own] = c == 0 ? 8 : (c == 1 ? 4 : (c == 2 ? 2 : (int64_t)widths(own)));
     const uint64_t cnt = one_of(c);
     const uint32_t scanned = wave_scan_inclusive(c < 3 ? 1u << (8 * c) : 0u);
@@ -201,7 +226,7 @@ __global__ __launch_bounds__(kThreads) void plan_count_kernel(W widths, int64_t 
     int c[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int k = 0; k < kPer; k++) {
-        if (base + k < nsc) c[width_class(widths(base + k))]++;
+        if (base + k < nsc) c[width_class(widths.width(base + k))]++;
     }
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -250,7 +275,7 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
     for (int k = 0; k < kPer; k++) {
         cls[k] = 3;
         if (base + k < nsc) {
-            const int64_t q = widths(base + k);
+            const int64_t q = widths.width(base + k);
             if (qbits_out) qbits_out[base + k] = q;
             cls[k] = width_class(q);
         }
@@ -556,11 +581,99 @@ hipError_t launch_group_plan(const int64_t *qbits, int64_t nsc, int32_t *order, 
     return run_plan(WidthsFromArray{qbits}, nullptr, nsc, order, work, nullptr, stream);
 }
 
+// ---- the thresholds of the width rule on the host ------------------------------------------------------
+//
+// The rule (dq_bitwidth.cuh: qbits_of_norm) is binary32 arithmetic with every result rounded to bf16 and the
+// library's polynomial log2: the same operations in the same order give the same bits on the host, so when u comes
+// as a number the two patterns at which the width becomes 4 and 8 are found here and travel with the kernel
+// arguments, and the plan kernel neither searches nor waits for the two waves that would.
+
+static inline uint32_t host_bits(float f) { uint32_t u; __builtin_memcpy(&u, &f, 4); return u; }
+static inline float host_float(uint32_t u) { float f; __builtin_memcpy(&f, &u, 4); return f; }
+
+static inline float host_round_bf16(float x) // round to nearest even, as v_cvt_pk_bf16_f32
+{
+    uint32_t b = host_bits(x);
+    if ((b & 0x7fffffffu) > 0x7f800000u) return host_float((b | 0x00400000u) & 0xffff0000u); // NaN stays NaN
+    b += 0x7fffu + ((b >> 16) & 1u);
+    return host_float(b & 0xffff0000u);
+}
+
+static float host_log2_det(float x) // log2_det of dq_device.cuh, operation by operation
+{
+    uint32_t ix = host_bits(x);
+    int k = 0;
+    if (ix >= 0x7f800000u) {
+        if (ix == 0x7f800000u) return x;
+        if ((ix & 0x7fffffffu) > 0x7f800000u) return x + x;
+        if ((ix << 1) == 0) return -__builtin_inff();
+        return host_float(0x7fc00000u);
+    }
+    if (ix < 0x00800000u) {
+        if (ix == 0) return -__builtin_inff();
+        x *= 8388608.0f;
+        ix = host_bits(x);
+        k = -23;
+    }
+    const uint32_t t = ix - 0x3f3504f3u;
+    k += (int)t >> 23;
+    const float z = host_float(ix - (t & 0xff800000u));
+    const float f = z - 1.0f;
+    float q = -0x1.d0dd08p-4f;
+    q = __builtin_fmaf(q, f, 0x1.7ad622p-3f);
+    q = __builtin_fmaf(q, f, -0x1.831b24p-3f);
+    q = __builtin_fmaf(q, f, 0x1.a33bdap-3f);
+    q = __builtin_fmaf(q, f, -0x1.eb492p-3f);
+    q = __builtin_fmaf(q, f, 0x1.277e38p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715762p-2f);
+    q = __builtin_fmaf(q, f, 0x1.ec7092p-2f);
+    q = __builtin_fmaf(q, f, -0x1.715476p-1f);
+    const float p = (f * f) * q;
+    float r = __builtin_fmaf(f, 0x1.4ae0cp-26f, p);
+    r = __builtin_fmaf(f, 0x1.715476p+0f, r);
+    return (float)k + r;
+}
+
+static int host_qbits_of_norm(uint32_t norm_bits, float u) // qbits_of_norm of dq_bitwidth.cuh
+{
+    const float eps = 1e-20f;
+    float x = host_float(norm_bits << 16);
+    x = (x != x) ? x : host_round_bf16(x > eps ? x : eps);
+    x = host_round_bf16(host_log2_det(x));
+    x = host_round_bf16(x * (float)(4.0 / (512.0 / 17.0)));
+    x = host_round_bf16(x + u);
+    x = (x != x) ? x : host_round_bf16(x > eps ? x : eps);
+    x = host_round_bf16(host_log2_det(x));
+    x = __builtin_floorf(x);
+    const int z = (x != x) ? 1 : (x < 1.0f ? 1 : (x > 3.0f ? 3 : (int)x));
+    return 1 << z;
+}
+
+// the smallest pattern in [0, kMaxPattern] whose width is >= target, kMaxPattern + 1 if none (the width is a
+// monotone step function of the pattern: width_thresholds() on the device relies on the same)
+static int host_width_threshold(float u, int target)
+{
+    int lo = 0, hi = kMaxPattern + 1; // the answer lies in [lo, hi]
+    while (lo < hi) {
+        const int mid = (lo + hi) / 2;
+        if (host_qbits_of_norm((uint32_t)mid, u) >= target)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    return lo;
+}
+
 // u_dev != nullptr: the offset is *u_dev at the time the kernels run, u is ignored
 hipError_t launch_group_plan_stats(const void *stats, float u, const double *u_dev, int64_t nsc, int64_t *qbits_out,
                                    int32_t *order, int32_t *work, uint32_t *hist, hipStream_t stream)
 {
-    return run_plan(WidthsFromStats{static_cast<const uint16_t *>(stats), u, u_dev}, qbits_out, nsc, order, work, hist, stream);
+    WidthsFromStats widths{static_cast<const uint16_t *>(stats), u, u_dev, {-1, -1}};
+    if (!u_dev && u == u) { // (a NaN offset: every width is 2, and the device search says so itself)
+        widths.thr_host[0] = host_width_threshold(u, 4);
+        widths.thr_host[1] = host_width_threshold(u, 8);
+    }
+    return run_plan(widths, qbits_out, nsc, order, work, hist, stream);
 }
 
 } // namespace dq
