@@ -33,7 +33,25 @@ struct MixedPlan {
     const int32_t *counts; // n8, n4, n2
     int chunk, world;
     int nsc;               // the counts are clamped so that their sum cannot exceed it
+    uint64_t inv40;        // ceil(2^40 / world) when world <= 2^16 and nsc + world < 2^24 (see divide_by_world), else 0
 };
+
+// world > 1.  With inv40 set, x / world for 0 <= x < 2^24 is (x * inv40) >> 40: inv40 = (2^40 + e) / world with
+// 0 <= e < world <= 2^16, so the product exceeds x / world * 2^40 by x e < 2^40, less than the 2^40 / world that
+// separate x / world from the next integer; and it stays below 2^64.  One scalar multiply instead of the expansion
+// of an integer division, which stands in front of the kernel's first load.
+__device__ __forceinline__ int divide_by_world(int x, const MixedPlan &p, bool magic)
+{
+    return magic ? (int)(((uint64_t)(uint32_t)x * p.inv40) >> 40) : x / p.world;
+}
+
+static MixedPlan make_plan(const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world, int64_t nsc)
+{
+    MixedPlan p{order, counts, ring_chunk, ring_world, (int)nsc, 0};
+    if (ring_world > 1 && ring_world <= 65536 && nsc + ring_world < (1 << 24))
+        p.inv40 = ((uint64_t)1 << 40) / (uint64_t)ring_world + (((uint64_t)1 << 40) % (uint64_t)ring_world ? 1 : 0);
+    return p;
+}
 
 struct Segment {
     int cls;          // 0: 8-bit, 1: 4-bit, 2: 2-bit, 3: nothing to do
@@ -44,9 +62,12 @@ struct Segment {
     int64_t byte_off; // where the run starts in the packed stream
 };
 
-// block -> the run (bit-width group of the ring chunk) it works in and its first tile there; a block takes `span` tiles
-__device__ __forceinline__ Segment locate(const MixedPlan &p, int block, int span)
+// block -> the run (bit-width group of the ring chunk) it works in and its first tile there; a block takes `span` tiles.
+// MODE 0: a ring of one rank (the whole bucket is the chunk: nothing to divide); 1: division by the world size as a
+// multiplication (divide_by_world); 2: as a division.
+template <int MODE> __device__ __forceinline__ Segment locate_in(const MixedPlan &p, int block, int span)
 {
+    constexpr bool SINGLE = MODE == 0;
     constexpr int kRec[3] = {Rec<8>::REC, Rec<4>::REC, Rec<2>::REC};
     Segment s;
     s.cls = 3; s.tile = 0; s.cnt = 0; s.row0 = 0; s.pos0 = 0; s.byte_off = 0;
@@ -57,8 +78,8 @@ __device__ __forceinline__ Segment locate(const MixedPlan &p, int block, int spa
 #pragma unroll
     for (int g = 0; g < 3; g++) {
         const int n = min(max(counts[g], 0), p.nsc - (int)pos); // a corrupt count cannot lead outside a region or the pool
-        const int per = (n + p.world - 1) / p.world;
-        const int begin = (int)min((int64_t)per * p.chunk, (int64_t)n);
+        const int per = SINGLE ? n : divide_by_world(n + p.world - 1, p, MODE == 1);
+        const int begin = SINGLE ? 0 : (int)min((int64_t)per * p.chunk, (int64_t)n);
         const int cnt = min(per, n - begin);
         const int tiles = ((cnt + kRowsPerWave - 1) / kRowsPerWave + span - 1) / span; // blocks of this run
         if (s.cls == 3 && t < tiles) {
@@ -69,6 +90,13 @@ __device__ __forceinline__ Segment locate(const MixedPlan &p, int block, int spa
         off += (int64_t)cnt * kRec[g];
     }
     return s;
+}
+
+__device__ __forceinline__ Segment locate(const MixedPlan &p, int block, int span)
+{
+    if (p.world == 1) return locate_in<0>(p, block, span);
+    if (p.inv40 != 0) return locate_in<1>(p, block, span);
+    return locate_in<2>(p, block, span);
 }
 
 template <int DT, int RDT, bool MEE, bool FUSED>
@@ -191,7 +219,7 @@ hipError_t launch_mixed_compress(const void *src, const float *center_mean, int 
                                  const uint8_t *recv, uint8_t *dst, const void *rnd, const RandKey *philox, int64_t nsc,
                                  int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
 {
-    const MixedPlan plan{order, counts, ring_chunk, ring_world, (int)nsc};
+    const MixedPlan plan = make_plan(order, counts, ring_chunk, ring_world, nsc);
     Center ctr;
     ctr.mean = center_mean;
     ctr.n_valid = n_valid;
@@ -219,7 +247,7 @@ hipError_t launch_mixed_decompress(const uint8_t *src, void *dst, const int32_t 
                                    int ring_chunk, int ring_world, const void *stats, int64_t limit, int64_t nsc,
                                    int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
 {
-    const MixedPlan plan{order, counts, ring_chunk, ring_world, (int)nsc};
+    const MixedPlan plan = make_plan(order, counts, ring_chunk, ring_world, nsc);
     const uint16_t *st = static_cast<const uint16_t *>(stats);
     if ((dtype & 0xf) == DQ_BF16)
         return mee ? run_decompress<DQ_BF16, true>(src, dst, plan, nsc, st, limit, mp, stream)

@@ -43,7 +43,8 @@ def segments(counts, chunk, world, nsc):
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("strategy", [2, 3])
 @pytest.mark.parametrize("nsc,world,weights", [(1037, 1, (1, 1, 1)), (1037, 3, (1, 2, 3)), (2, 1, (1, 1, 1)),
-                                               (515, 4, (1, 0, 1)), (64, 8, (0, 1, 0)), (6403, 8, (1, 6, 2))])
+                                               (515, 4, (1, 0, 1)), (64, 8, (0, 1, 0)), (6403, 8, (1, 6, 2)),
+                                               (2051, 7, (1, 3, 1)), (4099, 13, (2, 5, 1))])
 def test_mixed_matches_per_group_calls(capi, dt, strategy, nsc, world, weights):
     n_valid = nsc * 256 - 77
     q, order, work = make_plan(capi, nsc, nsc + world, weights)

@@ -163,3 +163,20 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode == 2 and "--gpus must be 1" in r.stderr and r.stdout.strip() == ""
+
+
+def test_division_by_the_world_size_as_a_multiplication():
+    """The mixed kernels split a group of n superchunks over the ring as ceil(n / world) per rank and compute the
+    quotient as (x * ceil(2^40 / world)) >> 40 for x < 2^24 and world <= 2^16 (dq_scaling_mixed.hip: divide_by_world).
+    Brute force over every world size and the operands where such a reciprocal goes wrong first: multiples of the
+    divisor minus one, the largest operands, and a random sample."""
+    import numpy as np
+    rng = np.random.default_rng(5)
+    top = (1 << 24) - 1
+    for d in range(2, 65537):
+        m = ((1 << 40) + d - 1) // d
+        k = np.concatenate([np.arange(1, 6, dtype=np.uint64), np.uint64(top // d) - np.arange(0, 4, dtype=np.uint64)])
+        x = np.concatenate([k * np.uint64(d) - np.uint64(1), k * np.uint64(d), np.array([top, top - 1, 0, 1], np.uint64),
+                            rng.integers(0, top + 1, 24, dtype=np.uint64)])
+        x = x[x <= top]
+        assert ((x * np.uint64(m)) >> np.uint64(40) == x // np.uint64(d)).all(), d
