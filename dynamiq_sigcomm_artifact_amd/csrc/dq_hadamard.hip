@@ -94,8 +94,9 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
     if (a.sbits == a.cbits) {
         origin = (int64_t)blockIdx.x << a.kt;
     } else {
-        const int64_t mids = (int64_t)1 << (a.sbits - a.cbits);
-        const int64_t hi = blockIdx.x / mids, mid = blockIdx.x % mids;
+        // (shift and mask, not quotient and remainder: see rht_strided_kernel)
+        const int mbits = a.sbits - a.cbits;
+        const int64_t hi = (int64_t)(blockIdx.x >> mbits), mid = (int64_t)(blockIdx.x & ((1u << mbits) - 1u));
         origin = (hi << (a.sbits + rbits)) + (mid << a.cbits);
     }
 

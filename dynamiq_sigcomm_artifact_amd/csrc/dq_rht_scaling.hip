@@ -430,8 +430,9 @@ __global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbi
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, nthreads = blockDim.x;
     const int tile = 1 << (rbits + 5);
-    const int64_t mids = (int64_t)1 << (sbits - 5);
-    const int64_t hi = blockIdx.x / mids, mid = blockIdx.x % mids;
+    // (shift and mask: written as a quotient and remainder by the power of two, the compiler expands a 64-bit
+    // division in front of the kernel's first loads)
+    const int64_t hi = (int64_t)(blockIdx.x >> (sbits - 5)), mid = (int64_t)(blockIdx.x & ((1u << (sbits - 5)) - 1u));
     const int64_t origin = (hi << (sbits + rbits)) + (mid << 5);
     const int col = tid & 31;
     const int groups = tile >> 9; // groups of sixteen rows
