@@ -110,12 +110,14 @@ def build_extension(verbose=True):
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared",
            "-DTORCH_EXTENSION_NAME=eden_utils", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           # c10's HIP stream / caching-allocator headers pull in the HIP runtime API (declarations only)
+           "-D__HIP_PLATFORM_AMD__=1", "-I" + os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "include"),
            "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
     cmd += ["-I" + p for p in ce.include_paths()]
     cmd += ["-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(PKG_DIR, "..", "include")]
     cmd += [os.path.join(CSRC, "eden_utils_module.cpp"), "-o", out]
     cmd += ["-L" + PKG_DIR, "-l:" + LIB_NAME, "-Wl,-rpath,$ORIGIN",
-            "-L" + torch_lib, "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_python",
+            "-L" + torch_lib, "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_python",
             "-Wl,-rpath," + torch_lib]
     dt = _run(cmd, "g++ eden_utils_module.cpp")
     if verbose:

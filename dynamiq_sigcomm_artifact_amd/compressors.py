@@ -34,6 +34,7 @@ def record_geometry(nbits, chunk_size, supergroup=_SUPERGROUP):
 
 class _DynamicRangeGPUKern(object):
     strategy = 2
+    given_pool_dtype = None           # dtype a pool passed in params["rand_pool_tensor"] is kept in (None: its own)
 
     def __init__(self, nbits, chunk_size, params, device="cuda", generator=None):
         eu = self.eden_utils = load_eden_utils()
@@ -69,6 +70,10 @@ class _DynamicRangeGPUKern(object):
             pool = torch.rand((rows, chunk_size), device=device, generator=generator).to(torch.bfloat16)   # values in [0, 1]
         else:
             pool = given.to(device=device)[:rows * chunk_size].view(rows, chunk_size)
+            if self.given_pool_dtype is not None:
+                # the MEE class keeps a loaded pool in binary16 (:488), the AEE class in the dtype of the file (:389): a
+                # bf16 caller of the MEE class therefore sees values rounded twice, and so must this one
+                pool = pool.to(dtype=self.given_pool_dtype)
         self.randomized_vec_pool = pool
         self.randomized_vec_pools[pool.dtype] = pool
 
@@ -146,22 +151,29 @@ class _DynamicRangeGPUKern(object):
 
     # ---- the same steps over a list of superchunk indices: index_select + the call above + index_copy_
     #      (comm_hooks.py:1001-1011) without the gathered copy; no counterpart in the reference ----
+    def _rows_supported(self):
+        if self.chunk_size != 16:
+            raise ValueError("the row-list kernels serve superchunks of 16 chunks of 16 elements; chunk_size is %d" % self.chunk_size)
+
     def compression_rows(self, full_tensor, rows, send_chunk):
         """send record k = compressed superchunk rows[k] of full_tensor"""
+        self._rows_supported()
         count = rows.numel()
         if count:
-            self.eden_utils.scaling_compress_rows(full_tensor, rows, send_chunk, self.rand_pool(count * 256, full_tensor.dtype),
+            self.eden_utils.scaling_compress_rows(full_tensor, rows, send_chunk, self.rand_pool(count * self._super_elems, full_tensor.dtype),
                                                   count, self.nbits, self._stream(), self.strategy)
 
     def dec_compression_rows(self, recv_chunk, full_tensor, rows, send_chunk):
+        self._rows_supported()
         count = rows.numel()
         if count:
             self.eden_utils.scaling_dec_comp_rows(recv_chunk, full_tensor, rows, send_chunk,
-                                                  self.rand_pool(count * 256, full_tensor.dtype), count, self.nbits,
+                                                  self.rand_pool(count * self._super_elems, full_tensor.dtype), count, self.nbits,
                                                   self._stream(), self.strategy)
 
     def decompression_rows(self, recv_chunk, full_output, rows, stats=None, n_limit=None):
         """superchunk rows[k] of full_output = decoded record k (+ its mean from stats)"""
+        self._rows_supported()
         count = rows.numel()
         if count:
             self.eden_utils.scaling_decompress_rows(recv_chunk, full_output, rows, stats,
@@ -177,6 +189,7 @@ class Aee_Dynamic_Range_GPU_kern(_DynamicRangeGPUKern):
 class Mee_Dynamic_Range_GPU_kern(_DynamicRangeGPUKern):
     """utils_aggregation.py:470-569 (hierarchical MEE, strategy 3)"""
     strategy = 3
+    given_pool_dtype = torch.float16
 
     def __init__(self, nbits, chunk_size, params, device="cuda", generator=None):
         super().__init__(nbits, chunk_size, params, device=device, generator=generator)

@@ -4,6 +4,7 @@
 #include <math.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 
@@ -63,8 +64,15 @@ int finish(hipError_t e)
 int select_device(int device)
 {
     int cur = -1;
-    if (hipGetDevice(&cur) == hipSuccess && cur == device) return DQ_OK;
-    if (hipSetDevice(device) != hipSuccess) return fail(DQ_ERR_DEVICE);
+    if (!(hipGetDevice(&cur) == hipSuccess && cur == device) && hipSetDevice(device) != hipSuccess) return fail(DQ_ERR_DEVICE);
+    // the first call on a device also resolves the address of the static scratch array of dq_eden_quantize_static,
+    // so that that entry point itself never has to (it may run under stream capture); a failure here is reported by
+    // that entry point, not by the caller at hand
+    static std::atomic<uint64_t> prepared{0};
+    if (device >= 0 && device < 64 && !(prepared.load(std::memory_order_acquire) >> device & 1)) {
+        if (dq::eden_static_prepare(device) != hipSuccess) (void)hipGetLastError();
+        prepared.fetch_or((uint64_t)1 << device, std::memory_order_release);
+    }
     return DQ_OK;
 }
 

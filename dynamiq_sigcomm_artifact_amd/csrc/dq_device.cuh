@@ -283,18 +283,62 @@ __host__ __device__ __forceinline__ void chunk_uniform_words(const RandKey &key,
 }
 
 // v / world, correctly rounded: world = 2^k multiplies by the exact reciprocal; otherwise the product with
-// the double reciprocal is within 2^-51 of the quotient, closer than a quotient of two binary32 numbers
-// can come to a rounding boundary without lying on it
+// the double reciprocal is within 2^-51 of the quotient, closer than a normal quotient of two binary32 numbers
+// can come to a rounding boundary without lying on it.  A subnormal quotient can lie exactly half-way between two
+// subnormal numbers (v = m 2^-150 world, m odd): `ties` says that this can happen for the element type and world size
+// at hand -- binary32 elements with any world size that is not a power of two, 16-bit elements (multiples of 2^-133
+// or 2^-24) only from world = 3 * 2^17 on -- and such quotients then take the division itself.
 struct WorldDiv {
     float inv;
     double inv_d;
     int pow2;
     int fuse16; // world = 2^k with k <= 16
-    __device__ __forceinline__ float operator()(float v) const { return pow2 ? v * inv : (float)((double)v * inv_d); }
+    int ties;
+    float world;
+    __device__ __forceinline__ static bool subnormal(float q) { return (__float_as_uint(q) & 0x7fffffffu) - 1u < 0x007fffffu; }
+    __device__ __forceinline__ float operator()(float v) const
+    {
+        if (pow2) return v * inv;
+        float q = (float)((double)v * inv_d);
+        if (ties && subnormal(q)) q = v / world;
+        return q;
+    }
+    // sixteen quotients at once when world is not a power of two; the divisions sit behind one branch of the wave (written
+    // as a choice per element, both quotients would be computed for every element)
+    __device__ __forceinline__ void divide16(float (&v)[16]) const
+    {
+        float q[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) q[k] = (float)((double)v[k] * inv_d);
+        if (ties) {
+            bool sub = false;
+#pragma unroll
+            for (int k = 0; k < 16; k++) sub |= __builtin_amdgcn_class(q[k], 0x90); // a subnormal number of either sign
+            if (__builtin_amdgcn_ballot_w64(sub) != 0) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) q[k] = subnormal(q[k]) ? v[k] / world : q[k];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 16; k++) v[k] = q[k];
+    }
     // With fuse16 set, (*this)(v) - mean for a v that came from a 16-bit element is fma(v, inv, -mean): the product with
     // 2^-k is then exact in binary32 (eight or eleven significant bits, no exponent below the binary32 range for world
     // sizes up to 2^16), so the fused operation rounds the same number once.
 };
+
+// elem_bytes: 2 or 4
+inline WorldDiv make_world_div(int world, int elem_bytes)
+{
+    WorldDiv wd;
+    wd.inv = 1.0f / (float)world;
+    wd.inv_d = 1.0 / (double)world;
+    wd.pow2 = (world & (world - 1)) == 0;
+    wd.fuse16 = wd.pow2 && world <= 65536;
+    wd.ties = !wd.pow2 && (elem_bytes == 4 || world >= (3 << 17));
+    wd.world = (float)world;
+    return wd;
+}
 
 // THC's uniform stochastic quantiser (testbed_evaluation/new_comm_hooks/thc_hooks.py:161-166):
 // x = clamp((v - lo) / delta, 0, levels - 1); level = floor(x) + (u < x - floor(x))

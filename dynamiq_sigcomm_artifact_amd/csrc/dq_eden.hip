@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
     }
     if (ordinary) {
 #pragma unroll
-        for (int k = 0; k < kEdenPerThread; k++) x[k] = div_by(v[k] * sqrt_n, yn);
+        for (int k = 0; k < kEdenPerThread; k++) x[k] = div_exact(v[k] * sqrt_n, norm, yn);
     } else {
 #pragma unroll
         for (int k = 0; k < kEdenPerThread; k++) x[k] = (v[k] * sqrt_n) / norm;
@@ -321,26 +321,39 @@ namespace dq {
 
 int64_t eden_static_max_n() { return kEdenStaticMaxTiles * (int64_t)kEdenTile; }
 
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex static_lock;
+double *static_scratch_of[kMaxDevices]; // device address of eden_static_scratch, per device
+} // namespace
+
+// Resolves the address of the static array on `device` (which the caller has made current), once per device.  Called
+// by the library's first call on a device, so that the entry point below has nothing left to look up when it runs
+// (e.g. under stream capture).
+hipError_t eden_static_prepare(int device)
+{
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> g(static_lock);
+    if (!static_scratch_of[device]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(eden_static_scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        static_scratch_of[device] = static_cast<double *>(p);
+    }
+    return hipSuccess;
+}
+
 hipError_t launch_eden_quantize_static(const float *vec, int64_t n, const float *boundaries, const float *centroids,
                                        int nbits, uint32_t *packed, float *result, int device, hipStream_t stream)
 {
-    constexpr int kMaxDevices = 64;
-    static std::mutex lock;
-    static double *scratch_of[kMaxDevices]; // device address of eden_static_scratch, per device
-    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
     if (eden_tiles(n) > kEdenStaticMaxTiles) return hipErrorInvalidValue;
+    const hipError_t e = eden_static_prepare(device);
+    if (e != hipSuccess) return e;
     double *scratch;
     {
-        std::lock_guard<std::mutex> g(lock);
-        if (!scratch_of[device]) {
-            // the caller has made `device` current
-            void *p = nullptr;
-            const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(eden_static_scratch));
-            if (e != hipSuccess) return e;
-            if (!p) return hipErrorInvalidSymbol;
-            scratch_of[device] = static_cast<double *>(p);
-        }
-        scratch = scratch_of[device];
+        std::lock_guard<std::mutex> g(static_lock);
+        scratch = static_scratch_of[device];
     }
     // every word of scratch that a kernel reads has been written by an earlier kernel of this same
     // call (sumsq -> norm, bins -> scale), so nothing has to be cleared between calls

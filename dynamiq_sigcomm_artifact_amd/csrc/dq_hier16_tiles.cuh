@@ -110,7 +110,10 @@ __device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int6
             for (int i = 0; i < 16; i++) t[i] = v.get(i) * ctr.wd.inv - mean;
         } else {
 #pragma unroll
-            for (int i = 0; i < 16; i++) t[i] = (float)((double)v.get(i) * ctr.wd.inv_d) - mean;
+            for (int i = 0; i < 16; i++) t[i] = v.get(i);
+            ctr.wd.divide16(t);
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] -= mean;
         }
     } else {
         // the ragged end of the vector: nothing at or beyond n_valid is read

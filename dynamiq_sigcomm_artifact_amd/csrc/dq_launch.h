@@ -155,6 +155,7 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
 // the same launches with the partial sums in the library's own static device array (no allocation anywhere);
 // `device` must be current
 int64_t eden_static_max_n();
+hipError_t eden_static_prepare(int device);
 hipError_t launch_eden_quantize_static(const float *vec, int64_t n, const float *boundaries, const float *centroids,
                                        int nbits, uint32_t *packed, float *result, int device,
                                        hipStream_t stream);

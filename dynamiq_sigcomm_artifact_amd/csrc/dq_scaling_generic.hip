@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
     if (!active) return;
 
     // pass 2: codes.  v / d is the correctly rounded quotient either way: with the chunk in registers and d an
-    // ordinary number it is the product with 1/d in double (see div_by), otherwise the IEEE division
+    // ordinary number it is the product with 1/d in double (see div_exact), otherwise the IEEE division
     BytePacker pk(cb);
     const auto codes = [&](auto fast) {
         const double yd = decltype(fast)::value ? recip_f64(d) : 0.0;
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kGenericBlock) void generic_compress_kernel(
         for (int i = 0; i < C; i++) {
             float v = CT ? ev.get(CT ? i : 0) : IO::load(src, base + i);
             float r = CT ? rv.get(CT ? i : 0) : ElemIO<RDT>::load(rnd, base + i);
-            float x = decltype(fast)::value ? div_by(v, yd) : v / d;
+            float x = decltype(fast)::value ? (DT == DQ_F16 ? div_by(v, yd) : div_exact(v, d, yd)) : v / d;
             int sv;
             if (DT == DQ_F16) {
                 x = rh(x);

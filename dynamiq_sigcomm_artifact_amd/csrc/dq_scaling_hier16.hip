@@ -56,7 +56,7 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     __shared__ __attribute__((aligned(16))) uint8_t win_out[RC::WIN];
     __shared__ __attribute__((aligned(16))) uint8_t win_in[FUSED ? RC::WIN : 16];
     __shared__ float table[(MEE && FUSED) ? (1 << NBITS) : 1];
-    const Center none{nullptr, 0, {0.0f, 0.0, 0, 0}};
+    const Center none{nullptr, 0, {0.0f, 0.0, 0, 0, 0, 0.0f}};
     compress_tile<DT, RDT, NBITS, MEE, FUSED>(src, recv, dst, rnd, row_ids_plain(rows), nsc, blockIdx.x, vec, key, none, mp, win_out,
                                               win_in, table, threadIdx.x);
 }

@@ -223,10 +223,7 @@ hipError_t launch_mixed_compress(const void *src, const float *center_mean, int 
     Center ctr;
     ctr.mean = center_mean;
     ctr.n_valid = n_valid;
-    ctr.wd.inv = 1.0f / (float)center_world;
-    ctr.wd.inv_d = 1.0 / (double)center_world;
-    ctr.wd.pow2 = (center_world & (center_world - 1)) == 0;
-    ctr.wd.fuse16 = ctr.wd.pow2 && center_world <= 65536;
+    ctr.wd = make_world_div(center_world, (dtype & 0xf) == DQ_F32 ? 4 : 2);
     const RandKey key = philox ? *philox : RandKey{0, 0};
     const bool rb16 = (dtype & DQ_RAND_BF16) != 0;
     dtype &= 0xf;

@@ -133,7 +133,8 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const float e = v.get(i);
-        float x = decltype(by_reciprocal)::value ? div_by(e, yd) : e / d;
+        // (a binary16 element divided by a binary16 scale is never subnormal in binary32)
+        float x = decltype(by_reciprocal)::value ? (DT == DQ_F16 ? div_by(e, yd) : div_exact(e, d, yd)) : e / d;
         int sv;
         if (DT == DQ_F16) {
             x = rh(x);

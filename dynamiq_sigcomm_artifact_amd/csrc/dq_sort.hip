@@ -9,6 +9,8 @@
 //   split    the first `top` values to the 8-bit list, the last `bottom` to the 2-bit list, the rest to the 4-bit list;
 //            work[0..3] = the counts
 // Everything lives in the caller's `work` buffer; no allocation, no host synchronisation.
+#include <algorithm>
+
 #include <hipcub/hipcub.hpp>
 
 #include "dq_bitwidth.cuh"
@@ -22,8 +24,22 @@ constexpr int kSortBlock = 256;
 
 __host__ __device__ inline size_t align256(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
 
-// upper bound of the radix sort's scratch with double buffers (measured: 0.034-0.10 bytes per item plus a constant)
-inline size_t sort_scratch_bound(int64_t nsc) { return align256((size_t)nsc / 8 + 65536); }
+// Scratch of the radix sort with double buffers: what the library itself asks for on this device for this many pairs (a
+// host-side query that launches nothing), padded by an eighth, and never less than nsc / 8 + 64 KiB (the sizes seen so far
+// are 0.034-0.10 bytes per item plus a constant).  Without a device to ask (a host that only sizes buffers) the floor alone.
+inline size_t sort_scratch_bound(int64_t nsc)
+{
+    size_t bound = align256((size_t)nsc / 8 + 65536);
+    hipcub::DoubleBuffer<uint16_t> keys(nullptr, nullptr);
+    hipcub::DoubleBuffer<int32_t> vals(nullptr, nullptr);
+    size_t asked = 0;
+    if (nsc <= (int64_t)0x7fffffff &&
+        hipcub::DeviceRadixSort::SortPairs(nullptr, asked, keys, vals, (int)nsc, 0, 16, nullptr) == hipSuccess)
+        bound = std::max(bound, align256(asked + asked / 8));
+    else
+        (void)hipGetLastError();
+    return bound;
+}
 
 struct LargePlanLayout {
     size_t keys[2], vals[2], scratch, total; // byte offsets into the workspace behind the 8-int header
@@ -92,12 +108,13 @@ hipError_t launch_group_plan_sorted_large(const void *stats, int64_t nsc, int64_
     // the arrays start at the first 256-byte boundary behind the header
     char *base = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(work + 8) + 255) & ~(uintptr_t)255);
     const LargePlanLayout l = layout_for(nsc);
+    const size_t scratch_room = l.total - l.scratch;
     hipcub::DoubleBuffer<uint16_t> keys(reinterpret_cast<uint16_t *>(base + l.keys[0]), reinterpret_cast<uint16_t *>(base + l.keys[1]));
     hipcub::DoubleBuffer<int32_t> vals(reinterpret_cast<int32_t *>(base + l.vals[0]), reinterpret_cast<int32_t *>(base + l.vals[1]));
     size_t scratch_bytes = 0;
     hipError_t e = hipcub::DeviceRadixSort::SortPairs(nullptr, scratch_bytes, keys, vals, (int)nsc, 0, 16, stream);
     if (e != hipSuccess) return e;
-    if (scratch_bytes > sort_scratch_bound(nsc)) return hipErrorOutOfMemory;
+    if (scratch_bytes > scratch_room) return hipErrorOutOfMemory;
     const unsigned blocks = (unsigned)((nsc + kSortBlock - 1) / kSortBlock);
     hipLaunchKernelGGL(sort_keys_kernel, dim3(blocks), dim3(kSortBlock), 0, stream, static_cast<const uint32_t *>(stats), nsc,
                        keys.Current(), vals.Current());

@@ -79,8 +79,7 @@ __global__ __launch_bounds__(64) void mean_center_tile_kernel(const void *__rest
 #pragma unroll
             for (int k = 0; k < 16; k++) v[k] = v[k] * wd.inv;
         } else {
-#pragma unroll
-            for (int k = 0; k < 16; k++) v[k] = (float)((double)v[k] * wd.inv_d);
+            wd.divide16(v);
         }
     } else {
 #pragma unroll
@@ -237,11 +236,7 @@ static hipError_t run_mean_center(const void *src, void *residual, void *stats, 
                          (reinterpret_cast<uintptr_t>(stats) & 3) == 0;
     if (aligned && n >= 256) {
         done = n / 256;
-        WorldDiv wd;
-        wd.inv = 1.0f / (float)world_size;
-        wd.inv_d = 1.0 / (double)world_size;
-        wd.pow2 = (world_size & (world_size - 1)) == 0;
-        wd.fuse16 = wd.pow2 && world_size <= 65536;
+        const WorldDiv wd = make_world_div(world_size, DT == DQ_F32 ? 4 : 2);
         hipLaunchKernelGGL(mean_center_tile_kernel<DT>, dim3((unsigned)((done + 3) / 4)), dim3(64), 0, stream, src, residual,
                            static_cast<uint32_t *>(stats), mean_out, done, wd);
         hipError_t e = hipGetLastError();

@@ -356,8 +356,25 @@ __device__ __forceinline__ double recip_f64(float b)
     return y;
 }
 
-// correctly rounded binary32 quotient a / b given yb ~= 1/b in double
+// binary32 quotient a / b given yb ~= 1/b in double.  The product carries a relative error below 2^-51, and a quotient of
+// two binary32 numbers that is a normal number comes no closer than 2^-49 (relative) to a rounding boundary without being
+// representable: for those this is the correctly rounded quotient.  A quotient in the subnormal range can lie exactly
+// half-way between two subnormal numbers (a = m 2^-150 b with m odd, possible when b is an even multiple of a power of
+// two), and there the error of the product decides the direction instead of the tie rule: where that can change a result,
+// use div_exact.
 __device__ __forceinline__ float div_by(float a, double yb) { return (float)((double)a * yb); }
+
+// q is a subnormal number other than zero
+__device__ __forceinline__ bool is_subnormal(float q) { return (__float_as_uint(q) & 0x7fffffffu) - 1u < 0x007fffffu; }
+
+// correctly rounded binary32 quotient a / b for every finite a: the product form, and the division itself when the product
+// comes out subnormal (a product that rounds to zero is below every tie, as is the quotient)
+__device__ __forceinline__ float div_exact(float a, float b, double yb)
+{
+    float q = div_by(a, yb);
+    if (is_subnormal(q)) q = a / b;
+    return q;
+}
 
 // log2_det() for a finite argument >= 1 (same operations, special cases dropped)
 __device__ __forceinline__ float log2_det_ge1(float x)
@@ -385,9 +402,11 @@ __device__ __forceinline__ float log2_det_ge1(float x)
 // One element of the fast quantiser, every operation as the reference orders them (three correctly rounded
 // divisions and the deterministic log2 for MEE): the signed code before clamping.
 template <bool MEE, class ARG>
-__device__ __forceinline__ int exact_code_fast(float vi, float ri, double yd, const ARG &mp)
+__device__ __forceinline__ int exact_code_fast(float vi, float ri, float d, double yd, const ARG &mp)
 {
-    float x = div_by(vi, yd);
+    // (the divisions further down are by constants above 1 of arguments that are zero or normal numbers, and a
+    // subnormal |x| / c disappears in the sum with 1)
+    float x = MEE ? div_by(vi, yd) : div_exact(vi, d, yd);
     if (MEE) {
         const float arg = div_by(__builtin_fabsf(x), mp.inv_c) + 1.0f;
         const float lat = div_by(log2_det_ge1(arg), mp.inv_l2b);
@@ -461,7 +480,7 @@ __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d
             if (__builtin_amdgcn_ballot_w64(doubt[i]) != 0) {
                 // (among them the zero elements -- padding, sparse input -- whose random value is exactly 0 or 1: their
                 // T is an integer, and the chain's ceil(-r) is 0, or -1 at r = 1)
-                const int sv = exact_code_fast<MEE>(v.get(i), r.get(i), yd, mp);
+                const int sv = exact_code_fast<MEE>(v.get(i), r.get(i), d, yd, mp);
                 if (doubt[i]) words_set<NBITS>(w, i, (uint32_t)(min(max(sv, -R), R) + R));
             }
         }

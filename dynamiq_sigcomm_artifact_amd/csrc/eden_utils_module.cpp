@@ -10,6 +10,8 @@
 // and 3/5/6/7-bit codes, plus rht_blocked, rand_diag, scaling_required_bytes,
 // set_quantization_seed and abi_version.
 #include <torch/extension.h>
+#include <c10/hip/HIPCachingAllocator.h>
+#include <c10/hip/HIPStream.h>
 
 #include <atomic>
 #include <vector>
@@ -63,6 +65,21 @@ void check_status(int status, const char *what)
 }
 
 dq_stream_t as_stream(uint64_t stream_p) { return reinterpret_cast<dq_stream_t>(static_cast<uintptr_t>(stream_p)); }
+
+// A tensor allocated here belongs to torch's current stream; the kernels that use it run on the caller's stream_p (the
+// reference's functions have the same split).  When the two differ the caching allocator is told, so that the block is
+// not handed out again (once the tensor is released) before the work queued on stream_p has finished with it.
+torch::Tensor on_stream(torch::Tensor t, uint64_t stream_p)
+{
+    if (!t.defined() || t.numel() == 0) return t;
+    const auto dev = t.device().index();
+    const hipStream_t s = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(stream_p));
+    if (c10::hip::getCurrentHIPStream(dev).stream() != s) {
+        const auto user = s == nullptr ? c10::hip::getDefaultHIPStream(dev) : c10::hip::getStreamFromExternal(s, dev);
+        c10::hip::HIPCachingAllocator::recordStream(t.storage().data_ptr(), user);
+    }
+    return t;
+}
 
 // ---- Hadamard --------------------------------------------------------------------
 
@@ -148,7 +165,7 @@ torch::Tensor rand_diag_bits(int64_t size, int64_t seed, torch::Device device, u
 {
     TORCH_CHECK(device.type() == torch::kCUDA, "device must be a CUDA device");
     TORCH_CHECK(size > 0 && size % 256 == 0, "size must be a positive multiple of 256");
-    auto bits = torch::empty({size / 32}, torch::TensorOptions().dtype(torch::kInt32).device(device));
+    auto bits = on_stream(torch::empty({size / 32}, torch::TensorOptions().dtype(torch::kInt32).device(device)), stream_p);
     check_status(dq_rand_diag_bits(reinterpret_cast<uint32_t *>(bits.data_ptr<int32_t>()), size, seed, bits.device().index(),
                                    as_stream(stream_p)),
                  "rand_diag_bits");
@@ -160,7 +177,7 @@ torch::Tensor pack_signs(torch::Tensor sign, uint64_t stream_p = 0)
     TORCH_CHECK(sign.device().type() == torch::kCUDA && sign.dtype() == torch::kFloat32 && sign.is_contiguous(),
                 "sign must be a contiguous torch.float32 CUDA tensor");
     TORCH_CHECK(sign.numel() > 0, "sign must not be empty");
-    auto bits = torch::empty({(sign.numel() + 31) / 32}, sign.options().dtype(torch::kInt32));
+    auto bits = on_stream(torch::empty({(sign.numel() + 31) / 32}, sign.options().dtype(torch::kInt32)), stream_p);
     check_status(dq_pack_signs(sign.data_ptr<float>(), reinterpret_cast<uint32_t *>(bits.data_ptr<int32_t>()), sign.numel(),
                                sign.device().index(), as_stream(stream_p)),
                  "pack_signs");
@@ -214,7 +231,7 @@ void scaling_decompress_irht(torch::Tensor src, c10::optional<torch::Tensor> sig
 torch::Tensor rand_diag(int64_t size, int64_t seed, torch::Device device, uint64_t stream_p = 0)
 {
     TORCH_CHECK(device.type() == torch::kCUDA, "device must be a CUDA device");
-    auto out = torch::empty({size}, torch::TensorOptions().device(device).dtype(torch::kFloat32));
+    auto out = on_stream(torch::empty({size}, torch::TensorOptions().device(device).dtype(torch::kFloat32)), stream_p);
     check_status(dq_rand_diag(out.data_ptr<float>(), size, seed, out.device().index(), as_stream(stream_p)), "rand_diag");
     return out;
 }
@@ -360,7 +377,7 @@ torch::Tensor group_plan(torch::Tensor qbits, torch::Tensor order, uint64_t stre
     const int64_t nsc = qbits.numel();
     TORCH_CHECK(nsc > 0, "qbits must not be empty");
     TORCH_CHECK(order.numel() >= 3 * nsc, "order has fewer than 3 * nsc entries");
-    auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
+    auto work = on_stream(torch::empty({dq_group_plan_work_ints(nsc)}, order.options()), stream_p);
     check_status(dq_group_plan(qbits.data_ptr<int64_t>(), nsc, order.data_ptr<int32_t>(), work.data_ptr<int32_t>(),
                                work.numel(), qbits.device().index(), as_stream(stream_p)),
                  "group_plan");
@@ -385,7 +402,7 @@ torch::Tensor group_plan_stats(torch::Tensor stats, double u, torch::Tensor orde
                     "qbits_out must be a contiguous torch.int64 CUDA tensor with one entry per superchunk");
         qptr = qbits_out->data_ptr<int64_t>();
     }
-    auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
+    auto work = on_stream(torch::empty({dq_group_plan_work_ints(nsc)}, order.options()), stream_p);
     check_status(dq_group_plan_stats(stats.data_ptr(), u, nsc, qptr, order.data_ptr<int32_t>(), work.data_ptr<int32_t>(),
                                      work.numel(), stats.device().index(), as_stream(stream_p)),
                  "group_plan_stats");
@@ -410,7 +427,7 @@ torch::Tensor group_plan_sorted(torch::Tensor stats, int64_t top_count, int64_t 
                     "qbits_out must be a contiguous torch.int64 CUDA tensor with one entry per superchunk");
         qptr = qbits_out->data_ptr<int64_t>();
     }
-    auto work = torch::empty({dq_group_plan_sorted_work_ints(nsc)}, order.options());
+    auto work = on_stream(torch::empty({dq_group_plan_sorted_work_ints(nsc)}, order.options()), stream_p);
     check_status(dq_group_plan_sorted(stats.data_ptr(), nsc, top_count, bottom_count, qptr, order.data_ptr<int32_t>(),
                                       work.data_ptr<int32_t>(), work.numel(), stats.device().index(), as_stream(stream_p)),
                  "group_plan_sorted");
@@ -438,7 +455,7 @@ torch::Tensor group_plan_stats_dev_u(torch::Tensor stats, torch::Tensor u, torch
                     "qbits_out must be a contiguous torch.int64 CUDA tensor with one entry per superchunk");
         qptr = qbits_out->data_ptr<int64_t>();
     }
-    auto work = torch::empty({dq_group_plan_work_ints(nsc)}, order.options());
+    auto work = on_stream(torch::empty({dq_group_plan_work_ints(nsc)}, order.options()), stream_p);
     uint32_t *hptr = nullptr;
     int64_t hlen = 0;
     if (hist.has_value()) {
@@ -477,7 +494,7 @@ torch::Tensor bitrate_search(torch::Tensor hist, int mode, double prev_u, double
     TORCH_CHECK(hist.dtype() == torch::kInt32 && hist.is_contiguous(), "hist must be a contiguous torch.int32 tensor");
     TORCH_CHECK(hist.numel() >= dq_bitrate_hist_ints(), "hist has fewer than bitrate_hist_ints() entries");
     TORCH_CHECK(mode == 0 || mode == 1, "mode must be 0 (bisection) or 1 (correction from prev_u)");
-    auto result = torch::empty({4}, hist.options().dtype(torch::kFloat64));
+    auto result = on_stream(torch::empty({4}, hist.options().dtype(torch::kFloat64)), stream_p);
     check_status(dq_bitrate_search(reinterpret_cast<uint32_t *>(hist.data_ptr<int32_t>()), hist.numel(), mode, prev_u, nullptr,
                                    target_avg_bits, result.data_ptr<double>(), hist.device().index(), as_stream(stream_p)),
                  "bitrate_search");
@@ -732,10 +749,10 @@ torch::Tensor EdenBinsToBits(torch::Tensor bins, int nbits)
     auto nbins = bins.size(-1);
     TORCH_CHECK(nbins == bins.numel(), "bins must be 1D");
     TORCH_CHECK((nbins & 31) == 0, "bins size must be a multiple of 32");
-    auto cbins = bins.clone();
+    auto cbins = on_stream(bins.clone(), 0);
     const int device = cbins.device().index();
     auto opts = torch::TensorOptions().device(bins.device().type(), device).dtype(torch::kInt32);
-    torch::Tensor carr = torch::zeros({(nbins >> 5) * nbits}, opts);
+    torch::Tensor carr = on_stream(torch::zeros({(nbins >> 5) * nbits}, opts), 0);
     if (nbins > 0)
         check_status(dq_bins_to_bits(cbins.data_ptr<int32_t>(), nbins, reinterpret_cast<uint32_t *>(carr.data_ptr<int32_t>()),
                                      (nbins >> 5) * nbits, nbits, device, nullptr),
@@ -749,11 +766,11 @@ torch::Tensor EdenBitsToBins(torch::Tensor arr, int nbits)
     TORCH_CHECK(arr.dtype() == torch::kInt32, "arr must be a torch.int32 CUDA tensor");
     auto narr = arr.size(-1);
     TORCH_CHECK(narr == arr.numel(), "arr must be 1D");
-    auto carr = arr.clone();
+    auto carr = on_stream(arr.clone(), 0);
     const int device = carr.device().index();
     auto opts = torch::TensorOptions().device(arr.device().type(), device).dtype(torch::kInt32);
     const int64_t nbins = (narr / nbits) << 5;
-    torch::Tensor cbins = torch::zeros({nbins}, opts);
+    torch::Tensor cbins = on_stream(torch::zeros({nbins}, opts), 0);
     if (nbins > 0)
         check_status(dq_bits_to_bins(cbins.data_ptr<int32_t>(), nbins, reinterpret_cast<const uint32_t *>(carr.data_ptr<int32_t>()),
                                      (nbins >> 5) * nbits, nbits, device, nullptr),
@@ -834,9 +851,9 @@ std::vector<torch::Tensor> eden_quantize(torch::Tensor vec, torch::Tensor bounda
     TORCH_CHECK(n > 0 && (n & 31) == 0, "vec size must be a positive multiple of 32");
     TORCH_CHECK(boundaries.numel() == (1 << nbits) - 1, "boundaries must hold 2^nbits - 1 values");
     TORCH_CHECK(centroids.numel() == (1 << nbits), "centroids must hold 2^nbits values");
-    auto packed = torch::empty({n / 32 * nbits}, vec.options().dtype(torch::kInt32));
-    auto result = torch::empty({4}, vec.options());
-    auto work = torch::empty({dq_eden_work_doubles(n)}, vec.options().dtype(torch::kFloat64));
+    auto packed = on_stream(torch::empty({n / 32 * nbits}, vec.options().dtype(torch::kInt32)), stream_p);
+    auto result = on_stream(torch::empty({4}, vec.options()), stream_p);
+    auto work = on_stream(torch::empty({dq_eden_work_doubles(n)}, vec.options().dtype(torch::kFloat64)), stream_p);
     check_status(dq_eden_quantize(vec.data_ptr<float>(), n, boundaries.data_ptr<float>(), centroids.data_ptr<float>(), nbits,
                                   reinterpret_cast<uint32_t *>(packed.data_ptr<int32_t>()), result.data_ptr<float>(),
                                   work.data_ptr<double>(), work.numel(), vec.device().index(), as_stream(stream_p)),
@@ -853,7 +870,7 @@ torch::Tensor eden_dequantize(torch::Tensor packed, torch::Tensor centroids, int
     TORCH_CHECK(packed.numel() > 0 && packed.numel() % nbits == 0, "packed size must be a multiple of nbits");
     TORCH_CHECK(centroids.numel() == (1 << nbits), "centroids must hold 2^nbits values");
     const int64_t n = packed.numel() / nbits * 32;
-    auto out = torch::empty({n}, centroids.options());
+    auto out = on_stream(torch::empty({n}, centroids.options()), stream_p);
     check_status(dq_eden_dequantize(reinterpret_cast<const uint32_t *>(packed.data_ptr<int32_t>()), n, centroids.data_ptr<float>(),
                                     nbits, out.data_ptr<float>(), packed.device().index(), as_stream(stream_p)),
                  "eden_dequantize");
@@ -870,7 +887,7 @@ torch::Tensor eden_dequantize_irht(torch::Tensor packed, torch::Tensor centroids
     TORCH_CHECK(packed.numel() > 0 && packed.numel() % nbits == 0, "packed size must be a multiple of nbits");
     TORCH_CHECK(centroids.numel() == (1 << nbits), "centroids must hold 2^nbits values");
     const int64_t n = packed.numel() / nbits * 32;
-    auto out = torch::empty({n}, centroids.options());
+    auto out = on_stream(torch::empty({n}, centroids.options()), stream_p);
     int sign_packed = 0;
     const void *sp = sign_arg(sign, out, n, &sign_packed);
     const float *ps = nullptr;
@@ -896,7 +913,7 @@ torch::Tensor thc_quantize(torch::Tensor rotated, torch::Tensor uniform, torch::
     TORCH_CHECK(uniform.numel() >= rotated.numel(), "uniform has fewer elements than rotated");
     TORCH_CHECK(lo.numel() == 1 && delta.numel() == 1, "lo and delta must hold one value");
     TORCH_CHECK(levels >= 2 && levels <= 256, "levels must be in [2, 256]");
-    auto out = torch::empty({rotated.numel()}, rotated.options().dtype(torch::kBFloat16));
+    auto out = on_stream(torch::empty({rotated.numel()}, rotated.options().dtype(torch::kBFloat16)), stream_p);
     check_status(dq_thc_quantize(rotated.data_ptr<float>(), uniform.data_ptr<float>(), out.data_ptr(), rotated.numel(),
                                  lo.data_ptr<float>(), delta.data_ptr<float>(), levels, rotated.device().index(),
                                  as_stream(stream_p)),

@@ -185,7 +185,11 @@ int dq_group_plan_stats(const void *stats, double u, int64_t nsc, int64_t *qbits
  * work holds 4 ints.  Longer buckets (the reference's training scripts give
  * DDP a 4000 MB bucket cap, testbed_evaluation/train_llm_causal.py:416): a
  * stable radix sort of the 16-bit keys inside `work`, which must then hold
- * dq_group_plan_sorted_work_ints(nsc) ints (about 12.2 bytes per superchunk).
+ * dq_group_plan_sorted_work_ints(nsc) ints (about 12.2 bytes per superchunk; the
+ * figure includes the scratch the sort library asks for on the current device,
+ * so call it with the device selected that will run the plan).  The long path
+ * runs the library's sort, whose launches include memset nodes: only the
+ * one-launch path (nsc <= 65535) may be captured into a HIP graph.
  * stats 4-byte aligned. */
 int64_t dq_group_plan_sorted_work_ints(int64_t nsc);
 int dq_group_plan_sorted(const void *stats, int64_t nsc, int64_t top_count, int64_t bottom_count,
@@ -345,7 +349,10 @@ int dq_eden_quantize(const float *vec, int64_t n, const float *boundaries, const
  * harnesses that forbid hipMalloc): the same launches and the same results, with
  * the per-tile partial sums in a static device array inside the library
  * (512 KiB per GPU, held until the process ends) instead of a caller's `work`.
- * Neither this call nor anything it runs allocates or frees memory.
+ * Neither this call nor anything it runs allocates or frees memory.  The
+ * array's device address is looked up once per GPU by the first call of any
+ * function of this library on that GPU; under stream capture, make one such
+ * call (any, e.g. this one as a warm-up) before the capture begins.
  * n is limited to dq_eden_quantize_static_max_n() = 2^28 elements; a larger n
  * is refused with DQ_ERR_SIZE.  All calls on one GPU share the array: calls
  * that may overlap on one GPU (two streams, two threads) race -- serialise them

@@ -288,6 +288,17 @@ def philox_uniform(n, seed, step):
     return out
 
 
+def philox_uniform_rows(rows, seed, step):
+    """the values of philox_uniform for the superchunks (256 elements each) listed in rows, concatenated"""
+    rows = np.ascontiguousarray(rows, np.int64)
+    out = np.zeros(rows.size * 256, np.float32)
+    f = lib().dqo_philox_uniform_rows
+    f.restype = None
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_uint64]
+    f(_p(out), _p(rows), rows.size, int(seed), int(step))
+    return out
+
+
 def eden_quantize(vec, boundaries, centroids, nbits):
     """-> (bins int32 [n], result float32 [4] = sumsq, dot, scale, norm)"""
     _chk(vec, np.float32, "vec")

@@ -847,6 +847,22 @@ void dqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t step)
     }
 }
 
+/* the same stream for a list of superchunks: out[256 k + e] = the value of element 256 rows[k] + e */
+void dqo_philox_uniform_rows(float *out, const int64_t *rows, int64_t nrows, uint64_t seed, uint64_t step)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    for (int64_t k = 0; k < nrows; k++) {
+        for (int j = 0; j < 16; j++) {
+            const int64_t chunk = rows[k] * 16 + j;
+            const uint32_t ctr[4] = {(uint32_t)chunk, (uint32_t)((uint64_t)chunk >> 32), (uint32_t)step, (uint32_t)(step >> 32)};
+            uint32_t w[4];
+            dqo_philox4x32_10(ctr, key, w);
+            for (int i = 0; i < 16; i++)
+                out[k * 256 + j * 16 + i] = (float)(((w[i >> 2] >> (8 * (i & 3))) & 0xffu) | 1u) * 0.00390625f;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------------ */
 /* EDEN Lloyd-Max quantiser, THC uniform quantiser                           */
 /* ------------------------------------------------------------------------ */

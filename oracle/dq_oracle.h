@@ -135,6 +135,7 @@ void dqo_bits_to_bins(const uint32_t *arr, int64_t narr, int32_t *bins, int nbit
  * random values are an input tensor): Philox4x32-10, pinned by the published known-answer vectors. */
 void dqo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
 void dqo_philox_uniform(float *out, int64_t n, uint64_t seed, uint64_t step);
+void dqo_philox_uniform_rows(float *out, const int64_t *rows, int64_t nrows, uint64_t seed, uint64_t step);
 
 /* cuda_kernels/src/srrcomp/srrcomp.py:356-361 (Eden._quantize) and :343-345; sums in double in the
  * library's documented order (torch's reduction order is unspecified: "parity unpinned" for the

@@ -161,7 +161,7 @@ def test_mixed_philox_matches_oracle(capi, oracle, dt, odt, strategy):
 
 
 @pytest.mark.parametrize("dt,odt", [(torch.bfloat16, BF16), (torch.float32, F32)])
-@pytest.mark.parametrize("world", [1, 2, 3, 8])
+@pytest.mark.parametrize("world", [1, 2, 3, 8, 6, 24])
 @pytest.mark.parametrize("n", [256 * 40, 256 * 41 - 200, 256 * 41 - 1, 77])
 def test_stats_and_centre_on_load(capi, oracle, dt, odt, world, n):
     """superchunk_stats == the oracle's statistics and binary32 means; compress with the centring folded into the
@@ -174,6 +174,15 @@ def test_stats_and_centre_on_load(capi, oracle, dt, odt, world, n):
         # the centred value must still be the one of the two-step arithmetic
         base[256:512] = torch.randn(256, generator=g) * 1e-39
         base[512:768] = torch.randn(256, generator=g) * 3e-38
+        # element / world exactly half-way between two subnormal numbers (m 2^-150, m odd; representable in binary32 for
+        # an even world size that is not a power of two), in pairs that cancel in the first step of the mean's tree:
+        # the mean is zero and the residual is the rounded quotient itself
+        m = torch.randint(0, 500, (128,), generator=g).double() * 2 + 1
+        tie = m * world * 2.0 ** -150
+        base = base.double()
+        base[768:896] = tie
+        base[896:1024] = -tie
+        base = base.float()
     src = torch.full((n + 64,), float("nan"), dtype=dt, device=DEV)     # a NaN beyond n must never be picked up
     src[:n] = base.to(dt)
     stats = torch.zeros(nsc, 2, dtype=torch.bfloat16, device=DEV)
@@ -190,8 +199,13 @@ def test_stats_and_centre_on_load(capi, oracle, dt, odt, world, n):
     stats3 = torch.zeros_like(stats)
     capi.superchunk_mean_center(src, residual, stats3, n, world)
     assert torch.equal(bits_t(stats), bits_t(stats3))
+    res_o, _ = oracle.superchunk_mean_center(to_bits(src[:n].cpu()), n, world, odt)
+    assert (to_bits(residual.cpu()).view(res_o.dtype if odt != F32 else np.uint32) ==
+            (res_o if odt != F32 else res_o.view(np.uint32))).all()
     q, order, work = make_plan(capi, nsc, n)
-    pool = torch.rand(nsc * 256, generator=g).to(dt).to(DEV)
+    pool = torch.rand(nsc * 256, generator=g)
+    pool[768:1024] = 0.0        # (a random value of 0 turns the lowest bit of a tiny quotient into a code)
+    pool = pool.to(dt).to(DEV)
     cap = capi.mixed_required_bytes(nsc, 1)
     for strategy in (2, 3):
         a = torch.zeros(cap, dtype=torch.uint8, device=DEV)

@@ -241,6 +241,55 @@ def test_estimate_route_at_the_ends_of_its_range(capi, oracle, dt, strategy, C):
         _dec_comp(capi, oracle, dt, n, nbits, C, strategy, src, (src.float() * -0.5).to(tdt), rnd, rnd.flip(0).contiguous(), tag)
 
 
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("strategy", [0, 1, 2, 3])
+@pytest.mark.parametrize("C", [16, 8, 32])
+def test_subnormal_quotients_half_way_between_two_subnormal_numbers(capi, oracle, dt, strategy, C):
+    """Elements v = m 2^-150 d (m odd, d the quantisation step of their chunk) with random value 0: the quotient v / d
+    is a tie between two subnormal numbers, which the division rounds to even and a product with an inexact reciprocal
+    of d does not, and with a random value of 0 the code is R for a quotient of 0 and R + 1 for anything above.  Such
+    a v exists when d is an even multiple of a power of two (binary32 elements) or a multiple of 2^17 (bfloat16): the
+    chunk maxima are chosen so that d = q 2^k."""
+    from helpers import unpack_stream
+    tdt = TORCH_DT[dt]
+    nsc = 40
+    n = nsc * 16 * C
+    g = torch.Generator().manual_seed(5150 + strategy + C)
+    ks = torch.tensor([1, 2, 3, 5, 17, 18, 20, 30, 40, 60])
+    qs = torch.tensor([255, 3, 5, 6, 7, 9, 10, 11, 12, 13, 14, 15, 20, 22, 100, 254])
+    placed = 0
+    for nbits in (2, 4, 8):
+        if (C * nbits) % 8:
+            continue
+        R = (1 << (nbits - 1)) - 1
+        amax = (qs.double() - torch.where(qs == 255, 0.0, 0.5)).view(1, 16) * (2.0 ** ks[torch.arange(nsc) % ks.numel()].double()).view(nsc, 1) * R
+        src = (torch.rand(nsc, 16, C, generator=g).double() - 0.5) * amax.view(nsc, 16, 1)
+        src[:, :, 0] = amax * torch.where(torch.rand(nsc, 16, generator=g) < 0.5, -1.0, 1.0)
+        src = src.reshape(-1).float().to(tdt)
+        enc = oracle.scaling_compress(to_bits(src), to_bits(torch.full((n,), 0.5).to(tdt)), n, nbits, C, strategy, dt)
+        _, (a0, a1) = unpack_stream(enc, n, nbits, C, strategy)
+        if strategy >= 2:
+            step = a0.astype(np.float64) * bits_to_f32(a1, BF16).astype(np.float64).repeat(16)
+        else:
+            step = bits_to_f32(a0, BF16).astype(np.float64)
+        vals = src.double().reshape(-1, C).clone()
+        rnd = torch.rand(n // C, C, generator=g)
+        for slot, m in enumerate((1, 3, 5, 7, 9, 11, 13), start=1):
+            if slot >= C:
+                break
+            cand = torch.from_numpy(step * m * 2.0 ** -150)
+            cand = torch.where(torch.rand(cand.shape, generator=g) < 0.5, -cand, cand)
+            ok = (cand.float().to(tdt).double() == cand) & (cand != 0)
+            vals[:, slot] = torch.where(ok, cand, vals[:, slot])
+            rnd[:, slot] = torch.where(ok, torch.tensor([0.0, 0.0, 1.0, 2.0 ** -20])[torch.randint(0, 4, ok.shape, generator=g)], rnd[:, slot])
+            placed += int(ok.sum())
+        src2 = vals.reshape(-1).float().to(tdt)
+        assert torch.equal(src2.double().reshape(-1, C)[:, 0], src.double().reshape(-1, C)[:, 0])
+        tag = "ties dt=%d C=%d b=%d s=%d" % (dt, C, nbits, strategy)
+        _roundtrip(capi, oracle, dt, n, nbits, C, strategy, src2, rnd.reshape(-1).to(tdt), tag)
+    assert placed > (400 if dt == F32 else 40), placed
+
+
 @pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [2, 3])
 @pytest.mark.parametrize("C", [16, 8, 32])

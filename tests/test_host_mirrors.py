@@ -80,6 +80,33 @@ def test_compressor_object_matches_reference_bookkeeping(eden_utils, oracle):
         assert (to_bits(out) == dec).all()
 
 
+@pytest.mark.gpu
+def test_loaded_random_pool_keeps_the_dtype_the_reference_keeps(eden_utils, oracle):
+    """the "correlated" mode loads its pool from a file: the AEE class keeps the file's dtype (utils_aggregation.py:389),
+    the MEE class casts it to float16 (:488), so a bfloat16 call of the MEE class rounds every value twice"""
+    from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern
+    d, W, n = 256 * 40, 2, 256 * 6
+    g = torch.Generator().manual_seed(8)
+    loaded = torch.rand(3 * ((d + 16) // 16) // W * 16 + 100, generator=g)
+    x = (torch.randn(n, generator=g) * 1e-3).to(torch.bfloat16)
+    twice = loaded.to(torch.float16).to(torch.bfloat16)
+    once = loaded.to(torch.bfloat16)
+    assert not torch.equal(twice, once)
+    for cls, strategy, seen, kept in ((Aee_Dynamic_Range_GPU_kern, 2, once, torch.float32),
+                                      (Mee_Dynamic_Range_GPU_kern, 3, twice, torch.float16)):
+        c = cls(4, 16, dict(_params(d, W), rand_pool_tensor=loaded))
+        assert c.randomized_vec_pool.dtype == kept
+        rows = c.randomized_vec_pool.shape[0]
+        assert rows == 3 * ((d + 16) // 16) // W
+        send = c.create_tensor(x, torch.uint8)
+        c.compression(x.to(DEV), send)
+        seed = ((4 * 998244353) & 0xFFFFFFFF) * 671431 + 1000000007 & 0xFFFFFFFF
+        randl = seed % (rows - n // 16 - 1)
+        rnd = seen[randl * 16:randl * 16 + n]
+        want = oracle.scaling_compress(to_bits(x), to_bits(rnd), n, 4, 16, strategy, BF16)
+        assert (send.cpu().numpy() == want).all()
+
+
 def _oracle_ring(oracle, vecs_bits, pools, nbits, strategy, W):
     """the same schedule on the CPU with oracle calls (ring_rdma.py:590-631)"""
     n = vecs_bits[0].size

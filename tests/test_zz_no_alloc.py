@@ -41,6 +41,48 @@ def test_static_scratch_matches_caller_scratch_twice_second_smaller(capi):
         assert np.isfinite(rb).all() and rb[0] > 0 and rb[2] > 0
 
 
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph(capi):
+    """a warmed call leaves the device's free-memory counter where it was, and the call captured into a HIP graph on one
+    stream gives the eager result on every replay (other work and synchronisations between the replays)"""
+    n, nbits = 4096 * 9 + 64, 4
+    g = torch.Generator().manual_seed(21)
+    x = (torch.randn(n, generator=g) * 3e-3).to(DEV)
+    cen = torch.from_numpy(GOLD["centroids_%d" % nbits]).to(DEV)
+    bnd = torch.from_numpy(GOLD["boundaries_%d" % nbits]).to(DEV)
+    words = n // 32 * nbits
+    eager = torch.zeros(words, dtype=torch.int32, device=DEV)
+    res_eager = torch.zeros(4, device=DEV)
+    capi.eden_quantize_static(x, bnd, cen, nbits, eager, res_eager)           # warm-up: the library is loaded and set up
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        capi.eden_quantize_static(x, bnd, cen, nbits, eager, res_eager)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+
+    packed = torch.zeros(words, dtype=torch.int32, device=DEV)
+    res = torch.zeros(4, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            capi.eden_quantize_static(x, bnd, cen, nbits, packed, res, stream=side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for k in range(3):
+        packed.fill_(-1)              # a fill kernel, not a memset node
+        res.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(packed, eager), k
+        assert torch.equal(res.view(torch.int32), res_eager.view(torch.int32)), k
+        y = (x * 2.0).sum()           # the program's own eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(y)
+
+
 def test_static_scratch_rejects_oversize_and_bad_arguments(capi):
     L = capi.lib()
     one = torch.zeros(64, device=DEV)
