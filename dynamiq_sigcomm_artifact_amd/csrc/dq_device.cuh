@@ -355,6 +355,22 @@ __device__ __forceinline__ float thc_level(float v, float u, float lo, float del
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// A 16-byte store of output that this kernel does not read again, with the non-temporal hint: the decoders' element
+// stores run a fifth faster with it on a 25 MB bucket (fp32 7.7 -> 6.25 us, bf16 5.6 -> 4.5 us with every launch
+// streaming to memory; 6.8 -> 6.0 and 5.4 -> 4.2 us replaying one bucket).  The same hint on the loads costs 15-20 %,
+// and on the encoder's small record stream it is within noise either way: neither carries it.
+__device__ __forceinline__ void stream_store(uint4 *p, uint4 v)
+{
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4 *>(p));
+}
+__device__ __forceinline__ void stream_store(float4 *p, float4 v)
+{
+    const u32x4 t = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4 *>(p));
+}
+
+
 // LDS accesses of one wave execute in order; the fence only stops the compiler
 // from moving them across the hand-over between lanes
 __device__ __forceinline__ void wave_lds_sync()
@@ -380,7 +396,7 @@ __device__ __forceinline__ void store_wave_words16(uint4 *tile, const uint32_t (
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int s = 64 * k + lane;
-        if (s < valid_slots) dst[s] = tile[swz(s)];
+        if (s < valid_slots) stream_store(dst + s, tile[swz(s)]);
     }
 }
 

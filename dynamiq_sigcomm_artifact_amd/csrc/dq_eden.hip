@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256) void thc_dequantize_kernel(const uint16_t *__r
         float p0 = bf16_bits_to_f32(l.x & 0xffffu) * step, p1 = bf16_bits_to_f32(l.x >> 16) * step;
         float p2 = bf16_bits_to_f32(l.y & 0xffffu) * step, p3 = bf16_bits_to_f32(l.y >> 16) * step;
         o.x = p0 + lo; o.y = p1 + lo; o.z = p2 + lo; o.w = p3 + lo;
-        *reinterpret_cast<float4 *>(out + i) = o;
+        stream_store(reinterpret_cast<float4 *>(out + i), o);
     } else {
         const int64_t i = begin + (int64_t)blockIdx.x * 256 + threadIdx.x;
         if (i >= n) return;

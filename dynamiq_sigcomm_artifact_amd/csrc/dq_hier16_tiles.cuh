@@ -343,7 +343,11 @@ __device__ __forceinline__ void decompress_tile(const uint8_t *__restrict__ src,
                 const int64_t e = d_slot[k] * 256 + (s % (16 * S)) * EP;
                 const uint4 val = tile_out[swz(s)];
                 if (e + EP <= limit) {
-                    *reinterpret_cast<uint4 *>(dbytes + e * ESZ) = val;
+                    // (the accumulating variant writes the lines it has just read: no streaming hint there)
+                    if (ADD)
+                        *reinterpret_cast<uint4 *>(dbytes + e * ESZ) = val;
+                    else
+                        stream_store(reinterpret_cast<uint4 *>(dbytes + e * ESZ), val);
                 } else {
                     const uint32_t part[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll

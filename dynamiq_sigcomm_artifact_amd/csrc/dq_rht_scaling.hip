@@ -257,7 +257,7 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
             float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
             v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale;
             flip4(v, a, g);
-            *reinterpret_cast<float4 *>(x + g) = v;
+            stream_store(reinterpret_cast<float4 *>(x + g), v);
         }
     } else {
         for (int i = tid; i < tile; i += nthreads) {
@@ -614,7 +614,7 @@ __global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel
                 float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
                 v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale;
                 flip4(v, a, half_origin + i);
-                *reinterpret_cast<float4 *>(x + half_origin + i) = v;
+                stream_store(reinterpret_cast<float4 *>(x + half_origin + i), v);
             }
         } else {
             for (int i = tid; i < (1 << kHalfBits); i += kSplitThreads)

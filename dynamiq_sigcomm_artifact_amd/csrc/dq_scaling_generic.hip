@@ -169,7 +169,7 @@ __device__ __forceinline__ void store_wave_slots(uint4 *tile, const uint4 (&slot
 #pragma unroll
     for (int k = 0; k < S; k++) {
         const int s = 64 * k + lane;
-        if (s < valid) dst[s] = tile[swz(s)];
+        if (s < valid) stream_store(dst + s, tile[swz(s)]);
     }
 }
 
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(kGenericBlock) void generic_decompress_kernel(
         }
         uint4 *wave_dst = reinterpret_cast<uint4 *>(static_cast<char *>(dst) + wave_first * ChunkShape<DT, CR>::kBytes);
         if constexpr (S == 1) {
-            if (active) wave_dst[lane] = slot[0];
+            if (active) stream_store(wave_dst + lane, slot[0]);
         } else {
             const int valid = (int)min((int64_t)64, nchunks - wave_first) * S;
             store_wave_slots<S>(tiles[threadIdx.x >> 6], slot, wave_dst, lane, valid);

@@ -57,7 +57,8 @@ __global__ __launch_bounds__(64) void hier16_compress_kernel(const void *__restr
     __shared__ __attribute__((aligned(16))) uint8_t win_in[FUSED ? RC::WIN : 16];
     __shared__ float table[(MEE && FUSED) ? (1 << NBITS) : 1];
     const Center none{nullptr, 0, {0.0f, 0.0, 0, 0, 0, 0.0f}};
-    compress_tile<DT, RDT, NBITS, MEE, FUSED>(src, recv, dst, rnd, row_ids_plain(rows), nsc, blockIdx.x, vec, key, none, mp, win_out,
+    const int64_t tile = blockIdx.x;
+    compress_tile<DT, RDT, NBITS, MEE, FUSED>(src, recv, dst, rnd, row_ids_plain(rows), nsc, tile, vec, key, none, mp, win_out,
                                               win_in, table, threadIdx.x);
 }
 
@@ -85,7 +86,8 @@ __global__ __launch_bounds__(64) void hier16_decompress_kernel(const uint8_t *__
             wave_lds_sync(); // window, table and output tile are reused by the next tile
         }
     } else {
-        decompress_tile<DT, NBITS, MEE, ADD>(src, dst, row_ids_plain(rows), stats, limit, nsc, blockIdx.x, vec, mp, win_in, tile_out,
+        const int64_t tile = blockIdx.x;
+        decompress_tile<DT, NBITS, MEE, ADD>(src, dst, row_ids_plain(rows), stats, limit, nsc, tile, vec, mp, win_in, tile_out,
                                              table);
     }
 }

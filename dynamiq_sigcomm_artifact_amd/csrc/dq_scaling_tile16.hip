@@ -257,7 +257,12 @@ __global__ __launch_bounds__(64) void tile16_decompress_kernel(const uint8_t *__
 #pragma unroll
         for (int k = 0; k < S; k++) {
             const int s = 64 * k + lane;
-            if (s < nslots) g[s] = tile_out[swz(s)];
+            if (s < nslots) {
+                if (ADD)
+                    g[s] = tile_out[swz(s)];
+                else
+                    stream_store(g + s, tile_out[swz(s)]);
+            }
         }
     } else if (active) {
         out.store(dst, e0 + lane * 16, false);

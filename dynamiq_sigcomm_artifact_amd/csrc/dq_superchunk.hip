@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void add_mean_copy_vec_kernel(const uint4 *__r
             w[k] = f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
         }
     }
-    dst[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    stream_store(dst + i, make_uint4(w[0], w[1], w[2], w[3]));
 }
 
 template <int DT>
