@@ -26,11 +26,29 @@ EXPORTS = [
     "dq_group_plan_stats_dev_u", "dq_group_plan_sorted", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
+    "dq_dynamic_bitrate_bucket",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_rht_scaling_compress_mfma16", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
     "dq_eden_work_doubles", "dq_eden_quantize", "dq_eden_quantize_static_max_n", "dq_eden_quantize_static", "dq_eden_dequantize", "dq_eden_dequantize_irht", "dq_thc_quantize", "dq_thc_dequantize", "dq_thc_rht_quantize", "dq_thc_dequantize_irht",
 ]
+
+STAGE_STATS, STAGE_PLAN, STAGE_COMPRESS, STAGE_DECOMPRESS = 1, 2, 4, 8
+STAGE_ALL = 15
+
+
+class Bucket(ctypes.Structure):
+    """dq_bucket_t of include/dynamiq_eden.h"""
+    _fields_ = [
+        ("src", ctypes.c_void_p), ("n", ctypes.c_int64), ("dtype", ctypes.c_int32), ("strategy", ctypes.c_int32),
+        ("center_world", ctypes.c_int32), ("ring_chunk", ctypes.c_int32), ("ring_world", ctypes.c_int32),
+        ("reserved", ctypes.c_int32), ("u", ctypes.c_double), ("u_dev", ctypes.c_void_p), ("stats", ctypes.c_void_p),
+        ("mean", ctypes.c_void_p), ("reduced_stats", ctypes.c_void_p), ("order", ctypes.c_void_p),
+        ("work", ctypes.c_void_p), ("work_ints", ctypes.c_int64), ("recv", ctypes.c_void_p), ("packed", ctypes.c_void_p),
+        ("packed_bytes", ctypes.c_int64), ("out", ctypes.c_void_p), ("hist", ctypes.c_void_p),
+        ("hist_ints", ctypes.c_int64), ("seed", ctypes.c_uint64), ("step", ctypes.c_uint64), ("step_dev", ctypes.c_void_p),
+    ]
+
 
 _lib = None
 
@@ -103,6 +121,8 @@ def lib():
         L.dq_mixed_decompress.argtypes = [vp, vp, vp, vp, i32, i32, vp, i64, i64, i32, i32, i32, vp]
         L.dq_superchunk_stats.restype = i32
         L.dq_superchunk_stats.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
+        L.dq_dynamic_bitrate_bucket.restype = i32
+        L.dq_dynamic_bitrate_bucket.argtypes = [c.POINTER(Bucket), i32, i32, vp]
         L.dq_superchunk_mean_center.restype = i32
         L.dq_superchunk_mean_center.argtypes = [vp, vp, vp, i64, i32, i32, i32, i32, vp]
         L.dq_superchunk_add_mean_copy.restype = i32
@@ -404,6 +424,61 @@ def mixed_decompress(src, dst, order, counts, nsc, strategy, stats=None, n_limit
     _call(lib().dq_mixed_decompress, _p(src), _p(dst), _p(order), _p(counts), ring_chunk,
                                      ring_world, _ptr(stats), nsc * 256 if n_limit is None else n_limit, nsc,
                                      dtype_code(dst), _dev(dst), strategy, _stream(stream))
+
+
+def bucket_descriptor(src, n, stats, mean, order, work, packed, strategy=2, out=None, u=0.0, reduced_stats=None,
+                      center_world=1, ring_chunk=0, ring_world=1, recv=None, hist=None, seed=0, step=0, step_dev=None):
+    """A dq_bucket_t for dynamic_bitrate_bucket, filled from tensors (each checked: contiguous, on one GPU, of the dtype
+    and size the stages need).  u: a number, or a float64 device tensor read when the plan runs.  The descriptor keeps
+    addresses, not tensors: whoever holds it keeps the tensors alive.  Returns (descriptor, device index)."""
+    nsc = (n + 255) // 256
+    code = dtype_code(src)
+    need = [(stats, torch.bfloat16, 2 * nsc, "stats"), (mean, torch.float32, nsc, "mean"), (order, torch.int32, 3 * nsc, "order"),
+            (work, torch.int32, group_plan_work_ints(nsc), "work"),
+            (packed, torch.uint8, mixed_required_bytes(nsc, ring_world), "packed")]
+    if out is not None:
+        need.append((out, src.dtype, n, "out"))
+    if reduced_stats is not None:
+        need.append((reduced_stats, torch.bfloat16, 2 * nsc, "reduced_stats"))
+    if recv is not None:
+        need.append((recv, torch.uint8, 0, "recv"))
+    if hist is not None:
+        need.append((hist, torch.int32, bitrate_hist_ints(), "hist"))
+    if step_dev is not None:
+        need.append((step_dev, torch.int64, 1, "step_dev"))
+    if src.numel() < n:
+        raise RuntimeError("bucket_descriptor: src has fewer than n elements")
+    for t, dt, count, name in need:
+        if t.dtype != dt or t.numel() < count:
+            raise RuntimeError("bucket_descriptor: %s must be %s with at least %d entries" % (name, dt, count))
+    b = Bucket()
+    b.src, b.n, b.dtype, b.strategy = _p(src), n, code, strategy
+    b.center_world, b.ring_chunk, b.ring_world = center_world, ring_chunk, ring_world
+    if isinstance(u, torch.Tensor):
+        if u.dtype != torch.float64 or u.numel() < 1:
+            raise RuntimeError("bucket_descriptor: a tensor u must be float64")
+        b.u, b.u_dev = 0.0, _p(u)
+    else:
+        b.u, b.u_dev = float(u), None
+    b.stats, b.mean, b.reduced_stats = _p(stats), _p(mean), _ptr(reduced_stats) or None
+    b.order, b.work, b.work_ints = _p(order), _p(work), work.numel()
+    b.recv, b.packed, b.packed_bytes = _ptr(recv) or None, _p(packed), packed.numel()
+    b.out = _ptr(out) or None
+    b.hist, b.hist_ints = _ptr(hist) or None, 0 if hist is None else hist.numel()
+    b.seed, b.step, b.step_dev = int(seed) & 0xFFFFFFFFFFFFFFFF, int(step) & 0xFFFFFFFFFFFFFFFF, _ptr(step_dev) or None
+    devices = _seen.devices
+    dev = devices[0]
+    if any(d != dev for d in devices):
+        del devices[:]
+        raise RuntimeError("tensor arguments live on different devices")
+    del devices[:]
+    return b, dev
+
+
+def dynamic_bitrate_bucket(desc, device, stages=STAGE_ALL, stream=None):
+    """one host call for any run of the stages statistics -> plan -> mixed compress -> mixed decompress of one bucket
+    (desc, device: from bucket_descriptor)"""
+    _check(lib().dq_dynamic_bitrate_bucket(ctypes.byref(desc), stages, device, _stream(stream)))
 
 
 def superchunk_stats(src, stats, mean, n, world_size, stream=None):

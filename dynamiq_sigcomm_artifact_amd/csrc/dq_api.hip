@@ -479,6 +479,54 @@ int dq_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, con
                                               strategy == 3, mp, static_cast<hipStream_t>(stream)));
 }
 
+int dq_dynamic_bitrate_bucket(const dq_bucket_t *b, int stages, int device, dq_stream_t stream)
+{
+    if (!b) return fail(DQ_ERR_NULL);
+    if (stages <= 0 || stages > 15) return fail(DQ_ERR_SIZE, "stages must be a combination of DQ_STAGE_*");
+    if (!(b->n > 0)) return fail(DQ_ERR_N);
+    const int64_t nsc = (b->n + 255) / 256;
+    const bool s_stats = stages & DQ_STAGE_STATS, s_plan = stages & DQ_STAGE_PLAN, s_comp = stages & DQ_STAGE_COMPRESS,
+               s_dec = stages & DQ_STAGE_DECOMPRESS;
+    // everything is checked before the first launch
+    int rc = check_mixed(nsc, b->ring_chunk, b->ring_world, b->dtype, b->strategy, false);
+    if (rc) return fail(rc);
+    if (!(b->center_world > 0)) return fail(DQ_ERR_WORLD_SIZE);
+    const void *reduced = b->reduced_stats ? b->reduced_stats : b->stats;
+    if (!b->src && (s_stats || s_comp)) return fail(DQ_ERR_NULL);
+    if (s_stats && (!b->stats || !b->mean)) return fail(DQ_ERR_NULL);
+    if (s_plan) {
+        if (!reduced || !b->order || !b->work) return fail(DQ_ERR_NULL);
+        if (b->work_ints < dq::group_plan_work_ints(nsc)) return fail(DQ_ERR_SIZE, "work buffer is too small");
+        if (b->hist && !b->u_dev) return fail(DQ_ERR_SIZE, "hist is filled by the plan only when u is read from device memory");
+        if (b->hist && b->hist_ints < dq::bitrate_hist_ints()) return fail(DQ_ERR_SIZE, "hist buffer is too small");
+        if (!b->u_dev && b->u != b->u) return fail(DQ_ERR_SIZE, "u must be a number");
+    }
+    if (s_comp || s_dec) {
+        if (!b->order || !b->work || !b->packed) return fail(DQ_ERR_NULL);
+        if (b->packed_bytes < dq::mixed_stream_bytes(nsc, b->ring_world))
+            return fail(DQ_ERR_SIZE, "packed buffer is too small (dq_mixed_required_bytes)");
+    }
+    if (s_comp && !b->mean) return fail(DQ_ERR_NULL);
+    if (s_dec && (!b->out || !reduced)) return fail(DQ_ERR_NULL);
+    if ((rc = select_device(device))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipSuccess;
+    if (s_stats) e = dq::launch_mean_center(b->src, nullptr, b->stats, b->mean, b->n, b->center_world, b->dtype, s);
+    if (e == hipSuccess && s_plan)
+        e = dq::launch_group_plan_stats(reduced, (float)b->u, b->u_dev, nsc, nullptr, b->order, b->work, b->hist, s);
+    if (e == hipSuccess && (s_comp || s_dec)) {
+        const dq::MeeParams mp[3] = {mee_params(8), mee_params(4), mee_params(2)};
+        const dq::RandKey key{b->seed, b->step};
+        if (s_comp)
+            e = dq::launch_mixed_compress(b->src, b->mean, b->center_world, b->n, b->order, b->work, b->ring_chunk, b->ring_world,
+                                          b->recv, b->packed, nullptr, &key, nsc, b->dtype, b->strategy == 3, mp, s, b->step_dev);
+        if (e == hipSuccess && s_dec)
+            e = dq::launch_mixed_decompress(b->packed, b->out, b->order, b->work, b->ring_chunk, b->ring_world, reduced, b->n, nsc,
+                                            b->dtype, b->strategy == 3, mp, s);
+    }
+    return finish(e);
+}
+
 int dq_scaling_compress_philox(const void *src, uint8_t *dst, int64_t n, int nbits, int chunk_size, int dtype, int device,
                                int strategy, uint64_t seed, uint64_t step, dq_stream_t stream)
 {

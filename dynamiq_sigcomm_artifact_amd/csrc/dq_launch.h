@@ -77,12 +77,14 @@ hipError_t launch_bitrate_search(uint32_t *hist, int mode, double prev_u, const 
                                  hipStream_t stream);
 
 // all bit-width groups of a planned bucket in one launch (dq_scaling_mixed.hip); mp: the MEE
-// parameters of 8, 4 and 2 bits in this order
+// parameters of 8, 4 and 2 bits in this order; step_dev (nullable, device memory): a value the kernel adds to
+// philox->step when it runs, so that a recorded launch can draw fresh rounding randomness on every replay
 int64_t mixed_stream_bytes(int64_t nsc, int world);
 hipError_t launch_mixed_compress(const void *src, const float *center_mean, int center_world, int64_t n_valid,
                                  const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world,
                                  const uint8_t *recv, uint8_t *dst, const void *rnd, const RandKey *philox,
-                                 int64_t nsc, int dtype, bool mee, const MeeParams *mp, hipStream_t stream);
+                                 int64_t nsc, int dtype, bool mee, const MeeParams *mp, hipStream_t stream,
+                                 const uint64_t *step_dev = nullptr);
 hipError_t launch_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, const int32_t *counts,
                                    int ring_chunk, int ring_world, const void *stats, int64_t limit, int64_t nsc,
                                    int dtype, bool mee, const MeeParams *mp, hipStream_t stream);

@@ -34,6 +34,7 @@ struct MixedPlan {
     int chunk, world;
     int nsc;               // the counts are clamped so that their sum cannot exceed it
     uint64_t inv40;        // ceil(2^40 / world) when world <= 2^16 and nsc + world < 2^24 (see divide_by_world), else 0
+    const uint64_t *step_dev; // null, or a value in device memory that the encoder adds to the step of its random stream
 };
 
 // world > 1.  With inv40 set, x / world for 0 <= x < 2^24 is (x * inv40) >> 40: inv40 = (2^40 + e) / world with
@@ -47,7 +48,7 @@ __device__ __forceinline__ int divide_by_world(int x, const MixedPlan &p, bool m
 
 static MixedPlan make_plan(const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world, int64_t nsc)
 {
-    MixedPlan p{order, counts, ring_chunk, ring_world, (int)nsc, 0};
+    MixedPlan p{order, counts, ring_chunk, ring_world, (int)nsc, 0, nullptr};
     if (ring_world > 1 && ring_world <= 65536 && nsc + ring_world < (1 << 24))
         p.inv40 = ((uint64_t)1 << 40) / (uint64_t)ring_world + (((uint64_t)1 << 40) % (uint64_t)ring_world ? 1 : 0);
     return p;
@@ -110,6 +111,7 @@ __global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restri
     __shared__ float table[(MEE && FUSED) ? 256 : 1];
     constexpr int RESZ = RDT == DQ_F32 ? 4 : 2;
 
+    if (RDT == DQ_PHILOX && plan.step_dev) key.step += *plan.step_dev; // (a scalar load that leaves with the three counts)
     const Segment s = locate(plan, blockIdx.x, 1);
     if (s.cls == 3) return;
     const RowIds rows = row_ids_plain(plan.order + s.row0);
@@ -217,9 +219,10 @@ int64_t mixed_stream_bytes(int64_t nsc, int world) { return (nsc / world + 3) * 
 hipError_t launch_mixed_compress(const void *src, const float *center_mean, int center_world, int64_t n_valid,
                                  const int32_t *order, const int32_t *counts, int ring_chunk, int ring_world,
                                  const uint8_t *recv, uint8_t *dst, const void *rnd, const RandKey *philox, int64_t nsc,
-                                 int dtype, bool mee, const MeeParams *mp, hipStream_t stream)
+                                 int dtype, bool mee, const MeeParams *mp, hipStream_t stream, const uint64_t *step_dev)
 {
-    const MixedPlan plan = make_plan(order, counts, ring_chunk, ring_world, nsc);
+    MixedPlan plan = make_plan(order, counts, ring_chunk, ring_world, nsc);
+    plan.step_dev = philox ? step_dev : nullptr;
     Center ctr;
     ctr.mean = center_mean;
     ctr.n_valid = n_valid;

@@ -14,6 +14,7 @@
 #include <c10/hip/HIPStream.h>
 
 #include <atomic>
+#include <cstring>
 #include <vector>
 
 #include "dynamiq_eden.h"
@@ -687,6 +688,79 @@ void superchunk_stats(torch::Tensor src, torch::Tensor stats, c10::optional<torc
                  "superchunk_stats");
 }
 
+// One bucket of the dynamic-bitrate path as one call: any run of the stages statistics (1) -> plan (2) -> mixed
+// compress (4) -> mixed decompress (8).  The arguments of a stage that is not asked for are not looked at.
+void dynamic_bitrate_bucket(torch::Tensor src, int64_t n, torch::Tensor stats, torch::Tensor mean, torch::Tensor order,
+                            torch::Tensor work, torch::Tensor packed, c10::optional<torch::Tensor> out, double u,
+                            c10::optional<torch::Tensor> u_dev, int stages = 15, c10::optional<torch::Tensor> reduced_stats = c10::nullopt,
+                            int center_world = 1, int ring_chunk = 0, int ring_world = 1,
+                            c10::optional<torch::Tensor> recv = c10::nullopt, c10::optional<torch::Tensor> hist = c10::nullopt,
+                            uint64_t seed = 0, uint64_t step = 0, c10::optional<torch::Tensor> step_dev = c10::nullopt,
+                            uint64_t stream_p = 0, int strategy = 2)
+{
+    auto dev_ok = [&](const torch::Tensor &t) { return t.device() == src.device() && t.is_contiguous(); };
+    TORCH_CHECK(src.device().type() == torch::kCUDA, "input must be a CUDA tensor");
+    TORCH_CHECK(src.scalar_type() == torch::kBFloat16 || src.scalar_type() == torch::kFloat32, "input must be torch.bfloat16 or torch.float32");
+    TORCH_CHECK(src.is_contiguous(), "buffers must be contiguous");
+    TORCH_CHECK(n > 0 && src.numel() >= n, "n must be positive and at most the number of input elements");
+    TORCH_CHECK(strategy == 2 || strategy == 3, "strategy must be 2 or 3");
+    TORCH_CHECK(stages > 0 && stages <= 15, "stages must be a combination of 1 (statistics), 2 (plan), 4 (compress), 8 (decompress)");
+    TORCH_CHECK(ring_world > 0 && ring_chunk >= 0 && ring_chunk < ring_world, "ring_chunk must lie in [0, ring_world)");
+    TORCH_CHECK(center_world > 0, "center_world must be positive");
+    const int64_t nsc = (n + 255) / 256;
+    TORCH_CHECK(dev_ok(stats) && stats.dtype() == torch::kBFloat16 && stats.numel() >= 2 * nsc, "stats must be a contiguous torch.bfloat16 tensor with a (mean, norm) pair per superchunk on the device of the input");
+    TORCH_CHECK(dev_ok(mean) && mean.dtype() == torch::kFloat32 && mean.numel() >= nsc, "mean must be a contiguous torch.float32 tensor with one entry per superchunk on the device of the input");
+    TORCH_CHECK(dev_ok(order) && order.dtype() == torch::kInt32 && order.numel() >= 3 * nsc, "order must be a contiguous torch.int32 tensor with 3 * nsc entries on the device of the input");
+    TORCH_CHECK(dev_ok(work) && work.dtype() == torch::kInt32 && work.numel() >= dq_group_plan_work_ints(nsc), "work must be a contiguous torch.int32 tensor with group_plan_work_ints(nsc) entries on the device of the input");
+    TORCH_CHECK(dev_ok(packed) && packed.dtype() == torch::kUInt8 && packed.numel() >= dq_mixed_required_bytes(nsc, ring_world), "packed must be a contiguous torch.uint8 tensor of mixed_required_bytes(nsc, ring_world) bytes on the device of the input");
+    dq_bucket_t b;
+    memset(&b, 0, sizeof(b));
+    b.src = src.data_ptr();
+    b.n = n;
+    b.dtype = dq_dtype_of(src.scalar_type());
+    b.strategy = strategy;
+    b.center_world = center_world;
+    b.ring_chunk = ring_chunk;
+    b.ring_world = ring_world;
+    b.u = u;
+    if (u_dev.has_value()) {
+        TORCH_CHECK(dev_ok(*u_dev) && u_dev->dtype() == torch::kFloat64 && u_dev->numel() >= 1, "u_dev must be a torch.float64 tensor on the device of the input");
+        b.u_dev = u_dev->data_ptr<double>();
+    }
+    b.stats = stats.data_ptr();
+    b.mean = mean.data_ptr<float>();
+    if (reduced_stats.has_value()) {
+        TORCH_CHECK(dev_ok(*reduced_stats) && reduced_stats->dtype() == torch::kBFloat16 && reduced_stats->numel() >= 2 * nsc, "reduced_stats must be a contiguous torch.bfloat16 tensor like stats");
+        b.reduced_stats = reduced_stats->data_ptr();
+    }
+    b.order = order.data_ptr<int32_t>();
+    b.work = work.data_ptr<int32_t>();
+    b.work_ints = work.numel();
+    if (recv.has_value()) {
+        TORCH_CHECK(dev_ok(*recv) && recv->dtype() == torch::kUInt8 && recv->numel() >= dq_mixed_required_bytes(nsc, ring_world), "recv must be a contiguous torch.uint8 tensor of mixed_required_bytes(nsc, ring_world) bytes");
+        b.recv = recv->data_ptr<uint8_t>();
+    }
+    b.packed = packed.data_ptr<uint8_t>();
+    b.packed_bytes = packed.numel();
+    if (out.has_value()) {
+        TORCH_CHECK(dev_ok(*out) && out->dtype() == src.dtype() && out->numel() >= n, "out must be a contiguous tensor of the input's dtype with at least n elements");
+        b.out = out->data_ptr();
+    }
+    TORCH_CHECK(!(stages & 8) || out.has_value(), "the decompress stage needs out");
+    if (hist.has_value()) {
+        TORCH_CHECK(dev_ok(*hist) && hist->dtype() == torch::kInt32 && hist->numel() >= dq_bitrate_hist_ints(), "hist must be a contiguous torch.int32 tensor with bitrate_hist_ints() entries");
+        b.hist = reinterpret_cast<uint32_t *>(hist->data_ptr<int32_t>());
+        b.hist_ints = hist->numel();
+    }
+    b.seed = seed;
+    b.step = step;
+    if (step_dev.has_value()) {
+        TORCH_CHECK(dev_ok(*step_dev) && step_dev->dtype() == torch::kInt64 && step_dev->numel() >= 1, "step_dev must be a torch.int64 tensor on the device of the input");
+        b.step_dev = reinterpret_cast<const uint64_t *>(step_dev->data_ptr<int64_t>());
+    }
+    check_status(dq_dynamic_bitrate_bucket(&b, stages, src.device().index(), as_stream(stream_p)), "dynamic_bitrate_bucket");
+}
+
 // ---- superchunk ops ---------------------------------------------------------------
 
 void superchunk_mean_center(torch::Tensor src, torch::Tensor residual, torch::Tensor stats, int n, int world_size,
@@ -1023,6 +1097,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, modul)
     modul.def("mixed_required_bytes", &mixed_required_bytes, "upper bound of the packed stream of one ring chunk over the three bit-width groups", py::arg("nsc"), py::arg("ring_world") = 1);
     modul.def("mixed_compress", &mixed_compress, "compress (or, with recv, decode-accumulate-recompress) ring chunk ring_chunk of all three bit-width groups of a planned bucket in one launch", py::arg("src"), py::arg("order"), py::arg("counts"), py::arg("dst"), py::arg("nsc"), py::arg("rand_pool") = py::none(), py::arg("recv") = py::none(), py::arg("center_mean") = py::none(), py::arg("center_world") = 1, py::arg("n") = 0, py::arg("ring_chunk") = 0, py::arg("ring_world") = 1, py::arg("seed") = 0, py::arg("step") = 0, py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("mixed_decompress", &mixed_decompress, "decode ring chunk ring_chunk of all three bit-width groups into their superchunks of dst, optionally adding the per-superchunk mean", py::arg("src"), py::arg("dst"), py::arg("order"), py::arg("counts"), py::arg("nsc"), py::arg("stats"), py::arg("n_limit"), py::arg("ring_chunk") = 0, py::arg("ring_world") = 1, py::arg("stream_p") = 0, py::arg("strategy") = 2);
+    modul.def("dynamic_bitrate_bucket", &dynamic_bitrate_bucket, "one bucket of the dynamic-bitrate path in one call: any run of the stages statistics (1), plan (2), mixed compress (4), mixed decompress (8)", py::arg("src"), py::arg("n"), py::arg("stats"), py::arg("mean"), py::arg("order"), py::arg("work"), py::arg("packed"), py::arg("out"), py::arg("u") = 0.0, py::arg("u_dev") = py::none(), py::arg("stages") = 15, py::arg("reduced_stats") = py::none(), py::arg("center_world") = 1, py::arg("ring_chunk") = 0, py::arg("ring_world") = 1, py::arg("recv") = py::none(), py::arg("hist") = py::none(), py::arg("seed") = 0, py::arg("step") = 0, py::arg("step_dev") = py::none(), py::arg("stream_p") = 0, py::arg("strategy") = 2);
     modul.def("superchunk_stats", &superchunk_stats, "the statistics of superchunk_mean_center without the residual, plus the unrounded float32 means", py::arg("src"), py::arg("stats"), py::arg("mean"), py::arg("n"), py::arg("world_size"), py::arg("stream_p") = 0);
     modul.def("scaling_compress_philox", &scaling_compress_philox, "scaling compress with the uniform values drawn in the kernel (Philox: key = seed, counter = chunk, step)", py::arg("src"), py::arg("dst"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0, py::arg("strategy") = 0);
     modul.def("scaling_dec_comp_philox", &scaling_dec_comp_philox, "scaling decompress and compress with the uniform values drawn in the kernel", py::arg("recv"), py::arg("inp"), py::arg("send"), py::arg("n"), py::arg("nbits"), py::arg("chunk_size"), py::arg("seed"), py::arg("step"), py::arg("stream_p") = 0, py::arg("strategy") = 0);

@@ -291,3 +291,137 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
         for r in range(W):
             decode(r, bufs[(step ^ 1) & 1][r], (r - step + W) % W)
     return outs, total, plan[:4]
+
+
+class SinglePassBuckets(object):
+    """The single-pass dynamic-bitrate path for a stream of buckets on one rank (a ring of one: statistics, widths,
+    partition, encode, decode, mean add -- what dynamic_bitrate_allreduce_single_pass does for W = 1), shaped for
+    25 MB buckets, where the four kernels of a bucket take about as long as four host calls and every launch waits
+    for the one before:
+
+      * one host call per bucket (capi.dynamic_bitrate_bucket) instead of four;
+      * with ``graphs=True`` the four launches of a (source, output) pair are captured once and replayed, so the host
+        cost per bucket is one graph launch.  DDP hands the hook the same bucket views on every step, so the pair is
+        the natural key; a replay reads whatever the source holds then;
+      * ``streams`` buckets are in flight at a time, each on a stream of its own with scratch of its own (statistics,
+        means, plan, packed stream): the latency-bound statistics and plan launches of one bucket overlap the codec
+        launches of its neighbour.
+
+    The offset u of the width rule is read from device memory when the plan runs (``set_u`` or a float64 tensor of the
+    caller's, e.g. the result of the offset search), and the rounding stream of the encoder is (seed, bucket ordinal *
+    2^32 + the step counter in device memory): ``begin_step`` advances the counter once per training step, so a
+    replayed launch draws fresh random values on every step.
+
+    run(x, out) enqueues a bucket and returns at once; join() makes the caller's current stream wait for everything
+    enqueued so far.  The caller must not overwrite x or read out before join()."""
+
+    def __init__(self, device, strategy=2, seed=0, streams=2, graphs=True, u=None, norm_histogram=None):
+        from . import capi
+        self.capi = capi
+        self.device = torch.device(device)
+        self.strategy, self.seed, self.graphs = strategy, int(seed), graphs
+        self.streams = [torch.cuda.Stream(device=self.device) for _ in range(max(1, int(streams)))]
+        self.scratch = [dict() for _ in self.streams]
+        self.pending = [False] * len(self.streams)
+        self.step_dev = torch.zeros(1, dtype=torch.int64, device=self.device)
+        self.u_dev = u if isinstance(u, torch.Tensor) else torch.full((1,), 60.0 if u is None else float(u), dtype=torch.float64,
+                                                                     device=self.device)
+        self.hist = norm_histogram
+        self.cache = {}          # (x.data_ptr(), out.data_ptr(), n, dtype, stream index) -> (descriptor, device, graph, ordinal)
+        self.ordinals = {}       # (x.data_ptr(), n) -> ordinal of the bucket in the random stream
+        self.superchunks = 0
+
+    # ---- once per training step ----------------------------------------------------------------------------
+    def set_u(self, u):
+        """the offset of the width rule for the buckets enqueued from now on (a number; a tensor was given at construction)"""
+        cur = torch.cuda.current_stream(self.device)
+        for k, st in enumerate(self.streams):
+            if self.pending[k]:
+                cur.wait_stream(st)
+        self.u_dev.fill_(float(u))
+        self._fence = torch.cuda.Event()
+        self._fence.record(cur)
+        for st in self.streams:
+            st.wait_event(self._fence)
+
+    def begin_step(self):
+        """advance the step counter of the rounding stream (one small kernel per training step)"""
+        cur = torch.cuda.current_stream(self.device)
+        for k, st in enumerate(self.streams):
+            if self.pending[k]:
+                cur.wait_stream(st)
+        self.step_dev.add_(1)
+        ev = torch.cuda.Event()
+        ev.record(cur)
+        for st in self.streams:
+            st.wait_event(ev)
+
+    # ---- per bucket ---------------------------------------------------------------------------------------------
+    def _scratch(self, k, nsc):
+        sc = self.scratch[k]
+        if sc.get("nsc", 0) < nsc:
+            capi, dev = self.capi, self.device
+            sc["nsc"] = nsc
+            sc["stats"] = torch.empty((nsc, 2), dtype=torch.bfloat16, device=dev)
+            sc["mean"] = torch.empty(nsc, dtype=torch.float32, device=dev)
+            sc["order"] = torch.empty(3 * nsc, dtype=torch.int32, device=dev)
+            sc["work"] = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
+            sc["packed"] = torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=dev)
+            # scratch of another size invalidates what was recorded against the old buffers
+            for key in [key for key in self.cache if key[4] == k]:
+                del self.cache[key]
+        return sc
+
+    def run(self, x, out):
+        """enqueue one bucket: out = decode(encode(x)) with the widths of its reduced norms; returns the index of the
+        stream it went to"""
+        capi = self.capi
+        n = x.numel()
+        nsc = (n + 255) // 256
+        # a source keeps its ordinal, and with it its stream and its recorded launches, from step to step
+        ordinal = self.ordinals.setdefault((x.data_ptr(), n), len(self.ordinals))
+        k = ordinal % len(self.streams)
+        st = self.streams[k]
+        key = (x.data_ptr(), out.data_ptr(), n, x.dtype, k)
+        entry = self.cache.get(key)
+        if entry is None:
+            sc = self._scratch(k, nsc)
+            desc, dev = capi.bucket_descriptor(x, n, sc["stats"][:nsc], sc["mean"], sc["order"], sc["work"], sc["packed"],
+                                               strategy=self.strategy, out=out, u=self.u_dev,
+                                               hist=None if self.hist is None else self.hist.hist, seed=self.seed,
+                                               step=ordinal << 32, step_dev=self.step_dev)
+            # (the first use of a pair runs eagerly, the second records the graph that later uses replay: a pair seen
+            # once costs no capture)
+            entry = [desc, dev, None, 0]
+            self.cache[key] = entry
+        desc, dev, graph, uses = entry
+        st.wait_stream(torch.cuda.current_stream(self.device))
+        if graph is not None:
+            with torch.cuda.stream(st):
+                graph.replay()
+        elif self.graphs and uses >= 1:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(st):
+                with torch.cuda.graph(graph, stream=st):
+                    capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
+                graph.replay()
+            entry[2] = graph
+        else:
+            capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
+        entry[3] = uses + 1
+        self.pending[k] = True
+        if self.hist is not None:
+            self.hist.count += nsc
+        self.superchunks += nsc
+        return k
+
+    def counts(self, k):
+        """device int32 tensor [n8, n4, n2, other] of the last bucket that ran on stream k"""
+        return self.scratch[k]["work"][:4]
+
+    def join(self):
+        cur = torch.cuda.current_stream(self.device)
+        for k, st in enumerate(self.streams):
+            if self.pending[k]:
+                cur.wait_stream(st)
+                self.pending[k] = False

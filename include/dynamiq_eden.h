@@ -316,6 +316,60 @@ int dq_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, con
 int dq_superchunk_stats(const void *src, void *stats, float *mean, int64_t n, int world_size,
                         int dtype, int device, dq_stream_t stream);
 
+/* ---- one bucket of the dynamic-bitrate path in one host call --------------
+ *
+ * The reference's hook runs a bucket as a sequence of Python-level steps
+ * (comm_hooks.py:932-1024: superchunk_mean_center, the stats all-reduce, the
+ * width rule, three nonzero / index_select / ring / index_copy_ rounds,
+ * superchunk_add_mean_copy).  With the calls above the same bucket is four
+ * launches -- dq_superchunk_stats, dq_group_plan_stats(_dev_u),
+ * dq_mixed_compress, dq_mixed_decompress -- and on a 25 MB bucket the host's
+ * cost of four calls is as long as the kernels.  dq_dynamic_bitrate_bucket
+ * enqueues any run of these stages for one bucket with one call; the stages,
+ * their arguments and their results are exactly those of the four calls.
+ *
+ *   DQ_STAGE_STATS       src -> stats (bf16 pairs), mean (binary32)   [dq_superchunk_stats, world = center_world]
+ *   DQ_STAGE_PLAN        reduced_stats (or stats when NULL), u or *u_dev -> order, work[0..3] (+ hist)
+ *   DQ_STAGE_COMPRESS    src centred on load with mean -> packed: ring chunk ring_chunk of ring_world, recv != NULL =
+ *                        the fused ring step; in-kernel rounding stream (seed, step + *step_dev)
+ *   DQ_STAGE_DECOMPRESS  packed -> out (+ the mean of reduced_stats), elements below n
+ *
+ * A ring of one rank (or a rank's local round trip) runs all four at once; in
+ * a ring of several ranks the stats all-reduce sits between STATS and PLAN and
+ * the exchanges between the codec stages, so a rank calls it once per run of
+ * consecutive stages.  step_dev (may be NULL): one uint64 in device memory that
+ * the encoder adds to `step` when it runs -- a launch recorded into a HIP graph
+ * then draws fresh rounding randomness on every replay if the owner advances
+ * that counter between replays.  No counterpart in the reference. */
+enum { DQ_STAGE_STATS = 1, DQ_STAGE_PLAN = 2, DQ_STAGE_COMPRESS = 4, DQ_STAGE_DECOMPRESS = 8 };
+
+typedef struct dq_bucket {
+    const void *src;            /* n elements of dtype (DQ_BF16 or DQ_F32) */
+    int64_t n;
+    int32_t dtype, strategy;    /* strategy 2 (AEE) or 3 (MEE) */
+    int32_t center_world;       /* the divisor of superchunk_mean_center */
+    int32_t ring_chunk, ring_world;
+    int32_t reserved;
+    double u;                   /* offset of the width rule, used when u_dev == NULL */
+    const double *u_dev;        /* ... or read from device memory when the plan runs */
+    void *stats;                /* bf16 [nsc, 2], nsc = ceil(n / 256): written by STATS */
+    float *mean;                /* float [nsc]: written by STATS, read by COMPRESS */
+    const void *reduced_stats;  /* the stats after the all-reduce; NULL = stats */
+    int32_t *order;             /* int32 [3 nsc] */
+    int32_t *work;              /* int32 [work_ints], work_ints >= dq_group_plan_work_ints(nsc) */
+    int64_t work_ints;
+    const uint8_t *recv;        /* may be NULL */
+    uint8_t *packed;            /* packed_bytes >= dq_mixed_required_bytes(nsc, ring_world) */
+    int64_t packed_bytes;
+    void *out;                  /* n elements of dtype: written by DECOMPRESS */
+    uint32_t *hist;             /* may be NULL; with u_dev only (see dq_group_plan_stats_dev_u) */
+    int64_t hist_ints;
+    uint64_t seed, step;
+    const uint64_t *step_dev;   /* may be NULL */
+} dq_bucket_t;
+
+int dq_dynamic_bitrate_bucket(const dq_bucket_t *bucket, int stages, int device, dq_stream_t stream);
+
 /* ---- consumers of the rotated vector: EDEN and THC ----------------------
  *
  * "reference" here: cuda_kernels/src/srrcomp/srrcomp.py (EDEN) and

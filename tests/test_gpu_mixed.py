@@ -450,3 +450,112 @@ def test_mixed_random_shapes(capi, block):
                 capi.scaling_dec_comp_rows(e, peer, rows, s, rnd, cnt, width, strategy)
                 assert torch.equal(enc[off:off + nb], e), tag + (chunk, width)
                 assert torch.equal(send[off:off + nb], s), tag + (chunk, width)
+
+
+def _llama_like(n, seed, dt=torch.bfloat16):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    nsc = (n + 255) // 256
+    scales = torch.exp(torch.randn(nsc, 1, generator=g, device=DEV) * 6.0) * 1e-3
+    return ((torch.randn(nsc, 256, generator=g, device=DEV) * scales).reshape(-1)[:n] + 1e-4).to(dt)
+
+
+def _four_calls(capi, x, n, u, strategy, seed, step, world=1):
+    nsc = (n + 255) // 256
+    stats = torch.zeros((nsc, 2), dtype=torch.bfloat16, device=DEV)
+    mean = torch.zeros(nsc, dtype=torch.float32, device=DEV)
+    order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    packed = torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=DEV)
+    out = torch.zeros_like(x)
+    capi.superchunk_stats(x, stats, mean, n, world)
+    capi.group_plan_stats(stats, u, None, order, work)
+    capi.mixed_compress(x, order, work, packed, nsc, strategy, seed=seed, step=step, center_mean=mean, center_world=world, n=n)
+    capi.mixed_decompress(packed, out, order, work, nsc, strategy, stats=stats, n_limit=n)
+    return stats, mean, order, work, packed, out
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_bucket_call_equals_the_four_calls(capi, eden_utils, dt, strategy):
+    """dq_dynamic_bitrate_bucket enqueues statistics -> plan -> mixed compress -> mixed decompress with one host call: every
+    buffer it writes equals what the four calls write, for all stages at once, for the stages one by one, with u in
+    device memory, through ctypes and through the module; step_dev adds to the step of the rounding stream"""
+    n, u, seed, step = 256 * 700 - 131, 6.0, 11, 5
+    nsc = (n + 255) // 256
+    x = _llama_like(n, 3, dt)
+    ref = _four_calls(capi, x, n, u, strategy, seed, step)
+    assert min(ref[3][:3].tolist()) > 0
+
+    def fresh():
+        return (torch.zeros((nsc, 2), dtype=torch.bfloat16, device=DEV), torch.zeros(nsc, dtype=torch.float32, device=DEV),
+                torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV),
+                torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV),
+                torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=DEV), torch.zeros_like(x))
+
+    def same(got):
+        counts = ref[3][:3].tolist()
+        used = sum(c * r for c, r in zip(counts, (274, 146, 82)))
+        assert torch.equal(bits_t(got[0]), bits_t(ref[0])) and torch.equal(bits_t(got[1]), bits_t(ref[1]))
+        assert got[3][:4].tolist() == ref[3][:4].tolist()
+        for g_, c in enumerate(counts):
+            assert torch.equal(got[2][g_ * nsc:g_ * nsc + c], ref[2][g_ * nsc:g_ * nsc + c])
+        assert torch.equal(got[4][:used], ref[4][:used])
+        assert torch.equal(bits_t(got[5]), bits_t(ref[5]))
+
+    # all stages, u a number
+    bufs = fresh()
+    desc, dev = capi.bucket_descriptor(x, n, *bufs[:5], strategy=strategy, out=bufs[5], u=u, seed=seed, step=step)
+    capi.dynamic_bitrate_bucket(desc, dev)
+    same(bufs)
+    # stage by stage, u and the step offset in device memory
+    bufs = fresh()
+    u_dev = torch.full((1,), u, dtype=torch.float64, device=DEV)
+    step_dev = torch.full((1,), 3, dtype=torch.int64, device=DEV)
+    desc, dev = capi.bucket_descriptor(x, n, *bufs[:5], strategy=strategy, out=bufs[5], u=u_dev, seed=seed, step=step - 3,
+                                       step_dev=step_dev)
+    for stage in (capi.STAGE_STATS, capi.STAGE_PLAN, capi.STAGE_COMPRESS, capi.STAGE_DECOMPRESS):
+        capi.dynamic_bitrate_bucket(desc, dev, stages=stage)
+    same(bufs)
+    # another value of the device-side step: other random values, other bytes
+    step_dev.fill_(4)
+    capi.dynamic_bitrate_bucket(desc, dev, stages=capi.STAGE_COMPRESS)
+    assert not torch.equal(bufs[4], ref[4])
+    # the module's twin
+    bufs = fresh()
+    eden_utils.dynamic_bitrate_bucket(x, n, *bufs[:5], bufs[5], u=u, seed=seed, step=step, strategy=strategy,
+                                      stream_p=torch.cuda.current_stream().cuda_stream)
+    same(bufs)
+    # refusals come before any launch
+    with pytest.raises(RuntimeError):
+        capi.bucket_descriptor(x, n, bufs[0], bufs[1], bufs[2], bufs[3], bufs[4][:100], strategy=strategy)
+    bad, dev = capi.bucket_descriptor(x, n, *bufs[:5], strategy=strategy, out=None, u=u)
+    with pytest.raises(RuntimeError):
+        capi.dynamic_bitrate_bucket(bad, dev)                     # the decode stage without an output
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("streams,graphs", [(1, False), (2, True), (3, True)])
+def test_single_pass_buckets_object(capi, streams, graphs):
+    """a stream of buckets through the pipeline object -- one host call per bucket, recorded once per (source, output)
+    pair and replayed, several buckets in flight on streams of their own -- gives, on every training step, the outputs of
+    the four calls with the rounding stream (seed, bucket ordinal * 2^32 + step)"""
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import SinglePassBuckets
+    sizes = [256 * 123, 256 * 300, 256 * 300 - 5, 256 * 300, 256 * 77 + 1]      # (a later, larger bucket makes a stream's scratch grow)
+    xs = [_llama_like(n, 40 + k) for k, n in enumerate(sizes)]
+    outs = [torch.zeros_like(x) for x in xs]
+    seed, u = 9, 6.0
+    pipe = SinglePassBuckets(DEV, strategy=2, seed=seed, streams=streams, graphs=graphs, u=u)
+    for step in range(1, 5):
+        if step == 3:
+            u = 7.5
+            pipe.set_u(u)
+        pipe.begin_step()
+        for x in xs:
+            x.mul_(1.25)                      # the sources change between steps; a replay must read the new values
+        for x, o in zip(xs, outs):
+            pipe.run(x, o)
+        pipe.join()
+        torch.cuda.synchronize()
+        for k, (x, o) in enumerate(zip(xs, outs)):
+            want = _four_calls(capi, x, x.numel(), u, 2, seed, (k << 32) + step)[5]
+            assert torch.equal(bits_t(o), bits_t(want)), (step, k)
