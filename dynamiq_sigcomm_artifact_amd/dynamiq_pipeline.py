@@ -299,13 +299,15 @@ class SinglePassBuckets(object):
     25 MB buckets, where the four kernels of a bucket take about as long as four host calls and every launch waits
     for the one before:
 
-      * one host call per bucket (capi.dynamic_bitrate_bucket) instead of four;
-      * with ``graphs=True`` the four launches of a (source, output) pair are captured once and replayed, so the host
-        cost per bucket is one graph launch.  DDP hands the hook the same bucket views on every step, so the pair is
-        the natural key; a replay reads whatever the source holds then;
+      * one host call per bucket (capi.dynamic_bitrate_bucket) instead of four (``run``);
       * ``streams`` buckets are in flight at a time, each on a stream of its own with scratch of its own (statistics,
         means, plan, packed stream): the latency-bound statistics and plan launches of one bucket overlap the codec
-        launches of its neighbour.
+        launches of its neighbour;
+      * with ``graphs=True``, ``run_all`` records a whole step's buckets once -- one graph per stream -- and replays
+        them: one graph launch per stream and step instead of one host call per bucket.  DDP hands the hook the same
+        bucket views on every step, so the list of (source, output) pairs is the natural key; a replay reads whatever
+        the sources hold then.  (A graph per bucket was measured and is slower than the eager call: launching a graph
+        costs the host more than one call that enqueues four kernels.)
 
     The offset u of the width rule is read from device memory when the plan runs (``set_u`` or a float64 tensor of the
     caller's, e.g. the result of the offset search), and the rounding stream of the encoder is (seed, bucket ordinal *
@@ -368,7 +370,7 @@ class SinglePassBuckets(object):
             sc["work"] = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=dev)
             sc["packed"] = torch.zeros(capi.mixed_required_bytes(nsc, 1), dtype=torch.uint8, device=dev)
             # scratch of another size invalidates what was recorded against the old buffers
-            for key in [key for key in self.cache if key[4] == k]:
+            for key in [key for key in self.cache if key[0] == "step" or key[4] == k]:
                 del self.cache[key]
         return sc
 
@@ -390,30 +392,68 @@ class SinglePassBuckets(object):
                                                strategy=self.strategy, out=out, u=self.u_dev,
                                                hist=None if self.hist is None else self.hist.hist, seed=self.seed,
                                                step=ordinal << 32, step_dev=self.step_dev)
-            # (the first use of a pair runs eagerly, the second records the graph that later uses replay: a pair seen
-            # once costs no capture)
             entry = [desc, dev, None, 0]
             self.cache[key] = entry
-        desc, dev, graph, uses = entry
+        desc, dev = entry[0], entry[1]
         st.wait_stream(torch.cuda.current_stream(self.device))
-        if graph is not None:
-            with torch.cuda.stream(st):
-                graph.replay()
-        elif self.graphs and uses >= 1:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.stream(st):
-                with torch.cuda.graph(graph, stream=st):
-                    capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
-                graph.replay()
-            entry[2] = graph
-        else:
-            capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
-        entry[3] = uses + 1
+        capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
         self.pending[k] = True
         if self.hist is not None:
             self.hist.count += nsc
         self.superchunks += nsc
         return k
+
+    def run_all(self, pairs):
+        """enqueue a whole step's buckets, [(x, out), ...].  A list that has been seen before (the same tensors in the
+        same order: DDP's buckets) is replayed from one recorded graph per stream -- one graph launch per stream and
+        step instead of one host call per bucket; the first time it runs bucket by bucket, the second time it records."""
+        key = tuple((x.data_ptr(), o.data_ptr(), x.numel(), x.dtype) for x, o in pairs)
+        entry = self.cache.get(("step", key))
+        cur = torch.cuda.current_stream(self.device)
+        if entry is None or not self.graphs:
+            for x, o in pairs:
+                self.run(x, o)
+            if entry is None:
+                self.cache[("step", key)] = [None, 1]
+            return
+        graphs, uses = entry
+        if graphs is None:
+            # per stream: the buckets that go to it, in order, recorded as one graph
+            share = [[] for _ in self.streams]
+            for x, o in pairs:
+                n = x.numel()
+                ordinal = self.ordinals.setdefault((x.data_ptr(), n), len(self.ordinals))
+                k = ordinal % len(self.streams)
+                item = self.cache.get((x.data_ptr(), o.data_ptr(), n, x.dtype, k))
+                if item is None:                # (cannot happen after a first eager pass with unchanged scratch)
+                    self.run(x, o)
+                    item = self.cache[(x.data_ptr(), o.data_ptr(), n, x.dtype, k)]
+                share[k].append(item)
+            self.join()
+            graphs = []
+            for k, st in enumerate(self.streams):
+                if not share[k]:
+                    graphs.append(None)
+                    continue
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(st):
+                    with torch.cuda.graph(g, stream=st):
+                        for desc, dev, _, _ in share[k]:
+                            self.capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
+                graphs.append(g)
+            entry[0] = graphs
+        for k, st in enumerate(self.streams):
+            if graphs[k] is None:
+                continue
+            st.wait_stream(cur)
+            with torch.cuda.stream(st):
+                graphs[k].replay()
+            self.pending[k] = True
+        entry[1] = uses + 1
+        total = sum((x.numel() + 255) // 256 for x, _ in pairs)
+        if self.hist is not None:
+            self.hist.count += total
+        self.superchunks += total
 
     def counts(self, k):
         """device int32 tensor [n8, n4, n2, other] of the last bucket that ran on stream k"""

@@ -534,26 +534,30 @@ def test_bucket_call_equals_the_four_calls(capi, eden_utils, dt, strategy):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("streams,graphs", [(1, False), (2, True), (3, True)])
-def test_single_pass_buckets_object(capi, streams, graphs):
-    """a stream of buckets through the pipeline object -- one host call per bucket, recorded once per (source, output)
-    pair and replayed, several buckets in flight on streams of their own -- gives, on every training step, the outputs of
-    the four calls with the rounding stream (seed, bucket ordinal * 2^32 + step)"""
+@pytest.mark.parametrize("streams,graphs,whole", [(1, False, False), (2, False, False), (2, True, True), (3, True, True),
+                                                  (2, False, True)])
+def test_single_pass_buckets_object(capi, streams, graphs, whole):
+    """a stream of buckets through the pipeline object -- one host call per bucket, or a whole step recorded once and
+    replayed (one graph per stream), several buckets in flight on streams of their own -- gives, on every training step,
+    the outputs of the four calls with the rounding stream (seed, bucket ordinal * 2^32 + step)"""
     from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import SinglePassBuckets
     sizes = [256 * 123, 256 * 300, 256 * 300 - 5, 256 * 300, 256 * 77 + 1]      # (a later, larger bucket makes a stream's scratch grow)
     xs = [_llama_like(n, 40 + k) for k, n in enumerate(sizes)]
     outs = [torch.zeros_like(x) for x in xs]
     seed, u = 9, 6.0
     pipe = SinglePassBuckets(DEV, strategy=2, seed=seed, streams=streams, graphs=graphs, u=u)
-    for step in range(1, 5):
-        if step == 3:
+    for step in range(1, 6):
+        if step == 4:
             u = 7.5
             pipe.set_u(u)
         pipe.begin_step()
         for x in xs:
             x.mul_(1.25)                      # the sources change between steps; a replay must read the new values
-        for x, o in zip(xs, outs):
-            pipe.run(x, o)
+        if whole:
+            pipe.run_all(list(zip(xs, outs)))
+        else:
+            for x, o in zip(xs, outs):
+                pipe.run(x, o)
         pipe.join()
         torch.cuda.synchronize()
         for k, (x, o) in enumerate(zip(xs, outs)):
