@@ -22,8 +22,7 @@
 // left: small tiles, strided passes over fewer than four bits, buffers without
 // 16-byte alignment.  Either kind can take a quantiser at the ends of the transform
 // (THC's levels, EDEN's bit planes and scale).  The LDS index is
-// padded by one float per 16 (i + i/16), which keeps every access pattern used
-// here free of bank conflicts.
+// padded by one float per 32 (dq_fwht.cuh).
 #include "dq_fwht.cuh"
 #include "dq_launch.h"
 
@@ -104,7 +103,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
     if (a.in_planes) {
         // sixteen consecutive bins per thread from its half word of every plane (two 8 x 8 bit transposes), their
         // centroids into one padded group of the tile; the centroid table sits behind the tile
-        float *cen = lds + tile + tile / 16 + 1;
+        float *cen = lds + padded_floats(tile);
         for (int k = tid; k < (1 << a.in_nbits); k += nthreads) cen[k] = a.in_centroids[k];
         __syncthreads();
         for (int i = tid * 16; i < tile; i += nthreads * 16) {
@@ -143,7 +142,7 @@ __global__ void fwht_tile_kernel(FwhtArgs a)
                 }
                 if (a.sign_mode == 1) apply_sign4(a, v, g);
             }
-            const int q = pad_idx(i); // i % 4 == 0: the four floats stay inside one padded group of 16
+            const int q = pad_idx(i); // i % 4 == 0: the four floats stay inside one padded group
             lds[q] = v.x; lds[q + 1] = v.y; lds[q + 2] = v.z; lds[q + 3] = v.w;
         }
     } else {
@@ -212,7 +211,7 @@ static hipError_t launch_tile(const FwhtArgs &a, int64_t ntiles, hipStream_t str
     const int tile = 1 << a.kt;
     int threads = tile / 16;
     threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
-    const size_t lds_bytes = (size_t)(tile + tile / 16 + 1 + (a.in_planes ? 256 : 0)) * sizeof(float);
+    const size_t lds_bytes = (size_t)(padded_floats(tile) + (a.in_planes ? 256 : 0)) * sizeof(float);
     if (lds_bytes > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(fwht_tile_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);

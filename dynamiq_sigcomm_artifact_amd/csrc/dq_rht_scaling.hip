@@ -7,9 +7,9 @@
 // workgroup: a workgroup owns a tile of 2^kt consecutive floats (whole transform blocks of up to 2^15) in
 // LDS.  One lane owns one chunk of 16 consecutive floats at both ends: it loads the chunk (64 bytes), flips
 // the signs and does the stages of strides 1..8 on its registers, the remaining stages run as LDS passes of
-// up to five stages each, and the lane then reads its chunk back and quantises it.  With the LDS index padded
-// by one float per 16 a chunk is 16 consecutive words and neighbouring lanes are 17 words apart, so these
-// accesses are free of bank conflicts.  The inverse kernel decodes records into registers, does the first
+// up to five stages each, and the lane then reads its chunk back and quantises it.  The LDS index is padded by
+// one float per 32 (dq_fwht.cuh): the chunk-wise accesses, the passes and the coalesced stores are then all free
+// of bank conflicts.  The inverse kernel decodes records into registers, does the first
 // stages there, finishes in LDS and stores fp32 with coalesced 16-byte stores.
 //
 // Results are bit for bit those of the two-call sequences: the butterflies run in the same order
@@ -98,11 +98,7 @@ __device__ __forceinline__ void load_chunk(float (&v)[16], const float *__restri
 }
 
 // floats of LDS holding the padded tile, rounded up so that what follows is 16-byte aligned
-__host__ __device__ inline int padded_tile_floats(int kt)
-{
-    const int tile = 1 << kt;
-    return (tile + tile / 16 + 1 + 3) & ~3;
-}
+__host__ __device__ inline int padded_tile_floats(int kt) { return padded_floats(1 << kt); }
 
 // The stages of strides 1..8 of 64 chunks as one matrix product on the matrix cores: Y = X H16, X the wave's 64 x 16
 // block of chunks, H16[i][j] = (-1)^popcount(i & j).  v_mfma_f32_16x16x4_f32 takes a 16 x 4 slice of X (lane l: row
@@ -131,7 +127,7 @@ __device__ __forceinline__ void chunk_stages_mfma16(const float *__restrict__ x,
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(q.z, h[2], acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(q.w, h[3], acc, 0, 0, 0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) lds[(chunk0 + 16 * b + 4 * kk + i) * 17 + m] = acc[i];
+        for (int i = 0; i < 4; i++) lds[chunk_word(chunk0 + 16 * b + 4 * kk + i) + m] = acc[i];
     }
 }
 
@@ -156,7 +152,7 @@ __global__ __attribute__((amdgpu_waves_per_eu(8, 8))) void rht_compress_kernel(c
         float v[16];
         load_chunk(v, x, a, origin + c * 16);
         chunk_stages(v, a.kb);
-        float *mine = lds + c * 17; // pad_idx(16 c + i) = 17 c + i
+        float *mine = lds + chunk_word(c);
 #pragma unroll
         for (int i = 0; i < 16; i++) mine[i] = v[i];
     }
@@ -180,7 +176,7 @@ __global__ __attribute__((amdgpu_waves_per_eu(8, 8))) void rht_compress_kernel(c
             r.generate(key, sc0 * 16 + lane);
         else
             r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
-        const float *mine = lds + (wave * 64 + lane) * 17; // pad_idx(16 c + i) = 17 c + i
+        const float *mine = lds + chunk_word(wave * 64 + lane);
 #pragma unroll
         for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint(mine[i] * a.scale);
     } else {
@@ -241,7 +237,7 @@ __global__ void irht_decompress_kernel(const uint8_t *__restrict__ src, float *_
         const int c = wave * 64 + lane;
         if (c * 16 < tile) {
             chunk_stages(t, a.kb);
-            float *mine = lds + c * 17;
+            float *mine = lds + chunk_word(c);
 #pragma unroll
             for (int i = 0; i < 16; i++) mine[i] = t[i];
         }
@@ -384,7 +380,7 @@ __global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_m
         fetch_chunk<ENDS>(w, x, in, e, cen, origin + (tid + nthreads) * 16);
         chunk_stages(v, a.kb);
         chunk_stages(w, a.kb);
-        float *mine = lds + tid * 17, *other = lds + (tid + nthreads) * 17;
+        float *mine = lds + chunk_word(tid), *other = lds + chunk_word(tid + nthreads);
 #pragma unroll
         for (int i = 0; i < 16; i++) mine[i] = v[i];
 #pragma unroll
@@ -394,7 +390,7 @@ __global__ void rht_tile_kernel(float *__restrict__ x, RhtTileArgs a, int sign_m
             float v[16];
             fetch_chunk<ENDS>(v, x, in, e, cen, origin + c * 16);
             chunk_stages(v, a.kb);
-            float *mine = lds + c * 17; // pad_idx(16 c + i) = 17 c + i
+            float *mine = lds + chunk_word(c);
 #pragma unroll
             for (int i = 0; i < 16; i++) mine[i] = v[i];
         }
@@ -461,8 +457,8 @@ __global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbi
         }
     }
     __syncthreads();
-#define DQ_PASS(P, M)                                     \
-    lds_pass<P, M>(lds, tile >> M, tid, nthreads);        \
+#define DQ_PASS(P, M)                                  \
+    lds_pass<P, M>(lds, rbits + 5, tid, nthreads);     \
     __syncthreads();
     switch (rbits - 4) {
     case 1: DQ_PASS(9, 1) break;
@@ -492,10 +488,10 @@ __global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbi
 
 // ---- blocks of 2^15: the tile in two halves -----------------------------------------------------------
 //
-// A 2^15 tile with its padding needs 139 KB of LDS: one workgroup per CU, whose load, butterfly and
+// A 2^15 tile with its padding needs 135 KB of LDS: one workgroup per CU, whose load, butterfly and
 // quantise phases cannot overlap with a neighbour's.  Here thread t owns chunk t of both halves of the
 // block: the stages of strides 1..8 run on registers, the stages of strides 16 .. 2^13 run in LDS one half
-// after the other (70 KB: two workgroups per CU), and the last stage (stride 2^14) pairs the thread's own
+// after the other (68 KB: two workgroups per CU), and the last stage (stride 2^14) pairs the thread's own
 // two chunks in registers.  The record windows (and the MEE table of the inverse kernel) share the LDS with
 // the tile: they are used only before the first half enters it or after the second has left.  Both kernels
 // ask for eight waves per SIMD (64 registers): two resident workgroups are worth more than the few values
@@ -505,7 +501,7 @@ constexpr int kSplitBits = 15, kHalfBits = 14, kSplitThreads = 1024;
 // stages of strides 16 .. 2^13 of the half block whose chunk t the thread holds in v (in and out)
 __device__ __forceinline__ void half_block_stages(float (&v)[16], float *lds, int tid)
 {
-    float *mine = lds + tid * 17;
+    float *mine = lds + chunk_word(tid);
 #pragma unroll
     for (int i = 0; i < 16; i++) mine[i] = v[i];
     fwht_lds_stages_after4(lds, kHalfBits, kHalfBits, tid, kSplitThreads);
@@ -601,7 +597,7 @@ __global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel
         vb[i] = p - q;
     }
     // store one half after the other through the LDS, so that every store instruction covers 1 KiB contiguously
-    float *mine = lds + tid * 17;
+    float *mine = lds + chunk_word(tid);
 #pragma unroll
     for (int h = 0; h < 2; h++) {
 #pragma unroll
@@ -647,7 +643,7 @@ __global__ __launch_bounds__(kSplitThreads, 8) void rht_tile_split_kernel(float 
         vb[i] = p - q;
     }
     // store one half after the other through the LDS, so that every store instruction covers 1 KiB contiguously
-    float *mine = lds + tid * 17;
+    float *mine = lds + chunk_word(tid);
 #pragma unroll
     for (int h = 0; h < 2; h++) {
 #pragma unroll

@@ -868,6 +868,28 @@ def mfma_experiment(dev, n=1 << 28, block=8192):
     _emit(mfma_experiment=True, bytes_differing=float((a != b).float().mean()), nmse_butterflies=_nmse(x, out_a), nmse_matrix_cores=_nmse(x, out_b))
 
 
+def fused_transform(dev, n=1 << 28, blocks=(1 << 10, 1 << 13, 1 << 15)):
+    """the blocked randomized Hadamard transform alone and fused with the 4-bit AEE codec (packed signs, in-kernel rounding
+    stream) for three block sizes: the launches whose LDS bank conflicts and vector-ALU load the counter runs look at"""
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn(n, generator=g, device=dev) * 1e-3
+    y = x.clone()
+    out = torch.empty_like(x)
+    sign = torch.empty(n // 32, dtype=torch.int32, device=dev)
+    capi.rand_diag_bits(sign, n, 1)
+    packed = torch.zeros(capi.required_bytes(n, 4, 16, 2), dtype=torch.uint8, device=dev)
+    pb = (4 + OV) / 8
+    for block in blocks:
+        scale = 1.0 / math.sqrt(block)
+        tc = _time_us(lambda: capi.rht_scaling_compress(x, sign, packed, block, scale, 4, 2, seed=3, step=1), 2, 5)
+        td = _time_us(lambda: capi.scaling_decompress_irht(packed, sign, out, block, scale, 4, 2), 2, 5)
+        tb = _time_us(lambda: capi.rht_blocked(y, sign, block, scale, False), 2, 5)
+        _emit(fused_transform=True, n=n, block=block, compress_us=round(tc, 1), decompress_us=round(td, 1), rht_blocked_us=round(tb, 1),
+              compress_frac_hbm=round((4 + 0.125 + pb) * n / tc / 1e3 / HBM_PEAK, 4),
+              decompress_frac_hbm=round((4 + 0.125 + pb) * n / td / 1e3 / HBM_PEAK, 4),
+              rht_blocked_frac_hbm=round((8 + 0.125) * n / tb / 1e3 / HBM_PEAK, 4))
+
+
 def reference_benchmark(dev, n=16 * 16 * 65536 * 16):
     """cuda_kernels/tests/benchmark_scaling_quantization.py:60-112 on this GPU, through the drop-in module: the same
     inputs (:31-39), the same eager timing loops (:41-57; 10 warm-up + 50 launches, 5 + 25 for the two ring-step
@@ -937,6 +959,8 @@ def main():
                     help="the kernels of the dynamic-bitrate pipeline at 2^26 and 2^28 bf16 elements in one bucket")
     ap.add_argument("--mfma-experiment", action="store_true",
                     help="the transform fused with the quantiser (blocks of 8192) with its first four stages as butterflies and on the matrix cores")
+    ap.add_argument("--fused-transform", action="store_true",
+                    help="the blocked transform alone and fused with the 4-bit codec at 2^28 elements for blocks of 2^10, 2^13, 2^15")
     ap.add_argument("--reference-benchmark", action="store_true",
                     help="the table of cuda_kernels/tests/benchmark_scaling_quantization.py with the fraction of the HBM peak")
     ap.add_argument("--limit", type=int, default=None, help="config 4: number of 25 MB buckets to process")
@@ -957,6 +981,9 @@ def main():
         return
     if args.mfma_experiment:
         mfma_experiment(dev, **({"n": args.n} if args.n else {}))
+        return
+    if args.fused_transform:
+        fused_transform(dev, **({"n": args.n} if args.n else {}))
         return
     if args.reference_benchmark:
         reference_benchmark(dev, **({"n": args.n} if args.n else {}))
