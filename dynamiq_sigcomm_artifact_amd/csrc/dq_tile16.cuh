@@ -419,17 +419,20 @@ __device__ __forceinline__ int exact_code_fast(float vi, float ri, float d, doub
 
 // The code of an element is clamp(ceil(L - r), -R, R) + R for the coordinate L the exact chain computes -- v / d (AEE)
 // or +-log2(|v / d| / c + 1) / log2(base) (MEE) -- because floor(L) + ceil(frac(L) - r) is that integer; and it is
-// min(floor(L - r + R + 1), 2R) (nothing below zero) as long as L - r is not an integer.  A cheap estimate T of
-// L - r + R + 1 gives the same code unless it comes within kDelta of an integer; such elements (one in a few thousand)
-// are redone with the exact chain, so the bytes are those of the exact chain throughout.
-//   AEE: T = fma(v, rcp(d), (R + 1) - r).  The hardware reciprocal is good to 1 ulp (|v rcp(d) - v / d| < (R + 1) 2^-23),
-//        (R + 1) - r is exact for the in-kernel random bytes and within (R + 1) 2^-26 otherwise, and the fma rounds a
-//        value below 2 (R + 1): its distance to the exact L - r + R + 1 stays below 0.27 (R + 1) 2^-20.
-//   MEE: T = fma(v_log_f32(fma(|v rcp(d)|, 1 / c, 1)), +-1 / log2(base), (R + 1) - r), v_log_f32 being good to 1 ulp;
-//        estimate and exact chain both approximate log2(|v| / (d c) + 1) / log2(base), their distance is bounded by
-//        (1.44 * 5e-7 + 2.7 ulp(log)) / log2(base) + 2 ulp(2 R): < 6.9e-5 for 6..8 bits (log2(base) = 0.0286, log < 4)
-//        and < 1.2e-5 below (log2(base) >= 0.09, log < 1.5); measured over 4e9 random operands per width: 1.5e-5
-//        and 4.8e-6 (without the offset in the last fma, which adds at most 3.8e-6 and 1e-6).
+// min(floor(L - r + R + 1), 2R) (nothing below zero) as long as L - r is not an integer.  A cheap estimate of
+// T = L - r + R + 1 that is within e < kDelta of it decides the code unless T comes within kDelta of an integer; such
+// elements (one in a few thousand) are redone with the exact chain, so the bytes are those of the exact chain
+// throughout.  The estimate is formed as T' = estimate + kDelta (kDelta is part of the constant the random value is
+// subtracted from): frac(T') >= 2 kDelta then puts T' - kDelta - e above floor(T') and T' - kDelta + e below
+// floor(T') + 1, so floor(T) = floor(T'), and the guard is one fraction and one comparison.
+//   AEE: estimate = fma(v, rcp(d), (R + 1 + kDelta) - r).  The hardware reciprocal is good to 1 ulp
+//        (|v rcp(d) - v / d| < (R + 1) 2^-23), the constant minus r is exact for the in-kernel random bytes and within
+//        (R + 1) 2^-26 otherwise, and the fma rounds a value below 2 (R + 1): e stays below 0.27 (R + 1) 2^-20.
+//   MEE: estimate = fma(v_log_f32(fma(|v rcp(d)|, 1 / c, 1)), +-1 / log2(base), (R + 1 + kDelta) - r), v_log_f32 being
+//        good to 1 ulp; estimate and exact chain both approximate log2(|v| / (d c) + 1) / log2(base), their distance is
+//        bounded by (1.44 * 5e-7 + 2.7 ulp(log)) / log2(base) + 2 ulp(2 R): < 6.9e-5 for 6..8 bits (log2(base) = 0.0286,
+//        log < 4) and < 1.2e-5 below (log2(base) >= 0.09, log < 1.5); measured over 4e9 random operands per width: 1.5e-5
+//        and 4.8e-6 (without the constant in the last fma, which adds at most 3.8e-6 and 1e-6).
 template <int NBITS, bool MEE> struct EstimateGuard {
     static constexpr float kDelta = MEE ? (NBITS >= 6 ? 0x1p-12f : 0x1p-14f) : (float)(1 << (NBITS - 1)) * 0x1p-20f;
 };
@@ -447,7 +450,7 @@ template <int NBITS, bool MEE, class RV, class RR>
 __device__ __forceinline__ float estimate_coordinate(const RV &v, const RR &r, int i, float rd, float rc, float rl2b)
 {
     const float vi = v.get(i);
-    const float off = below(r, i, (float)(Rec<NBITS>::R + 1));
+    const float off = below(r, i, (float)(Rec<NBITS>::R + 1) + EstimateGuard<NBITS, MEE>::kDelta); // the constant is exact: <= 21 bits
     if (MEE) {
         const float est = __builtin_amdgcn_logf(__builtin_fmaf(__builtin_fabsf(vi * rd), rc, 1.0f));
         return __builtin_fmaf(est, __builtin_copysignf(rl2b, vi), off);
@@ -469,7 +472,7 @@ __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const float t = estimate_coordinate<NBITS, MEE>(v, r, i, rd, rc, rl2b);
-        doubt[i] = __builtin_fabsf(__builtin_amdgcn_fractf(t) - 0.5f) > 0.5f - kDelta;
+        doubt[i] = __builtin_amdgcn_fractf(t) < 2.0f * kDelta;
         any |= doubt[i];
         words_put<NBITS>(w, i, (uint32_t)__builtin_amdgcn_fmed3f(t, 0.0f, (float)(2 * R))); // T < 2^20: exact
     }
