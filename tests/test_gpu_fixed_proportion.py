@@ -121,10 +121,11 @@ def test_sorted_plan_validation(capi):
 
 
 @pytest.mark.parametrize("strategy", [2, 3])
-def test_groups_feed_the_row_codec(capi, oracle, strategy):
+@pytest.mark.parametrize("widths", [(8, 4, 2), (7, 5, 3)])
+def test_groups_feed_the_row_codec(capi, oracle, strategy, widths):
     """one bucket end to end as the fixed-proportion hook runs it (one rank): groups in sorted order -> index_select ->
     compress (rand rows paired with the position in the group) -> decompress -> index_copy_, against the row-list
-    kernels fed by the device plan"""
+    kernels fed by the device plan; with the hook's widths and with the extension widths 7 / 5 / 3 in their place"""
     from dynamiq_sigcomm_artifact_amd import bitrate as B
     nsc = 1200
     g = torch.Generator().manual_seed(8)
@@ -136,7 +137,8 @@ def test_groups_feed_the_row_codec(capi, oracle, strategy):
     groups = B.fixed_proportion_groups(st[:, 1], thr)
     out = torch.zeros_like(x)
     want = torch.zeros_like(x)
-    for width, base, cnt, idx in ((8, 0, counts[0], groups[0]), (4, nsc, counts[1], groups[1]), (2, 2 * nsc, counts[2], groups[2])):
+    for width, base, cnt, idx in ((widths[0], 0, counts[0], groups[0]), (widths[1], nsc, counts[1], groups[1]),
+                                  (widths[2], 2 * nsc, counts[2], groups[2])):
         rand = torch.rand(cnt * 256, generator=g).to(torch.bfloat16).to(DEV)
         nbytes = capi.required_bytes(cnt * 256, width, 16, strategy)
         # the hook's sequence, through the oracle
