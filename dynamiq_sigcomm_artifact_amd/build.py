@@ -32,6 +32,7 @@ HIP_SOURCES = [
     "dq_hadamard.hip",
     "dq_packing.hip",
     "dq_eden.hip",
+    "dq_streams.hip",
 ]
 
 HIPCC_FLAGS = [

@@ -479,6 +479,14 @@ int dq_mixed_decompress(const uint8_t *src, void *dst, const int32_t *order, con
                                               strategy == 3, mp, static_cast<hipStream_t>(stream)));
 }
 
+int dq_streams_overlap(dq_stream_t a, dq_stream_t b, int device, int *overlap)
+{
+    if (!overlap) return fail(DQ_ERR_NULL);
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::probe_streams_overlap(static_cast<hipStream_t>(a), static_cast<hipStream_t>(b), overlap));
+}
+
 int dq_dynamic_bitrate_bucket(const dq_bucket_t *b, int stages, int device, dq_stream_t stream)
 {
     if (!b) return fail(DQ_ERR_NULL);

@@ -154,6 +154,10 @@ int64_t eden_work_doubles(int64_t n);
 hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids,
                                 int nbits, uint32_t *packed, float *result, double *work,
                                 hipStream_t stream);
+// *overlap = 1 when kernels enqueued on a and b run side by side, 0 when the two streams take turns (they share a
+// hardware queue, or are the same stream).  Synchronises with both streams: a set-up call, not for stream capture.
+hipError_t probe_streams_overlap(hipStream_t a, hipStream_t b, int *overlap);
+
 // the same launches with the partial sums in the library's own static device array (no allocation anywhere);
 // `device` must be current
 int64_t eden_static_max_n();

@@ -563,3 +563,29 @@ def test_single_pass_buckets_object(capi, streams, graphs, whole):
         for k, (x, o) in enumerate(zip(xs, outs)):
             want = _four_calls(capi, x, x.numel(), u, 2, seed, (k << 32) + step)[5]
             assert torch.equal(bits_t(o), bits_t(want)), (step, k)
+
+
+def test_streams_of_the_pipeline_object_run_side_by_side(capi):
+    """dq_streams_overlap: a stream against itself never overlaps; the streams SinglePassBuckets settles on overlap
+    with each other and with the caller's stream, also after the process has used up several streams of torch's pool
+    (the runtime maps streams onto four hardware queues at their first use, and a queue works in order)"""
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import SinglePassBuckets
+    index = torch.cuda.current_device()
+    st = torch.cuda.Stream()
+    assert capi.streams_overlap(st.cuda_stream, st.cuda_stream, index) is False
+    with pytest.raises(RuntimeError):
+        capi._check(capi.lib().dq_streams_overlap(None, None, index, None))
+    scratch = torch.zeros(64, device=DEV)
+    for used in range(5):
+        for streams in (2, 3):
+            pipe = SinglePassBuckets(DEV, strategy=2, seed=1, streams=streams, u=6.0)
+            assert pipe.side_by_side and len(pipe.streams) == streams
+            handles = [torch.cuda.current_stream().cuda_stream] + [s.cuda_stream for s in pipe.streams]
+            assert len(set(handles)) == streams + 1
+            for i in range(streams + 1):
+                for j in range(i + 1, streams + 1):
+                    assert capi.streams_overlap(handles[i], handles[j], index), (used, streams, i, j)
+        extra = torch.cuda.Stream()              # one more stream of the pool gets its queue
+        with torch.cuda.stream(extra):
+            scratch.add_(1.0)
+        torch.cuda.synchronize()
