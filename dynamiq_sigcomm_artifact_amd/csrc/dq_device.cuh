@@ -235,6 +235,19 @@ __device__ __forceinline__ float row16_max(float v)
     return v;
 }
 
+// the same maximum for values that are positive and finite: such floats are ordered like their bit patterns, and an
+// integer maximum takes its DPP operand directly (one instruction per step; the float form needs the move and a
+// canonicalising maximum in front of every step)
+__device__ __forceinline__ float row16_max_pos(float v)
+{
+    uint32_t u = __float_as_uint(v);
+    u = max(u, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)u, 0xB1, 0xf, 0xf, true));
+    u = max(u, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)u, 0x4E, 0xf, 0xf, true));
+    u = max(u, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)u, 0x141, 0xf, 0xf, true));
+    u = max(u, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)u, 0x140, 0xf, 0xf, true));
+    return __uint_as_float(u);
+}
+
 // parameters of the MEE lattice, built on the host and passed by value
 struct MeeParams {
     float c;   // (1+e^2)/(2e^2), binary16 widened

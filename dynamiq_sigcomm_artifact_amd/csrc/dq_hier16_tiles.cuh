@@ -70,7 +70,7 @@ __device__ __forceinline__ void chunk_encode_fast(const RV &v, const RR &r, uint
         s = div_by(a, mp.inv_cmm) + 1e-7f;
     else
         s = (R == 1 ? a : div_by(a, 1.0 / (double)R)) + 1e-7f; // >= 1e-7, finite
-    const float g = row16_max(s);
+    const float g = row16_max_pos(s); // s >= 1e-7, finite
     unit_bits = f32_to_bf16_bits(div_by(g, 1.0 / 255.0));
     const float unit = bf16_bits_to_f32(unit_bits);
     const float ratio = div_by(s, recip_f64(g)) * 255.0f;

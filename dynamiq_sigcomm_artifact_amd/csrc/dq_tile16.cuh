@@ -458,13 +458,29 @@ __device__ __forceinline__ float estimate_coordinate(const RV &v, const RR &r, i
     return __builtin_fmaf(vi, rd, off);
 }
 
+// Upper clamp of the packed codes of a chunk, for widths that divide 32: a field of an estimate_codes() word holds
+// floor(T) <= 2 R + 1 = all ones, and only that value is above 2 R.  A field is all ones when its low NBITS - 1 bits
+// carry into the top bit and the top bit is set; such fields lose their lowest bit.  A few integer instructions per
+// word instead of one clamp per element.
+template <int NBITS> __device__ __forceinline__ uint32_t clamp_fields(uint32_t w)
+{
+    static_assert(NBITS == 2 || NBITS == 4 || NBITS == 8, "fields must not straddle words");
+    if (NBITS == 2) return w ^ (w & (w >> 1) & 0x55555555u);
+    constexpr uint32_t one = NBITS == 4 ? 0x11111111u : 0x01010101u;
+    constexpr uint32_t top = one << (NBITS - 1), low = top - one;
+    const uint32_t full = ((w & low) + one) & w & top;
+    return w - (full >> (NBITS - 1));
+}
+
 // The codes of one chunk against the step d (normal, 2^-100 <= d <= 2^100) for elements that are finite (a NaN would
 // pass the guard unnoticed) with |v| <= (R + 1) d and random values in [0, 1]: estimate, guard, exact redo.  w must
-// be zeroed.
+// be zeroed.  -1 < T' < 2 R + 2, so the conversion to a signed integer (towards zero) is the lower clamp, and for the
+// widths that divide 32 the upper clamp is done on the packed words (clamp_fields).
 template <int NBITS, bool MEE, class RV, class RR, class ARG>
 __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d, const ARG &mp, uint32_t (&w)[Rec<NBITS>::WORDS])
 {
     constexpr int R = Rec<NBITS>::R;
+    constexpr bool kFields = NBITS == 2 || NBITS == 4 || NBITS == 8;
     const float rd = __builtin_amdgcn_rcpf(d);
     const float rc = MEE ? (float)mp.inv_c : 0.0f, rl2b = MEE ? (float)mp.inv_l2b : 0.0f;
     constexpr float kDelta = EstimateGuard<NBITS, MEE>::kDelta;
@@ -474,7 +490,14 @@ __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d
         const float t = estimate_coordinate<NBITS, MEE>(v, r, i, rd, rc, rl2b);
         doubt[i] = __builtin_amdgcn_fractf(t) < 2.0f * kDelta;
         any |= doubt[i];
-        words_put<NBITS>(w, i, (uint32_t)__builtin_amdgcn_fmed3f(t, 0.0f, (float)(2 * R))); // T < 2^20: exact
+        if (kFields)
+            words_put<NBITS>(w, i, (uint32_t)(int)t);
+        else
+            words_put<NBITS>(w, i, (uint32_t)__builtin_amdgcn_fmed3f(t, 0.0f, (float)(2 * R))); // T < 2^20: exact
+    }
+    if (kFields) {
+#pragma unroll
+        for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = clamp_fields<kFields ? NBITS : 2>(w[k]);
     }
     if (__builtin_amdgcn_ballot_w64(any) != 0) {
         const double yd = recip_f64(d);

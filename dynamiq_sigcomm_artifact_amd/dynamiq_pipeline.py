@@ -293,6 +293,33 @@ def dynamic_bitrate_allreduce_single_pass(rank_vecs, u, strategy=2, seed=0, out=
     return outs, total, plan[:4]
 
 
+def pick_streams(device, want, tries=16):
+    """`want` streams that run side by side with each other and with the caller's current stream; returns (streams, ok).
+    The runtime maps the streams of a process onto a few hardware queues when they are first used, and a queue works
+    through what it is given in order, whichever stream it came from.  Two streams on one queue take turns; and with the
+    caller's stream on the queue of one of them, an event that orders the *next* piece of work after the caller's
+    (recorded on the caller's stream) completes only after the piece enqueued just before it -- either way two buckets
+    "in flight" run as slowly as on one stream (measured: 31 against 18.5 us per 25 MB bucket).  Which streams share a
+    queue depends on what else the process has used, so candidates are taken from torch's pool until `want` of them
+    overlap with each other and with the current stream (capi.streams_overlap, about a millisecond per pair); if the
+    pool does not yield that many, the set is filled up and ok is False."""
+    from . import capi
+    device = torch.device(device)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    apart = [torch.cuda.current_stream(device).cuda_stream]
+    chosen = []
+    while len(chosen) < want and tries > 0:
+        tries -= 1
+        cand = torch.cuda.Stream(device=device)
+        if cand.cuda_stream not in apart and all(capi.streams_overlap(h, cand.cuda_stream, index) for h in apart):
+            chosen.append(cand)
+            apart.append(cand.cuda_stream)
+    ok = len(chosen) == want
+    while len(chosen) < want:
+        chosen.append(torch.cuda.Stream(device=device))
+    return chosen, ok
+
+
 class SinglePassBuckets(object):
     """The single-pass dynamic-bitrate path for a stream of buckets on one rank (a ring of one: statistics, widths,
     partition, encode, decode, mean add -- what dynamic_bitrate_allreduce_single_pass does for W = 1), shaped for
@@ -302,7 +329,7 @@ class SinglePassBuckets(object):
       * one host call per bucket (capi.dynamic_bitrate_bucket) instead of four (``run``);
       * ``streams`` buckets are in flight at a time, each on a stream of its own with scratch of its own (statistics,
         means, plan, packed stream): the latency-bound statistics and plan launches of one bucket overlap the codec
-        launches of its neighbour.  The streams are chosen so that they do run side by side (``_pick_streams``);
+        launches of its neighbour.  The streams are chosen so that they do run side by side (``pick_streams``);
       * with ``graphs=True``, ``run_all`` records a whole step's buckets once -- one graph per stream -- and replays
         them: one graph launch per stream and step instead of one host call per bucket.  DDP hands the hook the same
         bucket views on every step, so the list of (source, output) pairs is the natural key; a replay reads whatever
@@ -322,7 +349,7 @@ class SinglePassBuckets(object):
         self.capi = capi
         self.device = torch.device(device)
         self.strategy, self.seed, self.graphs = strategy, int(seed), graphs
-        self.streams, self.side_by_side = self._pick_streams(max(1, int(streams)))
+        self.streams, self.side_by_side = pick_streams(self.device, max(1, int(streams)))
         self.scratch = [dict() for _ in self.streams]
         self.pending = [False] * len(self.streams)
         # one step counter per stream, advanced on that stream: no hand-over between streams at a step boundary
@@ -337,31 +364,6 @@ class SinglePassBuckets(object):
         self.cache = {}          # (x.data_ptr(), out.data_ptr(), n, dtype, stream index) -> (descriptor, device, graph, ordinal)
         self.ordinals = {}       # (x.data_ptr(), n) -> ordinal of the bucket in the random stream
         self.superchunks = 0
-
-    def _pick_streams(self, want, tries=16):
-        """`want` streams that run side by side with each other and with the caller's current stream.  The runtime maps
-        the streams of a process onto a few hardware queues when they are first used, and a queue works through what
-        it is given in order, whichever stream it came from.  Two of our streams on one queue take turns; and with the
-        caller's stream on the queue of one of ours, the event that orders the *next* bucket after the caller's work
-        (recorded on the caller's stream) completes only after the bucket enqueued just before it -- either way two
-        buckets "in flight" run as slowly as on one stream (measured: 31 against 18.5 us per bucket).  Which streams
-        share a queue depends on what else the process has used, so candidates are taken from torch's pool until
-        `want` of them overlap with each other and with the current stream (capi.streams_overlap, about a
-        millisecond per pair); if the pool does not yield that many, the set is filled up and ``side_by_side`` is
-        False."""
-        index = self.device.index if self.device.index is not None else torch.cuda.current_device()
-        apart = [torch.cuda.current_stream(self.device).cuda_stream]
-        chosen = []
-        while len(chosen) < want and tries > 0:
-            tries -= 1
-            cand = torch.cuda.Stream(device=self.device)
-            if cand.cuda_stream not in apart and all(self.capi.streams_overlap(h, cand.cuda_stream, index) for h in apart):
-                chosen.append(cand)
-                apart.append(cand.cuda_stream)
-        ok = len(chosen) == want
-        while len(chosen) < want:
-            chosen.append(torch.cuda.Stream(device=self.device))
-        return chosen, ok
 
     # ---- once per training step ----------------------------------------------------------------------------
     def set_u(self, u):
@@ -470,7 +472,7 @@ class SinglePassBuckets(object):
                 graphs.append(g)
             entry[0] = graphs
         # one event for all streams, recorded before the first replay: an event recorded on the caller's stream between
-        # two replays could complete only after the first of them (see _pick_streams)
+        # two replays could complete only after the first of them (see pick_streams)
         fence = torch.cuda.Event()
         fence.record(cur)
         for k, st in enumerate(self.streams):

@@ -36,7 +36,7 @@ from dynamiq_sigcomm_artifact_amd import bitrate, capi                          
 from dynamiq_sigcomm_artifact_amd.compressors import Aee_Dynamic_Range_GPU_kern, Mee_Dynamic_Range_GPU_kern   # noqa: E402
 from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import (dynamic_bitrate_allreduce,     # noqa: E402
                                                            dynamic_bitrate_allreduce_grouped,
-                                                           dynamic_bitrate_allreduce_single_pass)
+                                                           dynamic_bitrate_allreduce_single_pass, pick_streams)
 from dynamiq_sigcomm_artifact_amd.ring_sim import ring_allreduce, split_chunks             # noqa: E402
 
 HBM_PEAK = 8000.0  # GB/s
@@ -481,7 +481,7 @@ def config4_streams(dev, u, nbuckets=48, rounds=8):
     # (streams, closed loop): in the closed loop the plans read u from device memory, every bucket adds its norms to the
     # histogram and a round ends with the correction of u for the next one -- a whole training step without a read-back
     for nstreams, closed in ((1, False), (2, False), (3, False), (4, False), (1, True), (2, True)):
-        streams = [torch.cuda.Stream() for _ in range(nstreams)]
+        streams, _ = pick_streams(dev, nstreams)          # streams that share no hardware queue with each other or with `main`
         graphs = []
         hist = bitrate.NormHistogram(dev) if closed else None
         if closed:
@@ -506,8 +506,11 @@ def config4_streams(dev, u, nbuckets=48, rounds=8):
         main = torch.cuda.current_stream()
 
         def replay_all():
+            fence = torch.cuda.Event()
+            fence.record(main)                   # one event before the first replay, not one between replays
+            for st in streams:
+                st.wait_event(fence)
             for g, st in zip(graphs, streams):
-                st.wait_stream(main)
                 with torch.cuda.stream(st):
                     g.replay()
             for st in streams:
