@@ -25,7 +25,7 @@ namespace dq {
 __device__ __forceinline__ int pad_idx(int i) { return i + (i >> 5); }
 
 // words of LDS for a padded tile of `tile` floats, rounded up to a multiple of four (what follows stays 16-byte aligned)
-__host__ __device__ inline int padded_floats(int tile) { return (tile + (tile >> 5) + 1 + 3) & ~3; }
+__host__ __device__ constexpr int padded_floats(int tile) { return (tile + (tile >> 5) + 1 + 3) & ~3; }
 
 // where the 16 consecutive elements of chunk c start: pad_idx(16 c + k) = 16 c + c / 2 + k for k < 16
 __device__ __forceinline__ int chunk_word(int c) { return 16 * c + (c >> 1); }

@@ -98,7 +98,7 @@ __device__ __forceinline__ void load_chunk(float (&v)[16], const float *__restri
 }
 
 // floats of LDS holding the padded tile, rounded up so that what follows is 16-byte aligned
-__host__ __device__ inline int padded_tile_floats(int kt) { return padded_floats(1 << kt); }
+__host__ __device__ constexpr int padded_tile_floats(int kt) { return padded_floats(1 << kt); }
 
 // The stages of strides 1..8 of 64 chunks as one matrix product on the matrix cores: Y = X H16, X the wave's 64 x 16
 // block of chunks, H16[i][j] = (-1)^popcount(i & j).  v_mfma_f32_16x16x4_f32 takes a 16 x 4 slice of X (lane l: row
@@ -510,8 +510,15 @@ __device__ __forceinline__ void half_block_stages(float (&v)[16], float *lds, in
     __syncthreads(); // the half has left the LDS
 }
 
+// bytes of LDS of the forward kernel: the half tile, and behind it the record windows of the sixteen waves where two
+// such workgroups still fit a CU (160 KB), i.e. up to 5-bit codes
+template <int NBITS> __host__ __device__ constexpr bool split_parks()
+{
+    return (size_t)padded_tile_floats(kHalfBits) * sizeof(float) + (kSplitThreads / 64) * Rec<NBITS>::WIN <= 80 * 1024;
+}
+
 template <int RDT, int NBITS, bool MEE>
-__global__ __launch_bounds__(kSplitThreads, 8) void rht_compress_split_kernel(const float *__restrict__ x, uint8_t *__restrict__ dst,
+__global__ __launch_bounds__(kSplitThreads, split_parks<NBITS>() ? 8 : 4) void rht_compress_split_kernel(const float *__restrict__ x, uint8_t *__restrict__ dst,
                                                                           const void *__restrict__ rnd, RhtTileArgs a,
                                                                           int rvec, RandKey key, MeeArg<NBITS, MEE> mp)
 {
@@ -525,15 +532,35 @@ __global__ __launch_bounds__(kSplitThreads, 8) void rht_compress_split_kernel(co
     butterflies<4>(va);
     butterflies<4>(vb);
     half_block_stages(va, lds, tid);
-    half_block_stages(vb, lds, tid);
+    float *mine = lds + chunk_word(tid);
+    uint8_t *win_out;
+    if constexpr (split_parks<NBITS>()) {
+        // The second half stays in the LDS after its stages: the thread pairs its two chunks there, keeps the sums
+        // and leaves the differences in its own slot until the sums are quantised.  With both halves in registers
+        // through the quantiser the kernel needs more than its 64 registers, and what it spills travels to memory
+        // and back (measured at 2^28 elements: 757 MB written and 1.52 GB read for 153 MB of records and 1.11 GB of
+        // input).  The record windows then lie behind the tile instead of inside it.
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const float p = va[i], q = vb[i];
-        va[i] = p + q;
-        vb[i] = p - q;
+        for (int i = 0; i < 16; i++) mine[i] = vb[i];
+        fwht_lds_stages_after4(lds, kHalfBits, kHalfBits, tid, kSplitThreads); // ends with a barrier; own slot only from here on
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float p = va[i], q = mine[i];
+            va[i] = p + q;
+            mine[i] = p - q;
+        }
+        win_out = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(kHalfBits)) + wave * RC::WIN;
+    } else {
+        half_block_stages(vb, lds, tid);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float p = va[i], q = vb[i];
+            va[i] = p + q;
+            vb[i] = p - q;
+        }
+        win_out = reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN;
     }
     // quantise: the wave's 64 chunks of a half are 4 superchunks, one run of records
-    uint8_t *win_out = reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN;
 #pragma unroll
     for (int h = 0; h < 2; h++) {
         const int64_t sc0 = (origin >> 8) + h * 64 + wave * kRowsPerWave;
@@ -544,7 +571,14 @@ __global__ __launch_bounds__(kSplitThreads, 8) void rht_compress_split_kernel(co
         else
             r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
 #pragma unroll
-        for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint((h ? vb[i] : va[i]) * a.scale);
+        for (int i = 0; i < 16; i++) {
+            float t;
+            if constexpr (split_parks<NBITS>())
+                t = h ? mine[i] : va[i];
+            else
+                t = h ? vb[i] : va[i];
+            v.w[i] = __float_as_uint(t * a.scale);
+        }
         encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, kRowsPerWave, win_out, threadIdx.x & 63);
         wave_lds_sync(); // the window is reused for the other half
     }
@@ -707,7 +741,8 @@ hipError_t run_compress(const float *src, const void *sign, int sign_bits, uint8
 {
     const Geometry g = geometry(src, sign, sign_bits, n, block, scale);
     if (g.a.kb == kSplitBits) {
-        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float);
+        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float) +
+                                (split_parks<NBITS>() ? (kSplitThreads / 64) * Rec<NBITS>::WIN : 0);
         auto split = rht_compress_split_kernel<RDT, NBITS, MEE>;
         hipError_t es = allow_lds(split, half_lds);
         if (es != hipSuccess) return es;

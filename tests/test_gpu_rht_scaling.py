@@ -67,6 +67,39 @@ def test_fused_equals_two_calls(capi, block, nbits, strategy):
     assert err < {2: 1.0, 4: 0.05, 5: 0.02, 8: 2e-3}[nbits]
 
 
+@pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("strategy", [2, 3])
+def test_blocks_of_32768_every_width(capi, nbits, strategy):
+    """the forward kernel for blocks of 2^15 keeps the second half of the block in the LDS up to 6-bit codes (its record
+    windows then lie behind the tile) and runs as one workgroup per CU above: every width, both rounding sources, against
+    the two calls"""
+    block, n = 32768, 3 * 32768
+    g, x, sign = _case(n, 77 + nbits)
+    bits = capi.pack_signs(sign)
+    scale = 1.0 / np.sqrt(block)
+    nb = capi.required_bytes(n, nbits, 16, strategy)
+    rot = x.clone()
+    capi.rht_blocked(rot, sign, block, scale, False)
+    for pool_dt in (None, torch.bfloat16, torch.float32):
+        want = torch.zeros(nb, dtype=torch.uint8, device=DEV)
+        if pool_dt is None:
+            pool = None
+            capi.scaling_compress_philox(rot, want, n, nbits, 16, strategy, 5, 9)
+        else:
+            pool = torch.rand(n, generator=g).to(pool_dt).to(DEV)
+            capi.scaling_compress(rot, want, pool, n, nbits, 16, strategy)
+        got = torch.full((nb + 32,), 0x5A, dtype=torch.uint8, device=DEV)
+        capi.rht_scaling_compress(x, bits, got, block, scale, nbits, strategy, rand_pool=pool, seed=5, step=9)
+        assert torch.equal(got[:nb], want), (nbits, strategy, pool_dt)
+        assert bool((got[nb:] == 0x5A).all())
+    dec = torch.empty(n, dtype=torch.float32, device=DEV)
+    capi.scaling_decompress(want, dec, n, nbits, 16, strategy)
+    capi.rht_blocked(dec, sign, block, scale, True)
+    back = torch.empty(n, dtype=torch.float32, device=DEV)
+    capi.scaling_decompress_irht(want, bits, back, block, scale, nbits, strategy)
+    assert torch.equal(back.view(torch.int32), dec.view(torch.int32))
+
+
 @pytest.mark.parametrize("n,block", [(256, 256), (256, 16), (512, 512), (768, 256), (1280, 256), (2048, 1024)])
 def test_small_vectors_no_sign_unaligned(capi, n, block):
     g, x, _ = _case(n, n + block)
