@@ -460,6 +460,13 @@ def config5_entries(capi, O, dev, reps, n=1 << 30):
     # the randomized Hadamard transform fused with the codec: packed Rademacher signs (one bit per element), in-kernel
     # rounding stream; the rotated vector never reaches memory
     sign = torch.empty(n // 32, dtype=torch.int32, device=dev)
+    # The first vector-ALU-bound measurements after a stretch of memory-bound work run on a GPU that is still raising its
+    # clock (whichever cell comes first reads 15-20 % slow): one measurement of the first cell is taken and thrown away.
+    settle = torch.zeros(capi.required_bytes(n, 2, 16, 2), dtype=torch.uint8, device=dev)
+    capi.rand_diag_bits(sign, n, 1 << 10)
+    for _ in range(2):
+        median_ms(lambda: capi.rht_scaling_compress(x, sign, settle, 1 << 10, 1.0 / 32.0, 2, 2, seed=1, step=0), 2, reps)
+    del settle
     for kb in (10, 11, 12, 13, 14, 15):
         block = 1 << kb
         scale = 1.0 / math.sqrt(block)
