@@ -492,66 +492,82 @@ __global__ void rht_strided_kernel(float *__restrict__ x, RhtTileArgs a, int rbi
 // quantise phases cannot overlap with a neighbour's.  Here thread t owns chunk t of both halves of the
 // block: the stages of strides 1..8 run on registers, the stages of strides 16 .. 2^13 run in LDS one half
 // after the other (68 KB: two workgroups per CU), and the last stage (stride 2^14) pairs the thread's own
-// two chunks in registers.  The record windows (and the MEE table of the inverse kernel) share the LDS with
-// the tile: they are used only before the first half enters it or after the second has left.  Both kernels
-// ask for eight waves per SIMD (64 registers): two resident workgroups are worth more than the few values
-// the forward kernel then spills (measured 1.55 against 1.69 ms at 2^30 elements).
+// two chunks.  In the inverse kernel and the plain transform the record windows (and the MEE table) share the
+// LDS with the tile: they are used only before the first half enters it or after the second has left.  The
+// forward kernel keeps its second half in the LDS through the pairing stage and the quantiser of the first
+// (see rht_compress_split_kernel).  All of them ask for eight waves per SIMD (64 registers): two resident
+// workgroups are worth more than anything the register file could hold instead.
 constexpr int kSplitBits = 15, kHalfBits = 14, kSplitThreads = 1024;
 
 // stages of strides 16 .. 2^13 of the half block whose chunk t the thread holds in v (in and out)
+template <int HB = kHalfBits>
 __device__ __forceinline__ void half_block_stages(float (&v)[16], float *lds, int tid)
 {
     float *mine = lds + chunk_word(tid);
 #pragma unroll
     for (int i = 0; i < 16; i++) mine[i] = v[i];
-    fwht_lds_stages_after4(lds, kHalfBits, kHalfBits, tid, kSplitThreads);
+    fwht_lds_stages_after4(lds, HB, HB, tid, 1 << (HB - 4));
 #pragma unroll
     for (int i = 0; i < 16; i++) v[i] = mine[i];
     __syncthreads(); // the half has left the LDS
 }
 
-// bytes of LDS of the forward kernel: the half tile, and behind it the record windows of the sixteen waves where two
-// such workgroups still fit a CU (160 KB), i.e. up to 5-bit codes
-template <int NBITS> __host__ __device__ constexpr bool split_parks()
+// The forward kernel takes blocks of 2^(HB + 1) in two halves of 2^HB, one chunk of each half per thread: HB = 14 for
+// blocks of 2^15 (1024 threads; a CU holds at most two such workgroups) and HB = 13 for blocks of 2^14 (512 threads, up
+// to four per CU; as one tile those blocks need 1024 threads of which half sit idle in both LDS passes).
+//
+// LDS: the half tile and, where the second half is parked in it through the quantiser, the record windows of the waves
+// behind it.  Parking needs the sum to leave room for as many workgroups as the thread count allows (two of 80 KB for
+// HB = 14: up to 6-bit codes); HB = 13 always parks (three workgroups per CU instead of four from 6-bit codes on).
+template <int NBITS, int HB> __host__ __device__ constexpr size_t split_lds_bytes(bool parked)
 {
-    return (size_t)padded_tile_floats(kHalfBits) * sizeof(float) + (kSplitThreads / 64) * Rec<NBITS>::WIN <= 80 * 1024;
+    return (size_t)padded_tile_floats(HB) * sizeof(float) + (parked ? ((1 << (HB - 4)) / 64) * Rec<NBITS>::WIN : 0);
+}
+template <int NBITS, int HB> __host__ __device__ constexpr bool split_parks()
+{
+    return HB < kHalfBits || split_lds_bytes<NBITS, HB>(true) <= 80 * 1024;
 }
 
-template <int RDT, int NBITS, bool MEE>
-__global__ __launch_bounds__(kSplitThreads, split_parks<NBITS>() ? 8 : 4) void rht_compress_split_kernel(const float *__restrict__ x, uint8_t *__restrict__ dst,
-                                                                          const void *__restrict__ rnd, RhtTileArgs a,
-                                                                          int rvec, RandKey key, MeeArg<NBITS, MEE> mp)
+// PAIR = false: the two halves are two whole blocks of 2^HB (no pairing stage): blocks of 2^10 on one wave.
+template <int RDT, int NBITS, bool MEE, int HB, bool PAIR = true>
+__global__ __launch_bounds__(1 << (HB - 4), (split_parks<NBITS, HB>() ? 8 : 4)) void rht_compress_split_kernel(
+    const float *__restrict__ x, uint8_t *__restrict__ dst, const void *__restrict__ rnd, RhtTileArgs a, int rvec, RandKey key,
+    MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
+    constexpr bool kParks = split_parks<NBITS, HB>();
+    constexpr int kThreads = 1 << (HB - 4), kWaves = kThreads / 64;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t origin = (int64_t)blockIdx.x << kSplitBits;
+    const int64_t origin = (int64_t)blockIdx.x << (HB + 1);
     float va[16], vb[16];
     load_chunk(va, x, a, origin + tid * 16);
-    load_chunk(vb, x, a, origin + (1 << kHalfBits) + tid * 16);
+    load_chunk(vb, x, a, origin + (1 << HB) + tid * 16);
     butterflies<4>(va);
     butterflies<4>(vb);
-    half_block_stages(va, lds, tid);
+    half_block_stages<HB>(va, lds, tid);
     float *mine = lds + chunk_word(tid);
     uint8_t *win_out;
-    if constexpr (split_parks<NBITS>()) {
+    if constexpr (kParks) {
         // The second half stays in the LDS after its stages: the thread pairs its two chunks there, keeps the sums
         // and leaves the differences in its own slot until the sums are quantised.  With both halves in registers
         // through the quantiser the kernel needs more than its 64 registers, and what it spills travels to memory
-        // and back (measured at 2^28 elements: 757 MB written and 1.52 GB read for 153 MB of records and 1.11 GB of
-        // input).  The record windows then lie behind the tile instead of inside it.
+        // and back (measured at 2^28 elements in blocks of 2^15: 757 MB written and 1.52 GB read for 153 MB of records
+        // and 1.11 GB of input).  The record windows then lie behind the tile instead of inside it.
 #pragma unroll
         for (int i = 0; i < 16; i++) mine[i] = vb[i];
-        fwht_lds_stages_after4(lds, kHalfBits, kHalfBits, tid, kSplitThreads); // ends with a barrier; own slot only from here on
+        fwht_lds_stages_after4(lds, HB, HB, tid, kThreads); // ends with a barrier; own slot only from here on
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const float p = va[i], q = mine[i];
-            va[i] = p + q;
-            mine[i] = p - q;
+            for (int i = 0; i < 16; i++) {
+                const float p = va[i], q = mine[i];
+                va[i] = p + q;
+                mine[i] = p - q;
+            }
         }
-        win_out = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(kHalfBits)) + wave * RC::WIN;
+        win_out = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(HB)) + wave * RC::WIN;
     } else {
-        half_block_stages(vb, lds, tid);
+        half_block_stages<HB>(vb, lds, tid);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const float p = va[i], q = vb[i];
@@ -563,7 +579,7 @@ __global__ __launch_bounds__(kSplitThreads, split_parks<NBITS>() ? 8 : 4) void r
     // quantise: the wave's 64 chunks of a half are 4 superchunks, one run of records
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        const int64_t sc0 = (origin >> 8) + h * 64 + wave * kRowsPerWave;
+        const int64_t sc0 = (origin >> 8) + h * (kWaves * kRowsPerWave) + wave * kRowsPerWave;
         Raw16<DQ_F32> v;
         Raw16<RDT> r;
         if constexpr (RDT == DQ_PHILOX)
@@ -573,7 +589,7 @@ __global__ __launch_bounds__(kSplitThreads, split_parks<NBITS>() ? 8 : 4) void r
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             float t;
-            if constexpr (split_parks<NBITS>())
+            if constexpr (kParks)
                 t = h ? mine[i] : va[i];
             else
                 t = h ? vb[i] : va[i];
@@ -584,26 +600,28 @@ __global__ __launch_bounds__(kSplitThreads, split_parks<NBITS>() ? 8 : 4) void r
     }
 }
 
-template <int NBITS, bool MEE>
-__global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel(const uint8_t *__restrict__ src,
+// the inverse: blocks of 2^(HB + 1) in two halves (PAIR), or two blocks of 2^HB per workgroup (PAIR = false)
+template <int NBITS, bool MEE, int HB, bool PAIR = true>
+__global__ __launch_bounds__(1 << (HB - 4), 8) void irht_decompress_split_kernel(const uint8_t *__restrict__ src,
                                                                              float *__restrict__ x, RhtTileArgs a,
                                                                              MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
+    constexpr int kThreads = 1 << (HB - 4), kWaves = kThreads / 64;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int row = lane >> 4, j = lane & 15;
-    const int64_t origin = (int64_t)blockIdx.x << kSplitBits;
+    const int64_t origin = (int64_t)blockIdx.x << (HB + 1);
     uint8_t *win_in = reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN;
-    float *table = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds) + (kSplitThreads / 64) * RC::WIN);
+    float *table = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(lds) + kWaves * RC::WIN);
     if (MEE) {
-        for (int k = tid; k < (1 << NBITS); k += kSplitThreads) table[k] = f16_bits_to_f32(mp.table[k]);
+        for (int k = tid; k < (1 << NBITS); k += kThreads) table[k] = f16_bits_to_f32(mp.table[k]);
         __syncthreads();
     }
     float va[16], vb[16];
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        const int64_t sc0 = (origin >> 8) + h * 64 + wave * kRowsPerWave;
+        const int64_t sc0 = (origin >> 8) + h * (kWaves * kRowsPerWave) + wave * kRowsPerWave;
         const int total = kRowsPerWave * RC::REC;
         const uint8_t *g = src + sc0 * RC::REC;
         const WinRegs wr = window_fetch(g, total, lane);
@@ -622,13 +640,15 @@ __global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel
     __syncthreads(); // windows and table are done with: the tile takes the LDS
     butterflies<4>(va);
     butterflies<4>(vb);
-    half_block_stages(va, lds, tid);
-    half_block_stages(vb, lds, tid);
+    half_block_stages<HB>(va, lds, tid);
+    half_block_stages<HB>(vb, lds, tid);
+    if constexpr (PAIR) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const float p = va[i], q = vb[i];
-        va[i] = p + q;
-        vb[i] = p - q;
+        for (int i = 0; i < 16; i++) {
+            const float p = va[i], q = vb[i];
+            va[i] = p + q;
+            vb[i] = p - q;
+        }
     }
     // store one half after the other through the LDS, so that every store instruction covers 1 KiB contiguously
     float *mine = lds + chunk_word(tid);
@@ -637,9 +657,9 @@ __global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel
 #pragma unroll
         for (int i = 0; i < 16; i++) mine[i] = h ? vb[i] : va[i];
         __syncthreads();
-        const int64_t half_origin = origin + ((int64_t)h << kHalfBits);
+        const int64_t half_origin = origin + ((int64_t)h << HB);
         if (a.vec) {
-            for (int i = tid * 4; i < (1 << kHalfBits); i += kSplitThreads * 4) {
+            for (int i = tid * 4; i < (1 << HB); i += kThreads * 4) {
                 const int q = pad_idx(i);
                 float4 v = make_float4(lds[q], lds[q + 1], lds[q + 2], lds[q + 3]);
                 v.x *= a.scale; v.y *= a.scale; v.z *= a.scale; v.w *= a.scale;
@@ -647,7 +667,7 @@ __global__ __launch_bounds__(kSplitThreads, 8) void irht_decompress_split_kernel
                 stream_store(reinterpret_cast<float4 *>(x + half_origin + i), v);
             }
         } else {
-            for (int i = tid; i < (1 << kHalfBits); i += kSplitThreads)
+            for (int i = tid; i < (1 << HB); i += kThreads)
                 x[half_origin + i] = flip1(lds[pad_idx(i)] * a.scale, a, half_origin + i);
         }
         __syncthreads();
@@ -740,15 +760,36 @@ hipError_t run_compress(const float *src, const void *sign, int sign_bits, uint8
                         float scale, const MeeParams &mp, RandKey key, hipStream_t stream)
 {
     const Geometry g = geometry(src, sign, sign_bits, n, block, scale);
-    if (g.a.kb == kSplitBits) {
-        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float) +
-                                (split_parks<NBITS>() ? (kSplitThreads / 64) * Rec<NBITS>::WIN : 0);
-        auto split = rht_compress_split_kernel<RDT, NBITS, MEE>;
-        hipError_t es = allow_lds(split, half_lds);
-        if (es != hipSuccess) return es;
-        hipLaunchKernelGGL(split, dim3((unsigned)(n >> kSplitBits)), dim3(kSplitThreads), half_lds, stream, src, dst, rnd, g.a,
-                           aligned16(rnd) ? 1 : 0, key, make_arg<NBITS, MEE>(mp));
+    if (g.a.kb == 10 && (n & 2047) == 0) {
+        // blocks of 2^10, two per wave
+        auto kernel = rht_compress_split_kernel<RDT, NBITS, MEE, 10, false>;
+        const size_t lds = split_lds_bytes<NBITS, 10>(true);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(n >> 11)), dim3(64), lds, stream, src, dst, rnd, g.a, aligned16(rnd) ? 1 : 0, key,
+                           make_arg<NBITS, MEE>(mp));
         return hipGetLastError();
+    }
+    if (g.a.kb >= kSplitBits - 4 && g.a.kb <= kSplitBits && (n & ((1 << g.a.kb) - 1)) == 0) {
+        // blocks of 2^11 .. 2^15: two halves per workgroup
+        auto launch = [&](auto kernel, size_t lds, int half_bits) -> hipError_t {
+            hipError_t es = allow_lds(kernel, lds);
+            if (es != hipSuccess) return es;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)(n >> (half_bits + 1))), dim3(1 << (half_bits - 4)), lds, stream, src, dst, rnd,
+                               g.a, aligned16(rnd) ? 1 : 0, key, make_arg<NBITS, MEE>(mp));
+            return hipGetLastError();
+        };
+        switch (g.a.kb) {
+        case kSplitBits:
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits>,
+                          split_lds_bytes<NBITS, kHalfBits>(split_parks<NBITS, kHalfBits>()), kHalfBits);
+        case kSplitBits - 1:
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 1>, split_lds_bytes<NBITS, kHalfBits - 1>(true), kHalfBits - 1);
+        case kSplitBits - 2:
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 2>, split_lds_bytes<NBITS, kHalfBits - 2>(true), kHalfBits - 2);
+        case kSplitBits - 3:
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 3>, split_lds_bytes<NBITS, kHalfBits - 3>(true), kHalfBits - 3);
+        default:
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 4>, split_lds_bytes<NBITS, kHalfBits - 4>(true), kHalfBits - 4);
+        }
     }
     if (g.a.kt >= kSplitBits) return hipErrorInvalidValue; // one run of records per wave needs tiles of at most 2^14
     const size_t windows = (size_t)(g.threads / 64) * Rec<NBITS>::WIN;
@@ -766,14 +807,26 @@ hipError_t run_decompress(const uint8_t *src, const void *sign, int sign_bits, f
                           const MeeParams &mp, hipStream_t stream)
 {
     const Geometry g = geometry(dst, sign, sign_bits, n, block, scale);
-    if (g.a.kb == kSplitBits) {
-        const size_t half_lds = (size_t)padded_tile_floats(kHalfBits) * sizeof(float);
-        auto split = irht_decompress_split_kernel<NBITS, MEE>;
-        hipError_t es = allow_lds(split, half_lds);
-        if (es != hipSuccess) return es;
-        hipLaunchKernelGGL(split, dim3((unsigned)(n >> kSplitBits)), dim3(kSplitThreads), half_lds, stream, src, dst, g.a,
-                           make_arg<NBITS, MEE>(mp));
-        return hipGetLastError();
+    if (g.a.kb >= 10 && g.a.kb <= kSplitBits && (n & ((g.a.kb == 10 ? 2048 : (1 << g.a.kb)) - 1)) == 0) {
+        // blocks of 2^11 .. 2^15 in two halves per workgroup, blocks of 2^10 two per wave
+        auto launch = [&](auto kernel, int half_bits) -> hipError_t {
+            const size_t tile = (size_t)padded_tile_floats(half_bits) * sizeof(float);
+            const size_t windows = (size_t)((1 << (half_bits - 4)) / 64) * Rec<NBITS>::WIN + (MEE ? (sizeof(float) << NBITS) : 0);
+            const size_t lds = std::max(tile, windows);
+            hipError_t es = allow_lds(kernel, lds);
+            if (es != hipSuccess) return es;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)(n >> (half_bits + 1))), dim3(1 << (half_bits - 4)), lds, stream, src, dst, g.a,
+                               make_arg<NBITS, MEE>(mp));
+            return hipGetLastError();
+        };
+        switch (g.a.kb) {
+        case 15: return launch(irht_decompress_split_kernel<NBITS, MEE, 14>, 14);
+        case 14: return launch(irht_decompress_split_kernel<NBITS, MEE, 13>, 13);
+        case 13: return launch(irht_decompress_split_kernel<NBITS, MEE, 12>, 12);
+        case 12: return launch(irht_decompress_split_kernel<NBITS, MEE, 11>, 11);
+        case 11: return launch(irht_decompress_split_kernel<NBITS, MEE, 10>, 10);
+        default: return launch(irht_decompress_split_kernel<NBITS, MEE, 10, false>, 10);
+        }
     }
     if (g.a.kt >= kSplitBits) return hipErrorInvalidValue;
     const size_t windows = (size_t)(g.threads / 64) * Rec<NBITS>::WIN + (MEE ? (sizeof(float) << NBITS) : 0);

@@ -69,11 +69,12 @@ def test_fused_equals_two_calls(capi, block, nbits, strategy):
 
 @pytest.mark.parametrize("nbits", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("strategy", [2, 3])
-def test_blocks_of_32768_every_width(capi, nbits, strategy):
-    """the forward kernel for blocks of 2^15 keeps the second half of the block in the LDS up to 6-bit codes (its record
-    windows then lie behind the tile) and runs as one workgroup per CU above: every width, both rounding sources, against
-    the two calls"""
-    block, n = 32768, 3 * 32768
+@pytest.mark.parametrize("block", [16384, 32768])
+def test_blocks_taken_in_two_halves_every_width(capi, nbits, strategy, block):
+    """the forward kernel for blocks of 2^14 and 2^15 takes a block in two halves and keeps the second one in the LDS
+    through the quantiser of the first (blocks of 2^15: up to 6-bit codes, its record windows then lie behind the tile;
+    one workgroup per CU above): every width, every rounding source, against the two calls"""
+    n = 3 * block
     g, x, sign = _case(n, 77 + nbits)
     bits = capi.pack_signs(sign)
     scale = 1.0 / np.sqrt(block)
