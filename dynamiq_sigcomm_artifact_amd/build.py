@@ -27,7 +27,7 @@ HIP_SOURCES = [
     "dq_scaling_tile16.hip",
     "dq_grouping.hip", "dq_bitrate.hip", "dq_sort.hip",
     "dq_scaling_mixed.hip",
-    "dq_rht_scaling.hip",
+    "dq_rht_scaling.hip", "dq_rht_compress_philox.hip", "dq_rht_compress_bf16.hip", "dq_rht_compress_f32.hip", "dq_rht_decompress.hip",
     "dq_superchunk.hip",
     "dq_hadamard.hip",
     "dq_packing.hip",

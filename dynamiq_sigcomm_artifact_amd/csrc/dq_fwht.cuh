@@ -1,6 +1,6 @@
 // Butterfly stages of the Walsh-Hadamard transform on a tile held in LDS, shared by the transform kernels
 // (dq_hadamard.hip) and the kernels that quantise the rotated tile before it leaves the workgroup
-// (dq_rht_scaling.hip).  Stages run in ascending stride with butterflies (a+b, a-b), the order of
+// (dq_rht_scaling_impl.cuh).  Stages run in ascending stride with butterflies (a+b, a-b), the order of
 // csrc/cuda_hadamard.cu:66-157,205-274, four or five index bits at a time on registers.
 //
 // Layout.  The LDS serves 32 lanes per cycle from 32 banks of one word, so an access of a wave is free of bank

@@ -16,7 +16,7 @@
 // result is bit-identical to a plain stage-by-stage FWHT.
 //
 // This file plans the passes.  Passes of at least 1024 elements go to the kernels of
-// dq_rht_scaling.hip, which do the first four stages on the registers a lane loads
+// dq_rht_scaling_impl.cuh, which do the first four stages on the registers a lane loads
 // into and need fewer LDS passes; the kernel here, fwht_tile_kernel, does the stages
 // of a tile four at a time (radix 16) between LDS and registers and serves what is
 // left: small tiles, strided passes over fewer than four bits, buffers without
@@ -247,7 +247,7 @@ static hipError_t fwht_blocks(float *x, const void *sign, bool sign_packed, int6
     a.out_levels = nullptr; a.uniform = thc.uniform; a.out_lo = thc.out_lo; a.out_delta = thc.out_delta;
     a.out_top = thc.out_top;
     const int sign_fwd = (sign && !inverse) ? 1 : 0, sign_inv = (sign && inverse) ? 2 : 0;
-    // Passes of at least 1024 elements run as the chunk-first kernels of dq_rht_scaling.hip; a quantiser at an end needs
+    // Passes of at least 1024 elements run as the chunk-first kernels of dq_rht_scaling_impl.cuh; a quantiser at an end needs
     // the 16-byte paths there
     const bool plain = !thc.in_levels && !thc.in_planes && !thc.out_levels && !thc.post_scale;
     const bool ends_ok = plain || (vec16 && (n & 31) == 0 && (reinterpret_cast<uintptr_t>(thc.in_levels) & 15) == 0);

@@ -116,7 +116,7 @@ hipError_t launch_thc_rht_quantize(float *vec, const void *sign, bool sign_packe
 hipError_t launch_thc_dequantize_irht(const void *levels_in, const void *sign, bool sign_packed, float *out, int64_t n,
                                       int64_t block, float scale, const float *step, const float *lo, hipStream_t stream);
 
-// blocked randomized Hadamard transform fused with the hierarchical chunk-16 quantiser (dq_rht_scaling.hip);
+// blocked randomized Hadamard transform fused with the hierarchical chunk-16 quantiser (dq_rht_scaling_impl.cuh and the translation units that include it);
 // rand_kind: DQ_F32 or DQ_BF16 pool, or 3 for the in-kernel stream (rnd ignored)
 hipError_t launch_pack_signs(const float *sign, uint32_t *bits, int64_t n, hipStream_t stream);
 // sign: fp32 +-1 values, or with sign_bits one bit per element (launch_pack_signs); may be null
