@@ -404,7 +404,7 @@ def config4_entries(capi, O, dev, reps):
         entry = {
             "workload": "config 4: single-pass dynamic-bitrate path (u = %.2f, %.2f code bits) per 25 MB bf16 bucket of a "
                         "Llama-3-8B shaped set, steps of %d distinct buckets back to back, %s, %d bucket(s) in flight; host calls included"
-                        % (u, avg, nb, "one recorded graph per stream and step" if graphs else "eager, one host call per bucket", streams),
+                        % (u, avg, nb, "one recorded graph per stream and step" if graphs else "eager, one host call per bucket, the first bucket of every round on the caller's own stream", streams),
             "us_per_bucket": round(per * 1e3, 2), "GBps_bf16_in": round(2.0 * n / (per * 1e-3) / 1e9, 1),
         }
         if not graphs and streams == 1:

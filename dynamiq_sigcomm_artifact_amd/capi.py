@@ -26,7 +26,7 @@ EXPORTS = [
     "dq_group_plan_stats_dev_u", "dq_group_plan_sorted", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
-    "dq_dynamic_bitrate_bucket", "dq_streams_overlap",
+    "dq_dynamic_bitrate_bucket", "dq_streams_overlap", "dq_stream_order_after",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_rht_scaling_compress_mfma16", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
@@ -123,6 +123,8 @@ def lib():
         L.dq_superchunk_stats.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
         L.dq_dynamic_bitrate_bucket.restype = i32
         L.dq_dynamic_bitrate_bucket.argtypes = [c.POINTER(Bucket), i32, i32, vp]
+        L.dq_stream_order_after.restype = i32
+        L.dq_stream_order_after.argtypes = [vp, vp, i32]
         L.dq_streams_overlap.restype = i32
         L.dq_streams_overlap.argtypes = [vp, vp, i32, c.POINTER(c.c_int)]
         L.dq_superchunk_mean_center.restype = i32
@@ -481,6 +483,12 @@ def dynamic_bitrate_bucket(desc, device, stages=STAGE_ALL, stream=None):
     """one host call for any run of the stages statistics -> plan -> mixed compress -> mixed decompress of one bucket
     (desc, device: from bucket_descriptor)"""
     _check(lib().dq_dynamic_bitrate_bucket(ctypes.byref(desc), stages, device, _stream(stream)))
+
+
+def stream_order_after(stream, after, device):
+    """`stream` waits for everything enqueued on `after` so far (raw handles or torch streams); an event from the library's
+    own ring, nothing allocated per call"""
+    _check(lib().dq_stream_order_after(_stream(stream), _stream(after), int(device)))
 
 
 def streams_overlap(a, b, device):

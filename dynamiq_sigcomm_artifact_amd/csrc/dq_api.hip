@@ -487,6 +487,13 @@ int dq_streams_overlap(dq_stream_t a, dq_stream_t b, int device, int *overlap)
     return finish(dq::probe_streams_overlap(static_cast<hipStream_t>(a), static_cast<hipStream_t>(b), overlap));
 }
 
+int dq_stream_order_after(dq_stream_t stream, dq_stream_t after, int device)
+{
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::stream_order_after(static_cast<hipStream_t>(stream), static_cast<hipStream_t>(after), device));
+}
+
 int dq_dynamic_bitrate_bucket(const dq_bucket_t *b, int stages, int device, dq_stream_t stream)
 {
     if (!b) return fail(DQ_ERR_NULL);

@@ -157,6 +157,8 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
 // *overlap = 1 when kernels enqueued on a and b run side by side, 0 when the two streams take turns (they share a
 // hardware queue, or are the same stream).  Synchronises with both streams: a set-up call, not for stream capture.
 hipError_t probe_streams_overlap(hipStream_t a, hipStream_t b, int *overlap);
+// `stream` waits for the work enqueued on `after` so far (pooled event, no allocation after the first 64 calls per device)
+hipError_t stream_order_after(hipStream_t stream, hipStream_t after, int device);
 
 // the same launches with the partial sums in the library's own static device array (no allocation anywhere);
 // `device` must be current

@@ -14,6 +14,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 namespace dq {
 
 namespace {
@@ -84,6 +86,30 @@ hipError_t probe_streams_overlap(hipStream_t a, hipStream_t b, int *overlap)
     }
     *overlap = both < 1.5f * alone;
     return hipSuccess;
+}
+
+// `stream` waits for everything enqueued on `after` so far: an event recorded on `after`, waited for by `stream`.  The events
+// come from a small ring per device, created on first use (timing disabled) and reused: a wait refers to the record that
+// was current when the wait was enqueued, so recording the event again later does not disturb it.  Meant for callers that
+// hand every bucket to a worker stream from a hot loop -- creating an event per hand-over, which is what a framework's
+// wait_stream does, costs the host as much as enqueueing the bucket's four kernels.
+hipError_t stream_order_after(hipStream_t stream, hipStream_t after, int device)
+{
+    if (stream == after) return hipSuccess;
+    constexpr int kRing = 64, kDevices = 64;
+    static std::mutex lock;
+    static hipEvent_t ring[kDevices][kRing];
+    static unsigned next[kDevices];
+    if (device < 0 || device >= kDevices) return hipErrorInvalidDevice;
+    hipEvent_t ev;
+    {
+        std::lock_guard<std::mutex> hold(lock);
+        const unsigned slot = next[device]++ % kRing;
+        if (!ring[device][slot]) DQ_TRY(hipEventCreateWithFlags(&ring[device][slot], hipEventDisableTiming));
+        ev = ring[device][slot];
+    }
+    DQ_TRY(hipEventRecord(ev, after));
+    return hipStreamWaitEvent(stream, ev, 0);
 }
 
 #undef DQ_TRY

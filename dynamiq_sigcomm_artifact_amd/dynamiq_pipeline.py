@@ -327,6 +327,9 @@ class SinglePassBuckets(object):
     for the one before:
 
       * one host call per bucket (capi.dynamic_bitrate_bucket) instead of four (``run``);
+      * eager buckets of the first of the ``streams`` slots run on the caller's own stream (``inline_first``): handing a
+        bucket to another stream costs an event record, a wait and a dearer first launch behind it -- measured 17 us of
+        host time against 13 us for the four kernels themselves;
       * ``streams`` buckets are in flight at a time, each on a stream of its own with scratch of its own (statistics,
         means, plan, packed stream): the latency-bound statistics and plan launches of one bucket overlap the codec
         launches of its neighbour.  The streams are chosen so that they do run side by side (``pick_streams``);
@@ -344,11 +347,11 @@ class SinglePassBuckets(object):
     run(x, out) enqueues a bucket and returns at once; join() makes the caller's current stream wait for everything
     enqueued so far.  The caller must not overwrite x or read out before join()."""
 
-    def __init__(self, device, strategy=2, seed=0, streams=2, graphs=True, u=None, norm_histogram=None):
+    def __init__(self, device, strategy=2, seed=0, streams=2, graphs=True, u=None, norm_histogram=None, inline_first=True):
         from . import capi
         self.capi = capi
         self.device = torch.device(device)
-        self.strategy, self.seed, self.graphs = strategy, int(seed), graphs
+        self.strategy, self.seed, self.graphs, self.inline_first = strategy, int(seed), graphs, bool(inline_first)
         self.streams, self.side_by_side = pick_streams(self.device, max(1, int(streams)))
         self.scratch = [dict() for _ in self.streams]
         self.pending = [False] * len(self.streams)
@@ -361,7 +364,9 @@ class SinglePassBuckets(object):
         ready.record(torch.cuda.current_stream(self.device))
         for st in self.streams:
             st.wait_event(ready)         # the counters and u are initialised on the caller's stream
-        self.cache = {}          # (x.data_ptr(), out.data_ptr(), n, dtype, stream index) -> (descriptor, device, graph, ordinal)
+        self.cache = {}          # (x.data_ptr(), out.data_ptr(), n, dtype) -> _entry(); ("step", keys) -> [graphs, uses]
+        self._enqueue = capi.lib().dq_dynamic_bitrate_bucket
+        self._order = capi.lib().dq_stream_order_after
         self.ordinals = {}       # (x.data_ptr(), n) -> ordinal of the bucket in the random stream
         self.superchunks = 0
 
@@ -381,9 +386,19 @@ class SinglePassBuckets(object):
     def begin_step(self):
         """advance the step counter of the rounding stream: one small kernel per stream and training step, enqueued on
         that stream, so it is ordered with the stream's buckets and nothing waits for another stream"""
-        for st, counter in zip(self.streams, self.step_devs):
-            with torch.cuda.stream(st):
+        for k, (st, counter) in enumerate(zip(self.streams, self.step_devs)):
+            if k == 0 and self.inline_first:
+                # slot 0 runs on the caller's stream when eager and on its worker stream when recorded: its counter is
+                # advanced on the caller's stream, after whatever the worker stream still has of the previous step (a
+                # recorded step orders the worker streams after the caller's before it starts)
+                if self.pending[0]:
+                    cur = torch.cuda.current_stream(self.device)
+                    cur.wait_stream(st)
+                    self.pending[0] = False
                 counter.add_(1)
+            else:
+                with torch.cuda.stream(st):
+                    counter.add_(1)
 
     # ---- per bucket ---------------------------------------------------------------------------------------------
     def _scratch(self, k, nsc):
@@ -399,34 +414,52 @@ class SinglePassBuckets(object):
             for name in ("stats", "mean", "order", "work", "packed"):
                 sc[name].record_stream(self.streams[k])     # allocated on the caller's stream, used on this one
             # scratch of another size invalidates what was recorded against the old buffers
-            for key in [key for key in self.cache if key[0] == "step" or key[4] == k]:
+            for key in [key for key, entry in self.cache.items() if key[0] == "step" or entry[3] == k]:
                 del self.cache[key]
         return sc
 
-    def run(self, x, out):
-        """enqueue one bucket: out = decode(encode(x)) with the widths of its reduced norms; returns the index of the
-        stream it went to"""
+    def _entry(self, x, out, n, key):
+        """descriptor of a bucket seen for the first time (or again after its stream's scratch grew)"""
+        import ctypes
         capi = self.capi
-        n = x.numel()
         nsc = (n + 255) // 256
         # a source keeps its ordinal, and with it its stream and its recorded launches, from step to step
-        ordinal = self.ordinals.setdefault((x.data_ptr(), n), len(self.ordinals))
+        ordinal = self.ordinals.setdefault((key[0], n), len(self.ordinals))
         k = ordinal % len(self.streams)
-        st = self.streams[k]
-        key = (x.data_ptr(), out.data_ptr(), n, x.dtype, k)
+        sc = self._scratch(k, nsc)
+        desc, dev = capi.bucket_descriptor(x, n, sc["stats"][:nsc], sc["mean"], sc["order"], sc["work"], sc["packed"],
+                                           strategy=self.strategy, out=out, u=self.u_dev,
+                                           hist=None if self.hist is None else self.hist.hist, seed=self.seed,
+                                           step=ordinal << 32, step_dev=self.step_devs[k])
+        # (descriptor, its reference for the call, device, stream index, superchunks, the stream's handle)
+        entry = (desc, ctypes.byref(desc), dev, k, nsc, ctypes.c_void_p(self.streams[k].cuda_stream))
+        self.cache[key] = entry
+        return entry
+
+    def run(self, x, out):
+        """enqueue one bucket: out = decode(encode(x)) with the widths of its reduced norms; returns the index of the
+        stream it went to.  The hot path of an eager caller: two library calls (order the worker stream after the
+        caller's, enqueue the bucket's four kernels) and one dictionary look-up."""
+        n = x.numel()
+        key = (x.data_ptr(), out.data_ptr(), n, x.dtype)
         entry = self.cache.get(key)
         if entry is None:
-            sc = self._scratch(k, nsc)
-            desc, dev = capi.bucket_descriptor(x, n, sc["stats"][:nsc], sc["mean"], sc["order"], sc["work"], sc["packed"],
-                                               strategy=self.strategy, out=out, u=self.u_dev,
-                                               hist=None if self.hist is None else self.hist.hist, seed=self.seed,
-                                               step=ordinal << 32, step_dev=self.step_devs[k])
-            entry = [desc, dev, None, 0]
-            self.cache[key] = entry
-        desc, dev = entry[0], entry[1]
-        st.wait_stream(torch.cuda.current_stream(self.device))
-        capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
-        self.pending[k] = True
+            entry = self._entry(x, out, n, key)
+        _, ref, dev, k, nsc, handle = entry
+        cur = torch.cuda.current_stream(self.device).cuda_stream
+        if k == 0 and self.inline_first:
+            # the first bucket of every round of `streams` goes to the caller's own stream: nothing to order, and ordering a
+            # worker stream after the caller's costs the host more than enqueueing the bucket's four kernels does
+            if self.pending[0]:                 # (a recorded step ran on the worker stream of this slot)
+                if self._order(cur, self.streams[0].cuda_stream, dev):
+                    raise RuntimeError(self.capi.lib().dq_last_error().decode())
+                self.pending[0] = False
+            if self._enqueue(ref, 15, dev, cur):
+                raise RuntimeError(self.capi.lib().dq_last_error().decode())
+        else:
+            if self._order(handle, cur, dev) or self._enqueue(ref, 15, dev, handle):
+                raise RuntimeError(self.capi.lib().dq_last_error().decode())
+            self.pending[k] = True
         if self.hist is not None:
             self.hist.count += nsc
         self.superchunks += nsc
@@ -449,15 +482,12 @@ class SinglePassBuckets(object):
         if graphs is None:
             # per stream: the buckets that go to it, in order, recorded as one graph
             share = [[] for _ in self.streams]
-            for x, o in pairs:
-                n = x.numel()
-                ordinal = self.ordinals.setdefault((x.data_ptr(), n), len(self.ordinals))
-                k = ordinal % len(self.streams)
-                item = self.cache.get((x.data_ptr(), o.data_ptr(), n, x.dtype, k))
+            for (x, o), bkey in zip(pairs, key):
+                item = self.cache.get(bkey)
                 if item is None:                # (cannot happen after a first eager pass with unchanged scratch)
                     self.run(x, o)
-                    item = self.cache[(x.data_ptr(), o.data_ptr(), n, x.dtype, k)]
-                share[k].append(item)
+                    item = self.cache[bkey]
+                share[item[3]].append(item)
             self.join()
             graphs = []
             for k, st in enumerate(self.streams):
@@ -467,8 +497,9 @@ class SinglePassBuckets(object):
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.stream(st):
                     with torch.cuda.graph(g, stream=st):
-                        for desc, dev, _, _ in share[k]:
-                            self.capi.dynamic_bitrate_bucket(desc, dev, stream=st.cuda_stream)
+                        for item in share[k]:
+                            if self._enqueue(item[1], 15, item[2], item[5]):
+                                raise RuntimeError(self.capi.lib().dq_last_error().decode())
                 graphs.append(g)
             entry[0] = graphs
         # one event for all streams, recorded before the first replay: an event recorded on the caller's stream between
@@ -495,8 +526,11 @@ class SinglePassBuckets(object):
         return self.scratch[k]["work"][:4]
 
     def join(self):
-        cur = torch.cuda.current_stream(self.device)
+        """the caller's current stream waits for everything enqueued so far"""
+        cur = torch.cuda.current_stream(self.device).cuda_stream
+        index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         for k, st in enumerate(self.streams):
             if self.pending[k]:
-                cur.wait_stream(st)
+                if self._order(cur, st.cuda_stream, index):
+                    raise RuntimeError(self.capi.lib().dq_last_error().decode())
                 self.pending[k] = False

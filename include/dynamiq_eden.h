@@ -380,6 +380,14 @@ int dq_dynamic_bitrate_bucket(const dq_bucket_t *bucket, int stages, int device,
  * both streams and creates events: a set-up call, not for stream capture. */
 int dq_streams_overlap(dq_stream_t a, dq_stream_t b, int device, int *overlap);
 
+/* No counterpart in the reference.  `stream` waits for everything enqueued on
+ * `after` so far (what a framework's wait_stream does), through an event taken
+ * from a ring the library keeps per device: nothing is created after the first
+ * 64 calls on a device, and the call costs the host two runtime calls.  A
+ * caller that hands each bucket to a worker stream as it becomes ready uses
+ * it in place of creating an event per bucket.  Not for stream capture. */
+int dq_stream_order_after(dq_stream_t stream, dq_stream_t after, int device);
+
 /* ---- consumers of the rotated vector: EDEN and THC ----------------------
  *
  * "reference" here: cuda_kernels/src/srrcomp/srrcomp.py (EDEN) and

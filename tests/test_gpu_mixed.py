@@ -589,3 +589,26 @@ def test_streams_of_the_pipeline_object_run_side_by_side(capi):
         with torch.cuda.stream(extra):
             scratch.add_(1.0)
         torch.cuda.synchronize()
+
+
+def test_stream_order_after_orders_two_streams(capi):
+    """dq_stream_order_after: work enqueued on the waiting stream afterwards sees what the other stream had been given
+    before the call -- also on the 65th and later calls, when the library's ring of events is being reused"""
+    index = torch.cuda.current_device()
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    big = torch.zeros(1 << 24, device=DEV)
+    flag = torch.zeros(8, device=DEV)
+    seen = torch.zeros(200, 8, device=DEV)
+    torch.cuda.synchronize()
+    for k in range(200):
+        with torch.cuda.stream(a):
+            for _ in range(3):
+                big.add_(1.0)                 # something for the flag's writer to queue behind
+            flag.fill_(float(k + 1))
+        capi.stream_order_after(b, a, index)
+        with torch.cuda.stream(b):
+            seen[k].copy_(flag)
+        capi.stream_order_after(a, b, index)  # the next round's fill must not overtake this copy
+    torch.cuda.synchronize()
+    assert torch.equal(seen[:, 0].cpu(), torch.arange(1, 201, dtype=torch.float32))
+    capi.stream_order_after(a, a, index)      # a stream after itself: nothing to do

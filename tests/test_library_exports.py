@@ -112,6 +112,7 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_scaling_decompress_irht(P, P, 1, P, 1024, 96, F1, 4, 0, 2, S), "power of 2")
     err(L.dq_pack_signs(P, N, 100, 0, S), "null pointer")
     err(L.dq_streams_overlap(S, S, 0, None), "null pointer")
+    err(L.dq_stream_order_after(S, S, -1), "device")
     err(L.dq_rand_diag_bits(P, 100, 1, 0, S), "multiple of 256")
     err(L.dq_rand_diag_bits(N, 256, 1, 0, S), "null pointer")
     err(L.dq_pack_signs(P, P, 0, 0, S), "n must be positive")
