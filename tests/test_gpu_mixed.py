@@ -612,3 +612,45 @@ def test_stream_order_after_orders_two_streams(capi):
     torch.cuda.synchronize()
     assert torch.equal(seen[:, 0].cpu(), torch.arange(1, 201, dtype=torch.float32))
     capi.stream_order_after(a, a, index)      # a stream after itself: nothing to do
+
+
+@pytest.mark.parametrize("streams", [1, 2, 3])
+def test_single_pass_buckets_alternating_between_recorded_and_eager_steps(capi, streams):
+    """the first slot of the pipeline object runs on the caller's stream when a bucket is enqueued eagerly and on its worker
+    stream when a recorded step is replayed: steps that alternate between the two (and a change of u in between) still
+    give the outputs of the four calls on every step"""
+    from dynamiq_sigcomm_artifact_amd.dynamiq_pipeline import SinglePassBuckets
+    sizes = [256 * 200, 256 * 200, 256 * 120 + 3, 256 * 200, 256 * 64]
+    xs = [_llama_like(n, 60 + k) for k, n in enumerate(sizes)]
+    outs = [torch.zeros_like(x) for x in xs]
+    seed, u = 4, 6.5
+    pipe = SinglePassBuckets(DEV, strategy=2, seed=seed, streams=streams, graphs=True, u=u)
+    pairs = list(zip(xs, outs))
+    modes = ["all", "all", "all", "each", "all", "each", "each", "all", "each", "all"]
+    x_then = [[None] * len(xs) for _ in modes]
+    o_then = [[None] * len(xs) for _ in modes]
+    us = []
+    # no synchronisation between the steps: only the object's own ordering keeps them apart
+    for step, mode in enumerate(modes, start=1):
+        if step == 5:
+            u = 7.25
+            pipe.set_u(u)
+        us.append(u)
+        pipe.begin_step()
+        for k, x in enumerate(xs):
+            x.mul_(1.125)
+            x_then[step - 1][k] = x.clone()
+        if mode == "all":
+            pipe.run_all(pairs)
+        else:
+            for x, o in pairs:
+                pipe.run(x, o)
+        pipe.join()
+        for k, o in enumerate(outs):
+            o_then[step - 1][k] = o.clone()
+    torch.cuda.synchronize()
+    for step, mode in enumerate(modes, start=1):
+        for k in range(len(xs)):
+            x = x_then[step - 1][k]
+            want = _four_calls(capi, x, x.numel(), us[step - 1], 2, seed, (k << 32) + step)[5]
+            assert torch.equal(bits_t(o_then[step - 1][k]), bits_t(want)), (step, mode, k)
