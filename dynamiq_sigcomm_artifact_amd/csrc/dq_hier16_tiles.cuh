@@ -126,14 +126,20 @@ __device__ __forceinline__ void center_chunk(Raw16<DT> &v, const void *src, int6
 // Quantise the wave's chunks (lane = chunk, 16 values in v, 16 uniform values in r; lanes of rows at or beyond
 // rows_here hold zeros) and stream the run of rows_here records to gout.  win_out: Rec<NBITS>::WIN bytes of LDS,
 // 16-byte aligned, owned by this wave.
-template <int NBITS, bool MEE, class RV, class RR>
+// WROWS < 4: the window holds WROWS records and the run leaves in 4 / WROWS pieces (win_out: window_bytes<NBITS>(WROWS)),
+// for kernels that cannot spare the LDS of a four-record window.
+template <int NBITS> __host__ __device__ constexpr int window_bytes(int rows)
+{
+    return ((rows * Rec<NBITS>::REC + 15 + 15) / 16) * 16;
+}
+
+template <int NBITS, bool MEE, int WROWS = kRowsPerWave, class RV, class RR>
 __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const MeeArg<NBITS, MEE> &mp, uint8_t *gout,
                                                  int rows_here, uint8_t *win_out, int lane)
 {
     typedef Rec<NBITS> RC;
+    static_assert(WROWS == 1 || WROWS == 2 || WROWS == 4, "the window holds 1, 2 or 4 records");
     const int row = lane >> 4, j = lane & 15;
-    const bool active = row < rows_here;
-    const int total = rows_here * RC::REC;
 
     uint32_t w[RC::WORDS], q, ub;
     const uint32_t amax = v.absmax_bits();
@@ -143,17 +149,24 @@ __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const
     else
         chunk_encode_guarded<NBITS, MEE>(v, r, mp, w, q, ub);
 
-    const int mis = (int)(reinterpret_cast<uintptr_t>(gout) & 15);
-    if (active) {
-        uint8_t *rec = win_out + mis + row * RC::REC;
-        chunk_write<NBITS>(rec + j * RC::CB, w, q);
-        if (j == 0) {
-            rec[16 * RC::CB] = (uint8_t)ub;
-            rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+#pragma unroll
+    for (int p = 0; p < kRowsPerWave; p += WROWS) {
+        if (p >= rows_here) break;
+        uint8_t *g = gout + p * RC::REC;
+        const int rows_now = min(WROWS, rows_here - p);
+        const int mis = (int)(reinterpret_cast<uintptr_t>(g) & 15);
+        if (row >= p && row < p + rows_now) {
+            uint8_t *rec = win_out + mis + (row - p) * RC::REC;
+            chunk_write<NBITS>(rec + j * RC::CB, w, q);
+            if (j == 0) {
+                rec[16 * RC::CB] = (uint8_t)ub;
+                rec[16 * RC::CB + 1] = (uint8_t)(ub >> 8);
+            }
         }
+        wave_lds_sync();
+        window_flush(win_out, g, mis, rows_now * RC::REC, lane);
+        if (WROWS < kRowsPerWave) wave_lds_sync(); // the window is written again
     }
-    wave_lds_sync();
-    window_flush(win_out, gout, mis, total, lane);
 }
 
 // The row list of the tiles a wave works through.  A wave that takes several tiles fetches their entries with one load

@@ -534,30 +534,32 @@ __device__ __forceinline__ void half_block_stages(float (&v)[16], float *lds, in
 }
 
 // The forward kernel takes blocks of 2^(HB + 1) in two halves of 2^HB, one chunk of each half per thread: HB = 14 for
-// blocks of 2^15 (1024 threads; a CU holds at most two such workgroups) and HB = 13 for blocks of 2^14 (512 threads, up
-// to four per CU; as one tile those blocks need 1024 threads of which half sit idle in both LDS passes).
+// blocks of 2^15 (1024 threads; a CU holds at most two such workgroups), HB = 13 for blocks of 2^14 (512 threads, up to
+// four per CU; as one tile those blocks need 1024 threads of which half sit idle in both LDS passes), ... HB = 10 for
+// blocks of 2^11 on one wave.
 //
-// LDS: the half tile and, where the second half is parked in it through the quantiser, the record windows of the waves
-// behind it.  Parking needs the sum to leave room for as many workgroups as the thread count allows (two of 80 KB for
-// HB = 14: up to 6-bit codes); HB = 13 always parks (three workgroups per CU instead of four from 6-bit codes on).
-template <int NBITS, int HB> __host__ __device__ constexpr size_t split_lds_bytes(bool parked)
+// LDS: the half tile, in which the second half is parked through the quantiser of the first, and the record windows of
+// the waves behind it.  For HB = 14 the sum must leave room for two workgroups per CU (80 KB each).
+// records per window: four (one run per wave) where two workgroups of 2^15-element blocks still fit a CU with the parked half,
+// two for the wider codes (7 and 8 bits), whose runs then leave in two pieces
+template <int NBITS, int HB> __host__ __device__ constexpr int split_window_rows()
 {
-    return (size_t)padded_tile_floats(HB) * sizeof(float) + (parked ? ((1 << (HB - 4)) / 64) * Rec<NBITS>::WIN : 0);
+    return HB < kHalfBits || (size_t)padded_tile_floats(HB) * sizeof(float) + ((1 << (HB - 4)) / 64) * window_bytes<NBITS>(4) <= 80 * 1024 ? 4 : 2;
 }
-template <int NBITS, int HB> __host__ __device__ constexpr bool split_parks()
+template <int NBITS, int HB> __host__ __device__ constexpr size_t split_lds_bytes()
 {
-    return HB < kHalfBits || split_lds_bytes<NBITS, HB>(true) <= 80 * 1024;
+    return (size_t)padded_tile_floats(HB) * sizeof(float) + ((1 << (HB - 4)) / 64) * window_bytes<NBITS>(split_window_rows<NBITS, HB>());
 }
 
 // PAIR = false: the two halves are two whole blocks of 2^HB (no pairing stage): blocks of 2^10 on one wave.
 template <int RDT, int NBITS, bool MEE, int HB, bool PAIR = true>
-__global__ __launch_bounds__(1 << (HB - 4), (split_parks<NBITS, HB>() ? 8 : 4)) void rht_compress_split_kernel(
+__global__ __launch_bounds__(1 << (HB - 4), 8) void rht_compress_split_kernel(
     const float *__restrict__ x, uint8_t *__restrict__ dst, const void *__restrict__ rnd, RhtTileArgs a, int rvec, RandKey key,
     MeeArg<NBITS, MEE> mp)
 {
     typedef Rec<NBITS> RC;
-    constexpr bool kParks = split_parks<NBITS, HB>();
     constexpr int kThreads = 1 << (HB - 4), kWaves = kThreads / 64;
+    constexpr int kWinRows = split_window_rows<NBITS, HB>();
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t origin = (int64_t)blockIdx.x << (HB + 1);
@@ -567,36 +569,24 @@ __global__ __launch_bounds__(1 << (HB - 4), (split_parks<NBITS, HB>() ? 8 : 4)) 
     butterflies<4>(va);
     butterflies<4>(vb);
     half_block_stages<HB>(va, lds, tid);
+    // The second half stays in the LDS after its stages: the thread pairs its two chunks there, keeps the sums and
+    // leaves the differences in its own slot until the sums are quantised.  With both halves in registers through the
+    // quantiser the kernel needs more than its 64 registers, and what it spills travels to memory and back (measured
+    // at 2^28 elements in blocks of 2^15: 757 MB written and 1.52 GB read for 153 MB of records and 1.11 GB of input).
+    // The record windows then lie behind the tile instead of inside it.
     float *mine = lds + chunk_word(tid);
-    uint8_t *win_out;
-    if constexpr (kParks) {
-        // The second half stays in the LDS after its stages: the thread pairs its two chunks there, keeps the sums
-        // and leaves the differences in its own slot until the sums are quantised.  With both halves in registers
-        // through the quantiser the kernel needs more than its 64 registers, and what it spills travels to memory
-        // and back (measured at 2^28 elements in blocks of 2^15: 757 MB written and 1.52 GB read for 153 MB of records
-        // and 1.11 GB of input).  The record windows then lie behind the tile instead of inside it.
 #pragma unroll
-        for (int i = 0; i < 16; i++) mine[i] = vb[i];
-        fwht_lds_stages_after4(lds, HB, HB, tid, kThreads); // ends with a barrier; own slot only from here on
-        if constexpr (PAIR) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float p = va[i], q = mine[i];
-                va[i] = p + q;
-                mine[i] = p - q;
-            }
-        }
-        win_out = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(HB)) + wave * RC::WIN;
-    } else {
-        half_block_stages<HB>(vb, lds, tid);
+    for (int i = 0; i < 16; i++) mine[i] = vb[i];
+    fwht_lds_stages_after4(lds, HB, HB, tid, kThreads); // ends with a barrier; own slot only from here on
+    if constexpr (PAIR) {
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const float p = va[i], q = vb[i];
+            const float p = va[i], q = mine[i];
             va[i] = p + q;
-            vb[i] = p - q;
+            mine[i] = p - q;
         }
-        win_out = reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN;
     }
+    uint8_t *win_out = reinterpret_cast<uint8_t *>(lds + padded_tile_floats(HB)) + wave * window_bytes<NBITS>(kWinRows);
     // quantise: the wave's 64 chunks of a half are 4 superchunks, one run of records
 #pragma unroll
     for (int h = 0; h < 2; h++) {
@@ -608,15 +598,8 @@ __global__ __launch_bounds__(1 << (HB - 4), (split_parks<NBITS, HB>() ? 8 : 4)) 
         else
             r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float t;
-            if constexpr (kParks)
-                t = h ? mine[i] : va[i];
-            else
-                t = h ? vb[i] : va[i];
-            v.w[i] = __float_as_uint(t * a.scale);
-        }
-        encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, kRowsPerWave, win_out, threadIdx.x & 63);
+        for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint((h ? mine[i] : va[i]) * a.scale);
+        encode_store_run<NBITS, MEE, kWinRows>(v, r, mp, dst + sc0 * RC::REC, kRowsPerWave, win_out, threadIdx.x & 63);
         wave_lds_sync(); // the window is reused for the other half
     }
 }
@@ -784,7 +767,7 @@ hipError_t run_compress(const float *src, const void *sign, int sign_bits, uint8
     if (g.a.kb == 10 && (n & 2047) == 0) {
         // blocks of 2^10, two per wave
         auto kernel = rht_compress_split_kernel<RDT, NBITS, MEE, 10, false>;
-        const size_t lds = split_lds_bytes<NBITS, 10>(true);
+        const size_t lds = split_lds_bytes<NBITS, 10>();
         hipLaunchKernelGGL(kernel, dim3((unsigned)(n >> 11)), dim3(64), lds, stream, src, dst, rnd, g.a, aligned16(rnd) ? 1 : 0, key,
                            make_arg<NBITS, MEE>(mp));
         return hipGetLastError();
@@ -800,16 +783,15 @@ hipError_t run_compress(const float *src, const void *sign, int sign_bits, uint8
         };
         switch (g.a.kb) {
         case kSplitBits:
-            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits>,
-                          split_lds_bytes<NBITS, kHalfBits>(split_parks<NBITS, kHalfBits>()), kHalfBits);
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits>, split_lds_bytes<NBITS, kHalfBits>(), kHalfBits);
         case kSplitBits - 1:
-            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 1>, split_lds_bytes<NBITS, kHalfBits - 1>(true), kHalfBits - 1);
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 1>, split_lds_bytes<NBITS, kHalfBits - 1>(), kHalfBits - 1);
         case kSplitBits - 2:
-            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 2>, split_lds_bytes<NBITS, kHalfBits - 2>(true), kHalfBits - 2);
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 2>, split_lds_bytes<NBITS, kHalfBits - 2>(), kHalfBits - 2);
         case kSplitBits - 3:
-            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 3>, split_lds_bytes<NBITS, kHalfBits - 3>(true), kHalfBits - 3);
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 3>, split_lds_bytes<NBITS, kHalfBits - 3>(), kHalfBits - 3);
         default:
-            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 4>, split_lds_bytes<NBITS, kHalfBits - 4>(true), kHalfBits - 4);
+            return launch(rht_compress_split_kernel<RDT, NBITS, MEE, kHalfBits - 4>, split_lds_bytes<NBITS, kHalfBits - 4>(), kHalfBits - 4);
         }
     }
     if (g.a.kt >= kSplitBits) return hipErrorInvalidValue; // one run of records per wave needs tiles of at most 2^14
