@@ -48,7 +48,12 @@ template <int M> __device__ __forceinline__ void butterflies(float (&v)[1 << M])
 // word offset of element j of a tuple of pass <P, M> from the tuple's first element: the index grows by j 2^P
 template <int P> __device__ __forceinline__ constexpr int tuple_step(int j)
 {
-    return P == 0 ? j : (P >= 5 ? j * ((1 << P) + (1 << (P - 5))) : 16 * j + (j >> 1)); // P == 4: bit 4 of the index is bit 0 of j
+    if constexpr (P == 0)
+        return j;
+    else if constexpr (P >= 5)
+        return j * ((1 << P) + (1 << (P - 5)));
+    else
+        return 16 * j + (j >> 1); // P == 4: bit 4 of the index is bit 0 of j
 }
 
 // Index of the first element of tuple u of a pass over index bits [P, P + M): the low P bits of u are the low P index
