@@ -133,7 +133,7 @@ template <int NBITS> __host__ __device__ constexpr int window_bytes(int rows)
     return ((rows * Rec<NBITS>::REC + 15 + 15) / 16) * 16;
 }
 
-template <int NBITS, bool MEE, int WROWS = kRowsPerWave, class RV, class RR>
+template <int NBITS, bool MEE, int WROWS = kRowsPerWave, bool STREAM = true, class RV, class RR>
 __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const MeeArg<NBITS, MEE> &mp, uint8_t *gout,
                                                  int rows_here, uint8_t *win_out, int lane)
 {
@@ -164,7 +164,7 @@ __device__ __forceinline__ void encode_store_run(const RV &v, const RR &r, const
             }
         }
         wave_lds_sync();
-        window_flush(win_out, g, mis, rows_now * RC::REC, lane);
+        window_flush<STREAM>(win_out, g, mis, rows_now * RC::REC, lane);
         if (WROWS < kRowsPerWave) wave_lds_sync(); // the window is written again
     }
 }

@@ -206,7 +206,7 @@ __global__ __attribute__((amdgpu_waves_per_eu(8, 8))) void rht_compress_kernel(c
     }
     __syncthreads();
     if (rows_here > 0)
-        encode_store_run<NBITS, MEE>(v, r, mp, dst + sc0 * RC::REC, rows_here, reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN, threadIdx.x & 63);
+        encode_store_run<NBITS, MEE, kRowsPerWave, false>(v, r, mp, dst + sc0 * RC::REC, rows_here, reinterpret_cast<uint8_t *>(lds) + wave * RC::WIN, threadIdx.x & 63);
 }
 
 template <int NBITS, bool MEE>
@@ -599,7 +599,7 @@ __global__ __launch_bounds__(1 << (HB - 4), 8) void rht_compress_split_kernel(
             r.load(rnd, (sc0 * 16 + lane) * 16, rvec);
 #pragma unroll
         for (int i = 0; i < 16; i++) v.w[i] = __float_as_uint((h ? mine[i] : va[i]) * a.scale);
-        encode_store_run<NBITS, MEE, kWinRows>(v, r, mp, dst + sc0 * RC::REC, kRowsPerWave, win_out, threadIdx.x & 63);
+        encode_store_run<NBITS, MEE, kWinRows, false>(v, r, mp, dst + sc0 * RC::REC, kRowsPerWave, win_out, threadIdx.x & 63);
         wave_lds_sync(); // the window is reused for the other half
     }
 }

@@ -279,7 +279,9 @@ __device__ __forceinline__ int window_commit(uint8_t *win, const WinRegs &r, con
     return mis;
 }
 
-// stream `total` bytes from win[mis ...] to g (g & 15 == mis)
+// stream `total` bytes from win[mis ...] to g (g & 15 == mis).  STREAM: whole 128-byte lines leave with the streaming hint
+// (for kernels that the memory system bounds; the address test per vector costs a kernel bound by its arithmetic 1-4 %).
+template <bool STREAM = true>
 __device__ __forceinline__ void window_flush(const uint8_t *win, uint8_t *g, int mis, int total, int lane)
 {
     int head = (16 - mis) & 15;
@@ -289,7 +291,19 @@ __device__ __forceinline__ void window_flush(const uint8_t *win, uint8_t *g, int
     if (lane < head) g[lane] = win[mis + lane];
     const uint4 *wv = reinterpret_cast<const uint4 *>(win + mis + head);
     uint4 *gv = reinterpret_cast<uint4 *>(g + head);
-    for (int v = lane; v < (body >> 4); v += 64) gv[v] = wv[v];
+    // 128-byte lines that lie wholly inside [g, g + total) leave with the streaming hint: they go out while the kernel
+    // runs instead of waiting in the L2 for the write-back at its end.  The ragged ends share their lines with the
+    // neighbouring waves' runs and are stored plainly, so that the L2 merges the pieces (as streaming stores they
+    // would reach memory as partial writes: measured slower than no hint at all).
+    const uintptr_t first = (reinterpret_cast<uintptr_t>(g) + 127) & ~(uintptr_t)127;
+    const uintptr_t last = (reinterpret_cast<uintptr_t>(g) + total) & ~(uintptr_t)127;
+    for (int v = lane; v < (body >> 4); v += 64) {
+        const uintptr_t at = reinterpret_cast<uintptr_t>(gv + v);
+        if (STREAM && at >= first && at < last)
+            stream_store(gv + v, wv[v]);
+        else
+            gv[v] = wv[v];
+    }
     const int tl = lane - 32; // lanes 32.. store the tail so head and tail overlap in time
     if (tl >= 0 && tl < tail) g[head + body + tl] = win[mis + head + body + tl];
 }
