@@ -653,6 +653,25 @@ def main():
     comp_ms = median_ms(compress, steps, reps)
     dec_ms = median_ms(decompress, steps, reps)
     torch.cuda.synchronize()
+
+    # ---- what launches of these shapes cost with the arithmetic taken away: the same tiles, the same accesses, over the same
+    #      ring (the packed buffers of the ring hold meaningless bytes afterwards; every later use writes them first) ----
+    floor_tiles = n // 1024
+    run_bytes = nb * 1024 // n if strategy in (2, 3) and n % 1024 == 0 and nbits in (2, 3, 4, 5, 6, 7, 8) else 0
+    comp_floor_ms = dec_floor_ms = None
+    if run_bytes and run_bytes % 8 == 0:
+        def compress_floor():
+            s_, r_, p_, _ = ring.next()
+            capi.tile_io_floor(0, s_, r_ if args.rand == "pool" else None, p_, run_bytes, floor_tiles)
+
+        def decompress_floor():
+            _, _, p_, o_ = ring.next()
+            capi.tile_io_floor(1, o_, None, p_, run_bytes, floor_tiles)
+
+        comp_floor_ms = median_ms(compress_floor, steps, reps)
+        dec_floor_ms = median_ms(decompress_floor, steps, reps)
+        torch.cuda.synchronize()
+
     t0 = time.perf_counter()
     eager_ms_per_step = eager_ms(step_ring, steps)
     torch.cuda.synchronize()
@@ -828,12 +847,21 @@ def main():
             "avg_launch_ms": round(comp_hbm_ms, 5),
             "avg_launch_ms_cache_assisted": round(comp_ms, 5),
             "timing": "median of %d replays of a HIP graph of %d launches" % (reps, steps),
+            "io_floor": None if comp_floor_ms is None else {
+                "avg_launch_ms": round(comp_floor_ms, 5),
+                "frac": round(comp_bytes / (comp_floor_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "kernel_over_floor": round(comp_hbm_ms / comp_floor_ms, 3),
+                "what": "dq_tile_io_floor: a kernel of the same launch shape (one wave per tile of 1,024 elements) that reads and "
+                        "writes the same bytes of the same ring with the same access pattern and computes nothing, timed the same way",
+            },
         },
         "kernels": {
             "compress": {"ms": round(comp_hbm_ms, 5), "algorithmic_GBps": round(comp_gbs, 1), "frac_hbm": round(comp_gbs / HBM_PEAK_GBS, 4),
-                         "ms_cache_assisted": round(comp_ms, 5)},
+                         "ms_cache_assisted": round(comp_ms, 5),
+                         "io_floor_ms": None if comp_floor_ms is None else round(comp_floor_ms, 5)},
             "decompress": {"ms": round(dec_hbm_ms, 5), "algorithmic_GBps": round(dec_gbs, 1), "frac_hbm": round(dec_gbs / HBM_PEAK_GBS, 4),
-                           "ms_cache_assisted": round(dec_ms, 5)},
+                           "ms_cache_assisted": round(dec_ms, 5),
+                           "io_floor_ms": None if dec_floor_ms is None else round(dec_floor_ms, 5)},
         },
         "frac_hbm_roundtrip": round((comp_bytes + dec_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "ms_per_step_replays": [round(t, 5) for t in step_hbm],

@@ -33,6 +33,7 @@ HIP_SOURCES = [
     "dq_packing.hip",
     "dq_eden.hip",
     "dq_streams.hip",
+    "dq_io_floor.hip",
 ]
 
 HIPCC_FLAGS = [

@@ -26,7 +26,7 @@ EXPORTS = [
     "dq_group_plan_stats_dev_u", "dq_group_plan_sorted", "dq_bitrate_hist_ints", "dq_norm_histogram", "dq_bitrate_search",
     "dq_scaling_compress_rows", "dq_scaling_dec_comp_rows", "dq_scaling_decompress_rows",
     "dq_mixed_required_bytes", "dq_mixed_compress", "dq_mixed_decompress", "dq_superchunk_stats",
-    "dq_dynamic_bitrate_bucket", "dq_streams_overlap", "dq_stream_order_after",
+    "dq_dynamic_bitrate_bucket", "dq_streams_overlap", "dq_stream_order_after", "dq_tile_io_floor",
     "dq_superchunk_mean_center", "dq_superchunk_add_mean_copy",
     "dq_hadamard", "dq_rht_blocked", "dq_rand_diag", "dq_rand_diag_bits", "dq_rht_scaling_compress", "dq_rht_scaling_compress_mfma16", "dq_scaling_decompress_irht", "dq_pack_signs",
     "dq_bins_to_bits", "dq_bits_to_bins", "dq_quantization",
@@ -123,6 +123,8 @@ def lib():
         L.dq_superchunk_stats.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
         L.dq_dynamic_bitrate_bucket.restype = i32
         L.dq_dynamic_bitrate_bucket.argtypes = [c.POINTER(Bucket), i32, i32, vp]
+        L.dq_tile_io_floor.restype = i32
+        L.dq_tile_io_floor.argtypes = [i32, vp, i32, vp, i32, vp, i32, i64, i32, vp]
         L.dq_stream_order_after.restype = i32
         L.dq_stream_order_after.argtypes = [vp, vp, i32]
         L.dq_streams_overlap.restype = i32
@@ -483,6 +485,18 @@ def dynamic_bitrate_bucket(desc, device, stages=STAGE_ALL, stream=None):
     """one host call for any run of the stages statistics -> plan -> mixed compress -> mixed decompress of one bucket
     (desc, device: from bucket_descriptor)"""
     _check(lib().dq_dynamic_bitrate_bucket(ctypes.byref(desc), stages, device, _stream(stream)))
+
+
+def tile_io_floor(direction, a, b, run, run_bytes_per_tile, tiles, stream=None):
+    """a launch with the shape and the memory accesses of the chunk-16 codec on `tiles` tiles of 1,024 elements and no
+    arithmetic: direction 0 reads the element tensor a and the pool b (may be None) and writes `run_bytes_per_tile` bytes per
+    tile to `run`; direction 1 reads `run` (and b) and overwrites a.  A measurement aid: what it writes has no meaning."""
+    a_bytes = 1024 * a.element_size()
+    b_bytes = 1024 * b.element_size() if b is not None else 0
+    if a.numel() < 1024 * tiles or (b is not None and b.numel() < 1024 * tiles) or run.numel() * run.element_size() < run_bytes_per_tile * tiles:
+        raise ValueError("a tensor is shorter than tiles * bytes per tile")
+    _call(lib().dq_tile_io_floor, int(direction), _ptr(a), a_bytes, _ptr(b), b_bytes, _ptr(run), int(run_bytes_per_tile),
+          int(tiles), a.device.index, _stream(stream))
 
 
 def stream_order_after(stream, after, device):

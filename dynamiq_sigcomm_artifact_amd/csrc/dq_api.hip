@@ -494,6 +494,22 @@ int dq_stream_order_after(dq_stream_t stream, dq_stream_t after, int device)
     return finish(dq::stream_order_after(static_cast<hipStream_t>(stream), static_cast<hipStream_t>(after), device));
 }
 
+int dq_tile_io_floor(int direction, void *a, int a_bytes_per_tile, const void *b, int b_bytes_per_tile, void *run, int run_bytes_per_tile,
+                     int64_t tiles, int device, dq_stream_t stream)
+{
+    if (direction != 0 && direction != 1) return fail(DQ_ERR_SIZE, "direction must be 0 (encoder shape) or 1 (decoder shape)");
+    if (!dq::tile_io_floor_shape_ok(a_bytes_per_tile, b_bytes_per_tile, run_bytes_per_tile))
+        return fail(DQ_ERR_SIZE, "a_bytes_per_tile must be 2048 or 4096, b_bytes_per_tile 0, 2048 or 4096, run_bytes_per_tile a multiple of 8 up to 8192");
+    if (!(tiles > 0) || tiles > 0x7fffffff) return fail(DQ_ERR_N);
+    if (!a || !run || (b_bytes_per_tile > 0 && !b)) return fail(DQ_ERR_NULL);
+    if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15) || (reinterpret_cast<uintptr_t>(run) & 7))
+        return fail(DQ_ERR_SIZE, "a and b must be 16-byte aligned, run 8-byte aligned");
+    int rc;
+    if ((rc = select_device(device))) return rc;
+    return finish(dq::launch_tile_io_floor(direction, a, a_bytes_per_tile, b, b_bytes_per_tile, run, run_bytes_per_tile, tiles,
+                                           static_cast<hipStream_t>(stream)));
+}
+
 int dq_dynamic_bitrate_bucket(const dq_bucket_t *b, int stages, int device, dq_stream_t stream)
 {
     if (!b) return fail(DQ_ERR_NULL);

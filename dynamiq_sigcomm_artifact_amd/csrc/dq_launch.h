@@ -159,6 +159,11 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
 hipError_t probe_streams_overlap(hipStream_t a, hipStream_t b, int *overlap);
 // `stream` waits for the work enqueued on `after` so far (pooled event, no allocation after the first 64 calls per device)
 hipError_t stream_order_after(hipStream_t stream, hipStream_t after, int device);
+// a kernel with the access pattern of the chunk-16 codec on `tiles` tiles and no arithmetic (dq_io_floor.hip); direction 0
+// reads a and b and writes run, direction 1 reads run (and b) and writes a
+bool tile_io_floor_shape_ok(int a_bytes, int b_bytes, int run_bytes);
+hipError_t launch_tile_io_floor(int direction, void *a, int a_bytes, const void *b, int b_bytes, void *run, int run_bytes, int64_t tiles,
+                                hipStream_t stream);
 
 // the same launches with the partial sums in the library's own static device array (no allocation anywhere);
 // `device` must be current

@@ -388,6 +388,24 @@ int dq_streams_overlap(dq_stream_t a, dq_stream_t b, int device, int *overlap);
  * it in place of creating an event per bucket.  Not for stream capture. */
 int dq_stream_order_after(dq_stream_t stream, dq_stream_t after, int device);
 
+/* No counterpart in the reference: a measurement aid.  Launches a kernel with
+ * the launch shape and the memory accesses of the chunk-16 codec kernels -- one
+ * wave per tile of 1,024 elements, each lane reading its chunk as 16-byte
+ * pieces, each wave writing one unaligned run of record bytes -- and no
+ * arithmetic beyond an exclusive-or of everything a lane loaded, which its
+ * stores carry.  Timed over the same buffers as a codec call, it tells how
+ * much of that call's time the launch itself and its memory traffic account
+ * for.  direction 0 (encoder shape): per tile read a_bytes_per_tile from `a`
+ * and b_bytes_per_tile from `b`, write run_bytes_per_tile to `run`.
+ * direction 1 (decoder shape): per tile read the run (and `b` when
+ * b_bytes_per_tile > 0), write `a` with streaming stores.  a_bytes_per_tile
+ * is 2048 or 4096 (1,024 bf16 or fp32 elements), b_bytes_per_tile 0, 2048 or
+ * 4096, run_bytes_per_tile a multiple of 8 up to 8192 (4 * record bytes).
+ * What it writes has no meaning; it overwrites `run` (direction 0) or `a`
+ * (direction 1) over tiles * bytes_per_tile bytes. */
+int dq_tile_io_floor(int direction, void *a, int a_bytes_per_tile, const void *b, int b_bytes_per_tile,
+                     void *run, int run_bytes_per_tile, int64_t tiles, int device, dq_stream_t stream);
+
 /* ---- consumers of the rotated vector: EDEN and THC ----------------------
  *
  * "reference" here: cuda_kernels/src/srrcomp/srrcomp.py (EDEN) and

@@ -255,3 +255,46 @@ def test_quantization_compression_module_stream(eden_utils, oracle):
         eden_utils.quantization_compression(q, 0.5, 10.0)
         want = oracle.quantization(v.numpy(), 0.5, 10.0, (123 + k * 0x9E3779B97F4A7C15) & (2 ** 64 - 1))
         assert (q.cpu().numpy() == want).all()
+
+
+@pytest.mark.parametrize("adt,bdt,run_bytes", [(torch.float32, torch.bfloat16, 584), (torch.bfloat16, torch.bfloat16, 328),
+                                               (torch.bfloat16, None, 1096)])
+def test_tile_io_floor_moves_exactly_the_bytes_of_the_codec_shape(capi, adt, bdt, run_bytes):
+    """dq_tile_io_floor, the launch of the codec's shape without the arithmetic: every store carries the exclusive-or of all
+    a lane loaded (so nothing it claims to read can be left out), it writes tiles * bytes per tile and not a byte more"""
+    tiles = 37
+    g = torch.Generator().manual_seed(run_bytes)
+    a = torch.randn(1024 * tiles, generator=g).to(adt).to(DEV)
+    b = torch.rand(1024 * tiles, generator=g).to(bdt).to(DEV) if bdt is not None else None
+    run = torch.full((run_bytes * tiles + 64,), 0xAB, dtype=torch.uint8, device=DEV)
+
+    def lane_words(t):          # [tiles, 64]: exclusive-or of the 32-bit words of each lane's chunk of 16 elements
+        w = t.cpu().contiguous().view(torch.uint8).numpy().view(np.uint32).reshape(tiles, 64, -1)
+        return np.bitwise_xor.reduce(w, axis=2)
+
+    x = np.arange(64, dtype=np.uint32)[None, :] ^ lane_words(a)
+    if b is not None:
+        x = x ^ lane_words(b)
+    capi.tile_io_floor(0, a, b, run, run_bytes, tiles)
+    got = run.cpu().numpy()
+    assert (got[run_bytes * tiles:] == 0xAB).all()
+    pieces = got[:run_bytes * tiles].view(np.uint32).reshape(tiles, run_bytes // 8, 2)
+    j = np.arange(run_bytes // 8)
+    assert (pieces[:, :, 0] == x[:, j % 64]).all()
+    assert (pieces[:, :, 1] == x[:, j % 64] + (j // 64).astype(np.uint32)[None, :]).all()
+
+    # decoder shape: reads the run just written (and b), overwrites a
+    y = np.broadcast_to(np.arange(64, dtype=np.uint32)[None, :], (tiles, 64)).copy()
+    for jj in range(run_bytes // 8):
+        y[:, jj % 64] ^= pieces[:, jj, 0] ^ pieces[:, jj, 1]
+    if b is not None:
+        y = y ^ lane_words(b)
+    guard = torch.full((1024 * (tiles + 1),), 3.0, dtype=adt, device=DEV)
+    capi.tile_io_floor(1, guard, b, run, run_bytes, tiles)
+    out = guard.cpu().view(torch.uint8).numpy().view(np.uint32).reshape(tiles + 1, -1, 64, 4)   # 16-byte piece 64 k + lane
+    k = np.arange(out.shape[1], dtype=np.uint32)[None, :, None]
+    assert (out[:tiles, :, :, 0] == y[:, None, :]).all() and (out[:tiles, :, :, 1] == y[:, None, :] + 1).all()
+    assert (out[:tiles, :, :, 2] == y[:, None, :] + 2).all() and (out[:tiles, :, :, 3] == y[:, None, :] + 3 + k).all()
+    assert bool((guard[1024 * tiles:] == 3.0).all())
+    with pytest.raises(ValueError):
+        capi.tile_io_floor(0, a, b, run, run_bytes, tiles + 1)

@@ -113,6 +113,12 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_pack_signs(P, N, 100, 0, S), "null pointer")
     err(L.dq_streams_overlap(S, S, 0, None), "null pointer")
     err(L.dq_stream_order_after(S, S, -1), "device")
+    err(L.dq_tile_io_floor(2, P, 4096, P, 2048, P, 584, 10, 0, S), "direction")
+    err(L.dq_tile_io_floor(0, P, 1000, P, 2048, P, 584, 10, 0, S), "a_bytes_per_tile")
+    err(L.dq_tile_io_floor(0, P, 4096, P, 2048, P, 580, 10, 0, S), "multiple of 8")
+    err(L.dq_tile_io_floor(0, P, 4096, P, 2048, P, 584, 0, 0, S), "n must be positive")
+    err(L.dq_tile_io_floor(0, P, 4096, N, 2048, P, 584, 10, 0, S), "null pointer")
+    err(L.dq_tile_io_floor(0, ctypes.c_void_p(0x1008), 4096, N, 0, P, 584, 10, 0, S), "aligned")
     err(L.dq_rand_diag_bits(P, 100, 1, 0, S), "multiple of 256")
     err(L.dq_rand_diag_bits(N, 256, 1, 0, S), "null pointer")
     err(L.dq_pack_signs(P, P, 0, 0, S), "n must be positive")
