@@ -386,7 +386,12 @@ __device__ __forceinline__ bool is_subnormal(float q) { return (__float_as_uint(
 __device__ __forceinline__ float div_exact(float a, float b, double yb)
 {
     float q = div_by(a, yb);
-    if (is_subnormal(q)) q = a / b;
+    if (__builtin_amdgcn_ballot_w64(is_subnormal(q)) != 0) {
+        // a branch of the wave, and one the compiler keeps: the division is a dozen instructions, which it would otherwise
+        // execute for every element and select from afterwards
+        asm volatile("");
+        if (is_subnormal(q)) q = a / b;
+    }
     return q;
 }
 
@@ -498,12 +503,16 @@ __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d
     const float rd = __builtin_amdgcn_rcpf(d);
     const float rc = MEE ? (float)mp.inv_c : 0.0f, rl2b = MEE ? (float)mp.inv_l2b : 0.0f;
     constexpr float kDelta = EstimateGuard<NBITS, MEE>::kDelta;
-    bool doubt[16], any = false;
+    // (the wave-wide view of each flag is taken where the comparison is made: there it is the comparison's own lane mask, and
+    // the tests further down are scalar)
+    bool doubt[16];
+    uint64_t lanes_in_doubt[16], any = 0;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const float t = estimate_coordinate<NBITS, MEE>(v, r, i, rd, rc, rl2b);
         doubt[i] = __builtin_amdgcn_fractf(t) < 2.0f * kDelta;
-        any |= doubt[i];
+        lanes_in_doubt[i] = __builtin_amdgcn_ballot_w64(doubt[i]);
+        any |= lanes_in_doubt[i];
         if (kFields)
             words_put<NBITS>(w, i, (uint32_t)(int)t);
         else
@@ -513,11 +522,11 @@ __device__ __forceinline__ void estimate_codes(const RV &v, const RR &r, float d
 #pragma unroll
         for (int k = 0; k < Rec<NBITS>::WORDS; k++) w[k] = clamp_fields<kFields ? NBITS : 2>(w[k]);
     }
-    if (__builtin_amdgcn_ballot_w64(any) != 0) {
+    if (any != 0) {
         const double yd = recip_f64(d);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            if (__builtin_amdgcn_ballot_w64(doubt[i]) != 0) {
+            if (lanes_in_doubt[i] != 0) {
                 // (among them the zero elements -- padding, sparse input -- whose random value is exactly 0 or 1: their
                 // T is an integer, and the chain's ceil(-r) is 0, or -1 at r = 1)
                 const int sv = exact_code_fast<MEE>(v.get(i), r.get(i), d, yd, mp);
