@@ -23,6 +23,8 @@
 #include "dq_bitwidth.cuh"
 #include "dq_launch.h"
 
+#include <type_traits>
+
 namespace dq {
 
 namespace {
@@ -44,11 +46,14 @@ struct WidthsFromArray {
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
     __device__ __forceinline__ int64_t width(int64_t i) const { return qbits[i]; }
     bool word_aligned() const { return true; }
+    bool quad_aligned() const { return false; }
+    __device__ __forceinline__ uint4 load_quad(int) const { return make_uint4(0, 0, 0, 0); } // (never taken)
+    struct Tally {};
     __device__ __forceinline__ const uint16_t *norm_stats() const { return nullptr; }
     const void *norm_stats_host() const { return nullptr; }
     __device__ __forceinline__ void resolve() {}
     __device__ __forceinline__ void prepare(int *, int, int) const {}
-    __device__ __forceinline__ bool known(int (&t)[2]) const // nothing to search for
+    __host__ __device__ __forceinline__ bool known(int (&t)[2]) const // nothing to search for
     {
         t[0] = t[1] = 0;
         return true;
@@ -78,20 +83,43 @@ struct WidthsFromStats {
         return (int)r >= thr_host[1] ? 8 : ((int)r >= thr_host[0] ? 4 : 2);
     }
     __device__ __forceinline__ void prepare(int *thr, int wave, int lane) const { width_thresholds(u, thr, wave, lane); }
-    __device__ __forceinline__ bool known(int (&t)[2]) const
+    __host__ __device__ __forceinline__ bool known(int (&t)[2]) const
     {
         t[0] = thr_host[0];
         t[1] = thr_host[1];
         return thr_host[0] >= 0;
     }
     bool word_aligned() const { return (reinterpret_cast<uintptr_t>(stats) & 3) == 0; } // load() reads pairs as one word
+    bool quad_aligned() const { return (reinterpret_cast<uintptr_t>(stats) & 15) == 0; } // load_quad(): four pairs, i % 4 == 0
     __device__ __forceinline__ Raw load(int i) const { return reinterpret_cast<const uint32_t *>(stats)[i]; }
+    __device__ __forceinline__ uint4 load_quad(int i) const { return *reinterpret_cast<const uint4 *>(stats + 2 * (int64_t)i); }
     __device__ __forceinline__ int cls(Raw pair, const int *thr) const
     {
         const uint32_t r = pair >> 16;
         if (r <= (uint32_t)kMaxPattern) return (int)r >= thr[1] ? 0 : ((int)r >= thr[0] ? 1 : 2);
         return width_class(qbits_of_norm(r, u)); // negative or NaN norms: the rule itself
     }
+    // the recount's form of cls(): counters without a branch.  The pattern is the high half of the pair, so r >= t is
+    // pair >= t << 16 for 0 <= t <= 0x8000 whatever the low half holds: `ge8` counts the pairs at or above the 8-bit
+    // threshold, `ge4` those at or above the 4-bit one, `top` keeps the largest pair seen (a pattern above kMaxPattern
+    // -- a negative or NaN norm -- is outside the thresholds' range, and whoever finds one counts the batch again with cls())
+    struct Tally {
+        uint32_t t8, t4, ge8, ge4, top;
+    };
+    __device__ __forceinline__ Tally tally_begin(const int *thr) const
+    {
+        return Tally{(uint32_t)min(max(thr[1], 0), 0x8000) << 16, (uint32_t)min(max(thr[0], 0), 0x8000) << 16, 0u, 0u, 0u};
+    }
+    __device__ __forceinline__ void tally(Tally &t, Raw pair) const
+    {
+        t.ge8 += pair >= t.t8 ? 1u : 0u;
+        t.ge4 += pair >= t.t4 ? 1u : 0u;
+        t.top = max(t.top, pair);
+    }
+    __device__ __forceinline__ bool tally_beyond(const Tally &t) const { return t.top >= ((uint32_t)kMaxPattern + 1u) << 16; }
+    // superchunks of the 8-bit and of the 4-bit class among those tallied (cls() asks for the 8-bit threshold first)
+    __device__ __forceinline__ uint32_t tally_n8(const Tally &t) const { return t.ge8; }
+    __device__ __forceinline__ uint32_t tally_n4(const Tally &t) const { return t.t4 <= t.t8 ? t.ge4 - t.ge8 : 0u; }
 };
 
 // three 21-bit counters in one word
@@ -128,7 +156,12 @@ constexpr int kOneBatch = 8;       // loads in flight per thread while recountin
 // HIST: the launch has a few workgroups more than tiles (one per 8192 superchunks); they add the norm patterns of the
 // bucket to `hist` (what the search for the next step's u works on) while the others plan, so the histogram costs no
 // launch of its own.
-template <class W, bool HIST>
+// QUAD: the recount of the tiles before reads four superchunks per load (a late tile's recount is a string of dependent
+// round trips to the L2, and a quarter as many requests make it a quarter as long).
+// SEARCH: the thresholds are not among the arguments (u is read from device memory) and two waves search for them; a
+// variant of its own, because with the choice left to run time the compiler moves the loop-invariant part of that search
+// (a hundred instructions) in front of the recount of every launch.
+template <class W, bool HIST, bool QUAD, bool SEARCH>
 __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t *__restrict__ qbits_out, int nsc,
                                                               int32_t *__restrict__ order, int32_t *__restrict__ work,
                                                               uint32_t *__restrict__ hist)
@@ -152,34 +185,76 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
     if (own < nsc) own_raw = widths.load(own);
     uint64_t mine = 0;
     int t2[2]; // the thresholds: from the kernel arguments, or searched by two waves and handed over through LDS
-    bool ready = widths.known(t2);
-    for (int i0 = 0; i0 < nbefore; i0 += kOneBatch * kOneThreads) {
-        typename W::Raw raw[kOneBatch];
+    bool ready = widths.known(t2) || !SEARCH;
+    constexpr int kStep = QUAD ? 4 : 1; // superchunks per load; nbefore is a whole number of tiles
+    for (int i0 = 0; i0 < nbefore; i0 += kOneBatch * kOneThreads * kStep) {
+        typename W::Raw raw[QUAD ? 1 : kOneBatch];
+        uint4 quad[QUAD ? kOneBatch : 1];
 #pragma unroll
         for (int j = 0; j < kOneBatch; j++) {
-            const int i = i0 + j * kOneThreads + (int)threadIdx.x;
-            if (i < nbefore) raw[j] = widths.load(i);
+            const int i = i0 + (j * kOneThreads + (int)threadIdx.x) * kStep;
+            if (i < nbefore) {
+                if constexpr (QUAD)
+                    quad[j] = widths.load_quad(i);
+                else
+                    raw[j] = widths.load(i);
+            }
         }
+        if constexpr (SEARCH) {
+            if (!ready) {
+                widths.prepare(thr, wave, lane);
+                __syncthreads();
+                t2[0] = thr[0];
+                t2[1] = thr[1];
+                ready = true;
+            }
+        }
+        if constexpr (QUAD && std::is_same<typename W::Raw, uint32_t>::value) {
+            // a late tile's recount is a few dozen classifications per thread on a compute unit that holds sixteen such
+            // waves: counted without branches, and once more the long way in the rare batch with a pattern outside the
+            // thresholds' range (a negative or NaN norm)
+            typename W::Tally tl = widths.tally_begin(t2);
+            uint32_t seen = 0;
+#pragma unroll
+            for (int j = 0; j < kOneBatch; j++) {
+                const int i = i0 + (j * kOneThreads + (int)threadIdx.x) * kStep;
+                if (i < nbefore) {
+                    widths.tally(tl, quad[j].x);
+                    widths.tally(tl, quad[j].y);
+                    widths.tally(tl, quad[j].z);
+                    widths.tally(tl, quad[j].w);
+                    seen += 4;
+                }
+            }
+            if (__builtin_amdgcn_ballot_w64(widths.tally_beyond(tl)) == 0) {
+                const uint32_t n8 = widths.tally_n8(tl), n4 = widths.tally_n4(tl);
+                mine += (uint64_t)n8 | ((uint64_t)n4 << 21) | ((uint64_t)(seen - n8 - n4) << 42);
+            } else {
+#pragma unroll // (a loop would index the loaded values by a variable: they would live in scratch memory)
+                for (int j = 0; j < kOneBatch; j++) {
+                    const int i = i0 + (j * kOneThreads + (int)threadIdx.x) * kStep;
+                    if (i < nbefore)
+                        mine += one_of(widths.cls(quad[j].x, t2)) + one_of(widths.cls(quad[j].y, t2)) +
+                                one_of(widths.cls(quad[j].z, t2)) + one_of(widths.cls(quad[j].w, t2));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < kOneBatch; j++) {
+                const int i = i0 + (j * kOneThreads + (int)threadIdx.x) * kStep;
+                if (i < nbefore) mine += one_of(widths.cls(raw[j], t2));
+            }
+        }
+    }
+    if constexpr (SEARCH) {
         if (!ready) {
             widths.prepare(thr, wave, lane);
             __syncthreads();
             t2[0] = thr[0];
             t2[1] = thr[1];
-            ready = true;
-        }
-#pragma unroll
-        for (int j = 0; j < kOneBatch; j++) {
-            const int i = i0 + j * kOneThreads + (int)threadIdx.x;
-            if (i < nbefore) mine += one_of(widths.cls(raw[j], t2));
         }
     }
-    if (!ready) {
-        widths.prepare(thr, wave, lane);
-        __syncthreads();
-        t2[0] = thr[0];
-        t2[1] = thr[1];
-    }
-    // the wave's total of the recount: a thread has counted at most 63 superchunks, a wave at most 4032 per class, so
+    // the wave's total of the recount: a thread has counted at most 64 superchunks, a wave at most 4096 per class, so
     // two classes share a word (lane 63 of the scan holds the total)
     const uint32_t mine01 = wave_scan_inclusive((uint32_t)field(mine, 0) | ((uint32_t)field(mine, 1) << 16));
     const uint32_t mine2 = wave_scan_inclusive((uint32_t)field(mine, 2));
@@ -557,12 +632,25 @@ static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *o
 {
     const int ntiles = (int)((nsc + kTile - 1) / kTile);
     if (ntiles <= kOneMaxTiles && widths.word_aligned()) {
-        if (hist)
-            hipLaunchKernelGGL((plan_one_kernel<W, true>), dim3(ntiles + (int)((nsc + kHistBatch - 1) / kHistBatch)),
-                               dim3(kOneThreads), 0, stream, widths, qbits_out, (int)nsc, order, work, hist);
-        else
-            hipLaunchKernelGGL((plan_one_kernel<W, false>), dim3(ntiles), dim3(kOneThreads), 0, stream, widths, qbits_out,
-                               (int)nsc, order, work, hist);
+        const dim3 grid(hist ? ntiles + (int)((nsc + kHistBatch - 1) / kHistBatch) : ntiles), block(kOneThreads);
+        const bool quad = std::is_same<typename W::Raw, uint32_t>::value && widths.quad_aligned();
+        int t2[2];
+        const bool search = !widths.known(t2);
+#define DQ_PLAN_ONE(HIST, QUAD)                                                                                            \
+    do {                                                                                                                   \
+        if (search)                                                                                                        \
+            hipLaunchKernelGGL((plan_one_kernel<W, HIST, QUAD, true>), grid, block, 0, stream, widths, qbits_out, (int)nsc, \
+                               order, work, hist);                                                                         \
+        else                                                                                                               \
+            hipLaunchKernelGGL((plan_one_kernel<W, HIST, QUAD, false>), grid, block, 0, stream, widths, qbits_out,          \
+                               (int)nsc, order, work, hist);                                                               \
+    } while (0)
+        if (hist) {
+            if (quad) DQ_PLAN_ONE(true, true); else DQ_PLAN_ONE(true, false);
+        } else {
+            if (quad) DQ_PLAN_ONE(false, true); else DQ_PLAN_ONE(false, false);
+        }
+#undef DQ_PLAN_ONE
         return hipGetLastError();
     }
     if (hist) {
