@@ -6,8 +6,9 @@
 //   order[nsc .. nsc + n4)         indices with qbits[i] == 4, ascending
 //   order[2 nsc .. 2 nsc + n2)     indices with qbits[i] == 2, ascending
 //   work[0..2] = n8, n4, n2;  work[3] = superchunks of any other width (in no group)
+//   work[4..5]                     the two threshold patterns (two-launch path with widths from statistics)
 //   work[8 ...]                    per-tile counts of the two-launch path (tile b = superchunks
-//                                  [1024 b, 1024 b + 1024))
+//                                  [1024 b, 1024 b + 1024)), four per tile; behind them the totals of every 64 tiles
 //
 // Every group has a region of its own, so where an index goes depends only on the superchunks before it.
 // Buckets of up to 65536 superchunks (64 tiles) take ONE launch: the workgroup of tile b counts the
@@ -380,6 +381,203 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
     }
 }
 
+// ---- two launches, widths from statistics (long buckets) ----------------------------------------------
+//
+// The kernels above let every workgroup of the second launch add up the counts of all tiles (four 4-byte loads per
+// tile): with T tiles that is T * T * 16 bytes of L2 reads -- 0.9 GB at the 7,630 tiles of a 2 * 10^9-element bucket,
+// 100 us for a plan whose own traffic is 60 MB.  Here the first launch takes a group of tiles per workgroup and leaves,
+// beside the count of every tile, the total of its group; a workgroup of the second launch then reads the totals of
+// the groups before its own and the counts of the tiles before it inside its group: at most 256 + 31 entries of 16
+// bytes (groups of 8 or 32 tiles, see group_tiles_for).  The first launch also leaves the two threshold patterns in work[4..5] (found on the host, or searched
+// by two waves of every workgroup when u is read from device memory), so the second neither searches nor evaluates
+// the rule; both classify four superchunks per 16-byte load.  Needs stats and work 16-byte aligned.
+
+// tiles per workgroup of the first launch: 8 (one per wave) up to 1,024 tiles, 32 (two per wave) beyond -- at most 256
+// groups up to 8,192 tiles, the 2^31 elements an int32 index reaches
+constexpr int kFewTiles = 1024;
+inline int group_tiles_for(int64_t ntiles) { return ntiles <= kFewTiles ? 8 : 32; }
+
+// the classes of up to four superchunks of a quad, counted into n[0..2]
+__device__ __forceinline__ void count_quad_slow(const WidthsFromStats &widths, uint4 q, int valid, const int *t2, uint32_t (&n)[3])
+{
+    const uint32_t v[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        if (k < valid) {
+            const int c = widths.cls(v[k], t2);
+#pragma unroll
+            for (int w = 0; w < 3; w++) n[w] += c == w ? 1u : 0u;
+        }
+    }
+}
+
+// superchunks [i, i + 4) of the statistics as four pairs; those at and beyond nsc read as zero pairs
+__device__ __forceinline__ uint4 load_quad_guarded(const WidthsFromStats &widths, int64_t i, int64_t nsc, int &valid)
+{
+    valid = (int)min((int64_t)4, max((int64_t)0, nsc - i));
+    if (valid == 4) return widths.load_quad((int)i);
+    uint4 q = make_uint4(0, 0, 0, 0);
+    if (valid > 0) q.x = widths.load((int)i);
+    if (valid > 1) q.y = widths.load((int)i + 1);
+    if (valid > 2) q.z = widths.load((int)i + 2);
+    return q;
+}
+
+template <bool SEARCH, int G, int THREADS>
+__global__ __launch_bounds__(THREADS) void plan_count_stats_kernel(WidthsFromStats widths, int64_t nsc, int ntiles,
+                                                                  int32_t *__restrict__ work)
+{
+    constexpr int kSuperTiles = G, kCountThreads = THREADS;
+    __shared__ int thr[2];
+    __shared__ uint32_t group_total[4];
+    widths.resolve();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int t2[2];
+    widths.known(t2);
+    if (threadIdx.x < 4) group_total[threadIdx.x] = 0;
+    if constexpr (SEARCH) widths.prepare(thr, wave, lane);
+    __syncthreads();
+    if constexpr (SEARCH) {
+        t2[0] = thr[0];
+        t2[1] = thr[1];
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        work[4] = t2[0];
+        work[5] = t2[1];
+    }
+    int4 *tile_counts = reinterpret_cast<int4 *>(work + 8);
+    const int tile0 = (int)blockIdx.x * kSuperTiles;
+    for (int k = wave; k < kSuperTiles && tile0 + k < ntiles; k += kCountThreads / 64) { // the bounds are the wave's own
+        const int tile = tile0 + k;
+        const int64_t base = (int64_t)tile * kTile + lane * 4;
+        uint4 q[4];
+        int valid[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) q[j] = load_quad_guarded(widths, base + j * 256, nsc, valid[j]);
+        WidthsFromStats::Tally tl = widths.tally_begin(t2);
+        uint32_t seen = 0;
+        bool ragged = false;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (valid[j] == 4) {
+                widths.tally(tl, q[j].x);
+                widths.tally(tl, q[j].y);
+                widths.tally(tl, q[j].z);
+                widths.tally(tl, q[j].w);
+                seen += 4;
+            } else if (valid[j] > 0) {
+                ragged = true;
+            }
+        }
+        uint32_t n[3];
+        if (__builtin_amdgcn_ballot_w64(ragged || widths.tally_beyond(tl)) == 0) {
+            n[0] = widths.tally_n8(tl);
+            n[1] = widths.tally_n4(tl);
+            n[2] = seen - n[0] - n[1];
+        } else { // the bucket's last tile, or a negative or NaN norm somewhere in this one: class by class
+            n[0] = n[1] = n[2] = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) count_quad_slow(widths, q[j], valid[j], t2, n);
+        }
+        // a lane has counted at most 16 superchunks, the wave 1024: two classes share a word
+        const uint32_t s01 = wave_scan_inclusive(n[0] | (n[1] << 16));
+        const uint32_t s2 = wave_scan_inclusive(n[2]);
+        if (lane == 63) {
+            const int c8 = (int)(s01 & 0xffffu), c4 = (int)(s01 >> 16), c2 = (int)s2;
+            tile_counts[tile] = make_int4(c8, c4, c2, 0);
+            atomicAdd(&group_total[0], (uint32_t)c8);
+            atomicAdd(&group_total[1], (uint32_t)c4);
+            atomicAdd(&group_total[2], (uint32_t)c2);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        tile_counts[ntiles + blockIdx.x] = make_int4((int)group_total[0], (int)group_total[1], (int)group_total[2], 0);
+}
+
+__global__ __launch_bounds__(kThreads) void plan_place_stats_kernel(WidthsFromStats widths, int64_t *__restrict__ qbits_out,
+                                                                   int64_t nsc, int ntiles, int kSuperTiles,
+                                                                   int32_t *__restrict__ order, int32_t *__restrict__ work)
+{
+    __shared__ int before[4], total[4];
+    __shared__ uint64_t wave_sum[kThreads / 64];
+    widths.resolve(); // (cls() evaluates the rule itself for a negative or NaN norm)
+    if (threadIdx.x < 4) {
+        before[threadIdx.x] = 0;
+        total[threadIdx.x] = 0;
+    }
+    __syncthreads();
+    const int t2[2] = {work[4], work[5]};
+    const int4 *tile_counts = reinterpret_cast<const int4 *>(work + 8);
+    const int group = (int)blockIdx.x / kSuperTiles, inside = (int)blockIdx.x % kSuperTiles;
+    const int ngroups = (ntiles + kSuperTiles - 1) / kSuperTiles;
+    {
+        // entries [0, group): the totals of the groups before; [group, group + inside): the tiles before inside the group
+        int b[3] = {0, 0, 0};
+        for (int e = threadIdx.x; e < group + inside; e += kThreads) {
+            const int4 c = e < group ? tile_counts[ntiles + e] : tile_counts[group * kSuperTiles + (e - group)];
+            b[0] += c.x;
+            b[1] += c.y;
+            b[2] += c.z;
+        }
+#pragma unroll
+        for (int w = 0; w < 3; w++) {
+            if (b[w]) atomicAdd(&before[w], b[w]);
+        }
+        if (blockIdx.x == 0) { // the group sizes of the whole bucket
+            int t[3] = {0, 0, 0};
+            for (int e = threadIdx.x; e < ngroups; e += kThreads) {
+                const int4 c = tile_counts[ntiles + e];
+                t[0] += c.x;
+                t[1] += c.y;
+                t[2] += c.z;
+            }
+#pragma unroll
+            for (int w = 0; w < 3; w++) {
+                if (t[w]) atomicAdd(&total[w], t[w]);
+            }
+        }
+    }
+    __syncthreads();
+    if (blockIdx.x == 0 && threadIdx.x < 4) work[threadIdx.x] = threadIdx.x < 3 ? total[threadIdx.x] : 0;
+
+    const int64_t base = (int64_t)blockIdx.x * kTile + threadIdx.x * kPer;
+    static_assert(kPer == 4, "a thread places the four superchunks of one 16-byte load");
+    int valid;
+    const uint4 q = load_quad_guarded(widths, base, nsc, valid);
+    const uint32_t v[4] = {q.x, q.y, q.z, q.w};
+    int cls[kPer];
+    uint64_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < kPer; k++) {
+        cls[k] = 3;
+        if (k < valid) {
+            cls[k] = widths.cls(v[k], t2);
+            if (qbits_out) qbits_out[base + k] = cls[k] == 0 ? 8 : (cls[k] == 1 ? 4 : 2);
+        }
+        mine += one_of(cls[k]);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t scanned = wave_scan_inclusive((uint32_t)field(mine, 0) | ((uint32_t)field(mine, 1) << 10) |
+                                                 ((uint32_t)field(mine, 2) << 20));
+    const uint64_t incl = (uint64_t)(scanned & 0x3ffu) | ((uint64_t)((scanned >> 10) & 0x3ffu) << 21) |
+                          ((uint64_t)((scanned >> 20) & 0x3ffu) << 42);
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    uint64_t excl = incl - mine;
+    for (int w = 0; w < wave; w++) excl += wave_sum[w];
+    int64_t pos[3];
+#pragma unroll
+    for (int w = 0; w < 3; w++) pos[w] = (int64_t)w * nsc + before[w] + field(excl, w);
+#pragma unroll
+    for (int k = 0; k < kPer; k++) {
+#pragma unroll
+        for (int w = 0; w < 3; w++) {
+            if (cls[k] == w) order[pos[w]++] = (int32_t)(base + k);
+        }
+    }
+}
+
 // ---- fixed-proportion groups: the stable descending sort of the norms in one launch -------------------
 //
 // testbed_evaluation/new_comm_hooks/comm_hooks.py:710-721: sorted = argsort(norms, descending, stable); the first
@@ -623,7 +821,13 @@ hipError_t launch_group_plan_sorted(const void *stats, int64_t nsc, int64_t top,
     return hipGetLastError();
 }
 
-int64_t group_plan_work_ints(int64_t nsc) { return 8 + 4 * ((nsc + kTile - 1) / kTile); }
+// header, four counts per tile, four per group of tiles
+int64_t group_plan_work_ints(int64_t nsc)
+{
+    const int64_t ntiles = (nsc + kTile - 1) / kTile;
+    const int64_t g = group_tiles_for(ntiles);
+    return 8 + 4 * ntiles + 4 * ((ntiles + g - 1) / g);
+}
 
 // hist (only with widths from statistics): the bucket's norm patterns are added to it
 template <class W>
@@ -656,6 +860,30 @@ static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *o
     if (hist) {
         const hipError_t eh = launch_norm_histogram(widths.norm_stats_host(), nsc, hist, stream);
         if (eh != hipSuccess) return eh;
+    }
+    if constexpr (std::is_same<W, WidthsFromStats>::value) {
+        if (widths.quad_aligned() && (reinterpret_cast<uintptr_t>(work) & 15) == 0) {
+            int t2[2];
+            const bool search = !widths.known(t2);
+            const int g = group_tiles_for(ntiles);
+            const dim3 groups((unsigned)((ntiles + g - 1) / g));
+#define DQ_PLAN_COUNT(SEARCH)                                                                                              \
+    do {                                                                                                                   \
+        if (g == 8)                                                                                                        \
+            hipLaunchKernelGGL((plan_count_stats_kernel<SEARCH, 8, 512>), groups, dim3(512), 0, stream, widths, nsc, ntiles, \
+                               work);                                                                                      \
+        else                                                                                                               \
+            hipLaunchKernelGGL((plan_count_stats_kernel<SEARCH, 32, 1024>), groups, dim3(1024), 0, stream, widths, nsc,     \
+                               ntiles, work);                                                                              \
+    } while (0)
+            if (search) DQ_PLAN_COUNT(true); else DQ_PLAN_COUNT(false);
+#undef DQ_PLAN_COUNT
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            hipLaunchKernelGGL(plan_place_stats_kernel, dim3(ntiles), dim3(kThreads), 0, stream, widths, qbits_out, nsc, ntiles, g,
+                               order, work);
+            return hipGetLastError();
+        }
     }
     hipLaunchKernelGGL(plan_count_kernel<W>, dim3(ntiles), dim3(kThreads), 0, stream, widths, nsc, work);
     hipError_t e = hipGetLastError();

@@ -206,3 +206,44 @@ def test_group_plan_stats_two_launch_paths(capi, oracle, nsc, shift):
         idx = np.nonzero(want == w)[0]
         assert (order_h[gi * nsc:gi * nsc + idx.size] == idx).all()
         assert (order_h[gi * nsc + idx.size:(gi + 1) * nsc] == -1).all()
+
+
+@pytest.mark.parametrize("u_on_device", [False, True])
+@pytest.mark.parametrize("nsc,shift", [(65537, 0), (70000, 0), (70001, 0), (70002, 2), (200003, 0), (1048576 + 1029, 0)])
+def test_group_plan_stats_long_buckets(capi, oracle, nsc, shift, u_on_device):
+    """more than 64 tiles with 16-byte aligned statistics: the first launch counts 64 tiles per workgroup, four
+    superchunks per load, and leaves the thresholds and the totals of its 64 tiles; the second reads those.  Ragged
+    ends, negative, NaN and infinite norms, u as a number and from device memory, and (shift 2) the statistics 4 bytes off,
+    which takes the older pair of kernels: all against the width rule of the oracle"""
+    g = torch.Generator().manual_seed(nsc + shift)
+    norms = torch.exp(torch.randn(nsc, generator=g) * 6.0).to(torch.bfloat16)
+    special = torch.randperm(nsc, generator=g)[:400]
+    norms[special[:100]] = -norms[special[:100]]
+    norms[special[100:200]] = float("nan")
+    norms[special[200:300]] = float("inf")
+    norms[special[300:400]] = 0.0
+    norms[nsc - 1] = float("nan")                      # in the ragged last quad where there is one
+    buf = torch.zeros(2 * nsc + 8, dtype=torch.bfloat16)
+    stats = buf[shift:shift + 2 * nsc].view(nsc, 2)
+    stats[:, 1] = norms
+    stats[:, 0] = torch.randn(nsc, generator=g).to(torch.bfloat16)   # the means in the low halves must not matter
+    stats_d = buf.to(DEV)[shift:shift + 2 * nsc].view(nsc, 2)
+    assert stats_d.data_ptr() % 16 == (2 * shift) % 16
+    order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    work = torch.full((capi.group_plan_work_ints(nsc),), -5, dtype=torch.int32, device=DEV)
+    qout = torch.empty(nsc, dtype=torch.int64, device=DEV)
+    u = 7.1
+    capi.group_plan_stats(stats_d, torch.tensor([u], dtype=torch.float64, device=DEV) if u_on_device else u, qout, order, work)
+    want = oracle.dynamic_bitrate_qbits(to_bits(norms), u)
+    assert (qout.cpu().numpy() == want).all()
+    counts = work[:4].tolist()
+    assert counts == [int((want == 8).sum()), int((want == 4).sum()), int((want == 2).sum()), 0] and min(counts[:3]) > 0
+    order_h = order.cpu().numpy()
+    for gi, w in enumerate((8, 4, 2)):
+        idx = np.nonzero(want == w)[0]
+        assert (order_h[gi * nsc:gi * nsc + idx.size] == idx).all()
+        assert (order_h[gi * nsc + idx.size:(gi + 1) * nsc] == -1).all()
+    # without the width output, and once more into the same work buffer (nothing of a plan may depend on what an earlier one left)
+    order2 = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
+    capi.group_plan_stats(stats_d, u, None, order2, work)
+    assert torch.equal(order, order2) and work[:4].tolist() == counts
