@@ -628,6 +628,18 @@ def kernels(dev, n=6553600):
                 if strategy >= 2 and tdt != torch.float16:
                     line("scaling_dec_comp (fused)", lambda: capi.scaling_dec_comp(packed, src, send, rnd, n, nbits, 16, strategy),
                          (sb + 2) * n + 2 * nb, **tag)
+        if tdt != torch.float16:
+            # the launch of the chunk-16 codec's shape with the arithmetic taken away, over the same buffers: what the 4-bit
+            # lines above can be held against (the bytes named are those of the codec call of that shape)
+            nb4 = capi.required_bytes(n, 4, 16, 2)
+            packed4 = torch.zeros(nb4, dtype=torch.uint8, device=dev)
+            run = nb4 * 1024 // n
+            line("tile_io_floor (encoder shape: elements + pool read, records written)",
+                 lambda: capi.tile_io_floor(0, src, rand, packed4, run, n // 1024), (sb + 2) * n + nb4, elements=name, nbits=4)
+            line("tile_io_floor (encoder shape without a pool)",
+                 lambda: capi.tile_io_floor(0, src, None, packed4, run, n // 1024), sb * n + nb4, elements=name, nbits=4)
+            line("tile_io_floor (decoder shape: records read, elements written)",
+                 lambda: capi.tile_io_floor(1, out, None, packed4, run, n // 1024), sb * n + nb4, elements=name, nbits=4)
         del src, rand, out
     # chunk sizes other than 16: the thread-per-chunk kernels
     src = x32.to(torch.bfloat16)
