@@ -209,12 +209,13 @@ def test_group_plan_stats_two_launch_paths(capi, oracle, nsc, shift):
 
 
 @pytest.mark.parametrize("u_on_device", [False, True])
-@pytest.mark.parametrize("nsc,shift", [(65537, 0), (70000, 0), (70001, 0), (70002, 2), (200003, 0), (1048576 + 1029, 0)])
+@pytest.mark.parametrize("nsc,shift", [(5000, 0), (5000, 2), (65537, 0), (70000, 0), (70001, 0), (70002, 2), (200003, 0), (1048576 + 1029, 0)])
 def test_group_plan_stats_long_buckets(capi, oracle, nsc, shift, u_on_device):
-    """more than 64 tiles with 16-byte aligned statistics: the first launch counts 64 tiles per workgroup, four
-    superchunks per load, and leaves the thresholds and the totals of its 64 tiles; the second reads those.  Ragged
+    """more than 64 tiles with 16-byte aligned statistics: the first launch counts a group of tiles per workgroup, four
+    superchunks per load, and leaves the thresholds and the totals of its group; the second reads those.  Ragged
     ends, negative, NaN and infinite norms, u as a number and from device memory, and (shift 2) the statistics 4 bytes off,
-    which takes the older pair of kernels: all against the width rule of the oracle"""
+    which takes the older pair of kernels; 5,000 superchunks: the same inputs through the one-launch kernel, with its
+    four-per-load recount and (shift 2) without: all against the width rule of the oracle"""
     g = torch.Generator().manual_seed(nsc + shift)
     norms = torch.exp(torch.randn(nsc, generator=g) * 6.0).to(torch.bfloat16)
     special = torch.randperm(nsc, generator=g)[:400]
