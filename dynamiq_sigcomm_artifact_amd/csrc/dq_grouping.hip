@@ -37,6 +37,10 @@ static_assert(64 * kPer < 1024, "the wave scan of the placing kernel packs three
 
 __device__ __forceinline__ int width_class(int64_t q) { return q == 8 ? 0 : q == 4 ? 1 : q == 2 ? 2 : 3; }
 
+// three 21-bit counters in one word
+__device__ __forceinline__ uint64_t one_of(int cls) { return cls < 3 ? (uint64_t)1 << (21 * cls) : 0; }
+__device__ __forceinline__ int field(uint64_t p, int cls) { return (int)((p >> (21 * cls)) & 0x1fffff); }
+
 // where the widths come from: an int64 array, or the norm column of the interleaved bf16 stats.
 //   operator()(i)           the width of superchunk i by the rule itself (two-launch path)
 //   prepare / load / cls    the one-launch path: prepare() fills thr[2] (no barrier inside), load() only
@@ -47,9 +51,35 @@ struct WidthsFromArray {
     __device__ __forceinline__ int64_t operator()(int64_t i) const { return qbits[i]; }
     __device__ __forceinline__ int64_t width(int64_t i) const { return qbits[i]; }
     bool word_aligned() const { return true; }
-    bool quad_aligned() const { return false; }
-    __device__ __forceinline__ uint4 load_quad(int) const { return make_uint4(0, 0, 0, 0); } // (never taken)
-    struct Tally {};
+    // the recount's loads: two widths per 16 bytes (i even), counted without branches; a width whose high half is
+    // set is outside what the three compares see, and whoever finds one counts the batch again with cls()
+    static constexpr int kPerLoad = 2;
+    bool quad_aligned() const { return (reinterpret_cast<uintptr_t>(qbits) & 15) == 0; }
+    __device__ __forceinline__ uint4 load_quad(int i) const { return *reinterpret_cast<const uint4 *>(qbits + i); }
+    struct Tally {
+        uint32_t n8, n4, n2, high;
+    };
+    __device__ __forceinline__ Tally tally_begin(const int *) const { return Tally{0u, 0u, 0u, 0u}; }
+    __device__ __forceinline__ void tally_one(Tally &t, uint32_t lo, uint32_t hi) const
+    {
+        t.n8 += lo == 8u ? 1u : 0u;
+        t.n4 += lo == 4u ? 1u : 0u;
+        t.n2 += lo == 2u ? 1u : 0u;
+        t.high |= hi;
+    }
+    __device__ __forceinline__ void tally_load(Tally &t, uint4 q) const
+    {
+        tally_one(t, q.x, q.y);
+        tally_one(t, q.z, q.w);
+    }
+    __device__ __forceinline__ bool tally_beyond(const Tally &t) const { return t.high != 0u; }
+    __device__ __forceinline__ uint32_t tally_n8(const Tally &t) const { return t.n8; }
+    __device__ __forceinline__ uint32_t tally_n4(const Tally &t) const { return t.n4; }
+    __device__ __forceinline__ uint32_t tally_n2(const Tally &t, uint32_t) const { return t.n2; }
+    __device__ __forceinline__ uint64_t count_slow(uint4 q, const int *thr) const
+    {
+        return one_of(cls((int64_t)(((uint64_t)q.y << 32) | q.x), thr)) + one_of(cls((int64_t)(((uint64_t)q.w << 32) | q.z), thr));
+    }
     __device__ __forceinline__ const uint16_t *norm_stats() const { return nullptr; }
     const void *norm_stats_host() const { return nullptr; }
     __device__ __forceinline__ void resolve() {}
@@ -121,11 +151,21 @@ struct WidthsFromStats {
     // superchunks of the 8-bit and of the 4-bit class among those tallied (cls() asks for the 8-bit threshold first)
     __device__ __forceinline__ uint32_t tally_n8(const Tally &t) const { return t.ge8; }
     __device__ __forceinline__ uint32_t tally_n4(const Tally &t) const { return t.t4 <= t.t8 ? t.ge4 - t.ge8 : 0u; }
+    __device__ __forceinline__ uint32_t tally_n2(const Tally &t, uint32_t seen) const { return seen - tally_n8(t) - tally_n4(t); }
+    static constexpr int kPerLoad = 4; // (mean, norm) pairs per 16 bytes
+    __device__ __forceinline__ void tally_load(Tally &t, uint4 q) const
+    {
+        tally(t, q.x);
+        tally(t, q.y);
+        tally(t, q.z);
+        tally(t, q.w);
+    }
+    __device__ __forceinline__ uint64_t count_slow(uint4 q, const int *thr) const
+    {
+        return one_of(cls(q.x, thr)) + one_of(cls(q.y, thr)) + one_of(cls(q.z, thr)) + one_of(cls(q.w, thr));
+    }
 };
 
-// three 21-bit counters in one word
-__device__ __forceinline__ uint64_t one_of(int cls) { return cls < 3 ? (uint64_t)1 << (21 * cls) : 0; }
-__device__ __forceinline__ int field(uint64_t p, int cls) { return (int)((p >> (21 * cls)) & 0x1fffff); }
 
 // Inclusive scan over the wave's 64 lanes with data-parallel-primitive moves (shifts by 1, 2, 4, 8 inside the rows of
 // sixteen lanes, then lane 15 of a row into the next row, lane 31 into the upper half): a dozen register-to-register
@@ -157,7 +197,7 @@ constexpr int kOneBatch = 8;       // loads in flight per thread while recountin
 // HIST: the launch has a few workgroups more than tiles (one per 8192 superchunks); they add the norm patterns of the
 // bucket to `hist` (what the search for the next step's u works on) while the others plan, so the histogram costs no
 // launch of its own.
-// QUAD: the recount of the tiles before reads four superchunks per load (a late tile's recount is a string of dependent
+// QUAD: the recount of the tiles before reads 16 bytes per load, four (mean, norm) pairs or two widths (a late tile's recount is a string of dependent
 // round trips to the L2, and a quarter as many requests make it a quarter as long).
 // SEARCH: the thresholds are not among the arguments (u is read from device memory) and two waves search for them; a
 // variant of its own, because with the choice left to run time the compiler moves the loop-invariant part of that search
@@ -187,7 +227,7 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
     uint64_t mine = 0;
     int t2[2]; // the thresholds: from the kernel arguments, or searched by two waves and handed over through LDS
     bool ready = widths.known(t2) || !SEARCH;
-    constexpr int kStep = QUAD ? 4 : 1; // superchunks per load; nbefore is a whole number of tiles
+    constexpr int kStep = QUAD ? W::kPerLoad : 1; // superchunks per load; nbefore is a whole number of tiles
     for (int i0 = 0; i0 < nbefore; i0 += kOneBatch * kOneThreads * kStep) {
         typename W::Raw raw[QUAD ? 1 : kOneBatch];
         uint4 quad[QUAD ? kOneBatch : 1];
@@ -210,7 +250,7 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
                 ready = true;
             }
         }
-        if constexpr (QUAD && std::is_same<typename W::Raw, uint32_t>::value) {
+        if constexpr (QUAD) {
             // a late tile's recount is a few dozen classifications per thread on a compute unit that holds sixteen such
             // waves: counted without branches, and once more the long way in the rare batch with a pattern outside the
             // thresholds' range (a negative or NaN norm)
@@ -220,23 +260,18 @@ __global__ __launch_bounds__(kOneThreads) void plan_one_kernel(W widths, int64_t
             for (int j = 0; j < kOneBatch; j++) {
                 const int i = i0 + (j * kOneThreads + (int)threadIdx.x) * kStep;
                 if (i < nbefore) {
-                    widths.tally(tl, quad[j].x);
-                    widths.tally(tl, quad[j].y);
-                    widths.tally(tl, quad[j].z);
-                    widths.tally(tl, quad[j].w);
-                    seen += 4;
+                    widths.tally_load(tl, quad[j]);
+                    seen += kStep;
                 }
             }
             if (__builtin_amdgcn_ballot_w64(widths.tally_beyond(tl)) == 0) {
                 const uint32_t n8 = widths.tally_n8(tl), n4 = widths.tally_n4(tl);
-                mine += (uint64_t)n8 | ((uint64_t)n4 << 21) | ((uint64_t)(seen - n8 - n4) << 42);
+                mine += (uint64_t)n8 | ((uint64_t)n4 << 21) | ((uint64_t)widths.tally_n2(tl, seen) << 42);
             } else {
 #pragma unroll // (a loop would index the loaded values by a variable: they would live in scratch memory)
                 for (int j = 0; j < kOneBatch; j++) {
                     const int i = i0 + (j * kOneThreads + (int)threadIdx.x) * kStep;
-                    if (i < nbefore)
-                        mine += one_of(widths.cls(quad[j].x, t2)) + one_of(widths.cls(quad[j].y, t2)) +
-                                one_of(widths.cls(quad[j].z, t2)) + one_of(widths.cls(quad[j].w, t2));
+                    if (i < nbefore) mine += widths.count_slow(quad[j], t2);
                 }
             }
         } else {
@@ -837,7 +872,7 @@ static hipError_t run_plan(W widths, int64_t *qbits_out, int64_t nsc, int32_t *o
     const int ntiles = (int)((nsc + kTile - 1) / kTile);
     if (ntiles <= kOneMaxTiles && widths.word_aligned()) {
         const dim3 grid(hist ? ntiles + (int)((nsc + kHistBatch - 1) / kHistBatch) : ntiles), block(kOneThreads);
-        const bool quad = std::is_same<typename W::Raw, uint32_t>::value && widths.quad_aligned();
+        const bool quad = widths.quad_aligned();
         int t2[2];
         const bool search = !widths.known(t2);
 #define DQ_PLAN_ONE(HIST, QUAD)                                                                                            \

@@ -20,6 +20,11 @@ def test_group_plan_matches_nonzero(capi, nsc):
     q = torch.tensor([2, 4, 8, 16])[torch.randint(0, 4 if nsc > 5 else 3, (nsc,), generator=g)].to(DEV)
     if nsc == 1023:
         q[:] = 8            # a single group
+    if nsc in (25600, 65536):
+        # widths that are none of 2, 4, 8 in every form: zero, odd, negative, and values whose low half reads 8, 4 or 2
+        odd = torch.tensor([0, 1, 3, -8, (1 << 32) + 8, (5 << 32) + 4, -(1 << 40) + 2, 1 << 62], device=DEV)
+        q[torch.randperm(nsc, generator=g)[:64].to(DEV)] = odd.repeat(8)
+        q = q.view(-1)
     order = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
     work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
     for rep in range(3):        # the same work buffer serves call after call
@@ -29,7 +34,7 @@ def test_group_plan_matches_nonzero(capi, nsc):
         capi.group_plan(q, order, work)
         counts = work[:4].tolist()
         want = [torch.nonzero(q == w).view(-1) for w in (8, 4, 2)]
-        assert counts[:3] == [w.numel() for w in want] and counts[3] == int((q == 16).sum())
+        assert counts[:3] == [w.numel() for w in want] and counts[3] == nsc - sum(w.numel() for w in want)
         for g in range(3):      # one region of nsc entries per width; nothing written beyond a group
             region = order[g * nsc:(g + 1) * nsc].cpu()
             assert torch.equal(region[:counts[g]], want[g].cpu().to(torch.int32))
