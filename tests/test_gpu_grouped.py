@@ -253,3 +253,46 @@ def test_group_plan_stats_long_buckets(capi, oracle, nsc, shift, u_on_device):
     order2 = torch.full((3 * nsc,), -1, dtype=torch.int32, device=DEV)
     capi.group_plan_stats(stats_d, u, None, order2, work)
     assert torch.equal(order, order2) and work[:4].tolist() == counts
+
+
+def test_group_plan_stats_thresholds_kept_in_the_work_buffer(capi, oracle):
+    """with u in device memory the one-launch plan leaves the thresholds it searched for in work[4..6] and a later launch on
+    the same buffer takes them from there when u has the same bits: same plans with and without, after a change of u, and
+    with anything else in those words (zeros, noise, the right u beside a broken seal, the entry of another u)"""
+    nsc = 30000
+    g = torch.Generator().manual_seed(5)
+    norms = torch.exp(torch.randn(nsc, generator=g) * 6.0).to(torch.bfloat16)
+    norms[torch.randperm(nsc, generator=g)[:50]] = float("nan")
+    stats = torch.zeros((nsc, 2), dtype=torch.bfloat16)
+    stats[:, 1] = norms
+    stats_d = stats.to(DEV)
+    order = torch.empty(3 * nsc, dtype=torch.int32, device=DEV)
+
+    def plan(u_dev, work):
+        order.fill_(-1)
+        q = torch.empty(nsc, dtype=torch.int64, device=DEV)
+        capi.group_plan_stats(stats_d, u_dev, q, order, work)
+        return q.cpu().numpy(), order.clone(), work[:4].tolist()
+
+    work = torch.zeros(capi.group_plan_work_ints(nsc), dtype=torch.int32, device=DEV)
+    u_dev = torch.tensor([7.1], dtype=torch.float64, device=DEV)
+    for u in (7.1, 7.1, 3.25, 3.25, 7.1, 60.0, -10.0, 7.1):
+        u_dev.fill_(u)
+        q, o, c = plan(u_dev, work)
+        want = oracle.dynamic_bitrate_qbits(to_bits(norms), u)
+        assert (q == want).all(), u
+        kept = work[4:8].cpu().numpy().view(np.uint32)
+        assert kept[0] == np.float32(u).view(np.uint32) and kept[2] == kept[0] ^ kept[1] ^ 0x9e3779b9, u
+        # the same through a fresh buffer (a search) and through one whose words 4..7 hold other things
+        for fill in ("zeros", "noise", "broken seal", "other u"):
+            w2 = torch.zeros_like(work)
+            if fill == "noise":
+                w2[4:8] = torch.randint(-2 ** 31, 2 ** 31 - 1, (4,), generator=g, dtype=torch.int64).to(torch.int32).to(DEV)
+            elif fill == "broken seal":
+                w2[4:8] = work[4:8]
+                w2[5] += 1
+            elif fill == "other u":
+                w2[4:8] = work[4:8]
+                w2[4] += 1
+            q2, o2, c2 = plan(u_dev, w2)
+            assert (q2 == want).all() and torch.equal(o2, o) and c2 == c, (u, fill)
