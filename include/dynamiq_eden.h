@@ -201,6 +201,11 @@ int dq_group_plan_sorted(const void *stats, int64_t nsc, int64_t top_count, int6
  * then needs no read-back of u at all.  hist (may be NULL; dq_bitrate_hist_ints()
  * uint32): the bucket's norm patterns are also added to it, as by
  * dq_norm_histogram, by a few more workgroups of the same launch (for nsc <= 65536).
+ * The launch leaves the two width thresholds it derived from u in work[4..6]
+ * (with the bits of u and a check word); the next call on the same work buffer
+ * with the same u takes them from there instead of searching again, so a
+ * caller that plans many buckets per step does well to keep one work buffer
+ * per stream.  Whatever else those words hold is recognised and ignored.
  * No counterpart in the reference, which keeps u on the host. */
 int dq_group_plan_stats_dev_u(const void *stats, const double *u_dev, int64_t nsc,
                               int64_t *qbits_out, int32_t *order, int32_t *work,
