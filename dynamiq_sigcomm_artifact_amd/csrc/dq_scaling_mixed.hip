@@ -111,9 +111,12 @@ __global__ __launch_bounds__(64) void mixed_compress_kernel(const void *__restri
     __shared__ float table[(MEE && FUSED) ? 256 : 1];
     constexpr int RESZ = RDT == DQ_F32 ? 4 : 2;
 
-    if (RDT == DQ_PHILOX && plan.step_dev) key.step += *plan.step_dev; // (a scalar load that leaves with the three counts)
+    // the step's addend leaves with the three counts and is used behind them: added here, its round trip would stand in
+    // front of theirs
+    const uint64_t step_add = (RDT == DQ_PHILOX && plan.step_dev) ? *plan.step_dev : 0;
     const Segment s = locate(plan, blockIdx.x, 1);
     if (s.cls == 3) return;
+    key.step += step_add;
     const RowIds rows = row_ids_plain(plan.order + s.row0);
     const void *r = RDT == DQ_PHILOX ? nullptr : static_cast<const char *>(rnd) + s.pos0 * 256 * RESZ;
     const uint8_t *in = FUSED ? recv + s.byte_off : nullptr;
