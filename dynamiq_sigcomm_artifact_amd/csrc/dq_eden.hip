@@ -3,7 +3,8 @@
 // (testbed_evaluation/new_comm_hooks/thc_hooks.py:149-181), which the reference runs as chains of
 // torch element-wise ops and reductions around eden_utils.Hadamard.
 //
-// EDEN quantise, four launches, no host synchronisation:
+// EDEN quantise, four launches (three for vectors of up to 2^22 elements, where every workgroup of `bins` folds the
+// partial sums of `sumsq` itself instead of waiting for a launch of one workgroup to do it), no host synchronisation:
 //   sumsq   tile b = elements [4096 b, 4096 b + 4096): thread t adds v^2 of elements t + 256 k (k ascending)
 //           in double, the 256 sums are halved (stride 128 .. 1) -> work[b]
 //   norm    one workgroup folds work[] the same way -> sumsq (double); norm = sqrtf((float)sumsq)
@@ -85,12 +86,16 @@ __global__ __launch_bounds__(kEdenThreads) void eden_norm_kernel(const double *_
 // bit plane in registers.  The boundaries sit in LDS in breadth-first order of the search tree (node 1 = the
 // middle boundary, children of node i at 2 i and 2 i + 1): the lanes of a wave read one level of the tree at a
 // time, consecutive words, where the sorted layout puts a whole level into a few banks.
-template <int NBITS>
+// FOLD: the norm is not in result[3] yet; the workgroup folds the `tiles` partial sums in `sums` the way eden_norm_kernel
+// does (the same association: the same bits), and workgroup 0 leaves result[0] and result[3] as that kernel would.  `work`
+// (the products) is then a region of its own: other workgroups are still reading `sums`.
+template <int NBITS, bool FOLD>
 __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__restrict__ vec, int64_t n,
                                                                 const float *__restrict__ boundaries,
                                                                 const float *__restrict__ centroids,
-                                                                const float *__restrict__ result, float sqrt_n,
-                                                                uint32_t *__restrict__ packed, double *__restrict__ work)
+                                                                float *__restrict__ result, float sqrt_n,
+                                                                uint32_t *__restrict__ packed, double *__restrict__ work,
+                                                                const double *__restrict__ sums, int64_t tiles)
 {
     constexpr int L = 1 << NBITS;
     __shared__ double lds[kEdenThreads];
@@ -104,7 +109,17 @@ __global__ __launch_bounds__(kEdenThreads) void eden_bins_kernel(const float *__
         }
     }
     __syncthreads();
-    const float norm = result[3];
+    float norm;
+    if constexpr (FOLD) {
+        const float s = (float)fold_array(sums, tiles, lds);
+        norm = __builtin_sqrtf(s);
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            result[0] = s;
+            result[3] = norm;
+        }
+    } else {
+        norm = result[3];
+    }
     const uint32_t nb = __float_as_uint(norm);
     const bool ordinary = nb >= 0x0d800000u && nb <= 0x71800000u; // uniform over the grid
     const double yn = ordinary ? recip_f64(norm) : 0.0;
@@ -281,7 +296,14 @@ inline int64_t eden_tiles(int64_t n) { return (n + kEdenTile - 1) / kEdenTile; }
 
 } // namespace
 
-int64_t eden_work_doubles(int64_t n) { return eden_tiles(n); }
+// vectors of up to kEdenFoldTiles tiles take three launches and keep the two kinds of partial sums apart
+constexpr int64_t kEdenFoldTiles = 1024;
+
+int64_t eden_work_doubles(int64_t n)
+{
+    const int64_t tiles = eden_tiles(n);
+    return tiles <= kEdenFoldTiles ? 2 * tiles : tiles;
+}
 
 hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *boundaries, const float *centroids, int nbits,
                                 uint32_t *packed, float *result, double *work, hipStream_t stream)
@@ -289,21 +311,31 @@ hipError_t launch_eden_quantize(const float *vec, int64_t n, const float *bounda
     const int64_t tiles = eden_tiles(n);
     const float sqrt_n = (float)sqrt((double)n);
     dim3 grid((unsigned)tiles), block(kEdenThreads);
+    const bool fold = tiles <= kEdenFoldTiles;
+    double *products = fold ? work + tiles : work;
     hipLaunchKernelGGL(eden_sumsq_kernel, grid, block, 0, stream, vec, n, work);
-    hipLaunchKernelGGL(eden_norm_kernel, dim3(1), block, 0, stream, work, tiles, result);
+    if (!fold) hipLaunchKernelGGL(eden_norm_kernel, dim3(1), block, 0, stream, work, tiles, result);
+#define DQ_EDEN_BINS(B)                                                                                                   \
+    do {                                                                                                                  \
+        if (fold)                                                                                                         \
+            hipLaunchKernelGGL((eden_bins_kernel<B, true>), grid, block, 0, stream, vec, n, boundaries, centroids, result, \
+                               sqrt_n, packed, products, work, tiles);                                                    \
+        else                                                                                                              \
+            hipLaunchKernelGGL((eden_bins_kernel<B, false>), grid, block, 0, stream, vec, n, boundaries, centroids, result, \
+                               sqrt_n, packed, products, work, tiles);                                                    \
+    } while (0)
     switch (nbits) {
-#define DQ_EDEN_CASE(B)                                                                                                  \
-    case B:                                                                                                              \
-        hipLaunchKernelGGL(eden_bins_kernel<B>, grid, block, 0, stream, vec, n, boundaries, centroids, result, sqrt_n, packed, \
-                           work);                                                                                        \
-        break;
-        DQ_EDEN_CASE(1) DQ_EDEN_CASE(2) DQ_EDEN_CASE(3) DQ_EDEN_CASE(4) DQ_EDEN_CASE(5) DQ_EDEN_CASE(6) DQ_EDEN_CASE(7)
-    default:
-        hipLaunchKernelGGL(eden_bins_kernel<8>, grid, block, 0, stream, vec, n, boundaries, centroids, result, sqrt_n, packed, work);
-        break;
-#undef DQ_EDEN_CASE
+    case 1: DQ_EDEN_BINS(1); break;
+    case 2: DQ_EDEN_BINS(2); break;
+    case 3: DQ_EDEN_BINS(3); break;
+    case 4: DQ_EDEN_BINS(4); break;
+    case 5: DQ_EDEN_BINS(5); break;
+    case 6: DQ_EDEN_BINS(6); break;
+    case 7: DQ_EDEN_BINS(7); break;
+    default: DQ_EDEN_BINS(8); break;
     }
-    hipLaunchKernelGGL(eden_scale_kernel, dim3(1), block, 0, stream, work, tiles, result);
+#undef DQ_EDEN_BINS
+    hipLaunchKernelGGL(eden_scale_kernel, dim3(1), block, 0, stream, products, tiles, result);
     return hipGetLastError();
 }
 
@@ -356,7 +388,8 @@ hipError_t launch_eden_quantize_static(const float *vec, int64_t n, const float 
         scratch = static_scratch_of[device];
     }
     // every word of scratch that a kernel reads has been written by an earlier kernel of this same
-    // call (sumsq -> norm, bins -> scale), so nothing has to be cleared between calls
+    // call (sumsq -> norm or bins, bins -> scale), so nothing has to be cleared between calls; the array
+    // holds the two regions of a short vector (2 * 1024 doubles) as it holds the one of a long vector
     return launch_eden_quantize(vec, n, boundaries, centroids, nbits, packed, result, scratch, stream);
 }
 

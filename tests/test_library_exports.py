@@ -172,7 +172,7 @@ def test_argument_errors_are_reported_before_any_device_work():
     err(L.dq_eden_dequantize_irht(P, 64, P, 4, P, 0, N, 64, F1, N, 0, S), "null pointer")
     err(L.dq_thc_dequantize_irht(P, P, 1, P, 0, 64, F1, P, P, 0, S), "multiple of block")
     err(L.dq_thc_dequantize(P, P, 64, N, P, 0, S), "null pointer")
-    assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 + 4 * 4 and capi.group_plan_work_ints(1048577) == 8 + 4 * 1025 + 4 * 33 and capi.eden_work_doubles(8192) == 2 and capi.bitrate_hist_ints() == 32768
+    assert capi.group_plan_work_ints(25600) == 8 + 4 * 25 + 4 * 4 and capi.group_plan_work_ints(1048577) == 8 + 4 * 1025 + 4 * 33 and capi.eden_work_doubles(8192) == 4 and capi.eden_work_doubles(4096 * 1025) == 1025 and capi.bitrate_hist_ints() == 32768
     # the sorted plan: four ints up to 65535 superchunks, the radix sort's buffers (about 12.2 bytes per superchunk) beyond
     assert capi.group_plan_sorted_work_ints(65535) == 4
     big = capi.group_plan_sorted_work_ints(8_000_000)
