@@ -6,8 +6,8 @@
 //   order[nsc .. nsc + n4)         indices with qbits[i] == 4, ascending
 //   order[2 nsc .. 2 nsc + n2)     indices with qbits[i] == 2, ascending
 //   work[0..2] = n8, n4, n2;  work[3] = superchunks of any other width (in no group)
-//   work[4..6]                     thresholds kept between launches: the two patterns (two-launch path with widths from
-//                                  statistics), or u's bits, the patterns and a seal (one launch, u from device memory)
+//   work[4..6]                     thresholds kept between launches (widths from statistics): u's bits, the two patterns in
+//                                  one word, and a seal
 //   work[8 ...]                    per-tile counts of the two-launch path (tile b = superchunks
 //                                  [1024 b, 1024 b + 1024)), four per tile; behind them the totals of every 64 tiles
 //
@@ -459,7 +459,7 @@ __global__ __launch_bounds__(kThreads) void plan_place_kernel(W widths, int64_t 
 // 100 us for a plan whose own traffic is 60 MB.  Here the first launch takes a group of tiles per workgroup and leaves,
 // beside the count of every tile, the total of its group; a workgroup of the second launch then reads the totals of
 // the groups before its own and the counts of the tiles before it inside its group: at most 256 + 31 entries of 16
-// bytes (groups of 8 or 32 tiles, see group_tiles_for).  The first launch also leaves the two threshold patterns in work[4..5] (found on the host, or searched
+// bytes (groups of 8 or 32 tiles, see group_tiles_for).  The first launch also leaves the two threshold patterns in work[4..6] (found on the host, or searched
 // by two waves of every workgroup when u is read from device memory), so the second neither searches nor evaluates
 // the rule; both classify four superchunks per 16-byte load.  Needs stats and work 16-byte aligned.
 
@@ -501,20 +501,32 @@ __global__ __launch_bounds__(THREADS) void plan_count_stats_kernel(WidthsFromSta
     constexpr int kSuperTiles = G, kCountThreads = THREADS;
     __shared__ int thr[2];
     __shared__ uint32_t group_total[4];
+    const uint4 kept = *reinterpret_cast<const uint4 *>(work + 4); // (work is 16-byte aligned on this path)
     widths.resolve();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int t2[2];
-    widths.known(t2);
+    bool ready = widths.known(t2);
     if (threadIdx.x < 4) group_total[threadIdx.x] = 0;
-    if constexpr (SEARCH) widths.prepare(thr, wave, lane);
+    if constexpr (SEARCH) {
+        // the thresholds an earlier plan on this work buffer found for the same u (see plan_one_kernel), or a search
+        if (kept.x == widths.u_key() && kept.z == (kept.x ^ kept.y ^ kThresholdSeal)) {
+            t2[0] = (int)(kept.y & 0xffffu);
+            t2[1] = (int)(kept.y >> 16);
+            ready = true;
+        }
+        if (!ready) widths.prepare(thr, wave, lane);
+    }
     __syncthreads();
     if constexpr (SEARCH) {
-        t2[0] = thr[0];
-        t2[1] = thr[1];
+        if (!ready) {
+            t2[0] = thr[0];
+            t2[1] = thr[1];
+        }
     }
+    // for the second launch, and for the next plan on this buffer: u's bits, both patterns (at most 0x7f81 each), the seal
     if (blockIdx.x == 0 && threadIdx.x == 0) {
-        work[4] = t2[0];
-        work[5] = t2[1];
+        const uint32_t both = (uint32_t)t2[0] | ((uint32_t)t2[1] << 16);
+        *reinterpret_cast<uint4 *>(work + 4) = make_uint4(widths.u_key(), both, widths.u_key() ^ both ^ kThresholdSeal, 0u);
     }
     int4 *tile_counts = reinterpret_cast<int4 *>(work + 8);
     const int tile0 = (int)blockIdx.x * kSuperTiles;
@@ -578,7 +590,7 @@ __global__ __launch_bounds__(kThreads) void plan_place_stats_kernel(WidthsFromSt
         total[threadIdx.x] = 0;
     }
     __syncthreads();
-    const int t2[2] = {work[4], work[5]};
+    const int t2[2] = {(int)((uint32_t)work[5] & 0xffffu), (int)((uint32_t)work[5] >> 16)}; // as the first launch left them
     const int4 *tile_counts = reinterpret_cast<const int4 *>(work + 8);
     const int group = (int)blockIdx.x / kSuperTiles, inside = (int)blockIdx.x % kSuperTiles;
     const int ngroups = (ntiles + kSuperTiles - 1) / kSuperTiles;

@@ -255,11 +255,12 @@ def test_group_plan_stats_long_buckets(capi, oracle, nsc, shift, u_on_device):
     assert torch.equal(order, order2) and work[:4].tolist() == counts
 
 
-def test_group_plan_stats_thresholds_kept_in_the_work_buffer(capi, oracle):
-    """with u in device memory the one-launch plan leaves the thresholds it searched for in work[4..6] and a later launch on
-    the same buffer takes them from there when u has the same bits: same plans with and without, after a change of u, and
-    with anything else in those words (zeros, noise, the right u beside a broken seal, the entry of another u)"""
-    nsc = 30000
+@pytest.mark.parametrize("nsc", [30000, 70000])
+def test_group_plan_stats_thresholds_kept_in_the_work_buffer(capi, oracle, nsc):
+    """with u in device memory the plan (one launch, or the pair for long buckets) leaves the thresholds it searched for in
+    work[4..6] and a later launch on the same buffer takes them from there when u has the same bits: same plans with and
+    without, after a change of u, and with anything else in those words (zeros, noise, the right u beside a broken seal, the
+    entry of another u)"""
     g = torch.Generator().manual_seed(5)
     norms = torch.exp(torch.randn(nsc, generator=g) * 6.0).to(torch.bfloat16)
     norms[torch.randperm(nsc, generator=g)[:50]] = float("nan")
