@@ -298,3 +298,25 @@ def test_tile_io_floor_moves_exactly_the_bytes_of_the_codec_shape(capi, adt, bdt
     assert bool((guard[1024 * tiles:] == 3.0).all())
     with pytest.raises(ValueError):
         capi.tile_io_floor(0, a, b, run, run_bytes, tiles + 1)
+
+
+@pytest.mark.parametrize("dt", [F16, BF16, F32])
+@pytest.mark.parametrize("n", [8, 255, 256 * 9 + 5, 256 * 40 + 4])
+def test_superchunk_add_mean_copy_alignments(capi, oracle, dt, n):
+    """the 16-byte kernel of add_mean_copy (two-byte and four-byte elements), the kernel for what it leaves over, and views
+    that are not 16-byte aligned give the oracle's bits and write nothing beyond n"""
+    tdt = TORCH_DT[dt]
+    g = torch.Generator().manual_seed(n)
+    nsc = (n + 255) // 256
+    res = (torch.randn(nsc * 256, generator=g) * 1e-2).to(tdt)
+    stats = (torch.randn(nsc * 2, generator=g) * 1e-2).to(torch.bfloat16)
+    want = oracle.superchunk_add_mean_copy(to_bits(res), to_bits(stats), n, dt)
+    for shift_in, shift_out in ((0, 0), (1, 0), (0, 1), (4, 4)):
+        rbuf = torch.zeros(nsc * 256 + 8, dtype=tdt, device=DEV)
+        rview = rbuf[shift_in:shift_in + nsc * 256]
+        rview.copy_(res)
+        obuf = torch.full((n + 16,), 5.0, dtype=tdt, device=DEV)
+        oview = obuf[shift_out:]
+        capi.superchunk_add_mean_copy(rview, oview, stats.to(DEV), n)
+        _eq("add_mean %d/%d" % (shift_in, shift_out), to_bits(oview[:n]), want)
+        assert bool((oview[n:] == 5.0).all()) and bool((obuf[:shift_out] == 5.0).all())
