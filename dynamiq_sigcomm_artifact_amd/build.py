@@ -3,6 +3,9 @@
   libdynamiq_eden.so   HIP kernels + C ABI (hipcc, gfx950)
   eden_utils*.so       pybind11 / libtorch binding with the reference module's
                        function names (g++), linked against libdynamiq_eden.so
+  tests/cxx/liblaunchers_probe.so
+                       test helper: a C++ caller of include/dynamiq_eden_launchers.hpp
+                       (amdclang++, host code only), linked against libdynamiq_eden.so
 
 Run as ``python -m dynamiq_sigcomm_artifact_amd.build`` or call ``build_all()``.
 hipcc cross-compiles for gfx950 without a GPU present.
@@ -127,9 +130,34 @@ def build_extension(verbose=True):
     return out
 
 
+PROBE_SRC = os.path.join(PKG_DIR, "..", "tests", "cxx", "launchers_probe.cpp")
+PROBE_PATH = os.path.join(PKG_DIR, "..", "tests", "cxx", "liblaunchers_probe.so")
+
+
+def launchers_probe_command(out, throw=False):
+    """the compile line of the C++ launcher header's test caller: plain C++ for the host, the HIP headers only for
+    their types"""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [os.path.join(rocm, "bin", "amdclang++"), "-O1", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Werror",
+           "-D__HIP_PLATFORM_AMD__=1", "-I" + os.path.join(rocm, "include"), "-I" + os.path.join(PKG_DIR, "..", "include")]
+    if throw:
+        cmd.append("-DDYNAMIQ_LAUNCHERS_THROW")
+    cmd += [PROBE_SRC, "-o", out, "-L" + PKG_DIR, "-l:" + LIB_NAME, "-Wl,-rpath," + PKG_DIR,
+            "-Wl,-rpath,$ORIGIN/../../dynamiq_sigcomm_artifact_amd"]
+    return cmd
+
+
+def build_launchers_probe(verbose=True):
+    dt = _run(launchers_probe_command(PROBE_PATH), "amdclang++ launchers_probe.cpp")
+    if verbose:
+        print("  clang %-28s %.1fs" % (os.path.basename(PROBE_PATH), dt))
+    return PROBE_PATH
+
+
 def build_all(verbose=True):
     lib = build_kernels(verbose)
     ext = build_extension(verbose)
+    build_launchers_probe(verbose)
     return lib, ext
 
 
@@ -139,3 +167,5 @@ if __name__ == "__main__":
         build_kernels(only_changed="--changed" in sys.argv)
     if only in ("all", "ext"):
         build_extension()
+    if only in ("all", "probe"):
+        build_launchers_probe()
