@@ -50,6 +50,52 @@ __device__ __forceinline__ bool ordinary_scale(float d)
     return b >= 0x0d800000u && b <= 0x71800000u;
 }
 
+// a / b correctly rounded to binary32 for binary16-valued a and b (b an ordinary scale or a lattice constant), given
+// y = RN32(1 / b): q0 = RN(a y) is within an ulp of the quotient, the remainder a - q0 b then fits binary32 and the fused
+// operation computes it exactly, and RN(q0 + rem y) is the correctly rounded quotient (Markstein's theorem; its one
+// exception, a divisor whose significand is all ones, needs 24 significant bits).  y is the double reciprocal rounded
+// to binary32: 1 / b with an 11-bit b stays 2^-36 (relative) clear of every binary32 rounding boundary unless it is
+// representable, so rounding the double (within 2^-51) rounds the reciprocal itself.  Quotients and remainders stay
+// normal numbers for these operands; the sign of a zero quotient is not kept (no code depends on it).
+__device__ __forceinline__ float div_half_operands(float a, float b, float y)
+{
+    const float q0 = a * y;
+    const float rem = __builtin_fmaf(-q0, b, a);
+    return __builtin_fmaf(rem, y, q0);
+}
+
+// The codes of a binary16 chunk with the half-precision operations done by the machine's own binary16 instructions
+// (IEEE, round to nearest even: the same value as the binary32 operation followed by one rounding that the op-by-op
+// chain below spells out, without the two conversions around every operation).  For a wave whose scales are all
+// ordinary, whose elements hold no NaN and whose random values lie in [0, 1]: every quotient is then finite and below
+// 2 R in magnitude, so none of the saturating conversions of the reference's chain can fire, floor, the two
+// differences, ceil and their sum are small integers or exact, and the clamp can be taken on the binary16 sum.
+// A zero quotient needs no case of its own under MEE: the lattice coordinate of 0 is log2(0 / c + 1) / l2b = +0.
+template <int NBITS, bool MEE, class RR, class ARG>
+__device__ __forceinline__ void half_codes_native(const Raw16<DQ_F16> &v, const RR &r, float d, double yd, const ARG &mp,
+                                                  uint32_t (&w)[Rec<NBITS>::WORDS])
+{
+    constexpr int R = Rec<NBITS>::R;
+    const float y = (float)yd;
+    const float yc = MEE ? (float)mp.inv_c : 0.0f, yl = MEE ? (float)mp.inv_l2b : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        _Float16 x = (_Float16)div_half_operands(v.get(i), d, y);
+        if (MEE) {
+            const _Float16 arg = (_Float16)div_half_operands((float)__builtin_fabsf16(x), mp.c, yc) + (_Float16)1.0f;
+            const _Float16 lg = (_Float16)log2_det_ge1((float)arg);
+            const _Float16 lat = (_Float16)div_half_operands((float)lg, mp.l2b, yl);
+            x = x < (_Float16)0.0f ? -lat : lat;
+        }
+        const _Float16 fl = __builtin_floorf16(x);
+        const _Float16 t = (x - fl) - (_Float16)r.get(i);
+        _Float16 c = fl + __builtin_ceilf16(t);
+        c = c < (_Float16)(-R) ? (_Float16)(-R) : c;
+        c = c > (_Float16)R ? (_Float16)R : c;
+        words_put<NBITS>(w, i, (uint32_t)(int)(c + (_Float16)R));
+    }
+}
+
 template <int DT, int RDT, int NBITS, bool HIER, bool MEE>
 __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restrict__ src, uint8_t *__restrict__ dst,
                                                             const void *__restrict__ rnd, int64_t nchunks, int vec,
@@ -79,11 +125,23 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
         r.zero();
     }
 
-    float a = __builtin_fabsf(v.get(0));
+    float a;
+    bool half_nan = false; // binary16 elements: the wave holds a NaN
+    if constexpr (DT == DQ_F16) {
+        // the largest magnitude as an integer maximum of the bit patterns; a NaN sorts above infinity, and only then does
+        // the reference's maximum (which passes over a NaN operand) need its own comparisons
+        const uint32_t amax = v.absmax_half_bits();
+        half_nan = __builtin_amdgcn_ballot_w64(amax > 0x7c00u) != 0;
+        a = f16_bits_to_f32(amax);
+        if (half_nan) {
+            a = __builtin_fabsf(v.get(0));
 #pragma unroll
-    for (int i = 1; i < 16; i++) {
-        const float e = __builtin_fabsf(v.get(i));
-        a = (DT == DQ_F16) ? h_max(a, e) : __builtin_fmaxf(a, e);
+            for (int i = 1; i < 16; i++) a = h_max(a, __builtin_fabsf(v.get(i)));
+        }
+    } else {
+        a = __builtin_fabsf(v.get(0));
+#pragma unroll
+        for (int i = 1; i < 16; i++) a = __builtin_fmaxf(a, __builtin_fabsf(v.get(i)));
     }
 
     float d;             // the scale the codes are computed against
@@ -127,6 +185,11 @@ __global__ __launch_bounds__(64) void tile16_compress_kernel(const void *__restr
         if (estimated) estimate_codes<NBITS, MEE>(v, r, d, mp, w);
     }
     const double yd = fast && !estimated ? recip_f64(d) : 0.0;
+    if constexpr (DT == DQ_F16) {
+        // (estimated doubles as "the codes are done")
+        estimated = fast && !half_nan && __builtin_amdgcn_ballot_w64(!r.unit_interval()) == 0;
+        if (estimated) half_codes_native<NBITS, MEE>(v, r, d, yd, mp, w);
+    }
     // the element-wise chain, compiled once per kind of division: with the choice made per element the compiler
     // computes both quotients and selects
     auto chain = [&](auto by_reciprocal) {

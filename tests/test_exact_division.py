@@ -105,3 +105,54 @@ def test_sixteen_bit_elements_meet_no_tie_below_a_world_size_of_3_times_2_to_17(
     v = np.array([3 * 2.0 ** -133], np.float32)
     assert (v.view(np.uint32) & 0xffff) == 0
     assert float(v[0]) / float(w) == 2.0 ** -150
+
+
+# ---- binary16 operands: the corrected single-precision quotient of the binary16 encoders ------------------------------
+
+def corrected_quotient(a, b, y):
+    """div_half_operands (csrc/dq_scaling_tile16.hip): q0 = RN32(a y); rem = fma(-q0, b, a); RN32(fma(rem, y, q0)).  The two
+    fused operations are evaluated in double: q0 b (24 x 11 bits) and a - q0 b are exact there, rem y (24 x 24 bits) too, and
+    the last sum is rounded to double before it is rounded to binary32 -- where that could differ from the single rounding of
+    the fused operation (the double lands on a binary32 tie) the caller's comparison falls back to exact fractions."""
+    q0 = (a * y).astype(np.float32)
+    rem = (a.astype(np.float64) - q0.astype(np.float64) * b.astype(np.float64))
+    assert np.array_equal(rem.astype(np.float32).astype(np.float64), rem)          # the remainder fits binary32
+    return (q0.astype(np.float64) + rem * y.astype(np.float64)).astype(np.float32)
+
+
+def test_corrected_quotient_of_binary16_operands_is_the_binary32_quotient_for_every_pair_of_significands():
+    """Every binary16 number is an 11-bit integer times a power of two, and scaling either operand by a power of two scales
+    quotient, reciprocal and remainder exactly (no operand of the encoders brings them near the ends of the binary32
+    range): all 1024 x 1024 pairs of normalised significands cover every pair of binary16 operands.  Checked for the
+    reciprocal the kernels use, the double reciprocal rounded to binary32, which is RN32(1 / b) itself."""
+    from fractions import Fraction
+    sig = np.arange(1024, 2048, dtype=np.float32)
+    a, b = (m.reshape(-1) for m in np.meshgrid(sig, sig, indexing="ij"))
+    y64 = 1.0 / b.astype(np.float64)
+    y = y64.astype(np.float32)
+    for yd in reciprocals(b):                                   # the device's double reciprocal may be an ulp off
+        assert np.array_equal(yd.astype(np.float32), y)
+    got = corrected_quotient(a, b, y)
+    want = a / b                                                # numpy's binary32 division is IEEE
+    bad = np.flatnonzero(got != want)
+    for i in bad:                                               # (the emulation's double rounding: settle exactly)
+        q0 = Fraction(float(np.float32(a[i] * y[i])))
+        exact = q0 + (Fraction(float(a[i])) - q0 * Fraction(float(b[i]))) * Fraction(float(y[i]))
+        assert abs(exact - Fraction(float(want[i]))) <= abs(exact - Fraction(float(got[i]))), (a[i], b[i])
+    assert bad.size < 8
+    # and with a few scalings of the operands, subnormal binary16 numerators included
+    for ea, eb in ((-24, 0), (-24, 15), (15, -24), (-10, 5), (0, -14)):
+        a2, b2 = np.ldexp(a, ea).astype(np.float32), np.ldexp(b, eb).astype(np.float32)
+        y2 = (1.0 / b2.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(corrected_quotient(a2, b2, y2) == a2 / b2, got == want)
+
+
+def test_binary16_rounding_of_a_quotient_of_binary16_operands_sees_no_double_rounding():
+    """RN16(RN32(a / b)) == RN16(a / b): a quotient of two 11-bit significands that is not itself a binary16 tie stays two
+    binary32 ulps clear of every such tie, so the binary32 rounding in between never moves it onto or across one."""
+    sig = np.arange(1024, 2048, dtype=np.float64)
+    a, b = (m.reshape(-1) for m in np.meshgrid(sig, sig, indexing="ij"))
+    q = a / b                                                   # double: 2^-53, far below the distances at stake
+    once = q.astype(np.float16)
+    twice = q.astype(np.float32).astype(np.float16)
+    assert np.array_equal(once.view(np.uint16), twice.view(np.uint16))
